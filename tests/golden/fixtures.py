@@ -1,0 +1,66 @@
+"""Loaders for the committed known-answer fixtures (see make_fixtures.py).
+
+Each loader returns float32 tensors shaped [1, neurons, T] ready for the
+dynamics API at w_scale = 4096 (the neuron classes' s_scale = 64 * 64), plus
+the expected output spike raster.  The reference's lava-side blocks emit a
+spike one step after the slayer-side tensor does, so ``expected`` is already
+aligned: expected[:, t] is the spike the dynamics must produce at step t,
+for t in [0, T-1).
+"""
+import os
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+W_SCALE = 4096
+
+
+def _unpack(b, T):
+    return np.unpackbits(b, axis=-1)[..., :T].astype(np.int64)
+
+
+def dense_lif():
+    """LIF dense block: vth=6, du=4095 (full current decay), dv=415.
+
+    Returns dict(x=[1,256,T] synaptic input, current_decay, voltage_decay,
+    threshold, expected=[256,T-1]).
+    """
+    z = np.load(os.path.join(HERE, 'netx_dense_lif.npz'))
+    T = int(z['num_steps'])
+    a = z['weight'].astype(np.int64) @ _unpack(z['in_bits'], T)      # [256, T]
+    x = torch.tensor(a * 64 / W_SCALE, dtype=torch.float32).reshape(1, 256, T)
+    return dict(x=x, current_decay=4096.0, voltage_decay=415.0,
+                threshold=6 / 64 + 0.01 / W_SCALE,
+                expected=_unpack(z['out_bits'], T)[:, 1:])
+
+
+def complex_dense_rf():
+    """RF dense block: vth=25, period=11, alpha=0.05 (no reset, phase spike)."""
+    z = np.load(os.path.join(HERE, 'netx_complex_dense_rf.npz'))
+    T = int(z['num_steps'])
+    s = _unpack(z['in_bits'], T)
+    ar = z['weight_real'].astype(np.int64) @ s
+    ai = z['weight_imag'].astype(np.int64) @ s
+    f = lambda a: torch.tensor(a * 64 / W_SCALE, dtype=torch.float32).reshape(1, 256, T)
+    return dict(xr=f(ar), xi=f(ai),
+                sin_decay=float(int(0.95 * np.sin(2 * np.pi / 11) * 4096)),
+                cos_decay=float(int(0.95 * np.cos(2 * np.pi / 11) * 4096)),
+                threshold=25 * 64 / W_SCALE,
+                expected=_unpack(z['out_bits'], T)[:, 1:])
+
+
+def complex_input_rf_iz():
+    """RF_IZ input block: vth=1.1, period=7, alpha=0.05; the same 0/1 input
+    drives the real and the imaginary port; spike = imag >= vth with reset
+    (real -> 0, imag -> vth - 1).  Here the lava block has no extra latency,
+    so expected[:, t] is the spike at step t for all t.
+    """
+    z = np.load(os.path.join(HERE, 'netx_complex_dense_rf.npz'))
+    T = int(z['num_steps'])
+    s = _unpack(z['in_bits'], T)
+    x = torch.tensor(s * 64 / W_SCALE, dtype=torch.float32).reshape(1, 200, T)
+    return dict(x=x,
+                sin_decay=float(int(0.95 * np.sin(2 * np.pi / 7) * 4096)),
+                cos_decay=float(int(0.95 * np.cos(2 * np.pi / 7) * 4096)),
+                threshold=1.1 * 64 / W_SCALE,
+                expected=_unpack(z['iz_out_bits'], T))
