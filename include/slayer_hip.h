@@ -1,0 +1,166 @@
+/*
+ * slayer_hip.h -- C ABI of libslayer_hip.so, the MI355X (gfx950) implementation of
+ * lava-dl SLAYER's neuron-dynamics and temporal-op kernels.
+ *
+ * Every entry point replaces one function of the reference's JIT-built CUDA
+ * modules (citations are relative to src/lava/lib/dl/slayer/ in lava-nc/lava-dl);
+ * the arithmetic follows the reference's CPU branch, which is the semantic
+ * definition (int64 states on the CPU, float32 tensors at every op boundary).
+ *
+ * Conventions
+ *   - All tensor pointers are DEVICE pointers to contiguous float32 data laid out
+ *     [M neurons][T steps], time innermost (M = numel / T).
+ *   - Nothing is allocated, freed or synchronised inside; work is enqueued on
+ *     `stream` (a hipStream_t passed as void*, NULL = the null stream) of the
+ *     device that is current when the call is made.
+ *   - Inputs are never written.  Outputs are fully overwritten.
+ *   - Return value: 0 on success, a positive hipError_t from the launch, or a
+ *     negative SLAYER_E* code for arguments the kernels cannot honour (nothing is
+ *     launched in that case).
+ *   - Per-neuron parameter addressing (decays) follows the reference kernels:
+ *     num_params == 1 -> shared;  otherwise neuron m uses
+ *     param[(m % neurons_per_batch) / (neurons_per_batch / num_params)]
+ *     (leaky_integrator.cu:46-52,145-147): num_params == C is per channel,
+ *     num_params == C*H*W is per neuron.
+ *   - States: num_states == 1 broadcasts one value, otherwise num_states == M.
+ *   - Integer states are held in 32 bits with 64-bit products (as the reference
+ *     kernels do, leaky_integrator.cu:43,61); results equal the int64 CPU branch
+ *     while every state stays inside +-(2^31 - 1).
+ */
+#ifndef SLAYER_HIP_H
+#define SLAYER_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SLAYER_ABI_VERSION 1
+
+#define SLAYER_EINVAL   (-1)   /* inconsistent sizes (M, T, neurons_per_batch, num_params, ...) */
+#define SLAYER_ENULL    (-2)   /* a required pointer is NULL */
+#define SLAYER_ERANGE   (-3)   /* a size exceeds what the kernels index (M*T >= 2^40, T >= 2^31, K > 4096 ...) */
+
+int slayer_abi_version(void);
+
+/* Text for a return code of this library (hipGetErrorString for positive codes). */
+const char *slayer_error_string(int code);
+
+/* ---- leaky integrator ---------------------------------------------------------------- */
+
+/* Replaces LIDynamicsFwd (neuron/dynamics/leaky_integrator.cu:112-153); arithmetic of
+ * _li_dynamics_fwd (neuron/dynamics/leaky_integrator.py:210-231).
+ * y = rs0(y * (4096 - trunc(decay)), 12) + trunc(w * in[t]);  out[t] = float(y) / w;
+ * if thr_scaled > 0 and float(y) >= float(thr_scaled):  y = 0.
+ * thr_scaled = threshold * w_scale computed by the caller in double (pass -w_scale for "no threshold"). */
+int slayer_li_fwd(float *out, const float *in, const float *decay, const float *state,
+                  double thr_scaled, int w_scale,
+                  int64_t M, int64_t neurons_per_batch, int64_t num_decays, int64_t num_states,
+                  int64_t T, void *stream);
+
+/* Replaces LIDynamicsBwd (leaky_integrator.cu:155-200); arithmetic of _li_dynamics_bwd
+ * (leaky_integrator.py:234-259).
+ * grad_in[T-1] = grad_out[T-1];  grad_in[t] = (1 - decay/4096) * grad_in[t+1] + grad_out[t];
+ * grad_decay[j] = sum over the neurons that use decay j of sum_t grad_in[t+1] * out[t].
+ * grad_decay (num_decays floats) may be NULL to skip the parameter gradient.
+ * workspace: M floats of scratch (per-neuron partial sums), required iff grad_decay != NULL. */
+int slayer_li_bwd(float *grad_in, float *grad_decay, const float *grad_out, const float *out,
+                  const float *decay, float *workspace,
+                  int64_t M, int64_t neurons_per_batch, int64_t num_decays,
+                  int64_t T, void *stream);
+
+/* ---- adaptive threshold + refractory ---------------------------------------------------- */
+
+/* Replaces AThDynamicsFwd (neuron/dynamics/adaptive_threshold.cu:81-131) with the CPU
+ * branch's rounding (_ath_dynamics_fwd, neuron/dynamics/adaptive_threshold.py:237-274):
+ * r = rs0(r * (4096 - rd), 12);  th = rs0((th - th0) * (4096 - td), 12) + th0;
+ * th_out[t] = th / w;  ref_out[t] = r / w;  s = trunc(w * in[t]) >= th + r;
+ * th += th_step * s;  r += 2 * th_before_step * s.
+ * th_step_scaled = int(th_scale * w_scale), th0_scaled = int(th0 * w_scale), both taken by the caller. */
+int slayer_ath_fwd(float *th_out, float *ref_out, const float *in,
+                   const float *ref_state, const float *ref_decay,
+                   const float *th_state, const float *th_decay,
+                   int64_t th_step_scaled, int64_t th0_scaled, int w_scale,
+                   int64_t M, int64_t neurons_per_batch,
+                   int64_t num_ref_decays, int64_t num_th_decays,
+                   int64_t num_ref_states, int64_t num_th_states,
+                   int64_t T, void *stream);
+
+/* ---- resonator ------------------------------------------------------------------------------ */
+
+/* Replaces ResDynamicsFwd (neuron/dynamics/resonator.cu:151-198); arithmetic of
+ * _res_dynamics_fwd (neuron/dynamics/resonator.py:333-376).
+ * re = rs0(c*re', 12) - rs0(s*im', 12) + trunc(w*re_in[t]);
+ * im = rs0(s*re', 12) + rs0(c*im', 12) + trunc(w*im_in[t]);   c, s = trunc(cos_decay), trunc(sin_decay)
+ * if thr_scaled >= 0 and float(im) >= float(thr_scaled): re' = 0, im' = trunc(float(thr_scaled - 1)). */
+int slayer_res_fwd(float *re_out, float *im_out, const float *re_in, const float *im_in,
+                   const float *sin_decay, const float *cos_decay,
+                   const float *re_state, const float *im_state,
+                   double thr_scaled, int w_scale,
+                   int64_t M, int64_t neurons_per_batch, int64_t num_decays,
+                   int64_t num_re_states, int64_t num_im_states,
+                   int64_t T, void *stream);
+
+/* Replaces ResDynamicsBwd (resonator.cu:200-262); arithmetic of _res_dynamics_bwd
+ * (resonator.py:379-467) without its host-side NaN scans (the Python caller does those).
+ * gr[t] = c*gr[t+1] + s*gi[t+1] + g_re[t];  gi[t] = -s*gr[t+1] + c*gi[t+1] + g_im[t];  c, s = decay/4096
+ * grad_sin[j] = sum(-gr[t+1]*im[t] + gi[t+1]*re[t]);  grad_cos[j] = sum(gr[t+1]*re[t] + gi[t+1]*im[t]).
+ * grad_sin/grad_cos (num_decays floats each) may both be NULL.
+ * workspace: 2*M floats, required iff the parameter gradients are requested. */
+int slayer_res_bwd(float *g_re_in, float *g_im_in, float *grad_sin, float *grad_cos,
+                   const float *g_re, const float *g_im, const float *re, const float *im,
+                   const float *sin_decay, const float *cos_decay, float *workspace,
+                   int64_t M, int64_t neurons_per_batch, int64_t num_decays,
+                   int64_t T, void *stream);
+
+/* ---- spike functions (elementwise; they replace chains of torch ops, not a .cu) ----------- */
+
+/* Spike.forward (spike/spike.py:64-87).  threshold: num_threshold == 1 -> scalar read from
+ * device memory, == numel -> elementwise.  graded != 0: out = (v >= th) * v / scale. */
+int slayer_spike_fwd(float *spikes, const float *voltage, const float *threshold,
+                     int64_t num_threshold, int graded, float scale, int64_t numel, void *stream);
+
+/* Spike.backward / _spike_backward (spike/spike.py:10-23,113-126).
+ * binary: rho/2/tau * exp(-|v - th| / tau) * g;   graded: rho * exp(min(v - th, 0) / tau) * g. */
+int slayer_spike_bwd(float *grad_voltage, const float *grad_spikes, const float *voltage,
+                     const float *threshold, int64_t num_threshold,
+                     float tau_rho, float scale_rho, int graded, int64_t numel, void *stream);
+
+/* complex.Spike.forward (spike/complex.py:49-92): (re >= th) * (im[t-1] < 0) * (im[t] >= 0)
+ * with im[-1] = imag_last[m] (num_last == 1 broadcasts).  graded != 0 multiplies by re / scale. */
+int slayer_cspike_fwd(float *spikes, const float *re, const float *im, const float *threshold,
+                      int64_t num_threshold, const float *imag_last, int64_t num_last,
+                      int graded, float scale, int64_t M, int64_t T, void *stream);
+
+/* complex.Spike.backward (spike/complex.py:117-167). */
+int slayer_cspike_bwd(float *grad_re, float *grad_im, const float *grad_spikes,
+                      const float *re, const float *im, const float *threshold,
+                      int64_t num_threshold, float tau_rho, float scale_rho, int graded,
+                      int64_t numel, void *stream);
+
+/* ---- time shift --------------------------------------------------------------------------- */
+
+/* Replaces both shift() overloads (utils/time/shift.cu:80-210); semantics of _shift_group /
+ * _shift_individual (utils/time/shift.py:46-91).  out[m][t] = in[m][t - k] (zero outside [0,T)),
+ * lut == NULL: every row moves by scalar_steps, the caller's int(shift / sampling_time) (python
+ * double arithmetic, as _shift_group does); otherwise lut holds neurons_per_batch device floats and
+ * row m moves by trunc(lut[m % neurons_per_batch] / sampling_time), divided in float32. */
+int slayer_shift(float *out, const float *in, const float *lut, int64_t scalar_steps,
+                 float sampling_time, int64_t M, int64_t neurons_per_batch, int64_t T, void *stream);
+
+/* ---- temporal filter ---------------------------------------------------------------------- */
+
+/* Replaces conv fwd (utils/filter/conv.cu:80-124): out[m][t] = Ts * sum_{i<K, t-i>=0} filt[i] * in[m][t-i]. */
+int slayer_conv(float *out, const float *in, const float *filt, int64_t K, float sampling_time,
+                int64_t M, int64_t T, void *stream);
+
+/* Replaces conv bwd (utils/filter/conv.cu:126-171): out[m][t] = Ts * sum_{i<K, t+i<T} filt[i] * in[m][t+i]. */
+int slayer_corr(float *out, const float *in, const float *filt, int64_t K, float sampling_time,
+                int64_t M, int64_t T, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SLAYER_HIP_H */

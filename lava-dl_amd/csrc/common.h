@@ -1,0 +1,30 @@
+// Host-side argument checks shared by the C-ABI entry points.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/slayer_hip.h"
+
+namespace slayer {
+
+constexpr int64_t kMaxT = (int64_t)1 << 30;
+constexpr int64_t kMaxNumel = (int64_t)1 << 40;
+
+inline int check_rows(int64_t M, int64_t T) {
+    if (M < 0 || T < 0) return SLAYER_EINVAL;
+    if (T > kMaxT || (T > 0 && M > kMaxNumel / T)) return SLAYER_ERANGE;
+    if ((M + 63) / 64 > 0x7fffffffLL) return SLAYER_ERANGE;
+    return 0;
+}
+
+// M rows split into batches of npb rows; a parameter vector of n entries maps onto one batch.
+inline int check_params(int64_t M, int64_t npb, int64_t n) {
+    if (npb <= 0 || M % npb != 0) return SLAYER_EINVAL;
+    if (n < 1 || (n > 1 && npb % n != 0)) return SLAYER_EINVAL;
+    return 0;
+}
+
+inline int check_states(int64_t M, int64_t n) { return (n == 1 || n == M) ? 0 : SLAYER_EINVAL; }
+
+inline bool is_pow2(int w) { return w > 0 && (w & (w - 1)) == 0; }
+
+}  // namespace slayer

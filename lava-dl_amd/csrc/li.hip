@@ -1,0 +1,151 @@
+// Leaky integrator: forward fixed-point recurrence and reverse-time gradient.
+#include "common.h"
+#include "tile.h"
+
+namespace slayer {
+
+// ---------------------------------------------------------------------------------- forward
+template <bool POW2>
+struct LiFwd {
+    static constexpr int kIn = 1, kOut = 1;
+    static constexpr bool kReverse = false;
+    struct Params {
+        const float* in[1];
+        float* out[1];
+        const float* decay;
+        const float* state;
+        float w, inv_w, thr;          // thr = +inf when the reset is disabled
+        int64_t npb, num_decays, num_states;
+    };
+    int y, mult;
+    float w, inv_w, thr;
+
+    __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
+        w = p.w; inv_w = p.inv_w; thr = p.thr;
+        y = 0; mult = 0;
+        if (valid) {
+            y = trunc_i32(p.state[p.num_states == 1 ? 0 : m] * w);
+            mult = 4096 - trunc_i32(p.decay[param_index(m, p.npb, p.num_decays)]);
+        }
+    }
+    __device__ __forceinline__ void step(const float (&x)[1], float (&o)[1]) {
+        const int yn = rs0_12(y, mult) + trunc_i32(w * x[0]);
+        const float yf = (float)yn;
+        o[0] = POW2 ? yf * inv_w : yf / w;
+        y = (yf >= thr) ? 0 : yn;
+    }
+    __device__ __forceinline__ void finish(const Params&, int64_t, bool) {}
+};
+
+// --------------------------------------------------------------------------------- backward
+struct LiBwd {
+    static constexpr int kIn = 2, kOut = 1;     // in: grad_out, saved forward output
+    static constexpr bool kReverse = true;
+    struct Params {
+        const float* in[2];
+        float* out[1];
+        const float* decay;
+        float* partial;               // per-neuron sum_t g[t+1] * out[t], or nullptr
+        int64_t npb, num_decays;
+    };
+    float a, g, acc;
+
+    __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
+        g = 0.f; acc = 0.f; a = 0.f;
+        if (valid) a = 1.0f - p.decay[param_index(m, p.npb, p.num_decays)] / 4096.0f;
+    }
+    __device__ __forceinline__ void step(const float (&x)[2], float (&o)[1]) {
+        acc = __fmaf_rn(g, x[1], acc);          // g still holds grad_in[t+1]
+        g = a * g + x[0];                       // separate multiply and add, as torch evaluates it
+        o[0] = g;
+    }
+    __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
+        if (valid && p.partial) p.partial[m] = acc;
+    }
+};
+
+// grad[j] = sum of partial[m] over all rows m whose parameter index is j, accumulated in
+// double in a fixed order (one workgroup per parameter, deterministic).
+__global__ __launch_bounds__(256) void reduce_param_grad(float* grad, const float* partial,
+                                                         int64_t M, int64_t npb, int64_t num_params) {
+    const int64_t j = blockIdx.x;
+    const int64_t block = num_params > 1 ? npb / num_params : npb;   // rows per batch for this parameter
+    const int64_t batches = M / npb;
+    const int64_t total = batches * block;
+    double s = 0.0;
+    for (int64_t i = threadIdx.x; i < total; i += blockDim.x) {
+        const int64_t n = i / block, b = i % block;
+        s += (double)partial[n * npb + j * block + b];
+    }
+    __shared__ double red[256];
+    red[threadIdx.x] = s;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) grad[j] = (float)red[0];
+}
+
+__global__ void zero_fill(float* p, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        p[i] = 0.0f;
+}
+
+// Clears n floats with a kernel (a memset node would not replay reliably inside a captured graph).
+int launch_zero_fill(float* p, int64_t n, hipStream_t stream) {
+    if (n <= 0) return 0;
+    hipLaunchKernelGGL(zero_fill, dim3(1), dim3(256), 0, stream, p, n);
+    return (int)hipGetLastError();
+}
+
+int launch_reduce_param_grad(float* grad, const float* partial, int64_t M, int64_t npb,
+                             int64_t num_params, hipStream_t stream) {
+    hipLaunchKernelGGL(reduce_param_grad, dim3((unsigned)num_params), dim3(256), 0, stream,
+                       grad, partial, M, npb, num_params);
+    return (int)hipGetLastError();
+}
+
+}  // namespace slayer
+
+using namespace slayer;
+
+extern "C" int slayer_li_fwd(float* out, const float* in, const float* decay, const float* state,
+                             double thr_scaled, int w_scale,
+                             int64_t M, int64_t neurons_per_batch, int64_t num_decays, int64_t num_states,
+                             int64_t T, void* stream) {
+    if (int e = check_rows(M, T)) return e;
+    if (M == 0 || T == 0) return 0;
+    if (!out || !in || !decay || !state) return SLAYER_ENULL;
+    if (int e = check_params(M, neurons_per_batch, num_decays)) return e;
+    if (int e = check_states(M, num_states)) return e;
+    if (w_scale == 0) return SLAYER_EINVAL;
+    const float w = (float)w_scale;
+    const float thr = thr_scaled > 0 ? (float)thr_scaled : __builtin_inff();
+    if (is_pow2(w_scale)) {
+        LiFwd<true>::Params p{{in}, {out}, decay, state, w, 1.0f / w, thr, neurons_per_batch, num_decays, num_states};
+        return launch_stream<LiFwd<true>, 64>(p, M, T, (hipStream_t)stream);
+    }
+    LiFwd<false>::Params p{{in}, {out}, decay, state, w, 1.0f / w, thr, neurons_per_batch, num_decays, num_states};
+    return launch_stream<LiFwd<false>, 64>(p, M, T, (hipStream_t)stream);
+}
+
+extern "C" int slayer_li_bwd(float* grad_in, float* grad_decay, const float* grad_out, const float* out,
+                             const float* decay, float* workspace,
+                             int64_t M, int64_t neurons_per_batch, int64_t num_decays,
+                             int64_t T, void* stream) {
+    if (int e = check_rows(M, T)) return e;
+    if (int e = check_params(M > 0 ? M : neurons_per_batch, neurons_per_batch, num_decays)) return e;
+    if (grad_decay && !workspace && M > 0) return SLAYER_ENULL;
+    if (M > 0 && T > 0) {
+        if (!grad_in || !grad_out || !out || !decay) return SLAYER_ENULL;
+        LiBwd::Params p{{grad_out, out}, {grad_in}, decay, grad_decay ? workspace : nullptr,
+                        neurons_per_batch, num_decays};
+        if (int e = launch_stream<LiBwd, 32>(p, M, T, (hipStream_t)stream)) return e;
+    }
+    if (grad_decay) {
+        if (M == 0 || T == 0) return launch_zero_fill(grad_decay, num_decays, (hipStream_t)stream);
+        return launch_reduce_param_grad(grad_decay, workspace, M, neurons_per_batch, num_decays, (hipStream_t)stream);
+    }
+    return 0;
+}

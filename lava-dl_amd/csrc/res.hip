@@ -1,0 +1,162 @@
+// Resonator: complex rotating-decay fixed-point recurrence and its reverse-time gradient.
+#include "common.h"
+#include "tile.h"
+
+namespace slayer {
+
+int launch_reduce_param_grad(float* grad, const float* partial, int64_t M, int64_t npb,
+                             int64_t num_params, hipStream_t stream);   // li.hip
+int launch_zero_fill(float* p, int64_t n, hipStream_t stream);          // li.hip
+
+template <bool POW2, bool HAS_THR>
+struct ResFwd {
+    static constexpr int kIn = 2, kOut = 2;
+    static constexpr bool kReverse = false;
+    struct Params {
+        const float* in[2];
+        float* out[2];
+        const float *sin_decay, *cos_decay, *re_state, *im_state;
+        float w, inv_w, thr;
+        int im_reset;
+        int64_t npb, num_decays, n_rs, n_is;
+    };
+    int re, im, s, c, im_reset;
+    float w, inv_w, thr;
+
+    __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
+        w = p.w; inv_w = p.inv_w; thr = p.thr; im_reset = p.im_reset;
+        re = im = s = c = 0;
+        if (valid) {
+            re = trunc_i32(p.re_state[p.n_rs == 1 ? 0 : m] * w);
+            im = trunc_i32(p.im_state[p.n_is == 1 ? 0 : m] * w);
+            const int64_t j = param_index(m, p.npb, p.num_decays);
+            s = trunc_i32(p.sin_decay[j]);
+            c = trunc_i32(p.cos_decay[j]);
+        }
+    }
+    __device__ __forceinline__ void step(const float (&x)[2], float (&o)[2]) {
+        const int re_n = rs0_12(c, re) - rs0_12(s, im) + trunc_i32(w * x[0]);
+        const int im_n = rs0_12(s, re) + rs0_12(c, im) + trunc_i32(w * x[1]);
+        const float ref = (float)re_n, imf = (float)im_n;
+        o[0] = POW2 ? ref * inv_w : ref / w;
+        o[1] = POW2 ? imf * inv_w : imf / w;
+        if (HAS_THR) {
+            // the kept imaginary state makes a float32 round trip, as the mixed int/float
+            // expression of the CPU branch does
+            const bool fired = imf >= thr;
+            re = fired ? 0 : re_n;
+            im = fired ? im_reset : trunc_i32(imf);
+        } else {
+            re = re_n;
+            im = im_n;
+        }
+    }
+    __device__ __forceinline__ void finish(const Params&, int64_t, bool) {}
+};
+
+struct ResBwd {
+    static constexpr int kIn = 4, kOut = 2;      // in: g_re, g_im, saved re, saved im
+    static constexpr bool kReverse = true;
+    struct Params {
+        const float* in[4];
+        float* out[2];
+        const float *sin_decay, *cos_decay;
+        float *partial_sin, *partial_cos;        // per-neuron sums, or nullptr
+        int64_t npb, num_decays;
+    };
+    float c, s, gr, gi, acc_s, acc_c;
+
+    __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
+        c = s = gr = gi = acc_s = acc_c = 0.f;
+        if (valid) {
+            const int64_t j = param_index(m, p.npb, p.num_decays);
+            c = p.cos_decay[j] / 4096.0f;
+            s = p.sin_decay[j] / 4096.0f;
+        }
+    }
+    __device__ __forceinline__ void step(const float (&x)[4], float (&o)[2]) {
+        // gr, gi still hold the gradients of step t+1; x[2], x[3] are re[t], im[t]
+        acc_s = __fmaf_rn(gi, x[2], __fmaf_rn(-gr, x[3], acc_s));
+        acc_c = __fmaf_rn(gi, x[3], __fmaf_rn(gr, x[2], acc_c));
+        const float ngr = (c * gr + s * gi) + x[0];
+        const float ngi = ((-s) * gr + c * gi) + x[1];
+        gr = ngr; gi = ngi;
+        o[0] = ngr; o[1] = ngi;
+    }
+    __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
+        if (valid && p.partial_sin) { p.partial_sin[m] = acc_s; p.partial_cos[m] = acc_c; }
+    }
+};
+
+}  // namespace slayer
+
+using namespace slayer;
+
+template <bool POW2, bool HAS_THR>
+static int res_fwd_launch(float* re_out, float* im_out, const float* re_in, const float* im_in,
+                          const float* sin_decay, const float* cos_decay, const float* re_state,
+                          const float* im_state, float thr, int im_reset, float w,
+                          int64_t M, int64_t npb, int64_t nd, int64_t n_rs, int64_t n_is, int64_t T,
+                          hipStream_t stream) {
+    using Op = ResFwd<POW2, HAS_THR>;
+    typename Op::Params p{{re_in, im_in}, {re_out, im_out}, sin_decay, cos_decay, re_state, im_state,
+                          w, 1.0f / w, thr, im_reset, npb, nd, n_rs, n_is};
+    return launch_stream<Op, 32>(p, M, T, stream);
+}
+
+extern "C" int slayer_res_fwd(float* re_out, float* im_out, const float* re_in, const float* im_in,
+                              const float* sin_decay, const float* cos_decay,
+                              const float* re_state, const float* im_state,
+                              double thr_scaled, int w_scale,
+                              int64_t M, int64_t neurons_per_batch, int64_t num_decays,
+                              int64_t num_re_states, int64_t num_im_states,
+                              int64_t T, void* stream) {
+    if (int e = check_rows(M, T)) return e;
+    if (M == 0 || T == 0) return 0;
+    if (!re_out || !im_out || !re_in || !im_in || !sin_decay || !cos_decay || !re_state || !im_state)
+        return SLAYER_ENULL;
+    if (int e = check_params(M, neurons_per_batch, num_decays)) return e;
+    if (int e = check_states(M, num_re_states)) return e;
+    if (int e = check_states(M, num_im_states)) return e;
+    if (w_scale == 0) return SLAYER_EINVAL;
+    const float w = (float)w_scale;
+    const bool has_thr = thr_scaled >= 0;
+    const float thr = (float)thr_scaled;
+    const int im_reset = has_thr ? (int)(float)(thr_scaled - 1.0) : 0;
+    hipStream_t st = (hipStream_t)stream;
+#define SLAYER_RES_ARGS re_out, im_out, re_in, im_in, sin_decay, cos_decay, re_state, im_state, thr, im_reset, w, \
+                        M, neurons_per_batch, num_decays, num_re_states, num_im_states, T, st
+    if (is_pow2(w_scale))
+        return has_thr ? res_fwd_launch<true, true>(SLAYER_RES_ARGS) : res_fwd_launch<true, false>(SLAYER_RES_ARGS);
+    return has_thr ? res_fwd_launch<false, true>(SLAYER_RES_ARGS) : res_fwd_launch<false, false>(SLAYER_RES_ARGS);
+#undef SLAYER_RES_ARGS
+}
+
+extern "C" int slayer_res_bwd(float* g_re_in, float* g_im_in, float* grad_sin, float* grad_cos,
+                              const float* g_re, const float* g_im, const float* re, const float* im,
+                              const float* sin_decay, const float* cos_decay, float* workspace,
+                              int64_t M, int64_t neurons_per_batch, int64_t num_decays,
+                              int64_t T, void* stream) {
+    if (int e = check_rows(M, T)) return e;
+    if (int e = check_params(M > 0 ? M : neurons_per_batch, neurons_per_batch, num_decays)) return e;
+    if ((grad_sin == nullptr) != (grad_cos == nullptr)) return SLAYER_ENULL;
+    const bool want = grad_sin != nullptr;
+    if (want && !workspace && M > 0) return SLAYER_ENULL;
+    hipStream_t st = (hipStream_t)stream;
+    if (M > 0 && T > 0) {
+        if (!g_re_in || !g_im_in || !g_re || !g_im || !re || !im || !sin_decay || !cos_decay) return SLAYER_ENULL;
+        ResBwd::Params p{{g_re, g_im, re, im}, {g_re_in, g_im_in}, sin_decay, cos_decay,
+                         want ? workspace : nullptr, want ? workspace + M : nullptr,
+                         neurons_per_batch, num_decays};
+        if (int e = launch_stream<ResBwd, 32>(p, M, T, st)) return e;
+    }
+    if (want) {
+        if (M == 0 || T == 0) {
+            if (int e = launch_zero_fill(grad_sin, num_decays, st)) return e;
+            return launch_zero_fill(grad_cos, num_decays, st);
+        }
+        if (int e = launch_reduce_param_grad(grad_sin, workspace, M, neurons_per_batch, num_decays, st)) return e;
+        return launch_reduce_param_grad(grad_cos, workspace + M, M, neurons_per_batch, num_decays, st);
+    }
+    return 0;
+}

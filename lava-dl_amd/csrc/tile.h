@@ -1,0 +1,193 @@
+// Neuron x time-chunk streaming engine shared by every sequential-in-time kernel.
+//
+// Tensors are [M][T] float32 with time innermost.  One 64-lane wavefront (one
+// workgroup) owns 64 consecutive neurons (rows) and walks the time axis in chunks
+// of TC steps:
+//
+//   global --dwordx4, coalesced along time--> registers --ds_write_b128--> LDS tile
+//   LDS tile: lane j runs the recurrence over row j, 4 steps per ds_read_b128,
+//             results overwrite the tile in place (ds_write_b128)
+//   LDS tile --ds_read_b128--> registers --dwordx4, coalesced--> global
+//
+// The loads for chunk k+1 are issued before chunk k is computed, so HBM latency
+// hides behind the sequential arithmetic.  Rows are padded by 4 floats (16 B):
+// with a pitch of TC+4 floats both access patterns (lane = (row, quad) for the
+// copies; lane = row for the recurrence) touch 8 distinct 16-byte bank groups
+// per 8 consecutive lanes, i.e. they run at the conflict-free b128 rate.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace slayer {
+
+constexpr int kWave = 64;
+
+// (a * b) >> 12 rounded toward zero.  The 64-bit product is biased by 4095 when it is
+// negative; its sign is the sign bit of a ^ b whenever the product is non-zero, and a
+// zero product gives 0 with either bias, so no second multiply is needed for the sign.
+__device__ __forceinline__ int rs0_12(int a, int b) {
+    const long long bias = (long long)(((a ^ b) >> 31) & 4095);
+    return (int)(((long long)a * (long long)b + bias) >> 12);
+}
+
+// float32 -> int32 toward zero; out-of-range values saturate (v_cvt_i32_f32).
+__device__ __forceinline__ int trunc_i32(float x) { return (int)x; }
+
+__device__ __forceinline__ int64_t param_index(int64_t m, int64_t npb, int64_t num_params) {
+    return num_params > 1 ? (m % npb) / (npb / num_params) : 0;
+}
+
+template <int TC>
+struct TileGeom {
+    static_assert(TC % 4 == 0 && TC >= 4 && TC <= 256 && (kWave * 4) % TC == 0, "bad chunk");
+    static constexpr int kPitch = TC + 4;               // floats per LDS row
+    static constexpr int kQuads = TC / 4;               // float4 per row
+    static constexpr int kRowsPerPass = kWave / kQuads; // rows one wave-wide access covers
+    static constexpr int kPasses = kWave / kRowsPerPass;
+    static constexpr int kTileFloats = kWave * kPitch;
+};
+
+// An Op provides:
+//   static constexpr int kIn, kOut;  static constexpr bool kReverse;
+//   struct Params { const float* in[kIn]; float* out[kOut]; ... };
+//   __device__ void init(const Params&, int64_t m, bool valid);
+//   __device__ void step(const float (&x)[kIn], float (&y)[kOut]);
+//   __device__ void finish(const Params&, int64_t m, bool valid);
+template <class Op, int TC, bool VEC4>
+__global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, int64_t M, int T) {
+    using G = TileGeom<TC>;
+    constexpr int NI = Op::kIn, NO = Op::kOut, NT = NI > NO ? NI : NO;
+    __shared__ __attribute__((aligned(16))) float tile[NT][G::kTileFloats];
+
+    const int lane = threadIdx.x;
+    const int64_t m0 = (int64_t)blockIdx.x * kWave;
+    const int rows = (int)((M - m0) < kWave ? (M - m0) : kWave);
+
+    Op op;
+    op.init(prm, m0 + lane, lane < rows);
+
+    const int nchunks = (T + TC - 1) / TC;
+    const int crow = lane / G::kQuads;      // row within a pass (copy pattern)
+    const int cq = lane % G::kQuads;        // quad within the row
+
+    float4 stage[NI][G::kPasses];
+
+    auto fetch = [&](int chunk) {
+        const int t = chunk * TC + 4 * cq;
+#pragma unroll
+        for (int p = 0; p < G::kPasses; ++p) {
+            const int r = p * G::kRowsPerPass + crow;
+            const size_t off = (size_t)(m0 + r) * (size_t)T + (size_t)t;
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (r < rows) {
+                    const float* src = prm.in[i] + off;
+                    if (VEC4) {
+                        if (t < T) v = *reinterpret_cast<const float4*>(src);
+                    } else {
+                        if (t + 0 < T) v.x = src[0];
+                        if (t + 1 < T) v.y = src[1];
+                        if (t + 2 < T) v.z = src[2];
+                        if (t + 3 < T) v.w = src[3];
+                    }
+                }
+                stage[i][p] = v;
+            }
+        }
+    };
+
+    fetch(Op::kReverse ? nchunks - 1 : 0);
+
+    for (int k = 0; k < nchunks; ++k) {
+        const int chunk = Op::kReverse ? nchunks - 1 - k : k;
+        const int t0 = chunk * TC;
+        const int len = (T - t0) < TC ? (T - t0) : TC;
+
+        // staged registers -> LDS
+#pragma unroll
+        for (int p = 0; p < G::kPasses; ++p) {
+            const int r = p * G::kRowsPerPass + crow;
+#pragma unroll
+            for (int i = 0; i < NI; ++i)
+                *reinterpret_cast<float4*>(&tile[i][r * G::kPitch + 4 * cq]) = stage[i][p];
+        }
+        __syncthreads();
+
+        if (k + 1 < nchunks) fetch(Op::kReverse ? chunk - 1 : chunk + 1);
+
+        // sequential recurrence: lane = neuron
+        const int nq = (len + 3) >> 2;
+#pragma unroll 2
+        for (int q = 0; q < nq; ++q) {
+            const int qq = Op::kReverse ? nq - 1 - q : q;
+            float xin[NI][4], yout[NO][4];
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                const float4 v = *reinterpret_cast<const float4*>(&tile[i][lane * G::kPitch + 4 * qq]);
+                xin[i][0] = v.x; xin[i][1] = v.y; xin[i][2] = v.z; xin[i][3] = v.w;
+            }
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const int ss = Op::kReverse ? 3 - s : s;
+                float x[NI], y[NO];
+#pragma unroll
+                for (int i = 0; i < NI; ++i) x[i] = xin[i][ss];
+                op.step(x, y);
+#pragma unroll
+                for (int o = 0; o < NO; ++o) yout[o][ss] = y[o];
+            }
+#pragma unroll
+            for (int o = 0; o < NO; ++o)
+                *reinterpret_cast<float4*>(&tile[o][lane * G::kPitch + 4 * qq]) =
+                    make_float4(yout[o][0], yout[o][1], yout[o][2], yout[o][3]);
+        }
+        __syncthreads();
+
+        // LDS -> global
+        {
+            const int t = t0 + 4 * cq;
+#pragma unroll
+            for (int p = 0; p < G::kPasses; ++p) {
+                const int r = p * G::kRowsPerPass + crow;
+                const size_t off = (size_t)(m0 + r) * (size_t)T + (size_t)t;
+#pragma unroll
+                for (int o = 0; o < NO; ++o) {
+                    const float4 v = *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]);
+                    if (r < rows) {
+                        float* dst = prm.out[o] + off;
+                        if (VEC4) {
+                            if (t < T) *reinterpret_cast<float4*>(dst) = v;
+                        } else {
+                            if (t + 0 < T) dst[0] = v.x;
+                            if (t + 1 < T) dst[1] = v.y;
+                            if (t + 2 < T) dst[2] = v.z;
+                            if (t + 3 < T) dst[3] = v.w;
+                        }
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    op.finish(prm, m0 + lane, lane < rows);
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Launch helper: picks the dwordx4 path when T and every pointer allow it.
+template <class Op, int TC>
+int launch_stream(const typename Op::Params& prm, int64_t M, int64_t T, hipStream_t stream) {
+    if (M == 0 || T == 0) return 0;
+    bool vec = (T % 4) == 0;
+    for (int i = 0; i < Op::kIn; ++i) vec = vec && aligned16(prm.in[i]);
+    for (int o = 0; o < Op::kOut; ++o) vec = vec && aligned16(prm.out[o]);
+    const dim3 grid((unsigned)((M + kWave - 1) / kWave)), block(kWave);
+    if (vec)
+        hipLaunchKernelGGL((stream_kernel<Op, TC, true>), grid, block, 0, stream, prm, M, (int)T);
+    else
+        hipLaunchKernelGGL((stream_kernel<Op, TC, false>), grid, block, 0, stream, prm, M, (int)T);
+    return (int)hipGetLastError();
+}
+
+}  // namespace slayer

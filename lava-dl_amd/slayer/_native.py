@@ -1,0 +1,109 @@
+"""ctypes binding of libslayer_hip.so (C ABI declared in include/slayer_hip.h).
+
+The shared library is the only implementation: there is no CPU or eager
+fallback.  Loading fails loudly when the library has not been built, and every
+operator raises when handed a tensor that is not float32 on a GPU.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, 'libslayer_hip.so')
+ABI_VERSION = 1
+
+_lib = None
+
+_P = ctypes.c_void_p
+_I64 = ctypes.c_int64
+_INT = ctypes.c_int
+_F = ctypes.c_float
+_D = ctypes.c_double
+
+_SIGNATURES = {
+    'slayer_abi_version': (_INT, []),
+    'slayer_error_string': (ctypes.c_char_p, [_INT]),
+    'slayer_li_fwd': (_INT, [_P, _P, _P, _P, _D, _INT, _I64, _I64, _I64, _I64, _I64, _P]),
+    'slayer_li_bwd': (_INT, [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _P]),
+    'slayer_ath_fwd': (_INT, [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _INT,
+                              _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P]),
+    'slayer_res_fwd': (_INT, [_P, _P, _P, _P, _P, _P, _P, _P, _D, _INT,
+                              _I64, _I64, _I64, _I64, _I64, _I64, _P]),
+    'slayer_res_bwd': (_INT, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _P]),
+    'slayer_spike_fwd': (_INT, [_P, _P, _P, _I64, _INT, _F, _I64, _P]),
+    'slayer_spike_bwd': (_INT, [_P, _P, _P, _P, _I64, _F, _F, _INT, _I64, _P]),
+    'slayer_cspike_fwd': (_INT, [_P, _P, _P, _P, _I64, _P, _I64, _INT, _F, _I64, _I64, _P]),
+    'slayer_cspike_bwd': (_INT, [_P, _P, _P, _P, _P, _P, _I64, _F, _F, _INT, _I64, _P]),
+    'slayer_shift': (_INT, [_P, _P, _P, _I64, _F, _I64, _I64, _I64, _P]),
+    'slayer_conv': (_INT, [_P, _P, _P, _I64, _F, _I64, _I64, _P]),
+    'slayer_corr': (_INT, [_P, _P, _P, _I64, _F, _I64, _I64, _P]),
+}
+
+EXPORTS = tuple(_SIGNATURES)
+
+
+def lib():
+    """The loaded library (torch is imported first so that its HIP runtime,
+    which has the same soname as the one the library was linked against, is the
+    single runtime in the process)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f'{LIB_PATH} is missing: build it with `make -C lava-dl_amd/csrc` '
+                '(hipcc, gfx950). There is no fallback implementation.')
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        if handle.slayer_abi_version() != ABI_VERSION:
+            raise RuntimeError('libslayer_hip.so ABI version mismatch; rebuild the library')
+        _lib = handle
+    return _lib
+
+
+def check(code):
+    if code != 0:
+        msg = lib().slayer_error_string(code).decode()
+        raise RuntimeError(f'libslayer_hip call failed ({code}): {msg}')
+
+
+def require_gpu(*tensors):
+    """Same conditions the reference kernels assert (CHECK_INPUT / CHECK_DEVICE,
+    neuron/dynamics/leaky_integrator.cu:14-17,120-124), raised as RuntimeError."""
+    dev = None
+    for t in tensors:
+        if not torch.is_tensor(t):
+            raise RuntimeError(f'expected a tensor, got {type(t)}')
+        if not t.is_cuda:
+            raise RuntimeError('slayer HIP kernels need tensors on an MI355X device; '
+                               'there is no CPU implementation in this package')
+        if t.dtype != torch.float32:
+            raise RuntimeError(f'slayer HIP kernels are float32 only, got {t.dtype}')
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError(f'tensors on different devices: {dev} and {t.device}')
+    return dev
+
+
+def ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def stream_handle():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def rows_and_steps(t):
+    T = t.shape[-1]
+    return (t.numel() // T if T > 0 else 0), T
+
+
+def neurons_per_batch(t):
+    n = 1
+    for s in t.shape[1:-1]:
+        n *= s
+    return n

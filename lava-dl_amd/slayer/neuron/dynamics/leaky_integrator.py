@@ -1,0 +1,93 @@
+"""Leaky integrator dynamics on the GPU.
+
+Interface of lava.lib.dl.slayer.neuron.dynamics.leaky_integrator
+(neuron/dynamics/leaky_integrator.py:50-119 in the reference); the body is
+slayer_li_fwd / slayer_li_bwd of libslayer_hip.so.
+"""
+import torch
+
+from ... import _native as N
+
+
+def dynamics(input, decay, state, w_scale, threshold=None, debug=False):
+    """y[t] = (1 - decay/4096) y[t-1] + x[t] in 12-bit fixed point, with an
+    optional spike-and-reset at ``threshold``.
+
+    Parameters
+    ----------
+    input : torch.Tensor
+        float32 GPU tensor [N, C, ..., T].
+    decay : torch.Tensor
+        unscaled integer decay(s): one value (shared), C values (per channel)
+        or one per neuron of a batch element.
+    state : torch.Tensor
+        initial state, one element or shaped like ``input.shape[:-1]``.
+    w_scale : int
+        scale of the integer state.
+    threshold : float or None
+        ``None`` disables the reset.
+    debug : bool
+        accepted for interface compatibility; the reference uses it to compare
+        its two implementations, here there is only one.
+
+    Returns
+    -------
+    torch.Tensor, same shape as ``input``.
+    """
+    if threshold is None:
+        threshold = -1
+    return _LIDynamics.apply(input, decay, state, threshold, w_scale)
+
+
+def persistent_state(state, spike):
+    """State to carry to the next call when the last step spiked (reset to 0)."""
+    spike = (spike > 0).to(state.dtype)
+    return state * (1 - spike)
+
+
+def _fwd(input, decay, state, threshold, w_scale):
+    dev = N.require_gpu(input, decay, state)
+    input, decay, state = input.contiguous(), decay.contiguous(), state.contiguous()
+    M, T = N.rows_and_steps(input)
+    if state.numel() not in (1, M):
+        raise RuntimeError(f'state has {state.numel()} elements, expected 1 or {M}')
+    output = torch.empty_like(input)
+    with torch.cuda.device(dev):
+        N.check(N.lib().slayer_li_fwd(
+            N.ptr(output), N.ptr(input), N.ptr(decay), N.ptr(state),
+            float(threshold * w_scale), int(w_scale),
+            M, N.neurons_per_batch(input), decay.numel(), state.numel(), T, N.stream_handle()))
+    return output
+
+
+def _bwd(grad_output, output, decay, need_decay_grad=True):
+    dev = N.require_gpu(grad_output, output, decay)
+    grad_output, output, decay = grad_output.contiguous(), output.contiguous(), decay.contiguous()
+    M, T = N.rows_and_steps(grad_output)
+    grad_input = torch.empty_like(grad_output)
+    grad_decay = workspace = None
+    if need_decay_grad:
+        grad_decay = torch.empty(decay.numel(), dtype=torch.float32, device=dev)
+        workspace = torch.empty(max(M, 1), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        N.check(N.lib().slayer_li_bwd(
+            N.ptr(grad_input), N.ptr(grad_decay), N.ptr(grad_output), N.ptr(output), N.ptr(decay),
+            N.ptr(workspace), M, N.neurons_per_batch(grad_output), decay.numel(), T, N.stream_handle()))
+    return grad_input, grad_decay
+
+
+class _LIDynamics(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input, decay, state, threshold, w_scale):
+        output = _fwd(input, decay.detach(), state.detach(), threshold, w_scale)
+        ctx.save_for_backward(output, decay)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        output, decay = ctx.saved_tensors
+        need = ctx.needs_input_grad[1]
+        grad_input, grad_decay = _bwd(grad_output, output, decay.detach(), need)
+        if grad_decay is not None:
+            grad_decay = grad_decay.reshape(decay.shape)
+        return grad_input, grad_decay, None, None, None

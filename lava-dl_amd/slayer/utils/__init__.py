@@ -1,0 +1,4 @@
+from . import time, filter, int_utils
+from .int_utils import right_shift_to_zero
+
+__all__ = ['time', 'filter', 'int_utils', 'right_shift_to_zero']

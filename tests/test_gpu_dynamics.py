@@ -1,0 +1,276 @@
+"""GPU parity of the fixed-point dynamics kernels against the CPU oracle, through the
+python operator interface (ctypes -> C ABI -> HIP kernels).  Integer-mode outputs must
+be bit-exact; float-mode gradients within 1e-5 relative."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import slayer_oracle as O
+from tests.golden import fixtures as G
+from tests.util import seed_of, dev, sparse_input, assert_exact, assert_rel
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope='module')
+def slayer():
+    import lava_dl_amd.slayer as s
+    return s
+
+
+def _decay(kind, shape, gen):
+    C = shape[1]
+    spatial = shape[1:-1]
+    if kind == 'shared':
+        return torch.tensor([float(torch.randint(0, 4097, (1,), generator=gen))])
+    if kind == 'channel':
+        return torch.randint(0, 4097, (C,), generator=gen).float()
+    return torch.randint(0, 4097, tuple(spatial), generator=gen).float()
+
+
+LI_CASES = [
+    # shape,               decay kind, w,    threshold,          state
+    ((4, 128, 200),        'shared',   64,   1.25,               'scalar'),
+    ((4, 128, 200),        'channel',  64,   None,               'full'),
+    ((2, 16, 8, 8, 300),   'channel',  64,   1.0,                'scalar'),
+    ((2, 3, 5, 7, 37),     'channel',  4096, 1.0 + 0.01 / 4096,  'full'),     # T % 4 != 0, M % 64 != 0
+    ((3, 70, 129),         'neuron',   100,  0.77,               'full'),     # w not a power of two
+    ((1, 5, 3),            'neuron',   64,   None,               'scalar'),   # T < 4
+    ((2, 64, 1),           'channel',  64,   0.5,                'full'),     # T == 1
+    ((1, 1, 260),          'shared',   4096, 2.0,                'scalar'),   # one neuron
+    ((2, 130, 64),         'channel',  64,   0.0,                'scalar'),   # threshold 0 = disabled
+]
+
+
+@pytest.mark.parametrize('shape,kind,w,thr,state_kind', LI_CASES)
+def test_li_fwd_bit_exact(slayer, shape, kind, w, thr, state_kind):
+    gen = torch.Generator().manual_seed(seed_of(shape, kind, w))
+    x = sparse_input(gen, shape, p=0.1, amp=2.0)
+    decay = _decay(kind, shape, gen)
+    state = torch.tensor([0.0]) if state_kind == 'scalar' else torch.randn(shape[:-1], generator=gen)
+    ref = O.li_fwd(x, decay, state, w, thr)
+    out = slayer.neuron.dynamics.leaky_integrator.dynamics(
+        x.to(dev()), decay.to(dev()), state.to(dev()), w, thr)
+    assert_exact(out, ref, f'li_fwd {shape}')
+
+
+def test_li_fwd_negative_and_edge_decays(slayer):
+    gen = torch.Generator().manual_seed(7)
+    x = sparse_input(gen, (2, 8, 96), p=0.5, amp=30.0)
+    decay = torch.tensor([0.0, 1.0, 2047.0, 4095.0, 4096.0, 1234.7, 5000.0, -17.0])
+    state = torch.randn(2, 8, generator=gen) * 50
+    for thr in (None, 3.0):
+        ref = O.li_fwd(x, decay, state, 64, thr)
+        out = slayer.neuron.dynamics.leaky_integrator.dynamics(x.to(dev()), decay.to(dev()), state.to(dev()), 64, thr)
+        assert_exact(out, ref, f'li_fwd edge decays thr={thr}')
+
+
+def test_li_fwd_non_contiguous_and_offset_views(slayer):
+    gen = torch.Generator().manual_seed(8)
+    base = sparse_input(gen, (3, 40, 101), p=0.2)
+    decay = torch.tensor([300.0])
+    zero = torch.tensor([0.0])
+    xg = base.to(dev())
+    # a view that starts 4 bytes into the allocation and has T % 4 != 0
+    v_cpu, v_gpu = base[:, :, 1:], xg[:, :, 1:]
+    assert_exact(slayer.neuron.dynamics.leaky_integrator.dynamics(v_gpu, decay.to(dev()), zero.to(dev()), 64, 1.0),
+                 O.li_fwd(v_cpu.contiguous(), decay, zero, 64, 1.0), 'li_fwd strided view')
+    # contiguous but misaligned base pointer with T % 4 == 0
+    flat = torch.zeros(2 * 64 * 100 + 1)
+    flat[1:] = sparse_input(gen, (2 * 64 * 100,), p=0.2)
+    fg = flat.to(dev())
+    v_cpu, v_gpu = flat[1:].reshape(2, 64, 100), fg[1:].reshape(2, 64, 100)
+    assert v_gpu.data_ptr() % 16 != 0
+    assert_exact(slayer.neuron.dynamics.leaky_integrator.dynamics(v_gpu, decay.to(dev()), zero.to(dev()), 64, 1.0),
+                 O.li_fwd(v_cpu, decay, zero, 64, 1.0), 'li_fwd misaligned base')
+
+
+def test_li_empty(slayer):
+    z = torch.zeros(0, 4, 10, device=dev())
+    out = slayer.neuron.dynamics.leaky_integrator.dynamics(z, torch.tensor([1.0], device=dev()),
+                                                           torch.tensor([0.0], device=dev()), 64)
+    assert out.shape == z.shape
+
+
+def test_li_rejects_cpu_and_wrong_dtype(slayer):
+    d = torch.tensor([1.0])
+    with pytest.raises(RuntimeError):
+        slayer.neuron.dynamics.leaky_integrator.dynamics(torch.zeros(1, 2, 8), d, d, 64)
+    with pytest.raises(RuntimeError):
+        slayer.neuron.dynamics.leaky_integrator.dynamics(torch.zeros(1, 2, 8, device=dev(), dtype=torch.float64),
+                                                         d.to(dev()), d.to(dev()), 64)
+    with pytest.raises(RuntimeError):   # 3 decays cannot map onto 4 channels
+        slayer.neuron.dynamics.leaky_integrator.dynamics(torch.zeros(1, 4, 8, device=dev()),
+                                                         torch.zeros(3, device=dev()), d.to(dev()), 64)
+
+
+def test_dense_lif_fixture_on_gpu(slayer):
+    """Reference-held known answer (netx gts/dense): CUBA current -> voltage -> spike."""
+    fx = G.dense_lif()
+    li = slayer.neuron.dynamics.leaky_integrator.dynamics
+    zero = torch.tensor([0.0], device=dev())
+    cur = li(fx['x'].to(dev()), torch.tensor([fx['current_decay']], device=dev()), zero, G.W_SCALE)
+    vol = li(cur, torch.tensor([fx['voltage_decay']], device=dev()), zero, G.W_SCALE, fx['threshold'])
+    spk = slayer.spike.Spike.apply(vol, fx['threshold'], 1.0, 1.0, False, 0, 1)
+    got = spk[0].cpu().numpy().astype(np.int64)[:, :fx['expected'].shape[1]]
+    assert int((got != fx['expected']).sum()) == 0
+    assert got.sum() == 1826
+
+
+@pytest.mark.parametrize('shape,kind', [((4, 128, 200), 'shared'), ((2, 16, 8, 8, 300), 'channel'),
+                                        ((3, 70, 129), 'channel'), ((2, 3, 5, 7, 37), 'neuron'),
+                                        ((2, 64, 1), 'channel'), ((1, 5, 3), 'shared')])
+def test_li_bwd(slayer, shape, kind):
+    gen = torch.Generator().manual_seed(seed_of(shape, kind))
+    go = torch.randn(shape, generator=gen)
+    out = torch.randn(shape, generator=gen)
+    decay = _decay(kind, shape, gen)
+    if kind == 'neuron':      # the reference reduces per-neuron decay gradients to [C]; not supported there either
+        ref_g, _ = O.li_bwd(go, out, decay)
+        ref_gd = (ref_g[..., 1:].double() * out[..., :-1].double()).sum(dim=(0, -1)).float()
+    else:
+        ref_g, ref_gd = O.li_bwd(go, out, decay)
+    from lava_dl_amd.slayer.neuron.dynamics import leaky_integrator as L
+    g, gd = L._bwd(go.to(dev()), out.to(dev()), decay.to(dev()))
+    assert_exact(g, ref_g, f'li_bwd grad_input {shape}')      # same op order, no contraction -> identical bits
+    exact = (ref_g[..., 1:].double() * out[..., :-1].double())
+    assert_rel(gd.reshape(ref_gd.shape), ref_gd, f'li_bwd grad_decay {shape}',
+               rel=1e-5 * max(1.0, float(exact.abs().sum() / max(ref_gd.abs().max(), 1e-30)) ** 0.5))
+
+
+def test_li_autograd_matches_oracle(slayer):
+    gen = torch.Generator().manual_seed(11)
+    x = sparse_input(gen, (2, 6, 4, 4, 60), p=0.1)
+    decay = torch.randint(0, 4096, (6,), generator=gen).float()
+    xg = x.to(dev()).requires_grad_()
+    dg = decay.to(dev()).requires_grad_()
+    out = slayer.neuron.dynamics.leaky_integrator.dynamics(xg, dg, torch.tensor([0.0], device=dev()), 64, 1.0)
+    go = torch.randn(x.shape, generator=gen)
+    out.backward(go.to(dev()))
+    ref_out = O.li_fwd(x, decay, torch.tensor([0.0]), 64, 1.0)
+    ref_g, ref_gd = O.li_bwd(go, ref_out, decay)
+    assert_exact(out, ref_out, 'autograd fwd')
+    assert_exact(xg.grad, ref_g, 'autograd grad_input')
+    assert dg.grad.shape == decay.shape
+    assert_rel(dg.grad, ref_gd, 'autograd grad_decay', rel=1e-4)
+
+
+# ------------------------------------------------------------------------------------- ATH
+ATH_CASES = [((4, 128, 200), 'channel', 64), ((2, 3, 5, 7, 37), 'channel', 4096), ((3, 70, 129), 'neuron', 100),
+             ((2, 64, 1), 'shared', 64), ((1, 5, 3), 'shared', 64)]
+
+
+@pytest.mark.parametrize('shape,kind,w', ATH_CASES)
+def test_ath_fwd_bit_exact(slayer, shape, kind, w):
+    gen = torch.Generator().manual_seed(seed_of(shape, kind, w, 'ath'))
+    x = sparse_input(gen, shape, p=0.3, amp=3.0)
+    rd, td = _decay(kind, shape, gen), _decay(kind, shape, gen)
+    th_state = torch.rand(shape[:-1], generator=gen) * 2        # includes th < th0
+    ref_state = torch.randn(shape[:-1], generator=gen)          # includes r < 0
+    ref_th, ref_r = O.ath_fwd(x, ref_state, rd, th_state, td, 0.5, 1.0, w)
+    th, r = slayer.neuron.dynamics.adaptive_threshold.dynamics(
+        x.to(dev()), ref_state.to(dev()), rd.to(dev()), th_state.to(dev()), td.to(dev()), 0.5, 1.0, w)
+    assert_exact(th, ref_th, f'ath threshold {shape}')
+    assert_exact(r, ref_r, f'ath refractory {shape}')
+
+
+def test_ath_scalar_states_and_no_grad(slayer):
+    gen = torch.Generator().manual_seed(21)
+    x = sparse_input(gen, (2, 32, 100), p=0.3, amp=3.0)
+    one, zero = torch.tensor([1.0]), torch.tensor([0.0])
+    rd, td = torch.tensor([300.0]), torch.tensor([100.0])
+    ref_th, ref_r = O.ath_fwd(x, zero, rd, one, td, 0.5, 1.0, 64)
+    xg = x.to(dev()).requires_grad_()
+    th, r = slayer.neuron.dynamics.adaptive_threshold.dynamics(
+        xg, zero.to(dev()), rd.to(dev()), one.to(dev()), td.to(dev()), 0.5, 1.0, 64)
+    assert_exact(th, ref_th, 'ath th')
+    assert_exact(r, ref_r, 'ath ref')
+    (th.sum() + r.sum() + (xg * 2).sum()).backward()
+    assert torch.equal(xg.grad.cpu(), torch.full(x.shape, 2.0))   # nothing flows back through the op
+
+
+# ------------------------------------------------------------------------------------- RES
+RES_CASES = [((4, 128, 200), 'channel', 64, None), ((2, 3, 5, 7, 37), 'channel', 4096, None),
+             ((3, 70, 129), 'neuron', 100, 1.5), ((2, 64, 1), 'shared', 64, 0.0), ((1, 5, 3), 'shared', 64, 2.3),
+             ((2, 40, 64), 'channel', 64, 1.0)]
+
+
+def _rot(kind, shape, gen):
+    n = _decay(kind, shape, gen).numel()
+    vshape = _decay(kind, shape, gen).shape
+    mag = torch.rand(n, generator=gen) * 4095
+    ph = torch.rand(n, generator=gen) * 2 * np.pi
+    return (mag * torch.sin(ph)).round().reshape(vshape), (mag * torch.cos(ph)).round().reshape(vshape)
+
+
+@pytest.mark.parametrize('shape,kind,w,thr', RES_CASES)
+def test_res_fwd_bit_exact(slayer, shape, kind, w, thr):
+    gen = torch.Generator().manual_seed(seed_of(shape, kind, w, 'res'))
+    xr = sparse_input(gen, shape, p=0.2, amp=2.0)
+    xi = sparse_input(gen, shape, p=0.2, amp=2.0)
+    sin, cos = _rot(kind, shape, gen)
+    rs = torch.randn(shape[:-1], generator=gen)
+    is_ = torch.randn(shape[:-1], generator=gen)
+    ref_re, ref_im = O.res_fwd(xr, xi, sin, cos, rs, is_, w, thr)
+    re, im = slayer.neuron.dynamics.resonator.dynamics(
+        xr.to(dev()), xi.to(dev()), sin.to(dev()), cos.to(dev()), rs.to(dev()), is_.to(dev()), w, thr)
+    assert_exact(re, ref_re, f'res real {shape}')
+    assert_exact(im, ref_im, f'res imag {shape}')
+
+
+def test_rf_fixtures_on_gpu(slayer):
+    """Reference-held known answers (netx gts/complex_dense): RF dense block (phase spike, no
+    reset) and RF_IZ input block (threshold mode with reset)."""
+    res = slayer.neuron.dynamics.resonator.dynamics
+    zero = torch.tensor([0.0], device=dev())
+    fx = G.complex_dense_rf()
+    re, im = res(fx['xr'].to(dev()), fx['xi'].to(dev()), torch.tensor([fx['sin_decay']], device=dev()),
+                 torch.tensor([fx['cos_decay']], device=dev()), zero, zero, G.W_SCALE)
+    spk = slayer.spike.complex.Spike.apply(re, im, fx['threshold'], 0.5, 10.0, False, 0, 1)
+    got = spk[0].cpu().numpy().astype(np.int64)[:, :fx['expected'].shape[1]]
+    assert int((got != fx['expected']).sum()) == 0 and got.sum() > 40000
+    fx = G.complex_input_rf_iz()
+    x = fx['x'].to(dev())
+    re, im = res(x, x, torch.tensor([fx['sin_decay']], device=dev()), torch.tensor([fx['cos_decay']], device=dev()),
+                 zero, zero, G.W_SCALE, fx['threshold'])
+    got = (im >= fx['threshold'])[0].cpu().numpy().astype(np.int64)
+    assert int((got != fx['expected']).sum()) == 0 and got.sum() == 13548
+
+
+@pytest.mark.parametrize('shape,kind', [((4, 128, 200), 'channel'), ((2, 3, 5, 7, 37), 'channel'),
+                                        ((3, 70, 129), 'shared'), ((2, 64, 1), 'channel')])
+def test_res_bwd(slayer, shape, kind):
+    gen = torch.Generator().manual_seed(seed_of(shape, kind, 'resb'))
+    f = lambda: torch.randn(shape, generator=gen)
+    g_re, g_im, re, im = f(), f(), f(), f()
+    sin, cos = _rot(kind, shape, gen)
+    ref = O.res_bwd(g_re, g_im, re, im, sin, cos)
+    from lava_dl_amd.slayer.neuron.dynamics import resonator as R
+    got = R._bwd(g_re.to(dev()), g_im.to(dev()), re.to(dev()), im.to(dev()), sin.to(dev()), cos.to(dev()))
+    assert_exact(got[0], ref[0], 'res_bwd grad_real_input')
+    assert_exact(got[1], ref[1], 'res_bwd grad_imag_input')
+    assert_rel(got[2].reshape(ref[2].shape), ref[2], 'res_bwd grad_sin', rel=1e-4)
+    assert_rel(got[3].reshape(ref[3].shape), ref[3], 'res_bwd grad_cos', rel=1e-4)
+
+
+def test_res_autograd_and_nan_guard(slayer):
+    gen = torch.Generator().manual_seed(31)
+    shape = (2, 8, 50)
+    xr = sparse_input(gen, shape, p=0.3).to(dev()).requires_grad_()
+    xi = sparse_input(gen, shape, p=0.3).to(dev()).requires_grad_()
+    sin = torch.full((8,), 2103.0, device=dev(), requires_grad=True)
+    cos = torch.full((8,), 3273.0, device=dev(), requires_grad=True)
+    zero = torch.tensor([0.0], device=dev())
+    re, im = slayer.neuron.dynamics.resonator.dynamics(xr, xi, sin, cos, zero, zero, 64)
+    (re.sum() + 2 * im.sum()).backward()
+    ref = O.res_bwd(torch.ones(shape), 2 * torch.ones(shape), re.detach().cpu(), im.detach().cpu(),
+                    sin.detach().cpu(), cos.detach().cpu())
+    assert_exact(xr.grad, ref[0], 'res autograd grad_real')
+    assert_exact(xi.grad, ref[1], 'res autograd grad_imag')
+    assert_rel(sin.grad, ref[2], 'res autograd grad_sin', rel=1e-4)
+    assert_rel(cos.grad, ref[3], 'res autograd grad_cos', rel=1e-4)
+    re, im = slayer.neuron.dynamics.resonator.dynamics(xr, xi, sin, cos, zero, zero, 64)
+    bad = torch.ones(shape, device=dev())
+    bad[0, 0, 10] = float('nan')
+    with pytest.raises(Exception):
+        torch.autograd.backward([re, im], [bad, torch.ones(shape, device=dev())])

@@ -1,0 +1,133 @@
+"""GPU parity of the spike functions, time shift and temporal filter against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import slayer_oracle as O
+from tests.util import seed_of, dev, sparse_input, assert_exact, assert_rel
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope='module')
+def slayer():
+    import lava_dl_amd.slayer as s
+    return s
+
+
+SHAPES = [(4, 128, 200), (2, 3, 5, 7, 37), (3, 70, 129), (1, 5, 3), (2, 64, 1)]
+
+
+@pytest.mark.parametrize('shape', SHAPES)
+@pytest.mark.parametrize('graded', [False, True])
+@pytest.mark.parametrize('tensor_th', [False, True])
+def test_spike_fwd_bwd(slayer, shape, graded, tensor_th):
+    gen = torch.Generator().manual_seed(seed_of(shape, graded, tensor_th))
+    v = torch.randn(shape, generator=gen) * 2
+    v[..., 0] = 0.7                                            # exact hits of the scalar threshold
+    th = (torch.randn(shape, generator=gen) if tensor_th else 0.7)
+    g = torch.randn(shape, generator=gen)
+    tau, rho, scale = 1.3, 0.9, 4
+    vg = v.to(dev()).requires_grad_()
+    thg = th.to(dev()) if tensor_th else th
+    s = slayer.spike.Spike.apply(vg, thg, tau, rho, graded, 0, scale)
+    assert_exact(s, O.spike_fwd(v, th, graded, scale), f'spike fwd {shape}')
+    s.backward(g.to(dev()))
+    assert_rel(vg.grad, O.spike_bwd(g, v, th, tau, rho, graded), f'spike bwd {shape}')
+
+
+@pytest.mark.parametrize('shape', SHAPES)
+@pytest.mark.parametrize('graded', [False, True])
+def test_cspike_fwd_bwd(slayer, shape, graded):
+    gen = torch.Generator().manual_seed(seed_of(shape, graded, 'c'))
+    re = torch.randn(shape, generator=gen) * 2
+    im = torch.randn(shape, generator=gen) * 2
+    im[..., -1] = 0.0                                          # imag == 0 counts as "not negative"
+    g = torch.randn(shape, generator=gen)
+    last = torch.randn(shape[:-1], generator=gen)
+    th, tau, rho, scale = 0.4, 0.5, 10.0, 8
+    rg, ig = re.to(dev()).requires_grad_(), im.to(dev()).requires_grad_()
+    s = slayer.spike.complex.Spike.apply(rg, ig, th, tau, rho, graded, last.to(dev()), scale)
+    assert_exact(s, O.cspike_fwd(re, im, th, last, graded, scale), f'cspike fwd {shape}')
+    s.backward(g.to(dev()))
+    ref_re, ref_im = O.cspike_bwd(g, re, im, th, tau, rho, graded)
+    assert_rel(rg.grad, ref_re, f'cspike bwd real {shape}')
+    assert_rel(ig.grad, ref_im, f'cspike bwd imag {shape}')
+    # scalar imag_last
+    s0 = slayer.spike.complex.Spike.apply(rg, ig, th, tau, rho, graded, -1.0, scale)
+    assert_exact(s0, O.cspike_fwd(re, im, th, -1.0, graded, scale), 'cspike scalar last')
+
+
+def test_shift_scalar_and_lut(slayer):
+    """The reference's own check (tests/.../utils/time/test_shift.py): +-10 scalar and a per-channel
+    ramp against plain slicing, here on [10, 200, 1000] plus odd shapes."""
+    gen = torch.Generator().manual_seed(50)
+    x = torch.rand((10, 200, 1000), generator=gen)
+    xg = x.to(dev())
+    for k in (10, -10, 0, 4, -8, 999, 1000, -1500, 2.7, -2.7):
+        assert_exact(slayer.utils.time.shift(xg, k), O.shift(x, k), f'shift scalar {k}')
+    assert_exact(slayer.utils.time.shift(xg, torch.tensor(7.0)), O.shift(x, 7), 'shift one-element tensor')
+    assert_exact(slayer.utils.time.shift(xg, 6, 2), O.shift(x, 3), 'shift sampling time')
+    lut = torch.arange(200, dtype=torch.float32) - 100
+    assert_exact(slayer.utils.time.shift(xg, lut.to(dev())), O.shift(x, lut), 'shift per-channel ramp')
+    lut = torch.rand(200, generator=gen) * 64 - 32          # fractional values are truncated toward zero
+    assert_exact(slayer.utils.time.shift(xg, lut.to(dev())), O.shift(x, lut), 'shift fractional lut')
+    for shape in [(2, 3, 5, 7, 37), (3, 70, 129), (1, 5, 3), (2, 64, 1)]:
+        x = torch.rand(shape, generator=gen)
+        lut = torch.randint(-5, 6, shape[1:-1], generator=gen).float()
+        assert_exact(slayer.utils.time.shift(x.to(dev()), lut.to(dev())), O.shift(x, lut), f'shift lut {shape}')
+        assert_exact(slayer.utils.time.shift(x.to(dev()), 2), O.shift(x, 2), f'shift scalar {shape}')
+    with pytest.raises(Exception):
+        slayer.utils.time.shift(xg, torch.zeros(7, device=dev()))
+    with pytest.raises(AssertionError):
+        slayer.utils.time.shift(torch.zeros(5, device=dev()), 1)
+
+
+@pytest.mark.parametrize('shape,K', [((200, 1000), 50), ((4, 32, 300), 64), ((2, 3, 5, 37), 7), ((3, 1500), 1),
+                                     ((2, 5, 20), 64), ((1000,), 50)])
+def test_conv_corr(slayer, shape, K):
+    """The reference's own check (tests/.../utils/filter/test_conv_filter.py) uses [200, 1000], K=50."""
+    gen = torch.Generator().manual_seed(seed_of(shape, K))
+    x = torch.rand(shape, generator=gen)
+    f = torch.rand(K, generator=gen)
+    x2 = x.reshape(1, -1) if x.dim() == 1 else x
+    for ts in (1, 0.5):
+        assert_rel(slayer.utils.filter.conv(x.to(dev()), f.to(dev()), ts), O.conv_fwd(x2, f, ts), f'conv {shape}')
+        assert_rel(slayer.utils.filter.corr(x.to(dev()), f.to(dev()), ts), O.conv_bwd(x2, f, ts), f'corr {shape}')
+    # float64 numpy.convolve on one row
+    row = x2.reshape(-1, x2.shape[-1])[0].double().numpy()
+    y = slayer.utils.filter.conv(x.to(dev()), f.to(dev())).reshape(-1, x2.shape[-1])[0].cpu().double().numpy()
+    assert np.allclose(y, np.convolve(row, f.double().numpy())[:row.size], rtol=1e-5, atol=1e-5)
+
+
+def test_conv_autograd_is_corr(slayer):
+    gen = torch.Generator().manual_seed(61)
+    x = torch.rand((3, 6, 90), generator=gen)
+    f = torch.rand(11, generator=gen)
+    g = torch.randn((3, 6, 90), generator=gen)
+    xg = x.to(dev()).requires_grad_()
+    slayer.utils.filter.conv(xg, f.to(dev()), 2).backward(g.to(dev()))
+    assert_rel(xg.grad, O.conv_bwd(g, f, 2), 'conv backward')
+    xg.grad = None
+    slayer.utils.filter.corr(xg, f.to(dev()), 2).backward(g.to(dev()))
+    assert_rel(xg.grad, O.conv_fwd(g, f, 2), 'corr backward')
+
+
+def test_delay_module(slayer):
+    gen = torch.Generator().manual_seed(70)
+    x = torch.rand((2, 5, 3, 40), generator=gen)
+    g = torch.randn((2, 5, 3, 40), generator=gen)
+    d = torch.tensor([0.0, 3.2, 7.9, 1.0, 12.5])
+    mod = slayer.axon.Delay(grad_scale=2.0)
+    mod.delay.data = d.to(dev())
+    mod.init = True
+    xg = x.to(dev()).requires_grad_()
+    y = mod(xg)
+    per_neuron = d.reshape(-1, 1).repeat(1, 3)
+    assert_exact(y, O.delay_fwd(x, per_neuron), 'delay forward')
+    y.backward(g.to(dev()))
+    ref_gi, ref_gd = O.delay_bwd(g, O.delay_fwd(x, per_neuron), per_neuron, grad_scale=2.0)
+    assert_exact(xg.grad, ref_gi, 'delay grad_input')
+    assert_rel(mod.delay.grad, ref_gd.sum(dim=1), 'delay grad_delay', rel=1e-4)
+    # functional form, default one step
+    assert_exact(slayer.axon.delay(x.to(dev())), O.shift(x, 1), 'delay()')
