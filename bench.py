@@ -127,15 +127,18 @@ def cpu_baseline(workload, inp, budget_s=20.0):
         return time.perf_counter() - t0
 
     dt = run(n_sub)
-    per_sample = dt
-    n_fit = max(1, min(N, int(budget_s / max(per_sample, 1e-9))))
-    if n_fit > n_sub:
-        n_sub = n_fit
-        dt = run(n_sub)
+    n_sub = max(1, min(N, int(budget_s / 4 / max(dt, 1e-9))))      # one run = at most a quarter of the budget
+    times, t_start = [], time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 50):
+        times.append(run(n_sub))
+    times.sort()
+    med = times[len(times) // 2]
     nt = n_sub * int(torch.tensor(inp['shape'][1:]).prod())
-    return dict(value=nt / dt, unit='neuron-timesteps/s', cores=torch.get_num_threads(), kind='port',
-                sample=f'oracle (torch CPU per-timestep loop) on batch[:{n_sub}] of {list(inp["shape"])}, '
-                       f'{dt:.1f} s, os.cpu_count()={os.cpu_count()}')
+    return dict(value=nt / med, unit='neuron-timesteps/s', cores=torch.get_num_threads(), kind='port',
+                sample=f'oracle (torch CPU per-timestep loop, same op sequence) on batch[:{n_sub}] of '
+                       f'{list(inp["shape"])}: median of {len(times)} runs, {med:.2f} s each, '
+                       f'{sum(times):.1f} s total; torch threads={torch.get_num_threads()}, '
+                       f'os.cpu_count()={os.cpu_count()}')
 
 
 def main():

@@ -65,7 +65,8 @@ int slayer_li_fwd(float *out, const float *in, const float *decay, const float *
  * grad_in[T-1] = grad_out[T-1];  grad_in[t] = (1 - decay/4096) * grad_in[t+1] + grad_out[t];
  * grad_decay[j] = sum over the neurons that use decay j of sum_t grad_in[t+1] * out[t].
  * grad_decay (num_decays floats) may be NULL to skip the parameter gradient.
- * workspace: M floats of scratch (per-neuron partial sums), required iff grad_decay != NULL. */
+ * workspace: M + 64 * num_decays floats of scratch (per-neuron partial sums, then slice sums),
+ * required iff grad_decay != NULL; its contents on return are unspecified. */
 int slayer_li_bwd(float *grad_in, float *grad_decay, const float *grad_out, const float *out,
                   const float *decay, float *workspace,
                   int64_t M, int64_t neurons_per_batch, int64_t num_decays,
@@ -108,7 +109,7 @@ int slayer_res_fwd(float *re_out, float *im_out, const float *re_in, const float
  * gr[t] = c*gr[t+1] + s*gi[t+1] + g_re[t];  gi[t] = -s*gr[t+1] + c*gi[t+1] + g_im[t];  c, s = decay/4096
  * grad_sin[j] = sum(-gr[t+1]*im[t] + gi[t+1]*re[t]);  grad_cos[j] = sum(gr[t+1]*re[t] + gi[t+1]*im[t]).
  * grad_sin/grad_cos (num_decays floats each) may both be NULL.
- * workspace: 2*M floats, required iff the parameter gradients are requested. */
+ * workspace: 2 * M + 128 * num_decays floats, required iff the parameter gradients are requested. */
 int slayer_res_bwd(float *g_re_in, float *g_im_in, float *grad_sin, float *grad_cos,
                    const float *g_re, const float *g_im, const float *re, const float *im,
                    const float *sin_decay, const float *cos_decay, float *workspace,

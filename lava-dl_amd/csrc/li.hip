@@ -2,6 +2,14 @@
 #include "common.h"
 #include "tile.h"
 
+// time-chunk lengths (steps per LDS tile); overridable for tuning builds
+#ifndef SLAYER_TC_LI_FWD
+#define SLAYER_TC_LI_FWD 64
+#endif
+#ifndef SLAYER_TC_LI_BWD
+#define SLAYER_TC_LI_BWD 32
+#endif
+
 namespace slayer {
 
 // ---------------------------------------------------------------------------------- forward
@@ -64,27 +72,44 @@ struct LiBwd {
     }
 };
 
-// grad[j] = sum of partial[m] over all rows m whose parameter index is j, accumulated in
-// double in a fixed order (one workgroup per parameter, deterministic).
-__global__ __launch_bounds__(256) void reduce_param_grad(float* grad, const float* partial,
-                                                         int64_t M, int64_t npb, int64_t num_params) {
+// Parameter-gradient reduction: grad[j] = sum of partial[m] over all rows m whose parameter
+// index is j.  Two deterministic passes: (j, s) workgroups each sum one slice in double and
+// write one float to scratch[j * split + s]; then one lane per parameter adds its `split`
+// slice sums in double.  `scratch` is the tail of the caller's workspace.
+constexpr int kRedBlock = 256;
+constexpr int kRedMaxSplit = 64;
+
+__global__ __launch_bounds__(kRedBlock) void reduce_param_slices(float* scratch, const float* partial,
+                                                                 int64_t M, int64_t npb, int64_t num_params,
+                                                                 int split) {
     const int64_t j = blockIdx.x;
-    const int64_t block = num_params > 1 ? npb / num_params : npb;   // rows per batch for this parameter
-    const int64_t batches = M / npb;
-    const int64_t total = batches * block;
-    double s = 0.0;
-    for (int64_t i = threadIdx.x; i < total; i += blockDim.x) {
-        const int64_t n = i / block, b = i % block;
-        s += (double)partial[n * npb + j * block + b];
+    const int s = blockIdx.y;
+    const int64_t block = num_params > 1 ? npb / num_params : npb;   // rows per batch element for parameter j
+    const int64_t total = (M / npb) * block;
+    const int64_t per = (total + split - 1) / split;
+    const int64_t lo = s * per, hi = (lo + per) < total ? (lo + per) : total;
+    double acc = 0.0;
+    for (int64_t i = lo + threadIdx.x; i < hi; i += kRedBlock) {
+        const int64_t n = i / block, b = i - n * block;
+        acc += (double)partial[n * npb + j * block + b];
     }
-    __shared__ double red[256];
-    red[threadIdx.x] = s;
+    __shared__ double red[kRedBlock];
+    red[threadIdx.x] = acc;
     __syncthreads();
-    for (int w = 128; w > 0; w >>= 1) {
+    for (int w = kRedBlock / 2; w > 0; w >>= 1) {
         if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
         __syncthreads();
     }
-    if (threadIdx.x == 0) grad[j] = (float)red[0];
+    if (threadIdx.x == 0) scratch[j * split + s] = (float)red[0];
+}
+
+__global__ __launch_bounds__(kRedBlock) void reduce_param_final(float* grad, const float* scratch,
+                                                                int64_t num_params, int split) {
+    const int64_t j = (int64_t)blockIdx.x * kRedBlock + threadIdx.x;
+    if (j >= num_params) return;
+    double acc = 0.0;
+    for (int s = 0; s < split; ++s) acc += (double)scratch[j * split + s];
+    grad[j] = (float)acc;
 }
 
 __global__ void zero_fill(float* p, int64_t n) {
@@ -99,10 +124,25 @@ int launch_zero_fill(float* p, int64_t n, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
-int launch_reduce_param_grad(float* grad, const float* partial, int64_t M, int64_t npb,
+// Slices per parameter: enough that a slice is a few thousand rows, at most kRedMaxSplit.
+int param_grad_split(int64_t M, int64_t npb, int64_t num_params) {
+    const int64_t block = num_params > 1 ? npb / num_params : npb;
+    const int64_t total = (M / npb) * block;
+    int64_t split = total / 2048;
+    if (split < 1) split = 1;
+    if (split > kRedMaxSplit) split = kRedMaxSplit;
+    return (int)split;
+}
+
+// scratch needs num_params * kRedMaxSplit floats.
+int launch_reduce_param_grad(float* grad, const float* partial, float* scratch, int64_t M, int64_t npb,
                              int64_t num_params, hipStream_t stream) {
-    hipLaunchKernelGGL(reduce_param_grad, dim3((unsigned)num_params), dim3(256), 0, stream,
-                       grad, partial, M, npb, num_params);
+    const int split = param_grad_split(M, npb, num_params);
+    hipLaunchKernelGGL(reduce_param_slices, dim3((unsigned)num_params, (unsigned)split), dim3(kRedBlock), 0, stream,
+                       scratch, partial, M, npb, num_params, split);
+    if (int e = (int)hipGetLastError()) return e;
+    hipLaunchKernelGGL(reduce_param_final, dim3((unsigned)((num_params + kRedBlock - 1) / kRedBlock)),
+                       dim3(kRedBlock), 0, stream, grad, scratch, num_params, split);
     return (int)hipGetLastError();
 }
 
@@ -124,10 +164,10 @@ extern "C" int slayer_li_fwd(float* out, const float* in, const float* decay, co
     const float thr = thr_scaled > 0 ? (float)thr_scaled : __builtin_inff();
     if (is_pow2(w_scale)) {
         LiFwd<true>::Params p{{in}, {out}, decay, state, w, 1.0f / w, thr, neurons_per_batch, num_decays, num_states};
-        return launch_stream<LiFwd<true>, 64>(p, M, T, (hipStream_t)stream);
+        return launch_stream<LiFwd<true>, SLAYER_TC_LI_FWD>(p, M, T, (hipStream_t)stream);
     }
     LiFwd<false>::Params p{{in}, {out}, decay, state, w, 1.0f / w, thr, neurons_per_batch, num_decays, num_states};
-    return launch_stream<LiFwd<false>, 64>(p, M, T, (hipStream_t)stream);
+    return launch_stream<LiFwd<false>, SLAYER_TC_LI_FWD>(p, M, T, (hipStream_t)stream);
 }
 
 extern "C" int slayer_li_bwd(float* grad_in, float* grad_decay, const float* grad_out, const float* out,
@@ -141,11 +181,12 @@ extern "C" int slayer_li_bwd(float* grad_in, float* grad_decay, const float* gra
         if (!grad_in || !grad_out || !out || !decay) return SLAYER_ENULL;
         LiBwd::Params p{{grad_out, out}, {grad_in}, decay, grad_decay ? workspace : nullptr,
                         neurons_per_batch, num_decays};
-        if (int e = launch_stream<LiBwd, 32>(p, M, T, (hipStream_t)stream)) return e;
+        if (int e = launch_stream<LiBwd, SLAYER_TC_LI_BWD>(p, M, T, (hipStream_t)stream)) return e;
     }
     if (grad_decay) {
         if (M == 0 || T == 0) return launch_zero_fill(grad_decay, num_decays, (hipStream_t)stream);
-        return launch_reduce_param_grad(grad_decay, workspace, M, neurons_per_batch, num_decays, (hipStream_t)stream);
+        return launch_reduce_param_grad(grad_decay, workspace, workspace + M, M, neurons_per_batch, num_decays,
+                                        (hipStream_t)stream);
     }
     return 0;
 }

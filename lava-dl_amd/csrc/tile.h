@@ -30,6 +30,25 @@ __device__ __forceinline__ int rs0_12(int a, int b) {
     return (int)(((long long)a * (long long)b + bias) >> 12);
 }
 
+// Streaming (non-temporal) 16-byte global accesses: tensors on this path are read once and
+// written once, so they should not displace each other in L2.
+typedef float vf4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 load4(const float* p, bool streaming) {
+    if (streaming) {
+        const vf4 v = __builtin_nontemporal_load(reinterpret_cast<const vf4*>(p));
+        return make_float4(v.x, v.y, v.z, v.w);
+    }
+    return *reinterpret_cast<const float4*>(p);
+}
+__device__ __forceinline__ void store4(float* p, float4 v, bool streaming) {
+    if (streaming) {
+        vf4 u; u.x = v.x; u.y = v.y; u.z = v.z; u.w = v.w;
+        __builtin_nontemporal_store(u, reinterpret_cast<vf4*>(p));
+    } else {
+        *reinterpret_cast<float4*>(p) = v;
+    }
+}
+
 // float32 -> int32 toward zero; out-of-range values saturate (v_cvt_i32_f32).
 __device__ __forceinline__ int trunc_i32(float x) { return (int)x; }
 
@@ -53,7 +72,14 @@ struct TileGeom {
 //   __device__ void init(const Params&, int64_t m, bool valid);
 //   __device__ void step(const float (&x)[kIn], float (&y)[kOut]);
 //   __device__ void finish(const Params&, int64_t m, bool valid);
-template <class Op, int TC, bool VEC4>
+//
+// Line alignment (VEC4 path).  A row of T floats starts wherever m*T falls, so a fixed
+// time grid would cut every row segment across 128-byte lines and each line would be
+// fetched (and partially written) twice.  Instead every row gets its own phase
+// a = (float index of the row start) mod 32 and tile column j of chunk k holds step
+// t = k*TC + j - a: the segments a wave-wide access touches then start on 128-byte
+// boundaries.  Lanes simply skip the columns that fall before step 0 or after step T-1.
+template <class Op, int TC, bool VEC4, bool STREAM>
 __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, int64_t M, int T) {
     using G = TileGeom<TC>;
     constexpr int NI = Op::kIn, NO = Op::kOut, NT = NI > NO ? NI : NO;
@@ -66,25 +92,39 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
     Op op;
     op.init(prm, m0 + lane, lane < rows);
 
-    const int nchunks = (T + TC - 1) / TC;
+    // phase of a row: float index of its first sample modulo one 128-byte line
+    const unsigned base_f = (unsigned)(reinterpret_cast<uintptr_t>(prm.in[0]) >> 2);
+    auto phase = [&](int r) -> int {
+        return VEC4 ? (int)((base_f + (unsigned)(m0 + r) * (unsigned)T) & 31u) : 0;
+    };
+    const int a_lane = phase(lane);
+
+    int last = (lane < rows) ? (a_lane + T - 1) / TC : 0;    // last chunk this row needs
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const int o = __shfl_xor(last, d);
+        last = o > last ? o : last;
+    }
+    const int nchunks = last + 1;
+
     const int crow = lane / G::kQuads;      // row within a pass (copy pattern)
     const int cq = lane % G::kQuads;        // quad within the row
 
     float4 stage[NI][G::kPasses];
 
     auto fetch = [&](int chunk) {
-        const int t = chunk * TC + 4 * cq;
 #pragma unroll
         for (int p = 0; p < G::kPasses; ++p) {
             const int r = p * G::kRowsPerPass + crow;
-            const size_t off = (size_t)(m0 + r) * (size_t)T + (size_t)t;
+            const int t = chunk * TC + 4 * cq - phase(r);
+            const int64_t off = (int64_t)(m0 + r) * (int64_t)T + (int64_t)t;
 #pragma unroll
             for (int i = 0; i < NI; ++i) {
                 float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (r < rows) {
                     const float* src = prm.in[i] + off;
                     if (VEC4) {
-                        if (t < T) v = *reinterpret_cast<const float4*>(src);
+                        if (t >= 0 && t < T) v = load4(src, STREAM);
                     } else {
                         if (t + 0 < T) v.x = src[0];
                         if (t + 1 < T) v.y = src[1];
@@ -101,8 +141,6 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
 
     for (int k = 0; k < nchunks; ++k) {
         const int chunk = Op::kReverse ? nchunks - 1 - k : k;
-        const int t0 = chunk * TC;
-        const int len = (T - t0) < TC ? (T - t0) : TC;
 
         // staged registers -> LDS
 #pragma unroll
@@ -116,54 +154,55 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
 
         if (k + 1 < nchunks) fetch(Op::kReverse ? chunk - 1 : chunk + 1);
 
-        // sequential recurrence: lane = neuron
-        const int nq = (len + 3) >> 2;
+        // sequential recurrence: lane = neuron; columns outside [0, T) are skipped
+        const int tl = chunk * TC - a_lane;           // step held by column 0 of this lane's row
 #pragma unroll 2
-        for (int q = 0; q < nq; ++q) {
-            const int qq = Op::kReverse ? nq - 1 - q : q;
-            float xin[NI][4], yout[NO][4];
+        for (int q = 0; q < G::kQuads; ++q) {
+            const int qq = Op::kReverse ? G::kQuads - 1 - q : q;
+            const int t = tl + 4 * qq;
+            if (t >= 0 && t < T) {
+                float xin[NI][4], yout[NO][4];
 #pragma unroll
-            for (int i = 0; i < NI; ++i) {
-                const float4 v = *reinterpret_cast<const float4*>(&tile[i][lane * G::kPitch + 4 * qq]);
-                xin[i][0] = v.x; xin[i][1] = v.y; xin[i][2] = v.z; xin[i][3] = v.w;
+                for (int i = 0; i < NI; ++i) {
+                    const float4 v = *reinterpret_cast<const float4*>(&tile[i][lane * G::kPitch + 4 * qq]);
+                    xin[i][0] = v.x; xin[i][1] = v.y; xin[i][2] = v.z; xin[i][3] = v.w;
+                }
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const int ss = Op::kReverse ? 3 - s : s;
+                    float x[NI], y[NO];
+#pragma unroll
+                    for (int i = 0; i < NI; ++i) x[i] = xin[i][ss];
+                    op.step(x, y);
+#pragma unroll
+                    for (int o = 0; o < NO; ++o) yout[o][ss] = y[o];
+                }
+#pragma unroll
+                for (int o = 0; o < NO; ++o)
+                    *reinterpret_cast<float4*>(&tile[o][lane * G::kPitch + 4 * qq]) =
+                        make_float4(yout[o][0], yout[o][1], yout[o][2], yout[o][3]);
             }
-#pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const int ss = Op::kReverse ? 3 - s : s;
-                float x[NI], y[NO];
-#pragma unroll
-                for (int i = 0; i < NI; ++i) x[i] = xin[i][ss];
-                op.step(x, y);
-#pragma unroll
-                for (int o = 0; o < NO; ++o) yout[o][ss] = y[o];
-            }
-#pragma unroll
-            for (int o = 0; o < NO; ++o)
-                *reinterpret_cast<float4*>(&tile[o][lane * G::kPitch + 4 * qq]) =
-                    make_float4(yout[o][0], yout[o][1], yout[o][2], yout[o][3]);
         }
         __syncthreads();
 
         // LDS -> global
-        {
-            const int t = t0 + 4 * cq;
 #pragma unroll
-            for (int p = 0; p < G::kPasses; ++p) {
-                const int r = p * G::kRowsPerPass + crow;
-                const size_t off = (size_t)(m0 + r) * (size_t)T + (size_t)t;
+        for (int p = 0; p < G::kPasses; ++p) {
+            const int r = p * G::kRowsPerPass + crow;
+            const int t = chunk * TC + 4 * cq - phase(r);
+            const int64_t off = (int64_t)(m0 + r) * (int64_t)T + (int64_t)t;
 #pragma unroll
-                for (int o = 0; o < NO; ++o) {
-                    const float4 v = *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]);
-                    if (r < rows) {
-                        float* dst = prm.out[o] + off;
-                        if (VEC4) {
-                            if (t < T) *reinterpret_cast<float4*>(dst) = v;
-                        } else {
-                            if (t + 0 < T) dst[0] = v.x;
-                            if (t + 1 < T) dst[1] = v.y;
-                            if (t + 2 < T) dst[2] = v.z;
-                            if (t + 3 < T) dst[3] = v.w;
-                        }
+            for (int o = 0; o < NO; ++o) {
+                const float4 v = *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]);
+                if (r < rows) {
+                    float* dst = prm.out[o] + off;
+                    if (VEC4) {
+                        if (t >= 0 && t < T) store4(dst, v, STREAM);
+                    } else {
+                        if (t + 0 < T) dst[0] = v.x;
+                        if (t + 1 < T) dst[1] = v.y;
+                        if (t + 2 < T) dst[2] = v.z;
+                        if (t + 3 < T) dst[3] = v.w;
                     }
                 }
             }
@@ -175,18 +214,22 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// Launch helper: picks the dwordx4 path when T and every pointer allow it.
+// Launch helper: picks the dwordx4 path when T and every pointer allow it, and non-temporal
+// global accesses when the tensors are too large to be reused out of the last-level cache.
 template <class Op, int TC>
 int launch_stream(const typename Op::Params& prm, int64_t M, int64_t T, hipStream_t stream) {
     if (M == 0 || T == 0) return 0;
     bool vec = (T % 4) == 0;
     for (int i = 0; i < Op::kIn; ++i) vec = vec && aligned16(prm.in[i]);
     for (int o = 0; o < Op::kOut; ++o) vec = vec && aligned16(prm.out[o]);
+    const bool streaming = M * T * 4 > ((int64_t)64 << 20);
     const dim3 grid((unsigned)((M + kWave - 1) / kWave)), block(kWave);
-    if (vec)
-        hipLaunchKernelGGL((stream_kernel<Op, TC, true>), grid, block, 0, stream, prm, M, (int)T);
+    if (!vec)
+        hipLaunchKernelGGL((stream_kernel<Op, TC, false, false>), grid, block, 0, stream, prm, M, (int)T);
+    else if (streaming)
+        hipLaunchKernelGGL((stream_kernel<Op, TC, true, true>), grid, block, 0, stream, prm, M, (int)T);
     else
-        hipLaunchKernelGGL((stream_kernel<Op, TC, false>), grid, block, 0, stream, prm, M, (int)T);
+        hipLaunchKernelGGL((stream_kernel<Op, TC, true, false>), grid, block, 0, stream, prm, M, (int)T);
     return (int)hipGetLastError();
 }
 

@@ -10,7 +10,8 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, 'libslayer_hip.so')
+# SLAYER_HIP_LIB points at an alternative build of the same library (e.g. a tuning build)
+LIB_PATH = os.environ.get('SLAYER_HIP_LIB') or os.path.join(_HERE, 'libslayer_hip.so')
 ABI_VERSION = 1
 
 _lib = None

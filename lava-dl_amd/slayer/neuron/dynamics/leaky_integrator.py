@@ -68,7 +68,7 @@ def _bwd(grad_output, output, decay, need_decay_grad=True):
     grad_decay = workspace = None
     if need_decay_grad:
         grad_decay = torch.empty(decay.numel(), dtype=torch.float32, device=dev)
-        workspace = torch.empty(max(M, 1), dtype=torch.float32, device=dev)
+        workspace = torch.empty(M + 64 * decay.numel(), dtype=torch.float32, device=dev)
     with torch.cuda.device(dev):
         N.check(N.lib().slayer_li_bwd(
             N.ptr(grad_input), N.ptr(grad_decay), N.ptr(grad_output), N.ptr(output), N.ptr(decay),

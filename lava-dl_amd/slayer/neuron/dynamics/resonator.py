@@ -74,7 +74,7 @@ def _bwd(grad_real, grad_imag, real, imag, sin_decay, cos_decay, need_decay_grad
     if need_decay_grad:
         g_sin = torch.empty(sin_decay.numel(), dtype=torch.float32, device=dev)
         g_cos = torch.empty(cos_decay.numel(), dtype=torch.float32, device=dev)
-        workspace = torch.empty(max(2 * M, 1), dtype=torch.float32, device=dev)
+        workspace = torch.empty(2 * M + 128 * sin_decay.numel(), dtype=torch.float32, device=dev)
     with torch.cuda.device(dev):
         N.check(N.lib().slayer_res_bwd(
             N.ptr(g_re_in), N.ptr(g_im_in), N.ptr(g_sin), N.ptr(g_cos),
