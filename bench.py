@@ -62,9 +62,9 @@ class Cuba:
         with t('li_fwd_voltage'):
             vol = L._fwd(cur, i['d_v'], self.zero, self.thr, self.w)
         with t('spike_fwd'):
-            spk, th = S._fwd(vol, self.thr, False, 1)
+            spk = S._fwd(vol, None, self.thr, False, 1)
         with t('spike_bwd'):
-            g_vol = S._bwd(i['g'], vol, th, 1.0, 1.0, False)
+            g_vol = S._bwd(i['g'], vol, None, self.thr, 1.0, 1.0, False)
         with t('li_bwd_voltage'):
             g_cur, gd_v = L._bwd(g_vol, vol, i['d_v'])
         with t('li_bwd_current'):
@@ -148,6 +148,9 @@ def main():
     ap.add_argument('--warmup', type=int, default=5)
     ap.add_argument('--workload', default='cuba')
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--calibration-copies', type=int, default=0,
+                    help='also run N plain device copies of one input tensor (a kernel of known traffic, '
+                         'used to scale hardware byte counters when profiling)')
     a = ap.parse_args()
     if a.gpus != 1:
         raise SystemExit('bench.py measures one GPU: this hot path has no multi-GPU component '
@@ -159,6 +162,8 @@ def main():
 
     inp = make_inputs(a.workload, dev)
     job = Cuba(inp)
+    for _ in range(a.calibration_copies):
+        torch.empty_like(inp['x']).copy_(inp['x'])
     nt = int(torch.tensor(inp['shape']).prod())
 
     for _ in range(a.warmup):

@@ -118,28 +118,34 @@ int slayer_res_bwd(float *g_re_in, float *g_im_in, float *grad_sin, float *grad_
 
 /* ---- spike functions (elementwise; they replace chains of torch ops, not a .cu) ----------- */
 
-/* Spike.forward (spike/spike.py:64-87).  threshold: num_threshold == 1 -> scalar read from
- * device memory, == numel -> elementwise.  graded != 0: out = (v >= th) * v / scale. */
+/* Threshold convention of the four spike entry points: threshold == NULL -> the scalar
+ * threshold_value applies everywhere; otherwise threshold points at num_threshold device floats,
+ * num_threshold == 1 (one value, read on the device) or == numel (elementwise). */
+
+/* Spike.forward (spike/spike.py:64-87).  graded != 0: out = (v >= th) * v / scale. */
 int slayer_spike_fwd(float *spikes, const float *voltage, const float *threshold,
-                     int64_t num_threshold, int graded, float scale, int64_t numel, void *stream);
+                     int64_t num_threshold, float threshold_value, int graded, float scale,
+                     int64_t numel, void *stream);
 
 /* Spike.backward / _spike_backward (spike/spike.py:10-23,113-126).
  * binary: rho/2/tau * exp(-|v - th| / tau) * g;   graded: rho * exp(min(v - th, 0) / tau) * g. */
 int slayer_spike_bwd(float *grad_voltage, const float *grad_spikes, const float *voltage,
-                     const float *threshold, int64_t num_threshold,
+                     const float *threshold, int64_t num_threshold, float threshold_value,
                      float tau_rho, float scale_rho, int graded, int64_t numel, void *stream);
 
 /* complex.Spike.forward (spike/complex.py:49-92): (re >= th) * (im[t-1] < 0) * (im[t] >= 0)
- * with im[-1] = imag_last[m] (num_last == 1 broadcasts).  graded != 0 multiplies by re / scale. */
+ * with im[-1] = imag_last[m] (num_last == 1 broadcasts; imag_last == NULL -> imag_last_value).
+ * graded != 0 multiplies by re / scale. */
 int slayer_cspike_fwd(float *spikes, const float *re, const float *im, const float *threshold,
-                      int64_t num_threshold, const float *imag_last, int64_t num_last,
+                      int64_t num_threshold, float threshold_value,
+                      const float *imag_last, int64_t num_last, float imag_last_value,
                       int graded, float scale, int64_t M, int64_t T, void *stream);
 
 /* complex.Spike.backward (spike/complex.py:117-167). */
 int slayer_cspike_bwd(float *grad_re, float *grad_im, const float *grad_spikes,
                       const float *re, const float *im, const float *threshold,
-                      int64_t num_threshold, float tau_rho, float scale_rho, int graded,
-                      int64_t numel, void *stream);
+                      int64_t num_threshold, float threshold_value,
+                      float tau_rho, float scale_rho, int graded, int64_t numel, void *stream);
 
 /* ---- time shift --------------------------------------------------------------------------- */
 

@@ -4,7 +4,7 @@
 
 // time-chunk lengths (steps per LDS tile); overridable for tuning builds
 #ifndef SLAYER_TC_LI_FWD
-#define SLAYER_TC_LI_FWD 64
+#define SLAYER_TC_LI_FWD 32
 #endif
 #ifndef SLAYER_TC_LI_BWD
 #define SLAYER_TC_LI_BWD 32

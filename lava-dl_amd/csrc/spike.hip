@@ -26,9 +26,9 @@ inline EltSplit elt_split(int64_t n, bool aligned) {
 
 template <bool TENSOR_TH, bool GRADED, bool STREAM>
 __global__ __launch_bounds__(kEltBlock) void spike_fwd_kernel(float* __restrict__ s, const float* __restrict__ v,
-                                                              const float* __restrict__ th, float scale, int64_t n,
-                                                              int64_t nq) {
-    const float th0 = TENSOR_TH ? 0.f : th[0];
+                                                              const float* __restrict__ th, float th0, float scale,
+                                                              int64_t n, int64_t nq) {
+    if (!TENSOR_TH && th) th0 = th[0];
     auto f = [&](float x, float t) -> float {
         const float h = (x >= t) ? 1.0f : 0.0f;
         return GRADED ? (h * x) / scale : h;
@@ -48,8 +48,8 @@ __global__ __launch_bounds__(kEltBlock) void spike_fwd_kernel(float* __restrict_
 template <bool TENSOR_TH, bool GRADED, bool STREAM>
 __global__ __launch_bounds__(kEltBlock) void spike_bwd_kernel(float* __restrict__ gv, const float* __restrict__ gs,
                                                               const float* __restrict__ v, const float* __restrict__ th,
-                                                              float tau, float rho, int64_t n, int64_t nq) {
-    const float th0 = TENSOR_TH ? 0.f : th[0];
+                                                              float th0, float tau, float rho, int64_t n, int64_t nq) {
+    if (!TENSOR_TH && th) th0 = th[0];
     const float lead = (rho / 2.0f) / tau;       // scale_rho / 2 / tau_rho, left to right
     auto f = [&](float x, float t, float g) -> float {
         const float d = x - t;
@@ -75,10 +75,11 @@ __global__ __launch_bounds__(kEltBlock) void spike_bwd_kernel(float* __restrict_
 template <bool TENSOR_TH, bool GRADED, bool VEC4>
 __global__ __launch_bounds__(kEltBlock) void cspike_fwd_kernel(float* __restrict__ s, const float* __restrict__ re,
                                                                const float* __restrict__ im,
-                                                               const float* __restrict__ th,
+                                                               const float* __restrict__ th, float th0,
                                                                const float* __restrict__ last, int64_t num_last,
-                                                               float scale, int64_t M, int T, int64_t items) {
-    const float th0 = TENSOR_TH ? 0.f : th[0];
+                                                               float last0, float scale, int64_t M, int T,
+                                                               int64_t items) {
+    if (!TENSOR_TH && th) th0 = th[0];
     auto f = [&](float r, float thr, float prev, float cur) -> float {
         const float a = (r >= thr) ? 1.0f : 0.0f, b = (prev < 0.0f) ? 1.0f : 0.0f, c = (cur >= 0.0f) ? 1.0f : 0.0f;
         return GRADED ? (((r * a) * b) * c) / scale : (a * b) * c;
@@ -90,7 +91,7 @@ __global__ __launch_bounds__(kEltBlock) void cspike_fwd_kernel(float* __restrict
         const int64_t m = i / T;
         const int t = (int)(i - m * T);
         const float4 c = load4(im + i, true), r = load4(re + i, true);
-        const float p0 = (t == 0) ? last[num_last == 1 ? 0 : m] : im[i - 1];
+        const float p0 = (t == 0) ? (last ? last[num_last == 1 ? 0 : m] : last0) : im[i - 1];
         float4 h = make_float4(th0, th0, th0, th0);
         if (TENSOR_TH) h = load4(th + i, true);
         store4(s + i, make_float4(f(r.x, h.x, p0, c.x), f(r.y, h.y, c.x, c.y), f(r.z, h.z, c.y, c.z),
@@ -98,7 +99,7 @@ __global__ __launch_bounds__(kEltBlock) void cspike_fwd_kernel(float* __restrict
     } else {
         const int64_t m = g / T;
         const int t = (int)(g - m * T);
-        const float prev = (t == 0) ? last[num_last == 1 ? 0 : m] : im[g - 1];
+        const float prev = (t == 0) ? (last ? last[num_last == 1 ? 0 : m] : last0) : im[g - 1];
         s[g] = f(re[g], TENSOR_TH ? th[g] : th0, prev, im[g]);
     }
 }
@@ -108,9 +109,9 @@ __global__ __launch_bounds__(kEltBlock) void cspike_bwd_kernel(float* __restrict
                                                                const float* __restrict__ gs,
                                                                const float* __restrict__ re,
                                                                const float* __restrict__ im,
-                                                               const float* __restrict__ th, float tau, float rho,
-                                                               int64_t n, int64_t nq) {
-    const float th0 = TENSOR_TH ? 0.f : th[0];
+                                                               const float* __restrict__ th, float th0, float tau,
+                                                               float rho, int64_t n, int64_t nq) {
+    if (!TENSOR_TH && th) th0 = th[0];
     const float half_over_tau = (1.0f / 2.0f) / tau;   // 1 / 2 / tau_rho
     const float two_tau = 2.0f * tau;
     const float neg_rho_over_tau = (-rho) / tau;
@@ -162,7 +163,8 @@ using namespace slayer;
         }                                                                                                  \
     } while (0)
 
-static int check_threshold(int64_t num_threshold, int64_t numel) {
+static int check_threshold(const float* threshold, int64_t num_threshold, int64_t numel) {
+    if (!threshold) return 0;
     return (num_threshold == 1 || num_threshold == numel) ? 0 : SLAYER_EINVAL;
 }
 
@@ -180,64 +182,68 @@ static int check_numel(int64_t numel) {
 }
 
 extern "C" int slayer_spike_fwd(float* spikes, const float* voltage, const float* threshold,
-                                int64_t num_threshold, int graded, float scale, int64_t numel, void* stream) {
+                                int64_t num_threshold, float threshold_value, int graded, float scale,
+                                int64_t numel, void* stream) {
     if (int e = check_numel(numel)) return e;
     if (numel == 0) return 0;
-    if (!spikes || !voltage || !threshold) return SLAYER_ENULL;
-    if (int e = check_threshold(num_threshold, numel)) return e;
-    const bool tt = num_threshold != 1;
+    if (!spikes || !voltage) return SLAYER_ENULL;
+    if (int e = check_threshold(threshold, num_threshold, numel)) return e;
+    const bool tt = threshold && num_threshold != 1;
     const EltSplit sp = elt_split(numel, all_aligned({spikes, voltage, tt ? threshold : nullptr}));
     hipStream_t st = (hipStream_t)stream;
     SLAYER_LAUNCH3(spike_fwd_kernel, tt, graded != 0, numel * 4 > kStreamingBytes, sp.grid, st,
-                   spikes, voltage, threshold, scale, numel, sp.nq);
+                   spikes, voltage, threshold, threshold_value, scale, numel, sp.nq);
     return (int)hipGetLastError();
 }
 
 extern "C" int slayer_spike_bwd(float* grad_voltage, const float* grad_spikes, const float* voltage,
-                                const float* threshold, int64_t num_threshold,
+                                const float* threshold, int64_t num_threshold, float threshold_value,
                                 float tau_rho, float scale_rho, int graded, int64_t numel, void* stream) {
     if (int e = check_numel(numel)) return e;
     if (numel == 0) return 0;
-    if (!grad_voltage || !grad_spikes || !voltage || !threshold) return SLAYER_ENULL;
-    if (int e = check_threshold(num_threshold, numel)) return e;
-    const bool tt = num_threshold != 1;
+    if (!grad_voltage || !grad_spikes || !voltage) return SLAYER_ENULL;
+    if (int e = check_threshold(threshold, num_threshold, numel)) return e;
+    const bool tt = threshold && num_threshold != 1;
     const EltSplit sp = elt_split(numel, all_aligned({grad_voltage, grad_spikes, voltage, tt ? threshold : nullptr}));
     hipStream_t st = (hipStream_t)stream;
     SLAYER_LAUNCH3(spike_bwd_kernel, tt, graded != 0, numel * 4 > kStreamingBytes, sp.grid, st,
-                   grad_voltage, grad_spikes, voltage, threshold, tau_rho, scale_rho, numel, sp.nq);
+                   grad_voltage, grad_spikes, voltage, threshold, threshold_value, tau_rho, scale_rho, numel, sp.nq);
     return (int)hipGetLastError();
 }
 
 extern "C" int slayer_cspike_fwd(float* spikes, const float* re, const float* im, const float* threshold,
-                                 int64_t num_threshold, const float* imag_last, int64_t num_last,
+                                 int64_t num_threshold, float threshold_value,
+                                 const float* imag_last, int64_t num_last, float imag_last_value,
                                  int graded, float scale, int64_t M, int64_t T, void* stream) {
     if (int e = check_rows(M, T)) return e;
     if (M == 0 || T == 0) return 0;
-    if (!spikes || !re || !im || !threshold || !imag_last) return SLAYER_ENULL;
-    if (int e = check_threshold(num_threshold, M * T)) return e;
-    if (int e = check_states(M, num_last)) return e;
-    const bool tt = num_threshold != 1;
+    if (!spikes || !re || !im) return SLAYER_ENULL;
+    if (int e = check_threshold(threshold, num_threshold, M * T)) return e;
+    if (imag_last)
+        if (int e = check_states(M, num_last)) return e;
+    const bool tt = threshold && num_threshold != 1;
     const bool vec = (T % 4 == 0) && all_aligned({spikes, re, im, tt ? threshold : nullptr});
     const int64_t items = vec ? M * T / 4 : M * T;
     const unsigned grid = (unsigned)((items + kEltBlock - 1) / kEltBlock);
     hipStream_t st = (hipStream_t)stream;
     SLAYER_LAUNCH3(cspike_fwd_kernel, tt, graded != 0, vec, grid, st,
-                   spikes, re, im, threshold, imag_last, num_last, scale, M, (int)T, items);
+                   spikes, re, im, threshold, threshold_value, imag_last, num_last, imag_last_value, scale, M, (int)T,
+                   items);
     return (int)hipGetLastError();
 }
 
 extern "C" int slayer_cspike_bwd(float* grad_re, float* grad_im, const float* grad_spikes,
                                  const float* re, const float* im, const float* threshold,
-                                 int64_t num_threshold, float tau_rho, float scale_rho, int graded,
-                                 int64_t numel, void* stream) {
+                                 int64_t num_threshold, float threshold_value, float tau_rho, float scale_rho,
+                                 int graded, int64_t numel, void* stream) {
     if (int e = check_numel(numel)) return e;
     if (numel == 0) return 0;
-    if (!grad_re || !grad_im || !grad_spikes || !re || !im || !threshold) return SLAYER_ENULL;
-    if (int e = check_threshold(num_threshold, numel)) return e;
-    const bool tt = num_threshold != 1;
+    if (!grad_re || !grad_im || !grad_spikes || !re || !im) return SLAYER_ENULL;
+    if (int e = check_threshold(threshold, num_threshold, numel)) return e;
+    const bool tt = threshold && num_threshold != 1;
     const EltSplit sp = elt_split(numel, all_aligned({grad_re, grad_im, grad_spikes, re, im, tt ? threshold : nullptr}));
     hipStream_t st = (hipStream_t)stream;
     SLAYER_LAUNCH3(cspike_bwd_kernel, tt, graded != 0, numel * 4 > kStreamingBytes, sp.grid, st,
-                   grad_re, grad_im, grad_spikes, re, im, threshold, tau_rho, scale_rho, numel, sp.nq);
+                   grad_re, grad_im, grad_spikes, re, im, threshold, threshold_value, tau_rho, scale_rho, numel, sp.nq);
     return (int)hipGetLastError();
 }

@@ -79,11 +79,19 @@ struct TileGeom {
 // a = (float index of the row start) mod 32 and tile column j of chunk k holds step
 // t = k*TC + j - a: the segments a wave-wide access touches then start on 128-byte
 // boundaries.  Lanes simply skip the columns that fall before step 0 or after step T-1.
+//
+// Boundary lines (VEC4 path).  Unless T is a multiple of 32, the last line of row r is also
+// the first line of row r+1.  Writing it in two pieces at two different times costs a
+// read-modify-write in memory for each piece (measured: ~16% of the kernel at T = 300), so
+// output quads that fall in such a shared line are collected in an LDS buffer of 65 lines
+// (one per row boundary of the wave) and written once, whole, after the last chunk.  Only
+// the two lines shared with neighbouring workgroups are still written in pieces.
 template <class Op, int TC, bool VEC4, bool STREAM>
 __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, int64_t M, int T) {
     using G = TileGeom<TC>;
     constexpr int NI = Op::kIn, NO = Op::kOut, NT = NI > NO ? NI : NO;
     __shared__ __attribute__((aligned(16))) float tile[NT][G::kTileFloats];
+    __shared__ __attribute__((aligned(16))) float bline[VEC4 ? NO : 1][VEC4 ? (kWave + 1) * 32 : 4];
 
     const int lane = threadIdx.x;
     const int64_t m0 = (int64_t)blockIdx.x * kWave;
@@ -106,6 +114,9 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
         last = o > last ? o : last;
     }
     const int nchunks = last + 1;
+
+    // rows shorter than a line could start and end inside the same line; they keep direct stores
+    const bool route = VEC4 && T >= 32;
 
     const int crow = lane / G::kQuads;      // row within a pass (copy pattern)
     const int cq = lane % G::kQuads;        // quad within the row
@@ -185,19 +196,30 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
         }
         __syncthreads();
 
-        // LDS -> global
+        // LDS -> global (quads of a line shared with a neighbouring row go to the boundary buffer)
 #pragma unroll
         for (int p = 0; p < G::kPasses; ++p) {
             const int r = p * G::kRowsPerPass + crow;
-            const int t = chunk * TC + 4 * cq - phase(r);
+            const int a = phase(r);
+            const int pos = chunk * TC + 4 * cq;          // position in the row's line-aligned window
+            const int t = pos - a;
             const int64_t off = (int64_t)(m0 + r) * (int64_t)T + (int64_t)t;
+            const int end = a + T;                        // window position one past the last step
+            const int last_full = end & ~31;
 #pragma unroll
             for (int o = 0; o < NO; ++o) {
                 const float4 v = *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]);
                 if (r < rows) {
                     float* dst = prm.out[o] + off;
                     if (VEC4) {
-                        if (t >= 0 && t < T) store4(dst, v, STREAM);
+                        if (t >= 0 && t < T) {
+                            if (route && a != 0 && pos < 32)
+                                *reinterpret_cast<float4*>(&bline[o][r * 32 + pos]) = v;
+                            else if (route && pos >= last_full)   // only when end is not a line multiple
+                                *reinterpret_cast<float4*>(&bline[o][(r + 1) * 32 + (pos - last_full)]) = v;
+                            else
+                                store4(dst, v, STREAM);
+                        }
                     } else {
                         if (t + 0 < T) dst[0] = v.x;
                         if (t + 1 < T) dst[1] = v.y;
@@ -208,6 +230,21 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
             }
         }
         __syncthreads();
+    }
+
+    if (route) {
+        // boundary line b holds the tail of row b-1 (columns < phase(b)) and the head of row b
+        for (int i = lane; i < (kWave + 1) * 8; i += kWave) {
+            const int b = i >> 3, col = (i & 7) * 4;
+            const int a = phase(b);
+            const bool owned = (col < a) ? (b >= 1 && b - 1 < rows) : (b < rows);
+            if (a != 0 && b <= rows && owned) {
+                const int64_t off = (int64_t)(m0 + b) * (int64_t)T - a + col;
+#pragma unroll
+                for (int o = 0; o < NO; ++o)
+                    store4(prm.out[o] + off, *reinterpret_cast<const float4*>(&bline[o][b * 32 + col]), STREAM);
+            }
+        }
     }
     op.finish(prm, m0 + lane, lane < rows);
 }

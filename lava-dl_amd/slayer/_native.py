@@ -32,10 +32,10 @@ _SIGNATURES = {
     'slayer_res_fwd': (_INT, [_P, _P, _P, _P, _P, _P, _P, _P, _D, _INT,
                               _I64, _I64, _I64, _I64, _I64, _I64, _P]),
     'slayer_res_bwd': (_INT, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _P]),
-    'slayer_spike_fwd': (_INT, [_P, _P, _P, _I64, _INT, _F, _I64, _P]),
-    'slayer_spike_bwd': (_INT, [_P, _P, _P, _P, _I64, _F, _F, _INT, _I64, _P]),
-    'slayer_cspike_fwd': (_INT, [_P, _P, _P, _P, _I64, _P, _I64, _INT, _F, _I64, _I64, _P]),
-    'slayer_cspike_bwd': (_INT, [_P, _P, _P, _P, _P, _P, _I64, _F, _F, _INT, _I64, _P]),
+    'slayer_spike_fwd': (_INT, [_P, _P, _P, _I64, _F, _INT, _F, _I64, _P]),
+    'slayer_spike_bwd': (_INT, [_P, _P, _P, _P, _I64, _F, _F, _F, _INT, _I64, _P]),
+    'slayer_cspike_fwd': (_INT, [_P, _P, _P, _P, _I64, _F, _P, _I64, _F, _INT, _F, _I64, _I64, _P]),
+    'slayer_cspike_bwd': (_INT, [_P, _P, _P, _P, _P, _P, _I64, _F, _F, _F, _INT, _I64, _P]),
     'slayer_shift': (_INT, [_P, _P, _P, _I64, _F, _I64, _I64, _I64, _P]),
     'slayer_conv': (_INT, [_P, _P, _P, _I64, _F, _I64, _I64, _P]),
     'slayer_corr': (_INT, [_P, _P, _P, _I64, _F, _I64, _I64, _P]),

@@ -9,34 +9,35 @@ import torch
 from .. import _native as N
 
 
-def _threshold_tensor(threshold, like):
+def split_threshold(threshold, like):
+    """(device tensor or None, scalar value): a python number travels by value, a tensor
+    stays on the device (one element, or expanded to the shape of ``like``)."""
     if torch.is_tensor(threshold):
         th = threshold.detach().to(device=like.device, dtype=like.dtype)
         if th.numel() != 1 and th.shape != like.shape:
             th = th.expand(like.shape)
-        return th.contiguous()
-    return torch.tensor([threshold], device=like.device, dtype=like.dtype)
+        return th.contiguous(), 0.0
+    return None, float(threshold)
 
 
-def _fwd(voltage, threshold, graded, scale):
+def _fwd(voltage, th, th_value, graded, scale):
     dev = N.require_gpu(voltage)
-    voltage = voltage.contiguous()
-    th = _threshold_tensor(threshold, voltage)
     spikes = torch.empty_like(voltage)
     with torch.cuda.device(dev):
         N.check(N.lib().slayer_spike_fwd(
-            N.ptr(spikes), N.ptr(voltage), N.ptr(th), th.numel(),
+            N.ptr(spikes), N.ptr(voltage), N.ptr(th), 0 if th is None else th.numel(), th_value,
             1 if graded else 0, float(scale), voltage.numel(), N.stream_handle()))
-    return spikes, th
+    return spikes
 
 
-def _bwd(grad_spikes, voltage, th, tau_rho, scale_rho, graded):
-    dev = N.require_gpu(grad_spikes, voltage, th)
+def _bwd(grad_spikes, voltage, th, th_value, tau_rho, scale_rho, graded):
+    dev = N.require_gpu(grad_spikes, voltage)
     grad_spikes = grad_spikes.contiguous()
     grad_voltage = torch.empty_like(voltage)
     with torch.cuda.device(dev):
         N.check(N.lib().slayer_spike_bwd(
-            N.ptr(grad_voltage), N.ptr(grad_spikes), N.ptr(voltage), N.ptr(th), th.numel(),
+            N.ptr(grad_voltage), N.ptr(grad_spikes), N.ptr(voltage), N.ptr(th),
+            0 if th is None else th.numel(), th_value,
             float(tau_rho), float(scale_rho), 1 if graded else 0, voltage.numel(), N.stream_handle()))
     return grad_voltage
 
@@ -53,13 +54,15 @@ class Spike(torch.autograd.Function):
     @staticmethod
     def forward(ctx, voltage, threshold, tau_rho, scale_rho, graded_spike, voltage_last, scale):
         graded = graded_spike is True
-        spikes, th = _fwd(voltage, threshold, graded, scale)
-        ctx.save_for_backward(voltage.contiguous(), th)
-        ctx.tau_rho, ctx.scale_rho, ctx.graded = float(tau_rho), float(scale_rho), graded
+        voltage = voltage.contiguous()
+        th, th_value = split_threshold(threshold, voltage)
+        spikes = _fwd(voltage, th, th_value, graded, scale)
+        ctx.save_for_backward(voltage, th)
+        ctx.th_value, ctx.tau_rho, ctx.scale_rho, ctx.graded = th_value, float(tau_rho), float(scale_rho), graded
         return spikes
 
     @staticmethod
     def backward(ctx, grad_spikes):
         voltage, th = ctx.saved_tensors
-        grad = _bwd(grad_spikes, voltage, th, ctx.tau_rho, ctx.scale_rho, ctx.graded)
+        grad = _bwd(grad_spikes, voltage, th, ctx.th_value, ctx.tau_rho, ctx.scale_rho, ctx.graded)
         return grad, None, None, None, None, None, None

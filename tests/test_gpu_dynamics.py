@@ -39,6 +39,11 @@ LI_CASES = [
     ((2, 64, 1),           'channel',  64,   0.5,                'full'),     # T == 1
     ((1, 1, 260),          'shared',   4096, 2.0,                'scalar'),   # one neuron
     ((2, 130, 64),         'channel',  64,   0.0,                'scalar'),   # threshold 0 = disabled
+    ((3, 50, 36),          'channel',  64,   1.0,                'scalar'),   # rows barely longer than a 128-byte line
+    ((3, 50, 28),          'channel',  64,   1.0,                'full'),     # rows shorter than a line
+    ((1, 67, 300),         'channel',  64,   1.0,                'scalar'),   # partial last wave, T % 32 == 12
+    ((2, 64, 100),         'neuron',   64,   1.0,                'scalar'),   # exactly one wave per batch element
+    ((5, 33, 1000),        'channel',  4096, 1.0,                'full'),     # T % 32 == 8
 ]
 
 
