@@ -22,6 +22,11 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per launch divided by algorithmic bytes, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# script scaled by a plain copy of known size (profiles/cuba_fwd_bwd_32x16x32x32x300.md).
+MEASURED_TRAFFIC_FACTOR = {'stream_kernel<LiFwd>': 1.038, 'stream_kernel<LiBwd>': 1.057,
+                           'spike_fwd_kernel': 1.000, 'spike_bwd_kernel': 1.000}
+
 
 def make_inputs(workload, dev):
     """Synthetic inputs generated on the CPU with a fixed seed, then copied to the GPU."""
@@ -200,7 +205,10 @@ def main():
         'hbm_frac_whole_step': value * total_bpn / 1e9 / HBM_PEAK_GBS,
         'roofline': {'bound': 'hbm', 'kernel': dom['kernel'], 'op': dom['op'],
                      'achieved': dom['achieved_GBps'], 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-                     'frac': dom['frac'], 'traffic': None},
+                     'frac': dom['frac'],
+                     'traffic': (nt * dom['bytes_per_nt'] * MEASURED_TRAFFIC_FACTOR[dom['kernel']]
+                                 if a.workload == 'cuba' else None),
+                     'traffic_unit': 'bytes per launch (rocprofv3 FETCH_SIZE x2 + WRITE_SIZE, see profiles/)'},
         'per_op': per_op,
     }
     if not a.no_cpu_baseline:

@@ -149,7 +149,7 @@ int slayer_cspike_bwd(float *grad_re, float *grad_im, const float *grad_spikes,
 
 /* ---- time shift --------------------------------------------------------------------------- */
 
-/* Replaces both shift() overloads (utils/time/shift.cu:80-210); semantics of _shift_group /
+/* Replaces both shift() overloads (utils/time/shift.cu:157-209, launchers :80-155); semantics of _shift_group /
  * _shift_individual (utils/time/shift.py:46-91).  out[m][t] = in[m][t - k] (zero outside [0,T)),
  * lut == NULL: every row moves by scalar_steps, the caller's int(shift / sampling_time) (python
  * double arithmetic, as _shift_group does); otherwise lut holds neurons_per_batch device floats and
@@ -159,11 +159,11 @@ int slayer_shift(float *out, const float *in, const float *lut, int64_t scalar_s
 
 /* ---- temporal filter ---------------------------------------------------------------------- */
 
-/* Replaces conv fwd (utils/filter/conv.cu:80-124): out[m][t] = Ts * sum_{i<K, t-i>=0} filt[i] * in[m][t-i]. */
+/* Replaces conv fwd (utils/filter/conv.cu:80-125): out[m][t] = Ts * sum_{i<K, t-i>=0} filt[i] * in[m][t-i]. */
 int slayer_conv(float *out, const float *in, const float *filt, int64_t K, float sampling_time,
                 int64_t M, int64_t T, void *stream);
 
-/* Replaces conv bwd (utils/filter/conv.cu:126-171): out[m][t] = Ts * sum_{i<K, t+i<T} filt[i] * in[m][t+i]. */
+/* Replaces conv bwd (utils/filter/conv.cu:127-172): out[m][t] = Ts * sum_{i<K, t+i<T} filt[i] * in[m][t+i]. */
 int slayer_corr(float *out, const float *in, const float *filt, int64_t K, float sampling_time,
                 int64_t M, int64_t T, void *stream);
 

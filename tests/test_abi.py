@@ -1,0 +1,94 @@
+"""Host-side checks that need no GPU: the C-ABI library loads, exports every symbol the header
+declares (and nothing the binding does not know), argument validation rejects bad sizes before any
+launch, and the python operators refuse CPU tensors."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, 'include', 'slayer_hip.h')
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+    return sorted(set(re.findall(r'\b(slayer_[a-z0-9_]+)\s*\(', text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from lava_dl_amd.slayer import _native
+    names = declared_symbols()
+    assert len(names) >= 14
+    handle = ctypes.CDLL(_native.LIB_PATH)
+    for n in names:
+        assert hasattr(handle, n), f'{n} declared in slayer_hip.h but not exported'
+    assert sorted(_native.EXPORTS) == names, 'python binding and header disagree'
+    assert _native.lib().slayer_abi_version() == 1
+    assert b'success' in _native.lib().slayer_error_string(0)
+    assert b'inconsistent' in _native.lib().slayer_error_string(-1)
+
+
+def test_argument_validation_happens_before_any_launch():
+    """Invalid sizes return SLAYER_E* without touching the device (safe without a GPU)."""
+    from lava_dl_amd.slayer import _native
+    L = _native.lib()
+    one = ctypes.c_void_p(16)          # non-null dummy pointers; never dereferenced on these paths
+    EINVAL, ENULL, ERANGE = -1, -2, -3
+    # M not a multiple of neurons_per_batch
+    assert L.slayer_li_fwd(one, one, one, one, 1.0, 64, 10, 3, 1, 1, 8, None) == EINVAL
+    # 3 decays do not divide 4 neurons per batch
+    assert L.slayer_li_fwd(one, one, one, one, 1.0, 64, 8, 4, 3, 1, 8, None) == EINVAL
+    # state count neither 1 nor M
+    assert L.slayer_li_fwd(one, one, one, one, 1.0, 64, 8, 4, 1, 5, 8, None) == EINVAL
+    assert L.slayer_li_fwd(one, one, one, one, 1.0, 0, 8, 4, 1, 1, 8, None) == EINVAL      # w_scale 0
+    assert L.slayer_li_fwd(None, one, one, one, 1.0, 64, 8, 4, 1, 1, 8, None) == ENULL
+    assert L.slayer_li_fwd(one, one, one, one, 1.0, 64, 8, 4, 1, 1, 1 << 31, None) == ERANGE
+    assert L.slayer_li_fwd(one, one, one, one, 1.0, 64, 0, 4, 1, 1, 8, None) == 0          # empty is fine
+    assert L.slayer_li_bwd(one, one, one, one, one, None, 8, 4, 1, 8, None) == ENULL       # grad wanted, no workspace
+    assert L.slayer_res_bwd(one, one, one, None, one, one, one, one, one, one, one, 8, 4, 1, 8, None) == ENULL
+    assert L.slayer_conv(one, one, one, 0, 1.0, 8, 8, None) == EINVAL
+    assert L.slayer_conv(one, one, one, 5000, 1.0, 8, 8, None) == ERANGE
+    assert L.slayer_shift(one, one, None, 1, 1.0, 8, 3, 8, None) == EINVAL
+    assert L.slayer_spike_fwd(one, one, one, 3, 0.0, 0, 1.0, 8, None) == EINVAL             # 3 thresholds for 8 samples
+    assert L.slayer_ath_fwd(one, one, one, one, one, one, one, 1 << 40, 0, 64, 8, 4, 1, 1, 1, 1, 8, None) == ERANGE
+
+
+def test_operators_refuse_cpu_tensors():
+    import lava_dl_amd.slayer as slayer
+    x = torch.zeros(2, 4, 16)
+    d = torch.tensor([100.0])
+    z = torch.tensor([0.0])
+    with pytest.raises(RuntimeError, match='no CPU implementation'):
+        slayer.neuron.dynamics.leaky_integrator.dynamics(x, d, z, 64)
+    with pytest.raises(RuntimeError):
+        slayer.neuron.dynamics.adaptive_threshold.dynamics(x, z, d, z, d, 0.5, 1.0, 64)
+    with pytest.raises(RuntimeError):
+        slayer.neuron.dynamics.resonator.dynamics(x, x, d, d, z, z, 64)
+    with pytest.raises(RuntimeError):
+        slayer.spike.Spike.apply(x, 1.0, 1.0, 1.0, False, 0, 1)
+    with pytest.raises(RuntimeError):
+        slayer.spike.complex.Spike.apply(x, x, 1.0, 1.0, 1.0, False, 0, 1)
+    with pytest.raises(RuntimeError):
+        slayer.utils.time.shift(x, 2)
+    with pytest.raises(RuntimeError):
+        slayer.utils.filter.conv(x, torch.ones(3))
+
+
+def test_product_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, 'lava-dl_amd')
+    for d, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith(('.py', '.hip', '.h')):
+                text = open(os.path.join(d, f)).read()
+                assert 'oracle' not in text, f'{f} mentions the oracle'
+
+
+def test_right_shift_to_zero():
+    import lava_dl_amd.slayer as slayer
+    x = torch.tensor([-8193, -4097, -4096, -4095, -1, 0, 1, 4095, 4096, 8191], dtype=torch.int64)
+    assert slayer.utils.int_utils.right_shift_to_zero(x, 12).tolist() == [-2, -1, -1, 0, 0, 0, 0, 0, 1, 1]
+    with pytest.raises(Exception):
+        slayer.utils.right_shift_to_zero(torch.zeros(2), 12)
