@@ -1,3 +1,3 @@
-from . import dynamics
+from . import dynamics, cuba, alif, rf
 
-__all__ = ['dynamics']
+__all__ = ['dynamics', 'cuba', 'alif', 'rf']

@@ -1,0 +1,68 @@
+"""Adaptive leaky integrate-and-fire neuron on the GPU dynamics kernels
+(counterpart of neuron/alif.py in the reference: call order :499-525, spike :557-591)."""
+import torch
+
+from .base import Neuron as _Base
+from .dynamics import leaky_integrator, adaptive_threshold
+from ..spike import Spike
+
+TAU_RHO_MULT = 100
+SCALE_RHO_MULT = 0.1
+
+
+class Neuron(_Base):
+    """``Neuron(threshold, threshold_step, current_decay, voltage_decay, threshold_decay,
+    refractory_decay, ...)``.  The voltage is not reset; a spike raises the threshold by
+    ``threshold_step`` and the refractory state by twice the threshold."""
+
+    def __init__(self, threshold, threshold_step, current_decay, voltage_decay, threshold_decay,
+                 refractory_decay, tau_grad=1, scale_grad=1, scale=1 << 6, norm=None, dropout=None,
+                 shared_param=True, persistent_state=False, requires_grad=False, graded_spike=False):
+        super().__init__(threshold, tau_grad, scale_grad, scale, norm, dropout, shared_param,
+                         persistent_state, requires_grad, graded_spike)
+        self.threshold_step = int(threshold_step * self.w_scale) / self.w_scale
+        self._register_decays(current_decay=current_decay, voltage_decay=voltage_decay,
+                              threshold_decay=threshold_decay, refractory_decay=refractory_decay)
+        self._register_states(current_state=0.0, voltage_state=0.0,
+                              threshold_state=lambda: self.threshold, refractory_state=0.0)
+        self.threshold_state.fill_(self.threshold)
+        self.clamp()
+
+    def dynamics(self, input):
+        """(current, voltage, threshold, refractory) traces."""
+        self._prepare(input)
+        if self.norm is not None:
+            input = self.norm(input)
+        current = leaky_integrator.dynamics(input, self._q('current_decay'), self.current_state.contiguous(),
+                                            self.s_scale, debug=self.debug)
+        voltage = leaky_integrator.dynamics(current, self._q('voltage_decay'), self.voltage_state.contiguous(),
+                                            self.s_scale, debug=self.debug)
+        threshold, refractory = adaptive_threshold.dynamics(
+            voltage, self.refractory_state.contiguous(), self._q('refractory_decay'),
+            self.threshold_state.contiguous(), self._q('threshold_decay'),
+            self.threshold_step, self.threshold, self.s_scale, debug=self.debug)
+        if self.persistent_state:
+            with torch.no_grad():
+                self.current_state = current[..., -1].clone()
+                self.voltage_state = voltage[..., -1].clone()
+                self.threshold_state = threshold[..., -1].clone()
+                self.refractory_state = refractory[..., -1].clone()
+        return current, voltage, threshold, refractory
+
+    def spike(self, voltage, threshold, refractory):
+        spike = Spike.apply(voltage, threshold + refractory, self.tau_rho * TAU_RHO_MULT,
+                            self.scale_rho * SCALE_RHO_MULT, self.graded_spike, self.voltage_state, 1)
+        if self.persistent_state:
+            with torch.no_grad():
+                last = spike[..., -1]
+                self.refractory_state = adaptive_threshold.persistent_ref_state(
+                    self.refractory_state, last, self.threshold_state).detach().clone()
+                self.threshold_state = adaptive_threshold.persistent_th_state(
+                    self.threshold_state, last, self.threshold_step).detach().clone()
+        if self.drop is not None:
+            spike = self.drop(spike)
+        return spike
+
+    def forward(self, input):
+        _, voltage, threshold, refractory = self.dynamics(input)
+        return self.spike(voltage, threshold, refractory)

@@ -1,0 +1,57 @@
+"""Current-based leaky integrate-and-fire neuron on the GPU dynamics kernels
+(counterpart of neuron/cuba.py in the reference: call order :356-374, spike :401-421)."""
+import torch
+
+from .base import Neuron as _Base
+from .dynamics import leaky_integrator
+from ..spike import Spike
+
+TAU_RHO_MULT = 100      # surrogate-gradient constants of the CUBA family (neuron/cuba.py:20-21)
+SCALE_RHO_MULT = 0.1
+
+
+class Neuron(_Base):
+    """``Neuron(threshold, current_decay, voltage_decay, ...)``; decays are fractions of 1
+    (stored times 4096), a [min, max] pair draws one value per channel when
+    ``shared_param=False``.  ``forward(x)`` returns the spike tensor."""
+
+    def __init__(self, threshold, current_decay, voltage_decay, tau_grad=1, scale_grad=1, scale=1 << 6,
+                 norm=None, dropout=None, shared_param=True, persistent_state=False, requires_grad=False,
+                 graded_spike=False):
+        super().__init__(threshold, tau_grad, scale_grad, scale, norm, dropout, shared_param,
+                         persistent_state, requires_grad, graded_spike)
+        # the dynamics spike at v >= threshold; hardware spikes at v > threshold
+        self.threshold_eps = 0.01 / self.s_scale
+        self._register_decays(current_decay=current_decay, voltage_decay=voltage_decay)
+        self._register_states(current_state=0.0, voltage_state=0.0)
+        self.clamp()
+
+    def dynamics(self, input):
+        """(current, voltage) traces; the voltage already carries the reset."""
+        self._prepare(input)
+        current = leaky_integrator.dynamics(input, self._q('current_decay'), self.current_state.contiguous(),
+                                            self.s_scale, debug=self.debug)
+        if self.norm is not None:
+            current = self.norm(current)
+        voltage = leaky_integrator.dynamics(current, self._q('voltage_decay'), self.voltage_state.contiguous(),
+                                            self.s_scale, self.threshold + self.threshold_eps, debug=self.debug)
+        if self.persistent_state:
+            with torch.no_grad():
+                self.current_state = current[..., -1].clone()
+                self.voltage_state = voltage[..., -1].clone()
+        return current, voltage
+
+    def spike(self, voltage):
+        spike = Spike.apply(voltage, self.threshold + self.threshold_eps, self.tau_rho * TAU_RHO_MULT,
+                            self.scale_rho * SCALE_RHO_MULT, self.graded_spike, self.voltage_state, 1)
+        if self.persistent_state:
+            with torch.no_grad():
+                self.voltage_state = leaky_integrator.persistent_state(
+                    self.voltage_state, spike[..., -1]).detach().clone()
+        if self.drop is not None:
+            spike = self.drop(spike)
+        return spike
+
+    def forward(self, input):
+        _, voltage = self.dynamics(input)
+        return self.spike(voltage)

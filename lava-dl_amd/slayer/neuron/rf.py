@@ -1,0 +1,104 @@
+"""Resonate-and-fire neuron on the GPU dynamics kernels
+(counterpart of neuron/rf.py in the reference: parameters :136-257, call order :429-471)."""
+import numpy as np
+import torch
+
+from .base import Neuron as _Base
+from .dynamics import resonator
+from ..spike import complex as complex_spike
+from ..utils.quantize import quantize
+
+TAU_RHO_MULT = 0.5      # surrogate-gradient constants of the RF family (neuron/rf.py:19-20)
+SCALE_RHO_MULT = 10
+
+
+class Neuron(_Base):
+    """``Neuron(threshold, period, decay, ...)``: the state rotates by 2 pi / period per step and
+    shrinks by (1 - decay); it spikes when the real part is above threshold while the imaginary
+    part crosses zero upwards.  ``forward((real_input, imag_input))`` returns the spikes."""
+
+    def __init__(self, threshold, period, decay, tau_grad=1, scale_grad=1, scale=1 << 6, norm=None,
+                 dropout=None, shared_param=True, persistent_state=False, requires_grad=False,
+                 graded_spike=False, log_init=True):
+        super().__init__(threshold, tau_grad, scale_grad, scale, None, dropout, shared_param,
+                         persistent_state, requires_grad, graded_spike)
+        self.real_norm = norm() if norm is not None else None
+        self.imag_norm = norm() if norm is not None else None
+        self.log_init = log_init
+
+        def check(p):
+            if p < 4:
+                raise AssertionError(f'Neuron period less than 4 does not make sense. Found period={p}.')
+
+        if shared_param:
+            if not np.isscalar(decay) or not np.isscalar(period):
+                raise AssertionError('Expected period and decay to be scalars when shared_param is True. '
+                                     f'Found {period=}, {decay=}.')
+            check(period)
+            start_p, start_d = period, decay
+        else:
+            pr = (period * 0.99, period * 1.01) if np.isscalar(period) else tuple(period)
+            dr = (decay * 0.99, decay * 1.01) if np.isscalar(decay) else tuple(decay)
+            if len(pr) != 2 or len(dr) != 2:
+                raise AssertionError(f'Expected [min, max] ranges. Found {period=}, {decay=}.')
+            check(period if np.isscalar(period) else min(period))
+            self._period_range, self._decay_range = pr, dr
+            start_p, start_d = pr[0], dr[0]
+        for name, fn in (('sin_decay', np.sin), ('cos_decay', np.cos)):
+            value = self.p_scale * fn(2 * np.pi / start_p) * (1 - start_d)
+            self.register_parameter(name, torch.nn.Parameter(torch.FloatTensor([value]),
+                                                             requires_grad=self.requires_grad))
+        self._register_states(real_state=0.0, imag_state=0.0)
+        self.clamp()
+
+    def clamp(self):
+        """Keep the gain below 1 (4095/4096), sin_decay >= 1 and cos_decay >= 0."""
+        with torch.no_grad():
+            gain = torch.sqrt(self.sin_decay ** 2 + self.cos_decay ** 2)
+            ratio = gain.clamp(0, self.p_scale - 1) / gain
+            self.sin_decay.data *= ratio
+            self.cos_decay.data *= ratio
+            self.sin_decay.data.clamp_(1)
+            self.cos_decay.data.clamp_(0)
+
+    def _draw_per_channel(self, channels, device):
+        (p_lo, p_hi), (d_lo, d_hi) = self._period_range, self._decay_range
+        if self.log_init:
+            frequency = torch.logspace(-np.log10(p_hi), -np.log10(p_lo), steps=channels).to(device)
+        else:
+            frequency = (1 / p_hi + (1 / p_lo - 1 / p_hi) * torch.rand(channels, dtype=torch.float)).to(device)
+        decay = d_lo + (d_hi - d_lo) * torch.rand(channels, dtype=torch.float).to(device)
+        self.sin_decay.data = self.p_scale * torch.sin(2 * np.pi * frequency) * (1 - decay)
+        self.cos_decay.data = self.p_scale * torch.cos(2 * np.pi * frequency) * (1 - decay)
+
+    def dynamics(self, input):
+        """(real, imag) traces for ``input = (real_input, imag_input)``."""
+        real_input, imag_input = input
+        if real_input.shape != imag_input.shape:
+            raise AssertionError(f'Real input tensor shape ({real_input.shape}) does not match '
+                                 f'with imaginary input shape ({imag_input.shape}).')
+        self._prepare(real_input)
+        if self.real_norm is not None:
+            real_input = self.real_norm(real_input)
+        if self.imag_norm is not None:
+            imag_input = self.imag_norm(imag_input)
+        real, imag = resonator.dynamics(real_input, imag_input, quantize(self.sin_decay), quantize(self.cos_decay),
+                                        self.real_state, self.imag_state, self.s_scale, debug=self.debug)
+        if self.persistent_state:
+            with torch.no_grad():
+                self.real_state = real[..., -1].clone()
+        return real, imag
+
+    def spike(self, real, imag):
+        spike = complex_spike.Spike.apply(real, imag, self.threshold, self.tau_rho * TAU_RHO_MULT,
+                                          self.scale_rho * SCALE_RHO_MULT, self.graded_spike, self.imag_state, 1)
+        if self.persistent_state:
+            with torch.no_grad():
+                self.imag_state = imag[..., -1].clone()
+        if self.drop is not None:
+            spike = self.drop(spike)
+        return spike
+
+    def forward(self, input):
+        real, imag = self.dynamics(input)
+        return self.spike(real, imag)

@@ -1,0 +1,30 @@
+"""Straight-through parameter quantiser (utils/quantize.py:18-94 in the reference)."""
+from enum import IntEnum, unique
+
+import torch
+
+
+@unique
+class MODE(IntEnum):
+    ROUND = 0
+    FLOOR = 1
+
+
+class _StraightThrough(torch.autograd.Function):
+    """Snap to a grid of ``step`` in the forward pass, identity in the backward pass."""
+
+    @staticmethod
+    def forward(ctx, input, step, use_floor):
+        scaled = input / step
+        return (torch.floor(scaled) if use_floor else torch.round(scaled)) * step
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return grad_output, None, None
+
+
+def quantize(input, step=1, mode=MODE.ROUND):
+    """Quantise ``input`` to multiples of ``step`` (round or floor); gradients pass through."""
+    if mode not in (MODE.ROUND, MODE.FLOOR):
+        raise ValueError(f'{mode=} is not recognized.')
+    return _StraightThrough.apply(input, step, mode == MODE.FLOOR)

@@ -1,0 +1,158 @@
+"""The thin CUBA / ALIF / RF neuron modules against the oracle's op chain, plus the invariants the
+reference's neuron tests assert (tests/lava/lib/dl/slayer/neuron/test_cuba.py:91-271 and siblings):
+batch consistency, integer states, persistent-state split invariance, backward runs."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import slayer_oracle as O
+from tests.util import dev, sparse_input, assert_exact, assert_rel
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope='module')
+def slayer():
+    import lava_dl_amd.slayer as s
+    return s
+
+
+def _oracle_cuba(x, cd, vd, thr, s_scale, tau, rho, cs=None, vs=None):
+    zero = torch.tensor([0.0])
+    cur = O.li_fwd(x, cd, zero if cs is None else cs, s_scale)
+    vol = O.li_fwd(cur, vd, zero if vs is None else vs, s_scale, thr)
+    return cur, vol, O.spike_fwd(vol, thr)
+
+
+def test_cuba_neuron_matches_oracle_chain(slayer):
+    gen = torch.Generator().manual_seed(100)
+    x = sparse_input(gen, (2, 6, 5, 80), p=0.2, amp=1.0)
+    n = slayer.neuron.cuba.Neuron(threshold=1.0, current_decay=0.25, voltage_decay=0.03,
+                                  tau_grad=1, scale_grad=1, requires_grad=True).to(dev())
+    xg = x.to(dev()).requires_grad_()
+    cur, vol = n.dynamics(xg)
+    spk = n.spike(vol)
+    thr = 1.0 + 0.01 / 4096
+    cd, vd = torch.tensor([1024.0]), torch.tensor([round(0.03 * 4096) * 1.0])
+    r_cur, r_vol, r_spk = _oracle_cuba(x, cd, vd, thr, 4096, 100.0, 0.1)
+    assert_exact(cur, r_cur, 'cuba current')
+    assert_exact(vol, r_vol, 'cuba voltage')
+    assert_exact(spk, r_spk, 'cuba spikes')
+    assert r_spk.sum() > 0
+    g = torch.randn(x.shape, generator=gen)
+    spk.backward(g.to(dev()))
+    r_gv = O.spike_bwd(g, r_vol, thr, 1.0 * 100, 1 * 0.1)
+    r_gc, r_gvd = O.li_bwd(r_gv, r_vol, vd)
+    r_gx, r_gcd = O.li_bwd(r_gc, r_cur, cd)
+    assert_rel(xg.grad, r_gx, 'cuba grad_input')
+    assert_rel(n.voltage_decay.grad, r_gvd, 'cuba grad voltage_decay', rel=1e-4)
+    assert_rel(n.current_decay.grad, r_gcd, 'cuba grad current_decay', rel=1e-4)
+    # integer states at the state scale, identical batch entries give identical outputs
+    assert torch.equal(torch.floor(vol * 4096), vol * 4096)
+    xb = x[:1].repeat(3, 1, 1, 1).to(dev())
+    n2 = slayer.neuron.cuba.Neuron(1.0, 0.25, 0.03).to(dev())
+    assert float(n2(xb).var(dim=0).max()) == 0.0
+
+
+@pytest.mark.parametrize('kind', ['cuba', 'alif', 'rf'])
+@pytest.mark.parametrize('shared', [True, False])
+def test_persistent_state_split_invariance(slayer, kind, shared):
+    """Running [:k] then [k:] with carried state equals the full run, for every trace and the spikes."""
+    gen = torch.Generator().manual_seed(101)
+    shape, k = (3, 8, 120), 47
+    torch.manual_seed(5)
+    if kind == 'cuba':
+        mk = lambda p: slayer.neuron.cuba.Neuron(1.0, [0.2, 0.4] if not shared else 0.25,
+                                                 [0.02, 0.2] if not shared else 0.03,
+                                                 shared_param=shared, persistent_state=p).to(dev())
+        x = sparse_input(gen, shape, p=0.3).to(dev())
+        run = lambda n, inp: (lambda cv: (cv[0], cv[1], n.spike(cv[1])))(n.dynamics(inp))
+    elif kind == 'alif':
+        rng = lambda a, b: [a, b] if not shared else a
+        mk = lambda p: slayer.neuron.alif.Neuron(1.0, 0.5, rng(0.25, 0.4), rng(0.03, 0.2), rng(0.1, 0.3),
+                                                 rng(0.1, 0.3), shared_param=shared, persistent_state=p).to(dev())
+        x = sparse_input(gen, shape, p=0.4, amp=2.0).to(dev())
+        run = lambda n, inp: (lambda t: t + (n.spike(t[1], t[2], t[3]),))(n.dynamics(inp))
+    else:
+        mk = lambda p: slayer.neuron.rf.Neuron(1.0, [5, 20] if not shared else 11,
+                                               [0.02, 0.1] if not shared else 0.05,
+                                               shared_param=shared, persistent_state=p).to(dev())
+        x = (sparse_input(gen, shape, p=0.3).to(dev()), sparse_input(gen, shape, p=0.3).to(dev()))
+        run = lambda n, inp: (lambda t: t + (n.spike(t[0], t[1]),))(n.dynamics(inp))
+    cut = (lambda a, b: tuple(t[..., a:b] for t in x)) if kind == 'rf' else (lambda a, b: x[..., a:b])
+    full_n, split_n = mk(False), mk(True)
+    full = run(full_n, x)
+    # same parameters in both modules
+    split_n._prepare(x[0] if kind == 'rf' else x)
+    for (na, pa), (nb, pb) in zip(full_n.named_parameters(), split_n.named_parameters()):
+        pb.data = pa.data.clone()
+    a = run(split_n, cut(0, k))
+    b = run(split_n, cut(k, shape[-1]))
+    assert sum(float(t.sum()) for t in (full[-1],)) > 0, 'no spikes in the test workload'
+    for i, (f, pa, pb) in enumerate(zip(full, a, b)):
+        assert torch.equal(torch.cat([pa, pb], dim=-1), f), f'{kind} trace {i} differs after the split'
+
+
+def test_alif_neuron_matches_oracle_chain(slayer):
+    gen = torch.Generator().manual_seed(102)
+    x = sparse_input(gen, (2, 12, 150), p=0.4, amp=2.0)
+    n = slayer.neuron.alif.Neuron(threshold=1.0, threshold_step=0.5, current_decay=0.25, voltage_decay=0.1,
+                                  threshold_decay=0.05, refractory_decay=0.2).to(dev())
+    xg = x.to(dev()).requires_grad_()
+    cur, vol, th, ref = n.dynamics(xg)
+    spk = n.spike(vol, th, ref)
+    one, zero = torch.tensor([1.0]), torch.tensor([0.0])
+    q = lambda v: torch.tensor([float(round(v * 4096))])
+    r_cur = O.li_fwd(x, q(0.25), zero, 4096)
+    r_vol = O.li_fwd(r_cur, q(0.1), zero, 4096)
+    r_th, r_ref = O.ath_fwd(r_vol, zero, q(0.2), one, q(0.05), 0.5, 1.0, 4096)
+    r_spk = O.spike_fwd(r_vol, r_th + r_ref)
+    for got, ref_t, name in ((cur, r_cur, 'current'), (vol, r_vol, 'voltage'), (th, r_th, 'threshold'),
+                             (ref, r_ref, 'refractory'), (spk, r_spk, 'spikes')):
+        assert_exact(got, ref_t, f'alif {name}')
+    assert r_spk.sum() > 0
+    g = torch.randn(x.shape, generator=gen)
+    spk.backward(g.to(dev()))
+    r_gv = O.spike_bwd(g, r_vol, r_th + r_ref, 100.0, 0.1)
+    r_gc, _ = O.li_bwd(r_gv, r_vol, q(0.1))
+    r_gx, _ = O.li_bwd(r_gc, r_cur, q(0.25))
+    assert_rel(xg.grad, r_gx, 'alif grad_input')
+
+
+def test_rf_neuron_matches_oracle_chain(slayer):
+    gen = torch.Generator().manual_seed(103)
+    shape = (2, 10, 200)
+    xr, xi = sparse_input(gen, shape, p=0.3), sparse_input(gen, shape, p=0.3)
+    n = slayer.neuron.rf.Neuron(threshold=1.0, period=11, decay=0.05).to(dev())
+    rg, ig = xr.to(dev()).requires_grad_(), xi.to(dev()).requires_grad_()
+    re, im = n.dynamics((rg, ig))
+    spk = n.spike(re, im)
+    sin = torch.round(n.sin_decay.detach().cpu())
+    cos = torch.round(n.cos_decay.detach().cpu())
+    assert (sin.item(), cos.item()) == (2104.0, 3273.0)
+    zero = torch.tensor([0.0])
+    r_re, r_im = O.res_fwd(xr, xi, sin, cos, zero, zero, 4096)
+    r_spk = O.cspike_fwd(r_re, r_im, 1.0, 0.0)
+    assert_exact(re, r_re, 'rf real')
+    assert_exact(im, r_im, 'rf imag')
+    assert_exact(spk, r_spk, 'rf spikes')
+    assert r_spk.sum() > 0
+    g = torch.randn(shape, generator=gen)
+    spk.backward(g.to(dev()))
+    g_re, g_im = O.cspike_bwd(g, r_re, r_im, 1.0, 0.5, 10.0)
+    r_gr, r_gi, _, _ = O.res_bwd(g_re, g_im, r_re, r_im, sin, cos)
+    assert_rel(rg.grad, r_gr, 'rf grad real input')
+    assert_rel(ig.grad, r_gi, 'rf grad imag input')
+
+
+def test_neuron_shape_checks(slayer):
+    n = slayer.neuron.cuba.Neuron(1.0, 0.25, 0.03).to(dev())
+    with pytest.raises(AssertionError):
+        n(torch.zeros(4, 10, device=dev()))
+    n(torch.zeros(2, 3, 10, device=dev()))
+    with pytest.raises(AssertionError):
+        n(torch.zeros(2, 4, 10, device=dev()))
+    with pytest.raises(AssertionError):
+        slayer.neuron.cuba.Neuron(1.0, [0.1, 0.2], 0.03)
+    with pytest.raises(AssertionError):
+        slayer.neuron.rf.Neuron(1.0, 3, 0.05)
