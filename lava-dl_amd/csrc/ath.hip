@@ -8,6 +8,7 @@ template <bool POW2>
 struct AthFwd {
     static constexpr int kIn = 1, kOut = 2;      // out: threshold trace, refractory trace
     static constexpr bool kReverse = false;
+    static constexpr int64_t kRows32Below = 65536, kRows16Below = 16384;
     struct Params {
         const float* in[1];
         float* out[2];
@@ -69,10 +70,10 @@ extern "C" int slayer_ath_fwd(float* th_out, float* ref_out, const float* in,
         AthFwd<true>::Params p{{in}, {th_out, ref_out}, ref_state, ref_decay, th_state, th_decay,
                                (int)th_step_scaled, (int)th0_scaled, w, 1.0f / w, neurons_per_batch,
                                num_ref_decays, num_th_decays, num_ref_states, num_th_states};
-        return launch_stream<AthFwd<true>, 32>(p, M, T, (hipStream_t)stream);
+        return launch_stream<AthFwd<true>>(p, M, T, (hipStream_t)stream);
     }
     AthFwd<false>::Params p{{in}, {th_out, ref_out}, ref_state, ref_decay, th_state, th_decay,
                             (int)th_step_scaled, (int)th0_scaled, w, 1.0f / w, neurons_per_batch,
                             num_ref_decays, num_th_decays, num_ref_states, num_th_states};
-    return launch_stream<AthFwd<false>, 32>(p, M, T, (hipStream_t)stream);
+    return launch_stream<AthFwd<false>>(p, M, T, (hipStream_t)stream);
 }

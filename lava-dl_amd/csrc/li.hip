@@ -2,14 +2,6 @@
 #include "common.h"
 #include "tile.h"
 
-// time-chunk lengths (steps per LDS tile); overridable for tuning builds
-#ifndef SLAYER_TC_LI_FWD
-#define SLAYER_TC_LI_FWD 32
-#endif
-#ifndef SLAYER_TC_LI_BWD
-#define SLAYER_TC_LI_BWD 32
-#endif
-
 namespace slayer {
 
 // ---------------------------------------------------------------------------------- forward
@@ -17,6 +9,7 @@ template <bool POW2>
 struct LiFwd {
     static constexpr int kIn = 1, kOut = 1;
     static constexpr bool kReverse = false;
+    static constexpr int64_t kRows32Below = kAlways, kRows16Below = 65536;
     struct Params {
         const float* in[1];
         float* out[1];
@@ -49,6 +42,7 @@ struct LiFwd {
 struct LiBwd {
     static constexpr int kIn = 2, kOut = 1;     // in: grad_out, saved forward output
     static constexpr bool kReverse = true;
+    static constexpr int64_t kRows32Below = kAlways, kRows16Below = kAlways;
     struct Params {
         const float* in[2];
         float* out[1];
@@ -164,10 +158,10 @@ extern "C" int slayer_li_fwd(float* out, const float* in, const float* decay, co
     const float thr = thr_scaled > 0 ? (float)thr_scaled : __builtin_inff();
     if (is_pow2(w_scale)) {
         LiFwd<true>::Params p{{in}, {out}, decay, state, w, 1.0f / w, thr, neurons_per_batch, num_decays, num_states};
-        return launch_stream<LiFwd<true>, SLAYER_TC_LI_FWD>(p, M, T, (hipStream_t)stream);
+        return launch_stream<LiFwd<true>>(p, M, T, (hipStream_t)stream);
     }
     LiFwd<false>::Params p{{in}, {out}, decay, state, w, 1.0f / w, thr, neurons_per_batch, num_decays, num_states};
-    return launch_stream<LiFwd<false>, SLAYER_TC_LI_FWD>(p, M, T, (hipStream_t)stream);
+    return launch_stream<LiFwd<false>>(p, M, T, (hipStream_t)stream);
 }
 
 extern "C" int slayer_li_bwd(float* grad_in, float* grad_decay, const float* grad_out, const float* out,
@@ -181,7 +175,7 @@ extern "C" int slayer_li_bwd(float* grad_in, float* grad_decay, const float* gra
         if (!grad_in || !grad_out || !out || !decay) return SLAYER_ENULL;
         LiBwd::Params p{{grad_out, out}, {grad_in}, decay, grad_decay ? workspace : nullptr,
                         neurons_per_batch, num_decays};
-        if (int e = launch_stream<LiBwd, SLAYER_TC_LI_BWD>(p, M, T, (hipStream_t)stream)) return e;
+        if (int e = launch_stream<LiBwd>(p, M, T, (hipStream_t)stream)) return e;
     }
     if (grad_decay) {
         if (M == 0 || T == 0) return launch_zero_fill(grad_decay, num_decays, (hipStream_t)stream);

@@ -12,6 +12,7 @@ template <bool POW2, bool HAS_THR>
 struct ResFwd {
     static constexpr int kIn = 2, kOut = 2;
     static constexpr bool kReverse = false;
+    static constexpr int64_t kRows32Below = 65536, kRows16Below = 16384;
     struct Params {
         const float* in[2];
         float* out[2];
@@ -57,6 +58,7 @@ struct ResFwd {
 struct ResBwd {
     static constexpr int kIn = 4, kOut = 2;      // in: g_re, g_im, saved re, saved im
     static constexpr bool kReverse = true;
+    static constexpr int64_t kRows32Below = 262144, kRows16Below = 262144;
     struct Params {
         const float* in[4];
         float* out[2];
@@ -101,7 +103,7 @@ static int res_fwd_launch(float* re_out, float* im_out, const float* re_in, cons
     using Op = ResFwd<POW2, HAS_THR>;
     typename Op::Params p{{re_in, im_in}, {re_out, im_out}, sin_decay, cos_decay, re_state, im_state,
                           w, 1.0f / w, thr, im_reset, npb, nd, n_rs, n_is};
-    return launch_stream<Op, 32>(p, M, T, stream);
+    return launch_stream<Op>(p, M, T, stream);
 }
 
 extern "C" int slayer_res_fwd(float* re_out, float* im_out, const float* re_in, const float* im_in,
@@ -148,7 +150,7 @@ extern "C" int slayer_res_bwd(float* g_re_in, float* g_im_in, float* grad_sin, f
         ResBwd::Params p{{g_re, g_im, re, im}, {g_re_in, g_im_in}, sin_decay, cos_decay,
                          want ? workspace : nullptr, want ? workspace + M : nullptr,
                          neurons_per_batch, num_decays};
-        if (int e = launch_stream<ResBwd, 32>(p, M, T, st)) return e;
+        if (int e = launch_stream<ResBwd>(p, M, T, st)) return e;
     }
     if (want) {
         if (M == 0 || T == 0) {

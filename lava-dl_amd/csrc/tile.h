@@ -2,7 +2,7 @@
 //
 // Tensors are [M][T] float32 with time innermost.  One 64-lane wavefront (one
 // workgroup) owns 64 consecutive neurons (rows) and walks the time axis in chunks
-// of TC steps:
+// of TC steps (TC = 32 for 64 rows):
 //
 //   global --dwordx4, coalesced along time--> registers --ds_write_b128--> LDS tile
 //   LDS tile: lane j runs the recurrence over row j, 4 steps per ds_read_b128,
@@ -56,18 +56,27 @@ __device__ __forceinline__ int64_t param_index(int64_t m, int64_t npb, int64_t n
     return num_params > 1 ? (m % npb) / (npb / num_params) : 0;
 }
 
-template <int TC>
+// A tile is R rows x TC steps with R * TC = 2048 samples (8 KB per tensor): R = 64 rows when
+// there are plenty of neurons, fewer rows and longer chunks when there are few, so that small
+// problems still spread over all compute units (lanes >= R only help with the copies).
+constexpr int kTileSamples = 2048;
+
+template <int R>
 struct TileGeom {
-    static_assert(TC % 4 == 0 && TC >= 4 && TC <= 256 && (kWave * 4) % TC == 0, "bad chunk");
-    static constexpr int kPitch = TC + 4;               // floats per LDS row
-    static constexpr int kQuads = TC / 4;               // float4 per row
-    static constexpr int kRowsPerPass = kWave / kQuads; // rows one wave-wide access covers
-    static constexpr int kPasses = kWave / kRowsPerPass;
-    static constexpr int kTileFloats = kWave * kPitch;
+    static constexpr int kRows = R;
+    static constexpr int kChunk = kTileSamples / R;          // TC: steps per chunk
+    static_assert(R == 64 || R == 32 || R == 16, "rows per wave");
+    static constexpr int kPitch = kChunk + 4;                // floats per LDS row
+    static constexpr int kQuads = kChunk / 4;                // float4 per row
+    static constexpr int kRowsPerPass = kWave / kQuads;      // rows one wave-wide access covers
+    static constexpr int kPasses = R / kRowsPerPass;
+    static_assert(kRowsPerPass >= 1 && kPasses >= 1, "tile geometry");
+    static constexpr int kTileFloats = R * kPitch;
 };
 
 // An Op provides:
 //   static constexpr int kIn, kOut;  static constexpr bool kReverse;
+//   static constexpr int64_t kRows32Below, kRows16Below;   (rows-per-wave policy, see launch_stream)
 //   struct Params { const float* in[kIn]; float* out[kOut]; ... };
 //   __device__ void init(const Params&, int64_t m, bool valid);
 //   __device__ void step(const float (&x)[kIn], float (&y)[kOut]);
@@ -86,16 +95,17 @@ struct TileGeom {
 // output quads that fall in such a shared line are collected in an LDS buffer of 65 lines
 // (one per row boundary of the wave) and written once, whole, after the last chunk.  Only
 // the two lines shared with neighbouring workgroups are still written in pieces.
-template <class Op, int TC, bool VEC4, bool STREAM>
+template <class Op, int R, bool VEC4, bool STREAM>
 __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, int64_t M, int T) {
-    using G = TileGeom<TC>;
+    using G = TileGeom<R>;
+    constexpr int TC = G::kChunk;
     constexpr int NI = Op::kIn, NO = Op::kOut, NT = NI > NO ? NI : NO;
     __shared__ __attribute__((aligned(16))) float tile[NT][G::kTileFloats];
-    __shared__ __attribute__((aligned(16))) float bline[VEC4 ? NO : 1][VEC4 ? (kWave + 1) * 32 : 4];
+    __shared__ __attribute__((aligned(16))) float bline[VEC4 ? NO : 1][VEC4 ? (R + 1) * 32 : 4];
 
     const int lane = threadIdx.x;
-    const int64_t m0 = (int64_t)blockIdx.x * kWave;
-    const int rows = (int)((M - m0) < kWave ? (M - m0) : kWave);
+    const int64_t m0 = (int64_t)blockIdx.x * R;
+    const int rows = (int)((M - m0) < R ? (M - m0) : R);
 
     Op op;
     op.init(prm, m0 + lane, lane < rows);
@@ -171,7 +181,7 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
         for (int q = 0; q < G::kQuads; ++q) {
             const int qq = Op::kReverse ? G::kQuads - 1 - q : q;
             const int t = tl + 4 * qq;
-            if (t >= 0 && t < T) {
+            if (lane < R && t >= 0 && t < T) {
                 float xin[NI][4], yout[NO][4];
 #pragma unroll
                 for (int i = 0; i < NI; ++i) {
@@ -234,7 +244,7 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
 
     if (route) {
         // boundary line b holds the tail of row b-1 (columns < phase(b)) and the head of row b
-        for (int i = lane; i < (kWave + 1) * 8; i += kWave) {
+        for (int i = lane; i < (R + 1) * 8; i += kWave) {
             const int b = i >> 3, col = (i & 7) * 4;
             const int a = phase(b);
             const bool owned = (col < a) ? (b >= 1 && b - 1 < rows) : (b < rows);
@@ -251,23 +261,41 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// Launch helper: picks the dwordx4 path when T and every pointer allow it, and non-temporal
-// global accesses when the tensors are too large to be reused out of the last-level cache.
-template <class Op, int TC>
+// Launch helper: picks the dwordx4 path when T and every pointer allow it, non-temporal global
+// accesses when the tensors are too large to be reused out of the last-level cache, and the
+// rows-per-wave geometry from the number of neurons.
+template <class Op, int R>
+int launch_stream_rows(const typename Op::Params& prm, int64_t M, int64_t T, bool vec, bool streaming,
+                       hipStream_t stream) {
+    const dim3 grid((unsigned)((M + R - 1) / R)), block(kWave);
+    if (!vec)
+        hipLaunchKernelGGL((stream_kernel<Op, R, false, false>), grid, block, 0, stream, prm, M, (int)T);
+    else if (streaming)
+        hipLaunchKernelGGL((stream_kernel<Op, R, true, true>), grid, block, 0, stream, prm, M, (int)T);
+    else
+        hipLaunchKernelGGL((stream_kernel<Op, R, true, false>), grid, block, 0, stream, prm, M, (int)T);
+    return (int)hipGetLastError();
+}
+
+// Rows per wave.  An Op states below how many neurons it wants 32 and 16 rows per wave
+// (kRows32Below, kRows16Below; measured on MI355X): arithmetic-heavy forward recurrences keep all
+// 64 lanes busy until the problem gets small, the light float backward passes prefer 16 rows
+// and 512-byte row segments at every size.
+constexpr int64_t kAlways = (int64_t)1 << 62;
+
+template <class Op>
 int launch_stream(const typename Op::Params& prm, int64_t M, int64_t T, hipStream_t stream) {
     if (M == 0 || T == 0) return 0;
     bool vec = (T % 4) == 0;
     for (int i = 0; i < Op::kIn; ++i) vec = vec && aligned16(prm.in[i]);
     for (int o = 0; o < Op::kOut; ++o) vec = vec && aligned16(prm.out[o]);
     const bool streaming = M * T * 4 > ((int64_t)64 << 20);
-    const dim3 grid((unsigned)((M + kWave - 1) / kWave)), block(kWave);
-    if (!vec)
-        hipLaunchKernelGGL((stream_kernel<Op, TC, false, false>), grid, block, 0, stream, prm, M, (int)T);
-    else if (streaming)
-        hipLaunchKernelGGL((stream_kernel<Op, TC, true, true>), grid, block, 0, stream, prm, M, (int)T);
-    else
-        hipLaunchKernelGGL((stream_kernel<Op, TC, true, false>), grid, block, 0, stream, prm, M, (int)T);
-    return (int)hipGetLastError();
+    if (M < Op::kRows16Below) return launch_stream_rows<Op, 16>(prm, M, T, vec, streaming, stream);
+    if constexpr (Op::kRows16Below < kAlways && Op::kRows16Below < Op::kRows32Below)
+        if (M < Op::kRows32Below) return launch_stream_rows<Op, 32>(prm, M, T, vec, streaming, stream);
+    if constexpr (Op::kRows32Below < kAlways)
+        return launch_stream_rows<Op, 64>(prm, M, T, vec, streaming, stream);
+    return 0;   // not reached: every neuron count is covered by the branches above
 }
 
 }  // namespace slayer

@@ -59,6 +59,47 @@ def test_li_fwd_bit_exact(slayer, shape, kind, w, thr, state_kind):
     assert_exact(out, ref, f'li_fwd {shape}')
 
 
+@pytest.mark.parametrize('M_per_batch', [70000, 35000, 9000, 2000])
+def test_all_tile_geometries(slayer, M_per_batch):
+    """Each kernel picks 64, 32 or 16 rows per wave from the neuron count (thresholds at 262144, 65536 and
+    16384 neurons depending on the kernel); every geometry must give the same bits.  The four sizes
+    here (280000, 140000, 36000, 8000 neurons) reach every instantiation."""
+    N, T = 4, 100
+    shape = (N, M_per_batch, T)
+    gen = torch.Generator().manual_seed(seed_of(shape))
+    x = sparse_input(gen, shape, p=0.1, amp=2.0)
+    d1 = torch.randint(0, 4097, (M_per_batch,), generator=gen).float()
+    d2 = torch.randint(0, 4097, (M_per_batch,), generator=gen).float()
+    zero, one = torch.tensor([0.0]), torch.tensor([1.0])
+    xg, d1g, d2g, zg, og = x.to(dev()), d1.to(dev()), d2.to(dev()), zero.to(dev()), one.to(dev())
+    D = slayer.neuron.dynamics
+    ref = O.li_fwd(x, d1, zero, 64, 1.0)
+    out = D.leaky_integrator.dynamics(xg, d1g, zg, 64, 1.0)
+    assert_exact(out, ref, 'li_fwd')
+    g = torch.randn(shape, generator=gen)
+    from lava_dl_amd.slayer.neuron.dynamics import leaky_integrator as L, resonator as R
+    gi, gd = L._bwd(g.to(dev()), out, d1g)
+    r_gi, r_gd = O.li_bwd(g, ref, d1)
+    assert_exact(gi, r_gi, 'li_bwd grad_input')
+    assert_rel(gd, r_gd, 'li_bwd grad_decay', rel=1e-4)
+    th, rf = D.adaptive_threshold.dynamics(xg, zg, d1g, og, d2g, 0.5, 1.0, 64)
+    r_th, r_rf = O.ath_fwd(x, zero, d1, one, d2, 0.5, 1.0, 64)
+    assert_exact(th, r_th, 'ath threshold')
+    assert_exact(rf, r_rf, 'ath refractory')
+    x2 = sparse_input(gen, shape, p=0.1, amp=2.0)
+    sin, cos = (d1 * 0.6).round(), (d2 * 0.7).round()
+    re, im = D.resonator.dynamics(xg, x2.to(dev()), sin.to(dev()), cos.to(dev()), zg, zg, 64)
+    r_re, r_im = O.res_fwd(x, x2, sin, cos, zero, zero, 64)
+    assert_exact(re, r_re, 'res real')
+    assert_exact(im, r_im, 'res imag')
+    got = R._bwd(g.to(dev()), xg, re, im, sin.to(dev()), cos.to(dev()))
+    want = O.res_bwd(g, x, r_re, r_im, sin, cos)
+    assert_exact(got[0], want[0], 'res_bwd grad_real')
+    assert_exact(got[1], want[1], 'res_bwd grad_imag')
+    assert_rel(got[2], want[2], 'res_bwd grad_sin', rel=1e-4)
+    assert_rel(got[3], want[3], 'res_bwd grad_cos', rel=1e-4)
+
+
 def test_li_fwd_negative_and_edge_decays(slayer):
     gen = torch.Generator().manual_seed(7)
     x = sparse_input(gen, (2, 8, 96), p=0.5, amp=30.0)
