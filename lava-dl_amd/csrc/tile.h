@@ -81,27 +81,57 @@ struct TileGeom {
 //   __device__ void init(const Params&, int64_t m, bool valid);
 //   __device__ void step(const float (&x)[kIn], float (&y)[kOut]);
 //   __device__ void finish(const Params&, int64_t m, bool valid);
+
+// ---------------------------------------------------------------------------------------------
+// Buffer addressing.  Global accesses of the dwordx4 path go through raw buffer instructions whose
+// descriptor covers exactly the rows of this wave: a lane that must not touch memory (column
+// outside [0, T), row beyond the tensor) gets an offset past the end, for which the hardware
+// returns zero / drops the store.  There are no branches around memory instructions, so their
+// count per chunk is static and the loads of chunk k+1 can be waited for with an exact vmcnt
+// while the stores of chunk k are still in flight.
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+constexpr int kOutOfRange = (int)0x80000000;
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const float* base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, (int)bytes, 0x00020000);
+}
+template <bool STREAM>
+__device__ __forceinline__ float4 buf_load4(__amdgpu_buffer_rsrc_t r, int byte_off) {
+    const v4u v = __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, STREAM ? 2 : 0);
+    return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
+}
+template <bool STREAM>
+__device__ __forceinline__ void buf_store4(__amdgpu_buffer_rsrc_t r, int byte_off, float4 f) {
+    v4u v;
+    v.x = __float_as_uint(f.x); v.y = __float_as_uint(f.y); v.z = __float_as_uint(f.z); v.w = __float_as_uint(f.w);
+    __builtin_amdgcn_raw_buffer_store_b128(v, r, byte_off, 0, STREAM ? 2 : 0);
+}
+
+// ---------------------------------------------------------------------------------------------
+// dwordx4 kernel (T % 4 == 0, 16-byte aligned bases).
 //
-// Line alignment (VEC4 path).  A row of T floats starts wherever m*T falls, so a fixed
-// time grid would cut every row segment across 128-byte lines and each line would be
-// fetched (and partially written) twice.  Instead every row gets its own phase
-// a = (float index of the row start) mod 32 and tile column j of chunk k holds step
-// t = k*TC + j - a: the segments a wave-wide access touches then start on 128-byte
-// boundaries.  Lanes simply skip the columns that fall before step 0 or after step T-1.
+// Line alignment.  A row of T floats starts wherever m*T falls, so a fixed time grid would cut
+// every row segment across 128-byte lines and each line would be fetched (and partially written)
+// twice.  Instead every row gets its own phase a = (float index of the row start) mod 32 and tile
+// column j of chunk k holds step t = k*TC + j - a: the segments a wave-wide access touches then
+// start on 128-byte boundaries.  Lanes skip the columns that fall before step 0 or after T-1.
 //
-// Boundary lines (VEC4 path).  Unless T is a multiple of 32, the last line of row r is also
-// the first line of row r+1.  Writing it in two pieces at two different times costs a
-// read-modify-write in memory for each piece (measured: ~16% of the kernel at T = 300), so
-// output quads that fall in such a shared line are collected in an LDS buffer of 65 lines
-// (one per row boundary of the wave) and written once, whole, after the last chunk.  Only
-// the two lines shared with neighbouring workgroups are still written in pieces.
-template <class Op, int R, bool VEC4, bool STREAM>
+// Boundary lines.  Unless T is a multiple of 32, the last line of row r is also the first line of
+// row r+1.  Writing it in two pieces at two different times costs a read-modify-write in memory
+// for each piece (measured: ~16% of the kernel at T = 300), so output quads that fall in such a
+// shared line are collected in an LDS buffer of R+1 lines (one per row boundary of the wave) and
+// written once, whole, after the last chunk.  Only the two lines shared with neighbouring
+// workgroups are still written in pieces.
+//
+// Interior chunks (every column of every row inside [0, T), no shared line) run a branch-free
+// recurrence loop; only the first and the last one or two chunks take the predicated path.
+template <class Op, int R, bool STREAM>
 __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, int64_t M, int T) {
     using G = TileGeom<R>;
     constexpr int TC = G::kChunk;
     constexpr int NI = Op::kIn, NO = Op::kOut, NT = NI > NO ? NI : NO;
     __shared__ __attribute__((aligned(16))) float tile[NT][G::kTileFloats];
-    __shared__ __attribute__((aligned(16))) float bline[VEC4 ? NO : 1][VEC4 ? (R + 1) * 32 : 4];
+    __shared__ __attribute__((aligned(16))) float bline[NO][(R + 1) * 32];
 
     const int lane = threadIdx.x;
     const int64_t m0 = (int64_t)blockIdx.x * R;
@@ -110,11 +140,16 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
     Op op;
     op.init(prm, m0 + lane, lane < rows);
 
+    __amdgpu_buffer_rsrc_t src[NI], dst[NO];
+    const unsigned wave_bytes = (unsigned)rows * (unsigned)T * 4u;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) src[i] = make_rsrc(prm.in[i] + m0 * (int64_t)T, wave_bytes);
+#pragma unroll
+    for (int o = 0; o < NO; ++o) dst[o] = make_rsrc(prm.out[o] + m0 * (int64_t)T, wave_bytes);
+
     // phase of a row: float index of its first sample modulo one 128-byte line
     const unsigned base_f = (unsigned)(reinterpret_cast<uintptr_t>(prm.in[0]) >> 2);
-    auto phase = [&](int r) -> int {
-        return VEC4 ? (int)((base_f + (unsigned)(m0 + r) * (unsigned)T) & 31u) : 0;
-    };
+    auto phase = [&](int r) -> int { return (int)((base_f + (unsigned)(m0 + r) * (unsigned)T) & 31u); };
     const int a_lane = phase(lane);
 
     int last = (lane < rows) ? (a_lane + T - 1) / TC : 0;    // last chunk this row needs
@@ -124,44 +159,72 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
         last = o > last ? o : last;
     }
     const int nchunks = last + 1;
-
+    // chunks [1, interior_end) hold only valid columns and touch no shared line, for every phase
+    const int interior_end = (T & ~31) / TC;
     // rows shorter than a line could start and end inside the same line; they keep direct stores
-    const bool route = VEC4 && T >= 32;
+    const bool route = T >= 32;
 
     const int crow = lane / G::kQuads;      // row within a pass (copy pattern)
     const int cq = lane % G::kQuads;        // quad within the row
+
+    // copy pattern, per pass: step of this lane's quad in chunk 0 and its byte offset in the wave's rows
+    int step0[G::kPasses], off0[G::kPasses];
+#pragma unroll
+    for (int p = 0; p < G::kPasses; ++p) {
+        const int r = p * G::kRowsPerPass + crow;
+        step0[p] = 4 * cq - phase(r);
+        off0[p] = (r * T + step0[p]) * 4;
+    }
 
     float4 stage[NI][G::kPasses];
 
     auto fetch = [&](int chunk) {
 #pragma unroll
         for (int p = 0; p < G::kPasses; ++p) {
-            const int r = p * G::kRowsPerPass + crow;
-            const int t = chunk * TC + 4 * cq - phase(r);
-            const int64_t off = (int64_t)(m0 + r) * (int64_t)T + (int64_t)t;
+            const bool ok = (unsigned)(step0[p] + chunk * TC) < (unsigned)T;
+            const int off = ok ? off0[p] + chunk * (TC * 4) : kOutOfRange;
 #pragma unroll
-            for (int i = 0; i < NI; ++i) {
-                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (r < rows) {
-                    const float* src = prm.in[i] + off;
-                    if (VEC4) {
-                        if (t >= 0 && t < T) v = load4(src, STREAM);
-                    } else {
-                        if (t + 0 < T) v.x = src[0];
-                        if (t + 1 < T) v.y = src[1];
-                        if (t + 2 < T) v.z = src[2];
-                        if (t + 3 < T) v.w = src[3];
-                    }
-                }
-                stage[i][p] = v;
-            }
+            for (int i = 0; i < NI; ++i) stage[i][p] = buf_load4<STREAM>(src[i], off);
         }
     };
 
+    auto run_quad = [&](int qq) {
+        float xin[NI][4], yout[NO][4];
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const float4 v = *reinterpret_cast<const float4*>(&tile[i][lane * G::kPitch + 4 * qq]);
+            xin[i][0] = v.x; xin[i][1] = v.y; xin[i][2] = v.z; xin[i][3] = v.w;
+        }
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const int ss = Op::kReverse ? 3 - s : s;
+            float x[NI], y[NO];
+#pragma unroll
+            for (int i = 0; i < NI; ++i) x[i] = xin[i][ss];
+            op.step(x, y);
+#pragma unroll
+            for (int o = 0; o < NO; ++o) yout[o][ss] = y[o];
+        }
+#pragma unroll
+        for (int o = 0; o < NO; ++o)
+            *reinterpret_cast<float4*>(&tile[o][lane * G::kPitch + 4 * qq]) =
+                make_float4(yout[o][0], yout[o][1], yout[o][2], yout[o][3]);
+    };
+
     fetch(Op::kReverse ? nchunks - 1 : 0);
+    // Stores that fall out of range (dropped by the hardware), as many as one chunk issues: the
+    // loop is then entered in the same state its back edge leaves -- a chunk of loads followed by
+    // a chunk of stores in flight -- and the wait for the loads at the top of every iteration
+    // can leave the stores of the previous chunk in flight instead of draining them.
+#pragma unroll
+    for (int p = 0; p < G::kPasses; ++p)
+#pragma unroll
+        for (int o = 0; o < NO; ++o)   // distinct offsets, or the compiler merges them into one store
+            buf_store4<STREAM>(dst[o], kOutOfRange + 16 * p, make_float4(0.f, 0.f, 0.f, 0.f));
 
     for (int k = 0; k < nchunks; ++k) {
         const int chunk = Op::kReverse ? nchunks - 1 - k : k;
+        const bool interior = chunk >= 1 && chunk < interior_end;
 
         // staged registers -> LDS
 #pragma unroll
@@ -173,15 +236,113 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
         }
         __syncthreads();
 
-        if (k + 1 < nchunks) fetch(Op::kReverse ? chunk - 1 : chunk + 1);
+        fetch(Op::kReverse ? chunk - 1 : chunk + 1);    // past the last chunk every lane is out of range
 
-        // sequential recurrence: lane = neuron; columns outside [0, T) are skipped
-        const int tl = chunk * TC - a_lane;           // step held by column 0 of this lane's row
-#pragma unroll 2
+        // sequential recurrence: lane = neuron
+        if (interior) {
+            if (lane < R) {
+#pragma unroll 4
+                for (int q = 0; q < G::kQuads; ++q) run_quad(Op::kReverse ? G::kQuads - 1 - q : q);
+            }
+        } else {
+            const int tl = chunk * TC - a_lane;       // step held by column 0 of this lane's row
+            for (int q = 0; q < G::kQuads; ++q) {
+                const int qq = Op::kReverse ? G::kQuads - 1 - q : q;
+                if (lane < R && (unsigned)(tl + 4 * qq) < (unsigned)T) run_quad(qq);
+            }
+        }
+        __syncthreads();
+
+        // LDS -> global; on edge chunks the quads of a line shared with a neighbouring row go to
+        // the boundary buffer instead (their global offset is pushed out of range)
+#pragma unroll
+        for (int p = 0; p < G::kPasses; ++p) {
+            const int r = p * G::kRowsPerPass + crow;
+            const int t = step0[p] + chunk * TC;
+            int off = ((unsigned)t < (unsigned)T) ? off0[p] + chunk * (TC * 4) : kOutOfRange;
+            float4 v[NO];
+#pragma unroll
+            for (int o = 0; o < NO; ++o) v[o] = *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]);
+            if (!interior && route && (unsigned)t < (unsigned)T && r < rows) {
+                const int a = 4 * cq - step0[p];
+                const int pos = t + a;                     // position in the row's line-aligned window
+                const int last_full = (a + T) & ~31;
+                int slot = -1;
+                if (a != 0 && pos < 32) slot = r * 32 + pos;
+                else if (pos >= last_full) slot = (r + 1) * 32 + (pos - last_full);
+                if (slot >= 0) {
+                    off = kOutOfRange;
+#pragma unroll
+                    for (int o = 0; o < NO; ++o) *reinterpret_cast<float4*>(&bline[o][slot]) = v[o];
+                }
+            }
+#pragma unroll
+            for (int o = 0; o < NO; ++o) buf_store4<STREAM>(dst[o], off, v[o]);
+        }
+        __syncthreads();
+    }
+
+    if (route) {
+        // boundary line b holds the tail of row b-1 (columns < phase(b)) and the head of row b
+        for (int i = lane; i < (R + 1) * 8; i += kWave) {
+            const int b = i >> 3, col = (i & 7) * 4;
+            const int a = phase(b);
+            const bool owned = (col < a) ? (b >= 1 && b - 1 < rows) : (b < rows);
+            const int off = (a != 0 && b <= rows && owned) ? (b * T - a + col) * 4 : kOutOfRange;
+#pragma unroll
+            for (int o = 0; o < NO; ++o)
+                buf_store4<STREAM>(dst[o], off, *reinterpret_cast<const float4*>(&bline[o][b * 32 + col]));
+        }
+    }
+    op.finish(prm, m0 + lane, lane < rows);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Fallback for T % 4 != 0 or bases that are not 16-byte aligned: same tiling, dword accesses,
+// no phase and no boundary buffer.  Bit-exact, not tuned.
+template <class Op, int R>
+__global__ __launch_bounds__(kWave) void stream_kernel_scalar(typename Op::Params prm, int64_t M, int T) {
+    using G = TileGeom<R>;
+    constexpr int TC = G::kChunk;
+    constexpr int NI = Op::kIn, NO = Op::kOut, NT = NI > NO ? NI : NO;
+    __shared__ __attribute__((aligned(16))) float tile[NT][G::kTileFloats];
+
+    const int lane = threadIdx.x;
+    const int64_t m0 = (int64_t)blockIdx.x * R;
+    const int rows = (int)((M - m0) < R ? (M - m0) : R);
+
+    Op op;
+    op.init(prm, m0 + lane, lane < rows);
+
+    const int nchunks = (T + TC - 1) / TC;
+    const int crow = lane / G::kQuads;
+    const int cq = lane % G::kQuads;
+
+    for (int k = 0; k < nchunks; ++k) {
+        const int chunk = Op::kReverse ? nchunks - 1 - k : k;
+        const int t = chunk * TC + 4 * cq;
+#pragma unroll
+        for (int p = 0; p < G::kPasses; ++p) {
+            const int r = p * G::kRowsPerPass + crow;
+            const int64_t off = (int64_t)(m0 + r) * (int64_t)T + (int64_t)t;
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);      // zero fill: steps past T-1 must be no-ops
+                if (r < rows) {
+                    const float* src = prm.in[i] + off;
+                    if (t + 0 < T) v.x = src[0];
+                    if (t + 1 < T) v.y = src[1];
+                    if (t + 2 < T) v.z = src[2];
+                    if (t + 3 < T) v.w = src[3];
+                }
+                *reinterpret_cast<float4*>(&tile[i][r * G::kPitch + 4 * cq]) = v;
+            }
+        }
+        __syncthreads();
+
         for (int q = 0; q < G::kQuads; ++q) {
             const int qq = Op::kReverse ? G::kQuads - 1 - q : q;
-            const int t = tl + 4 * qq;
-            if (lane < R && t >= 0 && t < T) {
+            if (lane < R && chunk * TC + 4 * qq < T) {
                 float xin[NI][4], yout[NO][4];
 #pragma unroll
                 for (int i = 0; i < NI; ++i) {
@@ -206,55 +367,23 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
         }
         __syncthreads();
 
-        // LDS -> global (quads of a line shared with a neighbouring row go to the boundary buffer)
 #pragma unroll
         for (int p = 0; p < G::kPasses; ++p) {
             const int r = p * G::kRowsPerPass + crow;
-            const int a = phase(r);
-            const int pos = chunk * TC + 4 * cq;          // position in the row's line-aligned window
-            const int t = pos - a;
             const int64_t off = (int64_t)(m0 + r) * (int64_t)T + (int64_t)t;
-            const int end = a + T;                        // window position one past the last step
-            const int last_full = end & ~31;
 #pragma unroll
             for (int o = 0; o < NO; ++o) {
                 const float4 v = *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]);
                 if (r < rows) {
-                    float* dst = prm.out[o] + off;
-                    if (VEC4) {
-                        if (t >= 0 && t < T) {
-                            if (route && a != 0 && pos < 32)
-                                *reinterpret_cast<float4*>(&bline[o][r * 32 + pos]) = v;
-                            else if (route && pos >= last_full)   // only when end is not a line multiple
-                                *reinterpret_cast<float4*>(&bline[o][(r + 1) * 32 + (pos - last_full)]) = v;
-                            else
-                                store4(dst, v, STREAM);
-                        }
-                    } else {
-                        if (t + 0 < T) dst[0] = v.x;
-                        if (t + 1 < T) dst[1] = v.y;
-                        if (t + 2 < T) dst[2] = v.z;
-                        if (t + 3 < T) dst[3] = v.w;
-                    }
+                    float* d = prm.out[o] + off;
+                    if (t + 0 < T) d[0] = v.x;
+                    if (t + 1 < T) d[1] = v.y;
+                    if (t + 2 < T) d[2] = v.z;
+                    if (t + 3 < T) d[3] = v.w;
                 }
             }
         }
         __syncthreads();
-    }
-
-    if (route) {
-        // boundary line b holds the tail of row b-1 (columns < phase(b)) and the head of row b
-        for (int i = lane; i < (R + 1) * 8; i += kWave) {
-            const int b = i >> 3, col = (i & 7) * 4;
-            const int a = phase(b);
-            const bool owned = (col < a) ? (b >= 1 && b - 1 < rows) : (b < rows);
-            if (a != 0 && b <= rows && owned) {
-                const int64_t off = (int64_t)(m0 + b) * (int64_t)T - a + col;
-#pragma unroll
-                for (int o = 0; o < NO; ++o)
-                    store4(prm.out[o] + off, *reinterpret_cast<const float4*>(&bline[o][b * 32 + col]), STREAM);
-            }
-        }
     }
     op.finish(prm, m0 + lane, lane < rows);
 }
@@ -269,11 +398,11 @@ int launch_stream_rows(const typename Op::Params& prm, int64_t M, int64_t T, boo
                        hipStream_t stream) {
     const dim3 grid((unsigned)((M + R - 1) / R)), block(kWave);
     if (!vec)
-        hipLaunchKernelGGL((stream_kernel<Op, R, false, false>), grid, block, 0, stream, prm, M, (int)T);
+        hipLaunchKernelGGL((stream_kernel_scalar<Op, R>), grid, block, 0, stream, prm, M, (int)T);
     else if (streaming)
-        hipLaunchKernelGGL((stream_kernel<Op, R, true, true>), grid, block, 0, stream, prm, M, (int)T);
+        hipLaunchKernelGGL((stream_kernel<Op, R, true>), grid, block, 0, stream, prm, M, (int)T);
     else
-        hipLaunchKernelGGL((stream_kernel<Op, R, true, false>), grid, block, 0, stream, prm, M, (int)T);
+        hipLaunchKernelGGL((stream_kernel<Op, R, false>), grid, block, 0, stream, prm, M, (int)T);
     return (int)hipGetLastError();
 }
 
@@ -286,7 +415,8 @@ constexpr int64_t kAlways = (int64_t)1 << 62;
 template <class Op>
 int launch_stream(const typename Op::Params& prm, int64_t M, int64_t T, hipStream_t stream) {
     if (M == 0 || T == 0) return 0;
-    bool vec = (T % 4) == 0;
+    // the dwordx4 kernel addresses a wave's rows with 32-bit byte offsets: 64 * T * 4 must stay below 2^31
+    bool vec = (T % 4) == 0 && T <= (1 << 22);
     for (int i = 0; i < Op::kIn; ++i) vec = vec && aligned16(prm.in[i]);
     for (int o = 0; o < Op::kOut; ++o) vec = vec && aligned16(prm.out[o]);
     const bool streaming = M * T * 4 > ((int64_t)64 << 20);
