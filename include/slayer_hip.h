@@ -167,6 +167,38 @@ int slayer_conv(float *out, const float *in, const float *filt, int64_t K, float
 int slayer_corr(float *out, const float *in, const float *filt, int64_t K, float sampling_time,
                 int64_t M, int64_t T, void *stream);
 
+/* ---- cross-check implementations (debug mode) ------------------------------------------------ */
+
+/* The reference's debug mode runs its CPU loop next to its kernel and raises on a difference
+ * (neuron/dynamics/leaky_integrator.py:134-155,168-205; adaptive_threshold.py:191-225;
+ * resonator.py:196-236,254-300).  These entry points are the second implementation for that check
+ * here: one thread per neuron, 64-bit integer state, plain global accesses.  Same arguments and
+ * results as the entry points without the suffix (the backward variants return grad_input only). */
+int slayer_li_fwd_naive(float *out, const float *in, const float *decay, const float *state,
+                        double thr_scaled, int w_scale,
+                        int64_t M, int64_t neurons_per_batch, int64_t num_decays, int64_t num_states,
+                        int64_t T, void *stream);
+int slayer_li_bwd_naive(float *grad_in, const float *grad_out, const float *decay,
+                        int64_t M, int64_t neurons_per_batch, int64_t num_decays, int64_t T, void *stream);
+int slayer_ath_fwd_naive(float *th_out, float *ref_out, const float *in,
+                         const float *ref_state, const float *ref_decay,
+                         const float *th_state, const float *th_decay,
+                         int64_t th_step_scaled, int64_t th0_scaled, int w_scale,
+                         int64_t M, int64_t neurons_per_batch,
+                         int64_t num_ref_decays, int64_t num_th_decays,
+                         int64_t num_ref_states, int64_t num_th_states,
+                         int64_t T, void *stream);
+int slayer_res_fwd_naive(float *re_out, float *im_out, const float *re_in, const float *im_in,
+                         const float *sin_decay, const float *cos_decay,
+                         const float *re_state, const float *im_state,
+                         double thr_scaled, int w_scale,
+                         int64_t M, int64_t neurons_per_batch, int64_t num_decays,
+                         int64_t num_re_states, int64_t num_im_states,
+                         int64_t T, void *stream);
+int slayer_res_bwd_naive(float *g_re_in, float *g_im_in, const float *g_re, const float *g_im,
+                         const float *sin_decay, const float *cos_decay,
+                         int64_t M, int64_t neurons_per_batch, int64_t num_decays, int64_t T, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -39,6 +39,13 @@ _SIGNATURES = {
     'slayer_shift': (_INT, [_P, _P, _P, _I64, _F, _I64, _I64, _I64, _P]),
     'slayer_conv': (_INT, [_P, _P, _P, _I64, _F, _I64, _I64, _P]),
     'slayer_corr': (_INT, [_P, _P, _P, _I64, _F, _I64, _I64, _P]),
+    'slayer_li_fwd_naive': (_INT, [_P, _P, _P, _P, _D, _INT, _I64, _I64, _I64, _I64, _I64, _P]),
+    'slayer_li_bwd_naive': (_INT, [_P, _P, _P, _I64, _I64, _I64, _I64, _P]),
+    'slayer_ath_fwd_naive': (_INT, [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _INT,
+                                    _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P]),
+    'slayer_res_fwd_naive': (_INT, [_P, _P, _P, _P, _P, _P, _P, _P, _D, _INT,
+                                    _I64, _I64, _I64, _I64, _I64, _I64, _P]),
+    'slayer_res_bwd_naive': (_INT, [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _P]),
 }
 
 EXPORTS = tuple(_SIGNATURES)
@@ -88,6 +95,16 @@ def require_gpu(*tensors):
         elif t.device != dev:
             raise RuntimeError(f'tensors on different devices: {dev} and {t.device}')
     return dev
+
+
+def raise_on_mismatch(what, fast, check):
+    """debug mode: the streaming kernel and the one-thread-per-neuron kernel must agree bit for bit."""
+    if not torch.equal(fast, check):
+        bad = fast != check
+        first = bad.nonzero()[0].tolist()
+        raise Exception(f'{what}: the two GPU implementations differ in {int(bad.sum())} of {bad.numel()} '
+                        f'elements, first at {first}: {fast[tuple(first)].item()!r} vs '
+                        f'{check[tuple(first)].item()!r} (a 32-bit state overflow shows up like this)')
 
 
 def ptr(t):

@@ -21,6 +21,7 @@ def dynamics(input, ref_state, ref_decay, th_state, th_decay, th_scale, th0, w_s
     (threshold, refractory) : tensors shaped like ``input`` (values before the
     spike update of each step).
     """
+    _ATHDynamics.DEBUG = debug
     return _ATHDynamics.apply(input, ref_state, ref_decay, th_state, th_decay, th_scale, th0, w_scale)
 
 
@@ -36,7 +37,7 @@ def persistent_th_state(th_state, spike, th_step):
     return th_state + spike * th_step
 
 
-def _fwd(input, ref_state, ref_decay, th_state, th_decay, th_scale, th0, w_scale):
+def _fwd(input, ref_state, ref_decay, th_state, th_decay, th_scale, th0, w_scale, entry='slayer_ath_fwd'):
     dev = N.require_gpu(input, ref_state, ref_decay, th_state, th_decay)
     input = input.contiguous()
     ref_state, ref_decay = ref_state.contiguous(), ref_decay.contiguous()
@@ -48,7 +49,7 @@ def _fwd(input, ref_state, ref_decay, th_state, th_decay, th_scale, th0, w_scale
     threshold = torch.empty_like(input)
     refractory = torch.empty_like(input)
     with torch.cuda.device(dev):
-        N.check(N.lib().slayer_ath_fwd(
+        N.check(getattr(N.lib(), entry)(
             N.ptr(threshold), N.ptr(refractory), N.ptr(input),
             N.ptr(ref_state), N.ptr(ref_decay), N.ptr(th_state), N.ptr(th_decay),
             int(th_scale * w_scale), int(th0 * w_scale), int(w_scale),
@@ -58,10 +59,18 @@ def _fwd(input, ref_state, ref_decay, th_state, th_decay, th_scale, th0, w_scale
 
 
 class _ATHDynamics(torch.autograd.Function):
+    DEBUG = False
+
     @staticmethod
     def forward(ctx, input, ref_state, ref_decay, th_state, th_decay, th_scale, th0, w_scale):
-        return _fwd(input.detach(), ref_state.detach(), ref_decay.detach(), th_state.detach(),
-                    th_decay.detach(), th_scale, th0, w_scale)
+        args = (input.detach(), ref_state.detach(), ref_decay.detach(), th_state.detach(),
+                th_decay.detach(), th_scale, th0, w_scale)
+        threshold, refractory = _fwd(*args)
+        if _ATHDynamics.DEBUG:
+            th_check, ref_check = _fwd(*args, entry='slayer_ath_fwd_naive')
+            N.raise_on_mismatch('adaptive_threshold threshold', threshold, th_check)
+            N.raise_on_mismatch('adaptive_threshold refractory', refractory, ref_check)
+        return threshold, refractory
 
     @staticmethod
     def backward(*_):

@@ -27,8 +27,8 @@ def dynamics(input, decay, state, w_scale, threshold=None, debug=False):
     threshold : float or None
         ``None`` disables the reset.
     debug : bool
-        accepted for interface compatibility; the reference uses it to compare
-        its two implementations, here there is only one.
+        also run the independent one-thread-per-neuron kernel (64-bit state) in
+        forward and backward and raise if the two results differ in any bit.
 
     Returns
     -------
@@ -36,6 +36,7 @@ def dynamics(input, decay, state, w_scale, threshold=None, debug=False):
     """
     if threshold is None:
         threshold = -1
+    _LIDynamics.DEBUG = debug
     return _LIDynamics.apply(input, decay, state, threshold, w_scale)
 
 
@@ -45,7 +46,7 @@ def persistent_state(state, spike):
     return state * (1 - spike)
 
 
-def _fwd(input, decay, state, threshold, w_scale):
+def _fwd(input, decay, state, threshold, w_scale, entry='slayer_li_fwd'):
     dev = N.require_gpu(input, decay, state)
     input, decay, state = input.contiguous(), decay.contiguous(), state.contiguous()
     M, T = N.rows_and_steps(input)
@@ -53,7 +54,7 @@ def _fwd(input, decay, state, threshold, w_scale):
         raise RuntimeError(f'state has {state.numel()} elements, expected 1 or {M}')
     output = torch.empty_like(input)
     with torch.cuda.device(dev):
-        N.check(N.lib().slayer_li_fwd(
+        N.check(getattr(N.lib(), entry)(
             N.ptr(output), N.ptr(input), N.ptr(decay), N.ptr(state),
             float(threshold * w_scale), int(w_scale),
             M, N.neurons_per_batch(input), decay.numel(), state.numel(), T, N.stream_handle()))
@@ -76,10 +77,29 @@ def _bwd(grad_output, output, decay, need_decay_grad=True):
     return grad_input, grad_decay
 
 
+def _bwd_naive(grad_output, decay):
+    dev = N.require_gpu(grad_output, decay)
+    grad_output, decay = grad_output.contiguous(), decay.contiguous()
+    M, T = N.rows_and_steps(grad_output)
+    grad_input = torch.empty_like(grad_output)
+    with torch.cuda.device(dev):
+        N.check(N.lib().slayer_li_bwd_naive(
+            N.ptr(grad_input), N.ptr(grad_output), N.ptr(decay), M, N.neurons_per_batch(grad_output),
+            decay.numel(), T, N.stream_handle()))
+    return grad_input
+
+
 class _LIDynamics(torch.autograd.Function):
+    DEBUG = False
+
     @staticmethod
     def forward(ctx, input, decay, state, threshold, w_scale):
         output = _fwd(input, decay.detach(), state.detach(), threshold, w_scale)
+        ctx.debug = _LIDynamics.DEBUG
+        if ctx.debug:
+            N.raise_on_mismatch('leaky_integrator forward', output,
+                                _fwd(input, decay.detach(), state.detach(), threshold, w_scale,
+                                     entry='slayer_li_fwd_naive'))
         ctx.save_for_backward(output, decay)
         return output
 
@@ -88,6 +108,8 @@ class _LIDynamics(torch.autograd.Function):
         output, decay = ctx.saved_tensors
         need = ctx.needs_input_grad[1]
         grad_input, grad_decay = _bwd(grad_output, output, decay.detach(), need)
+        if ctx.debug:
+            N.raise_on_mismatch('leaky_integrator backward', grad_input, _bwd_naive(grad_output, decay.detach()))
         if grad_decay is not None:
             grad_decay = grad_decay.reshape(decay.shape)
         return grad_input, grad_decay, None, None, None

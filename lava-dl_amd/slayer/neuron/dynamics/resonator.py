@@ -22,6 +22,7 @@ def dynamics(real_input, imag_input, sin_decay, cos_decay, real_state, imag_stat
     """
     if threshold is None:
         threshold = -1
+    _ResDynamics.DEBUG = debug
     return _ResDynamics.apply(real_input, imag_input, sin_decay, cos_decay,
                               real_state, imag_state, threshold, w_scale)
 
@@ -38,7 +39,8 @@ def persistent_imag_state(imag_state, spike, threshold, scale):
     return spike * (threshold - 1 / scale) + (1 - spike) * imag_state
 
 
-def _fwd(real_input, imag_input, sin_decay, cos_decay, real_state, imag_state, threshold, w_scale):
+def _fwd(real_input, imag_input, sin_decay, cos_decay, real_state, imag_state, threshold, w_scale,
+         entry='slayer_res_fwd'):
     dev = N.require_gpu(real_input, imag_input, sin_decay, cos_decay, real_state, imag_state)
     if real_input.shape != imag_input.shape:
         raise RuntimeError(f'real/imag input shapes differ: {real_input.shape} vs {imag_input.shape}')
@@ -54,7 +56,7 @@ def _fwd(real_input, imag_input, sin_decay, cos_decay, real_state, imag_state, t
     real = torch.empty_like(real_input)
     imag = torch.empty_like(imag_input)
     with torch.cuda.device(dev):
-        N.check(N.lib().slayer_res_fwd(
+        N.check(getattr(N.lib(), entry)(
             N.ptr(real), N.ptr(imag), N.ptr(real_input), N.ptr(imag_input),
             N.ptr(sin_decay), N.ptr(cos_decay), N.ptr(real_state), N.ptr(imag_state),
             float(threshold * w_scale), int(w_scale),
@@ -84,6 +86,19 @@ def _bwd(grad_real, grad_imag, real, imag, sin_decay, cos_decay, need_decay_grad
     return g_re_in, g_im_in, g_sin, g_cos
 
 
+def _bwd_naive(grad_real, grad_imag, sin_decay, cos_decay):
+    dev = N.require_gpu(grad_real, grad_imag, sin_decay, cos_decay)
+    grad_real, grad_imag = grad_real.contiguous(), grad_imag.contiguous()
+    M, T = N.rows_and_steps(grad_real)
+    g_re_in, g_im_in = torch.empty_like(grad_real), torch.empty_like(grad_imag)
+    with torch.cuda.device(dev):
+        N.check(N.lib().slayer_res_bwd_naive(
+            N.ptr(g_re_in), N.ptr(g_im_in), N.ptr(grad_real), N.ptr(grad_imag),
+            N.ptr(sin_decay.contiguous()), N.ptr(cos_decay.contiguous()),
+            M, N.neurons_per_batch(grad_real), sin_decay.numel(), T, N.stream_handle()))
+    return g_re_in, g_im_in
+
+
 def _raise_on_nan(**tensors):
     """The reference aborts the backward pass on NaN (resonator.py:421-439)."""
     for name, t in tensors.items():
@@ -92,11 +107,19 @@ def _raise_on_nan(**tensors):
 
 
 class _ResDynamics(torch.autograd.Function):
+    DEBUG = False
+
     @staticmethod
     def forward(ctx, real_input, imag_input, sin_decay, cos_decay, real_state, imag_state,
                 threshold, w_scale):
-        real, imag = _fwd(real_input, imag_input, sin_decay.detach(), cos_decay.detach(),
-                          real_state.detach(), imag_state.detach(), threshold, w_scale)
+        args = (real_input, imag_input, sin_decay.detach(), cos_decay.detach(),
+                real_state.detach(), imag_state.detach(), threshold, w_scale)
+        real, imag = _fwd(*args)
+        ctx.debug = _ResDynamics.DEBUG
+        if ctx.debug:
+            re_check, im_check = _fwd(*args, entry='slayer_res_fwd_naive')
+            N.raise_on_mismatch('resonator real', real, re_check)
+            N.raise_on_mismatch('resonator imag', imag, im_check)
         ctx.save_for_backward(real, imag, sin_decay, cos_decay)
         return real, imag
 
@@ -106,6 +129,10 @@ class _ResDynamics(torch.autograd.Function):
         need = ctx.needs_input_grad[2] or ctx.needs_input_grad[3]
         g_re, g_im, g_sin, g_cos = _bwd(grad_real, grad_imag, real, imag,
                                         sin_decay.detach(), cos_decay.detach(), need)
+        if ctx.debug:
+            c_re, c_im = _bwd_naive(grad_real, grad_imag, sin_decay.detach(), cos_decay.detach())
+            N.raise_on_mismatch('resonator grad real', g_re, c_re)
+            N.raise_on_mismatch('resonator grad imag', g_im, c_im)
         _raise_on_nan(grad_real=grad_real, grad_imag=grad_imag, grad_real_input=g_re,
                       grad_imag_input=g_im, grad_sin_decay=g_sin, grad_cos_decay=g_cos)
         if g_sin is not None:

@@ -320,3 +320,32 @@ def test_res_autograd_and_nan_guard(slayer):
     bad[0, 0, 10] = float('nan')
     with pytest.raises(Exception):
         torch.autograd.backward([re, im], [bad, torch.ones(shape, device=dev())])
+
+
+# --------------------------------------------------------------------------------- debug mode
+def test_debug_mode_cross_check_passes_and_catches_overflow(slayer):
+    """debug=True runs the independent one-thread-per-neuron kernels (64-bit state) next to the
+    streaming kernels: silent when they agree, an exception when a state leaves the 32-bit range."""
+    gen = torch.Generator().manual_seed(77)
+    shape = (2, 40, 132)
+    x = sparse_input(gen, shape, p=0.3, amp=2.0).to(dev()).requires_grad_()
+    x2 = sparse_input(gen, shape, p=0.3, amp=2.0).to(dev()).requires_grad_()
+    d = torch.randint(0, 4097, (40,), generator=gen).float().to(dev()).requires_grad_()
+    zero, one = torch.zeros(1, device=dev()), torch.ones(1, device=dev())
+    D = slayer.neuron.dynamics
+    y = D.leaky_integrator.dynamics(x, d, zero, 64, 1.0, debug=True)
+    ref = O.li_fwd(x.detach().cpu(), d.detach().cpu(), torch.tensor([0.0]), 64, 1.0)
+    assert_exact(y, ref, 'debug li_fwd')
+    y.sum().backward()
+    D.adaptive_threshold.dynamics(x.detach(), zero, d.detach(), one, d.detach(), 0.5, 1.0, 64, debug=True)
+    for thr in (None, 1.5):
+        re, im = D.resonator.dynamics(x, x2, (d * 0.5).round(), (d * 0.6).round(), zero, zero, 64, thr, debug=True)
+        (re.sum() + im.sum()).backward()
+    # an integrator (decay 0) driven beyond 2^31: the 32-bit streaming state saturates/wraps, the check fires
+    big = torch.full((1, 1, 64), 3.0e7, device=dev())
+    with pytest.raises(Exception, match='implementations differ'):
+        D.leaky_integrator.dynamics(big, zero, zero, 64, debug=True)
+    # the naive kernel itself follows the int64 oracle there
+    from lava_dl_amd.slayer.neuron.dynamics import leaky_integrator as L
+    got = L._fwd(big, zero, zero, -1, 64, entry='slayer_li_fwd_naive')
+    assert_exact(got, O.li_fwd(big.cpu(), torch.tensor([0.0]), torch.tensor([0.0]), 64), 'naive li_fwd beyond 2^31')
