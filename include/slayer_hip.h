@@ -89,6 +89,20 @@ int slayer_ath_fwd(float *th_out, float *ref_out, const float *in,
                    int64_t num_ref_states, int64_t num_th_states,
                    int64_t T, void *stream);
 
+/* Replaces APThDynamicsFwd (neuron/dynamics/adaptive_phase_th.cu:25-88 kernel, host function and
+ * exports at its end); arithmetic of _APTHDynamicsFwd (neuron/dynamics/adaptive_phase_th.py:234-284).
+ * Threshold / refractory recurrences as in slayer_ath_fwd; a step spikes when
+ * trunc(w*re_in[t]) >= th + r and trunc(w*im_in[t]) >= 0 and the previous imaginary sample was < 0
+ * (im_state seeds the previous sample of step 0). */
+int slayer_apth_fwd(float *th_out, float *ref_out, const float *re_in, const float *im_in,
+                    const float *im_state, const float *ref_state, const float *ref_decay,
+                    const float *th_state, const float *th_decay,
+                    int64_t th_step_scaled, int64_t th0_scaled, int w_scale,
+                    int64_t M, int64_t neurons_per_batch,
+                    int64_t num_ref_decays, int64_t num_th_decays,
+                    int64_t num_im_states, int64_t num_ref_states, int64_t num_th_states,
+                    int64_t T, void *stream);
+
 /* ---- resonator ------------------------------------------------------------------------------ */
 
 /* Replaces ResDynamicsFwd (neuron/dynamics/resonator.cu:151-198); arithmetic of
@@ -115,6 +129,23 @@ int slayer_res_bwd(float *g_re_in, float *g_im_in, float *grad_sin, float *grad_
                    const float *sin_decay, const float *cos_decay, float *workspace,
                    int64_t M, int64_t neurons_per_batch, int64_t num_decays,
                    int64_t T, void *stream);
+
+/* Replaces AdResDynamicsFwd (neuron/dynamics/adaptive_resonator.cu:25-126 kernel and its host
+ * function); arithmetic of _AdResDynamicsFwd (neuron/dynamics/adaptive_resonator.py:379-436):
+ * the resonator recurrence without reset plus threshold / refractory recurrences whose spike
+ * condition is im >= th + r (integer compare).  Its backward pass is slayer_res_bwd. */
+int slayer_adres_fwd(float *re_out, float *im_out, float *th_out, float *ref_out,
+                     const float *re_in, const float *im_in,
+                     const float *sin_decay, const float *cos_decay,
+                     const float *ref_decay, const float *th_decay,
+                     const float *re_state, const float *im_state,
+                     const float *ref_state, const float *th_state,
+                     int64_t th_step_scaled, int64_t th0_scaled, int w_scale,
+                     int64_t M, int64_t neurons_per_batch, int64_t num_decays,
+                     int64_t num_ref_decays, int64_t num_th_decays,
+                     int64_t num_re_states, int64_t num_im_states,
+                     int64_t num_ref_states, int64_t num_th_states,
+                     int64_t T, void *stream);
 
 /* ---- spike functions (elementwise; they replace chains of torch ops, not a .cu) ----------- */
 

@@ -55,6 +55,59 @@ struct ResFwd {
     __device__ __forceinline__ void finish(const Params&, int64_t, bool) {}
 };
 
+// Adaptive resonator: the resonator recurrence (no reset) with an adaptive threshold and a
+// refractory state driven by the imaginary part; four output traces.
+template <bool POW2>
+struct AdResFwd {
+    static constexpr int kIn = 2, kOut = 4;      // out: real, imag, threshold, refractory
+    static constexpr bool kReverse = false;
+    static constexpr int64_t kRows32Below = kAlways, kRows16Below = 16384;
+    struct Params {
+        const float* in[2];
+        float* out[4];
+        const float *sin_decay, *cos_decay, *ref_decay, *th_decay;
+        const float *re_state, *im_state, *ref_state, *th_state;
+        int step, base;
+        float w, inv_w;
+        int64_t npb, nd, n_rd, n_td, n_res, n_ims, n_rs, n_ts;
+    };
+    int re, im, s, c, th, r, mt, mr, th_step, base;
+    float w, inv_w;
+
+    __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
+        w = p.w; inv_w = p.inv_w; th_step = p.step; base = p.base;
+        re = im = s = c = th = r = mt = mr = 0;
+        if (valid) {
+            re = trunc_i32(p.re_state[p.n_res == 1 ? 0 : m] * w);
+            im = trunc_i32(p.im_state[p.n_ims == 1 ? 0 : m] * w);
+            th = trunc_i32(p.th_state[p.n_ts == 1 ? 0 : m] * w);
+            r = trunc_i32(p.ref_state[p.n_rs == 1 ? 0 : m] * w);
+            const int64_t j = param_index(m, p.npb, p.nd);
+            s = trunc_i32(p.sin_decay[j]);
+            c = trunc_i32(p.cos_decay[j]);
+            mt = 4096 - trunc_i32(p.th_decay[param_index(m, p.npb, p.n_td)]);
+            mr = 4096 - trunc_i32(p.ref_decay[param_index(m, p.npb, p.n_rd)]);
+        }
+    }
+    __device__ __forceinline__ void step(const float (&x)[2], float (&o)[4]) {
+        r = rs0_12(r, mr);
+        th = rs0_12(th - base, mt) + base;
+        const int re_n = rs0_12(c, re) - rs0_12(s, im) + trunc_i32(w * x[0]);
+        const int im_n = rs0_12(s, re) + rs0_12(c, im) + trunc_i32(w * x[1]);
+        const float ref = (float)re_n, imf = (float)im_n, thf = (float)th, rf = (float)r;
+        o[0] = POW2 ? ref * inv_w : ref / w;
+        o[1] = POW2 ? imf * inv_w : imf / w;
+        o[2] = POW2 ? thf * inv_w : thf / w;
+        o[3] = POW2 ? rf * inv_w : rf / w;
+        const bool fired = im_n >= th + r;
+        r += fired ? 2 * th : 0;
+        th += fired ? th_step : 0;
+        re = re_n;
+        im = im_n;
+    }
+    __device__ __forceinline__ void finish(const Params&, int64_t, bool) {}
+};
+
 struct ResBwd {
     static constexpr int kIn = 4, kOut = 2;      // in: g_re, g_im, saved re, saved im
     static constexpr bool kReverse = true;
@@ -164,4 +217,45 @@ extern "C" int slayer_res_bwd(float* g_re_in, float* g_im_in, float* grad_sin, f
                                         num_decays, st);
     }
     return 0;
+}
+
+extern "C" int slayer_adres_fwd(float* re_out, float* im_out, float* th_out, float* ref_out,
+                                const float* re_in, const float* im_in,
+                                const float* sin_decay, const float* cos_decay,
+                                const float* ref_decay, const float* th_decay,
+                                const float* re_state, const float* im_state,
+                                const float* ref_state, const float* th_state,
+                                int64_t th_step_scaled, int64_t th0_scaled, int w_scale,
+                                int64_t M, int64_t neurons_per_batch, int64_t num_decays,
+                                int64_t num_ref_decays, int64_t num_th_decays,
+                                int64_t num_re_states, int64_t num_im_states,
+                                int64_t num_ref_states, int64_t num_th_states,
+                                int64_t T, void* stream) {
+    if (int e = check_rows(M, T)) return e;
+    if (M == 0 || T == 0) return 0;
+    if (!re_out || !im_out || !th_out || !ref_out || !re_in || !im_in || !sin_decay || !cos_decay || !ref_decay ||
+        !th_decay || !re_state || !im_state || !ref_state || !th_state)
+        return SLAYER_ENULL;
+    if (int e = check_params(M, neurons_per_batch, num_decays)) return e;
+    if (int e = check_params(M, neurons_per_batch, num_ref_decays)) return e;
+    if (int e = check_params(M, neurons_per_batch, num_th_decays)) return e;
+    for (int64_t n : {num_re_states, num_im_states, num_ref_states, num_th_states})
+        if (int e = check_states(M, n)) return e;
+    if (w_scale == 0) return SLAYER_EINVAL;
+    const int64_t lim = 0x7fffffffLL;
+    if (th_step_scaled > lim || th_step_scaled < -lim || th0_scaled > lim || th0_scaled < -lim) return SLAYER_ERANGE;
+    const float w = (float)w_scale;
+    hipStream_t st = (hipStream_t)stream;
+    if (is_pow2(w_scale)) {
+        AdResFwd<true>::Params p{{re_in, im_in}, {re_out, im_out, th_out, ref_out}, sin_decay, cos_decay, ref_decay,
+                                 th_decay, re_state, im_state, ref_state, th_state, (int)th_step_scaled,
+                                 (int)th0_scaled, w, 1.0f / w, neurons_per_batch, num_decays, num_ref_decays,
+                                 num_th_decays, num_re_states, num_im_states, num_ref_states, num_th_states};
+        return launch_stream<AdResFwd<true>>(p, M, T, st);
+    }
+    AdResFwd<false>::Params p{{re_in, im_in}, {re_out, im_out, th_out, ref_out}, sin_decay, cos_decay, ref_decay,
+                              th_decay, re_state, im_state, ref_state, th_state, (int)th_step_scaled,
+                              (int)th0_scaled, w, 1.0f / w, neurons_per_batch, num_decays, num_ref_decays,
+                              num_th_decays, num_re_states, num_im_states, num_ref_states, num_th_states};
+    return launch_stream<AdResFwd<false>>(p, M, T, st);
 }

@@ -39,6 +39,9 @@ _SIGNATURES = {
     'slayer_shift': (_INT, [_P, _P, _P, _I64, _F, _I64, _I64, _I64, _P]),
     'slayer_conv': (_INT, [_P, _P, _P, _I64, _F, _I64, _I64, _P]),
     'slayer_corr': (_INT, [_P, _P, _P, _I64, _F, _I64, _I64, _P]),
+    'slayer_apth_fwd': (_INT, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _INT,
+                               _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P]),
+    'slayer_adres_fwd': (_INT, [_P] * 14 + [_I64, _I64, _INT] + [_I64] * 10 + [_P]),
     'slayer_li_fwd_naive': (_INT, [_P, _P, _P, _P, _D, _INT, _I64, _I64, _I64, _I64, _I64, _P]),
     'slayer_li_bwd_naive': (_INT, [_P, _P, _P, _I64, _I64, _I64, _I64, _P]),
     'slayer_ath_fwd_naive': (_INT, [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _INT,

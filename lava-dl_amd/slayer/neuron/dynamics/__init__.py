@@ -1,3 +1,3 @@
-from . import leaky_integrator, adaptive_threshold, resonator
+from . import leaky_integrator, adaptive_threshold, resonator, adaptive_phase_th, adaptive_resonator
 
-__all__ = ['leaky_integrator', 'adaptive_threshold', 'resonator']
+__all__ = ['leaky_integrator', 'adaptive_threshold', 'resonator', 'adaptive_phase_th', 'adaptive_resonator']

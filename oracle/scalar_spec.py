@@ -11,6 +11,8 @@ Rules restated (citations relative to /root/reference/src/lava/lib/dl/slayer/):
   LI        neuron/dynamics/leaky_integrator.py:214-231
   ATH       neuron/dynamics/adaptive_threshold.py:243-274
   RES       neuron/dynamics/resonator.py:343-376
+  APTH      neuron/dynamics/adaptive_phase_th.py:241-284
+  ADRES     neuron/dynamics/adaptive_resonator.py:386-436
 """
 
 import numpy as np
@@ -86,3 +88,56 @@ def res(xr, xi, sin_decay, cos_decay, re_state, im_state, w, threshold=None):
         else:
             re, im = re_n, im_n
     return re_out, im_out, fired_seq
+
+
+def apth(xr, xi, im_state, ref_state, ref_decay, th_state, th_decay, th_scale, th0, w):
+    """neuron/dynamics/adaptive_phase_th.py:241-284.  Returns (threshold, refractory, spikes)."""
+    th = to_int(f32(th_state) * f32(w))
+    r = to_int(f32(ref_state) * f32(w))
+    mt = 4096 - to_int(th_decay)
+    mr = 4096 - to_int(ref_decay)
+    step = int(th_scale * w)
+    base = int(th0 * w)
+    im_old = to_int(f32(w) * f32(im_state))
+    th_out, r_out, fired_seq = [], [], []
+    for a, b in zip(xr, xi):
+        r = trunc_div_4096(r * mr)
+        th = trunc_div_4096((th - base) * mt) + base
+        th_out.append(f32(th) / f32(w))
+        r_out.append(f32(r) / f32(w))
+        re, im = to_int(f32(w) * f32(a)), to_int(f32(w) * f32(b))
+        fired = re >= th + r and im >= 0 and im_old < 0
+        fired_seq.append(bool(fired))
+        if fired:
+            r += 2 * th
+            th += step
+        im_old = im
+    return th_out, r_out, fired_seq
+
+
+def adres(xr, xi, sin_decay, cos_decay, ref_decay, th_decay, re_state, im_state, ref_state, th_state,
+          th_scale, th0, w):
+    """neuron/dynamics/adaptive_resonator.py:386-436.  Returns (re, im, threshold, refractory, spikes)."""
+    re = to_int(f32(re_state) * f32(w))
+    im = to_int(f32(im_state) * f32(w))
+    th = to_int(f32(th_state) * f32(w))
+    r = to_int(f32(ref_state) * f32(w))
+    s, c = to_int(sin_decay), to_int(cos_decay)
+    mt = 4096 - to_int(th_decay)
+    mr = 4096 - to_int(ref_decay)
+    step = int(th_scale * w)
+    base = int(th0 * w)
+    outs = ([], [], [], [], [])
+    for a, b in zip(xr, xi):
+        r = trunc_div_4096(r * mr)
+        th = trunc_div_4096((th - base) * mt) + base
+        re, im = (trunc_div_4096(c * re) - trunc_div_4096(s * im) + to_int(f32(w) * f32(a)),
+                  trunc_div_4096(s * re) + trunc_div_4096(c * im) + to_int(f32(w) * f32(b)))
+        for o, v in zip(outs, (re, im, th, r)):
+            o.append(f32(v) / f32(w))
+        fired = im >= th + r
+        outs[4].append(bool(fired))
+        if fired:
+            r += 2 * th
+            th += step
+    return outs

@@ -16,6 +16,8 @@ Pin status (see tests/test_oracle_*.py):
                                   beyond 2**24 the float32 round trip of the reset
                                   expression is restated but PARITY UNPINNED
   ath_fwd                         scalar spec + closed forms + leak invariants
+  apth_fwd, adres_fwd             scalar spec; identity with the pinned pieces they are made of
+                                  (ath recurrences + complex spike condition; res_fwd + ath_fwd on imag)
   li_bwd, res_bwd                 torch autograd through a float IIR + scipy.signal.lfilter (float64)
   spike_bwd, cspike_bwd           closed forms evaluated in float64
   shift                           numpy slicing (the reference's own test_shift.py check)
@@ -169,6 +171,67 @@ def ath_persistent_ref_state(ref_state, spike, th_state):
 def ath_persistent_th_state(th_state, spike, th_step):
     """DYN/adaptive_threshold.py:154-172."""
     return th_state + (spike > 0).to(th_state.dtype) * th_step
+
+
+def apth_fwd(re_in, im_in, im_state, ref_state, ref_decay, th_state, th_decay, th_scale, th0, w_scale):
+    """Adaptive phase threshold forward.  DYN/adaptive_phase_th.py:51-131, 234-284.
+
+    Threshold / refractory recurrences of ath_fwd; the spike condition is
+    trunc(w*re) >= th + r  and  trunc(w*im) >= 0  and  previous trunc(w*im) < 0.
+    """
+    th_prev = (_full_state(th_state, re_in) * w_scale).detach().to(I64)
+    r_prev = (_full_state(ref_state, re_in) * w_scale).detach().to(I64)
+    th_mult = ONE - neuron_shaped(th_decay.detach(), re_in.shape).to(I64)
+    r_mult = ONE - neuron_shaped(ref_decay.detach(), re_in.shape).to(I64)
+    step = int(th_scale * w_scale)
+    base = int(th0 * w_scale)
+    im_old = (w_scale * _full_state(im_state, im_in)).to(I64)
+    th_out = torch.zeros_like(re_in)
+    r_out = torch.zeros_like(re_in)
+    for t in range(re_in.shape[-1]):
+        r = rs0(r_prev * r_mult)
+        th = rs0((th_prev - base) * th_mult) + base
+        re = (w_scale * re_in[..., t]).to(I64)
+        im = (w_scale * im_in[..., t]).to(I64)
+        fired = (re >= (th + r)) * (im >= 0) * (im_old < 0)
+        th_prev = th + step * (fired > 0.5)
+        r_prev = r + 2 * th * (fired > 0.5)
+        th_out[..., t] = th / w_scale
+        r_out[..., t] = r / w_scale
+        im_old = im
+    return th_out, r_out
+
+
+def adres_fwd(xr, xi, sin_decay, cos_decay, ref_decay, th_decay,
+              re_state, im_state, ref_state, th_state, th_scale, th0, w_scale):
+    """Adaptive resonator forward.  DYN/adaptive_resonator.py:49-158, 379-436.
+
+    res_fwd without reset, plus ath-style threshold / refractory recurrences whose spike
+    condition is the integer compare im >= th + r.  Backward is res_bwd (:439-520).
+    """
+    re_prev = (_full_state(re_state, xr) * w_scale).detach().to(I64)
+    im_prev = (_full_state(im_state, xi) * w_scale).detach().to(I64)
+    th_prev = (_full_state(th_state, xr) * w_scale).detach().to(I64)
+    r_prev = (_full_state(ref_state, xr) * w_scale).detach().to(I64)
+    s = neuron_shaped(sin_decay.detach(), xr.shape).to(I64)
+    c = neuron_shaped(cos_decay.detach(), xr.shape).to(I64)
+    th_mult = ONE - neuron_shaped(th_decay.detach(), xr.shape).to(I64)
+    r_mult = ONE - neuron_shaped(ref_decay.detach(), xr.shape).to(I64)
+    step = int(th_scale * w_scale)
+    base = int(th0 * w_scale)
+    outs = [torch.zeros_like(xr) for _ in range(4)]
+    for t in range(xr.shape[-1]):
+        r = rs0(r_prev * r_mult)
+        th = rs0((th_prev - base) * th_mult) + base
+        re = rs0(c * re_prev) - rs0(s * im_prev) + (w_scale * xr[..., t]).to(I64)
+        im = rs0(s * re_prev) + rs0(c * im_prev) + (w_scale * xi[..., t]).to(I64)
+        fired = (im >= (th + r)).to(I64)
+        re_prev, im_prev = re, im
+        th_prev = th + step * (fired > 0.5)
+        r_prev = r + 2 * th * (fired > 0.5)
+        for o, v in zip(outs, (re, im, th, r)):
+            o[..., t] = v / w_scale
+    return tuple(outs)
 
 
 # --------------------------------------------------------------------------

@@ -322,6 +322,52 @@ def test_res_autograd_and_nan_guard(slayer):
         torch.autograd.backward([re, im], [bad, torch.ones(shape, device=dev())])
 
 
+# ------------------------------------------------------------------------- APTH / adaptive RES
+@pytest.mark.parametrize('shape,kind,w', [((4, 128, 200), 'channel', 64), ((2, 3, 5, 7, 37), 'channel', 4096),
+                                          ((3, 70, 129), 'neuron', 100), ((4, 9000, 100), 'channel', 64),
+                                          ((4, 35000, 40), 'channel', 64), ((1, 5, 3), 'shared', 64)])
+def test_apth_and_adres_bit_exact(slayer, shape, kind, w):
+    gen = torch.Generator().manual_seed(seed_of(shape, kind, w, 'apth'))
+    xr = sparse_input(gen, shape, p=0.4, amp=3.0)
+    xi = torch.randn(shape, generator=gen)
+    rd, td = _decay(kind, shape, gen), _decay(kind, shape, gen)
+    sin, cos = _rot(kind, shape, gen)
+    st = lambda: torch.randn(shape[:-1], generator=gen)
+    ims, refs, ths, res = st(), st(), st() + 1.5, st()
+    D = slayer.neuron.dynamics
+    g = lambda t: t.to(dev())
+    r_th, r_ref = O.apth_fwd(xr, xi, ims, refs, rd, ths, td, 0.5, 1.0, w)
+    th, ref = D.adaptive_phase_th.dynamics(g(xr), g(xi), g(ims), g(refs), g(rd), g(ths), g(td), 0.5, 1.0, w)
+    assert_exact(th, r_th, f'apth threshold {shape}')
+    assert_exact(ref, r_ref, f'apth refractory {shape}')
+    want = O.adres_fwd(xr, xi, sin, cos, rd, td, res, ims, refs, ths, 0.5, 1.0, w)
+    got = D.adaptive_resonator.dynamics(g(xr), g(xi), g(sin), g(cos), g(rd), g(td), g(res), g(ims), g(refs),
+                                        g(ths), 0.5, 1.0, w)
+    for a, b, name in zip(got, want, ('real', 'imag', 'threshold', 'refractory')):
+        assert_exact(a, b, f'adres {name} {shape}')
+
+
+def test_adres_autograd(slayer):
+    gen = torch.Generator().manual_seed(91)
+    shape = (2, 8, 60)
+    xr = sparse_input(gen, shape, p=0.3).to(dev()).requires_grad_()
+    xi = sparse_input(gen, shape, p=0.3).to(dev()).requires_grad_()
+    sin = torch.full((8,), 2103.0, device=dev(), requires_grad=True)
+    cos = torch.full((8,), 3273.0, device=dev(), requires_grad=True)
+    d = torch.full((8,), 200.0, device=dev())
+    zero, one = torch.zeros(1, device=dev()), torch.ones(1, device=dev())
+    re, im, th, ref = slayer.neuron.dynamics.adaptive_resonator.dynamics(xr, xi, sin, cos, d, d, zero, zero, zero,
+                                                                         one, 0.5, 1.0, 64)
+    assert not th.requires_grad and not ref.requires_grad
+    (re.sum() + 2 * im.sum()).backward()
+    want = O.res_bwd(torch.ones(shape), 2 * torch.ones(shape), re.detach().cpu(), im.detach().cpu(),
+                     sin.detach().cpu(), cos.detach().cpu())
+    assert_exact(xr.grad, want[0], 'adres grad real')
+    assert_exact(xi.grad, want[1], 'adres grad imag')
+    assert_rel(sin.grad, want[2], 'adres grad sin', rel=1e-4)
+    assert_rel(cos.grad, want[3], 'adres grad cos', rel=1e-4)
+
+
 # --------------------------------------------------------------------------------- debug mode
 def test_debug_mode_cross_check_passes_and_catches_overflow(slayer):
     """debug=True runs the independent one-thread-per-neuron kernels (64-bit state) next to the

@@ -193,6 +193,64 @@ def test_ath_closed_forms():
     assert ref[0, 0].tolist() == [0.0, 2.0, 2.0]
 
 
+def test_apth_matches_scalar_spec_and_its_parts():
+    rng = np.random.default_rng(25)
+    T, C, w = 80, len(DECAYS), 64
+    xr = _rand_input(rng, (2, C, T), p=0.6, amp=3.0)
+    xi = torch.tensor(rng.standard_normal((2, C, T)), dtype=torch.float32)
+    rd, td = torch.tensor(DECAYS), torch.tensor(DECAYS[::-1])
+    th_state = torch.tensor(rng.random((2, C)) * 2, dtype=torch.float32)
+    ref_state = torch.tensor(rng.standard_normal((2, C)), dtype=torch.float32)
+    im_state = torch.tensor(rng.standard_normal((2, C)), dtype=torch.float32)
+    th, ref = O.apth_fwd(xr, xi, im_state, ref_state, rd, th_state, td, 0.5, 1.0, w)
+    spikes = 0
+    for n, c in itertools.product(range(2), range(C)):
+        t_ref, r_ref, fired = S.apth(xr[n, c].tolist(), xi[n, c].tolist(), float(im_state[n, c]),
+                                     float(ref_state[n, c]), DECAYS[c], float(th_state[n, c]),
+                                     DECAYS[::-1][c], 0.5, 1.0, w)
+        spikes += sum(fired)
+        assert np.array_equal(th[n, c].numpy(), np.array(t_ref, dtype=np.float32))
+        assert np.array_equal(ref[n, c].numpy(), np.array(r_ref, dtype=np.float32))
+    assert spikes > 0
+    # with an imaginary part that always crosses zero upwards the op reduces to ath_fwd on the real part
+    zig = torch.ones(2, C, T)
+    zig[..., ::2] = -1.0
+    up = torch.cat([-torch.ones(2, C, 1), zig[..., :-1]], -1)        # previous sample of each step
+    only_up = (zig >= 0) & (up < 0)
+    th_a, ref_a = O.apth_fwd(torch.where(only_up, xr, torch.full_like(xr, -100.0)), zig, -torch.ones(2, C),
+                             ref_state, rd, th_state, td, 0.5, 1.0, w)
+    th_b, ref_b = O.ath_fwd(torch.where(only_up, xr, torch.full_like(xr, -100.0)), ref_state, rd, th_state, td,
+                            0.5, 1.0, w)
+    assert torch.equal(th_a, th_b) and torch.equal(ref_a, ref_b)
+
+
+def test_adres_matches_scalar_spec_and_its_parts():
+    rng = np.random.default_rng(26)
+    T, w = 70, 64
+    sin = [2103.0, 1.0, 3000.5, -2000.0]
+    cos = [3273.0, 4095.0, 0.0, 2500.0]
+    rdl, tdl = [0.0, 100.0, 4096.0, 2000.0], [4095.0, 50.0, 0.0, 1234.0]
+    C = len(sin)
+    xr, xi = _rand_input(rng, (2, C, T)), _rand_input(rng, (2, C, T))
+    st = lambda: torch.tensor(rng.standard_normal((2, C)), dtype=torch.float32)
+    rs, is_, refs, ths = st(), st(), st(), st() + 1.5
+    outs = O.adres_fwd(xr, xi, torch.tensor(sin), torch.tensor(cos), torch.tensor(rdl), torch.tensor(tdl),
+                       rs, is_, refs, ths, 0.5, 1.0, w)
+    spikes = 0
+    for n, c in itertools.product(range(2), range(C)):
+        ref = S.adres(xr[n, c].tolist(), xi[n, c].tolist(), sin[c], cos[c], rdl[c], tdl[c],
+                      float(rs[n, c]), float(is_[n, c]), float(refs[n, c]), float(ths[n, c]), 0.5, 1.0, w)
+        spikes += sum(ref[4])
+        for got, want in zip(outs, ref[:4]):
+            assert np.array_equal(got[n, c].numpy(), np.array(want, dtype=np.float32))
+    assert spikes > 0
+    # it is the resonator followed by the adaptive threshold driven by the imaginary trace
+    re, im = O.res_fwd(xr, xi, torch.tensor(sin), torch.tensor(cos), rs, is_, w)
+    th, ref = O.ath_fwd(im, refs, torch.tensor(rdl), ths, torch.tensor(tdl), 0.5, 1.0, w)
+    for got, want in zip(outs, (re, im, th, ref)):
+        assert torch.equal(got, want)
+
+
 # ----------------------------------------------------------------------- RES
 @pytest.mark.parametrize('thr', [None, 0.0, 1.5, 2.3])
 def test_res_matches_scalar_spec(thr):
