@@ -198,6 +198,40 @@ int slayer_conv(float *out, const float *in, const float *filt, int64_t K, float
 int slayer_corr(float *out, const float *in, const float *filt, int64_t K, float sampling_time,
                 int64_t M, int64_t T, void *stream);
 
+/* ---- sigma-delta ---------------------------------------------------------------------------- */
+
+/* _DeltaUnit.forward (axon/delta.py:10-66; a python time loop in the reference, no kernel there):
+ * delta = in[t] - pre + residual;  delta_out[t] = delta;
+ * cum_error == 0:  y = |delta| >= thr ? delta : 0;
+ * cum_error != 0:  error += delta;  y = |error| >= thr ? delta : 0;  error = 0 after an event;
+ * residual = delta - y;  pre = in[t].  out[t] = y, or floor(y / quant_step) * quant_step when
+ * quant_step > 0 (the floor quantiser Delta.forward applies to its result, axon/delta.py:318).
+ * residual_out / error_out receive the final states (M floats each).  threshold follows the decay
+ * addressing (one value or one per channel); states are one value or M. */
+int slayer_delta_fwd(float *out, float *delta_out, float *residual_out, float *error_out,
+                     const float *in, const float *threshold, const float *pre_state,
+                     const float *residual_state, const float *error_state,
+                     int cum_error, float quant_step,
+                     int64_t M, int64_t neurons_per_batch, int64_t num_thresholds,
+                     int64_t num_pre, int64_t num_residual, int64_t num_error,
+                     int64_t T, void *stream);
+
+/* _DeltaUnit.backward (axon/delta.py:68-103): grad_in[t] = grad_out[t] - grad_out[t+1];
+ * grad_threshold[j] = sum of (|d| - thr > 0 ? -d * scale_grad * exp(-||d| - thr| / tau_grad) / thr
+ *                                          : -sign(d)) * grad_out over the neurons of threshold j.
+ * grad_threshold may be NULL; workspace: M + 64 * num_thresholds floats when it is not. */
+int slayer_delta_bwd(float *grad_in, float *grad_threshold, const float *grad_out,
+                     const float *delta, const float *threshold, float *workspace,
+                     float tau_grad, float scale_grad,
+                     int64_t M, int64_t neurons_per_batch, int64_t num_thresholds,
+                     int64_t T, void *stream);
+
+/* Running sum along time, sequential float32 adds (dendrite/sigma.py:63 uses torch.cumsum):
+ * out[t] = state + in[0] + ... + in[t]; reverse != 0 sums from the last step backwards (the
+ * gradient of the forward sum).  state == NULL starts from 0. */
+int slayer_cumsum(float *out, const float *in, const float *state, int64_t num_states,
+                  int reverse, int64_t M, int64_t T, void *stream);
+
 /* ---- cross-check implementations (debug mode) ------------------------------------------------ */
 
 /* The reference's debug mode runs its CPU loop next to its kernel and raises on a difference

@@ -1,0 +1,184 @@
+// Sigma-delta pair: delta encoder (difference + threshold, float state per neuron) forward and
+// backward, and the running sum of the sigma decoder in both time directions.  Same neuron x
+// time-chunk staging as the integer dynamics; the arithmetic is float32 in the reference's order.
+#include "common.h"
+#include "tile.h"
+
+namespace slayer {
+
+int launch_reduce_param_grad(float* grad, const float* partial, float* scratch, int64_t M, int64_t npb,
+                             int64_t num_params, hipStream_t stream);   // li.hip
+int launch_zero_fill(float* p, int64_t n, hipStream_t stream);          // li.hip
+
+template <bool CUM, bool QUANT>
+struct DeltaFwd {
+    static constexpr int kIn = 1, kOut = 2;          // out: (quantised) events, delta before thresholding
+    static constexpr bool kReverse = false;
+    static constexpr int64_t kRows32Below = kAlways, kRows16Below = 65536;
+    struct Params {
+        const float* in[1];
+        float* out[2];
+        const float *threshold, *pre_state, *residual_state, *error_state;
+        float *residual_out, *error_out;             // final states, one per neuron
+        float step;                                  // quantisation step of the events (QUANT)
+        int64_t npb, n_thr, n_pre, n_res, n_err;
+    };
+    float pre, residual, error, thr, q;
+
+    __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
+        pre = residual = error = 0.f; thr = 1.f; q = p.step;
+        if (valid) {
+            pre = p.pre_state[p.n_pre == 1 ? 0 : m];
+            residual = p.residual_state[p.n_res == 1 ? 0 : m];
+            error = p.error_state[p.n_err == 1 ? 0 : m];
+            thr = p.threshold[param_index(m, p.npb, p.n_thr)];
+        }
+    }
+    __device__ __forceinline__ void step(const float (&x)[1], float (&o)[2]) {
+        const float delta = (x[0] - pre) + residual;
+        float y;
+        if (CUM) {
+            error = error + delta;
+            y = (fabsf(error) >= thr) ? delta : 0.0f * delta;
+            error = error * ((fabsf(y) > 0.0f) ? 0.0f : 1.0f);
+        } else {
+            y = (fabsf(delta) >= thr) ? delta : 0.0f * delta;
+        }
+        residual = delta - y;
+        pre = x[0];
+        o[0] = QUANT ? floorf(y / q) * q : y;
+        o[1] = delta;
+    }
+    __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
+        if (valid) { p.residual_out[m] = residual; p.error_out[m] = error; }
+    }
+};
+
+struct DeltaBwd {
+    static constexpr int kIn = 2, kOut = 1;          // in: grad of the events, saved delta;  out: grad_input
+    static constexpr bool kReverse = true;
+    static constexpr int64_t kRows32Below = kAlways, kRows16Below = kAlways;
+    struct Params {
+        const float* in[2];
+        float* out[1];
+        const float* threshold;
+        float* partial;                              // per-neuron threshold gradient, or nullptr
+        float tau, scale;
+        int64_t npb, n_thr;
+    };
+    float g_next, acc, thr, tau, scale;
+
+    __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
+        g_next = acc = 0.f; thr = 1.f; tau = p.tau; scale = p.scale;
+        if (valid) thr = p.threshold[param_index(m, p.npb, p.n_thr)];
+    }
+    __device__ __forceinline__ void step(const float (&x)[2], float (&o)[1]) {
+        const float g = x[0], d = x[1];
+        o[0] = g - g_next;                           // grad[t] - grad[t+1]; the last step sees 0
+        g_next = g;
+        const float sub = fabsf(d) - thr;
+        const float sgn = d > 0.f ? 1.f : (d < 0.f ? -1.f : d);
+        const float gth = (sub > 0.f) ? ((-d) * (scale * expf(-fabsf(sub) / tau))) / thr : -sgn;
+        acc += gth * g;
+    }
+    __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
+        if (valid && p.partial) p.partial[m] = acc;
+    }
+};
+
+template <bool REVERSE>
+struct RunningSum {
+    static constexpr int kIn = 1, kOut = 1;
+    static constexpr bool kReverse = REVERSE;
+    static constexpr int64_t kRows32Below = kAlways, kRows16Below = kAlways;
+    struct Params {
+        const float* in[1];
+        float* out[1];
+        const float* state;                          // initial value per neuron, or nullptr for 0
+        int64_t n_state;
+    };
+    float y;
+    __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
+        y = (valid && p.state) ? p.state[p.n_state == 1 ? 0 : m] : 0.f;
+    }
+    __device__ __forceinline__ void step(const float (&x)[1], float (&o)[1]) { y = y + x[0]; o[0] = y; }
+    __device__ __forceinline__ void finish(const Params&, int64_t, bool) {}
+};
+
+template <bool CUM, bool QUANT>
+static int delta_fwd_launch(const typename DeltaFwd<CUM, QUANT>::Params& p, int64_t M, int64_t T, hipStream_t st) {
+    return launch_stream<DeltaFwd<CUM, QUANT>>(p, M, T, st);
+}
+
+}  // namespace slayer
+
+using namespace slayer;
+
+extern "C" int slayer_delta_fwd(float* out, float* delta_out, float* residual_out, float* error_out,
+                                const float* in, const float* threshold, const float* pre_state,
+                                const float* residual_state, const float* error_state,
+                                int cum_error, float quant_step,
+                                int64_t M, int64_t neurons_per_batch, int64_t num_thresholds,
+                                int64_t num_pre, int64_t num_residual, int64_t num_error,
+                                int64_t T, void* stream) {
+    if (int e = check_rows(M, T)) return e;
+    if (M == 0) return 0;
+    if (!residual_out || !error_out || !threshold || !pre_state || !residual_state || !error_state) return SLAYER_ENULL;
+    if (T > 0 && (!out || !delta_out || !in)) return SLAYER_ENULL;
+    if (int e = check_params(M, neurons_per_batch, num_thresholds)) return e;
+    for (int64_t n : {num_pre, num_residual, num_error})
+        if (int e = check_states(M, n)) return e;
+    if (T == 0) return SLAYER_EINVAL;                // the final states would not be defined by a launch
+    hipStream_t st = (hipStream_t)stream;
+    const bool quant = quant_step > 0.0f;
+#define SLAYER_DELTA(C, Q)                                                                                      \
+    do {                                                                                                        \
+        DeltaFwd<C, Q>::Params p{{in}, {out, delta_out}, threshold, pre_state, residual_state, error_state,       \
+                                 residual_out, error_out, quant_step, neurons_per_batch, num_thresholds,         \
+                                 num_pre, num_residual, num_error};                                              \
+        return delta_fwd_launch<C, Q>(p, M, T, st);                                                              \
+    } while (0)
+    if (cum_error) { if (quant) SLAYER_DELTA(true, true); else SLAYER_DELTA(true, false); }
+    if (quant) SLAYER_DELTA(false, true);
+    SLAYER_DELTA(false, false);
+#undef SLAYER_DELTA
+}
+
+extern "C" int slayer_delta_bwd(float* grad_in, float* grad_threshold, const float* grad_out,
+                                const float* delta, const float* threshold, float* workspace,
+                                float tau_grad, float scale_grad,
+                                int64_t M, int64_t neurons_per_batch, int64_t num_thresholds,
+                                int64_t T, void* stream) {
+    if (int e = check_rows(M, T)) return e;
+    if (int e = check_params(M > 0 ? M : neurons_per_batch, neurons_per_batch, num_thresholds)) return e;
+    if (grad_threshold && !workspace && M > 0) return SLAYER_ENULL;
+    hipStream_t st = (hipStream_t)stream;
+    if (M > 0 && T > 0) {
+        if (!grad_in || !grad_out || !delta || !threshold) return SLAYER_ENULL;
+        DeltaBwd::Params p{{grad_out, delta}, {grad_in}, threshold, grad_threshold ? workspace : nullptr,
+                           tau_grad, scale_grad, neurons_per_batch, num_thresholds};
+        if (int e = launch_stream<DeltaBwd>(p, M, T, st)) return e;
+    }
+    if (grad_threshold) {
+        if (M == 0 || T == 0) return launch_zero_fill(grad_threshold, num_thresholds, st);
+        return launch_reduce_param_grad(grad_threshold, workspace, workspace + M, M, neurons_per_batch,
+                                        num_thresholds, st);
+    }
+    return 0;
+}
+
+extern "C" int slayer_cumsum(float* out, const float* in, const float* state, int64_t num_states,
+                             int reverse, int64_t M, int64_t T, void* stream) {
+    if (int e = check_rows(M, T)) return e;
+    if (M == 0 || T == 0) return 0;
+    if (!out || !in) return SLAYER_ENULL;
+    if (state)
+        if (int e = check_states(M, num_states)) return e;
+    hipStream_t st = (hipStream_t)stream;
+    if (reverse) {
+        RunningSum<true>::Params p{{in}, {out}, state, num_states};
+        return launch_stream<RunningSum<true>>(p, M, T, st);
+    }
+    RunningSum<false>::Params p{{in}, {out}, state, num_states};
+    return launch_stream<RunningSum<false>>(p, M, T, st);
+}

@@ -355,7 +355,9 @@ __global__ __launch_bounds__(kWave) void stream_kernel_scalar(typename Op::Param
                     float x[NI], y[NO];
 #pragma unroll
                     for (int i = 0; i < NI; ++i) x[i] = xin[i][ss];
-                    op.step(x, y);
+#pragma unroll
+                    for (int o = 0; o < NO; ++o) y[o] = 0.f;
+                    if (chunk * TC + 4 * qq + ss < T) op.step(x, y);   // steps past T-1 must not touch the state
 #pragma unroll
                     for (int o = 0; o < NO; ++o) yout[o][ss] = y[o];
                 }

@@ -1,3 +1,4 @@
 from .delay import delay, Delay
+from .delta import Delta
 
-__all__ = ['delay', 'Delay']
+__all__ = ['delay', 'Delay', 'Delta']

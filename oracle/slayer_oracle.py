@@ -23,6 +23,8 @@ Pin status (see tests/test_oracle_*.py):
   shift                           numpy slicing (the reference's own test_shift.py check)
   conv_fwd / conv_bwd             numpy.convolve (the reference's own test_conv_filter.py check)
   delay_bwd                       finite-difference identity on the conv([-1,1]) form
+  delta_fwd / delta_bwd, sigma    hand-computed sequences, reconstruction invariant |x - sigma(delta(x))| < threshold,
+                                  float64 closed forms of the threshold gradient, numpy.cumsum
 """
 
 import numpy as np
@@ -439,3 +441,64 @@ def delay_bwd(grad_out, out, delay_val, grad_scale=1, sampling_time=1):
         .reshape(grad_out.shape[1:-1]) * sampling_time
     neg = -delay_val if torch.is_tensor(delay_val) else -delay_val
     return shift(grad_out, neg, sampling_time), g_delay * grad_scale
+
+
+# --------------------------------------------------------------------------
+# sigma-delta
+# --------------------------------------------------------------------------
+def delta_fwd(x, threshold, pre_state, residual_state, error_state, cum_error=False):
+    """Delta unit forward.  S/axon/delta.py:10-46.  Returns (events, delta_input, residual, error)."""
+    out = torch.zeros_like(x)
+    delta_input = torch.zeros_like(x)
+    pre = pre_state * torch.ones(x.shape[:-1])
+    residual = residual_state * torch.ones(x.shape[:-1])
+    error = (error_state * torch.ones(x.shape[:-1])).clone()
+    for t in range(x.shape[-1]):
+        delta = x[..., t] - pre + residual
+        delta_input[..., t] = delta
+        if cum_error:
+            error = error + delta
+            out[..., t] = torch.where(torch.abs(error) >= threshold, delta, 0 * delta)
+            error = error * (1 - (torch.abs(out[..., t]) > 0).to(x.dtype))
+        else:
+            out[..., t] = torch.where(torch.abs(delta) >= threshold, delta, 0 * delta)
+        residual = delta - out[..., t]
+        pre = x[..., t]
+    return out, delta_input, residual, error
+
+
+def delta_bwd(grad_out, delta_input, threshold, tau_grad, scale_grad):
+    """Delta unit backward.  S/axon/delta.py:68-103.  threshold has 1 or C elements.
+
+    The reference subtracts its [C, 1, ...] threshold from the [N, C, ..., T] delta without
+    adding the time axis, which mis-broadcasts (or raises) for per-channel thresholds; the
+    per-channel alignment its forward pass uses is what is restated here.
+    """
+    tau = torch.tensor(tau_grad, dtype=grad_out.dtype)
+    scale = torch.tensor(scale_grad, dtype=grad_out.dtype)
+    thr = threshold if threshold.numel() == 1 else threshold.reshape([-1] + [1] * (delta_input.dim() - 2))
+    sub = torch.abs(delta_input) - thr
+    g_thr = torch.where(sub > 0, -delta_input * (scale * torch.exp(-torch.abs(sub) / tau)) / thr,
+                        -torch.sign(delta_input)) * grad_out
+    g_in = torch.zeros_like(grad_out)
+    g_in[..., :-1] = grad_out[..., :-1] - grad_out[..., 1:]
+    g_in[..., -1] = grad_out[..., -1]
+    if threshold.numel() == 1:
+        g_thr = torch.unsqueeze(torch.sum(g_thr), dim=0)
+    else:
+        g_thr = torch.sum(g_thr.reshape(delta_input.shape[0], delta_input.shape[1], -1), dim=[0, -1]) \
+            .reshape(threshold.shape)
+    return g_in, g_thr
+
+
+def quantize_floor(x, step):
+    """S/utils/quantize.py:38-48 (forward of the floor quantiser)."""
+    return torch.floor(x / step) * step
+
+
+def sigma_fwd(x, pre_state=None):
+    """Sigma decoder.  S/dendrite/sigma.py:63-70: cumulative sum along time (+ carried state)."""
+    out = torch.cumsum(x, dim=-1)
+    if pre_state is not None:
+        out = out + pre_state.unsqueeze(-1)
+    return out

@@ -131,3 +131,85 @@ def test_delay_module(slayer):
     assert_rel(mod.delay.grad, ref_gd.sum(dim=1), 'delay grad_delay', rel=1e-4)
     # functional form, default one step
     assert_exact(slayer.axon.delay(x.to(dev())), O.shift(x, 1), 'delay()')
+
+
+# --------------------------------------------------------------------------------- sigma-delta
+@pytest.mark.parametrize('shape', [(3, 6, 200), (2, 3, 5, 7, 37), (4, 70, 129), (1, 5, 3), (4, 9000, 64)])
+@pytest.mark.parametrize('cum', [False, True])
+def test_delta_unit_and_sigma(slayer, shape, cum):
+    from lava_dl_amd.slayer.axon import delta as D
+    from lava_dl_amd.slayer.dendrite import sigma as SG
+    gen = torch.Generator().manual_seed(seed_of(shape, cum, 'delta'))
+    x = torch.cumsum(torch.randn(shape, generator=gen) * 0.3, dim=-1)
+    C = shape[1]
+    st = lambda: torch.randn(shape[:-1], generator=gen) * 0.2
+    pre, res, err = st(), st(), st() * 0
+    for thr in (torch.tensor([0.5]), (0.3 + torch.rand(C, generator=gen)).reshape([C] + [1] * (len(shape) - 3))):
+        r_out, r_din, r_res, r_err = O.delta_fwd(x, thr, pre, res, err, cum)
+        out, din, res_o, err_o = D._fwd(x.to(dev()), thr.to(dev()), pre.to(dev()), res.to(dev()), err.to(dev()), cum)
+        assert_exact(out, r_out, f'delta events {shape}')
+        assert_exact(din, r_din, f'delta input {shape}')
+        assert_exact(res_o, r_res, 'delta residual')
+        assert_exact(err_o, r_err, 'delta error')
+        outq = D._fwd(x.to(dev()), thr.to(dev()), pre.to(dev()), res.to(dev()), err.to(dev()), cum, 1 / 64)[0]
+        assert_exact(outq, O.quantize_floor(r_out, 1 / 64), 'delta quantised events')
+        g = torch.randn(shape, generator=gen)
+        w_in, w_thr = O.delta_bwd(g, r_din, thr, 0.8, 1.5)
+        g_in, g_thr = D._bwd(g.to(dev()), din, thr.to(dev()), 0.8, 1.5)
+        assert_exact(g_in, w_in, 'delta grad_input')
+        assert_rel(g_thr.reshape(w_thr.shape), w_thr, 'delta grad_threshold', rel=1e-4)
+    # running sum: float-mode against torch's cumsum, exact against strictly sequential float32 adds,
+    # and exact against torch's cumsum on quantised events (multiples of 1/64 add without rounding)
+    assert_rel(SG._cumsum(out), O.sigma_fwd(r_out), 'sigma running sum')
+    assert_exact(SG._cumsum(out), _seq_cumsum(r_out, torch.zeros(shape[:-1])), 'sigma sequential sum')
+    assert_exact(SG._cumsum(out, pre.to(dev())), _seq_cumsum(r_out, pre), 'sigma with carried state')
+    rq = O.quantize_floor(r_out, 1 / 64)
+    assert_exact(SG._cumsum(outq), O.sigma_fwd(rq), 'sigma on quantised events')
+    assert_exact(SG._cumsum(outq, None, reverse=True), torch.flip(O.sigma_fwd(torch.flip(rq, [-1])), [-1]),
+                 'sigma reverse sum')
+
+
+def _seq_cumsum(x, start):
+    """Sequential float32 running sum that starts from ``start`` (the kernel adds the state first)."""
+    out = torch.zeros_like(x)
+    y = start.clone()
+    for t in range(x.shape[-1]):
+        y = y + x[..., t]
+        out[..., t] = y
+    return out
+
+
+def test_delta_sigma_modules(slayer):
+    gen = torch.Generator().manual_seed(90)
+    x = torch.cumsum(torch.randn((2, 4, 3, 150), generator=gen) * 0.3, dim=-1)
+    for shared, cum in ((True, False), (False, True)):
+        enc = slayer.axon.Delta(threshold=0.5, cum_error=cum, shared_param=shared, requires_grad=True).to(dev())
+        dec = slayer.dendrite.Sigma().to(dev())
+        xg = x.to(dev()).requires_grad_()
+        ev = enc(xg)
+        thr = enc.threshold.detach().cpu()
+        zero = torch.zeros(x.shape[:-1])
+        r_out, r_din, _, _ = O.delta_fwd(x, thr, zero, zero, zero, cum)
+        assert_exact(ev, O.quantize_floor(r_out, 1 / 64), 'Delta module events')
+        y = dec(ev)
+        assert_exact(y, O.sigma_fwd(O.quantize_floor(r_out, 1 / 64)), 'Sigma module output')
+        g = torch.randn(x.shape, generator=gen)
+        y.backward(g.to(dev()))
+        # gradient of the running sum = running sum from the last step backwards (sequential float32 adds;
+        # a differently grouped sum would differ by an ulp of the partial sums, which the time difference
+        # in the delta backward then magnifies)
+        g_ev = torch.flip(_seq_cumsum(torch.flip(g, [-1]), torch.zeros(x.shape[:-1])), [-1])
+        w_in, w_thr = O.delta_bwd(g_ev, r_din, thr, 1, 1)
+        assert_exact(xg.grad, w_in, 'Delta module grad_input')
+        assert enc.threshold.grad.shape == enc.threshold.shape
+        assert_rel(enc.threshold.grad.reshape(w_thr.shape), w_thr, 'Delta module grad_threshold', rel=1e-4)
+    # persistent state: two halves equal one pass
+    enc_full = slayer.axon.Delta(0.5).to(dev())
+    enc_split = slayer.axon.Delta(0.5, persistent_state=True).to(dev())
+    dec_split = slayer.dendrite.Sigma(persistent_state=True).to(dev())
+    xg = x.to(dev())
+    full = enc_full(xg)
+    a, b = enc_split(xg[..., :70].contiguous()), enc_split(xg[..., 70:].contiguous())
+    assert torch.equal(torch.cat([a, b], -1), full)
+    ya, yb = dec_split(a), dec_split(b)
+    assert torch.equal(torch.cat([ya, yb], -1), slayer.dendrite.Sigma().to(dev())(full))

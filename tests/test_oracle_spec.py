@@ -454,3 +454,64 @@ def test_delay_bwd():
     diff[..., 0] = -o[..., 0]
     diff[..., 1:] = o[..., :-1] - o[..., 1:]
     assert np.allclose(gd.numpy(), 2.0 * (g.double().numpy() * diff).sum(axis=(0, 2)), rtol=1e-5, atol=1e-6)
+
+
+# --------------------------------------------------------------------------------- sigma-delta
+def test_delta_hand_sequences_and_reconstruction():
+    z = torch.zeros(1, 1)
+    x = torch.tensor([[[0.0, 0.4, 0.9, 1.0, 1.0, 0.2, -1.0]]])
+    thr = torch.tensor([0.5])
+    out, d_in, res, err = O.delta_fwd(x, thr, z, z, z)
+    # changes: .4 (kept as residual), .5+.4=.9 (event), .1 (residual), 0+.1 (residual .1), -.8+.1=-.7 (event), -1.2 (event)
+    assert np.allclose(out[0, 0].numpy(), [0, 0, 0.9, 0, 0, -0.7, -1.2], atol=1e-6)
+    assert np.allclose(d_in[0, 0].numpy(), [0, 0.4, 0.9, 0.1, 0.1, -0.7, -1.2], atol=1e-6)
+    assert abs(res.item()) < 1e-6
+    # cumulative error: 0.2 stays below 0.5 (residual 0.2); the next change 0.2 + 0.2 brings the error to 0.6,
+    # an event of 0.4 fires and the error restarts; the pattern repeats
+    x = torch.tensor([[[0.2, 0.4, 0.6, 0.8]]])
+    out, _, _, err = O.delta_fwd(x, thr, z, z, z, cum_error=True)
+    assert np.allclose(out[0, 0].numpy(), [0, 0.4, 0, 0.4], atol=1e-6) and abs(err.item()) < 1e-6
+    # without the cumulative error the same input never reaches the threshold in one step until the residual does
+    out, _, _, _ = O.delta_fwd(x, thr, z, z, z, cum_error=False)
+    assert np.allclose(out[0, 0].numpy(), [0, 0, 0.6, 0], atol=1e-6)
+    # reconstruction: the decoder follows the signal within one threshold, exactly where an event fired
+    rng = np.random.default_rng(80)
+    x = torch.tensor(np.cumsum(rng.standard_normal((3, 5, 200)) * 0.3, axis=-1), dtype=torch.float32)
+    zero = torch.zeros(3, 5)
+    for cum in (False, True):
+        out, _, res, _ = O.delta_fwd(x, thr, zero, zero, zero, cum)
+        rec = O.sigma_fwd(out)
+        assert float((x - rec).abs().max()) < (0.5 if not cum else 3.0) + 1e-4
+        fired = out != 0
+        assert fired.any()
+        if not cum:
+            assert float((x - rec)[fired].abs().max()) < 1e-4
+            assert np.allclose(res.numpy(), (x - rec)[..., -1].numpy(), atol=1e-4)
+    # carried state: splitting time gives the same events
+    out, _, _, _ = O.delta_fwd(x, thr, zero, zero, zero)
+    a, _, res_a, err_a = O.delta_fwd(x[..., :77], thr, zero, zero, zero)
+    b, _, _, _ = O.delta_fwd(x[..., 77:], thr, x[..., 76], res_a, err_a)
+    assert torch.equal(torch.cat([a, b], -1), out)
+    # torch's CPU cumsum does not add strictly one float32 at a time, so the running sum is a float-mode
+    # quantity (1e-5 relative); on event values that are multiples of 1/64 every order gives the same bits
+    assert np.allclose(O.sigma_fwd(out).numpy(), np.cumsum(out.double().numpy(), axis=-1), rtol=1e-5, atol=1e-5)
+    q = O.quantize_floor(out, 1 / 64)
+    assert np.array_equal(O.sigma_fwd(q).numpy(), np.cumsum(q.double().numpy(), axis=-1).astype(np.float32))
+
+
+def test_delta_bwd_closed_form():
+    rng = np.random.default_rng(81)
+    d = torch.tensor(rng.standard_normal((2, 3, 4, 30)), dtype=torch.float32)
+    g = torch.tensor(rng.standard_normal((2, 3, 4, 30)), dtype=torch.float32)
+    for thr in (torch.tensor([0.7]), torch.tensor([0.3, 0.7, 1.1]).reshape(3, 1)):
+        g_in, g_thr = O.delta_bwd(g, d, thr, 0.8, 1.5)
+        gn = g.double().numpy()
+        ref_in = gn.copy()
+        ref_in[..., :-1] -= gn[..., 1:]
+        assert np.allclose(g_in.numpy(), ref_in, atol=1e-6)
+        dn = d.double().numpy()
+        th = thr.double().numpy().reshape(-1, 1, 1) if thr.numel() > 1 else thr.double().numpy()
+        sub = np.abs(dn) - th
+        term = np.where(sub > 0, -dn * 1.5 * np.exp(-np.abs(sub) / 0.8) / th, -np.sign(dn)) * gn
+        want = term.sum() if thr.numel() == 1 else term.sum(axis=(0, 2, 3))
+        assert np.allclose(g_thr.numpy().ravel(), np.ravel(want), rtol=1e-5, atol=1e-5)
