@@ -232,6 +232,33 @@ int slayer_delta_bwd(float *grad_in, float *grad_threshold, const float *grad_ou
 int slayer_cumsum(float *out, const float *in, const float *state, int64_t num_states,
                   int reverse, int64_t M, int64_t T, void *stream);
 
+/* ---- fused CUBA neuron -------------------------------------------------------------------------- */
+
+/* No single counterpart in the reference: one launch for what cuba.Neuron.forward does with three
+ * (neuron/cuba.py:356-374 + :401-410 = leaky_integrator.dynamics, leaky_integrator.dynamics with
+ * threshold, Spike.forward).  Bit-identical to slayer_li_fwd -> slayer_li_fwd -> slayer_spike_fwd
+ * (each intermediate is rounded to float32 exactly as at the operator boundaries); it only saves the
+ * re-reading of the intermediates: 16 instead of 24 bytes per neuron-timestep.
+ * thr_scaled = (threshold + eps) * w_scale for the reset (double, <= 0 disables it),
+ * spike_threshold = threshold + eps for the spike compare on the float32 voltage. */
+int slayer_cuba_fwd(float *cur_out, float *vol_out, float *spk_out, const float *in,
+                    const float *i_decay, const float *v_decay,
+                    const float *i_state, const float *v_state,
+                    double thr_scaled, float spike_threshold, int graded, float spike_scale, int w_scale,
+                    int64_t M, int64_t neurons_per_batch, int64_t num_i_decays, int64_t num_v_decays,
+                    int64_t num_i_states, int64_t num_v_states, int64_t T, void *stream);
+
+/* Backward of the above = slayer_spike_bwd -> slayer_li_bwd (voltage) -> slayer_li_bwd (current) in
+ * one launch (16 instead of 36 bytes per neuron-timestep); grad_in is bit-identical to the chain.
+ * grad_i_decay / grad_v_decay may both be NULL; workspace: 2*M + 64*(num_i_decays + num_v_decays)
+ * floats when they are not. */
+int slayer_cuba_bwd(float *grad_in, float *grad_i_decay, float *grad_v_decay,
+                    const float *grad_spikes, const float *voltage, const float *current,
+                    const float *i_decay, const float *v_decay,
+                    float spike_threshold, float tau_rho, float scale_rho, int graded, float *workspace,
+                    int64_t M, int64_t neurons_per_batch, int64_t num_i_decays, int64_t num_v_decays,
+                    int64_t T, void *stream);
+
 /* ---- cross-check implementations (debug mode) ------------------------------------------------ */
 
 /* The reference's debug mode runs its CPU loop next to its kernel and raises on a difference

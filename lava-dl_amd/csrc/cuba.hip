@@ -1,0 +1,174 @@
+// Fused CUBA neuron: current integrator -> voltage integrator with reset -> spike in one pass
+// over the input (reads 4 B, writes 12 B per neuron-timestep instead of 24 B for the three
+// separate operators), and the matching backward pass (spike surrogate -> voltage gradient
+// -> current gradient; reads 12 B, writes 4 B instead of 36 B).  Every intermediate still makes
+// the float32 round trip it makes at the operator boundaries (state -> float32 / w -> trunc(w * .)),
+// so the results are bit-identical to chaining the separate kernels.
+#include "common.h"
+#include "tile.h"
+
+namespace slayer {
+
+int launch_reduce_param_grad(float* grad, const float* partial, float* scratch, int64_t M, int64_t npb,
+                             int64_t num_params, hipStream_t stream);   // li.hip
+int launch_zero_fill(float* p, int64_t n, hipStream_t stream);          // li.hip
+
+template <bool POW2, bool GRADED>
+struct CubaFwd {
+    static constexpr int kIn = 1, kOut = 3;          // out: current, voltage, spikes
+    static constexpr bool kReverse = false;
+    static constexpr int64_t kRows32Below = kAlways, kRows16Below = 32768;
+    struct Params {
+        const float* in[1];
+        float* out[3];
+        const float *i_decay, *v_decay, *i_state, *v_state;
+        float w, inv_w, thr, spike_thr, spike_scale;
+        int64_t npb, n_id, n_vd, n_is, n_vs;
+    };
+    int yc, yv, mi, mv;
+    float w, inv_w, thr, spike_thr, spike_scale;
+
+    __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
+        w = p.w; inv_w = p.inv_w; thr = p.thr; spike_thr = p.spike_thr; spike_scale = p.spike_scale;
+        yc = yv = mi = mv = 0;
+        if (valid) {
+            yc = trunc_i32(p.i_state[p.n_is == 1 ? 0 : m] * w);
+            yv = trunc_i32(p.v_state[p.n_vs == 1 ? 0 : m] * w);
+            mi = 4096 - trunc_i32(p.i_decay[param_index(m, p.npb, p.n_id)]);
+            mv = 4096 - trunc_i32(p.v_decay[param_index(m, p.npb, p.n_vd)]);
+        }
+    }
+    __device__ __forceinline__ void step(const float (&x)[1], float (&o)[3]) {
+        yc = rs0_12(yc, mi) + trunc_i32(w * x[0]);
+        const float cf = (float)yc;
+        const float cur = POW2 ? cf * inv_w : cf / w;
+        const int yn = rs0_12(yv, mv) + trunc_i32(w * cur);     // the voltage op reads the float32 current
+        const float vf = (float)yn;
+        const float vol = POW2 ? vf * inv_w : vf / w;
+        yv = (vf >= thr) ? 0 : yn;
+        const float h = (vol >= spike_thr) ? 1.0f : 0.0f;
+        o[0] = cur;
+        o[1] = vol;
+        o[2] = GRADED ? (h * vol) / spike_scale : h;
+    }
+    __device__ __forceinline__ void finish(const Params&, int64_t, bool) {}
+};
+
+template <bool GRADED>
+struct CubaBwd {
+    static constexpr int kIn = 3, kOut = 1;          // in: grad of spikes, saved voltage, saved current
+    static constexpr bool kReverse = true;
+    static constexpr int64_t kRows32Below = kAlways, kRows16Below = kAlways;
+    struct Params {
+        const float* in[3];
+        float* out[1];
+        const float *i_decay, *v_decay;
+        float *partial_i, *partial_v;                // per-neuron decay gradients, or nullptr
+        float spike_thr, tau, rho;
+        int64_t npb, n_id, n_vd;
+    };
+    float ai, av, gc, gx, acc_i, acc_v, spike_thr, tau, rho, lead;
+
+    __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
+        spike_thr = p.spike_thr; tau = p.tau; rho = p.rho;
+        lead = (rho / 2.0f) / tau;
+        ai = av = gc = gx = acc_i = acc_v = 0.f;
+        if (valid) {
+            ai = 1.0f - p.i_decay[param_index(m, p.npb, p.n_id)] / 4096.0f;
+            av = 1.0f - p.v_decay[param_index(m, p.npb, p.n_vd)] / 4096.0f;
+        }
+    }
+    __device__ __forceinline__ void step(const float (&x)[3], float (&o)[1]) {
+        const float d = x[1] - spike_thr;
+        const float gv = GRADED ? (rho * expf(fminf(d, 0.0f) / tau)) * x[0] : (lead * expf(-fabsf(d) / tau)) * x[0];
+        acc_v = __fmaf_rn(gc, x[1], acc_v);          // gc, gx still hold the gradients of step t+1
+        acc_i = __fmaf_rn(gx, x[2], acc_i);
+        gc = av * gc + gv;
+        gx = ai * gx + gc;
+        o[0] = gx;
+    }
+    __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
+        if (valid && p.partial_i) { p.partial_i[m] = acc_i; p.partial_v[m] = acc_v; }
+    }
+};
+
+}  // namespace slayer
+
+using namespace slayer;
+
+template <bool POW2, bool GRADED>
+static int cuba_fwd_launch(const typename CubaFwd<POW2, GRADED>::Params& p, int64_t M, int64_t T, hipStream_t st) {
+    return launch_stream<CubaFwd<POW2, GRADED>>(p, M, T, st);
+}
+
+extern "C" int slayer_cuba_fwd(float* cur_out, float* vol_out, float* spk_out, const float* in,
+                               const float* i_decay, const float* v_decay,
+                               const float* i_state, const float* v_state,
+                               double thr_scaled, float spike_threshold, int graded, float spike_scale, int w_scale,
+                               int64_t M, int64_t neurons_per_batch, int64_t num_i_decays, int64_t num_v_decays,
+                               int64_t num_i_states, int64_t num_v_states, int64_t T, void* stream) {
+    if (int e = check_rows(M, T)) return e;
+    if (M == 0 || T == 0) return 0;
+    if (!cur_out || !vol_out || !spk_out || !in || !i_decay || !v_decay || !i_state || !v_state) return SLAYER_ENULL;
+    if (int e = check_params(M, neurons_per_batch, num_i_decays)) return e;
+    if (int e = check_params(M, neurons_per_batch, num_v_decays)) return e;
+    if (int e = check_states(M, num_i_states)) return e;
+    if (int e = check_states(M, num_v_states)) return e;
+    if (w_scale == 0) return SLAYER_EINVAL;
+    const float w = (float)w_scale;
+    const float thr = thr_scaled > 0 ? (float)thr_scaled : __builtin_inff();
+    hipStream_t st = (hipStream_t)stream;
+#define SLAYER_CUBA(P, G)                                                                                        \
+    do {                                                                                                         \
+        CubaFwd<P, G>::Params p{{in}, {cur_out, vol_out, spk_out}, i_decay, v_decay, i_state, v_state, w,           \
+                                1.0f / w, thr, spike_threshold, spike_scale, neurons_per_batch, num_i_decays,      \
+                                num_v_decays, num_i_states, num_v_states};                                         \
+        return cuba_fwd_launch<P, G>(p, M, T, st);                                                                 \
+    } while (0)
+    if (is_pow2(w_scale)) { if (graded) SLAYER_CUBA(true, true); else SLAYER_CUBA(true, false); }
+    if (graded) SLAYER_CUBA(false, true);
+    SLAYER_CUBA(false, false);
+#undef SLAYER_CUBA
+}
+
+extern "C" int slayer_cuba_bwd(float* grad_in, float* grad_i_decay, float* grad_v_decay,
+                               const float* grad_spikes, const float* voltage, const float* current,
+                               const float* i_decay, const float* v_decay,
+                               float spike_threshold, float tau_rho, float scale_rho, int graded, float* workspace,
+                               int64_t M, int64_t neurons_per_batch, int64_t num_i_decays, int64_t num_v_decays,
+                               int64_t T, void* stream) {
+    if (int e = check_rows(M, T)) return e;
+    const int64_t mm = M > 0 ? M : neurons_per_batch;
+    if (int e = check_params(mm, neurons_per_batch, num_i_decays)) return e;
+    if (int e = check_params(mm, neurons_per_batch, num_v_decays)) return e;
+    if ((grad_i_decay == nullptr) != (grad_v_decay == nullptr)) return SLAYER_ENULL;
+    const bool want = grad_i_decay != nullptr;
+    if (want && !workspace && M > 0) return SLAYER_ENULL;
+    hipStream_t st = (hipStream_t)stream;
+    if (M > 0 && T > 0) {
+        if (!grad_in || !grad_spikes || !voltage || !current || !i_decay || !v_decay) return SLAYER_ENULL;
+        if (graded) {
+            CubaBwd<true>::Params p{{grad_spikes, voltage, current}, {grad_in}, i_decay, v_decay,
+                                    want ? workspace : nullptr, want ? workspace + M : nullptr,
+                                    spike_threshold, tau_rho, scale_rho, neurons_per_batch, num_i_decays, num_v_decays};
+            if (int e = launch_stream<CubaBwd<true>>(p, M, T, st)) return e;
+        } else {
+            CubaBwd<false>::Params p{{grad_spikes, voltage, current}, {grad_in}, i_decay, v_decay,
+                                     want ? workspace : nullptr, want ? workspace + M : nullptr,
+                                     spike_threshold, tau_rho, scale_rho, neurons_per_batch, num_i_decays, num_v_decays};
+            if (int e = launch_stream<CubaBwd<false>>(p, M, T, st)) return e;
+        }
+    }
+    if (want) {
+        if (M == 0 || T == 0) {
+            if (int e = launch_zero_fill(grad_i_decay, num_i_decays, st)) return e;
+            return launch_zero_fill(grad_v_decay, num_v_decays, st);
+        }
+        float* scratch = workspace + 2 * M;
+        if (int e = launch_reduce_param_grad(grad_i_decay, workspace, scratch, M, neurons_per_batch, num_i_decays, st))
+            return e;
+        return launch_reduce_param_grad(grad_v_decay, workspace + M, scratch + 64 * num_i_decays, M,
+                                        neurons_per_batch, num_v_decays, st);
+    }
+    return 0;
+}

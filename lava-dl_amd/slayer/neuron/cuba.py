@@ -3,7 +3,7 @@
 import torch
 
 from .base import Neuron as _Base
-from .dynamics import leaky_integrator
+from .dynamics import leaky_integrator, cuba_fused
 from ..spike import Spike
 
 TAU_RHO_MULT = 100      # surrogate-gradient constants of the CUBA family (neuron/cuba.py:20-21)
@@ -53,5 +53,22 @@ class Neuron(_Base):
         return spike
 
     def forward(self, input):
-        _, voltage = self.dynamics(input)
-        return self.spike(voltage)
+        """Spike response.  Without a normalisation between current and voltage the three steps run
+        as one fused kernel per direction (same bits as ``spike(dynamics(input)[1])``)."""
+        if self.norm is not None:
+            _, voltage = self.dynamics(input)
+            return self.spike(voltage)
+        self._prepare(input)
+        current, voltage, spike = cuba_fused.dynamics(
+            input, self._q('current_decay'), self._q('voltage_decay'),
+            self.current_state.contiguous(), self.voltage_state.contiguous(), self.s_scale,
+            self.threshold + self.threshold_eps, self.tau_rho * TAU_RHO_MULT, self.scale_rho * SCALE_RHO_MULT,
+            self.graded_spike, 1)
+        if self.persistent_state:
+            with torch.no_grad():
+                self.current_state = current[..., -1].clone()
+                self.voltage_state = leaky_integrator.persistent_state(
+                    voltage[..., -1], spike[..., -1]).detach().clone()
+        if self.drop is not None:
+            spike = self.drop(spike)
+        return spike

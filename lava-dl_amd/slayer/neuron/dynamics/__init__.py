@@ -1,3 +1,4 @@
-from . import leaky_integrator, adaptive_threshold, resonator, adaptive_phase_th, adaptive_resonator
+from . import leaky_integrator, adaptive_threshold, resonator, adaptive_phase_th, adaptive_resonator, cuba_fused
 
-__all__ = ['leaky_integrator', 'adaptive_threshold', 'resonator', 'adaptive_phase_th', 'adaptive_resonator']
+__all__ = ['leaky_integrator', 'adaptive_threshold', 'resonator', 'adaptive_phase_th', 'adaptive_resonator',
+           'cuba_fused']

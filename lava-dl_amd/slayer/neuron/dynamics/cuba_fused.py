@@ -1,0 +1,85 @@
+"""Fused CUBA neuron dynamics + spike on the GPU.
+
+No counterpart module in the reference: it does in one kernel launch per direction what
+``cuba.Neuron.forward`` (neuron/cuba.py:423-440 in the reference) does with
+``leaky_integrator.dynamics`` twice and ``Spike.apply``, with bit-identical results, reading the
+input once and never re-reading the intermediate current and voltage traces.
+"""
+import torch
+
+from ... import _native as N
+
+
+def dynamics(input, current_decay, voltage_decay, current_state, voltage_state, w_scale, threshold,
+             tau_rho, scale_rho, graded_spike=False, spike_scale=1):
+    """(current, voltage, spike) of a CUBA neuron.
+
+    ``threshold`` is used both for the voltage reset (compared in integer state units, as
+    ``leaky_integrator.dynamics`` does) and for the spike (compared on the float32 voltage, as
+    ``Spike`` does).  Gradients flow from ``spike`` to ``input`` and to both decays; the returned
+    current and voltage traces are detached.
+    """
+    return _CubaFused.apply(input, current_decay, voltage_decay, current_state, voltage_state,
+                            w_scale, threshold, tau_rho, scale_rho, graded_spike, spike_scale)
+
+
+def _fwd(input, i_decay, v_decay, i_state, v_state, w_scale, threshold, graded, spike_scale):
+    dev = N.require_gpu(input, i_decay, v_decay, i_state, v_state)
+    input, i_decay, v_decay = input.contiguous(), i_decay.contiguous(), v_decay.contiguous()
+    i_state, v_state = i_state.contiguous(), v_state.contiguous()
+    M, T = N.rows_and_steps(input)
+    for name, s in (('current_state', i_state), ('voltage_state', v_state)):
+        if s.numel() not in (1, M):
+            raise RuntimeError(f'{name} has {s.numel()} elements, expected 1 or {M}')
+    cur, vol, spk = (torch.empty_like(input) for _ in range(3))
+    with torch.cuda.device(dev):
+        N.check(N.lib().slayer_cuba_fwd(
+            N.ptr(cur), N.ptr(vol), N.ptr(spk), N.ptr(input), N.ptr(i_decay), N.ptr(v_decay),
+            N.ptr(i_state), N.ptr(v_state), float(threshold * w_scale), float(threshold),
+            1 if graded else 0, float(spike_scale), int(w_scale),
+            M, N.neurons_per_batch(input), i_decay.numel(), v_decay.numel(),
+            i_state.numel(), v_state.numel(), T, N.stream_handle()))
+    return cur, vol, spk
+
+
+def _bwd(grad_spikes, vol, cur, i_decay, v_decay, threshold, tau_rho, scale_rho, graded, need_decay_grad=True):
+    dev = N.require_gpu(grad_spikes, vol, cur, i_decay, v_decay)
+    grad_spikes, i_decay, v_decay = grad_spikes.contiguous(), i_decay.contiguous(), v_decay.contiguous()
+    M, T = N.rows_and_steps(grad_spikes)
+    grad_input = torch.empty_like(grad_spikes)
+    g_i = g_v = workspace = None
+    if need_decay_grad:
+        g_i = torch.empty(i_decay.numel(), dtype=torch.float32, device=dev)
+        g_v = torch.empty(v_decay.numel(), dtype=torch.float32, device=dev)
+        workspace = torch.empty(2 * M + 64 * (i_decay.numel() + v_decay.numel()), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        N.check(N.lib().slayer_cuba_bwd(
+            N.ptr(grad_input), N.ptr(g_i), N.ptr(g_v), N.ptr(grad_spikes), N.ptr(vol), N.ptr(cur),
+            N.ptr(i_decay), N.ptr(v_decay), float(threshold), float(tau_rho), float(scale_rho),
+            1 if graded else 0, N.ptr(workspace),
+            M, N.neurons_per_batch(grad_spikes), i_decay.numel(), v_decay.numel(), T, N.stream_handle()))
+    return grad_input, g_i, g_v
+
+
+class _CubaFused(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input, i_decay, v_decay, i_state, v_state, w_scale, threshold, tau_rho, scale_rho,
+                graded, spike_scale):
+        graded = graded is True
+        cur, vol, spk = _fwd(input, i_decay.detach(), v_decay.detach(), i_state.detach(), v_state.detach(),
+                             w_scale, threshold, graded, spike_scale)
+        ctx.save_for_backward(cur, vol, i_decay, v_decay)
+        ctx.cfg = (float(threshold), float(tau_rho), float(scale_rho), graded)
+        ctx.mark_non_differentiable(cur, vol)
+        return cur, vol, spk
+
+    @staticmethod
+    def backward(ctx, _g_cur, _g_vol, grad_spikes):
+        cur, vol, i_decay, v_decay = ctx.saved_tensors
+        threshold, tau_rho, scale_rho, graded = ctx.cfg
+        need = ctx.needs_input_grad[1] or ctx.needs_input_grad[2]
+        g_in, g_i, g_v = _bwd(grad_spikes, vol, cur, i_decay.detach(), v_decay.detach(),
+                              threshold, tau_rho, scale_rho, graded, need)
+        if g_i is not None:
+            g_i, g_v = g_i.reshape(i_decay.shape), g_v.reshape(v_decay.shape)
+        return (g_in, g_i, g_v) + (None,) * 8

@@ -156,3 +156,63 @@ def test_neuron_shape_checks(slayer):
         slayer.neuron.cuba.Neuron(1.0, [0.1, 0.2], 0.03)
     with pytest.raises(AssertionError):
         slayer.neuron.rf.Neuron(1.0, 3, 0.05)
+
+
+@pytest.mark.parametrize('shape,w,graded', [((4, 16, 8, 8, 300), 64, False), ((3, 70, 129), 100, False),
+                                            ((2, 3, 5, 7, 37), 4096, True), ((4, 9000, 64), 64, False),
+                                            ((4, 70000, 40), 64, False)])
+def test_fused_cuba_equals_the_operator_chain(slayer, shape, w, graded):
+    """The fused kernels must reproduce leaky_integrator -> leaky_integrator(threshold) -> Spike bit for bit,
+    forward (all three traces) and backward (grad_input), and the decay gradients to float tolerance."""
+    from tests.util import seed_of
+    gen = torch.Generator().manual_seed(seed_of(shape, w, graded, 'fused'))
+    C = shape[1]
+    x = sparse_input(gen, shape, p=0.1, amp=1.5).to(dev())
+    g = torch.randn(shape, generator=gen).to(dev())
+    d_i = torch.randint(0, 4097, (C,), generator=gen).float().to(dev())
+    d_v = torch.randint(0, 4097, (C,), generator=gen).float().to(dev())
+    s_i = torch.randn(shape[:-1], generator=gen).to(dev())
+    s_v = torch.randn(shape[:-1], generator=gen).to(dev()) * 0.3
+    thr, tau, rho = 1.0 + 0.01 / w, 1.3, 0.7
+    D = slayer.neuron.dynamics
+    # chain
+    x1, di1, dv1 = x.clone().requires_grad_(), d_i.clone().requires_grad_(), d_v.clone().requires_grad_()
+    cur = D.leaky_integrator.dynamics(x1, di1, s_i, w)
+    vol = D.leaky_integrator.dynamics(cur, dv1, s_v, w, thr)
+    spk = slayer.spike.Spike.apply(vol, thr, tau, rho, graded, 0, 2)
+    spk.backward(g)
+    # fused
+    x2, di2, dv2 = x.clone().requires_grad_(), d_i.clone().requires_grad_(), d_v.clone().requires_grad_()
+    f_cur, f_vol, f_spk = D.cuba_fused.dynamics(x2, di2, dv2, s_i, s_v, w, thr, tau, rho, graded, 2)
+    f_spk.backward(g)
+    assert float(spk.detach().abs().sum()) > 0
+    assert torch.equal(f_cur, cur.detach()), 'fused current differs'
+    assert torch.equal(f_vol, vol.detach()), 'fused voltage differs'
+    assert torch.equal(f_spk.detach(), spk.detach()), 'fused spikes differ'
+    assert torch.equal(x2.grad, x1.grad), 'fused grad_input differs'
+    assert_rel(di2.grad.cpu(), di1.grad.cpu(), 'fused grad current_decay', rel=1e-4)
+    assert_rel(dv2.grad.cpu(), dv1.grad.cpu(), 'fused grad voltage_decay', rel=1e-4)
+
+
+def test_cuba_neuron_forward_uses_fused_path_with_same_results(slayer):
+    gen = torch.Generator().manual_seed(104)
+    x = sparse_input(gen, (3, 6, 5, 90), p=0.2).to(dev())
+    torch.manual_seed(3)
+    a = slayer.neuron.cuba.Neuron(1.0, [0.2, 0.4], [0.02, 0.2], shared_param=False, requires_grad=True,
+                                  persistent_state=True).to(dev())
+    b = slayer.neuron.cuba.Neuron(1.0, [0.2, 0.4], [0.02, 0.2], shared_param=False, requires_grad=True,
+                                  persistent_state=True).to(dev())
+    b._prepare(x)
+    a._prepare(x)
+    for pa, pb in zip(a.parameters(), b.parameters()):
+        pb.data = pa.data.clone()
+    for k in range(2):                                    # two calls: the carried state must agree too
+        xa, xb = x.clone().requires_grad_(), x.clone().requires_grad_()
+        sa = a(xa)                                        # fused
+        _, vol = b.dynamics(xb)
+        sb = b.spike(vol)                                 # three operators
+        assert torch.equal(sa.detach(), sb.detach()), f'call {k}: spikes differ'
+        assert torch.equal(a.voltage_state, b.voltage_state) and torch.equal(a.current_state, b.current_state)
+        sa.sum().backward()
+        sb.sum().backward()
+        assert torch.equal(xa.grad, xb.grad)
