@@ -1,6 +1,6 @@
 """Benchmark of the SLAYER neuron-dynamics hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cuba|cuba_fwd_small|alif|rf|synapse]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cuba|cuba_fused|cuba_fwd_small|alif|rf|synapse]
 
 A step is one pass of the workload's op sequence over one batch of synthetic input that is already
 resident in HBM (outputs come from torch's caching allocator inside the timed region).  The default
@@ -147,6 +147,25 @@ class Cuba(Workload):
         g_vol = O.spike_bwd(g, vol, self.thr, 1.0, 1.0)
         g_cur, _ = O.li_bwd(g_vol, vol, c['d_v'])
         O.li_bwd(g_cur, cur, c['d_i'])
+
+
+class CubaFused(Cuba):
+    """Same tensor and parameters as `cuba`, run through the fused kernels: the intermediates are written
+    (autograd needs them) but never re-read by a separate operator.  Reported against its own byte count."""
+    name = 'CUBA conv-layer neuron tensor fwd+bwd, fused kernels'
+    ops = [('cuba_fwd', 'stream_kernel<CubaFwd>', 16), ('cuba_bwd', 'stream_kernel<CubaBwd>', 16)]
+
+    def __init__(self, dev):
+        super().__init__(dev)
+        from lava_dl_amd.slayer.neuron.dynamics import cuba_fused
+        self.F = cuba_fused
+
+    def step(self, t):
+        with t('cuba_fwd'):
+            cur, vol, spk = self.F._fwd(self.x, self.d_i, self.d_v, self.zero, self.zero, self.w, self.thr, False, 1)
+        with t('cuba_bwd'):
+            g_x, gd_i, gd_v = self.F._bwd(self.g, vol, cur, self.d_i, self.d_v, self.thr, 1.0, 1.0, False)
+        return spk, g_x, gd_v, gd_i
 
 
 class CubaFwdSmall(Workload):
@@ -320,7 +339,7 @@ class Synapse(Workload):
         O.conv_bwd(O.shift(g_z, -c['delay'], 1), c['filt'], 1)
 
 
-WORKLOADS = {'cuba': Cuba, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'rf': Rf, 'synapse': Synapse}
+WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'rf': Rf, 'synapse': Synapse}
 
 
 def cpu_baseline(job, budget_s=20.0):
