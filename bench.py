@@ -282,6 +282,24 @@ class Rf(Workload):
         O.res_bwd(g_re, g_im, re, im, c['sin'], c['cos'])
 
 
+class RfFused(Rf):
+    name = 'Resonator (RF) dynamics fwd+bwd, fused kernels'
+    ops = [('rf_fwd', 'stream_kernel<RfFwd>', 20), ('rf_bwd', 'stream_kernel<RfBwd>', 20)]
+
+    def __init__(self, dev):
+        super().__init__(dev)
+        from lava_dl_amd.slayer.neuron.dynamics import rf_fused
+        self.F = rf_fused
+
+    def step(self, t):
+        with t('rf_fwd'):
+            re, im, spk = self.F._fwd(self.xr, self.xi, self.sin, self.cos, self.zero, self.zero, self.zero, 64,
+                                      1.0, False, 1)
+        with t('rf_bwd'):
+            out = self.F._bwd(self.g, re, im, self.sin, self.cos, 1.0, 0.5, 10.0, False)
+        return spk, out
+
+
 class Synapse(Workload):
     name = 'SLAYER synapse stack (conv K=64 -> per-channel shift -> CUBA) fwd+bwd'
     shape = (32, 256, 1500)
@@ -339,7 +357,7 @@ class Synapse(Workload):
         O.conv_bwd(O.shift(g_z, -c['delay'], 1), c['filt'], 1)
 
 
-WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'rf': Rf, 'synapse': Synapse}
+WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'rf': Rf, 'rf_fused': RfFused, 'synapse': Synapse}
 
 
 def cpu_baseline(job, budget_s=20.0):

@@ -259,6 +259,29 @@ int slayer_cuba_bwd(float *grad_in, float *grad_i_decay, float *grad_v_decay,
                     int64_t M, int64_t neurons_per_batch, int64_t num_i_decays, int64_t num_v_decays,
                     int64_t T, void *stream);
 
+/* ---- fused resonate-and-fire neuron ------------------------------------------------------------- */
+
+/* One launch for what rf.Neuron.forward does with two operators (neuron/rf.py:429-436 + :463-471 =
+ * resonator.dynamics without threshold, complex.Spike.forward); bit-identical to slayer_res_fwd ->
+ * slayer_cspike_fwd, 20 instead of 28 bytes per neuron-timestep.  imag_last is the imaginary sample
+ * before step 0 (num_last == 1 broadcasts). */
+int slayer_rf_fwd(float *re_out, float *im_out, float *spk_out, const float *re_in, const float *im_in,
+                  const float *sin_decay, const float *cos_decay,
+                  const float *re_state, const float *im_state, const float *imag_last,
+                  float spike_threshold, int graded, float spike_scale, int w_scale,
+                  int64_t M, int64_t neurons_per_batch, int64_t num_decays,
+                  int64_t num_re_states, int64_t num_im_states, int64_t num_last,
+                  int64_t T, void *stream);
+
+/* Backward of the above = slayer_cspike_bwd -> slayer_res_bwd in one launch (20 instead of 44 bytes
+ * per neuron-timestep); the input gradients are bit-identical to the chain.  grad_sin / grad_cos may
+ * both be NULL; workspace: 2*M + 128*num_decays floats when they are not. */
+int slayer_rf_bwd(float *g_re_in, float *g_im_in, float *grad_sin, float *grad_cos,
+                  const float *grad_spikes, const float *re, const float *im,
+                  const float *sin_decay, const float *cos_decay,
+                  float spike_threshold, float tau_rho, float scale_rho, int graded, float *workspace,
+                  int64_t M, int64_t neurons_per_batch, int64_t num_decays, int64_t T, void *stream);
+
 /* ---- cross-check implementations (debug mode) ------------------------------------------------ */
 
 /* The reference's debug mode runs its CPU loop next to its kernel and raises on a difference

@@ -1,0 +1,183 @@
+// Fused resonate-and-fire neuron: resonator recurrence (no reset) + phase-threshold spike in one
+// pass (reads 8 B, writes 12 B per neuron-timestep instead of 28 B for the two operators), and the
+// matching backward pass (complex-spike surrogate -> reverse-time rotation; reads 12 B, writes 8 B
+// instead of 44 B).  Intermediates are rounded exactly as at the operator boundaries, so results
+// are bit-identical to chaining resonator.dynamics and complex.Spike.
+#include "common.h"
+#include "tile.h"
+
+namespace slayer {
+
+int launch_reduce_param_grad(float* grad, const float* partial, float* scratch, int64_t M, int64_t npb,
+                             int64_t num_params, hipStream_t stream);   // li.hip
+int launch_zero_fill(float* p, int64_t n, hipStream_t stream);          // li.hip
+
+template <bool POW2, bool GRADED>
+struct RfFwd {
+    static constexpr int kIn = 2, kOut = 3;          // out: real, imag, spikes
+    static constexpr bool kReverse = false;
+    static constexpr int64_t kRows32Below = 65536, kRows16Below = 16384;
+    struct Params {
+        const float* in[2];
+        float* out[3];
+        const float *sin_decay, *cos_decay, *re_state, *im_state, *imag_last;
+        float w, inv_w, spike_thr, spike_scale;
+        int64_t npb, nd, n_rs, n_is, n_last;
+    };
+    int re, im, s, c;
+    float w, inv_w, spike_thr, spike_scale, im_prev;
+
+    __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
+        w = p.w; inv_w = p.inv_w; spike_thr = p.spike_thr; spike_scale = p.spike_scale;
+        re = im = s = c = 0; im_prev = 0.f;
+        if (valid) {
+            re = trunc_i32(p.re_state[p.n_rs == 1 ? 0 : m] * w);
+            im = trunc_i32(p.im_state[p.n_is == 1 ? 0 : m] * w);
+            const int64_t j = param_index(m, p.npb, p.nd);
+            s = trunc_i32(p.sin_decay[j]);
+            c = trunc_i32(p.cos_decay[j]);
+            im_prev = p.imag_last[p.n_last == 1 ? 0 : m];
+        }
+    }
+    __device__ __forceinline__ void step(const float (&x)[2], float (&o)[3]) {
+        const int re_n = rs0_12(c, re) - rs0_12(s, im) + trunc_i32(w * x[0]);
+        const int im_n = rs0_12(s, re) + rs0_12(c, im) + trunc_i32(w * x[1]);
+        re = re_n; im = im_n;
+        const float ref = (float)re_n, imf = (float)im_n;
+        const float r = POW2 ? ref * inv_w : ref / w;
+        const float i = POW2 ? imf * inv_w : imf / w;
+        const float a = (r >= spike_thr) ? 1.0f : 0.0f, b = (im_prev < 0.0f) ? 1.0f : 0.0f, cc = (i >= 0.0f) ? 1.0f : 0.0f;
+        o[0] = r;
+        o[1] = i;
+        o[2] = GRADED ? (((r * a) * b) * cc) / spike_scale : (a * b) * cc;
+        im_prev = i;
+    }
+    __device__ __forceinline__ void finish(const Params&, int64_t, bool) {}
+};
+
+template <bool GRADED>
+struct RfBwd {
+    static constexpr int kIn = 3, kOut = 2;          // in: grad of spikes, saved real, saved imag
+    static constexpr bool kReverse = true;
+    static constexpr int64_t kRows32Below = 65536, kRows16Below = 16384;
+    struct Params {
+        const float* in[3];
+        float* out[2];
+        const float *sin_decay, *cos_decay;
+        float *partial_sin, *partial_cos;
+        float spike_thr, tau, rho;
+        int64_t npb, nd;
+    };
+    float c, s, gr, gi, acc_s, acc_c, thr, tau, rho, half_over_tau, two_tau, neg_rho_over_tau;
+
+    __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
+        thr = p.spike_thr; tau = p.tau; rho = p.rho;
+        half_over_tau = (1.0f / 2.0f) / tau;
+        two_tau = 2.0f * tau;
+        neg_rho_over_tau = (-rho) / tau;
+        c = s = gr = gi = acc_s = acc_c = 0.f;
+        if (valid) {
+            const int64_t j = param_index(m, p.npb, p.nd);
+            c = p.cos_decay[j] / 4096.0f;
+            s = p.sin_decay[j] / 4096.0f;
+        }
+    }
+    __device__ __forceinline__ void step(const float (&x)[3], float (&o)[2]) {
+        const float g = x[0], r = x[1], i = x[2];
+        // complex spike surrogate (same expression order as the stand-alone kernel)
+        float d_re;
+        if (GRADED) d_re = expf(-fmaxf(thr - r, 0.0f) / tau);
+        else d_re = half_over_tau * expf(-fabsf(r - thr) / tau);
+        const float d_im = half_over_tau * expf(-fabsf(i) / tau);
+        const float dr = r - thr;
+        const float sg_r = dr > 0.0f ? 1.0f : (dr < 0.0f ? -1.0f : (dr == 0.0f ? 0.0f : dr));
+        const float sg_i = i > 0.0f ? 1.0f : (i < 0.0f ? -1.0f : (i == 0.0f ? 0.0f : i));
+        const float step_re = 0.5f * (1.0f + sg_r * (1.0f - two_tau * d_re));
+        const float g_re = g * ((rho * d_re) * d_im);
+        const float g_im = g * (((neg_rho_over_tau * sg_i) * d_im) * step_re);
+        // reverse-time rotation; gr, gi still hold the gradients of step t+1
+        acc_s = __fmaf_rn(gi, r, __fmaf_rn(-gr, i, acc_s));
+        acc_c = __fmaf_rn(gi, i, __fmaf_rn(gr, r, acc_c));
+        const float ngr = (c * gr + s * gi) + g_re;
+        const float ngi = ((-s) * gr + c * gi) + g_im;
+        gr = ngr; gi = ngi;
+        o[0] = ngr; o[1] = ngi;
+    }
+    __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
+        if (valid && p.partial_sin) { p.partial_sin[m] = acc_s; p.partial_cos[m] = acc_c; }
+    }
+};
+
+}  // namespace slayer
+
+using namespace slayer;
+
+extern "C" int slayer_rf_fwd(float* re_out, float* im_out, float* spk_out, const float* re_in, const float* im_in,
+                             const float* sin_decay, const float* cos_decay,
+                             const float* re_state, const float* im_state, const float* imag_last,
+                             float spike_threshold, int graded, float spike_scale, int w_scale,
+                             int64_t M, int64_t neurons_per_batch, int64_t num_decays,
+                             int64_t num_re_states, int64_t num_im_states, int64_t num_last,
+                             int64_t T, void* stream) {
+    if (int e = check_rows(M, T)) return e;
+    if (M == 0 || T == 0) return 0;
+    if (!re_out || !im_out || !spk_out || !re_in || !im_in || !sin_decay || !cos_decay || !re_state || !im_state ||
+        !imag_last)
+        return SLAYER_ENULL;
+    if (int e = check_params(M, neurons_per_batch, num_decays)) return e;
+    for (int64_t n : {num_re_states, num_im_states, num_last})
+        if (int e = check_states(M, n)) return e;
+    if (w_scale == 0) return SLAYER_EINVAL;
+    const float w = (float)w_scale;
+    hipStream_t st = (hipStream_t)stream;
+#define SLAYER_RF(P, G)                                                                                          \
+    do {                                                                                                         \
+        RfFwd<P, G>::Params p{{re_in, im_in}, {re_out, im_out, spk_out}, sin_decay, cos_decay, re_state, im_state, \
+                              imag_last, w, 1.0f / w, spike_threshold, spike_scale, neurons_per_batch, num_decays, \
+                              num_re_states, num_im_states, num_last};                                             \
+        return launch_stream<RfFwd<P, G>>(p, M, T, st);                                                            \
+    } while (0)
+    if (is_pow2(w_scale)) { if (graded) SLAYER_RF(true, true); else SLAYER_RF(true, false); }
+    if (graded) SLAYER_RF(false, true);
+    SLAYER_RF(false, false);
+#undef SLAYER_RF
+}
+
+extern "C" int slayer_rf_bwd(float* g_re_in, float* g_im_in, float* grad_sin, float* grad_cos,
+                             const float* grad_spikes, const float* re, const float* im,
+                             const float* sin_decay, const float* cos_decay,
+                             float spike_threshold, float tau_rho, float scale_rho, int graded, float* workspace,
+                             int64_t M, int64_t neurons_per_batch, int64_t num_decays, int64_t T, void* stream) {
+    if (int e = check_rows(M, T)) return e;
+    if (int e = check_params(M > 0 ? M : neurons_per_batch, neurons_per_batch, num_decays)) return e;
+    if ((grad_sin == nullptr) != (grad_cos == nullptr)) return SLAYER_ENULL;
+    const bool want = grad_sin != nullptr;
+    if (want && !workspace && M > 0) return SLAYER_ENULL;
+    hipStream_t st = (hipStream_t)stream;
+    if (M > 0 && T > 0) {
+        if (!g_re_in || !g_im_in || !grad_spikes || !re || !im || !sin_decay || !cos_decay) return SLAYER_ENULL;
+        if (graded) {
+            RfBwd<true>::Params p{{grad_spikes, re, im}, {g_re_in, g_im_in}, sin_decay, cos_decay,
+                                  want ? workspace : nullptr, want ? workspace + M : nullptr,
+                                  spike_threshold, tau_rho, scale_rho, neurons_per_batch, num_decays};
+            if (int e = launch_stream<RfBwd<true>>(p, M, T, st)) return e;
+        } else {
+            RfBwd<false>::Params p{{grad_spikes, re, im}, {g_re_in, g_im_in}, sin_decay, cos_decay,
+                                   want ? workspace : nullptr, want ? workspace + M : nullptr,
+                                   spike_threshold, tau_rho, scale_rho, neurons_per_batch, num_decays};
+            if (int e = launch_stream<RfBwd<false>>(p, M, T, st)) return e;
+        }
+    }
+    if (want) {
+        if (M == 0 || T == 0) {
+            if (int e = launch_zero_fill(grad_sin, num_decays, st)) return e;
+            return launch_zero_fill(grad_cos, num_decays, st);
+        }
+        float* scratch = workspace + 2 * M;
+        if (int e = launch_reduce_param_grad(grad_sin, workspace, scratch, M, neurons_per_batch, num_decays, st))
+            return e;
+        return launch_reduce_param_grad(grad_cos, workspace + M, scratch + 64 * num_decays, M, neurons_per_batch,
+                                        num_decays, st);
+    }
+    return 0;
+}

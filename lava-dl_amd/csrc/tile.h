@@ -117,11 +117,12 @@ __device__ __forceinline__ void buf_store4(__amdgpu_buffer_rsrc_t r, int byte_of
 // start on 128-byte boundaries.  Lanes skip the columns that fall before step 0 or after T-1.
 //
 // Boundary lines.  Unless T is a multiple of 32, the last line of row r is also the first line of
-// row r+1.  Writing it in two pieces at two different times costs a read-modify-write in memory
-// for each piece (measured: ~16% of the kernel at T = 300), so output quads that fall in such a
-// shared line are collected in an LDS buffer of R+1 lines (one per row boundary of the wave) and
-// written once, whole, after the last chunk.  Only the two lines shared with neighbouring
-// workgroups are still written in pieces.
+// row r+1, and the two pieces are produced a whole row apart in time.  Written when produced, each
+// piece reaches memory as a partial line, which costs a read-modify-write there (measured: ~16% of
+// the kernel at T = 300).  So the piece that comes first (the head of row r+1 in a forward pass,
+// the tail of row r in a reverse pass) waits in registers, and the eight lanes that copy the first
+// line of row r+1 store the whole line with one instruction once the other piece exists.  Only
+// the lines shared with neighbouring workgroups are still written in pieces.
 //
 // Interior chunks (every column of every row inside [0, T), no shared line) run a branch-free
 // recurrence loop; only the first and the last one or two chunks take the predicated path.
@@ -131,7 +132,6 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
     constexpr int TC = G::kChunk;
     constexpr int NI = Op::kIn, NO = Op::kOut, NT = NI > NO ? NI : NO;
     __shared__ __attribute__((aligned(16))) float tile[NT][G::kTileFloats];
-    __shared__ __attribute__((aligned(16))) float bline[NO][(R + 1) * 32];
 
     const int lane = threadIdx.x;
     const int64_t m0 = (int64_t)blockIdx.x * R;
@@ -163,6 +163,11 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
     const int interior_end = (T & ~31) / TC;
     // rows shorter than a line could start and end inside the same line; they keep direct stores
     const bool route = T >= 32;
+    float4 keep[NO][G::kPasses];            // first-produced pieces of shared lines, one quad per pass
+#pragma unroll
+    for (int o = 0; o < NO; ++o)
+#pragma unroll
+        for (int p = 0; p < G::kPasses; ++p) keep[o][p] = make_float4(0.f, 0.f, 0.f, 0.f);
 
     const int crow = lane / G::kQuads;      // row within a pass (copy pattern)
     const int cq = lane % G::kQuads;        // quad within the row
@@ -253,47 +258,69 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
         }
         __syncthreads();
 
-        // LDS -> global; on edge chunks the quads of a line shared with a neighbouring row go to
-        // the boundary buffer instead (their global offset is pushed out of range)
+        // LDS -> global
+        if (interior) {
 #pragma unroll
-        for (int p = 0; p < G::kPasses; ++p) {
-            const int r = p * G::kRowsPerPass + crow;
-            const int t = step0[p] + chunk * TC;
-            int off = ((unsigned)t < (unsigned)T) ? off0[p] + chunk * (TC * 4) : kOutOfRange;
-            float4 v[NO];
+            for (int p = 0; p < G::kPasses; ++p) {
+                const int r = p * G::kRowsPerPass + crow;
+                const int off = off0[p] + chunk * (TC * 4);
 #pragma unroll
-            for (int o = 0; o < NO; ++o) v[o] = *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]);
-            if (!interior && route && (unsigned)t < (unsigned)T && r < rows) {
-                const int a = 4 * cq - step0[p];
-                const int pos = t + a;                     // position in the row's line-aligned window
-                const int last_full = (a + T) & ~31;
-                int slot = -1;
-                if (a != 0 && pos < 32) slot = r * 32 + pos;
-                else if (pos >= last_full) slot = (r + 1) * 32 + (pos - last_full);
-                if (slot >= 0) {
-                    off = kOutOfRange;
+                for (int o = 0; o < NO; ++o)
+                    buf_store4<STREAM>(dst[o], off, *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]));
+            }
+        } else {
+            // edge chunk.  The line shared by rows r-1 and r is assembled by the eight lanes that
+            // copy the first line of row r: quads at or after the row's phase are its head, the
+            // others the tail of row r-1, fetched from that row's tile in the chunk that holds it.
+            // Whichever piece is produced first waits in keep[][p].
+            const bool tails_here = chunk >= interior_end;   // chunks that can hold a row's partial last line
 #pragma unroll
-                    for (int o = 0; o < NO; ++o) *reinterpret_cast<float4*>(&bline[o][slot]) = v[o];
+            for (int p = 0; p < G::kPasses; ++p) {
+                const int r = p * G::kRowsPerPass + crow;
+                const int a = 4 * cq - step0[p];               // phase of row r
+                const int t = step0[p] + chunk * TC;
+                const bool valid = (unsigned)t < (unsigned)T;
+                int off = valid ? off0[p] + chunk * (TC * 4) : kOutOfRange;
+                const bool serves = route && r >= 1 && r < rows && a != 0 && cq < 8;   // lane holds quad cq of the shared line
+                const bool is_head = 4 * cq >= a;
+                const int tail_pos = (((a - T) & 31) + T) & ~31;   // window position of row r-1's partial last line
+                const int kp = tail_pos / TC;                      // chunk that holds it
+                const bool fetch_tail = serves && !is_head && chunk == kp;
+                const int tail_idx = fetch_tail ? (r - 1) * G::kPitch + (tail_pos - kp * TC) + 4 * cq : 0;
+                // quads of this row that another lane stores as part of an assembled line
+                const bool own_tail = route && valid && r + 1 < rows && 4 * cq + chunk * TC >= ((a + T) & ~31);
+                const bool own_head = serves && is_head && chunk == 0;
+                if (own_tail || (!Op::kReverse && own_head)) off = kOutOfRange;
+                if (Op::kReverse && serves && !is_head && chunk == 0) off = off0[p];
+#pragma unroll
+                for (int o = 0; o < NO; ++o) {
+                    float4 v = *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]);
+                    if (Op::kReverse) {
+                        // tails come first: fetch and hold them; chunk 0 stores head and held tail together
+                        if (tails_here) {
+                            const float4 tl = *reinterpret_cast<const float4*>(&tile[o][tail_idx]);
+                            if (fetch_tail) keep[o][p] = tl;
+                        }
+                        if (serves && !is_head && chunk == 0) v = keep[o][p];
+                    } else if (own_head) {
+                        keep[o][p] = v;                            // heads come first
+                    }
+                    buf_store4<STREAM>(dst[o], off, v);
+                }
+                if (!Op::kReverse && tails_here) {
+                    // the chunk with the tail of row r-1 stores it together with the held head of row r
+                    const int line_off = (serves && chunk == kp) ? off0[p] : kOutOfRange;
+#pragma unroll
+                    for (int o = 0; o < NO; ++o) {
+                        const float4 tl = *reinterpret_cast<const float4*>(&tile[o][tail_idx]);
+                        buf_store4<STREAM>(dst[o], line_off, is_head ? keep[o][p] : tl);
+                    }
                 }
             }
-#pragma unroll
-            for (int o = 0; o < NO; ++o) buf_store4<STREAM>(dst[o], off, v[o]);
         }
         __syncthreads();
     }
 
-    if (route) {
-        // boundary line b holds the tail of row b-1 (columns < phase(b)) and the head of row b
-        for (int i = lane; i < (R + 1) * 8; i += kWave) {
-            const int b = i >> 3, col = (i & 7) * 4;
-            const int a = phase(b);
-            const bool owned = (col < a) ? (b >= 1 && b - 1 < rows) : (b < rows);
-            const int off = (a != 0 && b <= rows && owned) ? (b * T - a + col) * 4 : kOutOfRange;
-#pragma unroll
-            for (int o = 0; o < NO; ++o)
-                buf_store4<STREAM>(dst[o], off, *reinterpret_cast<const float4*>(&bline[o][b * 32 + col]));
-        }
-    }
     op.finish(prm, m0 + lane, lane < rows);
 }
 

@@ -1,0 +1,92 @@
+"""Fused resonate-and-fire dynamics + phase-threshold spike on the GPU.
+
+No counterpart module in the reference: one kernel launch per direction for what
+``rf.Neuron.forward`` (neuron/rf.py:473-490 in the reference) does with ``resonator.dynamics``
+and ``complex.Spike.apply``, with bit-identical results.
+"""
+import torch
+
+from ... import _native as N
+from . import resonator as _res
+
+
+def dynamics(real_input, imag_input, sin_decay, cos_decay, real_state, imag_state, imag_last, w_scale,
+             threshold, tau_rho, scale_rho, graded_spike=False, spike_scale=1):
+    """(real, imag, spike) of an RF neuron (no reset).  ``imag_last`` is the imaginary response before
+    the first step (tensor shaped like the states, one element, or a number).  Gradients flow from
+    ``spike`` to both inputs and to sin_decay / cos_decay; real and imag are returned detached."""
+    return _RfFused.apply(real_input, imag_input, sin_decay, cos_decay, real_state, imag_state, imag_last,
+                          w_scale, threshold, tau_rho, scale_rho, graded_spike, spike_scale)
+
+
+def _fwd(real_input, imag_input, sin_decay, cos_decay, real_state, imag_state, imag_last, w_scale,
+         threshold, graded, spike_scale):
+    if not torch.is_tensor(imag_last):
+        imag_last = torch.tensor([float(imag_last)], dtype=real_input.dtype, device=real_input.device)
+    tensors = [real_input, imag_input, sin_decay, cos_decay, real_state, imag_state, imag_last]
+    dev = N.require_gpu(*tensors)
+    if real_input.shape != imag_input.shape:
+        raise RuntimeError(f'real/imag input shapes differ: {real_input.shape} vs {imag_input.shape}')
+    real_input, imag_input, sin_decay, cos_decay, real_state, imag_state, imag_last = \
+        [t.contiguous() for t in tensors]
+    M, T = N.rows_and_steps(real_input)
+    for name, s in (('real_state', real_state), ('imag_state', imag_state), ('imag_last', imag_last)):
+        if s.numel() not in (1, M):
+            raise RuntimeError(f'{name} has {s.numel()} elements, expected 1 or {M}')
+    real, imag, spk = (torch.empty_like(real_input) for _ in range(3))
+    with torch.cuda.device(dev):
+        N.check(N.lib().slayer_rf_fwd(
+            N.ptr(real), N.ptr(imag), N.ptr(spk), N.ptr(real_input), N.ptr(imag_input),
+            N.ptr(sin_decay), N.ptr(cos_decay), N.ptr(real_state), N.ptr(imag_state), N.ptr(imag_last),
+            float(threshold), 1 if graded else 0, float(spike_scale), int(w_scale),
+            M, N.neurons_per_batch(real_input), sin_decay.numel(),
+            real_state.numel(), imag_state.numel(), imag_last.numel(), T, N.stream_handle()))
+    return real, imag, spk
+
+
+def _bwd(grad_spikes, real, imag, sin_decay, cos_decay, threshold, tau_rho, scale_rho, graded,
+         need_decay_grad=True):
+    dev = N.require_gpu(grad_spikes, real, imag, sin_decay, cos_decay)
+    grad_spikes, sin_decay, cos_decay = grad_spikes.contiguous(), sin_decay.contiguous(), cos_decay.contiguous()
+    M, T = N.rows_and_steps(grad_spikes)
+    g_re, g_im = torch.empty_like(grad_spikes), torch.empty_like(grad_spikes)
+    g_sin = g_cos = workspace = None
+    if need_decay_grad:
+        g_sin = torch.empty(sin_decay.numel(), dtype=torch.float32, device=dev)
+        g_cos = torch.empty(cos_decay.numel(), dtype=torch.float32, device=dev)
+        workspace = torch.empty(2 * M + 128 * sin_decay.numel(), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        N.check(N.lib().slayer_rf_bwd(
+            N.ptr(g_re), N.ptr(g_im), N.ptr(g_sin), N.ptr(g_cos), N.ptr(grad_spikes), N.ptr(real), N.ptr(imag),
+            N.ptr(sin_decay), N.ptr(cos_decay), float(threshold), float(tau_rho), float(scale_rho),
+            1 if graded else 0, N.ptr(workspace),
+            M, N.neurons_per_batch(grad_spikes), sin_decay.numel(), T, N.stream_handle()))
+    return g_re, g_im, g_sin, g_cos
+
+
+class _RfFused(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, real_input, imag_input, sin_decay, cos_decay, real_state, imag_state, imag_last,
+                w_scale, threshold, tau_rho, scale_rho, graded, spike_scale):
+        graded = graded is True
+        last = imag_last.detach() if torch.is_tensor(imag_last) else imag_last
+        real, imag, spk = _fwd(real_input, imag_input, sin_decay.detach(), cos_decay.detach(),
+                               real_state.detach(), imag_state.detach(), last, w_scale, threshold, graded,
+                               spike_scale)
+        ctx.save_for_backward(real, imag, sin_decay, cos_decay)
+        ctx.cfg = (float(threshold), float(tau_rho), float(scale_rho), graded)
+        ctx.mark_non_differentiable(real, imag)
+        return real, imag, spk
+
+    @staticmethod
+    def backward(ctx, _g_re, _g_im, grad_spikes):
+        real, imag, sin_decay, cos_decay = ctx.saved_tensors
+        threshold, tau_rho, scale_rho, graded = ctx.cfg
+        need = ctx.needs_input_grad[2] or ctx.needs_input_grad[3]
+        g_re, g_im, g_sin, g_cos = _bwd(grad_spikes, real, imag, sin_decay.detach(), cos_decay.detach(),
+                                        threshold, tau_rho, scale_rho, graded, need)
+        _res._raise_on_nan(grad_spikes=grad_spikes, grad_real_input=g_re, grad_imag_input=g_im,
+                           grad_sin_decay=g_sin, grad_cos_decay=g_cos)
+        if g_sin is not None:
+            g_sin, g_cos = g_sin.reshape(sin_decay.shape), g_cos.reshape(cos_decay.shape)
+        return (g_re, g_im, g_sin, g_cos) + (None,) * 9

@@ -4,7 +4,7 @@ import numpy as np
 import torch
 
 from .base import Neuron as _Base
-from .dynamics import resonator
+from .dynamics import resonator, rf_fused
 from ..spike import complex as complex_spike
 from ..utils.quantize import quantize
 
@@ -100,5 +100,24 @@ class Neuron(_Base):
         return spike
 
     def forward(self, input):
-        real, imag = self.dynamics(input)
-        return self.spike(real, imag)
+        """Spike response to ``(real_input, imag_input)``.  Without input normalisation the dynamics
+        and the spike run as one fused kernel per direction (same bits as ``spike(*dynamics(input))``)."""
+        if self.real_norm is not None or self.imag_norm is not None:
+            real, imag = self.dynamics(input)
+            return self.spike(real, imag)
+        real_input, imag_input = input
+        if real_input.shape != imag_input.shape:
+            raise AssertionError(f'Real input tensor shape ({real_input.shape}) does not match '
+                                 f'with imaginary input shape ({imag_input.shape}).')
+        self._prepare(real_input)
+        real, imag, spike = rf_fused.dynamics(
+            real_input, imag_input, quantize(self.sin_decay), quantize(self.cos_decay),
+            self.real_state, self.imag_state, self.imag_state, self.s_scale, self.threshold,
+            self.tau_rho * TAU_RHO_MULT, self.scale_rho * SCALE_RHO_MULT, self.graded_spike, 1)
+        if self.persistent_state:
+            with torch.no_grad():
+                self.real_state = real[..., -1].clone()
+                self.imag_state = imag[..., -1].clone()
+        if self.drop is not None:
+            spike = self.drop(spike)
+        return spike

@@ -216,3 +216,59 @@ def test_cuba_neuron_forward_uses_fused_path_with_same_results(slayer):
         sa.sum().backward()
         sb.sum().backward()
         assert torch.equal(xa.grad, xb.grad)
+
+
+@pytest.mark.parametrize('shape,w,graded', [((4, 128, 200), 64, False), ((3, 70, 129), 100, False),
+                                            ((2, 3, 5, 7, 37), 4096, True), ((4, 9000, 64), 64, False),
+                                            ((4, 70000, 40), 64, False)])
+def test_fused_rf_equals_the_operator_chain(slayer, shape, w, graded):
+    from tests.util import seed_of
+    gen = torch.Generator().manual_seed(seed_of(shape, w, graded, 'rf fused'))
+    C = shape[1]
+    xr = sparse_input(gen, shape, p=0.2, amp=1.5).to(dev())
+    xi = sparse_input(gen, shape, p=0.2, amp=1.5).to(dev())
+    g = torch.randn(shape, generator=gen).to(dev())
+    mag = torch.rand(C, generator=gen) * 4000
+    ph = torch.rand(C, generator=gen) * 1.5
+    sin, cos = (mag * torch.sin(ph)).round().to(dev()), (mag * torch.cos(ph)).round().to(dev())
+    rs = torch.randn(shape[:-1], generator=gen).to(dev())
+    is_ = torch.randn(shape[:-1], generator=gen).to(dev())
+    last = torch.randn(shape[:-1], generator=gen).to(dev())
+    thr, tau, rho = 0.6, 0.5, 10.0
+    D = slayer.neuron.dynamics
+    a = [t.clone().requires_grad_() for t in (xr, xi, sin, cos)]
+    re, im = D.resonator.dynamics(a[0], a[1], a[2], a[3], rs, is_, w)
+    spk = slayer.spike.complex.Spike.apply(re, im, thr, tau, rho, graded, last, 2)
+    spk.backward(g)
+    b = [t.clone().requires_grad_() for t in (xr, xi, sin, cos)]
+    f_re, f_im, f_spk = D.rf_fused.dynamics(b[0], b[1], b[2], b[3], rs, is_, last, w, thr, tau, rho, graded, 2)
+    f_spk.backward(g)
+    assert float(spk.detach().abs().sum()) > 0
+    assert torch.equal(f_re, re.detach()) and torch.equal(f_im, im.detach()), 'fused traces differ'
+    assert torch.equal(f_spk.detach(), spk.detach()), 'fused spikes differ'
+    assert torch.equal(b[0].grad, a[0].grad) and torch.equal(b[1].grad, a[1].grad), 'fused input gradients differ'
+    assert_rel(b[2].grad.cpu(), a[2].grad.cpu(), 'fused grad sin', rel=1e-4)
+    assert_rel(b[3].grad.cpu(), a[3].grad.cpu(), 'fused grad cos', rel=1e-4)
+
+
+def test_rf_neuron_forward_uses_fused_path_with_same_results(slayer):
+    gen = torch.Generator().manual_seed(105)
+    shape = (3, 12, 150)
+    xr, xi = sparse_input(gen, shape, p=0.3).to(dev()), sparse_input(gen, shape, p=0.3).to(dev())
+    mk = lambda: slayer.neuron.rf.Neuron(1.0, [5, 20], [0.02, 0.1], shared_param=False, requires_grad=True,
+                                         persistent_state=True).to(dev())
+    a, b = mk(), mk()
+    a._prepare(xr)
+    b._prepare(xr)
+    for pa, pb in zip(a.parameters(), b.parameters()):
+        pb.data = pa.data.clone()
+    for k in range(2):
+        ia = (xr.clone().requires_grad_(), xi.clone().requires_grad_())
+        ib = (xr.clone().requires_grad_(), xi.clone().requires_grad_())
+        sa = a(ia)
+        sb = b.spike(*b.dynamics(ib))
+        assert torch.equal(sa.detach(), sb.detach()), f'call {k}: spikes differ'
+        assert torch.equal(a.real_state, b.real_state) and torch.equal(a.imag_state, b.imag_state)
+        sa.sum().backward()
+        sb.sum().backward()
+        assert torch.equal(ia[0].grad, ib[0].grad) and torch.equal(ia[1].grad, ib[1].grad)
