@@ -282,6 +282,34 @@ int slayer_rf_bwd(float *g_re_in, float *g_im_in, float *grad_sin, float *grad_c
                   float spike_threshold, float tau_rho, float scale_rho, int graded, float *workspace,
                   int64_t M, int64_t neurons_per_batch, int64_t num_decays, int64_t T, void *stream);
 
+/* ---- fused adaptive-threshold LIF neuron ---------------------------------------------------- */
+
+/* One launch for what alif.Neuron.forward does with five operators (neuron/alif.py:499-525 + :557-568 =
+ * leaky_integrator.dynamics twice without reset, adaptive_threshold.dynamics, threshold + refractory,
+ * Spike.forward); bit-identical to that chain, 20 instead of 52 bytes per neuron-timestep.
+ * theta_out receives threshold + refractory (what the spike compares against and what the backward pass
+ * needs); th_last_out / ref_last_out ([M], both or neither NULL) receive the threshold and refractory
+ * values of the last step, i.e. threshold[..., -1] and refractory[..., -1] of the separate operator. */
+int slayer_alif_fwd(float *cur_out, float *vol_out, float *theta_out, float *spk_out,
+                    float *th_last_out, float *ref_last_out, const float *in,
+                    const float *i_decay, const float *v_decay, const float *th_decay, const float *ref_decay,
+                    const float *i_state, const float *v_state, const float *th_state, const float *ref_state,
+                    int64_t th_step_scaled, int64_t th0_scaled, int graded, float spike_scale, int w_scale,
+                    int64_t M, int64_t neurons_per_batch,
+                    int64_t num_i_decays, int64_t num_v_decays, int64_t num_th_decays, int64_t num_ref_decays,
+                    int64_t num_i_states, int64_t num_v_states, int64_t num_th_states, int64_t num_ref_states,
+                    int64_t T, void *stream);
+
+/* Backward of the above = slayer_spike_bwd with a threshold tensor -> slayer_li_bwd twice, in one launch
+ * (20 instead of 40 bytes per neuron-timestep); grad_in is bit-identical to the chain.  grad_i_decay /
+ * grad_v_decay may both be NULL; workspace: 2*M + 64*(num_i_decays + num_v_decays) floats otherwise. */
+int slayer_alif_bwd(float *grad_in, float *grad_i_decay, float *grad_v_decay,
+                    const float *grad_spikes, const float *voltage, const float *theta, const float *current,
+                    const float *i_decay, const float *v_decay,
+                    float tau_rho, float scale_rho, int graded, float *workspace,
+                    int64_t M, int64_t neurons_per_batch, int64_t num_i_decays, int64_t num_v_decays,
+                    int64_t T, void *stream);
+
 /* ---- cross-check implementations (debug mode) ------------------------------------------------ */
 
 /* The reference's debug mode runs its CPU loop next to its kernel and raises on a difference

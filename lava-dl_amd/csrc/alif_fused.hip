@@ -1,0 +1,196 @@
+// Fused adaptive-threshold LIF neuron: current integrator -> voltage integrator (no reset) ->
+// threshold / refractory recurrences -> spike against threshold + refractory, in one pass over the
+// input (reads 4 B, writes 16 B per neuron-timestep instead of 52 B for the five separate
+// operators), and the matching backward pass (spike surrogate with a per-step threshold -> voltage
+// gradient -> current gradient; reads 16 B, writes 4 B instead of 40 B).  Intermediates make the
+// same float32 round trips as at the operator boundaries, so results are bit-identical to the chain.
+#include "common.h"
+#include "tile.h"
+
+namespace slayer {
+
+int launch_reduce_param_grad(float* grad, const float* partial, float* scratch, int64_t M, int64_t npb,
+                             int64_t num_params, hipStream_t stream);   // li.hip
+int launch_zero_fill(float* p, int64_t n, hipStream_t stream);          // li.hip
+
+template <bool POW2, bool GRADED>
+struct AlifFwd {
+    static constexpr int kIn = 1, kOut = 4;          // out: current, voltage, threshold + refractory, spikes
+    static constexpr bool kReverse = false;
+    static constexpr int64_t kRows32Below = 65536, kRows16Below = 16384;
+    struct Params {
+        const float* in[1];
+        float* out[4];
+        float *th_last, *ref_last;                   // [M] threshold / refractory of the last step, or nullptr
+        const float *i_decay, *v_decay, *th_decay, *ref_decay, *i_state, *v_state, *th_state, *ref_state;
+        int step, base;
+        float w, inv_w, spike_scale;
+        int64_t npb, n_id, n_vd, n_td, n_rd, n_is, n_vs, n_ts, n_rs;
+    };
+    int yc, yv, th, r, mi, mv, mt, mr, th_step, base;
+    float w, inv_w, spike_scale, th_f, ref_f;
+
+    __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
+        w = p.w; inv_w = p.inv_w; spike_scale = p.spike_scale; th_step = p.step; base = p.base;
+        yc = yv = th = r = mi = mv = mt = mr = 0;
+        th_f = ref_f = 0.f;
+        if (valid) {
+            yc = trunc_i32(p.i_state[p.n_is == 1 ? 0 : m] * w);
+            yv = trunc_i32(p.v_state[p.n_vs == 1 ? 0 : m] * w);
+            th = trunc_i32(p.th_state[p.n_ts == 1 ? 0 : m] * w);
+            r = trunc_i32(p.ref_state[p.n_rs == 1 ? 0 : m] * w);
+            mi = 4096 - trunc_i32(p.i_decay[param_index(m, p.npb, p.n_id)]);
+            mv = 4096 - trunc_i32(p.v_decay[param_index(m, p.npb, p.n_vd)]);
+            mt = 4096 - trunc_i32(p.th_decay[param_index(m, p.npb, p.n_td)]);
+            mr = 4096 - trunc_i32(p.ref_decay[param_index(m, p.npb, p.n_rd)]);
+        }
+    }
+    __device__ __forceinline__ void step(const float (&x)[1], float (&o)[4]) {
+        yc = rs0_12(yc, mi) + trunc_i32(w * x[0]);
+        const float cf = (float)yc;
+        const float cur = POW2 ? cf * inv_w : cf / w;
+        yv = rs0_12(yv, mv) + trunc_i32(w * cur);               // the voltage op reads the float32 current
+        const float vf = (float)yv;
+        const float vol = POW2 ? vf * inv_w : vf / w;
+        r = rs0_12(r, mr);
+        th = rs0_12(th - base, mt) + base;
+        const float thf = (float)th, rf = (float)r;
+        th_f = POW2 ? thf * inv_w : thf / w;
+        ref_f = POW2 ? rf * inv_w : rf / w;
+        const bool fired = trunc_i32(w * vol) >= th + r;        // the threshold op reads the float32 voltage
+        r += fired ? 2 * th : 0;
+        th += fired ? th_step : 0;
+        const float theta = th_f + ref_f;
+        const float h = (vol >= theta) ? 1.0f : 0.0f;
+        o[0] = cur;
+        o[1] = vol;
+        o[2] = theta;
+        o[3] = GRADED ? (h * vol) / spike_scale : h;
+    }
+    __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
+        if (valid && p.th_last) { p.th_last[m] = th_f; p.ref_last[m] = ref_f; }
+    }
+};
+
+template <bool GRADED>
+struct AlifBwd {
+    static constexpr int kIn = 4, kOut = 1;          // in: grad of spikes, saved voltage, threshold + refractory, current
+    static constexpr bool kReverse = true;
+    static constexpr int64_t kRows32Below = 65536, kRows16Below = 16384;
+    struct Params {
+        const float* in[4];
+        float* out[1];
+        const float *i_decay, *v_decay;
+        float *partial_i, *partial_v;                // per-neuron decay gradients, or nullptr
+        float tau, rho;
+        int64_t npb, n_id, n_vd;
+    };
+    float ai, av, gc, gx, acc_i, acc_v, tau, rho, lead;
+
+    __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
+        tau = p.tau; rho = p.rho;
+        lead = (rho / 2.0f) / tau;
+        ai = av = gc = gx = acc_i = acc_v = 0.f;
+        if (valid) {
+            ai = 1.0f - p.i_decay[param_index(m, p.npb, p.n_id)] / 4096.0f;
+            av = 1.0f - p.v_decay[param_index(m, p.npb, p.n_vd)] / 4096.0f;
+        }
+    }
+    __device__ __forceinline__ void step(const float (&x)[4], float (&o)[1]) {
+        const float d = x[1] - x[2];
+        const float gv = GRADED ? (rho * expf(fminf(d, 0.0f) / tau)) * x[0] : (lead * expf(-fabsf(d) / tau)) * x[0];
+        acc_v = __fmaf_rn(gc, x[1], acc_v);          // gc, gx still hold the gradients of step t+1
+        acc_i = __fmaf_rn(gx, x[3], acc_i);
+        gc = av * gc + gv;
+        gx = ai * gx + gc;
+        o[0] = gx;
+    }
+    __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
+        if (valid && p.partial_i) { p.partial_i[m] = acc_i; p.partial_v[m] = acc_v; }
+    }
+};
+
+}  // namespace slayer
+
+using namespace slayer;
+
+extern "C" int slayer_alif_fwd(float* cur_out, float* vol_out, float* theta_out, float* spk_out,
+                               float* th_last_out, float* ref_last_out, const float* in,
+                               const float* i_decay, const float* v_decay, const float* th_decay, const float* ref_decay,
+                               const float* i_state, const float* v_state, const float* th_state, const float* ref_state,
+                               int64_t th_step_scaled, int64_t th0_scaled, int graded, float spike_scale, int w_scale,
+                               int64_t M, int64_t neurons_per_batch,
+                               int64_t num_i_decays, int64_t num_v_decays, int64_t num_th_decays, int64_t num_ref_decays,
+                               int64_t num_i_states, int64_t num_v_states, int64_t num_th_states, int64_t num_ref_states,
+                               int64_t T, void* stream) {
+    if (int e = check_rows(M, T)) return e;
+    if (M == 0 || T == 0) return 0;
+    if (!cur_out || !vol_out || !theta_out || !spk_out || !in || !i_decay || !v_decay || !th_decay || !ref_decay ||
+        !i_state || !v_state || !th_state || !ref_state)
+        return SLAYER_ENULL;
+    if ((th_last_out == nullptr) != (ref_last_out == nullptr)) return SLAYER_ENULL;
+    for (int64_t n : {num_i_decays, num_v_decays, num_th_decays, num_ref_decays})
+        if (int e = check_params(M, neurons_per_batch, n)) return e;
+    for (int64_t n : {num_i_states, num_v_states, num_th_states, num_ref_states})
+        if (int e = check_states(M, n)) return e;
+    if (w_scale == 0) return SLAYER_EINVAL;
+    const int64_t lim = 0x7fffffffLL;
+    if (th_step_scaled > lim || th_step_scaled < -lim || th0_scaled > lim || th0_scaled < -lim) return SLAYER_ERANGE;
+    const float w = (float)w_scale;
+    hipStream_t st = (hipStream_t)stream;
+#define SLAYER_ALIF(P, G)                                                                                         \
+    do {                                                                                                          \
+        AlifFwd<P, G>::Params p{{in}, {cur_out, vol_out, theta_out, spk_out}, th_last_out, ref_last_out,            \
+                                i_decay, v_decay, th_decay, ref_decay, i_state, v_state, th_state, ref_state,       \
+                                (int)th_step_scaled, (int)th0_scaled, w, 1.0f / w, spike_scale, neurons_per_batch,  \
+                                num_i_decays, num_v_decays, num_th_decays, num_ref_decays,                          \
+                                num_i_states, num_v_states, num_th_states, num_ref_states};                         \
+        return launch_stream<AlifFwd<P, G>>(p, M, T, st);                                                           \
+    } while (0)
+    if (is_pow2(w_scale)) { if (graded) SLAYER_ALIF(true, true); else SLAYER_ALIF(true, false); }
+    if (graded) SLAYER_ALIF(false, true);
+    SLAYER_ALIF(false, false);
+#undef SLAYER_ALIF
+}
+
+extern "C" int slayer_alif_bwd(float* grad_in, float* grad_i_decay, float* grad_v_decay,
+                               const float* grad_spikes, const float* voltage, const float* theta, const float* current,
+                               const float* i_decay, const float* v_decay,
+                               float tau_rho, float scale_rho, int graded, float* workspace,
+                               int64_t M, int64_t neurons_per_batch, int64_t num_i_decays, int64_t num_v_decays,
+                               int64_t T, void* stream) {
+    if (int e = check_rows(M, T)) return e;
+    const int64_t mm = M > 0 ? M : neurons_per_batch;
+    if (int e = check_params(mm, neurons_per_batch, num_i_decays)) return e;
+    if (int e = check_params(mm, neurons_per_batch, num_v_decays)) return e;
+    if ((grad_i_decay == nullptr) != (grad_v_decay == nullptr)) return SLAYER_ENULL;
+    const bool want = grad_i_decay != nullptr;
+    if (want && !workspace && M > 0) return SLAYER_ENULL;
+    hipStream_t st = (hipStream_t)stream;
+    if (M > 0 && T > 0) {
+        if (!grad_in || !grad_spikes || !voltage || !theta || !current || !i_decay || !v_decay) return SLAYER_ENULL;
+        if (graded) {
+            AlifBwd<true>::Params p{{grad_spikes, voltage, theta, current}, {grad_in}, i_decay, v_decay,
+                                    want ? workspace : nullptr, want ? workspace + M : nullptr,
+                                    tau_rho, scale_rho, neurons_per_batch, num_i_decays, num_v_decays};
+            if (int e = launch_stream<AlifBwd<true>>(p, M, T, st)) return e;
+        } else {
+            AlifBwd<false>::Params p{{grad_spikes, voltage, theta, current}, {grad_in}, i_decay, v_decay,
+                                     want ? workspace : nullptr, want ? workspace + M : nullptr,
+                                     tau_rho, scale_rho, neurons_per_batch, num_i_decays, num_v_decays};
+            if (int e = launch_stream<AlifBwd<false>>(p, M, T, st)) return e;
+        }
+    }
+    if (want) {
+        if (M == 0 || T == 0) {
+            if (int e = launch_zero_fill(grad_i_decay, num_i_decays, st)) return e;
+            return launch_zero_fill(grad_v_decay, num_v_decays, st);
+        }
+        float* scratch = workspace + 2 * M;
+        if (int e = launch_reduce_param_grad(grad_i_decay, workspace, scratch, M, neurons_per_batch, num_i_decays, st))
+            return e;
+        return launch_reduce_param_grad(grad_v_decay, workspace + M, scratch + 64 * num_i_decays, M,
+                                        neurons_per_batch, num_v_decays, st);
+    }
+    return 0;
+}

@@ -3,7 +3,7 @@
 import torch
 
 from .base import Neuron as _Base
-from .dynamics import leaky_integrator, adaptive_threshold
+from .dynamics import leaky_integrator, adaptive_threshold, alif_fused
 from ..spike import Spike
 
 TAU_RHO_MULT = 100
@@ -64,5 +64,25 @@ class Neuron(_Base):
         return spike
 
     def forward(self, input):
-        _, voltage, threshold, refractory = self.dynamics(input)
-        return self.spike(voltage, threshold, refractory)
+        """Spike response.  Without a norm the whole neuron runs as one fused kernel per direction
+        (same bits as ``spike(*dynamics(input)[1:])``)."""
+        if self.norm is not None:
+            _, voltage, threshold, refractory = self.dynamics(input)
+            return self.spike(voltage, threshold, refractory)
+        self._prepare(input)
+        current, voltage, _, spike, th_last, ref_last = alif_fused.dynamics(
+            input, self._q('current_decay'), self._q('voltage_decay'), self._q('threshold_decay'),
+            self._q('refractory_decay'), self.current_state, self.voltage_state, self.threshold_state,
+            self.refractory_state, self.threshold_step, self.threshold, self.s_scale,
+            self.tau_rho * TAU_RHO_MULT, self.scale_rho * SCALE_RHO_MULT, self.graded_spike, 1)
+        if self.persistent_state:
+            with torch.no_grad():
+                last = spike[..., -1]
+                self.current_state = current[..., -1].clone()
+                self.voltage_state = voltage[..., -1].clone()
+                self.refractory_state = adaptive_threshold.persistent_ref_state(ref_last, last, th_last).detach().clone()
+                self.threshold_state = adaptive_threshold.persistent_th_state(
+                    th_last, last, self.threshold_step).detach().clone()
+        if self.drop is not None:
+            spike = self.drop(spike)
+        return spike

@@ -1,5 +1,5 @@
 from . import (leaky_integrator, adaptive_threshold, resonator, adaptive_phase_th, adaptive_resonator,
-               cuba_fused, rf_fused)
+               cuba_fused, rf_fused, alif_fused)
 
 __all__ = ['leaky_integrator', 'adaptive_threshold', 'resonator', 'adaptive_phase_th', 'adaptive_resonator',
-           'cuba_fused', 'rf_fused']
+           'cuba_fused', 'rf_fused', 'alif_fused']

@@ -1,0 +1,92 @@
+"""Fused adaptive-threshold LIF dynamics + spike on the GPU.
+
+No counterpart module in the reference: one kernel launch per direction for what
+``alif.Neuron.forward`` (neuron/alif.py:499-525 and :557-591 in the reference) does with
+``leaky_integrator.dynamics`` twice, ``adaptive_threshold.dynamics``, a tensor add and
+``Spike.apply``, with bit-identical results.
+"""
+import torch
+
+from ... import _native as N
+
+
+def dynamics(input, current_decay, voltage_decay, threshold_decay, refractory_decay,
+             current_state, voltage_state, threshold_state, refractory_state,
+             threshold_step, threshold_base, w_scale, tau_rho, scale_rho, graded_spike=False, spike_scale=1):
+    """(current, voltage, theta, spike, threshold_last, refractory_last) of an ALIF neuron, where
+    ``theta = threshold + refractory`` is what the spike compares the voltage against and the two
+    ``*_last`` tensors (shaped like the states) are the threshold and refractory values of the last
+    step.  Gradients flow from ``spike`` to ``input`` and to the current / voltage decays (the
+    threshold dynamics has none, as in the separate operator); the other outputs are detached."""
+    return _AlifFused.apply(input, current_decay, voltage_decay, threshold_decay, refractory_decay,
+                            current_state, voltage_state, threshold_state, refractory_state,
+                            threshold_step, threshold_base, w_scale, tau_rho, scale_rho, graded_spike, spike_scale)
+
+
+def _fwd(input, decays, states, threshold_step, threshold_base, w_scale, graded, spike_scale, want_last=True):
+    """decays = (current, voltage, threshold, refractory), states likewise."""
+    dev = N.require_gpu(input, *decays, *states)
+    input = input.contiguous()
+    decays = [d.contiguous() for d in decays]
+    states = [s.contiguous() for s in states]
+    M, T = N.rows_and_steps(input)
+    for name, s in zip(('current_state', 'voltage_state', 'threshold_state', 'refractory_state'), states):
+        if s.numel() not in (1, M):
+            raise RuntimeError(f'{name} has {s.numel()} elements, expected 1 or {M}')
+    cur, vol, theta, spk = (torch.empty_like(input) for _ in range(4))
+    th_last = ref_last = None
+    if want_last:
+        th_last = torch.empty(input.shape[:-1], dtype=input.dtype, device=dev)
+        ref_last = torch.empty(input.shape[:-1], dtype=input.dtype, device=dev)
+    with torch.cuda.device(dev):
+        N.check(N.lib().slayer_alif_fwd(
+            N.ptr(cur), N.ptr(vol), N.ptr(theta), N.ptr(spk), N.ptr(th_last), N.ptr(ref_last), N.ptr(input),
+            *[N.ptr(d) for d in decays], *[N.ptr(s) for s in states],
+            int(threshold_step * w_scale), int(threshold_base * w_scale), 1 if graded else 0, float(spike_scale),
+            int(w_scale), M, N.neurons_per_batch(input), *[d.numel() for d in decays],
+            *[s.numel() for s in states], T, N.stream_handle()))
+    return cur, vol, theta, spk, th_last, ref_last
+
+
+def _bwd(grad_spikes, vol, theta, cur, i_decay, v_decay, tau_rho, scale_rho, graded, need_decay_grad=True):
+    dev = N.require_gpu(grad_spikes, vol, theta, cur, i_decay, v_decay)
+    grad_spikes, i_decay, v_decay = grad_spikes.contiguous(), i_decay.contiguous(), v_decay.contiguous()
+    M, T = N.rows_and_steps(grad_spikes)
+    grad_input = torch.empty_like(grad_spikes)
+    g_i = g_v = workspace = None
+    if need_decay_grad:
+        g_i = torch.empty(i_decay.numel(), dtype=torch.float32, device=dev)
+        g_v = torch.empty(v_decay.numel(), dtype=torch.float32, device=dev)
+        workspace = torch.empty(2 * M + 64 * (i_decay.numel() + v_decay.numel()), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        N.check(N.lib().slayer_alif_bwd(
+            N.ptr(grad_input), N.ptr(g_i), N.ptr(g_v), N.ptr(grad_spikes), N.ptr(vol), N.ptr(theta), N.ptr(cur),
+            N.ptr(i_decay), N.ptr(v_decay), float(tau_rho), float(scale_rho), 1 if graded else 0, N.ptr(workspace),
+            M, N.neurons_per_batch(grad_spikes), i_decay.numel(), v_decay.numel(), T, N.stream_handle()))
+    return grad_input, g_i, g_v
+
+
+class _AlifFused(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input, i_decay, v_decay, th_decay, ref_decay, i_state, v_state, th_state, ref_state,
+                threshold_step, threshold_base, w_scale, tau_rho, scale_rho, graded, spike_scale):
+        graded = graded is True
+        outs = _fwd(input, [d.detach() for d in (i_decay, v_decay, th_decay, ref_decay)],
+                    [s.detach() for s in (i_state, v_state, th_state, ref_state)],
+                    threshold_step, threshold_base, w_scale, graded, spike_scale)
+        cur, vol, theta, spk, th_last, ref_last = outs
+        ctx.save_for_backward(cur, vol, theta, i_decay, v_decay)
+        ctx.cfg = (float(tau_rho), float(scale_rho), graded)
+        ctx.mark_non_differentiable(cur, vol, theta, th_last, ref_last)
+        return outs
+
+    @staticmethod
+    def backward(ctx, _g_cur, _g_vol, _g_theta, grad_spikes, _g_th, _g_ref):
+        cur, vol, theta, i_decay, v_decay = ctx.saved_tensors
+        tau_rho, scale_rho, graded = ctx.cfg
+        need = ctx.needs_input_grad[1] or ctx.needs_input_grad[2]
+        g_in, g_i, g_v = _bwd(grad_spikes, vol, theta, cur, i_decay.detach(), v_decay.detach(),
+                              tau_rho, scale_rho, graded, need)
+        if g_i is not None:
+            g_i, g_v = g_i.reshape(i_decay.shape), g_v.reshape(v_decay.shape)
+        return (g_in, g_i, g_v) + (None,) * 13

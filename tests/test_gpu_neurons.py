@@ -272,3 +272,63 @@ def test_rf_neuron_forward_uses_fused_path_with_same_results(slayer):
         sa.sum().backward()
         sb.sum().backward()
         assert torch.equal(ia[0].grad, ib[0].grad) and torch.equal(ia[1].grad, ib[1].grad)
+
+
+@pytest.mark.parametrize('shape,w,graded', [((4, 128, 200), 64, False), ((3, 70, 129), 100, False),
+                                            ((2, 3, 5, 7, 37), 4096, True), ((4, 9000, 64), 64, False),
+                                            ((4, 70000, 40), 64, True)])
+def test_fused_alif_equals_the_operator_chain(slayer, shape, w, graded):
+    from tests.util import seed_of
+    gen = torch.Generator().manual_seed(seed_of(shape, w, graded, 'alif fused'))
+    C = shape[1]
+    x = sparse_input(gen, shape, p=0.3, amp=2.0).to(dev())
+    g = torch.randn(shape, generator=gen).to(dev())
+    d_i, d_v, d_th, d_ref = (torch.randint(0, 4096, (C,), generator=gen).float().to(dev()) for _ in range(4))
+    s_i, s_v = (torch.randn(shape[:-1], generator=gen).to(dev()) for _ in range(2))
+    s_th = (1.0 + torch.rand(shape[:-1], generator=gen)).to(dev())
+    s_ref = torch.rand(shape[:-1], generator=gen).to(dev())
+    step, base, tau, rho = 0.5, 1.0, 0.7, 1.5
+    D = slayer.neuron.dynamics
+    a = [t.clone().requires_grad_() for t in (x, d_i, d_v)]
+    cur = D.leaky_integrator.dynamics(a[0], a[1], s_i, w)
+    vol = D.leaky_integrator.dynamics(cur, a[2], s_v, w)
+    th, ref = D.adaptive_threshold.dynamics(vol, s_ref, d_ref, s_th, d_th, step, base, w)
+    spk = slayer.spike.Spike.apply(vol, th + ref, tau, rho, graded, s_v, 2)
+    spk.backward(g)
+    b = [t.clone().requires_grad_() for t in (x, d_i, d_v)]
+    f_cur, f_vol, f_theta, f_spk, f_th, f_ref = D.alif_fused.dynamics(
+        b[0], b[1], b[2], d_th, d_ref, s_i, s_v, s_th, s_ref, step, base, w, tau, rho, graded, 2)
+    f_spk.backward(g)
+    assert 0 < float((spk.detach() != 0).float().mean()) < 1
+    assert torch.equal(f_cur, cur.detach()) and torch.equal(f_vol, vol.detach()), 'fused traces differ'
+    assert torch.equal(f_theta, (th + ref).detach()), 'fused threshold + refractory differs'
+    assert torch.equal(f_th, th[..., -1]) and torch.equal(f_ref, ref[..., -1]), 'fused final states differ'
+    assert torch.equal(f_spk.detach(), spk.detach()), 'fused spikes differ'
+    assert torch.equal(b[0].grad, a[0].grad), 'fused input gradient differs'
+    assert_rel(b[1].grad.cpu(), a[1].grad.cpu(), 'fused grad current decay', rel=1e-4)
+    assert_rel(b[2].grad.cpu(), a[2].grad.cpu(), 'fused grad voltage decay', rel=1e-4)
+
+
+def test_alif_neuron_forward_uses_fused_path_with_same_results(slayer):
+    gen = torch.Generator().manual_seed(106)
+    shape = (3, 12, 150)
+    x = sparse_input(gen, shape, p=0.3, amp=2.0).to(dev())
+    mk = lambda: slayer.neuron.alif.Neuron(1.0, 0.5, [0.25, 0.3], [0.05, 0.1], [0.1, 0.2], [0.2, 0.3],
+                                           shared_param=False, requires_grad=True, persistent_state=True).to(dev())
+    a, b = mk(), mk()
+    a._prepare(x)                                   # per-channel decays are drawn at random on the first call
+    b._prepare(x)
+    for pa, pb in zip(a.parameters(), b.parameters()):
+        pb.data = pa.data.clone()
+    for k in range(3):
+        xa, xb = x.clone().requires_grad_(), x.clone().requires_grad_()
+        sa = a(xa)
+        _, vol, th, ref = b.dynamics(xb)
+        sb = b.spike(vol, th, ref)
+        assert torch.equal(sa.detach(), sb.detach()), f'call {k}: spikes differ'
+        for name in ('current_state', 'voltage_state', 'threshold_state', 'refractory_state'):
+            assert torch.equal(getattr(a, name), getattr(b, name)), f'call {k}: {name} differs'
+        sa.sum().backward()
+        sb.sum().backward()
+        assert torch.equal(xa.grad, xb.grad), f'call {k}: input gradients differ'
+    assert float(sa.detach().sum()) > 0
