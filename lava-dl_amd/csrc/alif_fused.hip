@@ -17,7 +17,7 @@ template <bool POW2, bool GRADED>
 struct AlifFwd {
     static constexpr int kIn = 1, kOut = 4;          // out: current, voltage, threshold + refractory, spikes
     static constexpr bool kReverse = false;
-    static constexpr int64_t kRows32Below = 65536, kRows16Below = 16384;
+    static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
     struct Params {
         const float* in[1];
         float* out[4];
@@ -76,7 +76,7 @@ template <bool GRADED>
 struct AlifBwd {
     static constexpr int kIn = 4, kOut = 1;          // in: grad of spikes, saved voltage, threshold + refractory, current
     static constexpr bool kReverse = true;
-    static constexpr int64_t kRows32Below = 65536, kRows16Below = 16384;
+    static constexpr int64_t kRows32Below = 4096, kRows16Below = 4096;     // exp per step: keep all lanes busy
     struct Params {
         const float* in[4];
         float* out[1];

@@ -8,7 +8,7 @@ template <bool POW2>
 struct AthFwd {
     static constexpr int kIn = 1, kOut = 2;      // out: threshold trace, refractory trace
     static constexpr bool kReverse = false;
-    static constexpr int64_t kRows32Below = 65536, kRows16Below = 16384;
+    static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
     struct Params {
         const float* in[1];
         float* out[2];
@@ -49,7 +49,7 @@ template <bool POW2>
 struct ApthFwd {
     static constexpr int kIn = 2, kOut = 2;      // in: real, imag;  out: threshold, refractory
     static constexpr bool kReverse = false;
-    static constexpr int64_t kRows32Below = 65536, kRows16Below = 16384;
+    static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
     struct Params {
         const float* in[2];
         float* out[2];

@@ -17,7 +17,7 @@ template <bool POW2, bool GRADED>
 struct CubaFwd {
     static constexpr int kIn = 1, kOut = 3;          // out: current, voltage, spikes
     static constexpr bool kReverse = false;
-    static constexpr int64_t kRows32Below = 65536, kRows16Below = 16384;
+    static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
     struct Params {
         const float* in[1];
         float* out[3];
@@ -58,7 +58,7 @@ template <bool GRADED>
 struct CubaBwd {
     static constexpr int kIn = 3, kOut = 1;          // in: grad of spikes, saved voltage, saved current
     static constexpr bool kReverse = true;
-    static constexpr int64_t kRows32Below = 65536, kRows16Below = 16384;   // exp per step: keep all lanes busy
+    static constexpr int64_t kRows32Below = 4096, kRows16Below = 4096;     // exp per step: keep all lanes busy
     struct Params {
         const float* in[3];
         float* out[1];

@@ -9,7 +9,7 @@ template <bool POW2>
 struct LiFwd {
     static constexpr int kIn = 1, kOut = 1;
     static constexpr bool kReverse = false;
-    static constexpr int64_t kRows32Below = kAlways, kRows16Below = 65536;
+    static constexpr int64_t kRows32Below = 32768, kRows16Below = 8192;
     struct Params {
         const float* in[1];
         float* out[1];

@@ -12,7 +12,7 @@ template <bool POW2, bool HAS_THR>
 struct ResFwd {
     static constexpr int kIn = 2, kOut = 2;
     static constexpr bool kReverse = false;
-    static constexpr int64_t kRows32Below = 65536, kRows16Below = 16384;
+    static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
     struct Params {
         const float* in[2];
         float* out[2];
@@ -111,7 +111,7 @@ struct AdResFwd {
 struct ResBwd {
     static constexpr int kIn = 4, kOut = 2;      // in: g_re, g_im, saved re, saved im
     static constexpr bool kReverse = true;
-    static constexpr int64_t kRows32Below = 262144, kRows16Below = 262144;
+    static constexpr int64_t kRows32Below = kAlways, kRows16Below = 16384;
     struct Params {
         const float* in[4];
         float* out[2];

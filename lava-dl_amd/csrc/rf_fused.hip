@@ -16,7 +16,7 @@ template <bool POW2, bool GRADED>
 struct RfFwd {
     static constexpr int kIn = 2, kOut = 3;          // out: real, imag, spikes
     static constexpr bool kReverse = false;
-    static constexpr int64_t kRows32Below = 65536, kRows16Below = 16384;
+    static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
     struct Params {
         const float* in[2];
         float* out[3];
@@ -59,7 +59,7 @@ template <bool GRADED>
 struct RfBwd {
     static constexpr int kIn = 3, kOut = 2;          // in: grad of spikes, saved real, saved imag
     static constexpr bool kReverse = true;
-    static constexpr int64_t kRows32Below = 65536, kRows16Below = 16384;
+    static constexpr int64_t kRows32Below = 4096, kRows16Below = 4096;     // exp per step: keep all lanes busy
     struct Params {
         const float* in[3];
         float* out[2];
