@@ -15,7 +15,8 @@ int launch_zero_fill(float* p, int64_t n, hipStream_t stream);          // li.hi
 
 template <bool POW2, bool GRADED>
 struct AlifFwd {
-    static constexpr int kIn = 1, kOut = 4;          // out: current, voltage, threshold + refractory, spikes
+    static constexpr int kIn = 1, kOut = 3;          // out: current, voltage, threshold + refractory
+    static constexpr int kDerived = 1;               // spikes: a function of voltage and threshold + refractory
     static constexpr bool kReverse = false;
     static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
     struct Params {
@@ -45,7 +46,7 @@ struct AlifFwd {
             mr = 4096 - trunc_i32(p.ref_decay[param_index(m, p.npb, p.n_rd)]);
         }
     }
-    __device__ __forceinline__ void step(const float (&x)[1], float (&o)[4]) {
+    __device__ __forceinline__ void step(const float (&x)[1], float (&o)[3]) {
         yc = rs0_12(yc, mi) + trunc_i32(w * x[0]);
         const float cf = (float)yc;
         const float cur = POW2 ? cf * inv_w : cf / w;
@@ -60,12 +61,17 @@ struct AlifFwd {
         const bool fired = trunc_i32(w * vol) >= th + r;        // the threshold op reads the float32 voltage
         r += fired ? 2 * th : 0;
         th += fired ? th_step : 0;
-        const float theta = th_f + ref_f;
-        const float h = (vol >= theta) ? 1.0f : 0.0f;
         o[0] = cur;
         o[1] = vol;
-        o[2] = theta;
-        o[3] = GRADED ? (h * vol) / spike_scale : h;
+        o[2] = th_f + ref_f;
+    }
+    __device__ __forceinline__ float spike(float vol, float theta) const {
+        const float h = (vol >= theta) ? 1.0f : 0.0f;
+        return GRADED ? (h * vol) / spike_scale : h;
+    }
+    __device__ __forceinline__ float4 derive(const float4 (&y)[3]) const {
+        return make_float4(spike(y[1].x, y[2].x), spike(y[1].y, y[2].y), spike(y[1].z, y[2].z),
+                           spike(y[1].w, y[2].w));
     }
     __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
         if (valid && p.th_last) { p.th_last[m] = th_f; p.ref_last[m] = ref_f; }

@@ -15,7 +15,8 @@ int launch_zero_fill(float* p, int64_t n, hipStream_t stream);          // li.hi
 
 template <bool POW2, bool GRADED>
 struct CubaFwd {
-    static constexpr int kIn = 1, kOut = 3;          // out: current, voltage, spikes
+    static constexpr int kIn = 1, kOut = 2;          // out: current, voltage
+    static constexpr int kDerived = 1;               // spikes: a function of the voltage alone
     static constexpr bool kReverse = false;
     static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
     struct Params {
@@ -38,18 +39,22 @@ struct CubaFwd {
             mv = 4096 - trunc_i32(p.v_decay[param_index(m, p.npb, p.n_vd)]);
         }
     }
-    __device__ __forceinline__ void step(const float (&x)[1], float (&o)[3]) {
+    __device__ __forceinline__ void step(const float (&x)[1], float (&o)[2]) {
         yc = rs0_12(yc, mi) + trunc_i32(w * x[0]);
         const float cf = (float)yc;
         const float cur = POW2 ? cf * inv_w : cf / w;
         const int yn = rs0_12(yv, mv) + trunc_i32(w * cur);     // the voltage op reads the float32 current
         const float vf = (float)yn;
-        const float vol = POW2 ? vf * inv_w : vf / w;
         yv = (vf >= thr) ? 0 : yn;
-        const float h = (vol >= spike_thr) ? 1.0f : 0.0f;
         o[0] = cur;
-        o[1] = vol;
-        o[2] = GRADED ? (h * vol) / spike_scale : h;
+        o[1] = POW2 ? vf * inv_w : vf / w;
+    }
+    __device__ __forceinline__ float spike(float vol) const {
+        const float h = (vol >= spike_thr) ? 1.0f : 0.0f;
+        return GRADED ? (h * vol) / spike_scale : h;
+    }
+    __device__ __forceinline__ float4 derive(const float4 (&y)[2]) const {
+        return make_float4(spike(y[1].x), spike(y[1].y), spike(y[1].z), spike(y[1].w));
     }
     __device__ __forceinline__ void finish(const Params&, int64_t, bool) {}
 };

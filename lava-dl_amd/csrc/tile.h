@@ -76,11 +76,21 @@ struct TileGeom {
 
 // An Op provides:
 //   static constexpr int kIn, kOut;  static constexpr bool kReverse;
+//   optionally static constexpr int kDerived = 1 and
+//     __device__ float4 derive(const float4 (&y)[kOut]) const;   (uses wave-uniform members only)
+//     an extra output, Params::out[kOut], that is an elementwise function of the other outputs of
+//     the same step: it is computed while a quad is copied out and needs neither an LDS tile nor
+//     boundary registers
 //   static constexpr int64_t kRows32Below, kRows16Below;   (rows-per-wave policy, see launch_stream)
 //   struct Params { const float* in[kIn]; float* out[kOut]; ... };
 //   __device__ void init(const Params&, int64_t m, bool valid);
 //   __device__ void step(const float (&x)[kIn], float (&y)[kOut]);
 //   __device__ void finish(const Params&, int64_t m, bool valid);
+
+template <class Op, class = void>
+struct DerivedCount { static constexpr int value = 0; };
+template <class Op>
+struct DerivedCount<Op, decltype((void)Op::kDerived)> { static constexpr int value = Op::kDerived; };
 
 // ---------------------------------------------------------------------------------------------
 // Buffer addressing.  Global accesses of the dwordx4 path go through raw buffer instructions whose
@@ -120,9 +130,9 @@ __device__ __forceinline__ void buf_store4(__amdgpu_buffer_rsrc_t r, int byte_of
 // row r+1, and the two pieces are produced a whole row apart in time.  Written when produced, each
 // piece reaches memory as a partial line, which costs a read-modify-write there (measured: ~16% of
 // the kernel at T = 300).  So the piece that comes first (the head of row r+1 in a forward pass,
-// the tail of row r in a reverse pass) waits in registers, and the eight lanes that copy the first
-// line of row r+1 store the whole line with one instruction once the other piece exists.  Only
-// the lines shared with neighbouring workgroups are still written in pieces.
+// the tail of row r in a reverse pass) waits in registers of the lanes that will store the other
+// piece, and the eight lanes that cover the line store it whole with one instruction.  Only the
+// lines shared with neighbouring workgroups are still written in pieces.
 //
 // Interior chunks (every column of every row inside [0, T), no shared line) run a branch-free
 // recurrence loop; only the first and the last one or two chunks take the predicated path.
@@ -130,7 +140,8 @@ template <class Op, int R, bool STREAM>
 __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, int64_t M, int T) {
     using G = TileGeom<R>;
     constexpr int TC = G::kChunk;
-    constexpr int NI = Op::kIn, NO = Op::kOut, NT = NI > NO ? NI : NO;
+    constexpr int NI = Op::kIn, NO = Op::kOut, ND = DerivedCount<Op>::value, NT = NI > NO ? NI : NO;
+    static_assert(ND == 0 || ND == 1, "at most one derived output");
     __shared__ __attribute__((aligned(16))) float tile[NT][G::kTileFloats];
 
     const int lane = threadIdx.x;
@@ -140,12 +151,19 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
     Op op;
     op.init(prm, m0 + lane, lane < rows);
 
-    __amdgpu_buffer_rsrc_t src[NI], dst[NO];
+    __amdgpu_buffer_rsrc_t src[NI], dst[NO + ND];
     const unsigned wave_bytes = (unsigned)rows * (unsigned)T * 4u;
 #pragma unroll
     for (int i = 0; i < NI; ++i) src[i] = make_rsrc(prm.in[i] + m0 * (int64_t)T, wave_bytes);
 #pragma unroll
-    for (int o = 0; o < NO; ++o) dst[o] = make_rsrc(prm.out[o] + m0 * (int64_t)T, wave_bytes);
+    for (int o = 0; o < NO + ND; ++o) dst[o] = make_rsrc(prm.out[o] + m0 * (int64_t)T, wave_bytes);
+
+    // stores the quad of every output (tile outputs y, then the derived one) at byte offset off
+    auto store_quads = [&](const float4 (&y)[NO], int off) {
+#pragma unroll
+        for (int o = 0; o < NO; ++o) buf_store4<STREAM>(dst[o], off, y[o]);
+        if constexpr (ND == 1) buf_store4<STREAM>(dst[NO], off, op.derive(y));
+    };
 
     // phase of a row: float index of its first sample modulo one 128-byte line
     const unsigned base_f = (unsigned)(reinterpret_cast<uintptr_t>(prm.in[0]) >> 2);
@@ -224,7 +242,7 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
 #pragma unroll
     for (int p = 0; p < G::kPasses; ++p)
 #pragma unroll
-        for (int o = 0; o < NO; ++o)   // distinct offsets, or the compiler merges them into one store
+        for (int o = 0; o < NO + ND; ++o)   // distinct offsets, or the compiler merges them into one store
             buf_store4<STREAM>(dst[o], kOutOfRange + 16 * p, make_float4(0.f, 0.f, 0.f, 0.f));
 
     for (int k = 0; k < nchunks; ++k) {
@@ -258,65 +276,61 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
         }
         __syncthreads();
 
-        // LDS -> global
-        if (interior) {
+        // LDS -> global.  On edge chunks the line shared by rows r and r+1 is completed before it is
+        // stored: in a forward pass the lanes that copy the last line of row r fill its slots past
+        // the end of the row with the head of row r+1, which they fetched from that row's tile in
+        // chunk 0; in a reverse pass the lanes that copy the first line of row r+1 fill its slots
+        // before the start of the row with the tail of row r, fetched in the chunk that held it.
+        // Either way the fetched quad waits in keep[][p] and leaves with the regular store of its
+        // lane, so every chunk issues the same number of stores.
 #pragma unroll
-            for (int p = 0; p < G::kPasses; ++p) {
-                const int r = p * G::kRowsPerPass + crow;
-                const int off = off0[p] + chunk * (TC * 4);
+        for (int p = 0; p < G::kPasses; ++p) {
+            const int r = p * G::kRowsPerPass + crow;
+            const int t = step0[p] + chunk * TC;
+            int off = off0[p] + chunk * (TC * 4);
+            float4 v[NO];
 #pragma unroll
-                for (int o = 0; o < NO; ++o)
-                    buf_store4<STREAM>(dst[o], off, *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]));
-            }
-        } else {
-            // edge chunk.  The line shared by rows r-1 and r is assembled by the eight lanes that
-            // copy the first line of row r: quads at or after the row's phase are its head, the
-            // others the tail of row r-1, fetched from that row's tile in the chunk that holds it.
-            // Whichever piece is produced first waits in keep[][p].
-            const bool tails_here = chunk >= interior_end;   // chunks that can hold a row's partial last line
-#pragma unroll
-            for (int p = 0; p < G::kPasses; ++p) {
-                const int r = p * G::kRowsPerPass + crow;
-                const int a = 4 * cq - step0[p];               // phase of row r
-                const int t = step0[p] + chunk * TC;
+            for (int o = 0; o < NO; ++o) v[o] = *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]);
+            if (!interior) {
+                const int a = 4 * cq - step0[p];                   // phase of row r
                 const bool valid = (unsigned)t < (unsigned)T;
-                int off = valid ? off0[p] + chunk * (TC * 4) : kOutOfRange;
-                const bool serves = route && r >= 1 && r < rows && a != 0 && cq < 8;   // lane holds quad cq of the shared line
-                const bool is_head = 4 * cq >= a;
-                const int tail_pos = (((a - T) & 31) + T) & ~31;   // window position of row r-1's partial last line
-                const int kp = tail_pos / TC;                      // chunk that holds it
-                const bool fetch_tail = serves && !is_head && chunk == kp;
-                const int tail_idx = fetch_tail ? (r - 1) * G::kPitch + (tail_pos - kp * TC) + 4 * cq : 0;
-                // quads of this row that another lane stores as part of an assembled line
-                const bool own_tail = route && valid && r + 1 < rows && 4 * cq + chunk * TC >= ((a + T) & ~31);
-                const bool own_head = serves && is_head && chunk == 0;
-                if (own_tail || (!Op::kReverse && own_head)) off = kOutOfRange;
-                if (Op::kReverse && serves && !is_head && chunk == 0) off = off0[p];
+                if (!valid) off = kOutOfRange;
+                const int a_next = (a + T) & 31;                   // phase of row r+1
+                const int tail_pos = (a + T) & ~31;                // window position of row r's partial last line
+                const int prev_tail_pos = (((a - T) & 31) + T) & ~31;   // the same for row r-1
+                // the pieces of a line shared with a neighbouring row of this wave
+                const bool own_head = route && r >= 1 && r < rows && a != 0 && cq < 8 && 4 * cq >= a;
+                const bool own_tail = route && valid && r + 1 < rows && 4 * cq + chunk * TC >= tail_pos;
+                bool fetch, release;
+                int idx;                                           // tile position of the quad to fetch
+                if (Op::kReverse) {
+                    // slot cq of row r's first line, before the row starts: tail of row r-1
+                    const bool slot = route && r >= 1 && r < rows && a != 0 && cq < 8 && 4 * cq < a;
+                    const int kp = prev_tail_pos / TC;
+                    fetch = slot && chunk == kp;
+                    release = slot && chunk == 0;
+                    idx = (r - 1) * G::kPitch + (prev_tail_pos - kp * TC) + 4 * cq;
+                    if (own_tail) off = kOutOfRange;               // stored by row r+1's lanes in chunk 0
+                } else {
+                    // slot j of row r's last line, past the end of the row: head of row r+1
+                    const int kt = tail_pos / TC;
+                    const int j = cq - (tail_pos - kt * TC) / 4;
+                    const bool slot = route && r + 1 < rows && a_next != 0 && j >= 0 && j < 8 && 4 * j >= a_next;
+                    fetch = slot && chunk == 0;
+                    release = slot && chunk == kt;
+                    idx = (r + 1) * G::kPitch + 4 * j;
+                    if (own_head && chunk == 0) off = kOutOfRange; // stored by row r-1's lanes with its tail
+                }
+                if (!fetch) idx = 0;
+                if (release) off = off0[p] + chunk * (TC * 4);
 #pragma unroll
                 for (int o = 0; o < NO; ++o) {
-                    float4 v = *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]);
-                    if (Op::kReverse) {
-                        // tails come first: fetch and hold them; chunk 0 stores head and held tail together
-                        if (tails_here) {
-                            const float4 tl = *reinterpret_cast<const float4*>(&tile[o][tail_idx]);
-                            if (fetch_tail) keep[o][p] = tl;
-                        }
-                        if (serves && !is_head && chunk == 0) v = keep[o][p];
-                    } else if (own_head) {
-                        keep[o][p] = v;                            // heads come first
-                    }
-                    buf_store4<STREAM>(dst[o], off, v);
-                }
-                if (!Op::kReverse && tails_here) {
-                    // the chunk with the tail of row r-1 stores it together with the held head of row r
-                    const int line_off = (serves && chunk == kp) ? off0[p] : kOutOfRange;
-#pragma unroll
-                    for (int o = 0; o < NO; ++o) {
-                        const float4 tl = *reinterpret_cast<const float4*>(&tile[o][tail_idx]);
-                        buf_store4<STREAM>(dst[o], line_off, is_head ? keep[o][p] : tl);
-                    }
+                    const float4 other = *reinterpret_cast<const float4*>(&tile[o][idx]);
+                    if (fetch) keep[o][p] = other;
+                    if (release) v[o] = keep[o][p];
                 }
             }
+            store_quads(v, off);
         }
         __syncthreads();
     }
@@ -331,7 +345,7 @@ template <class Op, int R>
 __global__ __launch_bounds__(kWave) void stream_kernel_scalar(typename Op::Params prm, int64_t M, int T) {
     using G = TileGeom<R>;
     constexpr int TC = G::kChunk;
-    constexpr int NI = Op::kIn, NO = Op::kOut, NT = NI > NO ? NI : NO;
+    constexpr int NI = Op::kIn, NO = Op::kOut, ND = DerivedCount<Op>::value, NT = NI > NO ? NI : NO;
     __shared__ __attribute__((aligned(16))) float tile[NT][G::kTileFloats];
 
     const int lane = threadIdx.x;
@@ -400,15 +414,23 @@ __global__ __launch_bounds__(kWave) void stream_kernel_scalar(typename Op::Param
         for (int p = 0; p < G::kPasses; ++p) {
             const int r = p * G::kRowsPerPass + crow;
             const int64_t off = (int64_t)(m0 + r) * (int64_t)T + (int64_t)t;
+            float4 v[NO + ND];
 #pragma unroll
-            for (int o = 0; o < NO; ++o) {
-                const float4 v = *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]);
+            for (int o = 0; o < NO; ++o) v[o] = *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]);
+            if constexpr (ND == 1) {
+                float4 y[NO];
+#pragma unroll
+                for (int o = 0; o < NO; ++o) y[o] = v[o];
+                v[NO] = op.derive(y);
+            }
+#pragma unroll
+            for (int o = 0; o < NO + ND; ++o) {
                 if (r < rows) {
                     float* d = prm.out[o] + off;
-                    if (t + 0 < T) d[0] = v.x;
-                    if (t + 1 < T) d[1] = v.y;
-                    if (t + 2 < T) d[2] = v.z;
-                    if (t + 3 < T) d[3] = v.w;
+                    if (t + 0 < T) d[0] = v[o].x;
+                    if (t + 1 < T) d[1] = v[o].y;
+                    if (t + 2 < T) d[2] = v[o].z;
+                    if (t + 3 < T) d[3] = v[o].w;
                 }
             }
         }
@@ -447,7 +469,7 @@ int launch_stream(const typename Op::Params& prm, int64_t M, int64_t T, hipStrea
     // the dwordx4 kernel addresses a wave's rows with 32-bit byte offsets: 64 * T * 4 must stay below 2^31
     bool vec = (T % 4) == 0 && T <= (1 << 22);
     for (int i = 0; i < Op::kIn; ++i) vec = vec && aligned16(prm.in[i]);
-    for (int o = 0; o < Op::kOut; ++o) vec = vec && aligned16(prm.out[o]);
+    for (int o = 0; o < Op::kOut + DerivedCount<Op>::value; ++o) vec = vec && aligned16(prm.out[o]);
     const bool streaming = M * T * 4 > ((int64_t)64 << 20);
     if (M < Op::kRows16Below) return launch_stream_rows<Op, 16>(prm, M, T, vec, streaming, stream);
     if constexpr (Op::kRows16Below < kAlways && Op::kRows16Below < Op::kRows32Below)
