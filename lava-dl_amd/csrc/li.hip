@@ -42,6 +42,7 @@ struct LiFwd {
 struct LiBwd {
     static constexpr int kIn = 2, kOut = 1;     // in: grad_out, saved forward output
     static constexpr bool kReverse = true;
+    static constexpr int kDuoRows = 32;          // light float recurrence: shorter rows per wave, longer segments
     static constexpr int64_t kRows32Below = kAlways, kRows16Below = kAlways;
     struct Params {
         const float* in[2];

@@ -57,6 +57,7 @@ struct DeltaFwd {
 struct DeltaBwd {
     static constexpr int kIn = 2, kOut = 1;          // in: grad of the events, saved delta;  out: grad_input
     static constexpr bool kReverse = true;
+    static constexpr int kDuoRows = 32;          // light float recurrence: shorter rows per wave, longer segments
     static constexpr int64_t kRows32Below = kAlways, kRows16Below = kAlways;
     struct Params {
         const float* in[2];
@@ -90,6 +91,7 @@ template <bool REVERSE>
 struct RunningSum {
     static constexpr int kIn = 1, kOut = 1;
     static constexpr bool kReverse = REVERSE;
+    static constexpr int kDuoRows = 32;          // light float recurrence: shorter rows per wave, longer segments
     static constexpr int64_t kRows32Below = kAlways, kRows16Below = kAlways;
     struct Params {
         const float* in[1];

@@ -136,72 +136,51 @@ __device__ __forceinline__ void buf_store4(__amdgpu_buffer_rsrc_t r, int byte_of
 //
 // Interior chunks (every column of every row inside [0, T), no shared line) run a branch-free
 // recurrence loop; only the first and the last one or two chunks take the predicated path.
+// Everything a wave needs to move the tiles of its R rows between global memory and LDS: buffer
+// descriptors, the per-pass copy pattern, the registers the next chunk is prefetched into and the
+// registers that hold boundary quads.
 template <class Op, int R, bool STREAM>
-__global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, int64_t M, int T) {
+struct Copier {
     using G = TileGeom<R>;
-    constexpr int TC = G::kChunk;
-    constexpr int NI = Op::kIn, NO = Op::kOut, ND = DerivedCount<Op>::value, NT = NI > NO ? NI : NO;
+    static constexpr int TC = G::kChunk, NI = Op::kIn, NO = Op::kOut, ND = DerivedCount<Op>::value;
     static_assert(ND == 0 || ND == 1, "at most one derived output");
-    __shared__ __attribute__((aligned(16))) float tile[NT][G::kTileFloats];
-
-    const int lane = threadIdx.x;
-    const int64_t m0 = (int64_t)blockIdx.x * R;
-    const int rows = (int)((M - m0) < R ? (M - m0) : R);
-
-    Op op;
-    op.init(prm, m0 + lane, lane < rows);
+    using Tiles = float (*)[G::kTileFloats];
 
     __amdgpu_buffer_rsrc_t src[NI], dst[NO + ND];
-    const unsigned wave_bytes = (unsigned)rows * (unsigned)T * 4u;
-#pragma unroll
-    for (int i = 0; i < NI; ++i) src[i] = make_rsrc(prm.in[i] + m0 * (int64_t)T, wave_bytes);
-#pragma unroll
-    for (int o = 0; o < NO + ND; ++o) dst[o] = make_rsrc(prm.out[o] + m0 * (int64_t)T, wave_bytes);
+    int step0[G::kPasses], off0[G::kPasses];    // step of this lane's quad in chunk 0, its byte offset in the wave's rows
+    float4 stage[NI][G::kPasses];               // prefetched inputs
+    float4 keep[NO][G::kPasses];                // first-produced pieces of shared lines, one quad per pass
+    int rows, T, crow, cq, interior_end;
+    bool route;
 
-    // stores the quad of every output (tile outputs y, then the derived one) at byte offset off
-    auto store_quads = [&](const float4 (&y)[NO], int off) {
+    __device__ __forceinline__ void init(const typename Op::Params& prm, int64_t m0, int rows_, int T_, int lane,
+                                         unsigned base_f) {
+        rows = rows_; T = T_;
+        const unsigned wave_bytes = (unsigned)rows * (unsigned)T * 4u;
 #pragma unroll
-        for (int o = 0; o < NO; ++o) buf_store4<STREAM>(dst[o], off, y[o]);
-        if constexpr (ND == 1) buf_store4<STREAM>(dst[NO], off, op.derive(y));
-    };
-
-    // phase of a row: float index of its first sample modulo one 128-byte line
-    const unsigned base_f = (unsigned)(reinterpret_cast<uintptr_t>(prm.in[0]) >> 2);
-    auto phase = [&](int r) -> int { return (int)((base_f + (unsigned)(m0 + r) * (unsigned)T) & 31u); };
-    const int a_lane = phase(lane);
-
-    int last = (lane < rows) ? (a_lane + T - 1) / TC : 0;    // last chunk this row needs
+        for (int i = 0; i < NI; ++i) src[i] = make_rsrc(prm.in[i] + m0 * (int64_t)T, wave_bytes);
 #pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-        const int o = __shfl_xor(last, d);
-        last = o > last ? o : last;
-    }
-    const int nchunks = last + 1;
-    // chunks [1, interior_end) hold only valid columns and touch no shared line, for every phase
-    const int interior_end = (T & ~31) / TC;
-    // rows shorter than a line could start and end inside the same line; they keep direct stores
-    const bool route = T >= 32;
-    float4 keep[NO][G::kPasses];            // first-produced pieces of shared lines, one quad per pass
+        for (int o = 0; o < NO + ND; ++o) dst[o] = make_rsrc(prm.out[o] + m0 * (int64_t)T, wave_bytes);
+        crow = lane / G::kQuads;                // row within a pass
+        cq = lane % G::kQuads;                  // quad within the row
+        // chunks [1, interior_end) hold only valid columns and touch no shared line, for every phase
+        interior_end = (T & ~31) / TC;
+        // rows shorter than a line could start and end inside the same line; they keep direct stores
+        route = T >= 32;
 #pragma unroll
-    for (int o = 0; o < NO; ++o)
+        for (int p = 0; p < G::kPasses; ++p) {
+            const int r = p * G::kRowsPerPass + crow;
+            step0[p] = 4 * cq - (int)((base_f + (unsigned)(m0 + r) * (unsigned)T) & 31u);
+            off0[p] = (r * T + step0[p]) * 4;
 #pragma unroll
-        for (int p = 0; p < G::kPasses; ++p) keep[o][p] = make_float4(0.f, 0.f, 0.f, 0.f);
-
-    const int crow = lane / G::kQuads;      // row within a pass (copy pattern)
-    const int cq = lane % G::kQuads;        // quad within the row
-
-    // copy pattern, per pass: step of this lane's quad in chunk 0 and its byte offset in the wave's rows
-    int step0[G::kPasses], off0[G::kPasses];
-#pragma unroll
-    for (int p = 0; p < G::kPasses; ++p) {
-        const int r = p * G::kRowsPerPass + crow;
-        step0[p] = 4 * cq - phase(r);
-        off0[p] = (r * T + step0[p]) * 4;
+            for (int o = 0; o < NO; ++o) keep[o][p] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
     }
 
-    float4 stage[NI][G::kPasses];
+    __device__ __forceinline__ bool interior(int chunk) const { return chunk >= 1 && chunk < interior_end; }
 
-    auto fetch = [&](int chunk) {
+    // global -> registers; past the last chunk every lane is out of range
+    __device__ __forceinline__ void fetch(int chunk) {
 #pragma unroll
         for (int p = 0; p < G::kPasses; ++p) {
             const bool ok = (unsigned)(step0[p] + chunk * TC) < (unsigned)T;
@@ -209,8 +188,113 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
 #pragma unroll
             for (int i = 0; i < NI; ++i) stage[i][p] = buf_load4<STREAM>(src[i], off);
         }
-    };
+    }
 
+    // registers -> LDS
+    __device__ __forceinline__ void stage_to_tiles(Tiles tile) const {
+#pragma unroll
+        for (int p = 0; p < G::kPasses; ++p) {
+            const int r = p * G::kRowsPerPass + crow;
+#pragma unroll
+            for (int i = 0; i < NI; ++i)
+                *reinterpret_cast<float4*>(&tile[i][r * G::kPitch + 4 * cq]) = stage[i][p];
+        }
+    }
+
+    // Stores that fall out of range (dropped by the hardware), as many as one chunk issues: the
+    // chunk loop is then entered in the same state its back edge leaves -- a chunk of loads
+    // followed by a chunk of stores in flight -- and the wait for the loads at the top of every
+    // iteration can leave the stores of the previous chunk in flight instead of draining them.
+    __device__ __forceinline__ void prime_stores() const {
+#pragma unroll
+        for (int p = 0; p < G::kPasses; ++p)
+#pragma unroll
+            for (int o = 0; o < NO + ND; ++o)   // distinct offsets, or the compiler merges them into one store
+                buf_store4<STREAM>(dst[o], kOutOfRange + 16 * p, make_float4(0.f, 0.f, 0.f, 0.f));
+    }
+
+    // LDS -> global.  On edge chunks the line shared by rows r and r+1 is completed before it is
+    // stored: in a forward pass the lanes that copy the last line of row r fill its slots past
+    // the end of the row with the head of row r+1, which they fetched from that row's tile in
+    // chunk 0; in a reverse pass the lanes that copy the first line of row r+1 fill its slots
+    // before the start of the row with the tail of row r, fetched in the chunk that held it.
+    // Either way the fetched quad waits in keep[][p] and leaves with the regular store of its
+    // lane, so every chunk issues the same number of stores.
+    __device__ __forceinline__ void copy_out(const Op& op, Tiles tile, int chunk) {
+        const bool inner = interior(chunk);
+#pragma unroll
+        for (int p = 0; p < G::kPasses; ++p) {
+            const int r = p * G::kRowsPerPass + crow;
+            const int t = step0[p] + chunk * TC;
+            int off = off0[p] + chunk * (TC * 4);
+            float4 v[NO];
+#pragma unroll
+            for (int o = 0; o < NO; ++o) v[o] = *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]);
+            if (!inner) {
+                const int a = 4 * cq - step0[p];                   // phase of row r
+                const bool valid = (unsigned)t < (unsigned)T;
+                if (!valid) off = kOutOfRange;
+                const int a_next = (a + T) & 31;                   // phase of row r+1
+                const int tail_pos = (a + T) & ~31;                // window position of row r's partial last line
+                const int prev_tail_pos = (((a - T) & 31) + T) & ~31;   // the same for row r-1
+                // the pieces of a line shared with a neighbouring row of this wave
+                const bool own_head = route && r >= 1 && r < rows && a != 0 && cq < 8 && 4 * cq >= a;
+                const bool own_tail = route && valid && r + 1 < rows && 4 * cq + chunk * TC >= tail_pos;
+                bool take, release;
+                int idx;                                           // tile position of the quad to take
+                if (Op::kReverse) {
+                    // slot cq of row r's first line, before the row starts: tail of row r-1
+                    const bool slot = route && r >= 1 && r < rows && a != 0 && cq < 8 && 4 * cq < a;
+                    const int kp = prev_tail_pos / TC;
+                    take = slot && chunk == kp;
+                    release = slot && chunk == 0;
+                    idx = (r - 1) * G::kPitch + (prev_tail_pos - kp * TC) + 4 * cq;
+                    if (own_tail) off = kOutOfRange;               // stored by row r+1's lanes in chunk 0
+                } else {
+                    // slot j of row r's last line, past the end of the row: head of row r+1
+                    const int kt = tail_pos / TC;
+                    const int j = cq - (tail_pos - kt * TC) / 4;
+                    const bool slot = route && r + 1 < rows && a_next != 0 && j >= 0 && j < 8 && 4 * j >= a_next;
+                    take = slot && chunk == 0;
+                    release = slot && chunk == kt;
+                    idx = (r + 1) * G::kPitch + 4 * j;
+                    if (own_head && chunk == 0) off = kOutOfRange; // stored by row r-1's lanes with its tail
+                }
+                if (!take) idx = 0;
+                if (release) off = off0[p] + chunk * (TC * 4);
+#pragma unroll
+                for (int o = 0; o < NO; ++o) {
+                    const float4 other = *reinterpret_cast<const float4*>(&tile[o][idx]);
+                    if (take) keep[o][p] = other;
+                    if (release) v[o] = keep[o][p];
+                }
+            }
+#pragma unroll
+            for (int o = 0; o < NO; ++o) buf_store4<STREAM>(dst[o], off, v[o]);
+            if constexpr (ND == 1) buf_store4<STREAM>(dst[NO], off, op.derive(v));
+        }
+    }
+};
+
+// Phase of a row (float index of its first sample modulo one 128-byte line) and the number of
+// chunks the wave's rows span, the same value in every lane.
+template <int TC>
+__device__ __forceinline__ int chunk_count(int a_lane, bool valid, int T) {
+    int last = valid ? (a_lane + T - 1) / TC : 0;    // last chunk this row needs
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const int o = __shfl_xor(last, d);
+        last = o > last ? o : last;
+    }
+    return last + 1;
+}
+
+// The sequential part: lane = neuron, one chunk of the tiles in place.
+template <class Op, int R>
+__device__ __forceinline__ void run_chunk(Op& op, float (*tile)[TileGeom<R>::kTileFloats], int lane, int chunk,
+                                          bool inner, int a_lane, int T) {
+    using G = TileGeom<R>;
+    constexpr int NI = Op::kIn, NO = Op::kOut;
     auto run_quad = [&](int qq) {
         float xin[NI][4], yout[NO][4];
 #pragma unroll
@@ -233,109 +317,107 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
             *reinterpret_cast<float4*>(&tile[o][lane * G::kPitch + 4 * qq]) =
                 make_float4(yout[o][0], yout[o][1], yout[o][2], yout[o][3]);
     };
+    if (inner) {
+        if (lane < R) {
+#pragma unroll 4
+            for (int q = 0; q < G::kQuads; ++q) run_quad(Op::kReverse ? G::kQuads - 1 - q : q);
+        }
+    } else {
+        const int tl = chunk * G::kChunk - a_lane;       // step held by column 0 of this lane's row
+        for (int q = 0; q < G::kQuads; ++q) {
+            const int qq = Op::kReverse ? G::kQuads - 1 - q : q;
+            if (lane < R && (unsigned)(tl + 4 * qq) < (unsigned)T) run_quad(qq);
+        }
+    }
+}
 
-    fetch(Op::kReverse ? nchunks - 1 : 0);
-    // Stores that fall out of range (dropped by the hardware), as many as one chunk issues: the
-    // loop is then entered in the same state its back edge leaves -- a chunk of loads followed by
-    // a chunk of stores in flight -- and the wait for the loads at the top of every iteration
-    // can leave the stores of the previous chunk in flight instead of draining them.
-#pragma unroll
-    for (int p = 0; p < G::kPasses; ++p)
-#pragma unroll
-        for (int o = 0; o < NO + ND; ++o)   // distinct offsets, or the compiler merges them into one store
-            buf_store4<STREAM>(dst[o], kOutOfRange + 16 * p, make_float4(0.f, 0.f, 0.f, 0.f));
+template <class Op, int R, bool STREAM>
+__global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, int64_t M, int T) {
+    using G = TileGeom<R>;
+    constexpr int TC = G::kChunk;
+    constexpr int NI = Op::kIn, NO = Op::kOut, NT = NI > NO ? NI : NO;
+    __shared__ __attribute__((aligned(16))) float tile[NT][G::kTileFloats];
+
+    const int lane = threadIdx.x;
+    const int64_t m0 = (int64_t)blockIdx.x * R;
+    const int rows = (int)((M - m0) < R ? (M - m0) : R);
+
+    Op op;
+    op.init(prm, m0 + lane, lane < rows);
+
+    const unsigned base_f = (unsigned)(reinterpret_cast<uintptr_t>(prm.in[0]) >> 2);
+    const int a_lane = (int)((base_f + (unsigned)(m0 + lane) * (unsigned)T) & 31u);
+    const int nchunks = chunk_count<TC>(a_lane, lane < rows, T);
+
+    Copier<Op, R, STREAM> io;
+    io.init(prm, m0, rows, T, lane, base_f);
+    io.fetch(Op::kReverse ? nchunks - 1 : 0);
+    io.prime_stores();
 
     for (int k = 0; k < nchunks; ++k) {
         const int chunk = Op::kReverse ? nchunks - 1 - k : k;
-        const bool interior = chunk >= 1 && chunk < interior_end;
-
-        // staged registers -> LDS
-#pragma unroll
-        for (int p = 0; p < G::kPasses; ++p) {
-            const int r = p * G::kRowsPerPass + crow;
-#pragma unroll
-            for (int i = 0; i < NI; ++i)
-                *reinterpret_cast<float4*>(&tile[i][r * G::kPitch + 4 * cq]) = stage[i][p];
-        }
+        io.stage_to_tiles(tile);
         __syncthreads();
-
-        fetch(Op::kReverse ? chunk - 1 : chunk + 1);    // past the last chunk every lane is out of range
-
-        // sequential recurrence: lane = neuron
-        if (interior) {
-            if (lane < R) {
-#pragma unroll 4
-                for (int q = 0; q < G::kQuads; ++q) run_quad(Op::kReverse ? G::kQuads - 1 - q : q);
-            }
-        } else {
-            const int tl = chunk * TC - a_lane;       // step held by column 0 of this lane's row
-            for (int q = 0; q < G::kQuads; ++q) {
-                const int qq = Op::kReverse ? G::kQuads - 1 - q : q;
-                if (lane < R && (unsigned)(tl + 4 * qq) < (unsigned)T) run_quad(qq);
-            }
-        }
+        io.fetch(Op::kReverse ? chunk - 1 : chunk + 1);
+        run_chunk<Op, R>(op, tile, lane, chunk, io.interior(chunk), a_lane, T);
         __syncthreads();
-
-        // LDS -> global.  On edge chunks the line shared by rows r and r+1 is completed before it is
-        // stored: in a forward pass the lanes that copy the last line of row r fill its slots past
-        // the end of the row with the head of row r+1, which they fetched from that row's tile in
-        // chunk 0; in a reverse pass the lanes that copy the first line of row r+1 fill its slots
-        // before the start of the row with the tail of row r, fetched in the chunk that held it.
-        // Either way the fetched quad waits in keep[][p] and leaves with the regular store of its
-        // lane, so every chunk issues the same number of stores.
-#pragma unroll
-        for (int p = 0; p < G::kPasses; ++p) {
-            const int r = p * G::kRowsPerPass + crow;
-            const int t = step0[p] + chunk * TC;
-            int off = off0[p] + chunk * (TC * 4);
-            float4 v[NO];
-#pragma unroll
-            for (int o = 0; o < NO; ++o) v[o] = *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]);
-            if (!interior) {
-                const int a = 4 * cq - step0[p];                   // phase of row r
-                const bool valid = (unsigned)t < (unsigned)T;
-                if (!valid) off = kOutOfRange;
-                const int a_next = (a + T) & 31;                   // phase of row r+1
-                const int tail_pos = (a + T) & ~31;                // window position of row r's partial last line
-                const int prev_tail_pos = (((a - T) & 31) + T) & ~31;   // the same for row r-1
-                // the pieces of a line shared with a neighbouring row of this wave
-                const bool own_head = route && r >= 1 && r < rows && a != 0 && cq < 8 && 4 * cq >= a;
-                const bool own_tail = route && valid && r + 1 < rows && 4 * cq + chunk * TC >= tail_pos;
-                bool fetch, release;
-                int idx;                                           // tile position of the quad to fetch
-                if (Op::kReverse) {
-                    // slot cq of row r's first line, before the row starts: tail of row r-1
-                    const bool slot = route && r >= 1 && r < rows && a != 0 && cq < 8 && 4 * cq < a;
-                    const int kp = prev_tail_pos / TC;
-                    fetch = slot && chunk == kp;
-                    release = slot && chunk == 0;
-                    idx = (r - 1) * G::kPitch + (prev_tail_pos - kp * TC) + 4 * cq;
-                    if (own_tail) off = kOutOfRange;               // stored by row r+1's lanes in chunk 0
-                } else {
-                    // slot j of row r's last line, past the end of the row: head of row r+1
-                    const int kt = tail_pos / TC;
-                    const int j = cq - (tail_pos - kt * TC) / 4;
-                    const bool slot = route && r + 1 < rows && a_next != 0 && j >= 0 && j < 8 && 4 * j >= a_next;
-                    fetch = slot && chunk == 0;
-                    release = slot && chunk == kt;
-                    idx = (r + 1) * G::kPitch + 4 * j;
-                    if (own_head && chunk == 0) off = kOutOfRange; // stored by row r-1's lanes with its tail
-                }
-                if (!fetch) idx = 0;
-                if (release) off = off0[p] + chunk * (TC * 4);
-#pragma unroll
-                for (int o = 0; o < NO; ++o) {
-                    const float4 other = *reinterpret_cast<const float4*>(&tile[o][idx]);
-                    if (fetch) keep[o][p] = other;
-                    if (release) v[o] = keep[o][p];
-                }
-            }
-            store_quads(v, off);
-        }
+        io.copy_out(op, tile, chunk);
         __syncthreads();
     }
-
     op.finish(prm, m0 + lane, lane < rows);
+}
+
+// Two-wave variant for problems too small to fill the machine with one wave per R rows.  There the
+// run time is the number of steps times the latency of one step of the sequential wave, so that
+// wave does nothing else: wave 0 runs the recurrence chunk after chunk, wave 1 moves the tiles
+// (prefetch, LDS fill, boundary lines, stores) through a second set of tiles, one barrier per chunk.
+//   barrier j: chunk j is in tiles[j & 1] and the recurrence of chunk j-1 is done.
+template <class Op, int R, bool STREAM>
+__global__ __launch_bounds__(2 * kWave) void stream_kernel_duo(typename Op::Params prm, int64_t M, int T) {
+    using G = TileGeom<R>;
+    constexpr int TC = G::kChunk;
+    constexpr int NI = Op::kIn, NO = Op::kOut, NT = NI > NO ? NI : NO;
+    __shared__ __attribute__((aligned(16))) float tiles[2][NT][G::kTileFloats];
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int role = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));   // wave-uniform
+    const int64_t m0 = (int64_t)blockIdx.x * R;
+    const int rows = (int)((M - m0) < R ? (M - m0) : R);
+    const unsigned base_f = (unsigned)(reinterpret_cast<uintptr_t>(prm.in[0]) >> 2);
+    const int a_lane = (int)((base_f + (unsigned)(m0 + lane) * (unsigned)T) & 31u);
+    const int nchunks = chunk_count<TC>(a_lane, lane < rows, T);
+    const int interior_end = (T & ~31) / TC;
+
+    if (role == 0) {
+        Op op;
+        op.init(prm, m0 + lane, lane < rows);
+        for (int k = 0; k < nchunks; ++k) {
+            const int chunk = Op::kReverse ? nchunks - 1 - k : k;
+            __syncthreads();                                   // barrier k
+            run_chunk<Op, R>(op, tiles[k & 1], lane, chunk, chunk >= 1 && chunk < interior_end, a_lane, T);
+        }
+        __syncthreads();                                       // barrier nchunks
+        op.finish(prm, m0 + lane, lane < rows);
+    } else {
+        Op uni;                                                // wave-uniform members only (derive)
+        uni.init(prm, 0, false);
+        Copier<Op, R, STREAM> io;
+        io.init(prm, m0, rows, T, lane, base_f);
+        auto chunk_of = [&](int k) { return Op::kReverse ? nchunks - 1 - k : k; };
+        io.fetch(chunk_of(0));
+        io.prime_stores();
+        io.stage_to_tiles(tiles[0]);
+        io.fetch(chunk_of(1));
+        __syncthreads();                                       // barrier 0
+        for (int k = 0; k < nchunks; ++k) {
+            // wave 0 works on tiles[k & 1]; the other set still holds the results of chunk k-1
+            io.copy_out(uni, tiles[(k + 1) & 1], chunk_of(k - 1));   // k == 0: no such chunk, every store falls out of range
+            io.stage_to_tiles(tiles[(k + 1) & 1]);             // chunk k+1 (zeros past the end)
+            io.fetch(chunk_of(k + 2));
+            __syncthreads();                                   // barrier k+1
+        }
+        io.copy_out(uni, tiles[(nchunks - 1) & 1], chunk_of(nchunks - 1));
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -441,9 +523,37 @@ __global__ __launch_bounds__(kWave) void stream_kernel_scalar(typename Op::Param
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// Launch helper: picks the dwordx4 path when T and every pointer allow it, non-temporal global
-// accesses when the tensors are too large to be reused out of the last-level cache, and the
-// rows-per-wave geometry from the number of neurons.
+constexpr int64_t kAlways = (int64_t)1 << 62;
+
+// Rows per workgroup of the two-wave kernel: 64 unless the Op says otherwise (kDuoRows).
+template <class Op, class = void>
+struct DuoRows { static constexpr int value = 64; };
+template <class Op>
+struct DuoRows<Op, decltype((void)Op::kDuoRows)> { static constexpr int value = Op::kDuoRows; };
+
+// Two-wave workgroups of this kernel that one compute unit holds at a time (LDS and registers).
+template <class Op, int R, bool STREAM>
+int duo_groups_per_cu() {
+    static const int n = [] {
+        int v = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&v, stream_kernel_duo<Op, R, STREAM>, 2 * kWave, 0) != hipSuccess)
+            v = 0;
+        return v;
+    }();
+    return n;
+}
+
+inline int compute_units() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess) cached[dev] = n;
+    }
+    return cached[dev];
+}
+
 template <class Op, int R>
 int launch_stream_rows(const typename Op::Params& prm, int64_t M, int64_t T, bool vec, bool streaming,
                        hipStream_t stream) {
@@ -457,20 +567,36 @@ int launch_stream_rows(const typename Op::Params& prm, int64_t M, int64_t T, boo
     return (int)hipGetLastError();
 }
 
-// Rows per wave.  An Op states below how many neurons it wants 32 and 16 rows per wave
-// (kRows32Below, kRows16Below; measured on MI355X): arithmetic-heavy forward recurrences keep all
-// 64 lanes busy until the problem gets small, the light float backward passes prefer 16 rows
-// and 512-byte row segments at every size.
-constexpr int64_t kAlways = (int64_t)1 << 62;
-
+// Launch policy (thresholds measured on MI355X).
+//  * dwordx4 path when T and every pointer allow it, else the dword fallback;
+//  * non-temporal global accesses when the tensors are too large to be reused out of the
+//    last-level cache;
+//  * while every workgroup of the two-wave kernel is resident at once, run time is set by the
+//    latency of the sequential wave and that kernel is 10-40% faster (all 64 lanes hold a row);
+//  * beyond that the one-wave kernel, with the rows per wave the Op asks for (kRows32Below,
+//    kRows16Below): integer forward recurrences and backward passes with an exp per step keep all
+//    64 lanes busy, the light float backward passes prefer 16 rows and 512-byte row segments.
 template <class Op>
 int launch_stream(const typename Op::Params& prm, int64_t M, int64_t T, hipStream_t stream) {
     if (M == 0 || T == 0) return 0;
-    // the dwordx4 kernel addresses a wave's rows with 32-bit byte offsets: 64 * T * 4 must stay below 2^31
+    // the dwordx4 kernels address a wave's rows with 32-bit byte offsets: 64 * T * 4 must stay below 2^31
     bool vec = (T % 4) == 0 && T <= (1 << 22);
     for (int i = 0; i < Op::kIn; ++i) vec = vec && aligned16(prm.in[i]);
     for (int o = 0; o < Op::kOut + DerivedCount<Op>::value; ++o) vec = vec && aligned16(prm.out[o]);
     const bool streaming = M * T * 4 > ((int64_t)64 << 20);
+    if (vec) {
+        constexpr int RD = DuoRows<Op>::value;
+        const int64_t groups = (M + RD - 1) / RD;
+        const int per_cu = streaming ? duo_groups_per_cu<Op, RD, true>() : duo_groups_per_cu<Op, RD, false>();
+        if (groups <= (int64_t)per_cu * compute_units()) {
+            const dim3 grid((unsigned)groups), block(2 * kWave);
+            if (streaming)
+                hipLaunchKernelGGL((stream_kernel_duo<Op, RD, true>), grid, block, 0, stream, prm, M, (int)T);
+            else
+                hipLaunchKernelGGL((stream_kernel_duo<Op, RD, false>), grid, block, 0, stream, prm, M, (int)T);
+            return (int)hipGetLastError();
+        }
+    }
     if (M < Op::kRows16Below) return launch_stream_rows<Op, 16>(prm, M, T, vec, streaming, stream);
     if constexpr (Op::kRows16Below < kAlways && Op::kRows16Below < Op::kRows32Below)
         if (M < Op::kRows32Below) return launch_stream_rows<Op, 32>(prm, M, T, vec, streaming, stream);
