@@ -15,25 +15,40 @@ struct LiFwd {
         float* out[1];
         const float* decay;
         const float* state;
-        float w, inv_w, thr;          // thr = +inf when the reset is disabled
+        float w, inv_w;
+        int fire_above;               // reset when the state exceeds this (INT_MAX: reset disabled)
         int64_t npb, num_decays, num_states;
     };
-    int y, mult;
-    float w, inv_w, thr;
+    // The tiles hold integers (bit patterns in float registers): the input is scaled and truncated
+    // on its way into LDS, the state is converted and scaled back on its way out, and the
+    // sequential loop is left with the recurrence alone.
+    static constexpr bool kTransforms = true;
+    int y, mult, fire_above;
+    float w, inv_w;
 
     __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
-        w = p.w; inv_w = p.inv_w; thr = p.thr;
+        w = p.w; inv_w = p.inv_w; fire_above = p.fire_above;
         y = 0; mult = 0;
         if (valid) {
             y = trunc_i32(p.state[p.num_states == 1 ? 0 : m] * w);
             mult = 4096 - trunc_i32(p.decay[param_index(m, p.npb, p.num_decays)]);
         }
     }
+    __device__ __forceinline__ float to_state(float x) const { return __int_as_float(trunc_i32(w * x)); }
+    __device__ __forceinline__ float from_state(float s) const {
+        const float yf = (float)__float_as_int(s);
+        return POW2 ? yf * inv_w : yf / w;
+    }
+    __device__ __forceinline__ void pre(float4 (&x)[1]) const {
+        x[0] = make_float4(to_state(x[0].x), to_state(x[0].y), to_state(x[0].z), to_state(x[0].w));
+    }
+    __device__ __forceinline__ void post(float4 (&o)[1]) const {
+        o[0] = make_float4(from_state(o[0].x), from_state(o[0].y), from_state(o[0].z), from_state(o[0].w));
+    }
     __device__ __forceinline__ void step(const float (&x)[1], float (&o)[1]) {
-        const int yn = rs0_12(y, mult) + trunc_i32(w * x[0]);
-        const float yf = (float)yn;
-        o[0] = POW2 ? yf * inv_w : yf / w;
-        y = (yf >= thr) ? 0 : yn;
+        const int yn = rs0_12(y, mult) + __float_as_int(x[0]);
+        o[0] = __int_as_float(yn);
+        y = (yn > fire_above) ? 0 : yn;              // (float)yn >= threshold, decided on the integer
     }
     __device__ __forceinline__ void finish(const Params&, int64_t, bool) {}
 };
@@ -156,12 +171,12 @@ extern "C" int slayer_li_fwd(float* out, const float* in, const float* decay, co
     if (int e = check_states(M, num_states)) return e;
     if (w_scale == 0) return SLAYER_EINVAL;
     const float w = (float)w_scale;
-    const float thr = thr_scaled > 0 ? (float)thr_scaled : __builtin_inff();
+    const int fa = fire_above(thr_scaled > 0 ? (float)thr_scaled : __builtin_inff());
     if (is_pow2(w_scale)) {
-        LiFwd<true>::Params p{{in}, {out}, decay, state, w, 1.0f / w, thr, neurons_per_batch, num_decays, num_states};
+        LiFwd<true>::Params p{{in}, {out}, decay, state, w, 1.0f / w, fa, neurons_per_batch, num_decays, num_states};
         return launch_stream<LiFwd<true>>(p, M, T, (hipStream_t)stream);
     }
-    LiFwd<false>::Params p{{in}, {out}, decay, state, w, 1.0f / w, thr, neurons_per_batch, num_decays, num_states};
+    LiFwd<false>::Params p{{in}, {out}, decay, state, w, 1.0f / w, fa, neurons_per_batch, num_decays, num_states};
     return launch_stream<LiFwd<false>>(p, M, T, (hipStream_t)stream);
 }
 

@@ -30,6 +30,18 @@ __device__ __forceinline__ int rs0_12(int a, int b) {
     return (int)(((long long)a * (long long)b + bias) >> 12);
 }
 
+// Largest integer y whose float32 conversion is below thr: (float)y >= thr  <=>  y > fire_above(thr),
+// so a recurrence can take its reset decision on the integer state.  INT_MAX (never fires) for
+// thresholds beyond the int range, NaN or +inf.
+inline int fire_above(float thr) {
+    if (!(thr <= 2147483648.0f)) return 0x7fffffff;
+    if (thr <= -2147483648.0f) return (int)0x80000000;     // every state fires except the most negative one
+    long long c = (long long)__builtin_ceil((double)thr);   // candidate for the smallest firing state
+    while (c > -2147483648LL && (float)(c - 1) >= thr) --c;
+    while (c <= 2147483647LL && (float)c < thr) ++c;
+    return (int)(c - 1);
+}
+
 // Streaming (non-temporal) 16-byte global accesses: tensors on this path are read once and
 // written once, so they should not displace each other in L2.
 typedef float vf4 __attribute__((ext_vector_type(4)));
@@ -76,6 +88,12 @@ struct TileGeom {
 
 // An Op provides:
 //   static constexpr int kIn, kOut;  static constexpr bool kReverse;
+//   optionally static constexpr bool kTransforms = true and
+//     __device__ void pre(float4 (&x)[kIn]) const;  __device__ void post(float4 (&y)[kOut]) const;
+//     elementwise maps (wave-uniform members only) applied to the input quads on their way into LDS
+//     and to the output quads on their way out, so that work that does not belong to the
+//     sequential dependency chain (scaling, int <-> float conversion) is done by all 64 lanes in
+//     the copy phases, or by the copy wave of the two-wave kernel;
 //   optionally static constexpr int kDerived = 1 and
 //     __device__ float4 derive(const float4 (&y)[kOut]) const;   (uses wave-uniform members only)
 //     an extra output, Params::out[kOut], that is an elementwise function of the other outputs of
@@ -86,6 +104,11 @@ struct TileGeom {
 //   __device__ void init(const Params&, int64_t m, bool valid);
 //   __device__ void step(const float (&x)[kIn], float (&y)[kOut]);
 //   __device__ void finish(const Params&, int64_t m, bool valid);
+
+template <class Op, class = void>
+struct HasTransforms { static constexpr bool value = false; };
+template <class Op>
+struct HasTransforms<Op, decltype((void)Op::kTransforms)> { static constexpr bool value = Op::kTransforms; };
 
 template <class Op, class = void>
 struct DerivedCount { static constexpr int value = 0; };
@@ -139,23 +162,27 @@ __device__ __forceinline__ void buf_store4(__amdgpu_buffer_rsrc_t r, int byte_of
 // Everything a wave needs to move the tiles of its R rows between global memory and LDS: buffer
 // descriptors, the per-pass copy pattern, the registers the next chunk is prefetched into and the
 // registers that hold boundary quads.
-template <class Op, int R, bool STREAM>
+//
+// A wave can share the job with others: it then owns PASSES of the G::kPasses wave-wide accesses
+// that cover a tile, starting at pass first_pass.
+template <class Op, int R, bool STREAM, int PASSES = TileGeom<R>::kPasses>
 struct Copier {
     using G = TileGeom<R>;
     static constexpr int TC = G::kChunk, NI = Op::kIn, NO = Op::kOut, ND = DerivedCount<Op>::value;
+    static constexpr int kPasses = PASSES;
     static_assert(ND == 0 || ND == 1, "at most one derived output");
     using Tiles = float (*)[G::kTileFloats];
 
     __amdgpu_buffer_rsrc_t src[NI], dst[NO + ND];
-    int step0[G::kPasses], off0[G::kPasses];    // step of this lane's quad in chunk 0, its byte offset in the wave's rows
-    float4 stage[NI][G::kPasses];               // prefetched inputs
-    float4 keep[NO][G::kPasses];                // first-produced pieces of shared lines, one quad per pass
-    int rows, T, crow, cq, interior_end;
+    int step0[kPasses], off0[kPasses];    // step of this lane's quad in chunk 0, its byte offset in the wave's rows
+    float4 stage[NI][kPasses];               // prefetched inputs
+    float4 keep[NO][kPasses];                // first-produced pieces of shared lines, one quad per pass
+    int rows, T, crow, cq, interior_end, first_pass;
     bool route;
 
     __device__ __forceinline__ void init(const typename Op::Params& prm, int64_t m0, int rows_, int T_, int lane,
-                                         unsigned base_f) {
-        rows = rows_; T = T_;
+                                         unsigned base_f, int first_pass_ = 0) {
+        rows = rows_; T = T_; first_pass = first_pass_;
         const unsigned wave_bytes = (unsigned)rows * (unsigned)T * 4u;
 #pragma unroll
         for (int i = 0; i < NI; ++i) src[i] = make_rsrc(prm.in[i] + m0 * (int64_t)T, wave_bytes);
@@ -168,8 +195,8 @@ struct Copier {
         // rows shorter than a line could start and end inside the same line; they keep direct stores
         route = T >= 32;
 #pragma unroll
-        for (int p = 0; p < G::kPasses; ++p) {
-            const int r = p * G::kRowsPerPass + crow;
+        for (int p = 0; p < kPasses; ++p) {
+            const int r = (first_pass + p) * G::kRowsPerPass + crow;
             step0[p] = 4 * cq - (int)((base_f + (unsigned)(m0 + r) * (unsigned)T) & 31u);
             off0[p] = (r * T + step0[p]) * 4;
 #pragma unroll
@@ -179,25 +206,30 @@ struct Copier {
 
     __device__ __forceinline__ bool interior(int chunk) const { return chunk >= 1 && chunk < interior_end; }
 
-    // global -> registers; past the last chunk every lane is out of range
-    __device__ __forceinline__ void fetch(int chunk) {
+    // global -> registers; past the last chunk (or before the first) every lane is out of range
+    __device__ __forceinline__ void fetch_into(float4 (&buf)[NI][kPasses], int chunk) const {
 #pragma unroll
-        for (int p = 0; p < G::kPasses; ++p) {
+        for (int p = 0; p < kPasses; ++p) {
             const bool ok = (unsigned)(step0[p] + chunk * TC) < (unsigned)T;
             const int off = ok ? off0[p] + chunk * (TC * 4) : kOutOfRange;
 #pragma unroll
-            for (int i = 0; i < NI; ++i) stage[i][p] = buf_load4<STREAM>(src[i], off);
+            for (int i = 0; i < NI; ++i) buf[i][p] = buf_load4<STREAM>(src[i], off);
         }
     }
+    __device__ __forceinline__ void fetch(int chunk) { fetch_into(stage, chunk); }
 
     // registers -> LDS
-    __device__ __forceinline__ void stage_to_tiles(Tiles tile) const {
+    __device__ __forceinline__ void stage_to_tiles(const Op& op, Tiles tile) const { to_tiles(op, tile, stage); }
+    __device__ __forceinline__ void to_tiles(const Op& op, Tiles tile, const float4 (&buf)[NI][kPasses]) const {
 #pragma unroll
-        for (int p = 0; p < G::kPasses; ++p) {
-            const int r = p * G::kRowsPerPass + crow;
+        for (int p = 0; p < kPasses; ++p) {
+            const int r = (first_pass + p) * G::kRowsPerPass + crow;
+            float4 x[NI];
 #pragma unroll
-            for (int i = 0; i < NI; ++i)
-                *reinterpret_cast<float4*>(&tile[i][r * G::kPitch + 4 * cq]) = stage[i][p];
+            for (int i = 0; i < NI; ++i) x[i] = buf[i][p];
+            if constexpr (HasTransforms<Op>::value) op.pre(x);
+#pragma unroll
+            for (int i = 0; i < NI; ++i) *reinterpret_cast<float4*>(&tile[i][r * G::kPitch + 4 * cq]) = x[i];
         }
     }
 
@@ -207,7 +239,7 @@ struct Copier {
     // iteration can leave the stores of the previous chunk in flight instead of draining them.
     __device__ __forceinline__ void prime_stores() const {
 #pragma unroll
-        for (int p = 0; p < G::kPasses; ++p)
+        for (int p = 0; p < kPasses; ++p)
 #pragma unroll
             for (int o = 0; o < NO + ND; ++o)   // distinct offsets, or the compiler merges them into one store
                 buf_store4<STREAM>(dst[o], kOutOfRange + 16 * p, make_float4(0.f, 0.f, 0.f, 0.f));
@@ -223,8 +255,8 @@ struct Copier {
     __device__ __forceinline__ void copy_out(const Op& op, Tiles tile, int chunk) {
         const bool inner = interior(chunk);
 #pragma unroll
-        for (int p = 0; p < G::kPasses; ++p) {
-            const int r = p * G::kRowsPerPass + crow;
+        for (int p = 0; p < kPasses; ++p) {
+            const int r = (first_pass + p) * G::kRowsPerPass + crow;
             const int t = step0[p] + chunk * TC;
             int off = off0[p] + chunk * (TC * 4);
             float4 v[NO];
@@ -269,6 +301,7 @@ struct Copier {
                     if (release) v[o] = keep[o][p];
                 }
             }
+            if constexpr (HasTransforms<Op>::value) op.post(v);
 #pragma unroll
             for (int o = 0; o < NO; ++o) buf_store4<STREAM>(dst[o], off, v[o]);
             if constexpr (ND == 1) buf_store4<STREAM>(dst[NO], off, op.derive(v));
@@ -290,7 +323,7 @@ __device__ __forceinline__ int chunk_count(int a_lane, bool valid, int T) {
 }
 
 // The sequential part: lane = neuron, one chunk of the tiles in place.
-template <class Op, int R>
+template <class Op, int R, int UNROLL>
 __device__ __forceinline__ void run_chunk(Op& op, float (*tile)[TileGeom<R>::kTileFloats], int lane, int chunk,
                                           bool inner, int a_lane, int T) {
     using G = TileGeom<R>;
@@ -319,7 +352,7 @@ __device__ __forceinline__ void run_chunk(Op& op, float (*tile)[TileGeom<R>::kTi
     };
     if (inner) {
         if (lane < R) {
-#pragma unroll 4
+#pragma unroll UNROLL
             for (int q = 0; q < G::kQuads; ++q) run_quad(Op::kReverse ? G::kQuads - 1 - q : q);
         }
     } else {
@@ -356,10 +389,10 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
 
     for (int k = 0; k < nchunks; ++k) {
         const int chunk = Op::kReverse ? nchunks - 1 - k : k;
-        io.stage_to_tiles(tile);
+        io.stage_to_tiles(op, tile);
         __syncthreads();
         io.fetch(Op::kReverse ? chunk - 1 : chunk + 1);
-        run_chunk<Op, R>(op, tile, lane, chunk, io.interior(chunk), a_lane, T);
+        run_chunk<Op, R, 4>(op, tile, lane, chunk, io.interior(chunk), a_lane, T);
         __syncthreads();
         io.copy_out(op, tile, chunk);
         __syncthreads();
@@ -367,16 +400,22 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
     op.finish(prm, m0 + lane, lane < rows);
 }
 
-// Two-wave variant for problems too small to fill the machine with one wave per R rows.  There the
-// run time is the number of steps times the latency of one step of the sequential wave, so that
-// wave does nothing else: wave 0 runs the recurrence chunk after chunk, wave 1 moves the tiles
-// (prefetch, LDS fill, boundary lines, stores) through a second set of tiles, one barrier per chunk.
+// Variant for problems too small to fill the machine with one wave per R rows.  There the run
+// time is the number of steps times the latency of one step of the sequential wave, so that wave
+// does nothing else: wave 0 runs the recurrence chunk after chunk, NCOPY more waves move the tiles
+// (prefetch, LDS fill, boundary lines, stores) through a second set of tiles, each owning an equal
+// share of the wave-wide accesses that cover a tile; one barrier per chunk.
 //   barrier j: chunk j is in tiles[j & 1] and the recurrence of chunk j-1 is done.
-template <class Op, int R, bool STREAM>
-__global__ __launch_bounds__(2 * kWave) void stream_kernel_duo(typename Op::Params prm, int64_t M, int T) {
+// A chunk is a few hundred nanoseconds of recurrence, less than a trip to memory, so the copy
+// waves keep the loads of two chunks in flight (chunk j waits in fetched[j & 1]).  All waves run
+// an even number of chunks; a surplus chunk lies outside every row and neither computes nor stores.
+template <class Op, int R, bool STREAM, int NCOPY>
+__global__ __launch_bounds__((1 + NCOPY) * kWave) void stream_kernel_duo(typename Op::Params prm, int64_t M, int T) {
     using G = TileGeom<R>;
     constexpr int TC = G::kChunk;
     constexpr int NI = Op::kIn, NO = Op::kOut, NT = NI > NO ? NI : NO;
+    constexpr int PASSES = G::kPasses / NCOPY;
+    static_assert(PASSES * NCOPY == G::kPasses, "copy waves share the passes evenly");
     __shared__ __attribute__((aligned(16))) float tiles[2][NT][G::kTileFloats];
 
     const int lane = threadIdx.x & (kWave - 1);
@@ -386,37 +425,46 @@ __global__ __launch_bounds__(2 * kWave) void stream_kernel_duo(typename Op::Para
     const unsigned base_f = (unsigned)(reinterpret_cast<uintptr_t>(prm.in[0]) >> 2);
     const int a_lane = (int)((base_f + (unsigned)(m0 + lane) * (unsigned)T) & 31u);
     const int nchunks = chunk_count<TC>(a_lane, lane < rows, T);
+    const int nloop = (nchunks + 1) & ~1;
     const int interior_end = (T & ~31) / TC;
+    // k-th chunk in processing order; values outside [0, nchunks) name no chunk
+    auto chunk_of = [&](int k) { return Op::kReverse ? nchunks - 1 - k : k; };
 
     if (role == 0) {
         Op op;
         op.init(prm, m0 + lane, lane < rows);
-        for (int k = 0; k < nchunks; ++k) {
-            const int chunk = Op::kReverse ? nchunks - 1 - k : k;
+        for (int k = 0; k < nloop; ++k) {
+            const int chunk = chunk_of(k);
             __syncthreads();                                   // barrier k
-            run_chunk<Op, R>(op, tiles[k & 1], lane, chunk, chunk >= 1 && chunk < interior_end, a_lane, T);
+            if (k < nchunks)
+                run_chunk<Op, R, 4>(op, tiles[k & 1], lane, chunk, chunk >= 1 && chunk < interior_end, a_lane, T);
         }
-        __syncthreads();                                       // barrier nchunks
+        __syncthreads();                                       // barrier nloop
         op.finish(prm, m0 + lane, lane < rows);
     } else {
-        Op uni;                                                // wave-uniform members only (derive)
+        Op uni;                                                // wave-uniform members only (pre, post, derive)
         uni.init(prm, 0, false);
-        Copier<Op, R, STREAM> io;
-        io.init(prm, m0, rows, T, lane, base_f);
-        auto chunk_of = [&](int k) { return Op::kReverse ? nchunks - 1 - k : k; };
-        io.fetch(chunk_of(0));
+        Copier<Op, R, STREAM, PASSES> io;
+        io.init(prm, m0, rows, T, lane, base_f, (role - 1) * PASSES);
+        float4 fetched[2][NI][PASSES];
+        io.fetch_into(fetched[0], chunk_of(0));
+        io.fetch_into(fetched[1], chunk_of(1));
         io.prime_stores();
-        io.stage_to_tiles(tiles[0]);
-        io.fetch(chunk_of(1));
+        io.to_tiles(uni, tiles[0], fetched[0]);
+        io.fetch_into(fetched[0], chunk_of(2));
         __syncthreads();                                       // barrier 0
-        for (int k = 0; k < nchunks; ++k) {
-            // wave 0 works on tiles[k & 1]; the other set still holds the results of chunk k-1
-            io.copy_out(uni, tiles[(k + 1) & 1], chunk_of(k - 1));   // k == 0: no such chunk, every store falls out of range
-            io.stage_to_tiles(tiles[(k + 1) & 1]);             // chunk k+1 (zeros past the end)
-            io.fetch(chunk_of(k + 2));
+        for (int k = 0; k < nloop; k += 2) {
+            // wave 0 works on tiles[0] (chunk k); tiles[1] still holds the results of chunk k-1
+            io.copy_out(uni, tiles[1], chunk_of(k - 1));
+            io.to_tiles(uni, tiles[1], fetched[1]);            // chunk k+1
+            io.fetch_into(fetched[1], chunk_of(k + 3));
             __syncthreads();                                   // barrier k+1
+            io.copy_out(uni, tiles[0], chunk_of(k));
+            io.to_tiles(uni, tiles[0], fetched[0]);            // chunk k+2
+            io.fetch_into(fetched[0], chunk_of(k + 4));
+            __syncthreads();                                   // barrier k+2
         }
-        io.copy_out(uni, tiles[(nchunks - 1) & 1], chunk_of(nchunks - 1));
+        io.copy_out(uni, tiles[1], chunk_of(nloop - 1));
     }
 }
 
@@ -448,6 +496,7 @@ __global__ __launch_bounds__(kWave) void stream_kernel_scalar(typename Op::Param
         for (int p = 0; p < G::kPasses; ++p) {
             const int r = p * G::kRowsPerPass + crow;
             const int64_t off = (int64_t)(m0 + r) * (int64_t)T + (int64_t)t;
+            float4 x[NI];
 #pragma unroll
             for (int i = 0; i < NI; ++i) {
                 float4 v = make_float4(0.f, 0.f, 0.f, 0.f);      // zero fill: steps past T-1 must be no-ops
@@ -458,8 +507,11 @@ __global__ __launch_bounds__(kWave) void stream_kernel_scalar(typename Op::Param
                     if (t + 2 < T) v.z = src[2];
                     if (t + 3 < T) v.w = src[3];
                 }
-                *reinterpret_cast<float4*>(&tile[i][r * G::kPitch + 4 * cq]) = v;
+                x[i] = v;
             }
+            if constexpr (HasTransforms<Op>::value) op.pre(x);
+#pragma unroll
+            for (int i = 0; i < NI; ++i) *reinterpret_cast<float4*>(&tile[i][r * G::kPitch + 4 * cq]) = x[i];
         }
         __syncthreads();
 
@@ -496,15 +548,13 @@ __global__ __launch_bounds__(kWave) void stream_kernel_scalar(typename Op::Param
         for (int p = 0; p < G::kPasses; ++p) {
             const int r = p * G::kRowsPerPass + crow;
             const int64_t off = (int64_t)(m0 + r) * (int64_t)T + (int64_t)t;
-            float4 v[NO + ND];
+            float4 y[NO], v[NO + ND];
 #pragma unroll
-            for (int o = 0; o < NO; ++o) v[o] = *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]);
-            if constexpr (ND == 1) {
-                float4 y[NO];
+            for (int o = 0; o < NO; ++o) y[o] = *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]);
+            if constexpr (HasTransforms<Op>::value) op.post(y);
 #pragma unroll
-                for (int o = 0; o < NO; ++o) y[o] = v[o];
-                v[NO] = op.derive(y);
-            }
+            for (int o = 0; o < NO; ++o) v[o] = y[o];
+            if constexpr (ND == 1) v[NO] = op.derive(y);
 #pragma unroll
             for (int o = 0; o < NO + ND; ++o) {
                 if (r < rows) {
@@ -531,12 +581,16 @@ struct DuoRows { static constexpr int value = 64; };
 template <class Op>
 struct DuoRows<Op, decltype((void)Op::kDuoRows)> { static constexpr int value = Op::kDuoRows; };
 
-// Two-wave workgroups of this kernel that one compute unit holds at a time (LDS and registers).
+// Copy waves per workgroup of the multi-wave kernel.
+constexpr int kCopyWaves = 1;
+
+// Workgroups of the multi-wave kernel that one compute unit holds at a time (LDS and registers).
 template <class Op, int R, bool STREAM>
 int duo_groups_per_cu() {
     static const int n = [] {
         int v = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&v, stream_kernel_duo<Op, R, STREAM>, 2 * kWave, 0) != hipSuccess)
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&v, stream_kernel_duo<Op, R, STREAM, kCopyWaves>,
+                                                         (1 + kCopyWaves) * kWave, 0) != hipSuccess)
             v = 0;
         return v;
     }();
@@ -589,11 +643,11 @@ int launch_stream(const typename Op::Params& prm, int64_t M, int64_t T, hipStrea
         const int64_t groups = (M + RD - 1) / RD;
         const int per_cu = streaming ? duo_groups_per_cu<Op, RD, true>() : duo_groups_per_cu<Op, RD, false>();
         if (groups <= (int64_t)per_cu * compute_units()) {
-            const dim3 grid((unsigned)groups), block(2 * kWave);
+            const dim3 grid((unsigned)groups), block((1 + kCopyWaves) * kWave);
             if (streaming)
-                hipLaunchKernelGGL((stream_kernel_duo<Op, RD, true>), grid, block, 0, stream, prm, M, (int)T);
+                hipLaunchKernelGGL((stream_kernel_duo<Op, RD, true, kCopyWaves>), grid, block, 0, stream, prm, M, (int)T);
             else
-                hipLaunchKernelGGL((stream_kernel_duo<Op, RD, false>), grid, block, 0, stream, prm, M, (int)T);
+                hipLaunchKernelGGL((stream_kernel_duo<Op, RD, false, kCopyWaves>), grid, block, 0, stream, prm, M, (int)T);
             return (int)hipGetLastError();
         }
     }

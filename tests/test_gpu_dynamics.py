@@ -100,6 +100,26 @@ def test_all_tile_geometries(slayer, M_per_batch):
     assert_rel(got[3], want[3], 'res_bwd grad_cos', rel=1e-4)
 
 
+@pytest.mark.parametrize('thr', [4100.0, 4096.0 + 1.0 / 4096, 7000.3, 16384.0])
+def test_li_fwd_reset_decision_on_states_beyond_float32_integers(slayer, thr):
+    """The kernel decides the reset on the integer state; the reference compares float32(state) with
+    float32(threshold * w).  Beyond 2**24 the conversion rounds, so states next to such a threshold
+    check that both decisions agree."""
+    gen = torch.Generator().manual_seed(seed_of('big states', thr))
+    shape, w = (2, 64, 400), 4096
+    # no decay; now and then a jump to just below threshold * w >= 2**24, then steps of a few LSB
+    jump = (torch.rand(shape, generator=gen) < 0.1).float()
+    x = jump * (thr - torch.randint(0, 6, shape, generator=gen).float() / w) \
+        + (1 - jump) * torch.randint(-2, 4, shape, generator=gen).float() / w
+    decay = torch.tensor([0.0])
+    state = torch.tensor([0.0])
+    ref = O.li_fwd(x, decay, state, w, thr)
+    fired = (ref * w >= thr * w).float().mean()
+    assert 0.02 < float(fired) < 0.5, 'the case must cross the threshold both ways'
+    out = slayer.neuron.dynamics.leaky_integrator.dynamics(x.to(dev()), decay.to(dev()), state.to(dev()), w, thr)
+    assert_exact(out, ref, f'li_fwd big states thr={thr}')
+
+
 def test_li_fwd_negative_and_edge_decays(slayer):
     gen = torch.Generator().manual_seed(7)
     x = sparse_input(gen, (2, 8, 96), p=0.5, amp=30.0)
