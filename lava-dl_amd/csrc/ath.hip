@@ -17,6 +17,7 @@ struct AthFwd {
         float w, inv_w;
         int64_t npb, n_rd, n_td, n_rs, n_ts;
     };
+    static constexpr bool kTransforms = true;    // integer tiles, see to_state / from_state
     int th, r, mt, mr, th_step, base;
     float w, inv_w;
 
@@ -30,13 +31,17 @@ struct AthFwd {
             mr = 4096 - trunc_i32(p.ref_decay[param_index(m, p.npb, p.n_rd)]);
         }
     }
+    __device__ __forceinline__ void pre(float4 (&x)[1]) const { x[0] = to_state(x[0], w); }
+    __device__ __forceinline__ void post(float4 (&o)[2]) const {
+        o[0] = from_state<POW2>(o[0], w, inv_w);
+        o[1] = from_state<POW2>(o[1], w, inv_w);
+    }
     __device__ __forceinline__ void step(const float (&x)[1], float (&o)[2]) {
         r = rs0_12(r, mr);
         th = rs0_12(th - base, mt) + base;
-        const float thf = (float)th, rf = (float)r;
-        o[0] = POW2 ? thf * inv_w : thf / w;
-        o[1] = POW2 ? rf * inv_w : rf / w;
-        const bool fired = trunc_i32(w * x[0]) >= th + r;
+        o[0] = __int_as_float(th);
+        o[1] = __int_as_float(r);
+        const bool fired = __float_as_int(x[0]) >= th + r;
         r += fired ? 2 * th : 0;
         th += fired ? th_step : 0;
     }

@@ -23,14 +23,16 @@ struct CubaFwd {
         const float* in[1];
         float* out[3];
         const float *i_decay, *v_decay, *i_state, *v_state;
-        float w, inv_w, thr, spike_thr, spike_scale;
+        float w, inv_w, spike_thr, spike_scale;
+        int fire_above;                              // voltage reset when the state exceeds this
         int64_t npb, n_id, n_vd, n_is, n_vs;
     };
-    int yc, yv, mi, mv;
-    float w, inv_w, thr, spike_thr, spike_scale;
+    static constexpr bool kTransforms = true;        // integer tiles, see to_state / from_state
+    int yc, yv, mi, mv, fire_above;
+    float w, inv_w, spike_thr, spike_scale;
 
     __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
-        w = p.w; inv_w = p.inv_w; thr = p.thr; spike_thr = p.spike_thr; spike_scale = p.spike_scale;
+        w = p.w; inv_w = p.inv_w; fire_above = p.fire_above; spike_thr = p.spike_thr; spike_scale = p.spike_scale;
         yc = yv = mi = mv = 0;
         if (valid) {
             yc = trunc_i32(p.i_state[p.n_is == 1 ? 0 : m] * w);
@@ -39,15 +41,20 @@ struct CubaFwd {
             mv = 4096 - trunc_i32(p.v_decay[param_index(m, p.npb, p.n_vd)]);
         }
     }
+    __device__ __forceinline__ void pre(float4 (&x)[1]) const { x[0] = to_state(x[0], w); }
+    __device__ __forceinline__ void post(float4 (&o)[2]) const {
+        o[0] = from_state<POW2>(o[0], w, inv_w);
+        o[1] = from_state<POW2>(o[1], w, inv_w);
+    }
     __device__ __forceinline__ void step(const float (&x)[1], float (&o)[2]) {
-        yc = rs0_12(yc, mi) + trunc_i32(w * x[0]);
+        yc = rs0_12(yc, mi) + __float_as_int(x[0]);
+        // the voltage op reads the float32 current: trunc(w * (float(yc) / w)); for a power of two
+        // the scaling is exact and only the int -> float32 rounding remains
         const float cf = (float)yc;
-        const float cur = POW2 ? cf * inv_w : cf / w;
-        const int yn = rs0_12(yv, mv) + trunc_i32(w * cur);     // the voltage op reads the float32 current
-        const float vf = (float)yn;
-        yv = (vf >= thr) ? 0 : yn;
-        o[0] = cur;
-        o[1] = POW2 ? vf * inv_w : vf / w;
+        const int yn = rs0_12(yv, mv) + (POW2 ? trunc_i32(cf) : trunc_i32(w * (cf / w)));
+        yv = (yn > fire_above) ? 0 : yn;             // float(yn) >= threshold, decided on the integer
+        o[0] = __int_as_float(yc);
+        o[1] = __int_as_float(yn);
     }
     __device__ __forceinline__ float spike(float vol) const {
         const float h = (vol >= spike_thr) ? 1.0f : 0.0f;
@@ -121,12 +128,12 @@ extern "C" int slayer_cuba_fwd(float* cur_out, float* vol_out, float* spk_out, c
     if (int e = check_states(M, num_v_states)) return e;
     if (w_scale == 0) return SLAYER_EINVAL;
     const float w = (float)w_scale;
-    const float thr = thr_scaled > 0 ? (float)thr_scaled : __builtin_inff();
+    const int fa = fire_above(thr_scaled > 0 ? (float)thr_scaled : __builtin_inff());
     hipStream_t st = (hipStream_t)stream;
 #define SLAYER_CUBA(P, G)                                                                                        \
     do {                                                                                                         \
         CubaFwd<P, G>::Params p{{in}, {cur_out, vol_out, spk_out}, i_decay, v_decay, i_state, v_state, w,           \
-                                1.0f / w, thr, spike_threshold, spike_scale, neurons_per_batch, num_i_decays,      \
+                                1.0f / w, spike_threshold, spike_scale, fa, neurons_per_batch, num_i_decays,       \
                                 num_v_decays, num_i_states, num_v_states};                                         \
         return cuba_fwd_launch<P, G>(p, M, T, st);                                                                 \
     } while (0)

@@ -34,17 +34,8 @@ struct LiFwd {
             mult = 4096 - trunc_i32(p.decay[param_index(m, p.npb, p.num_decays)]);
         }
     }
-    __device__ __forceinline__ float to_state(float x) const { return __int_as_float(trunc_i32(w * x)); }
-    __device__ __forceinline__ float from_state(float s) const {
-        const float yf = (float)__float_as_int(s);
-        return POW2 ? yf * inv_w : yf / w;
-    }
-    __device__ __forceinline__ void pre(float4 (&x)[1]) const {
-        x[0] = make_float4(to_state(x[0].x), to_state(x[0].y), to_state(x[0].z), to_state(x[0].w));
-    }
-    __device__ __forceinline__ void post(float4 (&o)[1]) const {
-        o[0] = make_float4(from_state(o[0].x), from_state(o[0].y), from_state(o[0].z), from_state(o[0].w));
-    }
+    __device__ __forceinline__ void pre(float4 (&x)[1]) const { x[0] = to_state(x[0], w); }
+    __device__ __forceinline__ void post(float4 (&o)[1]) const { o[0] = from_state<POW2>(o[0], w, inv_w); }
     __device__ __forceinline__ void step(const float (&x)[1], float (&o)[1]) {
         const int yn = rs0_12(y, mult) + __float_as_int(x[0]);
         o[0] = __int_as_float(yn);

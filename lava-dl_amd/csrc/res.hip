@@ -17,15 +17,16 @@ struct ResFwd {
         const float* in[2];
         float* out[2];
         const float *sin_decay, *cos_decay, *re_state, *im_state;
-        float w, inv_w, thr;
-        int im_reset;
+        float w, inv_w;
+        int fire_above, im_reset;                // reset when the imaginary state exceeds fire_above
         int64_t npb, num_decays, n_rs, n_is;
     };
-    int re, im, s, c, im_reset;
-    float w, inv_w, thr;
+    static constexpr bool kTransforms = true;    // integer tiles, see to_state / from_state
+    int re, im, s, c, fire_above, im_reset;
+    float w, inv_w;
 
     __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
-        w = p.w; inv_w = p.inv_w; thr = p.thr; im_reset = p.im_reset;
+        w = p.w; inv_w = p.inv_w; fire_above = p.fire_above; im_reset = p.im_reset;
         re = im = s = c = 0;
         if (valid) {
             re = trunc_i32(p.re_state[p.n_rs == 1 ? 0 : m] * w);
@@ -35,18 +36,25 @@ struct ResFwd {
             c = trunc_i32(p.cos_decay[j]);
         }
     }
+    __device__ __forceinline__ void pre(float4 (&x)[2]) const {
+        x[0] = to_state(x[0], w);
+        x[1] = to_state(x[1], w);
+    }
+    __device__ __forceinline__ void post(float4 (&o)[2]) const {
+        o[0] = from_state<POW2>(o[0], w, inv_w);
+        o[1] = from_state<POW2>(o[1], w, inv_w);
+    }
     __device__ __forceinline__ void step(const float (&x)[2], float (&o)[2]) {
-        const int re_n = rs0_12(c, re) - rs0_12(s, im) + trunc_i32(w * x[0]);
-        const int im_n = rs0_12(s, re) + rs0_12(c, im) + trunc_i32(w * x[1]);
-        const float ref = (float)re_n, imf = (float)im_n;
-        o[0] = POW2 ? ref * inv_w : ref / w;
-        o[1] = POW2 ? imf * inv_w : imf / w;
+        const int re_n = rs0_12(c, re) - rs0_12(s, im) + __float_as_int(x[0]);
+        const int im_n = rs0_12(s, re) + rs0_12(c, im) + __float_as_int(x[1]);
+        o[0] = __int_as_float(re_n);
+        o[1] = __int_as_float(im_n);
         if (HAS_THR) {
-            // the kept imaginary state makes a float32 round trip, as the mixed int/float
-            // expression of the CPU branch does
-            const bool fired = imf >= thr;
+            // float(im_n) >= threshold, decided on the integer; the kept imaginary state makes a
+            // float32 round trip, as the mixed int/float expression of the CPU branch does
+            const bool fired = im_n > fire_above;
             re = fired ? 0 : re_n;
-            im = fired ? im_reset : trunc_i32(imf);
+            im = fired ? im_reset : trunc_i32((float)im_n);
         } else {
             re = re_n;
             im = im_n;
@@ -155,7 +163,7 @@ static int res_fwd_launch(float* re_out, float* im_out, const float* re_in, cons
                           hipStream_t stream) {
     using Op = ResFwd<POW2, HAS_THR>;
     typename Op::Params p{{re_in, im_in}, {re_out, im_out}, sin_decay, cos_decay, re_state, im_state,
-                          w, 1.0f / w, thr, im_reset, npb, nd, n_rs, n_is};
+                          w, 1.0f / w, fire_above(thr), im_reset, npb, nd, n_rs, n_is};
     return launch_stream<Op>(p, M, T, stream);
 }
 

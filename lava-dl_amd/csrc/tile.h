@@ -42,6 +42,24 @@ inline int fire_above(float thr) {
     return (int)(c - 1);
 }
 
+// Integer tiles: an Op with kTransforms can keep its fixed-point states in LDS as integers (bit
+// patterns in float registers).  Inputs are scaled and truncated on the way in, states converted
+// and scaled back on the way out.
+__device__ __forceinline__ float to_state(float x, float w) { return __int_as_float((int)(w * x)); }
+__device__ __forceinline__ float4 to_state(float4 x, float w) {
+    return make_float4(to_state(x.x, w), to_state(x.y, w), to_state(x.z, w), to_state(x.w, w));
+}
+template <bool POW2>
+__device__ __forceinline__ float from_state(float s, float w, float inv_w) {
+    const float f = (float)__float_as_int(s);
+    return POW2 ? f * inv_w : f / w;
+}
+template <bool POW2>
+__device__ __forceinline__ float4 from_state(float4 s, float w, float inv_w) {
+    return make_float4(from_state<POW2>(s.x, w, inv_w), from_state<POW2>(s.y, w, inv_w),
+                       from_state<POW2>(s.z, w, inv_w), from_state<POW2>(s.w, w, inv_w));
+}
+
 // Streaming (non-temporal) 16-byte global accesses: tensors on this path are read once and
 // written once, so they should not displace each other in L2.
 typedef float vf4 __attribute__((ext_vector_type(4)));
