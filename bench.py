@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch divided by algorithmic bytes, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # script scaled by a plain copy of known size (profiles/cuba_fwd_bwd_32x16x32x32x300.md).
-MEASURED_TRAFFIC_FACTOR = {'stream_kernel<LiFwd>': 1.041, 'stream_kernel<LiBwd>': 1.058,
+MEASURED_TRAFFIC_FACTOR = {'stream_kernel<LiFwd>': 1.037, 'stream_kernel<LiBwd>': 1.058,
                            'spike_fwd_kernel': 1.000, 'spike_bwd_kernel': 1.000}
 
 

@@ -415,3 +415,20 @@ def test_debug_mode_cross_check_passes_and_catches_overflow(slayer):
     from lava_dl_amd.slayer.neuron.dynamics import leaky_integrator as L
     got = L._fwd(big, zero, zero, -1, 64, entry='slayer_li_fwd_naive')
     assert_exact(got, O.li_fwd(big.cpu(), torch.tensor([0.0]), torch.tensor([0.0]), 64), 'naive li_fwd beyond 2^31')
+
+
+def test_rows_longer_than_the_vector_path_allows(slayer):
+    """T > 2**22 leaves the dwordx4 kernels (32-bit byte offsets per wave) for the dword kernel;
+    too long for the CPU oracle, so the independent one-thread-per-neuron kernel is the checker
+    (debug=True raises on any mismatch) and the head of the rows is compared with the oracle."""
+    gen = torch.Generator().manual_seed(77)
+    T = (1 << 22) + 8
+    x = sparse_input(gen, (1, 3, T), p=0.05, amp=1.5).to(dev()).requires_grad_()
+    d = torch.tensor([300.0, 1000.0, 4000.0], device=dev(), requires_grad=True)
+    zero = torch.zeros(1, device=dev())
+    y = slayer.neuron.dynamics.leaky_integrator.dynamics(x, d, zero, 64, 1.0, debug=True)
+    y.backward(torch.ones_like(y) * 1e-3)
+    head = 2048
+    ref = O.li_fwd(x.detach().cpu()[..., :head], d.detach().cpu(), torch.tensor([0.0]), 64, 1.0)
+    assert_exact(y.detach()[..., :head], ref, 'li_fwd long rows, head')
+    assert torch.isfinite(x.grad).all() and float(x.grad.abs().sum()) > 0
