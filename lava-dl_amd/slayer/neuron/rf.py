@@ -12,14 +12,14 @@ TAU_RHO_MULT = 0.5      # surrogate-gradient constants of the RF family (neuron/
 SCALE_RHO_MULT = 10
 
 
-class Neuron(_Base):
-    """``Neuron(threshold, period, decay, ...)``: the state rotates by 2 pi / period per step and
-    shrinks by (1 - decay); it spikes when the real part is above threshold while the imaginary
-    part crosses zero upwards.  ``forward((real_input, imag_input))`` returns the spikes."""
+class ResonatorNeuron(_Base):
+    """What the resonator family shares (rf, rf_iz, adrf, adrf_iz in the reference): the rotation
+    parameters sin_decay / cos_decay from (period, decay), their clamp to the first quadrant of the
+    unit circle, per-channel initialisation, one norm per input component, and the complex state."""
 
     def __init__(self, threshold, period, decay, tau_grad=1, scale_grad=1, scale=1 << 6, norm=None,
                  dropout=None, shared_param=True, persistent_state=False, requires_grad=False,
-                 graded_spike=False, log_init=True):
+                 graded_spike=False, log_init=True, extra_decays=None, extra_states=None):
         super().__init__(threshold, tau_grad, scale_grad, scale, None, dropout, shared_param,
                          persistent_state, requires_grad, graded_spike)
         self.real_norm = norm() if norm is not None else None
@@ -48,12 +48,18 @@ class Neuron(_Base):
             value = self.p_scale * fn(2 * np.pi / start_p) * (1 - start_d)
             self.register_parameter(name, torch.nn.Parameter(torch.FloatTensor([value]),
                                                              requires_grad=self.requires_grad))
-        self._register_states(real_state=0.0, imag_state=0.0)
+        if extra_decays:
+            self._register_decays(**extra_decays)
+        self._register_states(real_state=0.0, imag_state=0.0, **(extra_states or {}))
         self.clamp()
 
     def clamp(self):
-        """Keep the gain below 1 (4095/4096), sin_decay >= 1 and cos_decay >= 0."""
+        """Keep the gain below 1 (4095/4096), sin_decay >= 1 and cos_decay >= 0 (and the other
+        decays inside [0, 1])."""
         with torch.no_grad():
+            for name, prm in self.named_parameters(recurse=False):
+                if name not in ('sin_decay', 'cos_decay'):
+                    prm.data.clamp_(0, self.p_scale)
             gain = torch.sqrt(self.sin_decay ** 2 + self.cos_decay ** 2)
             ratio = gain.clamp(0, self.p_scale - 1) / gain
             self.sin_decay.data *= ratio
@@ -70,9 +76,10 @@ class Neuron(_Base):
         decay = d_lo + (d_hi - d_lo) * torch.rand(channels, dtype=torch.float).to(device)
         self.sin_decay.data = self.p_scale * torch.sin(2 * np.pi * frequency) * (1 - decay)
         self.cos_decay.data = self.p_scale * torch.cos(2 * np.pi * frequency) * (1 - decay)
+        super()._draw_per_channel(channels, device)          # the other decays, if any
 
-    def dynamics(self, input):
-        """(real, imag) traces for ``input = (real_input, imag_input)``."""
+    def _inputs(self, input):
+        """Shape checks, state preparation and input norms; returns (real_input, imag_input)."""
         real_input, imag_input = input
         if real_input.shape != imag_input.shape:
             raise AssertionError(f'Real input tensor shape ({real_input.shape}) does not match '
@@ -82,6 +89,20 @@ class Neuron(_Base):
             real_input = self.real_norm(real_input)
         if self.imag_norm is not None:
             imag_input = self.imag_norm(imag_input)
+        return real_input, imag_input
+
+    def forward(self, input):
+        return self.spike(*self.dynamics(input))
+
+
+class Neuron(ResonatorNeuron):
+    """``Neuron(threshold, period, decay, ...)``: the state rotates by 2 pi / period per step and
+    shrinks by (1 - decay); it spikes when the real part is above threshold while the imaginary
+    part crosses zero upwards.  ``forward((real_input, imag_input))`` returns the spikes."""
+
+    def dynamics(self, input):
+        """(real, imag) traces for ``input = (real_input, imag_input)``."""
+        real_input, imag_input = self._inputs(input)
         real, imag = resonator.dynamics(real_input, imag_input, quantize(self.sin_decay), quantize(self.cos_decay),
                                         self.real_state, self.imag_state, self.s_scale, debug=self.debug)
         if self.persistent_state:
