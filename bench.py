@@ -168,6 +168,23 @@ class CubaFused(Cuba):
         return spk, g_x, gd_v, gd_i
 
 
+class CubaFusedLean(Cuba):
+    name = 'CUBA neuron fwd+bwd, fused kernels without the current trace (no decay gradients)'
+    ops = [('cuba_fwd', 'stream_kernel<CubaFwd>', 12), ('cuba_bwd', 'stream_kernel<CubaBwd>', 12)]
+
+    def __init__(self, dev):
+        super().__init__(dev)
+        from lava_dl_amd.slayer.neuron.dynamics import cuba_fused
+        self.F = cuba_fused
+
+    def step(self, t):
+        with t('cuba_fwd'):
+            _, vol, spk = self.F._fwd(self.x, self.d_i, self.d_v, self.zero, self.zero, self.w, self.thr, False, 1, True)
+        with t('cuba_bwd'):
+            g_x, _, _ = self.F._bwd(self.g, vol, None, self.d_i, self.d_v, self.thr, 1.0, 1.0, False, False)
+        return spk, g_x
+
+
 class CubaFwdSmall(Workload):
     name = 'CUBA LIF dynamics forward only (latency-bound: 512 neurons)'
     shape = (4, 128, 200)
@@ -376,7 +393,7 @@ class Synapse(Workload):
         O.conv_bwd(O.shift(g_z, -c['delay'], 1), c['filt'], 1)
 
 
-WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'alif_fused': AlifFused, 'rf': Rf, 'rf_fused': RfFused, 'synapse': Synapse}
+WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fused_lean': CubaFusedLean, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'alif_fused': AlifFused, 'rf': Rf, 'rf_fused': RfFused, 'synapse': Synapse}
 
 
 def cpu_baseline(job, budget_s=20.0):

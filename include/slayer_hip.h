@@ -240,8 +240,11 @@ int slayer_cumsum(float *out, const float *in, const float *state, int64_t num_s
  * (each intermediate is rounded to float32 exactly as at the operator boundaries); it only saves the
  * re-reading of the intermediates: 16 instead of 24 bytes per neuron-timestep.
  * thr_scaled = (threshold + eps) * w_scale for the reset (double, <= 0 disables it),
- * spike_threshold = threshold + eps for the spike compare on the float32 voltage. */
-int slayer_cuba_fwd(float *cur_out, float *vol_out, float *spk_out, const float *in,
+ * spike_threshold = threshold + eps for the spike compare on the float32 voltage.
+ * cur_out may be NULL when the current trace is not wanted (no decay gradient in the backward pass):
+ * 12 bytes per neuron-timestep.  cur_last_out ([M], may be NULL) receives the current of the last
+ * step, i.e. current[..., -1], which is what a persistent state needs. */
+int slayer_cuba_fwd(float *cur_out, float *vol_out, float *spk_out, float *cur_last_out, const float *in,
                     const float *i_decay, const float *v_decay,
                     const float *i_state, const float *v_state,
                     double thr_scaled, float spike_threshold, int graded, float spike_scale, int w_scale,
@@ -250,8 +253,8 @@ int slayer_cuba_fwd(float *cur_out, float *vol_out, float *spk_out, const float 
 
 /* Backward of the above = slayer_spike_bwd -> slayer_li_bwd (voltage) -> slayer_li_bwd (current) in
  * one launch (16 instead of 36 bytes per neuron-timestep); grad_in is bit-identical to the chain.
- * grad_i_decay / grad_v_decay may both be NULL; workspace: 2*M + 64*(num_i_decays + num_v_decays)
- * floats when they are not. */
+ * grad_i_decay / grad_v_decay may both be NULL (then current may be NULL too and is not read: 12 bytes
+ * per neuron-timestep); workspace: 2*M + 64*(num_i_decays + num_v_decays) floats when they are not. */
 int slayer_cuba_bwd(float *grad_in, float *grad_i_decay, float *grad_v_decay,
                     const float *grad_spikes, const float *voltage, const float *current,
                     const float *i_decay, const float *v_decay,

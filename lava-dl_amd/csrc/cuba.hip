@@ -13,15 +13,19 @@ int launch_reduce_param_grad(float* grad, const float* partial, float* scratch, 
                              int64_t num_params, hipStream_t stream);   // li.hip
 int launch_zero_fill(float* p, int64_t n, hipStream_t stream);          // li.hip
 
-template <bool POW2, bool GRADED>
+// KEEP_CURRENT = false leaves the current trace out (a caller that wants no decay gradient does not
+// need it): 12 instead of 16 bytes per neuron-timestep.
+template <bool POW2, bool GRADED, bool KEEP_CURRENT>
 struct CubaFwd {
-    static constexpr int kIn = 1, kOut = 2;          // out: current, voltage
+    static constexpr int kIn = 1, kOut = KEEP_CURRENT ? 2 : 1;     // out: [current,] voltage
+    static constexpr int kVol = kOut - 1;
     static constexpr int kDerived = 1;               // spikes: a function of the voltage alone
     static constexpr bool kReverse = false;
     static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
     struct Params {
         const float* in[1];
-        float* out[3];
+        float* out[kOut + 1];
+        float* cur_last;                             // [M] current of the last step, or nullptr
         const float *i_decay, *v_decay, *i_state, *v_state;
         float w, inv_w, spike_thr, spike_scale;
         int fire_above;                              // voltage reset when the state exceeds this
@@ -42,40 +46,44 @@ struct CubaFwd {
         }
     }
     __device__ __forceinline__ void pre(float4 (&x)[1]) const { x[0] = to_state(x[0], w); }
-    __device__ __forceinline__ void post(float4 (&o)[2]) const {
-        o[0] = from_state<POW2>(o[0], w, inv_w);
-        o[1] = from_state<POW2>(o[1], w, inv_w);
+    __device__ __forceinline__ void post(float4 (&o)[kOut]) const {
+#pragma unroll
+        for (int i = 0; i < kOut; ++i) o[i] = from_state<POW2>(o[i], w, inv_w);
     }
-    __device__ __forceinline__ void step(const float (&x)[1], float (&o)[2]) {
+    __device__ __forceinline__ void step(const float (&x)[1], float (&o)[kOut]) {
         yc = rs0_12(yc, mi) + __float_as_int(x[0]);
         // the voltage op reads the float32 current: trunc(w * (float(yc) / w)); for a power of two
         // the scaling is exact and only the int -> float32 rounding remains
         const float cf = (float)yc;
         const int yn = rs0_12(yv, mv) + (POW2 ? trunc_i32(cf) : trunc_i32(w * (cf / w)));
         yv = (yn > fire_above) ? 0 : yn;             // float(yn) >= threshold, decided on the integer
-        o[0] = __int_as_float(yc);
-        o[1] = __int_as_float(yn);
+        if (KEEP_CURRENT) o[0] = __int_as_float(yc);
+        o[kVol] = __int_as_float(yn);
     }
     __device__ __forceinline__ float spike(float vol) const {
         const float h = (vol >= spike_thr) ? 1.0f : 0.0f;
         return GRADED ? (h * vol) / spike_scale : h;
     }
-    __device__ __forceinline__ float4 derive(const float4 (&y)[2]) const {
-        return make_float4(spike(y[1].x), spike(y[1].y), spike(y[1].z), spike(y[1].w));
+    __device__ __forceinline__ float4 derive(const float4 (&y)[kOut]) const {
+        return make_float4(spike(y[kVol].x), spike(y[kVol].y), spike(y[kVol].z), spike(y[kVol].w));
     }
-    __device__ __forceinline__ void finish(const Params&, int64_t, bool) {}
+    __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
+        if (valid && p.cur_last) p.cur_last[m] = from_state<POW2>(__int_as_float(yc), w, inv_w);
+    }
 };
 
-template <bool GRADED>
+// DECAY_GRAD = false drops the saved current and both decay-gradient sums: 12 instead of 16 bytes
+// per neuron-timestep.
+template <bool GRADED, bool DECAY_GRAD>
 struct CubaBwd {
-    static constexpr int kIn = 3, kOut = 1;          // in: grad of spikes, saved voltage, saved current
+    static constexpr int kIn = DECAY_GRAD ? 3 : 2, kOut = 1;   // in: grad of spikes, saved voltage[, saved current]
     static constexpr bool kReverse = true;
     static constexpr int64_t kRows32Below = 4096, kRows16Below = 4096;     // exp per step: keep all lanes busy
     struct Params {
-        const float* in[3];
+        const float* in[kIn];
         float* out[1];
         const float *i_decay, *v_decay;
-        float *partial_i, *partial_v;                // per-neuron decay gradients, or nullptr
+        float *partial_i, *partial_v;                // per-neuron decay gradients (DECAY_GRAD only)
         float spike_thr, tau, rho;
         int64_t npb, n_id, n_vd;
     };
@@ -90,17 +98,19 @@ struct CubaBwd {
             av = 1.0f - p.v_decay[param_index(m, p.npb, p.n_vd)] / 4096.0f;
         }
     }
-    __device__ __forceinline__ void step(const float (&x)[3], float (&o)[1]) {
+    __device__ __forceinline__ void step(const float (&x)[kIn], float (&o)[1]) {
         const float d = x[1] - spike_thr;
         const float gv = GRADED ? (rho * expf(fminf(d, 0.0f) / tau)) * x[0] : (lead * expf(-fabsf(d) / tau)) * x[0];
-        acc_v = __fmaf_rn(gc, x[1], acc_v);          // gc, gx still hold the gradients of step t+1
-        acc_i = __fmaf_rn(gx, x[2], acc_i);
+        if (DECAY_GRAD) {
+            acc_v = __fmaf_rn(gc, x[1], acc_v);      // gc, gx still hold the gradients of step t+1
+            acc_i = __fmaf_rn(gx, x[kIn - 1], acc_i);
+        }
         gc = av * gc + gv;
         gx = ai * gx + gc;
         o[0] = gx;
     }
     __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
-        if (valid && p.partial_i) { p.partial_i[m] = acc_i; p.partial_v[m] = acc_v; }
+        if (DECAY_GRAD && valid && p.partial_i) { p.partial_i[m] = acc_i; p.partial_v[m] = acc_v; }
     }
 };
 
@@ -108,12 +118,7 @@ struct CubaBwd {
 
 using namespace slayer;
 
-template <bool POW2, bool GRADED>
-static int cuba_fwd_launch(const typename CubaFwd<POW2, GRADED>::Params& p, int64_t M, int64_t T, hipStream_t st) {
-    return launch_stream<CubaFwd<POW2, GRADED>>(p, M, T, st);
-}
-
-extern "C" int slayer_cuba_fwd(float* cur_out, float* vol_out, float* spk_out, const float* in,
+extern "C" int slayer_cuba_fwd(float* cur_out, float* vol_out, float* spk_out, float* cur_last_out, const float* in,
                                const float* i_decay, const float* v_decay,
                                const float* i_state, const float* v_state,
                                double thr_scaled, float spike_threshold, int graded, float spike_scale, int w_scale,
@@ -121,7 +126,7 @@ extern "C" int slayer_cuba_fwd(float* cur_out, float* vol_out, float* spk_out, c
                                int64_t num_i_states, int64_t num_v_states, int64_t T, void* stream) {
     if (int e = check_rows(M, T)) return e;
     if (M == 0 || T == 0) return 0;
-    if (!cur_out || !vol_out || !spk_out || !in || !i_decay || !v_decay || !i_state || !v_state) return SLAYER_ENULL;
+    if (!vol_out || !spk_out || !in || !i_decay || !v_decay || !i_state || !v_state) return SLAYER_ENULL;
     if (int e = check_params(M, neurons_per_batch, num_i_decays)) return e;
     if (int e = check_params(M, neurons_per_batch, num_v_decays)) return e;
     if (int e = check_states(M, num_i_states)) return e;
@@ -132,10 +137,18 @@ extern "C" int slayer_cuba_fwd(float* cur_out, float* vol_out, float* spk_out, c
     hipStream_t st = (hipStream_t)stream;
 #define SLAYER_CUBA(P, G)                                                                                        \
     do {                                                                                                         \
-        CubaFwd<P, G>::Params p{{in}, {cur_out, vol_out, spk_out}, i_decay, v_decay, i_state, v_state, w,           \
-                                1.0f / w, spike_threshold, spike_scale, fa, neurons_per_batch, num_i_decays,       \
-                                num_v_decays, num_i_states, num_v_states};                                         \
-        return cuba_fwd_launch<P, G>(p, M, T, st);                                                                 \
+        if (cur_out) {                                                                                           \
+            CubaFwd<P, G, true>::Params p{{in}, {cur_out, vol_out, spk_out}, cur_last_out, i_decay, v_decay,      \
+                                          i_state, v_state, w, 1.0f / w, spike_threshold, spike_scale, fa,       \
+                                          neurons_per_batch, num_i_decays, num_v_decays, num_i_states,           \
+                                          num_v_states};                                                         \
+            return launch_stream<CubaFwd<P, G, true>>(p, M, T, st);                                              \
+        }                                                                                                        \
+        CubaFwd<P, G, false>::Params p{{in}, {vol_out, spk_out}, cur_last_out, i_decay, v_decay, i_state,         \
+                                       v_state, w, 1.0f / w, spike_threshold, spike_scale, fa,                   \
+                                       neurons_per_batch, num_i_decays, num_v_decays, num_i_states,              \
+                                       num_v_states};                                                            \
+        return launch_stream<CubaFwd<P, G, false>>(p, M, T, st);                                                 \
     } while (0)
     if (is_pow2(w_scale)) { if (graded) SLAYER_CUBA(true, true); else SLAYER_CUBA(true, false); }
     if (graded) SLAYER_CUBA(false, true);
@@ -158,18 +171,23 @@ extern "C" int slayer_cuba_bwd(float* grad_in, float* grad_i_decay, float* grad_
     if (want && !workspace && M > 0) return SLAYER_ENULL;
     hipStream_t st = (hipStream_t)stream;
     if (M > 0 && T > 0) {
-        if (!grad_in || !grad_spikes || !voltage || !current || !i_decay || !v_decay) return SLAYER_ENULL;
-        if (graded) {
-            CubaBwd<true>::Params p{{grad_spikes, voltage, current}, {grad_in}, i_decay, v_decay,
-                                    want ? workspace : nullptr, want ? workspace + M : nullptr,
-                                    spike_threshold, tau_rho, scale_rho, neurons_per_batch, num_i_decays, num_v_decays};
-            if (int e = launch_stream<CubaBwd<true>>(p, M, T, st)) return e;
-        } else {
-            CubaBwd<false>::Params p{{grad_spikes, voltage, current}, {grad_in}, i_decay, v_decay,
-                                     want ? workspace : nullptr, want ? workspace + M : nullptr,
-                                     spike_threshold, tau_rho, scale_rho, neurons_per_batch, num_i_decays, num_v_decays};
-            if (int e = launch_stream<CubaBwd<false>>(p, M, T, st)) return e;
-        }
+        if (!grad_in || !grad_spikes || !voltage || !i_decay || !v_decay || (want && !current)) return SLAYER_ENULL;
+#define SLAYER_CUBA_BWD(G)                                                                                       \
+    do {                                                                                                         \
+        if (want) {                                                                                              \
+            CubaBwd<G, true>::Params p{{grad_spikes, voltage, current}, {grad_in}, i_decay, v_decay, workspace,   \
+                                       workspace + M, spike_threshold, tau_rho, scale_rho, neurons_per_batch,    \
+                                       num_i_decays, num_v_decays};                                              \
+            if (int e = launch_stream<CubaBwd<G, true>>(p, M, T, st)) return e;                                  \
+        } else {                                                                                                 \
+            CubaBwd<G, false>::Params p{{grad_spikes, voltage}, {grad_in}, i_decay, v_decay, nullptr, nullptr,    \
+                                        spike_threshold, tau_rho, scale_rho, neurons_per_batch, num_i_decays,    \
+                                        num_v_decays};                                                           \
+            if (int e = launch_stream<CubaBwd<G, false>>(p, M, T, st)) return e;                                 \
+        }                                                                                                        \
+    } while (0)
+        if (graded) SLAYER_CUBA_BWD(true); else SLAYER_CUBA_BWD(false);
+#undef SLAYER_CUBA_BWD
     }
     if (want) {
         if (M == 0 || T == 0) {

@@ -63,10 +63,11 @@ class Neuron(_Base):
             input, self._q('current_decay'), self._q('voltage_decay'),
             self.current_state.contiguous(), self.voltage_state.contiguous(), self.s_scale,
             self.threshold + self.threshold_eps, self.tau_rho * TAU_RHO_MULT, self.scale_rho * SCALE_RHO_MULT,
-            self.graded_spike, 1)
+            self.graded_spike, 1, keep_current=self.requires_grad)
         if self.persistent_state:
             with torch.no_grad():
-                self.current_state = current[..., -1].clone()
+                # without trainable decays the kernel skips the current trace and returns its last step
+                self.current_state = (current[..., -1] if self.requires_grad else current).clone()
                 self.voltage_state = leaky_integrator.persistent_state(
                     voltage[..., -1], spike[..., -1]).detach().clone()
         if self.drop is not None:

@@ -11,19 +11,25 @@ from ... import _native as N
 
 
 def dynamics(input, current_decay, voltage_decay, current_state, voltage_state, w_scale, threshold,
-             tau_rho, scale_rho, graded_spike=False, spike_scale=1):
+             tau_rho, scale_rho, graded_spike=False, spike_scale=1, keep_current=True):
     """(current, voltage, spike) of a CUBA neuron.
+
+    With ``keep_current=False`` and decays that do not require a gradient the current trace is
+    neither written nor read back (24 instead of 32 bytes per neuron-timestep for forward plus
+    backward) and ``current`` holds only the last step, shaped like the states.
 
     ``threshold`` is used both for the voltage reset (compared in integer state units, as
     ``leaky_integrator.dynamics`` does) and for the spike (compared on the float32 voltage, as
     ``Spike`` does).  Gradients flow from ``spike`` to ``input`` and to both decays; the returned
     current and voltage traces are detached.
     """
+    lean = not keep_current and not (current_decay.requires_grad or voltage_decay.requires_grad)
     return _CubaFused.apply(input, current_decay, voltage_decay, current_state, voltage_state,
-                            w_scale, threshold, tau_rho, scale_rho, graded_spike, spike_scale)
+                            w_scale, threshold, tau_rho, scale_rho, graded_spike, spike_scale, lean)
 
 
-def _fwd(input, i_decay, v_decay, i_state, v_state, w_scale, threshold, graded, spike_scale):
+def _fwd(input, i_decay, v_decay, i_state, v_state, w_scale, threshold, graded, spike_scale, lean=False):
+    """lean: no current trace; the first result is then current[..., -1]."""
     dev = N.require_gpu(input, i_decay, v_decay, i_state, v_state)
     input, i_decay, v_decay = input.contiguous(), i_decay.contiguous(), v_decay.contiguous()
     i_state, v_state = i_state.contiguous(), v_state.contiguous()
@@ -31,19 +37,24 @@ def _fwd(input, i_decay, v_decay, i_state, v_state, w_scale, threshold, graded, 
     for name, s in (('current_state', i_state), ('voltage_state', v_state)):
         if s.numel() not in (1, M):
             raise RuntimeError(f'{name} has {s.numel()} elements, expected 1 or {M}')
-    cur, vol, spk = (torch.empty_like(input) for _ in range(3))
+    vol, spk = torch.empty_like(input), torch.empty_like(input)
+    cur = None if lean else torch.empty_like(input)
+    cur_last = torch.empty(input.shape[:-1], dtype=input.dtype, device=dev) if lean else None
     with torch.cuda.device(dev):
         N.check(N.lib().slayer_cuba_fwd(
-            N.ptr(cur), N.ptr(vol), N.ptr(spk), N.ptr(input), N.ptr(i_decay), N.ptr(v_decay),
+            N.ptr(cur), N.ptr(vol), N.ptr(spk), N.ptr(cur_last), N.ptr(input), N.ptr(i_decay), N.ptr(v_decay),
             N.ptr(i_state), N.ptr(v_state), float(threshold * w_scale), float(threshold),
             1 if graded else 0, float(spike_scale), int(w_scale),
             M, N.neurons_per_batch(input), i_decay.numel(), v_decay.numel(),
             i_state.numel(), v_state.numel(), T, N.stream_handle()))
-    return cur, vol, spk
+    return (cur_last if lean else cur), vol, spk
 
 
 def _bwd(grad_spikes, vol, cur, i_decay, v_decay, threshold, tau_rho, scale_rho, graded, need_decay_grad=True):
-    dev = N.require_gpu(grad_spikes, vol, cur, i_decay, v_decay)
+    dev = N.require_gpu(grad_spikes, vol, i_decay, v_decay) if cur is None else \
+        N.require_gpu(grad_spikes, vol, cur, i_decay, v_decay)
+    if cur is None and need_decay_grad:
+        raise RuntimeError('the decay gradients need the current trace')
     grad_spikes, i_decay, v_decay = grad_spikes.contiguous(), i_decay.contiguous(), v_decay.contiguous()
     M, T = N.rows_and_steps(grad_spikes)
     grad_input = torch.empty_like(grad_spikes)
@@ -64,11 +75,11 @@ def _bwd(grad_spikes, vol, cur, i_decay, v_decay, threshold, tau_rho, scale_rho,
 class _CubaFused(torch.autograd.Function):
     @staticmethod
     def forward(ctx, input, i_decay, v_decay, i_state, v_state, w_scale, threshold, tau_rho, scale_rho,
-                graded, spike_scale):
+                graded, spike_scale, lean):
         graded = graded is True
         cur, vol, spk = _fwd(input, i_decay.detach(), v_decay.detach(), i_state.detach(), v_state.detach(),
-                             w_scale, threshold, graded, spike_scale)
-        ctx.save_for_backward(cur, vol, i_decay, v_decay)
+                             w_scale, threshold, graded, spike_scale, lean)
+        ctx.save_for_backward(None if lean else cur, vol, i_decay, v_decay)
         ctx.cfg = (float(threshold), float(tau_rho), float(scale_rho), graded)
         ctx.mark_non_differentiable(cur, vol)
         return cur, vol, spk
@@ -77,9 +88,9 @@ class _CubaFused(torch.autograd.Function):
     def backward(ctx, _g_cur, _g_vol, grad_spikes):
         cur, vol, i_decay, v_decay = ctx.saved_tensors
         threshold, tau_rho, scale_rho, graded = ctx.cfg
-        need = ctx.needs_input_grad[1] or ctx.needs_input_grad[2]
+        need = (ctx.needs_input_grad[1] or ctx.needs_input_grad[2]) and cur is not None
         g_in, g_i, g_v = _bwd(grad_spikes, vol, cur, i_decay.detach(), v_decay.detach(),
                               threshold, tau_rho, scale_rho, graded, need)
         if g_i is not None:
             g_i, g_v = g_i.reshape(i_decay.shape), g_v.reshape(v_decay.shape)
-        return (g_in, g_i, g_v) + (None,) * 8
+        return (g_in, g_i, g_v) + (None,) * 9

@@ -332,3 +332,30 @@ def test_alif_neuron_forward_uses_fused_path_with_same_results(slayer):
         sb.sum().backward()
         assert torch.equal(xa.grad, xb.grad), f'call {k}: input gradients differ'
     assert float(sa.detach().sum()) > 0
+
+
+@pytest.mark.parametrize('shape,w', [((4, 128, 200), 64), ((3, 70, 129), 100), ((4, 9000, 64), 4096)])
+def test_fused_cuba_without_current_trace(slayer, shape, w):
+    """keep_current=False skips the current trace: same voltage, spikes and input gradient, and the
+    last current comes back per neuron."""
+    from tests.util import seed_of
+    gen = torch.Generator().manual_seed(seed_of(shape, w, 'lean cuba'))
+    C = shape[1]
+    x = sparse_input(gen, shape, p=0.2, amp=1.5).to(dev())
+    g = torch.randn(shape, generator=gen).to(dev())
+    d_i, d_v = (torch.randint(0, 4096, (C,), generator=gen).float().to(dev()) for _ in range(2))
+    s_i, s_v = (torch.randn(shape[:-1], generator=gen).to(dev()) for _ in range(2))
+    F = slayer.neuron.dynamics.cuba_fused
+    a, b = x.clone().requires_grad_(), x.clone().requires_grad_()
+    cur, vol, spk = F.dynamics(a, d_i, d_v, s_i, s_v, w, 1.0, 0.7, 1.5)
+    spk.backward(g)
+    cur_last, vol2, spk2 = F.dynamics(b, d_i, d_v, s_i, s_v, w, 1.0, 0.7, 1.5, keep_current=False)
+    spk2.backward(g)
+    assert cur_last.shape == shape[:-1] and torch.equal(cur_last, cur[..., -1])
+    assert torch.equal(vol2, vol) and torch.equal(spk2.detach(), spk.detach()) and float(spk.detach().sum()) > 0
+    assert torch.equal(b.grad, a.grad)
+    # trainable decays still get their gradients: the flag is ignored then
+    dd = d_i.clone().requires_grad_()
+    c3, _, s3 = F.dynamics(x, dd, d_v, s_i, s_v, w, 1.0, 0.7, 1.5, keep_current=False)
+    s3.backward(g)
+    assert c3.shape == shape and dd.grad is not None and torch.isfinite(dd.grad).all()
