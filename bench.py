@@ -1,6 +1,6 @@
 """Benchmark of the SLAYER neuron-dynamics hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cuba|cuba_fused|cuba_fwd_small|alif|alif_fused|rf|rf_fused|synapse]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cuba|cuba_fused|cuba_fused_lean|cuba_fwd_small|alif|alif_fused|alif_fused_lean|rf|rf_fused|synapse]
 
 A step is one pass of the workload's op sequence over one batch of synthetic input that is already
 resident in HBM (outputs come from torch's caching allocator inside the timed region).  The default
@@ -277,6 +277,25 @@ class AlifFused(Alif):
         return spk, g_x
 
 
+class AlifFusedLean(Alif):
+    name = 'ALIF fwd+bwd, fused kernels without the current trace (no decay gradients)'
+    ops = [('alif_fwd', 'stream_kernel<AlifFwd>', 16), ('alif_bwd', 'stream_kernel<AlifBwd>', 16)]
+
+    def __init__(self, dev):
+        super().__init__(dev)
+        from lava_dl_amd.slayer.neuron.dynamics import alif_fused
+        self.F = alif_fused
+
+    def step(self, t):
+        with t('alif_fwd'):
+            _, vol, theta, spk, _, _ = self.F._fwd(
+                self.x, (self.d_i, self.d_v, self.d_th, self.d_ref), (self.zero, self.zero, self.one, self.zero),
+                0.5, 1.0, 64, False, 1, True, True)
+        with t('alif_bwd'):
+            g_x = self.F._bwd(self.g, vol, theta, None, self.d_i, self.d_v, 1.0, 1.0, False, False)
+        return spk, g_x
+
+
 class Rf(Workload):
     name = 'Resonator (RF) dynamics fwd+bwd'
     shape = (64, 1024, 2000)
@@ -393,7 +412,7 @@ class Synapse(Workload):
         O.conv_bwd(O.shift(g_z, -c['delay'], 1), c['filt'], 1)
 
 
-WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fused_lean': CubaFusedLean, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'alif_fused': AlifFused, 'rf': Rf, 'rf_fused': RfFused, 'synapse': Synapse}
+WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fused_lean': CubaFusedLean, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'alif_fused': AlifFused, 'alif_fused_lean': AlifFusedLean, 'rf': Rf, 'rf_fused': RfFused, 'synapse': Synapse}
 
 
 def cpu_baseline(job, budget_s=20.0):

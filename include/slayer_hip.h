@@ -292,9 +292,11 @@ int slayer_rf_bwd(float *g_re_in, float *g_im_in, float *grad_sin, float *grad_c
  * Spike.forward); bit-identical to that chain, 20 instead of 52 bytes per neuron-timestep.
  * theta_out receives threshold + refractory (what the spike compares against and what the backward pass
  * needs); th_last_out / ref_last_out ([M], both or neither NULL) receive the threshold and refractory
- * values of the last step, i.e. threshold[..., -1] and refractory[..., -1] of the separate operator. */
+ * values of the last step, i.e. threshold[..., -1] and refractory[..., -1] of the separate operator.
+ * cur_out may be NULL when the current trace is not wanted (no decay gradient in the backward pass):
+ * 16 bytes per neuron-timestep; cur_last_out ([M], may be NULL) receives current[..., -1]. */
 int slayer_alif_fwd(float *cur_out, float *vol_out, float *theta_out, float *spk_out,
-                    float *th_last_out, float *ref_last_out, const float *in,
+                    float *cur_last_out, float *th_last_out, float *ref_last_out, const float *in,
                     const float *i_decay, const float *v_decay, const float *th_decay, const float *ref_decay,
                     const float *i_state, const float *v_state, const float *th_state, const float *ref_state,
                     int64_t th_step_scaled, int64_t th0_scaled, int graded, float spike_scale, int w_scale,
@@ -305,7 +307,8 @@ int slayer_alif_fwd(float *cur_out, float *vol_out, float *theta_out, float *spk
 
 /* Backward of the above = slayer_spike_bwd with a threshold tensor -> slayer_li_bwd twice, in one launch
  * (20 instead of 40 bytes per neuron-timestep); grad_in is bit-identical to the chain.  grad_i_decay /
- * grad_v_decay may both be NULL; workspace: 2*M + 64*(num_i_decays + num_v_decays) floats otherwise. */
+ * grad_v_decay may both be NULL (then current may be NULL too and is not read: 16 bytes per
+ * neuron-timestep); workspace: 2*M + 64*(num_i_decays + num_v_decays) floats otherwise. */
 int slayer_alif_bwd(float *grad_in, float *grad_i_decay, float *grad_v_decay,
                     const float *grad_spikes, const float *voltage, const float *theta, const float *current,
                     const float *i_decay, const float *v_decay,

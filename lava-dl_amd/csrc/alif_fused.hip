@@ -13,28 +13,31 @@ int launch_reduce_param_grad(float* grad, const float* partial, float* scratch, 
                              int64_t num_params, hipStream_t stream);   // li.hip
 int launch_zero_fill(float* p, int64_t n, hipStream_t stream);          // li.hip
 
-template <bool POW2, bool GRADED>
+// KEEP_CURRENT = false leaves the current trace out (a caller that wants no decay gradient does not
+// need it): 16 instead of 20 bytes per neuron-timestep.
+template <bool POW2, bool GRADED, bool KEEP_CURRENT>
 struct AlifFwd {
-    static constexpr int kIn = 1, kOut = 3;          // out: current, voltage, threshold + refractory
+    static constexpr int kIn = 1, kOut = KEEP_CURRENT ? 3 : 2;   // out: [current,] voltage, threshold + refractory
+    static constexpr int kVol = kOut - 2, kTheta = kOut - 1;
     static constexpr int kDerived = 1;               // spikes: a function of voltage and threshold + refractory
     static constexpr bool kReverse = false;
     static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
     struct Params {
         const float* in[1];
-        float* out[4];
-        float *th_last, *ref_last;                   // [M] threshold / refractory of the last step, or nullptr
+        float* out[kOut + 1];
+        float *cur_last, *th_last, *ref_last;        // [M] values of the last step, or nullptr
         const float *i_decay, *v_decay, *th_decay, *ref_decay, *i_state, *v_state, *th_state, *ref_state;
         int step, base;
         float w, inv_w, spike_scale;
         int64_t npb, n_id, n_vd, n_td, n_rd, n_is, n_vs, n_ts, n_rs;
     };
     int yc, yv, th, r, mi, mv, mt, mr, th_step, base;
-    float w, inv_w, spike_scale, th_f, ref_f;
+    float w, inv_w, spike_scale, th_f, ref_f, cur_f;
 
     __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
         w = p.w; inv_w = p.inv_w; spike_scale = p.spike_scale; th_step = p.step; base = p.base;
         yc = yv = th = r = mi = mv = mt = mr = 0;
-        th_f = ref_f = 0.f;
+        th_f = ref_f = cur_f = 0.f;
         if (valid) {
             yc = trunc_i32(p.i_state[p.n_is == 1 ? 0 : m] * w);
             yv = trunc_i32(p.v_state[p.n_vs == 1 ? 0 : m] * w);
@@ -46,7 +49,7 @@ struct AlifFwd {
             mr = 4096 - trunc_i32(p.ref_decay[param_index(m, p.npb, p.n_rd)]);
         }
     }
-    __device__ __forceinline__ void step(const float (&x)[1], float (&o)[3]) {
+    __device__ __forceinline__ void step(const float (&x)[1], float (&o)[kOut]) {
         yc = rs0_12(yc, mi) + trunc_i32(w * x[0]);
         const float cf = (float)yc;
         const float cur = POW2 ? cf * inv_w : cf / w;
@@ -61,30 +64,33 @@ struct AlifFwd {
         const bool fired = trunc_i32(w * vol) >= th + r;        // the threshold op reads the float32 voltage
         r += fired ? 2 * th : 0;
         th += fired ? th_step : 0;
-        o[0] = cur;
-        o[1] = vol;
-        o[2] = th_f + ref_f;
+        if (KEEP_CURRENT) o[0] = cur;
+        cur_f = cur;
+        o[kVol] = vol;
+        o[kTheta] = th_f + ref_f;
     }
     __device__ __forceinline__ float spike(float vol, float theta) const {
         const float h = (vol >= theta) ? 1.0f : 0.0f;
         return GRADED ? (h * vol) / spike_scale : h;
     }
-    __device__ __forceinline__ float4 derive(const float4 (&y)[3]) const {
-        return make_float4(spike(y[1].x, y[2].x), spike(y[1].y, y[2].y), spike(y[1].z, y[2].z),
-                           spike(y[1].w, y[2].w));
+    __device__ __forceinline__ float4 derive(const float4 (&y)[kOut]) const {
+        return make_float4(spike(y[kVol].x, y[kTheta].x), spike(y[kVol].y, y[kTheta].y),
+                           spike(y[kVol].z, y[kTheta].z), spike(y[kVol].w, y[kTheta].w));
     }
     __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
         if (valid && p.th_last) { p.th_last[m] = th_f; p.ref_last[m] = ref_f; }
+        if (valid && p.cur_last) p.cur_last[m] = cur_f;
     }
 };
 
-template <bool GRADED>
+// DECAY_GRAD = false drops the saved current and both decay-gradient sums (16 instead of 20 bytes).
+template <bool GRADED, bool DECAY_GRAD>
 struct AlifBwd {
-    static constexpr int kIn = 4, kOut = 1;          // in: grad of spikes, saved voltage, threshold + refractory, current
+    static constexpr int kIn = DECAY_GRAD ? 4 : 3, kOut = 1;   // in: grad of spikes, voltage, threshold + refractory[, current]
     static constexpr bool kReverse = true;
     static constexpr int64_t kRows32Below = 4096, kRows16Below = 4096;     // exp per step: keep all lanes busy
     struct Params {
-        const float* in[4];
+        const float* in[kIn];
         float* out[1];
         const float *i_decay, *v_decay;
         float *partial_i, *partial_v;                // per-neuron decay gradients, or nullptr
@@ -102,17 +108,19 @@ struct AlifBwd {
             av = 1.0f - p.v_decay[param_index(m, p.npb, p.n_vd)] / 4096.0f;
         }
     }
-    __device__ __forceinline__ void step(const float (&x)[4], float (&o)[1]) {
+    __device__ __forceinline__ void step(const float (&x)[kIn], float (&o)[1]) {
         const float d = x[1] - x[2];
         const float gv = GRADED ? (rho * expf(fminf(d, 0.0f) / tau)) * x[0] : (lead * expf(-fabsf(d) / tau)) * x[0];
-        acc_v = __fmaf_rn(gc, x[1], acc_v);          // gc, gx still hold the gradients of step t+1
-        acc_i = __fmaf_rn(gx, x[3], acc_i);
+        if (DECAY_GRAD) {
+            acc_v = __fmaf_rn(gc, x[1], acc_v);      // gc, gx still hold the gradients of step t+1
+            acc_i = __fmaf_rn(gx, x[kIn - 1], acc_i);
+        }
         gc = av * gc + gv;
         gx = ai * gx + gc;
         o[0] = gx;
     }
     __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
-        if (valid && p.partial_i) { p.partial_i[m] = acc_i; p.partial_v[m] = acc_v; }
+        if (DECAY_GRAD && valid && p.partial_i) { p.partial_i[m] = acc_i; p.partial_v[m] = acc_v; }
     }
 };
 
@@ -121,7 +129,7 @@ struct AlifBwd {
 using namespace slayer;
 
 extern "C" int slayer_alif_fwd(float* cur_out, float* vol_out, float* theta_out, float* spk_out,
-                               float* th_last_out, float* ref_last_out, const float* in,
+                               float* cur_last_out, float* th_last_out, float* ref_last_out, const float* in,
                                const float* i_decay, const float* v_decay, const float* th_decay, const float* ref_decay,
                                const float* i_state, const float* v_state, const float* th_state, const float* ref_state,
                                int64_t th_step_scaled, int64_t th0_scaled, int graded, float spike_scale, int w_scale,
@@ -131,7 +139,7 @@ extern "C" int slayer_alif_fwd(float* cur_out, float* vol_out, float* theta_out,
                                int64_t T, void* stream) {
     if (int e = check_rows(M, T)) return e;
     if (M == 0 || T == 0) return 0;
-    if (!cur_out || !vol_out || !theta_out || !spk_out || !in || !i_decay || !v_decay || !th_decay || !ref_decay ||
+    if (!vol_out || !theta_out || !spk_out || !in || !i_decay || !v_decay || !th_decay || !ref_decay ||
         !i_state || !v_state || !th_state || !ref_state)
         return SLAYER_ENULL;
     if ((th_last_out == nullptr) != (ref_last_out == nullptr)) return SLAYER_ENULL;
@@ -144,19 +152,24 @@ extern "C" int slayer_alif_fwd(float* cur_out, float* vol_out, float* theta_out,
     if (th_step_scaled > lim || th_step_scaled < -lim || th0_scaled > lim || th0_scaled < -lim) return SLAYER_ERANGE;
     const float w = (float)w_scale;
     hipStream_t st = (hipStream_t)stream;
+#define SLAYER_ALIF_ARGS cur_last_out, th_last_out, ref_last_out, i_decay, v_decay, th_decay, ref_decay, i_state,       \
+                         v_state, th_state, ref_state, (int)th_step_scaled, (int)th0_scaled, w, 1.0f / w,         \
+                         spike_scale, neurons_per_batch, num_i_decays, num_v_decays, num_th_decays,               \
+                         num_ref_decays, num_i_states, num_v_states, num_th_states, num_ref_states
 #define SLAYER_ALIF(P, G)                                                                                         \
     do {                                                                                                          \
-        AlifFwd<P, G>::Params p{{in}, {cur_out, vol_out, theta_out, spk_out}, th_last_out, ref_last_out,            \
-                                i_decay, v_decay, th_decay, ref_decay, i_state, v_state, th_state, ref_state,       \
-                                (int)th_step_scaled, (int)th0_scaled, w, 1.0f / w, spike_scale, neurons_per_batch,  \
-                                num_i_decays, num_v_decays, num_th_decays, num_ref_decays,                          \
-                                num_i_states, num_v_states, num_th_states, num_ref_states};                         \
-        return launch_stream<AlifFwd<P, G>>(p, M, T, st);                                                           \
+        if (cur_out) {                                                                                            \
+            AlifFwd<P, G, true>::Params p{{in}, {cur_out, vol_out, theta_out, spk_out}, SLAYER_ALIF_ARGS};          \
+            return launch_stream<AlifFwd<P, G, true>>(p, M, T, st);                                               \
+        }                                                                                                         \
+        AlifFwd<P, G, false>::Params p{{in}, {vol_out, theta_out, spk_out}, SLAYER_ALIF_ARGS};                      \
+        return launch_stream<AlifFwd<P, G, false>>(p, M, T, st);                                                  \
     } while (0)
     if (is_pow2(w_scale)) { if (graded) SLAYER_ALIF(true, true); else SLAYER_ALIF(true, false); }
     if (graded) SLAYER_ALIF(false, true);
     SLAYER_ALIF(false, false);
 #undef SLAYER_ALIF
+#undef SLAYER_ALIF_ARGS
 }
 
 extern "C" int slayer_alif_bwd(float* grad_in, float* grad_i_decay, float* grad_v_decay,
@@ -174,18 +187,24 @@ extern "C" int slayer_alif_bwd(float* grad_in, float* grad_i_decay, float* grad_
     if (want && !workspace && M > 0) return SLAYER_ENULL;
     hipStream_t st = (hipStream_t)stream;
     if (M > 0 && T > 0) {
-        if (!grad_in || !grad_spikes || !voltage || !theta || !current || !i_decay || !v_decay) return SLAYER_ENULL;
-        if (graded) {
-            AlifBwd<true>::Params p{{grad_spikes, voltage, theta, current}, {grad_in}, i_decay, v_decay,
-                                    want ? workspace : nullptr, want ? workspace + M : nullptr,
-                                    tau_rho, scale_rho, neurons_per_batch, num_i_decays, num_v_decays};
-            if (int e = launch_stream<AlifBwd<true>>(p, M, T, st)) return e;
-        } else {
-            AlifBwd<false>::Params p{{grad_spikes, voltage, theta, current}, {grad_in}, i_decay, v_decay,
-                                     want ? workspace : nullptr, want ? workspace + M : nullptr,
-                                     tau_rho, scale_rho, neurons_per_batch, num_i_decays, num_v_decays};
-            if (int e = launch_stream<AlifBwd<false>>(p, M, T, st)) return e;
-        }
+        if (!grad_in || !grad_spikes || !voltage || !theta || !i_decay || !v_decay || (want && !current))
+            return SLAYER_ENULL;
+#define SLAYER_ALIF_BWD(G)                                                                                        \
+    do {                                                                                                          \
+        if (want) {                                                                                               \
+            AlifBwd<G, true>::Params p{{grad_spikes, voltage, theta, current}, {grad_in}, i_decay, v_decay,         \
+                                       workspace, workspace + M, tau_rho, scale_rho, neurons_per_batch,           \
+                                       num_i_decays, num_v_decays};                                               \
+            if (int e = launch_stream<AlifBwd<G, true>>(p, M, T, st)) return e;                                   \
+        } else {                                                                                                  \
+            AlifBwd<G, false>::Params p{{grad_spikes, voltage, theta}, {grad_in}, i_decay, v_decay, nullptr,        \
+                                        nullptr, tau_rho, scale_rho, neurons_per_batch, num_i_decays,             \
+                                        num_v_decays};                                                            \
+            if (int e = launch_stream<AlifBwd<G, false>>(p, M, T, st)) return e;                                  \
+        }                                                                                                         \
+    } while (0)
+        if (graded) SLAYER_ALIF_BWD(true); else SLAYER_ALIF_BWD(false);
+#undef SLAYER_ALIF_BWD
     }
     if (want) {
         if (M == 0 || T == 0) {

@@ -74,11 +74,13 @@ class Neuron(_Base):
             input, self._q('current_decay'), self._q('voltage_decay'), self._q('threshold_decay'),
             self._q('refractory_decay'), self.current_state, self.voltage_state, self.threshold_state,
             self.refractory_state, self.threshold_step, self.threshold, self.s_scale,
-            self.tau_rho * TAU_RHO_MULT, self.scale_rho * SCALE_RHO_MULT, self.graded_spike, 1)
+            self.tau_rho * TAU_RHO_MULT, self.scale_rho * SCALE_RHO_MULT, self.graded_spike, 1,
+            keep_current=self.requires_grad)
         if self.persistent_state:
             with torch.no_grad():
                 last = spike[..., -1]
-                self.current_state = current[..., -1].clone()
+                # without trainable decays the kernel skips the current trace and returns its last step
+                self.current_state = (current[..., -1] if self.requires_grad else current).clone()
                 self.voltage_state = voltage[..., -1].clone()
                 self.refractory_state = adaptive_threshold.persistent_ref_state(ref_last, last, th_last).detach().clone()
                 self.threshold_state = adaptive_threshold.persistent_th_state(

@@ -12,19 +12,26 @@ from ... import _native as N
 
 def dynamics(input, current_decay, voltage_decay, threshold_decay, refractory_decay,
              current_state, voltage_state, threshold_state, refractory_state,
-             threshold_step, threshold_base, w_scale, tau_rho, scale_rho, graded_spike=False, spike_scale=1):
+             threshold_step, threshold_base, w_scale, tau_rho, scale_rho, graded_spike=False, spike_scale=1,
+             keep_current=True):
     """(current, voltage, theta, spike, threshold_last, refractory_last) of an ALIF neuron, where
     ``theta = threshold + refractory`` is what the spike compares the voltage against and the two
     ``*_last`` tensors (shaped like the states) are the threshold and refractory values of the last
     step.  Gradients flow from ``spike`` to ``input`` and to the current / voltage decays (the
-    threshold dynamics has none, as in the separate operator); the other outputs are detached."""
+    threshold dynamics has none, as in the separate operator); the other outputs are detached.
+    With ``keep_current=False`` and decays that do not require a gradient the current trace is neither
+    written nor read back and ``current`` holds only the last step, shaped like the states."""
+    lean = not keep_current and not (current_decay.requires_grad or voltage_decay.requires_grad)
     return _AlifFused.apply(input, current_decay, voltage_decay, threshold_decay, refractory_decay,
                             current_state, voltage_state, threshold_state, refractory_state,
-                            threshold_step, threshold_base, w_scale, tau_rho, scale_rho, graded_spike, spike_scale)
+                            threshold_step, threshold_base, w_scale, tau_rho, scale_rho, graded_spike, spike_scale,
+                            lean)
 
 
-def _fwd(input, decays, states, threshold_step, threshold_base, w_scale, graded, spike_scale, want_last=True):
-    """decays = (current, voltage, threshold, refractory), states likewise."""
+def _fwd(input, decays, states, threshold_step, threshold_base, w_scale, graded, spike_scale, want_last=True,
+         lean=False):
+    """decays = (current, voltage, threshold, refractory), states likewise.  lean: no current trace,
+    the first result is then current[..., -1]."""
     dev = N.require_gpu(input, *decays, *states)
     input = input.contiguous()
     decays = [d.contiguous() for d in decays]
@@ -33,23 +40,29 @@ def _fwd(input, decays, states, threshold_step, threshold_base, w_scale, graded,
     for name, s in zip(('current_state', 'voltage_state', 'threshold_state', 'refractory_state'), states):
         if s.numel() not in (1, M):
             raise RuntimeError(f'{name} has {s.numel()} elements, expected 1 or {M}')
-    cur, vol, theta, spk = (torch.empty_like(input) for _ in range(4))
+    vol, theta, spk = (torch.empty_like(input) for _ in range(3))
+    cur = None if lean else torch.empty_like(input)
+    cur_last = torch.empty(input.shape[:-1], dtype=input.dtype, device=dev) if lean else None
     th_last = ref_last = None
     if want_last:
         th_last = torch.empty(input.shape[:-1], dtype=input.dtype, device=dev)
         ref_last = torch.empty(input.shape[:-1], dtype=input.dtype, device=dev)
     with torch.cuda.device(dev):
         N.check(N.lib().slayer_alif_fwd(
-            N.ptr(cur), N.ptr(vol), N.ptr(theta), N.ptr(spk), N.ptr(th_last), N.ptr(ref_last), N.ptr(input),
+            N.ptr(cur), N.ptr(vol), N.ptr(theta), N.ptr(spk), N.ptr(cur_last), N.ptr(th_last), N.ptr(ref_last),
+            N.ptr(input),
             *[N.ptr(d) for d in decays], *[N.ptr(s) for s in states],
             int(threshold_step * w_scale), int(threshold_base * w_scale), 1 if graded else 0, float(spike_scale),
             int(w_scale), M, N.neurons_per_batch(input), *[d.numel() for d in decays],
             *[s.numel() for s in states], T, N.stream_handle()))
-    return cur, vol, theta, spk, th_last, ref_last
+    return (cur_last if lean else cur), vol, theta, spk, th_last, ref_last
 
 
 def _bwd(grad_spikes, vol, theta, cur, i_decay, v_decay, tau_rho, scale_rho, graded, need_decay_grad=True):
-    dev = N.require_gpu(grad_spikes, vol, theta, cur, i_decay, v_decay)
+    dev = N.require_gpu(grad_spikes, vol, theta, i_decay, v_decay) if cur is None else \
+        N.require_gpu(grad_spikes, vol, theta, cur, i_decay, v_decay)
+    if cur is None and need_decay_grad:
+        raise RuntimeError('the decay gradients need the current trace')
     grad_spikes, i_decay, v_decay = grad_spikes.contiguous(), i_decay.contiguous(), v_decay.contiguous()
     M, T = N.rows_and_steps(grad_spikes)
     grad_input = torch.empty_like(grad_spikes)
@@ -69,13 +82,13 @@ def _bwd(grad_spikes, vol, theta, cur, i_decay, v_decay, tau_rho, scale_rho, gra
 class _AlifFused(torch.autograd.Function):
     @staticmethod
     def forward(ctx, input, i_decay, v_decay, th_decay, ref_decay, i_state, v_state, th_state, ref_state,
-                threshold_step, threshold_base, w_scale, tau_rho, scale_rho, graded, spike_scale):
+                threshold_step, threshold_base, w_scale, tau_rho, scale_rho, graded, spike_scale, lean):
         graded = graded is True
         outs = _fwd(input, [d.detach() for d in (i_decay, v_decay, th_decay, ref_decay)],
                     [s.detach() for s in (i_state, v_state, th_state, ref_state)],
-                    threshold_step, threshold_base, w_scale, graded, spike_scale)
+                    threshold_step, threshold_base, w_scale, graded, spike_scale, True, lean)
         cur, vol, theta, spk, th_last, ref_last = outs
-        ctx.save_for_backward(cur, vol, theta, i_decay, v_decay)
+        ctx.save_for_backward(None if lean else cur, vol, theta, i_decay, v_decay)
         ctx.cfg = (float(tau_rho), float(scale_rho), graded)
         ctx.mark_non_differentiable(cur, vol, theta, th_last, ref_last)
         return outs
@@ -84,9 +97,9 @@ class _AlifFused(torch.autograd.Function):
     def backward(ctx, _g_cur, _g_vol, _g_theta, grad_spikes, _g_th, _g_ref):
         cur, vol, theta, i_decay, v_decay = ctx.saved_tensors
         tau_rho, scale_rho, graded = ctx.cfg
-        need = ctx.needs_input_grad[1] or ctx.needs_input_grad[2]
+        need = (ctx.needs_input_grad[1] or ctx.needs_input_grad[2]) and cur is not None
         g_in, g_i, g_v = _bwd(grad_spikes, vol, theta, cur, i_decay.detach(), v_decay.detach(),
                               tau_rho, scale_rho, graded, need)
         if g_i is not None:
             g_i, g_v = g_i.reshape(i_decay.shape), g_v.reshape(v_decay.shape)
-        return (g_in, g_i, g_v) + (None,) * 13
+        return (g_in, g_i, g_v) + (None,) * 14

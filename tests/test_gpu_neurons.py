@@ -359,3 +359,26 @@ def test_fused_cuba_without_current_trace(slayer, shape, w):
     c3, _, s3 = F.dynamics(x, dd, d_v, s_i, s_v, w, 1.0, 0.7, 1.5, keep_current=False)
     s3.backward(g)
     assert c3.shape == shape and dd.grad is not None and torch.isfinite(dd.grad).all()
+
+
+@pytest.mark.parametrize('shape,w', [((4, 128, 200), 64), ((3, 70, 129), 100)])
+def test_fused_alif_without_current_trace(slayer, shape, w):
+    from tests.util import seed_of
+    gen = torch.Generator().manual_seed(seed_of(shape, w, 'lean alif'))
+    C = shape[1]
+    x = sparse_input(gen, shape, p=0.3, amp=2.0).to(dev())
+    g = torch.randn(shape, generator=gen).to(dev())
+    decays = [torch.randint(0, 4096, (C,), generator=gen).float().to(dev()) for _ in range(4)]
+    states = [torch.rand(shape[:-1], generator=gen).to(dev()) for _ in range(4)]
+    states[2] = states[2] + 1.0
+    F = slayer.neuron.dynamics.alif_fused
+    a, b = x.clone().requires_grad_(), x.clone().requires_grad_()
+    full = F.dynamics(a, *decays, *states, 0.5, 1.0, w, 0.7, 1.5)
+    full[3].backward(g)
+    lean = F.dynamics(b, *decays, *states, 0.5, 1.0, w, 0.7, 1.5, keep_current=False)
+    lean[3].backward(g)
+    assert lean[0].shape == shape[:-1] and torch.equal(lean[0], full[0][..., -1])
+    for i in (1, 2, 4, 5):
+        assert torch.equal(lean[i], full[i]), f'output {i} differs'
+    assert torch.equal(lean[3].detach(), full[3].detach()) and float(full[3].detach().sum()) > 0
+    assert torch.equal(b.grad, a.grad)
