@@ -1,6 +1,6 @@
 """Benchmark of the SLAYER neuron-dynamics hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cuba|cuba_fused|cuba_fused_lean|cuba_fwd_small|alif|alif_fused|alif_fused_lean|rf|rf_fused|synapse]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cuba|cuba_fused|cuba_fused_lean|cuba_inference|cuba_fwd_small|alif|alif_fused|alif_fused_lean|rf|rf_fused|synapse]
 
 A step is one pass of the workload's op sequence over one batch of synthetic input that is already
 resident in HBM (outputs come from torch's caching allocator inside the timed region).  The default
@@ -183,6 +183,21 @@ class CubaFusedLean(Cuba):
         with t('cuba_bwd'):
             g_x, _, _ = self.F._bwd(self.g, vol, None, self.d_i, self.d_v, self.thr, 1.0, 1.0, False, False)
         return spk, g_x
+
+
+class CubaInference(Cuba):
+    name = 'CUBA neuron forward, spikes only (inference)'
+    ops = [('cuba_fwd', 'stream_kernel<CubaFwd>', 8)]
+
+    def __init__(self, dev):
+        super().__init__(dev)
+        from lava_dl_amd.slayer.neuron.dynamics import cuba_fused
+        self.F = cuba_fused
+
+    def step(self, t):
+        with t('cuba_fwd'):
+            out = self.F._fwd(self.x, self.d_i, self.d_v, self.zero, self.zero, self.w, self.thr, False, 1, True, True)
+        return out
 
 
 class CubaFwdSmall(Workload):
@@ -412,7 +427,7 @@ class Synapse(Workload):
         O.conv_bwd(O.shift(g_z, -c['delay'], 1), c['filt'], 1)
 
 
-WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fused_lean': CubaFusedLean, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'alif_fused': AlifFused, 'alif_fused_lean': AlifFusedLean, 'rf': Rf, 'rf_fused': RfFused, 'synapse': Synapse}
+WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fused_lean': CubaFusedLean, 'cuba_inference': CubaInference, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'alif_fused': AlifFused, 'alif_fused_lean': AlifFusedLean, 'rf': Rf, 'rf_fused': RfFused, 'synapse': Synapse}
 
 
 def cpu_baseline(job, budget_s=20.0):

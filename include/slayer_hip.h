@@ -242,9 +242,12 @@ int slayer_cumsum(float *out, const float *in, const float *state, int64_t num_s
  * thr_scaled = (threshold + eps) * w_scale for the reset (double, <= 0 disables it),
  * spike_threshold = threshold + eps for the spike compare on the float32 voltage.
  * cur_out may be NULL when the current trace is not wanted (no decay gradient in the backward pass):
- * 12 bytes per neuron-timestep.  cur_last_out ([M], may be NULL) receives the current of the last
- * step, i.e. current[..., -1], which is what a persistent state needs. */
-int slayer_cuba_fwd(float *cur_out, float *vol_out, float *spk_out, float *cur_last_out, const float *in,
+ * 12 bytes per neuron-timestep; vol_out may be NULL as well when no backward pass will follow
+ * (inference): 8 bytes.  cur_last_out / vol_last_out ([M], may be NULL) receive the current and the
+ * voltage of the last step, i.e. current[..., -1] and voltage[..., -1], which is what a persistent
+ * state needs. */
+int slayer_cuba_fwd(float *cur_out, float *vol_out, float *spk_out, float *cur_last_out, float *vol_last_out,
+                    const float *in,
                     const float *i_decay, const float *v_decay,
                     const float *i_state, const float *v_state,
                     double thr_scaled, float spike_threshold, int graded, float spike_scale, int w_scale,

@@ -25,17 +25,18 @@ struct CubaFwd {
     struct Params {
         const float* in[1];
         float* out[kOut + 1];
-        float* cur_last;                             // [M] current of the last step, or nullptr
+        float *cur_last, *vol_last;                  // [M] current / voltage of the last step, or nullptr
         const float *i_decay, *v_decay, *i_state, *v_state;
         float w, inv_w, spike_thr, spike_scale;
         int fire_above;                              // voltage reset when the state exceeds this
         int64_t npb, n_id, n_vd, n_is, n_vs;
     };
     static constexpr bool kTransforms = true;        // integer tiles, see to_state / from_state
-    int yc, yv, mi, mv, fire_above;
+    int yc, yv, yv_out, mi, mv, fire_above;
     float w, inv_w, spike_thr, spike_scale;
 
     __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
+        yv_out = 0;
         w = p.w; inv_w = p.inv_w; fire_above = p.fire_above; spike_thr = p.spike_thr; spike_scale = p.spike_scale;
         yc = yv = mi = mv = 0;
         if (valid) {
@@ -57,6 +58,7 @@ struct CubaFwd {
         const float cf = (float)yc;
         const int yn = rs0_12(yv, mv) + (POW2 ? trunc_i32(cf) : trunc_i32(w * (cf / w)));
         yv = (yn > fire_above) ? 0 : yn;             // float(yn) >= threshold, decided on the integer
+        yv_out = yn;
         if (KEEP_CURRENT) o[0] = __int_as_float(yc);
         o[kVol] = __int_as_float(yn);
     }
@@ -69,6 +71,7 @@ struct CubaFwd {
     }
     __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
         if (valid && p.cur_last) p.cur_last[m] = from_state<POW2>(__int_as_float(yc), w, inv_w);
+        if (valid && p.vol_last) p.vol_last[m] = from_state<POW2>(__int_as_float(yv_out), w, inv_w);
     }
 };
 
@@ -118,7 +121,8 @@ struct CubaBwd {
 
 using namespace slayer;
 
-extern "C" int slayer_cuba_fwd(float* cur_out, float* vol_out, float* spk_out, float* cur_last_out, const float* in,
+extern "C" int slayer_cuba_fwd(float* cur_out, float* vol_out, float* spk_out, float* cur_last_out,
+                               float* vol_last_out, const float* in,
                                const float* i_decay, const float* v_decay,
                                const float* i_state, const float* v_state,
                                double thr_scaled, float spike_threshold, int graded, float spike_scale, int w_scale,
@@ -126,7 +130,7 @@ extern "C" int slayer_cuba_fwd(float* cur_out, float* vol_out, float* spk_out, f
                                int64_t num_i_states, int64_t num_v_states, int64_t T, void* stream) {
     if (int e = check_rows(M, T)) return e;
     if (M == 0 || T == 0) return 0;
-    if (!vol_out || !spk_out || !in || !i_decay || !v_decay || !i_state || !v_state) return SLAYER_ENULL;
+    if (!spk_out || !in || !i_decay || !v_decay || !i_state || !v_state) return SLAYER_ENULL;
     if (int e = check_params(M, neurons_per_batch, num_i_decays)) return e;
     if (int e = check_params(M, neurons_per_batch, num_v_decays)) return e;
     if (int e = check_states(M, num_i_states)) return e;
@@ -138,14 +142,15 @@ extern "C" int slayer_cuba_fwd(float* cur_out, float* vol_out, float* spk_out, f
 #define SLAYER_CUBA(P, G)                                                                                        \
     do {                                                                                                         \
         if (cur_out) {                                                                                           \
-            CubaFwd<P, G, true>::Params p{{in}, {cur_out, vol_out, spk_out}, cur_last_out, i_decay, v_decay,      \
-                                          i_state, v_state, w, 1.0f / w, spike_threshold, spike_scale, fa,       \
+            CubaFwd<P, G, true>::Params p{{in}, {cur_out, vol_out, spk_out}, cur_last_out, vol_last_out, i_decay,    \
+                                          v_decay, i_state, v_state, w, 1.0f / w, spike_threshold, spike_scale,  \
+                                          fa,                                                                    \
                                           neurons_per_batch, num_i_decays, num_v_decays, num_i_states,           \
                                           num_v_states};                                                         \
             return launch_stream<CubaFwd<P, G, true>>(p, M, T, st);                                              \
         }                                                                                                        \
-        CubaFwd<P, G, false>::Params p{{in}, {vol_out, spk_out}, cur_last_out, i_decay, v_decay, i_state,         \
-                                       v_state, w, 1.0f / w, spike_threshold, spike_scale, fa,                   \
+        CubaFwd<P, G, false>::Params p{{in}, {vol_out, spk_out}, cur_last_out, vol_last_out, i_decay, v_decay,    \
+                                       i_state, v_state, w, 1.0f / w, spike_threshold, spike_scale, fa,          \
                                        neurons_per_batch, num_i_decays, num_v_decays, num_i_states,              \
                                        num_v_states};                                                            \
         return launch_stream<CubaFwd<P, G, false>>(p, M, T, st);                                                 \

@@ -118,7 +118,7 @@ struct TileGeom {
 //     the same step: it is computed while a quad is copied out and needs neither an LDS tile nor
 //     boundary registers
 //   static constexpr int64_t kRows32Below, kRows16Below;   (rows-per-wave policy, see launch_stream)
-//   struct Params { const float* in[kIn]; float* out[kOut]; ... };
+//   struct Params { const float* in[kIn]; float* out[kOut]; ... };   (a null out[] entry is not stored)
 //   __device__ void init(const Params&, int64_t m, bool valid);
 //   __device__ void step(const float (&x)[kIn], float (&y)[kOut]);
 //   __device__ void finish(const Params&, int64_t m, bool valid);
@@ -205,7 +205,8 @@ struct Copier {
 #pragma unroll
         for (int i = 0; i < NI; ++i) src[i] = make_rsrc(prm.in[i] + m0 * (int64_t)T, wave_bytes);
 #pragma unroll
-        for (int o = 0; o < NO + ND; ++o) dst[o] = make_rsrc(prm.out[o] + m0 * (int64_t)T, wave_bytes);
+        for (int o = 0; o < NO + ND; ++o)    // an output the caller does not want: every store falls out of range
+            dst[o] = prm.out[o] ? make_rsrc(prm.out[o] + m0 * (int64_t)T, wave_bytes) : make_rsrc(nullptr, 0);
         crow = lane / G::kQuads;                // row within a pass
         cq = lane % G::kQuads;                  // quad within the row
         // chunks [1, interior_end) hold only valid columns and touch no shared line, for every phase
@@ -575,7 +576,7 @@ __global__ __launch_bounds__(kWave) void stream_kernel_scalar(typename Op::Param
             if constexpr (ND == 1) v[NO] = op.derive(y);
 #pragma unroll
             for (int o = 0; o < NO + ND; ++o) {
-                if (r < rows) {
+                if (r < rows && prm.out[o]) {
                     float* d = prm.out[o] + off;
                     if (t + 0 < T) d[0] = v[o].x;
                     if (t + 1 < T) d[1] = v[o].y;

@@ -45,7 +45,7 @@ _SIGNATURES = {
     'slayer_delta_fwd': (_INT, [_P] * 9 + [_INT, _F] + [_I64] * 7 + [_P]),
     'slayer_delta_bwd': (_INT, [_P] * 6 + [_F, _F] + [_I64] * 4 + [_P]),
     'slayer_cumsum': (_INT, [_P, _P, _P, _I64, _INT, _I64, _I64, _P]),
-    'slayer_cuba_fwd': (_INT, [_P] * 9 + [_D, _F, _INT, _F, _INT] + [_I64] * 7 + [_P]),
+    'slayer_cuba_fwd': (_INT, [_P] * 10 + [_D, _F, _INT, _F, _INT] + [_I64] * 7 + [_P]),
     'slayer_cuba_bwd': (_INT, [_P] * 8 + [_F, _F, _F, _INT, _P] + [_I64] * 5 + [_P]),
     'slayer_rf_fwd': (_INT, [_P] * 10 + [_F, _INT, _F, _INT] + [_I64] * 7 + [_P]),
     'slayer_rf_bwd': (_INT, [_P] * 9 + [_F, _F, _F, _INT, _P] + [_I64] * 4 + [_P]),

@@ -59,17 +59,24 @@ class Neuron(_Base):
             _, voltage = self.dynamics(input)
             return self.spike(voltage)
         self._prepare(input)
-        current, voltage, spike = cuba_fused.dynamics(
-            input, self._q('current_decay'), self._q('voltage_decay'),
-            self.current_state.contiguous(), self.voltage_state.contiguous(), self.s_scale,
-            self.threshold + self.threshold_eps, self.tau_rho * TAU_RHO_MULT, self.scale_rho * SCALE_RHO_MULT,
-            self.graded_spike, 1, keep_current=self.requires_grad)
+        args = (input, self._q('current_decay'), self._q('voltage_decay'),
+                self.current_state.contiguous(), self.voltage_state.contiguous(), self.s_scale,
+                self.threshold + self.threshold_eps)
+        if not (torch.is_grad_enabled() and (input.requires_grad or self.requires_grad)):
+            # nothing to differentiate: only the spikes are written, the last current / voltage come per neuron
+            current_last, voltage_last, spike = cuba_fused.spikes(*args, self.graded_spike, 1)
+        else:
+            # without trainable decays the kernel skips the current trace and returns its last step
+            current, voltage, spike = cuba_fused.dynamics(
+                *args, self.tau_rho * TAU_RHO_MULT, self.scale_rho * SCALE_RHO_MULT, self.graded_spike, 1,
+                keep_current=self.requires_grad)
+            current_last = current[..., -1] if self.requires_grad else current
+            voltage_last = voltage[..., -1]
         if self.persistent_state:
             with torch.no_grad():
-                # without trainable decays the kernel skips the current trace and returns its last step
-                self.current_state = (current[..., -1] if self.requires_grad else current).clone()
+                self.current_state = current_last.clone()
                 self.voltage_state = leaky_integrator.persistent_state(
-                    voltage[..., -1], spike[..., -1]).detach().clone()
+                    voltage_last, spike[..., -1]).detach().clone()
         if self.drop is not None:
             spike = self.drop(spike)
         return spike

@@ -28,8 +28,19 @@ def dynamics(input, current_decay, voltage_decay, current_state, voltage_state, 
                             w_scale, threshold, tau_rho, scale_rho, graded_spike, spike_scale, lean)
 
 
-def _fwd(input, i_decay, v_decay, i_state, v_state, w_scale, threshold, graded, spike_scale, lean=False):
-    """lean: no current trace; the first result is then current[..., -1]."""
+def spikes(input, current_decay, voltage_decay, current_state, voltage_state, w_scale, threshold,
+           graded_spike=False, spike_scale=1):
+    """Inference form: (current_last, voltage_last, spike) with only the spikes written per step
+    (8 bytes per neuron-timestep); no gradient."""
+    with torch.no_grad():
+        return _fwd(input, current_decay, voltage_decay, current_state, voltage_state, w_scale, threshold,
+                    graded_spike is True, spike_scale, lean=True, spikes_only=True)
+
+
+def _fwd(input, i_decay, v_decay, i_state, v_state, w_scale, threshold, graded, spike_scale, lean=False,
+         spikes_only=False):
+    """lean: no current trace; the first result is then current[..., -1].  spikes_only (with lean):
+    no voltage trace either; the second result is then voltage[..., -1]."""
     dev = N.require_gpu(input, i_decay, v_decay, i_state, v_state)
     input, i_decay, v_decay = input.contiguous(), i_decay.contiguous(), v_decay.contiguous()
     i_state, v_state = i_state.contiguous(), v_state.contiguous()
@@ -37,17 +48,22 @@ def _fwd(input, i_decay, v_decay, i_state, v_state, w_scale, threshold, graded, 
     for name, s in (('current_state', i_state), ('voltage_state', v_state)):
         if s.numel() not in (1, M):
             raise RuntimeError(f'{name} has {s.numel()} elements, expected 1 or {M}')
-    vol, spk = torch.empty_like(input), torch.empty_like(input)
+    if spikes_only and not lean:
+        raise RuntimeError('spikes_only implies lean')
+    spk = torch.empty_like(input)
+    vol = None if spikes_only else torch.empty_like(input)
     cur = None if lean else torch.empty_like(input)
     cur_last = torch.empty(input.shape[:-1], dtype=input.dtype, device=dev) if lean else None
+    vol_last = torch.empty(input.shape[:-1], dtype=input.dtype, device=dev) if spikes_only else None
     with torch.cuda.device(dev):
         N.check(N.lib().slayer_cuba_fwd(
-            N.ptr(cur), N.ptr(vol), N.ptr(spk), N.ptr(cur_last), N.ptr(input), N.ptr(i_decay), N.ptr(v_decay),
+            N.ptr(cur), N.ptr(vol), N.ptr(spk), N.ptr(cur_last), N.ptr(vol_last), N.ptr(input),
+            N.ptr(i_decay), N.ptr(v_decay),
             N.ptr(i_state), N.ptr(v_state), float(threshold * w_scale), float(threshold),
             1 if graded else 0, float(spike_scale), int(w_scale),
             M, N.neurons_per_batch(input), i_decay.numel(), v_decay.numel(),
             i_state.numel(), v_state.numel(), T, N.stream_handle()))
-    return (cur_last if lean else cur), vol, spk
+    return (cur_last if lean else cur), (vol_last if spikes_only else vol), spk
 
 
 def _bwd(grad_spikes, vol, cur, i_decay, v_decay, threshold, tau_rho, scale_rho, graded, need_decay_grad=True):

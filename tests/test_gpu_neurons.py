@@ -382,3 +382,27 @@ def test_fused_alif_without_current_trace(slayer, shape, w):
         assert torch.equal(lean[i], full[i]), f'output {i} differs'
     assert torch.equal(lean[3].detach(), full[3].detach()) and float(full[3].detach().sum()) > 0
     assert torch.equal(b.grad, a.grad)
+
+
+@pytest.mark.parametrize('shared', [True, False])
+def test_cuba_neuron_inference_form_matches_training_form(slayer, shared):
+    """Under no_grad only the spikes are written; spikes and the carried states must equal the
+    training form over several calls with persistent state."""
+    gen = torch.Generator().manual_seed(107)
+    shape = (3, 12, 6, 152)
+    x = sparse_input(gen, shape, p=0.3, amp=1.5).to(dev())
+    mk = lambda: slayer.neuron.cuba.Neuron(1.0, [0.2, 0.4] if not shared else 0.25, [0.02, 0.2] if not shared else 0.03,
+                                           shared_param=shared, persistent_state=True).to(dev())
+    a, b = mk(), mk()
+    a._prepare(x); b._prepare(x)
+    for pa, pb in zip(a.parameters(), b.parameters()):
+        pb.data = pa.data.clone()
+    total = 0.0
+    for k in range(3):
+        sa = a(x.clone().requires_grad_())
+        with torch.no_grad():
+            sb = b(x)
+        assert torch.equal(sa.detach(), sb), f'call {k}: spikes differ'
+        assert torch.equal(a.current_state, b.current_state) and torch.equal(a.voltage_state, b.voltage_state)
+        total += float(sb.sum())
+    assert total > 0
