@@ -27,4 +27,7 @@ def quantize(input, step=1, mode=MODE.ROUND):
     """Quantise ``input`` to multiples of ``step`` (round or floor); gradients pass through."""
     if mode not in (MODE.ROUND, MODE.FLOOR):
         raise ValueError(f'{mode=} is not recognized.')
+    if not (torch.is_grad_enabled() and input.requires_grad):      # nothing to pass a gradient to
+        scaled = input / step
+        return (torch.floor(scaled) if mode == MODE.FLOOR else torch.round(scaled)) * step
     return _StraightThrough.apply(input, step, mode == MODE.FLOOR)
