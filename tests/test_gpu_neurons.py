@@ -406,3 +406,42 @@ def test_cuba_neuron_inference_form_matches_training_form(slayer, shared):
         assert torch.equal(a.current_state, b.current_state) and torch.equal(a.voltage_state, b.voltage_state)
         total += float(sb.sum())
     assert total > 0
+
+
+def test_fused_cuba_under_graph_capture_replays(slayer):
+    """The entry points enqueue kernels only (no memset nodes, no allocation of their own), so a step
+    can be captured in a graph; every replay, with eager work in between, must equal the eager result."""
+    gen = torch.Generator().manual_seed(108)
+    shape = (4, 16, 8, 96)
+    F = slayer.neuron.dynamics.cuba_fused
+    d_i, d_v = (torch.randint(0, 4096, (16,), generator=gen).float().to(dev()) for _ in range(2))
+    zero = torch.zeros(1, device=dev())
+    x = sparse_input(gen, shape, p=0.2, amp=1.5).to(dev())
+    g = torch.randn(shape, generator=gen).to(dev())
+
+    def step():
+        cur, vol, spk = F._fwd(x, d_i, d_v, zero, zero, 64, 1.0, False, 1)
+        g_x, g_i, g_v = F._bwd(g, vol, cur, d_i, d_v, 1.0, 1.0, 1.0, False)
+        return spk, g_x, g_i, g_v
+
+    step()                                      # warm-up outside the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        step()
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            outs = step()
+    torch.cuda.synchronize()
+    for k in range(4):
+        x.copy_(sparse_input(gen, shape, p=0.2, amp=1.5).to(dev()))
+        g.copy_(torch.randn(shape, generator=gen).to(dev()))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in outs]
+        want = step()                           # eager work between the replays
+        torch.cuda.synchronize()
+        assert float(want[0].sum()) > 0
+        for i, (a, b) in enumerate(zip(got, want)):
+            assert torch.equal(a, b), f'replay {k}: output {i} differs from the eager result'
