@@ -91,10 +91,10 @@ __device__ __forceinline__ int64_t param_index(int64_t m, int64_t npb, int64_t n
 // problems still spread over all compute units (lanes >= R only help with the copies).
 constexpr int kTileSamples = 2048;
 
-template <int R>
+template <int R, int S = kTileSamples>
 struct TileGeom {
     static constexpr int kRows = R;
-    static constexpr int kChunk = kTileSamples / R;          // TC: steps per chunk
+    static constexpr int kChunk = S / R;                     // TC: steps per chunk
     static_assert(R == 64 || R == 32 || R == 16, "rows per wave");
     static constexpr int kPitch = kChunk + 4;                // floats per LDS row
     static constexpr int kQuads = kChunk / 4;                // float4 per row
@@ -183,9 +183,9 @@ __device__ __forceinline__ void buf_store4(__amdgpu_buffer_rsrc_t r, int byte_of
 //
 // A wave can share the job with others: it then owns PASSES of the G::kPasses wave-wide accesses
 // that cover a tile, starting at pass first_pass.
-template <class Op, int R, bool STREAM, int PASSES = TileGeom<R>::kPasses>
+template <class Op, int R, bool STREAM, int PASSES = TileGeom<R>::kPasses, int S = kTileSamples>
 struct Copier {
-    using G = TileGeom<R>;
+    using G = TileGeom<R, S>;
     static constexpr int TC = G::kChunk, NI = Op::kIn, NO = Op::kOut, ND = DerivedCount<Op>::value;
     static constexpr int kPasses = PASSES;
     static_assert(ND == 0 || ND == 1, "at most one derived output");
@@ -342,10 +342,10 @@ __device__ __forceinline__ int chunk_count(int a_lane, bool valid, int T) {
 }
 
 // The sequential part: lane = neuron, one chunk of the tiles in place.
-template <class Op, int R, int UNROLL>
-__device__ __forceinline__ void run_chunk(Op& op, float (*tile)[TileGeom<R>::kTileFloats], int lane, int chunk,
+template <class Op, int R, int UNROLL, int S = kTileSamples>
+__device__ __forceinline__ void run_chunk(Op& op, float (*tile)[TileGeom<R, S>::kTileFloats], int lane, int chunk,
                                           bool inner, int a_lane, int T) {
-    using G = TileGeom<R>;
+    using G = TileGeom<R, S>;
     constexpr int NI = Op::kIn, NO = Op::kOut;
     auto run_quad = [&](int qq) {
         float xin[NI][4], yout[NO][4];
@@ -428,9 +428,9 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
 // A chunk is a few hundred nanoseconds of recurrence, less than a trip to memory, so the copy
 // waves keep the loads of two chunks in flight (chunk j waits in fetched[j & 1]).  All waves run
 // an even number of chunks; a surplus chunk lies outside every row and neither computes nor stores.
-template <class Op, int R, bool STREAM, int NCOPY>
+template <class Op, int R, bool STREAM, int NCOPY, int S = kTileSamples>
 __global__ __launch_bounds__((1 + NCOPY) * kWave) void stream_kernel_duo(typename Op::Params prm, int64_t M, int T) {
-    using G = TileGeom<R>;
+    using G = TileGeom<R, S>;
     constexpr int TC = G::kChunk;
     constexpr int NI = Op::kIn, NO = Op::kOut, NT = NI > NO ? NI : NO;
     constexpr int PASSES = G::kPasses / NCOPY;
@@ -456,14 +456,14 @@ __global__ __launch_bounds__((1 + NCOPY) * kWave) void stream_kernel_duo(typenam
             const int chunk = chunk_of(k);
             __syncthreads();                                   // barrier k
             if (k < nchunks)
-                run_chunk<Op, R, 4>(op, tiles[k & 1], lane, chunk, chunk >= 1 && chunk < interior_end, a_lane, T);
+                run_chunk<Op, R, 4, S>(op, tiles[k & 1], lane, chunk, chunk >= 1 && chunk < interior_end, a_lane, T);
         }
         __syncthreads();                                       // barrier nloop
         op.finish(prm, m0 + lane, lane < rows);
     } else {
         Op uni;                                                // wave-uniform members only (pre, post, derive)
         uni.init(prm, 0, false);
-        Copier<Op, R, STREAM, PASSES> io;
+        Copier<Op, R, STREAM, PASSES, S> io;
         io.init(prm, m0, rows, T, lane, base_f, (role - 1) * PASSES);
         float4 fetched[2][NI][PASSES];
         io.fetch_into(fetched[0], chunk_of(0));
