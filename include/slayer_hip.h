@@ -270,8 +270,11 @@ int slayer_cuba_bwd(float *grad_in, float *grad_i_decay, float *grad_v_decay,
 /* One launch for what rf.Neuron.forward does with two operators (neuron/rf.py:429-436 + :463-471 =
  * resonator.dynamics without threshold, complex.Spike.forward); bit-identical to slayer_res_fwd ->
  * slayer_cspike_fwd, 20 instead of 28 bytes per neuron-timestep.  imag_last is the imaginary sample
- * before step 0 (num_last == 1 broadcasts). */
-int slayer_rf_fwd(float *re_out, float *im_out, float *spk_out, const float *re_in, const float *im_in,
+ * before step 0 (num_last == 1 broadcasts).  re_out / im_out may both be NULL when no backward pass
+ * will follow (inference: 12 bytes); re_last_out / im_last_out ([M], both or neither NULL) receive
+ * real[..., -1] and imag[..., -1] for a persistent state. */
+int slayer_rf_fwd(float *re_out, float *im_out, float *spk_out, float *re_last_out, float *im_last_out,
+                  const float *re_in, const float *im_in,
                   const float *sin_decay, const float *cos_decay,
                   const float *re_state, const float *im_state, const float *imag_last,
                   float spike_threshold, int graded, float spike_scale, int w_scale,
@@ -297,9 +300,12 @@ int slayer_rf_bwd(float *g_re_in, float *g_im_in, float *grad_sin, float *grad_c
  * needs); th_last_out / ref_last_out ([M], both or neither NULL) receive the threshold and refractory
  * values of the last step, i.e. threshold[..., -1] and refractory[..., -1] of the separate operator.
  * cur_out may be NULL when the current trace is not wanted (no decay gradient in the backward pass):
- * 16 bytes per neuron-timestep; cur_last_out ([M], may be NULL) receives current[..., -1]. */
+ * 16 bytes per neuron-timestep; vol_out and theta_out may be NULL as well (together with cur_out) when
+ * no backward pass will follow (inference: 8 bytes).  cur_last_out / vol_last_out ([M], may be NULL)
+ * receive current[..., -1] and voltage[..., -1]. */
 int slayer_alif_fwd(float *cur_out, float *vol_out, float *theta_out, float *spk_out,
-                    float *cur_last_out, float *th_last_out, float *ref_last_out, const float *in,
+                    float *cur_last_out, float *vol_last_out, float *th_last_out, float *ref_last_out,
+                    const float *in,
                     const float *i_decay, const float *v_decay, const float *th_decay, const float *ref_decay,
                     const float *i_state, const float *v_state, const float *th_state, const float *ref_state,
                     int64_t th_step_scaled, int64_t th0_scaled, int graded, float spike_scale, int w_scale,

@@ -25,19 +25,19 @@ struct AlifFwd {
     struct Params {
         const float* in[1];
         float* out[kOut + 1];
-        float *cur_last, *th_last, *ref_last;        // [M] values of the last step, or nullptr
+        float *cur_last, *vol_last, *th_last, *ref_last;   // [M] values of the last step, or nullptr
         const float *i_decay, *v_decay, *th_decay, *ref_decay, *i_state, *v_state, *th_state, *ref_state;
         int step, base;
         float w, inv_w, spike_scale;
         int64_t npb, n_id, n_vd, n_td, n_rd, n_is, n_vs, n_ts, n_rs;
     };
     int yc, yv, th, r, mi, mv, mt, mr, th_step, base;
-    float w, inv_w, spike_scale, th_f, ref_f, cur_f;
+    float w, inv_w, spike_scale, th_f, ref_f, cur_f, vol_f;
 
     __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
         w = p.w; inv_w = p.inv_w; spike_scale = p.spike_scale; th_step = p.step; base = p.base;
         yc = yv = th = r = mi = mv = mt = mr = 0;
-        th_f = ref_f = cur_f = 0.f;
+        th_f = ref_f = cur_f = vol_f = 0.f;
         if (valid) {
             yc = trunc_i32(p.i_state[p.n_is == 1 ? 0 : m] * w);
             yv = trunc_i32(p.v_state[p.n_vs == 1 ? 0 : m] * w);
@@ -66,6 +66,7 @@ struct AlifFwd {
         th += fired ? th_step : 0;
         if (KEEP_CURRENT) o[0] = cur;
         cur_f = cur;
+        vol_f = vol;
         o[kVol] = vol;
         o[kTheta] = th_f + ref_f;
     }
@@ -80,6 +81,7 @@ struct AlifFwd {
     __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
         if (valid && p.th_last) { p.th_last[m] = th_f; p.ref_last[m] = ref_f; }
         if (valid && p.cur_last) p.cur_last[m] = cur_f;
+        if (valid && p.vol_last) p.vol_last[m] = vol_f;
     }
 };
 
@@ -129,7 +131,8 @@ struct AlifBwd {
 using namespace slayer;
 
 extern "C" int slayer_alif_fwd(float* cur_out, float* vol_out, float* theta_out, float* spk_out,
-                               float* cur_last_out, float* th_last_out, float* ref_last_out, const float* in,
+                               float* cur_last_out, float* vol_last_out, float* th_last_out, float* ref_last_out,
+                               const float* in,
                                const float* i_decay, const float* v_decay, const float* th_decay, const float* ref_decay,
                                const float* i_state, const float* v_state, const float* th_state, const float* ref_state,
                                int64_t th_step_scaled, int64_t th0_scaled, int graded, float spike_scale, int w_scale,
@@ -139,10 +142,11 @@ extern "C" int slayer_alif_fwd(float* cur_out, float* vol_out, float* theta_out,
                                int64_t T, void* stream) {
     if (int e = check_rows(M, T)) return e;
     if (M == 0 || T == 0) return 0;
-    if (!vol_out || !theta_out || !spk_out || !in || !i_decay || !v_decay || !th_decay || !ref_decay ||
+    if (!spk_out || !in || !i_decay || !v_decay || !th_decay || !ref_decay ||
         !i_state || !v_state || !th_state || !ref_state)
         return SLAYER_ENULL;
     if ((th_last_out == nullptr) != (ref_last_out == nullptr)) return SLAYER_ENULL;
+    if ((vol_out == nullptr) != (theta_out == nullptr) || (vol_out == nullptr && cur_out != nullptr)) return SLAYER_ENULL;
     for (int64_t n : {num_i_decays, num_v_decays, num_th_decays, num_ref_decays})
         if (int e = check_params(M, neurons_per_batch, n)) return e;
     for (int64_t n : {num_i_states, num_v_states, num_th_states, num_ref_states})
@@ -152,7 +156,7 @@ extern "C" int slayer_alif_fwd(float* cur_out, float* vol_out, float* theta_out,
     if (th_step_scaled > lim || th_step_scaled < -lim || th0_scaled > lim || th0_scaled < -lim) return SLAYER_ERANGE;
     const float w = (float)w_scale;
     hipStream_t st = (hipStream_t)stream;
-#define SLAYER_ALIF_ARGS cur_last_out, th_last_out, ref_last_out, i_decay, v_decay, th_decay, ref_decay, i_state,       \
+#define SLAYER_ALIF_ARGS cur_last_out, vol_last_out, th_last_out, ref_last_out, i_decay, v_decay, th_decay, ref_decay, i_state,       \
                          v_state, th_state, ref_state, (int)th_step_scaled, (int)th0_scaled, w, 1.0f / w,         \
                          spike_scale, neurons_per_batch, num_i_decays, num_v_decays, num_th_decays,               \
                          num_ref_decays, num_i_states, num_v_states, num_th_states, num_ref_states

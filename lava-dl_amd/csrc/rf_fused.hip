@@ -20,16 +20,17 @@ struct RfFwd {
     struct Params {
         const float* in[2];
         float* out[3];
+        float *re_last, *im_last;                   // [M] real / imaginary part of the last step, or nullptr
         const float *sin_decay, *cos_decay, *re_state, *im_state, *imag_last;
         float w, inv_w, spike_thr, spike_scale;
         int64_t npb, nd, n_rs, n_is, n_last;
     };
     int re, im, s, c;
-    float w, inv_w, spike_thr, spike_scale, im_prev;
+    float w, inv_w, spike_thr, spike_scale, im_prev, re_prev;
 
     __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
         w = p.w; inv_w = p.inv_w; spike_thr = p.spike_thr; spike_scale = p.spike_scale;
-        re = im = s = c = 0; im_prev = 0.f;
+        re = im = s = c = 0; im_prev = re_prev = 0.f;
         if (valid) {
             re = trunc_i32(p.re_state[p.n_rs == 1 ? 0 : m] * w);
             im = trunc_i32(p.im_state[p.n_is == 1 ? 0 : m] * w);
@@ -51,8 +52,11 @@ struct RfFwd {
         o[1] = i;
         o[2] = GRADED ? (((r * a) * b) * cc) / spike_scale : (a * b) * cc;
         im_prev = i;
+        re_prev = r;
     }
-    __device__ __forceinline__ void finish(const Params&, int64_t, bool) {}
+    __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
+        if (valid && p.re_last) { p.re_last[m] = re_prev; p.im_last[m] = im_prev; }
+    }
 };
 
 template <bool GRADED>
@@ -112,7 +116,8 @@ struct RfBwd {
 
 using namespace slayer;
 
-extern "C" int slayer_rf_fwd(float* re_out, float* im_out, float* spk_out, const float* re_in, const float* im_in,
+extern "C" int slayer_rf_fwd(float* re_out, float* im_out, float* spk_out, float* re_last_out, float* im_last_out,
+                             const float* re_in, const float* im_in,
                              const float* sin_decay, const float* cos_decay,
                              const float* re_state, const float* im_state, const float* imag_last,
                              float spike_threshold, int graded, float spike_scale, int w_scale,
@@ -121,8 +126,9 @@ extern "C" int slayer_rf_fwd(float* re_out, float* im_out, float* spk_out, const
                              int64_t T, void* stream) {
     if (int e = check_rows(M, T)) return e;
     if (M == 0 || T == 0) return 0;
-    if (!re_out || !im_out || !spk_out || !re_in || !im_in || !sin_decay || !cos_decay || !re_state || !im_state ||
-        !imag_last)
+    if (!spk_out || !re_in || !im_in || !sin_decay || !cos_decay || !re_state || !im_state || !imag_last)
+        return SLAYER_ENULL;
+    if ((re_out == nullptr) != (im_out == nullptr) || (re_last_out == nullptr) != (im_last_out == nullptr))
         return SLAYER_ENULL;
     if (int e = check_params(M, neurons_per_batch, num_decays)) return e;
     for (int64_t n : {num_re_states, num_im_states, num_last})
@@ -132,8 +138,9 @@ extern "C" int slayer_rf_fwd(float* re_out, float* im_out, float* spk_out, const
     hipStream_t st = (hipStream_t)stream;
 #define SLAYER_RF(P, G)                                                                                          \
     do {                                                                                                         \
-        RfFwd<P, G>::Params p{{re_in, im_in}, {re_out, im_out, spk_out}, sin_decay, cos_decay, re_state, im_state, \
-                              imag_last, w, 1.0f / w, spike_threshold, spike_scale, neurons_per_batch, num_decays, \
+        RfFwd<P, G>::Params p{{re_in, im_in}, {re_out, im_out, spk_out}, re_last_out, im_last_out, sin_decay, cos_decay, re_state,   \
+                              im_state, imag_last, w, 1.0f / w, spike_threshold, spike_scale, neurons_per_batch,   \
+                              num_decays,                                                                          \
                               num_re_states, num_im_states, num_last};                                             \
         return launch_stream<RfFwd<P, G>>(p, M, T, st);                                                            \
     } while (0)

@@ -70,18 +70,24 @@ class Neuron(_Base):
             _, voltage, threshold, refractory = self.dynamics(input)
             return self.spike(voltage, threshold, refractory)
         self._prepare(input)
-        current, voltage, _, spike, th_last, ref_last = alif_fused.dynamics(
-            input, self._q('current_decay'), self._q('voltage_decay'), self._q('threshold_decay'),
-            self._q('refractory_decay'), self.current_state, self.voltage_state, self.threshold_state,
-            self.refractory_state, self.threshold_step, self.threshold, self.s_scale,
-            self.tau_rho * TAU_RHO_MULT, self.scale_rho * SCALE_RHO_MULT, self.graded_spike, 1,
-            keep_current=self.requires_grad)
+        args = (input, self._q('current_decay'), self._q('voltage_decay'), self._q('threshold_decay'),
+                self._q('refractory_decay'), self.current_state, self.voltage_state, self.threshold_state,
+                self.refractory_state, self.threshold_step, self.threshold, self.s_scale)
+        if not (torch.is_grad_enabled() and (input.requires_grad or self.requires_grad)):
+            # nothing to differentiate: only the spikes are written, the last states come per neuron
+            current_last, voltage_last, _, spike, th_last, ref_last = alif_fused.spikes(*args, self.graded_spike, 1)
+        else:
+            # without trainable decays the kernel skips the current trace and returns its last step
+            current, voltage, _, spike, th_last, ref_last = alif_fused.dynamics(
+                *args, self.tau_rho * TAU_RHO_MULT, self.scale_rho * SCALE_RHO_MULT, self.graded_spike, 1,
+                keep_current=self.requires_grad)
+            current_last = current[..., -1] if self.requires_grad else current
+            voltage_last = voltage[..., -1]
         if self.persistent_state:
             with torch.no_grad():
                 last = spike[..., -1]
-                # without trainable decays the kernel skips the current trace and returns its last step
-                self.current_state = (current[..., -1] if self.requires_grad else current).clone()
-                self.voltage_state = voltage[..., -1].clone()
+                self.current_state = current_last.clone()
+                self.voltage_state = voltage_last.clone()
                 self.refractory_state = adaptive_threshold.persistent_ref_state(ref_last, last, th_last).detach().clone()
                 self.threshold_state = adaptive_threshold.persistent_th_state(
                     th_last, last, self.threshold_step).detach().clone()

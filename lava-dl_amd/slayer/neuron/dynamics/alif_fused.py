@@ -28,10 +28,22 @@ def dynamics(input, current_decay, voltage_decay, threshold_decay, refractory_de
                             lean)
 
 
+def spikes(input, current_decay, voltage_decay, threshold_decay, refractory_decay,
+           current_state, voltage_state, threshold_state, refractory_state,
+           threshold_step, threshold_base, w_scale, graded_spike=False, spike_scale=1):
+    """Inference form: (current_last, voltage_last, None, spike, threshold_last, refractory_last) with only
+    the spikes written per step; no gradient."""
+    with torch.no_grad():
+        return _fwd(input, (current_decay, voltage_decay, threshold_decay, refractory_decay),
+                    (current_state, voltage_state, threshold_state, refractory_state),
+                    threshold_step, threshold_base, w_scale, graded_spike is True, spike_scale, True, True, True)
+
+
 def _fwd(input, decays, states, threshold_step, threshold_base, w_scale, graded, spike_scale, want_last=True,
-         lean=False):
+         lean=False, spikes_only=False):
     """decays = (current, voltage, threshold, refractory), states likewise.  lean: no current trace,
-    the first result is then current[..., -1]."""
+    the first result is then current[..., -1].  spikes_only (with lean): no voltage / theta traces
+    either; the second result is then voltage[..., -1] and the third None."""
     dev = N.require_gpu(input, *decays, *states)
     input = input.contiguous()
     decays = [d.contiguous() for d in decays]
@@ -40,22 +52,27 @@ def _fwd(input, decays, states, threshold_step, threshold_base, w_scale, graded,
     for name, s in zip(('current_state', 'voltage_state', 'threshold_state', 'refractory_state'), states):
         if s.numel() not in (1, M):
             raise RuntimeError(f'{name} has {s.numel()} elements, expected 1 or {M}')
-    vol, theta, spk = (torch.empty_like(input) for _ in range(3))
+    if spikes_only and not lean:
+        raise RuntimeError('spikes_only implies lean')
+    spk = torch.empty_like(input)
+    vol, theta = (None, None) if spikes_only else (torch.empty_like(input), torch.empty_like(input))
     cur = None if lean else torch.empty_like(input)
     cur_last = torch.empty(input.shape[:-1], dtype=input.dtype, device=dev) if lean else None
+    vol_last = torch.empty(input.shape[:-1], dtype=input.dtype, device=dev) if spikes_only else None
     th_last = ref_last = None
     if want_last:
         th_last = torch.empty(input.shape[:-1], dtype=input.dtype, device=dev)
         ref_last = torch.empty(input.shape[:-1], dtype=input.dtype, device=dev)
     with torch.cuda.device(dev):
         N.check(N.lib().slayer_alif_fwd(
-            N.ptr(cur), N.ptr(vol), N.ptr(theta), N.ptr(spk), N.ptr(cur_last), N.ptr(th_last), N.ptr(ref_last),
+            N.ptr(cur), N.ptr(vol), N.ptr(theta), N.ptr(spk), N.ptr(cur_last), N.ptr(vol_last), N.ptr(th_last),
+            N.ptr(ref_last),
             N.ptr(input),
             *[N.ptr(d) for d in decays], *[N.ptr(s) for s in states],
             int(threshold_step * w_scale), int(threshold_base * w_scale), 1 if graded else 0, float(spike_scale),
             int(w_scale), M, N.neurons_per_batch(input), *[d.numel() for d in decays],
             *[s.numel() for s in states], T, N.stream_handle()))
-    return (cur_last if lean else cur), vol, theta, spk, th_last, ref_last
+    return (cur_last if lean else cur), (vol_last if spikes_only else vol), theta, spk, th_last, ref_last
 
 
 def _bwd(grad_spikes, vol, theta, cur, i_decay, v_decay, tau_rho, scale_rho, graded, need_decay_grad=True):

@@ -19,8 +19,17 @@ def dynamics(real_input, imag_input, sin_decay, cos_decay, real_state, imag_stat
                           w_scale, threshold, tau_rho, scale_rho, graded_spike, spike_scale)
 
 
+def spikes(real_input, imag_input, sin_decay, cos_decay, real_state, imag_state, imag_last, w_scale,
+           threshold, graded_spike=False, spike_scale=1):
+    """Inference form: (real_last, imag_last, spike) with only the spikes written per step; no gradient."""
+    with torch.no_grad():
+        return _fwd(real_input, imag_input, sin_decay, cos_decay, real_state, imag_state, imag_last, w_scale,
+                    threshold, graded_spike is True, spike_scale, spikes_only=True)
+
+
 def _fwd(real_input, imag_input, sin_decay, cos_decay, real_state, imag_state, imag_last, w_scale,
-         threshold, graded, spike_scale):
+         threshold, graded, spike_scale, spikes_only=False):
+    """spikes_only: no real / imag traces; the first two results are then real[..., -1], imag[..., -1]."""
     if not torch.is_tensor(imag_last):
         imag_last = torch.tensor([float(imag_last)], dtype=real_input.dtype, device=real_input.device)
     tensors = [real_input, imag_input, sin_decay, cos_decay, real_state, imag_state, imag_last]
@@ -33,15 +42,21 @@ def _fwd(real_input, imag_input, sin_decay, cos_decay, real_state, imag_state, i
     for name, s in (('real_state', real_state), ('imag_state', imag_state), ('imag_last', imag_last)):
         if s.numel() not in (1, M):
             raise RuntimeError(f'{name} has {s.numel()} elements, expected 1 or {M}')
-    real, imag, spk = (torch.empty_like(real_input) for _ in range(3))
+    spk = torch.empty_like(real_input)
+    real = imag = re_last = im_last = None
+    if spikes_only:
+        re_last, im_last = (torch.empty(real_input.shape[:-1], dtype=real_input.dtype, device=dev) for _ in range(2))
+    else:
+        real, imag = torch.empty_like(real_input), torch.empty_like(real_input)
     with torch.cuda.device(dev):
         N.check(N.lib().slayer_rf_fwd(
-            N.ptr(real), N.ptr(imag), N.ptr(spk), N.ptr(real_input), N.ptr(imag_input),
+            N.ptr(real), N.ptr(imag), N.ptr(spk), N.ptr(re_last), N.ptr(im_last), N.ptr(real_input),
+            N.ptr(imag_input),
             N.ptr(sin_decay), N.ptr(cos_decay), N.ptr(real_state), N.ptr(imag_state), N.ptr(imag_last),
             float(threshold), 1 if graded else 0, float(spike_scale), int(w_scale),
             M, N.neurons_per_batch(real_input), sin_decay.numel(),
             real_state.numel(), imag_state.numel(), imag_last.numel(), T, N.stream_handle()))
-    return real, imag, spk
+    return (re_last, im_last, spk) if spikes_only else (real, imag, spk)
 
 
 def _bwd(grad_spikes, real, imag, sin_decay, cos_decay, threshold, tau_rho, scale_rho, graded,

@@ -131,14 +131,20 @@ class Neuron(ResonatorNeuron):
             raise AssertionError(f'Real input tensor shape ({real_input.shape}) does not match '
                                  f'with imaginary input shape ({imag_input.shape}).')
         self._prepare(real_input)
-        real, imag, spike = rf_fused.dynamics(
-            real_input, imag_input, quantize(self.sin_decay), quantize(self.cos_decay),
-            self.real_state, self.imag_state, self.imag_state, self.s_scale, self.threshold,
-            self.tau_rho * TAU_RHO_MULT, self.scale_rho * SCALE_RHO_MULT, self.graded_spike, 1)
+        args = (real_input, imag_input, quantize(self.sin_decay), quantize(self.cos_decay),
+                self.real_state, self.imag_state, self.imag_state, self.s_scale, self.threshold)
+        needs_grad = real_input.requires_grad or imag_input.requires_grad or self.requires_grad
+        if not (torch.is_grad_enabled() and needs_grad):
+            # nothing to differentiate: only the spikes are written, the last state comes per neuron
+            real_last, imag_last, spike = rf_fused.spikes(*args, self.graded_spike, 1)
+        else:
+            real, imag, spike = rf_fused.dynamics(*args, self.tau_rho * TAU_RHO_MULT,
+                                                  self.scale_rho * SCALE_RHO_MULT, self.graded_spike, 1)
+            real_last, imag_last = real[..., -1], imag[..., -1]
         if self.persistent_state:
             with torch.no_grad():
-                self.real_state = real[..., -1].clone()
-                self.imag_state = imag[..., -1].clone()
+                self.real_state = real_last.clone()
+                self.imag_state = imag_last.clone()
         if self.drop is not None:
             spike = self.drop(spike)
         return spike

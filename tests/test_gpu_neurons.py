@@ -384,28 +384,42 @@ def test_fused_alif_without_current_trace(slayer, shape, w):
     assert torch.equal(b.grad, a.grad)
 
 
+@pytest.mark.parametrize('kind', ['cuba', 'alif', 'rf'])
 @pytest.mark.parametrize('shared', [True, False])
-def test_cuba_neuron_inference_form_matches_training_form(slayer, shared):
+def test_neuron_inference_form_matches_training_form(slayer, kind, shared):
     """Under no_grad only the spikes are written; spikes and the carried states must equal the
     training form over several calls with persistent state."""
     gen = torch.Generator().manual_seed(107)
     shape = (3, 12, 6, 152)
-    x = sparse_input(gen, shape, p=0.3, amp=1.5).to(dev())
-    mk = lambda: slayer.neuron.cuba.Neuron(1.0, [0.2, 0.4] if not shared else 0.25, [0.02, 0.2] if not shared else 0.03,
-                                           shared_param=shared, persistent_state=True).to(dev())
+    rng = lambda a, b: [a, b] if not shared else a
+    if kind == 'cuba':
+        mk = lambda: slayer.neuron.cuba.Neuron(1.0, rng(0.2, 0.4), rng(0.02, 0.2), shared_param=shared,
+                                               persistent_state=True).to(dev())
+    elif kind == 'alif':
+        mk = lambda: slayer.neuron.alif.Neuron(1.0, 0.5, rng(0.25, 0.4), rng(0.03, 0.2), rng(0.1, 0.3), rng(0.1, 0.3),
+                                               shared_param=shared, persistent_state=True).to(dev())
+    else:
+        mk = lambda: slayer.neuron.rf.Neuron(1.0, rng(5, 20) if not shared else 11, rng(0.02, 0.1),
+                                             shared_param=shared, persistent_state=True).to(dev())
+    x = sparse_input(gen, shape, p=0.3, amp=2.0).to(dev())
+    x2 = sparse_input(gen, shape, p=0.3, amp=2.0).to(dev())
+    inp = (lambda grad: (x.clone().requires_grad_(grad), x2.clone().requires_grad_(grad))) if kind == 'rf' \
+        else (lambda grad: x.clone().requires_grad_(grad))
     a, b = mk(), mk()
     a._prepare(x); b._prepare(x)
     for pa, pb in zip(a.parameters(), b.parameters()):
         pb.data = pa.data.clone()
+    states = [n for n, _ in a.named_buffers() if n.endswith('_state')]
     total = 0.0
     for k in range(3):
-        sa = a(x.clone().requires_grad_())
+        sa = a(inp(True))
         with torch.no_grad():
-            sb = b(x)
+            sb = b(inp(False))
         assert torch.equal(sa.detach(), sb), f'call {k}: spikes differ'
-        assert torch.equal(a.current_state, b.current_state) and torch.equal(a.voltage_state, b.voltage_state)
+        for name in states:
+            assert torch.equal(getattr(a, name), getattr(b, name)), f'call {k}: {name} differs'
         total += float(sb.sum())
-    assert total > 0
+    assert total > 0 and len(states) >= 2
 
 
 def test_fused_cuba_under_graph_capture_replays(slayer):
