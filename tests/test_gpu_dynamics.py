@@ -432,3 +432,38 @@ def test_rows_longer_than_the_vector_path_allows(slayer):
     ref = O.li_fwd(x.detach().cpu()[..., :head], d.detach().cpu(), torch.tensor([0.0]), 64, 1.0)
     assert_exact(y.detach()[..., :head], ref, 'li_fwd long rows, head')
     assert torch.isfinite(x.grad).all() and float(x.grad.abs().sum()) > 0
+
+
+def test_two_streams_and_two_threads(slayer):
+    """Entry points take the caller's stream and keep no per-call global state: launches from two
+    host threads on two streams, interleaved, give the same bits as serial launches."""
+    import threading
+    gen = torch.Generator().manual_seed(91)
+    shapes = [(4, 64, 33, 300), (2, 40, 17, 128)]
+    xs = [sparse_input(gen, s, p=0.2, amp=1.5).to(dev()) for s in shapes]
+    ds = [torch.randint(0, 4096, (s[1],), generator=gen).float().to(dev()) for s in shapes]
+    zero = torch.zeros(1, device=dev())
+    D = slayer.neuron.dynamics.leaky_integrator
+    want = [D.dynamics(x, d, zero, 64, 1.0) for x, d in zip(xs, ds)]
+    torch.cuda.synchronize()
+    got, errors = [None, None], []
+
+    def work(i):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for _ in range(20):
+                    y = D.dynamics(xs[i], ds[i], zero, 64, 1.0)
+                stream.synchronize()
+            got[i] = y
+        except Exception as e:      # surfaced in the main thread below
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for i in range(2):
+        assert torch.equal(got[i], want[i]), f'stream {i}: result differs from the serial launch'
