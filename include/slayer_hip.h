@@ -325,6 +325,33 @@ int slayer_alif_bwd(float *grad_in, float *grad_i_decay, float *grad_v_decay,
                     int64_t M, int64_t neurons_per_batch, int64_t num_i_decays, int64_t num_v_decays,
                     int64_t T, void *stream);
 
+/* ---- recurrent CUBA layer --------------------------------------------------------------------- */
+
+/* The time loop of utils/recurrent.py:45-81 (CustomRecurrent.forward) for a CUBA neuron with binary
+ * spikes, in one launch:  feedback[t] = R s[t-1],  s[t] = neuron(z[t] + feedback[t]),  s[-1] = 0.
+ * z, spk_out, vol_out: [N][C][T]; rec_t = R^T followed by a row of zeros, [C + 1][C] (row j = the
+ * weights from neuron j; the kernel pads its spike lists with the index of the zero row);
+ * decays [1] or [C]; states [1] or [N*C] are the neuron's persistent current / voltage before the
+ * first step.  vol_out is the voltage trace the backward pass needs; cur_last_out / vol_last_out
+ * ([N*C]) are the current and the (un-reset) voltage of the last step.  C <= 1024.
+ * Equal to calling the neuron one step at a time (the state between two calls makes the same float32
+ * round trip) whenever the feedback sums are exact in float32, e.g. with quantised weights. */
+int slayer_cuba_recurrent_fwd(float *spk_out, float *vol_out, float *cur_last_out, float *vol_last_out,
+                              const float *z, const float *rec_t,
+                              const float *i_decay, const float *v_decay,
+                              const float *i_state, const float *v_state,
+                              float spike_threshold, int w_scale,
+                              int64_t N, int64_t C, int64_t num_i_decays, int64_t num_v_decays,
+                              int64_t num_i_states, int64_t num_v_states, int64_t T, void *stream);
+
+/* Backward of the loop as utils/recurrent.py:83-112 differentiates it (the carried neuron state is a
+ * constant, a step contributes its spike surrogate, the gradient reaches step t-1 through R):
+ * grad_z[t] = surrogate(voltage[t]) * (grad_spikes[t] + (grad_z[t+1] R));  rec = R, [C][C].
+ * The gradient of R is the product grad_z[:, :, 1:] x spikes[:, :, :-1] and is left to the caller. */
+int slayer_cuba_recurrent_bwd(float *grad_z, const float *grad_spikes, const float *voltage, const float *rec,
+                              float spike_threshold, float tau_rho, float scale_rho,
+                              int64_t N, int64_t C, int64_t T, void *stream);
+
 /* ---- cross-check implementations (debug mode) ------------------------------------------------ */
 
 /* The reference's debug mode runs its CPU loop next to its kernel and raises on a difference

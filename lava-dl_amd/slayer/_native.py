@@ -51,6 +51,8 @@ _SIGNATURES = {
     'slayer_rf_bwd': (_INT, [_P] * 9 + [_F, _F, _F, _INT, _P] + [_I64] * 4 + [_P]),
     'slayer_alif_fwd': (_INT, [_P] * 17 + [_I64, _I64, _INT, _F, _INT] + [_I64] * 11 + [_P]),
     'slayer_alif_bwd': (_INT, [_P] * 9 + [_F, _F, _INT, _P] + [_I64] * 5 + [_P]),
+    'slayer_cuba_recurrent_fwd': (_INT, [_P] * 10 + [_F, _INT] + [_I64] * 7 + [_P]),
+    'slayer_cuba_recurrent_bwd': (_INT, [_P] * 4 + [_F, _F, _F] + [_I64] * 3 + [_P]),
     'slayer_li_fwd_naive': (_INT, [_P, _P, _P, _P, _D, _INT, _I64, _I64, _I64, _I64, _I64, _P]),
     'slayer_li_bwd_naive': (_INT, [_P, _P, _P, _I64, _I64, _I64, _I64, _P]),
     'slayer_ath_fwd_naive': (_INT, [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _INT,

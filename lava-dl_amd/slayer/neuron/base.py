@@ -49,6 +49,12 @@ class Neuron(torch.nn.Module):
     def threshold(self):
         return self._threshold
 
+    def quantize_8bit(self, weight, descale=False):
+        """Weight quantiser to link with a synapse (``synapse.pre_hook_fx = neuron.quantize_8bit``):
+        steps of 2 / scale, clamped to the 8-bit range; ``descale`` returns integers."""
+        q = quantize(weight, step=2 / self.w_scale).clamp(-256 / self.w_scale, 254 / self.w_scale)
+        return q * self.w_scale if descale else q
+
     def _register_decays(self, **decays):
         """Shared: one value each.  Per channel: remember [min, max] (a scalar means +-1 %)
         and draw the values when the channel count is known."""

@@ -502,3 +502,44 @@ def sigma_fwd(x, pre_state=None):
     if pre_state is not None:
         out = out + pre_state.unsqueeze(-1)
     return out
+
+
+# --------------------------------------------------------------------------- recurrent layer
+def recurrent_cuba_fwd(z, rec, i_decay, v_decay, i_state, v_state, w_scale, threshold):
+    """Recurrent CUBA layer, S/utils/recurrent.py:45-81 with the CUBA neuron called one step at a
+    time (S/neuron/cuba.py:356-421, persistent state): feedback = s[t-1] @ R^T, the neuron's current
+    and voltage LI run one step each from the carried float32 states, a spike resets the carried
+    voltage.  z: [N, C, T]; rec = R [C, C].  Returns (spikes, voltage, current_state, voltage_state)."""
+    spikes = torch.zeros_like(z)
+    voltage = torch.zeros_like(z)
+    cur_state = _full_state(i_state, z[..., :1])
+    vol_state = _full_state(v_state, z[..., :1])
+    s = torch.zeros(z.shape[:-1])
+    rec_t = rec.transpose(0, 1)
+    for t in range(z.shape[-1]):
+        dend = (z[..., t] + torch.matmul(s, rec_t)).unsqueeze(-1)
+        cur = li_fwd(dend, i_decay, cur_state, w_scale)
+        vol = li_fwd(cur, v_decay, vol_state, w_scale, threshold)
+        spk = spike_fwd(vol, threshold)
+        cur_state = cur[..., -1]
+        vol_state = li_persistent_state(vol[..., -1], spk[..., -1])
+        s = spk[..., 0]
+        spikes[..., t] = s
+        voltage[..., t] = vol[..., 0]
+    return spikes, voltage, cur_state, vol_state
+
+
+def recurrent_cuba_bwd(grad_x, spikes, voltage, rec, threshold, tau_rho, scale_rho):
+    """S/utils/recurrent.py:83-112: the carried neuron state is a constant, so a step contributes the
+    spike surrogate (the two one-step LI backward passes are identities); the gradient reaches step
+    t-1 through R.  Returns (grad_z, grad_R)."""
+    grad_z = torch.zeros_like(grad_x)
+    carry = torch.zeros(grad_x.shape[:-1])
+    for t in range(grad_x.shape[-1] - 1, -1, -1):
+        gs = carry + grad_x[..., t]
+        gd = spike_bwd(gs.unsqueeze(-1), voltage[..., t:t + 1], threshold, tau_rho, scale_rho)[..., 0]
+        grad_z[..., t] = gd
+        carry = torch.matmul(gd, rec)
+    grad_out = grad_z[..., 1:].transpose(0, 1).reshape(grad_z.shape[1], -1)
+    spikes_in = spikes[..., :-1].transpose(1, 2).reshape(-1, spikes.shape[1])
+    return grad_z, torch.matmul(grad_out, spikes_in)
