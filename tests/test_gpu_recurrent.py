@@ -99,6 +99,6 @@ def test_other_neurons_take_the_generic_loop(slayer):
     syn_a, syn_b = (_Dense(c, torch.Generator().manual_seed(3)).to(dev()) for _ in range(2))
     out = slayer.utils.recurrent.custom_recurrent(z, a, syn_a)
     ref = slayer.utils.recurrent.custom_recurrent_ground_truth_2(z.detach(), b, syn_b)
-    assert torch.equal(out, ref.detach()) and float(out.sum()) > 0
+    assert torch.equal(out, ref.detach()) and float(out.detach().sum()) > 0
     out.sum().backward()
     assert torch.isfinite(z.grad).all() and syn_a.weight.grad is not None
