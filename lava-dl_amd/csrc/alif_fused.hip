@@ -110,9 +110,21 @@ struct AlifBwd {
             av = 1.0f - p.v_decay[param_index(m, p.npb, p.n_vd)] / 4096.0f;
         }
     }
+    // The surrogate does not depend on the recurrence, so it is evaluated on the way into LDS (by all
+    // 64 lanes, or by the copy wave of the multi-wave kernel) and takes the place of the incoming gradient.
+    static constexpr bool kTransforms = true;
+    static constexpr int kCopyWaves = 4;
+    __device__ __forceinline__ float surrogate(float g, float v, float theta) const {
+        const float d = v - theta;
+        return GRADED ? (rho * expf(fminf(d, 0.0f) / tau)) * g : (lead * expf(-fabsf(d) / tau)) * g;
+    }
+    __device__ __forceinline__ void pre(float4 (&x)[kIn]) const {
+        x[0] = make_float4(surrogate(x[0].x, x[1].x, x[2].x), surrogate(x[0].y, x[1].y, x[2].y),
+                           surrogate(x[0].z, x[1].z, x[2].z), surrogate(x[0].w, x[1].w, x[2].w));
+    }
+    __device__ __forceinline__ void post(float4 (&)[1]) const {}
     __device__ __forceinline__ void step(const float (&x)[kIn], float (&o)[1]) {
-        const float d = x[1] - x[2];
-        const float gv = GRADED ? (rho * expf(fminf(d, 0.0f) / tau)) * x[0] : (lead * expf(-fabsf(d) / tau)) * x[0];
+        const float gv = x[0];
         if (DECAY_GRAD) {
             acc_v = __fmaf_rn(gc, x[1], acc_v);      // gc, gx still hold the gradients of step t+1
             acc_i = __fmaf_rn(gx, x[kIn - 1], acc_i);

@@ -600,16 +600,20 @@ struct DuoRows { static constexpr int value = 64; };
 template <class Op>
 struct DuoRows<Op, decltype((void)Op::kDuoRows)> { static constexpr int value = Op::kDuoRows; };
 
-// Copy waves per workgroup of the multi-wave kernel.
-constexpr int kCopyWaves = 1;
+// Copy waves per workgroup of the multi-wave kernel: 1 unless the Op says otherwise (kCopyWaves; an Op
+// whose pre() is expensive wants more, so that the sequential wave does not wait for its tiles).
+template <class Op, class = void>
+struct CopyWaves { static constexpr int value = 1; };
+template <class Op>
+struct CopyWaves<Op, decltype((void)Op::kCopyWaves)> { static constexpr int value = Op::kCopyWaves; };
 
 // Workgroups of the multi-wave kernel that one compute unit holds at a time (LDS and registers).
 template <class Op, int R, bool STREAM>
 int duo_groups_per_cu() {
     static const int n = [] {
         int v = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&v, stream_kernel_duo<Op, R, STREAM, kCopyWaves>,
-                                                         (1 + kCopyWaves) * kWave, 0) != hipSuccess)
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&v, stream_kernel_duo<Op, R, STREAM, CopyWaves<Op>::value>,
+                                                         (1 + CopyWaves<Op>::value) * kWave, 0) != hipSuccess)
             v = 0;
         return v;
     }();
@@ -662,11 +666,12 @@ int launch_stream(const typename Op::Params& prm, int64_t M, int64_t T, hipStrea
         const int64_t groups = (M + RD - 1) / RD;
         const int per_cu = streaming ? duo_groups_per_cu<Op, RD, true>() : duo_groups_per_cu<Op, RD, false>();
         if (groups <= (int64_t)per_cu * compute_units()) {
-            const dim3 grid((unsigned)groups), block((1 + kCopyWaves) * kWave);
+            constexpr int NC = CopyWaves<Op>::value;
+            const dim3 grid((unsigned)groups), block((1 + NC) * kWave);
             if (streaming)
-                hipLaunchKernelGGL((stream_kernel_duo<Op, RD, true, kCopyWaves>), grid, block, 0, stream, prm, M, (int)T);
+                hipLaunchKernelGGL((stream_kernel_duo<Op, RD, true, NC>), grid, block, 0, stream, prm, M, (int)T);
             else
-                hipLaunchKernelGGL((stream_kernel_duo<Op, RD, false, kCopyWaves>), grid, block, 0, stream, prm, M, (int)T);
+                hipLaunchKernelGGL((stream_kernel_duo<Op, RD, false, NC>), grid, block, 0, stream, prm, M, (int)T);
             return (int)hipGetLastError();
         }
     }
