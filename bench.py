@@ -1,6 +1,6 @@
 """Benchmark of the SLAYER neuron-dynamics hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cuba|cuba_fused|cuba_fused_lean|cuba_inference|cuba_fwd_small|alif|alif_fused|alif_fused_lean|rf|rf_fused|rf_inference|synapse]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cuba|cuba_fused|cuba_fused_lean|cuba_inference|cuba_fwd_small|alif|alif_fused|alif_fused_lean|rf|rf_fused|rf_fused_lean|rf_inference|synapse]
 
 A step is one pass of the workload's op sequence over one batch of synthetic input that is already
 resident in HBM (outputs come from torch's caching allocator inside the timed region).  The default
@@ -370,6 +370,18 @@ class RfFused(Rf):
         return spk, out
 
 
+class RfFusedLean(RfFused):
+    name = 'Resonator (RF) dynamics fwd+bwd, fused kernels, no decay gradients'
+
+    def step(self, t):
+        with t('rf_fwd'):
+            re, im, spk = self.F._fwd(self.xr, self.xi, self.sin, self.cos, self.zero, self.zero, self.zero, 64,
+                                      1.0, False, 1)
+        with t('rf_bwd'):
+            out = self.F._bwd(self.g, re, im, self.sin, self.cos, 1.0, 0.5, 10.0, False, False)
+        return spk, out
+
+
 class RfInference(Rf):
     name = 'Resonator (RF) neuron forward, spikes only (inference)'
     ops = [('rf_fwd', 'stream_kernel<RfFwd>', 12)]
@@ -443,7 +455,7 @@ class Synapse(Workload):
         O.conv_bwd(O.shift(g_z, -c['delay'], 1), c['filt'], 1)
 
 
-WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fused_lean': CubaFusedLean, 'cuba_inference': CubaInference, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'alif_fused': AlifFused, 'alif_fused_lean': AlifFusedLean, 'rf': Rf, 'rf_fused': RfFused, 'rf_inference': RfInference, 'synapse': Synapse}
+WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fused_lean': CubaFusedLean, 'cuba_inference': CubaInference, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'alif_fused': AlifFused, 'alif_fused_lean': AlifFusedLean, 'rf': Rf, 'rf_fused': RfFused, 'rf_fused_lean': RfFusedLean, 'rf_inference': RfInference, 'synapse': Synapse}
 
 
 def cpu_baseline(job, budget_s=20.0):

@@ -59,9 +59,14 @@ struct RfFwd {
     }
 };
 
-template <bool GRADED>
+// DECAY_GRAD = false: the saved real / imag parts are needed by the spike surrogate only, which does not
+// depend on the recurrence; it is then evaluated on the way into LDS (by all 64 lanes, or by the copy
+// waves of the multi-wave kernel) and its two results take the places of real and imag.
+template <bool GRADED, bool DECAY_GRAD>
 struct RfBwd {
     static constexpr int kIn = 3, kOut = 2;          // in: grad of spikes, saved real, saved imag
+    static constexpr bool kTransforms = !DECAY_GRAD;
+    static constexpr int kCopyWaves = DECAY_GRAD ? 1 : 4;
     static constexpr bool kReverse = true;
     static constexpr int64_t kRows32Below = 4096, kRows16Below = 4096;     // exp per step: keep all lanes busy
     struct Params {
@@ -86,9 +91,8 @@ struct RfBwd {
             s = p.sin_decay[j] / 4096.0f;
         }
     }
-    __device__ __forceinline__ void step(const float (&x)[3], float (&o)[2]) {
-        const float g = x[0], r = x[1], i = x[2];
-        // complex spike surrogate (same expression order as the stand-alone kernel)
+    // complex spike surrogate (same expression order as the stand-alone kernel)
+    __device__ __forceinline__ void surrogate(float g, float r, float i, float& g_re, float& g_im) const {
         float d_re;
         if (GRADED) d_re = expf(-fmaxf(thr - r, 0.0f) / tau);
         else d_re = half_over_tau * expf(-fabsf(r - thr) / tau);
@@ -97,18 +101,39 @@ struct RfBwd {
         const float sg_r = dr > 0.0f ? 1.0f : (dr < 0.0f ? -1.0f : (dr == 0.0f ? 0.0f : dr));
         const float sg_i = i > 0.0f ? 1.0f : (i < 0.0f ? -1.0f : (i == 0.0f ? 0.0f : i));
         const float step_re = 0.5f * (1.0f + sg_r * (1.0f - two_tau * d_re));
-        const float g_re = g * ((rho * d_re) * d_im);
-        const float g_im = g * (((neg_rho_over_tau * sg_i) * d_im) * step_re);
-        // reverse-time rotation; gr, gi still hold the gradients of step t+1
-        acc_s = __fmaf_rn(gi, r, __fmaf_rn(-gr, i, acc_s));
-        acc_c = __fmaf_rn(gi, i, __fmaf_rn(gr, r, acc_c));
+        g_re = g * ((rho * d_re) * d_im);
+        g_im = g * (((neg_rho_over_tau * sg_i) * d_im) * step_re);
+    }
+    __device__ __forceinline__ void pre(float4 (&x)[3]) const {
+        float4 a, b;
+        surrogate(x[0].x, x[1].x, x[2].x, a.x, b.x);
+        surrogate(x[0].y, x[1].y, x[2].y, a.y, b.y);
+        surrogate(x[0].z, x[1].z, x[2].z, a.z, b.z);
+        surrogate(x[0].w, x[1].w, x[2].w, a.w, b.w);
+        x[1] = a;
+        x[2] = b;
+    }
+    __device__ __forceinline__ void post(float4 (&)[2]) const {}
+    __device__ __forceinline__ void step(const float (&x)[3], float (&o)[2]) {
+        float g_re, g_im;
+        if (DECAY_GRAD) {
+            const float r = x[1], i = x[2];
+            surrogate(x[0], r, i, g_re, g_im);
+            // gr, gi still hold the gradients of step t+1
+            acc_s = __fmaf_rn(gi, r, __fmaf_rn(-gr, i, acc_s));
+            acc_c = __fmaf_rn(gi, i, __fmaf_rn(gr, r, acc_c));
+        } else {
+            g_re = x[1];
+            g_im = x[2];
+        }
+        // reverse-time rotation
         const float ngr = (c * gr + s * gi) + g_re;
         const float ngi = ((-s) * gr + c * gi) + g_im;
         gr = ngr; gi = ngi;
         o[0] = ngr; o[1] = ngi;
     }
     __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
-        if (valid && p.partial_sin) { p.partial_sin[m] = acc_s; p.partial_cos[m] = acc_c; }
+        if (DECAY_GRAD && valid && p.partial_sin) { p.partial_sin[m] = acc_s; p.partial_cos[m] = acc_c; }
     }
 };
 
@@ -163,17 +188,23 @@ extern "C" int slayer_rf_bwd(float* g_re_in, float* g_im_in, float* grad_sin, fl
     hipStream_t st = (hipStream_t)stream;
     if (M > 0 && T > 0) {
         if (!g_re_in || !g_im_in || !grad_spikes || !re || !im || !sin_decay || !cos_decay) return SLAYER_ENULL;
-        if (graded) {
-            RfBwd<true>::Params p{{grad_spikes, re, im}, {g_re_in, g_im_in}, sin_decay, cos_decay,
-                                  want ? workspace : nullptr, want ? workspace + M : nullptr,
-                                  spike_threshold, tau_rho, scale_rho, neurons_per_batch, num_decays};
-            if (int e = launch_stream<RfBwd<true>>(p, M, T, st)) return e;
-        } else {
-            RfBwd<false>::Params p{{grad_spikes, re, im}, {g_re_in, g_im_in}, sin_decay, cos_decay,
-                                   want ? workspace : nullptr, want ? workspace + M : nullptr,
-                                   spike_threshold, tau_rho, scale_rho, neurons_per_batch, num_decays};
-            if (int e = launch_stream<RfBwd<false>>(p, M, T, st)) return e;
-        }
+#define SLAYER_RF_BWD(G, D)                                                                                       \
+    do {                                                                                                          \
+        RfBwd<G, D>::Params p{{grad_spikes, re, im}, {g_re_in, g_im_in}, sin_decay, cos_decay,                      \
+                              want ? workspace : nullptr, want ? workspace + M : nullptr,                         \
+                              spike_threshold, tau_rho, scale_rho, neurons_per_batch, num_decays};                \
+        if (D || stream_fits_multiwave<RfBwd<G, D>>(p, M, T)) {                                                   \
+            if (int e = launch_stream<RfBwd<G, D>>(p, M, T, st)) return e;                                        \
+            done = true;                                                                                          \
+        }                                                                                                         \
+    } while (0)
+        // Without decay gradients the surrogate can run in the copy waves of the multi-wave kernel (three
+        // times faster there); the one-wave kernel gains nothing from that split, so large tensors take
+        // the other form with its partial sums dropped.
+        bool done = false;
+        if (!want) { if (graded) SLAYER_RF_BWD(true, false); else SLAYER_RF_BWD(false, false); }
+        if (!done) { if (graded) SLAYER_RF_BWD(true, true); else SLAYER_RF_BWD(false, true); }
+#undef SLAYER_RF_BWD
     }
     if (want) {
         if (M == 0 || T == 0) {

@@ -653,27 +653,41 @@ int launch_stream_rows(const typename Op::Params& prm, int64_t M, int64_t T, boo
 //  * beyond that the one-wave kernel, with the rows per wave the Op asks for (kRows32Below,
 //    kRows16Below): integer forward recurrences and backward passes with an exp per step keep all
 //    64 lanes busy, the light float backward passes prefer 16 rows and 512-byte row segments.
+// True when launch_stream would pick the dwordx4 path for these operands.
 template <class Op>
-int launch_stream(const typename Op::Params& prm, int64_t M, int64_t T, hipStream_t stream) {
-    if (M == 0 || T == 0) return 0;
+bool stream_vectorizes(const typename Op::Params& prm, int64_t T) {
     // the dwordx4 kernels address a wave's rows with 32-bit byte offsets: 64 * T * 4 must stay below 2^31
     bool vec = (T % 4) == 0 && T <= (1 << 22);
     for (int i = 0; i < Op::kIn; ++i) vec = vec && aligned16(prm.in[i]);
     for (int o = 0; o < Op::kOut + DerivedCount<Op>::value; ++o) vec = vec && aligned16(prm.out[o]);
-    const bool streaming = M * T * 4 > ((int64_t)64 << 20);
-    if (vec) {
+    return vec;
+}
+
+inline bool stream_is_large(int64_t M, int64_t T) { return M * T * 4 > ((int64_t)64 << 20); }
+
+// True when launch_stream would run the multi-wave kernel: dwordx4 path and every workgroup resident at once.
+template <class Op>
+bool stream_fits_multiwave(const typename Op::Params& prm, int64_t M, int64_t T) {
+    if (M == 0 || T == 0 || !stream_vectorizes<Op>(prm, T)) return false;
+    constexpr int RD = DuoRows<Op>::value;
+    const int per_cu = stream_is_large(M, T) ? duo_groups_per_cu<Op, RD, true>() : duo_groups_per_cu<Op, RD, false>();
+    return (M + RD - 1) / RD <= (int64_t)per_cu * compute_units();
+}
+
+template <class Op>
+int launch_stream(const typename Op::Params& prm, int64_t M, int64_t T, hipStream_t stream) {
+    if (M == 0 || T == 0) return 0;
+    const bool vec = stream_vectorizes<Op>(prm, T);
+    const bool streaming = stream_is_large(M, T);
+    if (stream_fits_multiwave<Op>(prm, M, T)) {
         constexpr int RD = DuoRows<Op>::value;
-        const int64_t groups = (M + RD - 1) / RD;
-        const int per_cu = streaming ? duo_groups_per_cu<Op, RD, true>() : duo_groups_per_cu<Op, RD, false>();
-        if (groups <= (int64_t)per_cu * compute_units()) {
-            constexpr int NC = CopyWaves<Op>::value;
-            const dim3 grid((unsigned)groups), block((1 + NC) * kWave);
-            if (streaming)
-                hipLaunchKernelGGL((stream_kernel_duo<Op, RD, true, NC>), grid, block, 0, stream, prm, M, (int)T);
-            else
-                hipLaunchKernelGGL((stream_kernel_duo<Op, RD, false, NC>), grid, block, 0, stream, prm, M, (int)T);
-            return (int)hipGetLastError();
-        }
+        constexpr int NC = CopyWaves<Op>::value;
+        const dim3 grid((unsigned)((M + RD - 1) / RD)), block((1 + NC) * kWave);
+        if (streaming)
+            hipLaunchKernelGGL((stream_kernel_duo<Op, RD, true, NC>), grid, block, 0, stream, prm, M, (int)T);
+        else
+            hipLaunchKernelGGL((stream_kernel_duo<Op, RD, false, NC>), grid, block, 0, stream, prm, M, (int)T);
+        return (int)hipGetLastError();
     }
     if (M < Op::kRows16Below) return launch_stream_rows<Op, 16>(prm, M, T, vec, streaming, stream);
     if constexpr (Op::kRows16Below < kAlways && Op::kRows16Below < Op::kRows32Below)

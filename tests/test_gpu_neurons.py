@@ -249,6 +249,11 @@ def test_fused_rf_equals_the_operator_chain(slayer, shape, w, graded):
     assert torch.equal(b[0].grad, a[0].grad) and torch.equal(b[1].grad, a[1].grad), 'fused input gradients differ'
     assert_rel(b[2].grad.cpu(), a[2].grad.cpu(), 'fused grad sin', rel=1e-4)
     assert_rel(b[3].grad.cpu(), a[3].grad.cpu(), 'fused grad cos', rel=1e-4)
+    # without trainable decays the surrogate moves out of the sequential loop: same input gradients
+    c = [xr.clone().requires_grad_(), xi.clone().requires_grad_()]
+    l_spk = D.rf_fused.dynamics(c[0], c[1], sin, cos, rs, is_, last, w, thr, tau, rho, graded, 2)[2]
+    l_spk.backward(g)
+    assert torch.equal(c[0].grad, a[0].grad) and torch.equal(c[1].grad, a[1].grad), 'lean input gradients differ'
 
 
 def test_rf_neuron_forward_uses_fused_path_with_same_results(slayer):
