@@ -12,9 +12,11 @@ S/neuron/dynamics/).
 Pin status (see tests/test_oracle_*.py):
   li_fwd, spike_fwd (binary)      reference-held fixture gts/dense + scalar spec + closed forms
   res_fwd (no threshold), cspike  reference-held fixture gts/complex_dense + scalar spec
-  res_fwd (threshold mode)        scalar spec + invariants for abs(state) <= 2**24;
-                                  beyond 2**24 the float32 round trip of the reset
-                                  expression is restated but PARITY UNPINNED
+  res_fwd (threshold mode)        reference-held fixture gts/complex_dense (RF_IZ input block) + scalar spec;
+                                  beyond 2**24, where the reset expression rounds through float32:
+                                  vectors computed by the reference's CPU branch
+                                  (tests/golden/make_reference_vectors.py)
+  li_fwd beyond 2**24             the same vectors (float32 reset compare)
   ath_fwd                         scalar spec + closed forms + leak invariants
   apth_fwd, adres_fwd             scalar spec; identity with the pinned pieces they are made of
                                   (ath recurrences + complex spike condition; res_fwd + ath_fwd on imag)

@@ -64,3 +64,26 @@ def complex_input_rf_iz():
                 cos_decay=float(int(0.95 * np.cos(2 * np.pi / 7) * 4096)),
                 threshold=1.1 * 64 / W_SCALE,
                 expected=_unpack(z['iz_out_bits'], T))
+
+
+def reference_big_state_vectors():
+    """Vectors written by make_reference_vectors.py from the reference's CPU branch: states beyond 2**24 at
+    w_scale = 4096 next to a threshold.  Returns (li_cases, res_cases); each case is a dict of float32
+    tensors, expected outputs already divided by w_scale (exact: integers below 2**31 times 2**-12)."""
+    z = np.load(os.path.join(HERE, 'reference_big_state_vectors.npz'))
+
+    def state(a):
+        return (torch.tensor(a.astype(np.float64)) / W_SCALE).float()
+
+    li, res = [], []
+    k = 0
+    while f'li{k}_thr' in z:
+        li.append(dict(threshold=float(z[f'li{k}_thr']), x=torch.tensor(z[f'li{k}_x']), out=state(z[f'li{k}_out'])))
+        k += 1
+    k = 0
+    while f'res{k}_thr' in z:
+        res.append(dict(threshold=float(z[f'res{k}_thr']), xr=torch.tensor(z[f'res{k}_xr']),
+                        xi=torch.tensor(z[f'res{k}_xi']), sin=torch.tensor(z[f'res{k}_sin']),
+                        cos=torch.tensor(z[f'res{k}_cos']), re=state(z[f'res{k}_re']), im=state(z[f'res{k}_im'])))
+        k += 1
+    return li, res

@@ -120,6 +120,24 @@ def test_li_fwd_reset_decision_on_states_beyond_float32_integers(slayer, thr):
     assert_exact(out, ref, f'li_fwd big states thr={thr}')
 
 
+def test_big_state_vectors_of_the_reference_cpu_branch(slayer):
+    """Vectors computed by the reference itself (tests/golden/make_reference_vectors.py): leaky integrator and
+    thresholded resonator with states beyond 2**24, vector kernels and one-thread-per-neuron kernels."""
+    li, res = G.reference_big_state_vectors()
+    D = slayer.neuron.dynamics
+    zero = torch.tensor([0.0], device=dev())
+    for case in li:
+        for debug in (False, True):
+            out = D.leaky_integrator.dynamics(case['x'].to(dev()), zero, zero, G.W_SCALE, case['threshold'], debug=debug)
+            assert_exact(out, case['out'], f"li reference vectors thr={case['threshold']} debug={debug}")
+    for case in res:
+        for debug in (False, True):
+            re, im = D.resonator.dynamics(case['xr'].to(dev()), case['xi'].to(dev()), case['sin'].to(dev()),
+                                          case['cos'].to(dev()), zero, zero, G.W_SCALE, case['threshold'], debug=debug)
+            assert_exact(re, case['re'], f"res reference vectors real thr={case['threshold']} debug={debug}")
+            assert_exact(im, case['im'], f"res reference vectors imag thr={case['threshold']} debug={debug}")
+
+
 def test_li_fwd_negative_and_edge_decays(slayer):
     gen = torch.Generator().manual_seed(7)
     x = sparse_input(gen, (2, 8, 96), p=0.5, amp=30.0)

@@ -96,3 +96,26 @@ def test_rf_iz_fixture_is_sensitive():
     # a different threshold (71 instead of 70.4 in scaled units)
     s, _, _ = _rf_iz(fx, thr=71.5 / W)
     assert _mismatch(s, fx['expected']) > 0
+
+
+def test_li_reset_beyond_float32_integers_matches_reference_vectors():
+    """States beyond 2**24 next to a threshold: vectors computed by the reference's CPU branch
+    (tests/golden/make_reference_vectors.py)."""
+    li, _ = G.reference_big_state_vectors()
+    assert len(li) == 4
+    zero = torch.tensor([0.0])
+    for case in li:
+        assert float(case['out'].abs().max()) * G.W_SCALE > 2 ** 24
+        got = O.li_fwd(case['x'], zero, zero, G.W_SCALE, case['threshold'])
+        assert torch.equal(got, case['out']), case['threshold']
+
+
+def test_resonator_threshold_mode_beyond_float32_integers_matches_reference_vectors():
+    _, res = G.reference_big_state_vectors()
+    assert len(res) == 3
+    zero = torch.tensor([0.0])
+    for case in res:
+        assert float(case['im'].abs().max()) * G.W_SCALE > 2 ** 24
+        re, im = O.res_fwd(case['xr'], case['xi'], case['sin'], case['cos'], zero, zero, G.W_SCALE, case['threshold'])
+        assert torch.equal(re, case['re']), case['threshold']
+        assert torch.equal(im, case['im']), case['threshold']
