@@ -203,3 +203,47 @@ def test_synapse_stack_full_size(slayer):
     lhs = (y.detach().double() * g.double()).sum()
     rhs = (x.double() * slayer.utils.filter.corr(g, filt.to(dev()), 1).double()).sum()
     assert abs(float(lhs - rhs)) <= 1e-5 * abs(float(lhs))
+
+
+@pytest.mark.parametrize('C,T', [(300000, 1000), (150000, 999)])
+def test_tensors_beyond_four_gib(slayer, C, T):
+    """[8, 300000, 1000] float32 is 9.6 GB per tensor (dwordx4 kernels), [8, 150000, 999] 4.8 GB (dword
+    kernels): byte offsets pass 2**32 and, in the first, element offsets pass 2**31 inside the tensor.  Row
+    slabs at the start, around those two lines and at the end are recomputed by the oracle; the fused CUBA
+    block must equal the chain everywhere."""
+    N = 8
+    shape = (N, C, T)
+    D = slayer.neuron.dynamics
+    L = D.leaky_integrator
+    x = gpu_events(shape, 0.03, 0.6, 31 + T)
+    g = gpu_randn(shape, 32 + T)
+    d_i, d_v = torch.tensor([1024.0]), torch.tensor([128.0])
+    zero = torch.zeros(1, device=dev())
+    cur = L.dynamics(x, d_i.to(dev()), zero, 64)
+    vol = L.dynamics(cur, d_v.to(dev()), zero, 64, 1.25)
+    spk = slayer.spike.spike._fwd(vol, None, 1.25, False, 1.0)
+    g_vol = slayer.spike.spike._bwd(g, vol, None, 1.25, 1.0, 1.0, False)
+    g_cur, _ = L._bwd(g_vol, vol, d_v.to(dev()), False)
+    slabs = [(0, slice(0, 70)), (N - 1, slice(C - 70, C))]
+    for line in (1 << 30, 1 << 31):                 # element index of byte 2**32 and element 2**31
+        if line < N * C * T:
+            n0, c0 = divmod(line // T, C)
+            slabs.append((n0, slice(max(c0 - 40, 0), min(c0 + 40, C))))
+    for n, cs in slabs:
+        xs, gs = x[n:n + 1, cs].cpu(), g[n:n + 1, cs].cpu()
+        r_cur = O.li_fwd(xs, d_i, torch.tensor([0.0]), 64)
+        r_vol = O.li_fwd(r_cur, d_v, torch.tensor([0.0]), 64, 1.25)
+        r_spk = O.spike_fwd(r_vol, 1.25)
+        r_gv = O.spike_bwd(gs, r_vol, 1.25, 1.0, 1.0)
+        r_gc, _ = O.li_bwd(g_vol[n:n + 1, cs].cpu(), r_vol, d_v)     # the GPU's own surrogate values: exact compare
+        assert_exact(cur[n:n + 1, cs], r_cur, f'current slab {n} T={T}')
+        assert_exact(vol[n:n + 1, cs], r_vol, f'voltage slab {n} T={T}')
+        assert_exact(spk[n:n + 1, cs], r_spk, f'spike slab {n} T={T}')
+        assert_rel(g_vol[n:n + 1, cs], r_gv, f'spike grad slab {n} T={T}')
+        assert_exact(g_cur[n:n + 1, cs], r_gc, f'li_bwd slab {n} T={T}')
+    assert float(spk.sum()) > 1000
+    del g, g_vol, g_cur
+    f_cur, f_vol, f_spk = D.cuba_fused._fwd(x, d_i.to(dev()), d_v.to(dev()), zero, zero, 64, 1.25, False, 1.0)[:3]
+    assert torch.equal(f_cur, cur) and torch.equal(f_vol, vol) and torch.equal(f_spk, spk)
+    del f_cur, f_vol, f_spk, cur, vol, spk, x
+    torch.cuda.empty_cache()
