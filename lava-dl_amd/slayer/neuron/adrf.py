@@ -3,7 +3,9 @@
 import numpy as np
 import torch
 
+from .base import hardware_decay
 from .rf import ResonatorNeuron
+from . import rf as _rf
 from .dynamics import resonator, adaptive_phase_th
 from ..spike import complex as complex_spike
 from ..utils.quantize import quantize
@@ -15,6 +17,20 @@ SCALE_RHO_MULT = 0.1
 def _exact_range(value):
     """Per-channel ranges of the threshold / refractory decays: a scalar means exactly that value."""
     return [value, value] if np.isscalar(value) else value
+
+
+def neuron_params(device_params, scale=1 << 6, p_scale=1 << 12):
+    """Constructor arguments from a hardware parameter dictionary (neuron/adrf.py:25-55; the step
+    is read from the threshold mantissa there as well)."""
+    params = _rf.neuron_params(device_params, scale, p_scale)
+    return {
+        'threshold': params['threshold'],
+        'threshold_step': device_params['vThMant'] / scale,
+        'period': params['period'],
+        'decay': params['decay'],
+        'threshold_decay': device_params['thDecay'] / p_scale,
+        'refractory_decay': device_params['refDecay'] / p_scale,
+    }
 
 
 class AdaptiveResonatorNeuron(ResonatorNeuron):
@@ -33,6 +49,26 @@ class AdaptiveResonatorNeuron(ResonatorNeuron):
         self.threshold_step = int(threshold_step * self.w_scale) / self.w_scale
         self.threshold_state.fill_(self.threshold)
 
+    cx_threshold_decay = hardware_decay('threshold_decay')
+    cx_refractory_decay = hardware_decay('refractory_decay')
+
+    @property
+    def v_th_step(self):
+        return int(self.threshold_step * self.w_scale)
+
+    @property
+    def device_params(self):
+        return {
+            'type': self.DEVICE_TYPE,
+            'sinDecay': self.cx_sin_decay,
+            'cosDecay': self.cx_cos_decay,
+            'thDecay': self.cx_threshold_decay,
+            'refDecay': self.cx_refractory_decay,
+            'vThMant': self.v_th_mant,
+            'vThStep': self.v_th_step,
+            'gradedSpike': self.graded_spike,
+        }
+
     def _spike_updates_adaptation(self, spike):
         last = spike[..., -1]
         self.refractory_state = adaptive_phase_th.persistent_ref_state(
@@ -47,6 +83,7 @@ class AdaptiveResonatorNeuron(ResonatorNeuron):
 class Neuron(AdaptiveResonatorNeuron):
     """Spikes when the real part reaches threshold + refractory while the imaginary part crosses
     zero upwards; no reset of the resonator state."""
+    DEVICE_TYPE = 'ADRF_PHASE'
 
     def dynamics(self, input):
         """(real, imag, threshold, refractory) traces for ``input = (real_input, imag_input)``."""

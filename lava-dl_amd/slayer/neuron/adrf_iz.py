@@ -2,7 +2,7 @@
 (counterpart of neuron/adrf_iz.py in the reference: call order :574-594, spike :616-645)."""
 import torch
 
-from .adrf import AdaptiveResonatorNeuron
+from .adrf import AdaptiveResonatorNeuron, neuron_params     # noqa: F401  (same translation as adrf)
 from .dynamics import adaptive_resonator
 from ..spike import Spike
 from ..utils.quantize import quantize
@@ -17,6 +17,7 @@ class Neuron(AdaptiveResonatorNeuron):
 
     The reference's ``forward`` hands ``spike`` three arguments where it takes four
     (neuron/adrf_iz.py:669-670) and cannot run; here ``forward`` is ``spike(*dynamics(input))``."""
+    DEVICE_TYPE = 'ADRF_IZHIKEVICH'
 
     def dynamics(self, input):
         """(real, imag, threshold, refractory) traces for ``input = (real_input, imag_input)``."""

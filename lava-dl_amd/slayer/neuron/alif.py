@@ -2,12 +2,25 @@
 (counterpart of neuron/alif.py in the reference: call order :499-525, spike :557-591)."""
 import torch
 
-from .base import Neuron as _Base
+from .base import Neuron as _Base, hardware_decay
 from .dynamics import leaky_integrator, adaptive_threshold, alif_fused
 from ..spike import Spike
 
 TAU_RHO_MULT = 100
 SCALE_RHO_MULT = 0.1
+
+
+def neuron_params(device_params, scale=1 << 6, p_scale=1 << 12):
+    """Constructor arguments from a hardware parameter dictionary (neuron/alif.py:26-52; the step
+    is read from the threshold mantissa there as well)."""
+    return {
+        'threshold': device_params['vThMant'] / scale,
+        'threshold_step': device_params['vThMant'] / scale,
+        'current_decay': device_params['iDecay'] / p_scale,
+        'voltage_decay': device_params['vDecay'] / p_scale,
+        'threshold_decay': device_params['thDecay'] / p_scale,
+        'refractory_decay': device_params['refDecay'] / p_scale,
+    }
 
 
 class Neuron(_Base):
@@ -27,6 +40,33 @@ class Neuron(_Base):
                               threshold_state=lambda: self.threshold, refractory_state=0.0)
         self.threshold_state.fill_(self.threshold)
         self.clamp()
+
+    cx_current_decay = hardware_decay('current_decay')
+    cx_voltage_decay = hardware_decay('voltage_decay')
+    cx_threshold_decay = hardware_decay('threshold_decay')
+    cx_refractory_decay = hardware_decay('refractory_decay')
+
+    @property
+    def v_th_step(self):
+        return int(self.threshold_step * self.w_scale)
+
+    @property
+    def ref_delay(self):
+        return 1
+
+    @property
+    def device_params(self):
+        return {
+            'type': 'ALIF',
+            'iDecay': self.cx_current_decay,
+            'vDecay': self.cx_voltage_decay,
+            'thDecay': self.cx_threshold_decay,
+            'refDecay': self.cx_refractory_decay,
+            'vThMant': self.v_th_mant,
+            'vThStep': self.v_th_step,
+            'refDelay': self.ref_delay,
+            'gradedSpike': self.graded_spike,
+        }
 
     def dynamics(self, input):
         """(current, voltage, threshold, refractory) traces."""

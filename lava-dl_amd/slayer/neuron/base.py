@@ -4,8 +4,7 @@ These modules reproduce what the reference's neuron classes do around the
 dynamics kernels (neuron/base.py:60-217, neuron/cuba.py:108-440 in the
 reference): parameter scaling and quantisation, lazily shaped state buffers,
 persistent state across calls, the threshold epsilon and the surrogate-gradient
-constants.  Export helpers (device_params, cx_* properties) are not part of the
-compute path and are left out.
+constants, and the hardware view of the parameters (cx_* integers, device_params).
 """
 import numpy as np
 import torch
@@ -13,6 +12,17 @@ import torch
 from ..utils.quantize import quantize
 
 P_SCALE = 1 << 12      # decays are stored as 12-bit integers
+
+
+def hardware_decay(name):
+    """Property returning a decay parameter as the integer(s) the hardware is configured with:
+    clamped, rounded, a plain int when shared and an int array per channel otherwise
+    (neuron/cuba.py:231-251 in the reference)."""
+    def get(self):
+        self.clamp()
+        val = quantize(getattr(self, name)).cpu().data.numpy().astype(int)
+        return val[0] if len(val) == 1 else val
+    return property(get, doc=f'{name} as configured on the hardware (12-bit integer).')
 
 
 class Neuron(torch.nn.Module):
@@ -54,6 +64,21 @@ class Neuron(torch.nn.Module):
         steps of 2 / scale, clamped to the 8-bit range; ``descale`` returns integers."""
         q = quantize(weight, step=2 / self.w_scale).clamp(-256 / self.w_scale, 254 / self.w_scale)
         return q * self.w_scale if descale else q
+
+    # --------------------------------------------------------------- hardware view
+    @property
+    def scale(self):
+        """Factor between this representation of the states and the hardware's."""
+        return self.w_scale
+
+    @property
+    def weight_exponent(self):
+        return int(np.log2(self.s_scale // self.w_scale) - 6)
+
+    @property
+    def v_th_mant(self):
+        """Threshold mantissa."""
+        return int(self.threshold * self.w_scale)
 
     def _register_decays(self, **decays):
         """Shared: one value each.  Per channel: remember [min, max] (a scalar means +-1 %)

@@ -2,12 +2,21 @@
 (counterpart of neuron/cuba.py in the reference: call order :356-374, spike :401-421)."""
 import torch
 
-from .base import Neuron as _Base
+from .base import Neuron as _Base, hardware_decay
 from .dynamics import leaky_integrator, cuba_fused
 from ..spike import Spike
 
 TAU_RHO_MULT = 100      # surrogate-gradient constants of the CUBA family (neuron/cuba.py:20-21)
 SCALE_RHO_MULT = 0.1
+
+
+def neuron_params(device_params, scale=1 << 6, p_scale=1 << 12):
+    """Constructor arguments from a hardware parameter dictionary (neuron/cuba.py:26-49)."""
+    return {
+        'threshold': device_params['vThMant'] / scale,
+        'current_decay': device_params['iDecay'] / p_scale,
+        'voltage_decay': device_params['vDecay'] / p_scale,
+    }
 
 
 class Neuron(_Base):
@@ -25,6 +34,24 @@ class Neuron(_Base):
         self._register_decays(current_decay=current_decay, voltage_decay=voltage_decay)
         self._register_states(current_state=0.0, voltage_state=0.0)
         self.clamp()
+
+    cx_current_decay = hardware_decay('current_decay')
+    cx_voltage_decay = hardware_decay('voltage_decay')
+
+    @property
+    def ref_delay(self):
+        return 1
+
+    @property
+    def device_params(self):
+        return {
+            'type': 'CUBA',
+            'iDecay': self.cx_current_decay,
+            'vDecay': self.cx_voltage_decay,
+            'vThMant': self.v_th_mant,
+            'refDelay': self.ref_delay,
+            'gradedSpike': self.graded_spike,
+        }
 
     def dynamics(self, input):
         """(current, voltage) traces; the voltage already carries the reset."""

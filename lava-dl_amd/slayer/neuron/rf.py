@@ -3,13 +3,24 @@
 import numpy as np
 import torch
 
-from .base import Neuron as _Base
+from .base import Neuron as _Base, hardware_decay
 from .dynamics import resonator, rf_fused
 from ..spike import complex as complex_spike
 from ..utils.quantize import quantize
 
 TAU_RHO_MULT = 0.5      # surrogate-gradient constants of the RF family (neuron/rf.py:19-20)
 SCALE_RHO_MULT = 10
+
+
+def neuron_params(device_params, scale=1 << 6, p_scale=1 << 12):
+    """Constructor arguments from a hardware parameter dictionary (neuron/rf.py:23-50)."""
+    sin_decay = device_params['sinDecay'] / p_scale
+    cos_decay = device_params['cosDecay'] / p_scale
+    return {
+        'threshold': device_params['vThMant'] / scale,
+        'period': 1 / (np.arctan2(sin_decay, cos_decay) / 2 / np.pi),
+        'decay': 1 - np.sqrt(sin_decay ** 2 + cos_decay ** 2),
+    }
 
 
 class ResonatorNeuron(_Base):
@@ -67,6 +78,43 @@ class ResonatorNeuron(_Base):
             self.sin_decay.data.clamp_(1)
             self.cos_decay.data.clamp_(0)
 
+    DEVICE_TYPE = None
+    cx_sin_decay = hardware_decay('sin_decay')
+    cx_cos_decay = hardware_decay('cos_decay')
+
+    @property
+    def decay(self):
+        """1 - gain per step, from the rounded rotation parameters."""
+        self.clamp()
+        s = quantize(self.sin_decay).cpu().data.numpy() / self.p_scale
+        c = quantize(self.cos_decay).cpu().data.numpy() / self.p_scale
+        return 1 - np.sqrt(s ** 2 + c ** 2)
+
+    @property
+    def lam(self):
+        return -np.log(1 - self.decay)
+
+    @property
+    def frequency(self):
+        """Rotations per step."""
+        self.clamp()
+        return np.arctan2(quantize(self.sin_decay).cpu().data.numpy(),
+                          quantize(self.cos_decay).cpu().data.numpy()) / 2 / np.pi
+
+    @property
+    def period(self):
+        return 1 / self.frequency
+
+    @property
+    def device_params(self):
+        return {
+            'type': self.DEVICE_TYPE,
+            'sinDecay': self.cx_sin_decay,
+            'cosDecay': self.cx_cos_decay,
+            'vThMant': self.v_th_mant,
+            'gradedSpike': self.graded_spike,
+        }
+
     def _draw_per_channel(self, channels, device):
         (p_lo, p_hi), (d_lo, d_hi) = self._period_range, self._decay_range
         if self.log_init:
@@ -99,6 +147,7 @@ class Neuron(ResonatorNeuron):
     """``Neuron(threshold, period, decay, ...)``: the state rotates by 2 pi / period per step and
     shrinks by (1 - decay); it spikes when the real part is above threshold while the imaginary
     part crosses zero upwards.  ``forward((real_input, imag_input))`` returns the spikes."""
+    DEVICE_TYPE = 'RF_PHASE'
 
     def dynamics(self, input):
         """(real, imag) traces for ``input = (real_input, imag_input)``."""

@@ -2,7 +2,7 @@
 (counterpart of neuron/rf_iz.py in the reference: call order :433-441, spike :463-489)."""
 import torch
 
-from .rf import ResonatorNeuron
+from .rf import ResonatorNeuron, neuron_params     # noqa: F401  (same translation as rf)
 from .dynamics import resonator
 from ..spike import Spike
 from ..utils.quantize import quantize
@@ -15,6 +15,7 @@ class Neuron(ResonatorNeuron):
     """``Neuron(threshold, period, decay, ...)``: a resonator that spikes when its imaginary part
     reaches the threshold; the spike resets the real part to zero and the imaginary part to just
     below the threshold."""
+    DEVICE_TYPE = 'RF_IZHIKEVICH'
 
     def dynamics(self, input):
         """(real, imag) traces for ``input = (real_input, imag_input)``."""

@@ -8,6 +8,11 @@ from ..axon.delta import Delta
 from ..dendrite.sigma import Sigma
 
 
+def neuron_params(device_params, scale=1 << 6):
+    """Constructor arguments from a hardware parameter dictionary (neuron/sigma_delta.py:15-33)."""
+    return {'threshold': device_params['vThMant'] / scale}
+
+
 class Neuron(_Base):
     """``Neuron(threshold, activation, ...)``: ``delta(activation(sigma(input) [+ bias]))``; the
     output events are graded.  ``set_bias`` adds a per-neuron bias before the activation."""
@@ -31,6 +36,14 @@ class Neuron(_Base):
     @property
     def threshold(self):
         return self.delta.threshold
+
+    @property
+    def device_params(self):
+        return {
+            'type': 'SDNN',
+            'activation': self.activation.__name__,
+            'vThMant': self.v_th_mant,
+        }
 
     def set_bias(self, bias):
         self.bias.data = (bias if self.shape is None else bias.reshape(self.shape)).to(self.bias.device)

@@ -10,3 +10,16 @@ def right_shift_to_zero(x, bits):
         raise Exception(f'Expected torch.int32 or torch.int64 data, found {x.dtype}.')
     magnitude = torch.abs(x) >> bits
     return (torch.sign(x) * magnitude).to(x.dtype)
+
+
+class Q2Zero(torch.autograd.Function):
+    """Truncation toward zero of a float tensor with an identity gradient (utils/int_utils.py:35-50
+    in the reference; a verification aid, not used by the kernels)."""
+
+    @staticmethod
+    def forward(ctx, x):
+        return torch.trunc(x).to(torch.int32).to(x.dtype)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return grad_output

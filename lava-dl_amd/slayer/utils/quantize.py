@@ -31,3 +31,12 @@ def quantize(input, step=1, mode=MODE.ROUND):
         scaled = input / step
         return (torch.floor(scaled) if mode == MODE.FLOOR else torch.round(scaled)) * step
     return _StraightThrough.apply(input, step, mode == MODE.FLOOR)
+
+
+def quantize_hook_fx(x, scale=1 << 6, num_bits=8, descale=False):
+    """Synapse pre-hook quantiser (utils/quantize.py:84-115 in the reference): even multiples of
+    1 / scale, limited to the signed ``num_bits`` weight range; ``descale`` returns integers."""
+    lo = -2 * (1 << num_bits) / scale
+    hi = 2 * ((1 << num_bits) - 1) / scale
+    q = quantize(x, step=2 / scale).clamp(lo, hi)
+    return q * scale if descale else q

@@ -1,3 +1,4 @@
+from .replicate import replicate
 from .shift import shift
 
-__all__ = ['shift']
+__all__ = ['replicate', 'shift']
