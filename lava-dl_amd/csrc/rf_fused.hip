@@ -59,18 +59,21 @@ struct RfFwd {
     }
 };
 
-// DECAY_GRAD = false: the saved real / imag parts are needed by the spike surrogate only, which does not
-// depend on the recurrence; it is then evaluated on the way into LDS (by all 64 lanes, or by the copy
-// waves of the multi-wave kernel) and its two results take the places of real and imag.
-template <bool GRADED, bool DECAY_GRAD>
+// The spike surrogate does not depend on the recurrence.  STAGED = true evaluates it on the way into LDS (by
+// the copy waves of the multi-wave kernel) and the sequential wave keeps only the rotation: without decay
+// gradients its two results take the places of real and imag; with them real and imag are still needed for
+// the partial sums, so a fourth input slot without a tensor behind it receives the second result.
+template <bool GRADED, bool DECAY_GRAD, bool STAGED>
 struct RfBwd {
-    static constexpr int kIn = 3, kOut = 2;          // in: grad of spikes, saved real, saved imag
-    static constexpr bool kTransforms = !DECAY_GRAD;
-    static constexpr int kCopyWaves = DECAY_GRAD ? 1 : 4;
+    static_assert(DECAY_GRAD || STAGED, "without decay gradients the surrogate is always staged");
+    static constexpr int kIn = (DECAY_GRAD && STAGED) ? 4 : 3;     // grad of spikes, saved real, saved imag[, free slot]
+    static constexpr int kOut = 2;
+    static constexpr bool kTransforms = STAGED;
+    static constexpr int kCopyWaves = STAGED ? 4 : 1;
     static constexpr bool kReverse = true;
     static constexpr int64_t kRows32Below = 4096, kRows16Below = 4096;     // exp per step: keep all lanes busy
     struct Params {
-        const float* in[3];
+        const float* in[kIn];
         float* out[2];
         const float *sin_decay, *cos_decay;
         float *partial_sin, *partial_cos;
@@ -104,21 +107,22 @@ struct RfBwd {
         g_re = g * ((rho * d_re) * d_im);
         g_im = g * (((neg_rho_over_tau * sg_i) * d_im) * step_re);
     }
-    __device__ __forceinline__ void pre(float4 (&x)[3]) const {
+    __device__ __forceinline__ void pre(float4 (&x)[kIn]) const {
         float4 a, b;
         surrogate(x[0].x, x[1].x, x[2].x, a.x, b.x);
         surrogate(x[0].y, x[1].y, x[2].y, a.y, b.y);
         surrogate(x[0].z, x[1].z, x[2].z, a.z, b.z);
         surrogate(x[0].w, x[1].w, x[2].w, a.w, b.w);
-        x[1] = a;
-        x[2] = b;
+        if (DECAY_GRAD) { x[0] = a; x[kIn - 1] = b; }
+        else { x[1] = a; x[2] = b; }
     }
     __device__ __forceinline__ void post(float4 (&)[2]) const {}
-    __device__ __forceinline__ void step(const float (&x)[3], float (&o)[2]) {
+    __device__ __forceinline__ void step(const float (&x)[kIn], float (&o)[2]) {
         float g_re, g_im;
         if (DECAY_GRAD) {
             const float r = x[1], i = x[2];
-            surrogate(x[0], r, i, g_re, g_im);
+            if (STAGED) { g_re = x[0]; g_im = x[kIn - 1]; }
+            else surrogate(x[0], r, i, g_re, g_im);
             // gr, gi still hold the gradients of step t+1
             acc_s = __fmaf_rn(gi, r, __fmaf_rn(-gr, i, acc_s));
             acc_c = __fmaf_rn(gi, i, __fmaf_rn(gr, r, acc_c));
@@ -188,22 +192,24 @@ extern "C" int slayer_rf_bwd(float* g_re_in, float* g_im_in, float* grad_sin, fl
     hipStream_t st = (hipStream_t)stream;
     if (M > 0 && T > 0) {
         if (!g_re_in || !g_im_in || !grad_spikes || !re || !im || !sin_decay || !cos_decay) return SLAYER_ENULL;
-#define SLAYER_RF_BWD(G, D)                                                                                       \
+#define SLAYER_RF_BWD(G, D, S)                                                                                    \
     do {                                                                                                          \
-        RfBwd<G, D>::Params p{{grad_spikes, re, im}, {g_re_in, g_im_in}, sin_decay, cos_decay,                      \
-                              want ? workspace : nullptr, want ? workspace + M : nullptr,                         \
-                              spike_threshold, tau_rho, scale_rho, neurons_per_batch, num_decays};                \
-        if (D || stream_fits_multiwave<RfBwd<G, D>>(p, M, T)) {                                                   \
-            if (int e = launch_stream<RfBwd<G, D>>(p, M, T, st)) return e;                                        \
+        using Op = RfBwd<G, D, S>;                                                                                \
+        Op::Params p{{grad_spikes, re, im}, {g_re_in, g_im_in}, sin_decay, cos_decay,                             \
+                     want ? workspace : nullptr, want ? workspace + M : nullptr,                                  \
+                     spike_threshold, tau_rho, scale_rho, neurons_per_batch, num_decays};                         \
+        if (!S || stream_fits_multiwave<Op>(p, M, T)) {                                                           \
+            if (int e = launch_stream<Op>(p, M, T, st)) return e;                                                 \
             done = true;                                                                                          \
         }                                                                                                         \
     } while (0)
-        // Without decay gradients the surrogate can run in the copy waves of the multi-wave kernel (three
-        // times faster there); the one-wave kernel gains nothing from that split, so large tensors take
-        // the other form with its partial sums dropped.
+        // The staged forms pay off in the multi-wave kernel (three times faster there); the one-wave kernel
+        // gains nothing from the split, so large tensors take the unstaged form (partial sums dropped when
+        // the decay gradients are not wanted).
         bool done = false;
-        if (!want) { if (graded) SLAYER_RF_BWD(true, false); else SLAYER_RF_BWD(false, false); }
-        if (!done) { if (graded) SLAYER_RF_BWD(true, true); else SLAYER_RF_BWD(false, true); }
+        if (graded) { if (want) SLAYER_RF_BWD(true, true, true); else SLAYER_RF_BWD(true, false, true); }
+        else { if (want) SLAYER_RF_BWD(false, true, true); else SLAYER_RF_BWD(false, false, true); }
+        if (!done) { if (graded) SLAYER_RF_BWD(true, true, false); else SLAYER_RF_BWD(false, true, false); }
 #undef SLAYER_RF_BWD
     }
     if (want) {

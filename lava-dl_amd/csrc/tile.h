@@ -118,7 +118,8 @@ struct TileGeom {
 //     the same step: it is computed while a quad is copied out and needs neither an LDS tile nor
 //     boundary registers
 //   static constexpr int64_t kRows32Below, kRows16Below;   (rows-per-wave policy, see launch_stream)
-//   struct Params { const float* in[kIn]; float* out[kOut]; ... };   (a null out[] entry is not stored)
+//   struct Params { const float* in[kIn]; float* out[kOut]; ... };   (a null out[] entry is not stored, a null
+//     in[] entry other than in[0] reads as zeros: a slot for pre() to fill)
 //   __device__ void init(const Params&, int64_t m, bool valid);
 //   __device__ void step(const float (&x)[kIn], float (&y)[kOut]);
 //   __device__ void finish(const Params&, int64_t m, bool valid);
@@ -203,7 +204,8 @@ struct Copier {
         rows = rows_; T = T_; first_pass = first_pass_;
         const unsigned wave_bytes = (unsigned)rows * (unsigned)T * 4u;
 #pragma unroll
-        for (int i = 0; i < NI; ++i) src[i] = make_rsrc(prm.in[i] + m0 * (int64_t)T, wave_bytes);
+        for (int i = 0; i < NI; ++i)         // an input the caller does not have: every load falls out of range, reads 0
+            src[i] = prm.in[i] ? make_rsrc(prm.in[i] + m0 * (int64_t)T, wave_bytes) : make_rsrc(nullptr, 0);
 #pragma unroll
         for (int o = 0; o < NO + ND; ++o)    // an output the caller does not want: every store falls out of range
             dst[o] = prm.out[o] ? make_rsrc(prm.out[o] + m0 * (int64_t)T, wave_bytes) : make_rsrc(nullptr, 0);
@@ -519,7 +521,7 @@ __global__ __launch_bounds__(kWave) void stream_kernel_scalar(typename Op::Param
 #pragma unroll
             for (int i = 0; i < NI; ++i) {
                 float4 v = make_float4(0.f, 0.f, 0.f, 0.f);      // zero fill: steps past T-1 must be no-ops
-                if (r < rows) {
+                if (r < rows && prm.in[i]) {
                     const float* src = prm.in[i] + off;
                     if (t + 0 < T) v.x = src[0];
                     if (t + 1 < T) v.y = src[1];
