@@ -272,7 +272,8 @@ int slayer_cuba_bwd(float *grad_in, float *grad_i_decay, float *grad_v_decay,
  * slayer_cspike_fwd, 20 instead of 28 bytes per neuron-timestep.  imag_last is the imaginary sample
  * before step 0 (num_last == 1 broadcasts).  re_out / im_out may both be NULL when no backward pass
  * will follow (inference: 12 bytes); re_last_out / im_last_out ([M], both or neither NULL) receive
- * real[..., -1] and imag[..., -1] for a persistent state. */
+ * real[..., -1] and imag[..., -1] for a persistent state.  w_scale must be positive (SLAYER_EINVAL
+ * otherwise): the spike conditions are decided on the integer states. */
 int slayer_rf_fwd(float *re_out, float *im_out, float *spk_out, float *re_last_out, float *im_last_out,
                   const float *re_in, const float *im_in,
                   const float *sin_decay, const float *cos_decay,

@@ -12,50 +12,70 @@ int launch_reduce_param_grad(float* grad, const float* partial, float* scratch, 
                              int64_t num_params, hipStream_t stream);   // li.hip
 int launch_zero_fill(float* p, int64_t n, hipStream_t stream);          // li.hip
 
+// Integer tiles: inputs are scaled and truncated on the way into LDS, the states leave the sequential
+// loop as integers together with the spike decision (taken on the integers: real part above the largest
+// state whose output value is still below the threshold, previous imaginary state negative, new one not),
+// and become output values and spikes on the way out.
 template <bool POW2, bool GRADED>
 struct RfFwd {
     static constexpr int kIn = 2, kOut = 3;          // out: real, imag, spikes
     static constexpr bool kReverse = false;
+    static constexpr bool kTransforms = true;
     static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
     struct Params {
         const float* in[2];
         float* out[3];
         float *re_last, *im_last;                   // [M] real / imaginary part of the last step, or nullptr
         const float *sin_decay, *cos_decay, *re_state, *im_state, *imag_last;
-        float w, inv_w, spike_thr, spike_scale;
+        float w, inv_w, spike_scale;
+        int fire_above;                             // a real state above this is at or over the spike threshold
         int64_t npb, nd, n_rs, n_is, n_last;
     };
-    int re, im, s, c;
-    float w, inv_w, spike_thr, spike_scale, im_prev, re_prev;
+    int re, im, im_prev, s, c, fire_above;
+    float w, inv_w, spike_scale;
 
     __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
-        w = p.w; inv_w = p.inv_w; spike_thr = p.spike_thr; spike_scale = p.spike_scale;
-        re = im = s = c = 0; im_prev = re_prev = 0.f;
+        w = p.w; inv_w = p.inv_w; spike_scale = p.spike_scale; fire_above = p.fire_above;
+        re = im = im_prev = s = c = 0;
         if (valid) {
             re = trunc_i32(p.re_state[p.n_rs == 1 ? 0 : m] * w);
             im = trunc_i32(p.im_state[p.n_is == 1 ? 0 : m] * w);
             const int64_t j = param_index(m, p.npb, p.nd);
             s = trunc_i32(p.sin_decay[j]);
             c = trunc_i32(p.cos_decay[j]);
-            im_prev = p.imag_last[p.n_last == 1 ? 0 : m];
+            im_prev = (p.imag_last[p.n_last == 1 ? 0 : m] < 0.0f) ? -1 : 0;      // only its sign matters
         }
     }
+    __device__ __forceinline__ void pre(float4 (&x)[2]) const {
+        x[0] = to_state(x[0], w);
+        x[1] = to_state(x[1], w);
+    }
     __device__ __forceinline__ void step(const float (&x)[2], float (&o)[3]) {
-        const int re_n = rs0_12(c, re) - rs0_12(s, im) + trunc_i32(w * x[0]);
-        const int im_n = rs0_12(s, re) + rs0_12(c, im) + trunc_i32(w * x[1]);
-        re = re_n; im = im_n;
-        const float ref = (float)re_n, imf = (float)im_n;
-        const float r = POW2 ? ref * inv_w : ref / w;
-        const float i = POW2 ? imf * inv_w : imf / w;
-        const float a = (r >= spike_thr) ? 1.0f : 0.0f, b = (im_prev < 0.0f) ? 1.0f : 0.0f, cc = (i >= 0.0f) ? 1.0f : 0.0f;
-        o[0] = r;
-        o[1] = i;
-        o[2] = GRADED ? (((r * a) * b) * cc) / spike_scale : (a * b) * cc;
-        im_prev = i;
-        re_prev = r;
+        const int re_n = rs0_12(c, re) - rs0_12(s, im) + __float_as_int(x[0]);
+        const int im_n = rs0_12(s, re) + rs0_12(c, im) + __float_as_int(x[1]);
+        const bool fired = (re_n > fire_above) & (im_prev < 0) & (im_n >= 0);
+        re = re_n; im = im_n; im_prev = im_n;
+        o[0] = __int_as_float(re_n);
+        o[1] = __int_as_float(im_n);
+        o[2] = __int_as_float(fired ? 1 : 0);
+    }
+    // the reference multiplies the real part by the three conditions one after the other: a spike that
+    // does not fire is a zero with the sign of the real part
+    __device__ __forceinline__ float spike(float r, float flag) const {
+        const bool fired = __float_as_int(flag) != 0;
+        if (GRADED) return (fired ? r : r * 0.0f) / spike_scale;
+        return fired ? 1.0f : 0.0f;
+    }
+    __device__ __forceinline__ void post(float4 (&y)[3]) const {
+        y[0] = from_state<POW2>(y[0], w, inv_w);
+        y[1] = from_state<POW2>(y[1], w, inv_w);
+        y[2] = make_float4(spike(y[0].x, y[2].x), spike(y[0].y, y[2].y), spike(y[0].z, y[2].z), spike(y[0].w, y[2].w));
     }
     __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
-        if (valid && p.re_last) { p.re_last[m] = re_prev; p.im_last[m] = im_prev; }
+        if (valid && p.re_last) {
+            p.re_last[m] = from_state<POW2>(__int_as_float(re), w, inv_w);
+            p.im_last[m] = from_state<POW2>(__int_as_float(im), w, inv_w);
+        }
     }
 };
 
@@ -162,13 +182,14 @@ extern "C" int slayer_rf_fwd(float* re_out, float* im_out, float* spk_out, float
     if (int e = check_params(M, neurons_per_batch, num_decays)) return e;
     for (int64_t n : {num_re_states, num_im_states, num_last})
         if (int e = check_states(M, n)) return e;
-    if (w_scale == 0) return SLAYER_EINVAL;
+    if (w_scale <= 0) return SLAYER_EINVAL;
     const float w = (float)w_scale;
+    const int fire = fire_above_scaled(spike_threshold, w, is_pow2(w_scale));
     hipStream_t st = (hipStream_t)stream;
 #define SLAYER_RF(P, G)                                                                                          \
     do {                                                                                                         \
         RfFwd<P, G>::Params p{{re_in, im_in}, {re_out, im_out, spk_out}, re_last_out, im_last_out, sin_decay, cos_decay, re_state,   \
-                              im_state, imag_last, w, 1.0f / w, spike_threshold, spike_scale, neurons_per_batch,   \
+                              im_state, imag_last, w, 1.0f / w, spike_scale, fire, neurons_per_batch,              \
                               num_decays,                                                                          \
                               num_re_states, num_im_states, num_last};                                             \
         return launch_stream<RfFwd<P, G>>(p, M, T, st);                                                            \

@@ -42,6 +42,25 @@ inline int fire_above(float thr) {
     return (int)(c - 1);
 }
 
+// The same for a compare made on the converted state: largest integer y whose output value
+// (float32(y) * (1 / w) for a power-of-two w, float32(y) / w otherwise, w > 0) is below thr, found by
+// bisection with the very operations the kernels use (both are monotone in y).
+inline int fire_above_scaled(float thr, float w, bool pow2) {
+    const float inv_w = 1.0f / w;
+    auto below = [&](long long y) {
+        const float f = (float)y;
+        return (pow2 ? f * inv_w : f / w) < thr;
+    };
+    long long lo = -2147483648LL, hi = 2147483647LL;
+    if (!below(lo)) return (int)lo;          // every state fires except the most negative one
+    if (below(hi) || !(thr == thr)) return (int)hi;
+    while (hi - lo > 1) {
+        const long long mid = lo + (hi - lo) / 2;
+        if (below(mid)) lo = mid; else hi = mid;
+    }
+    return (int)lo;
+}
+
 // Integer tiles: an Op with kTransforms can keep its fixed-point states in LDS as integers (bit
 // patterns in float registers).  Inputs are scaled and truncated on the way in, states converted
 // and scaled back on the way out.
