@@ -15,29 +15,33 @@ int launch_zero_fill(float* p, int64_t n, hipStream_t stream);          // li.hi
 
 // KEEP_CURRENT = false leaves the current trace out (a caller that wants no decay gradient does not
 // need it): 16 instead of 20 bytes per neuron-timestep.
+//
+// Integer tiles: the input is scaled and truncated on the way into LDS; current, voltage, threshold and
+// refractory state leave the sequential loop as integers in four tiles and become current, voltage,
+// threshold + refractory and spikes on the way out (the tile of the refractory state carries the spikes
+// to memory).
 template <bool POW2, bool GRADED, bool KEEP_CURRENT>
 struct AlifFwd {
-    static constexpr int kIn = 1, kOut = KEEP_CURRENT ? 3 : 2;   // out: [current,] voltage, threshold + refractory
-    static constexpr int kVol = kOut - 2, kTheta = kOut - 1;
-    static constexpr int kDerived = 1;               // spikes: a function of voltage and threshold + refractory
+    static constexpr int kIn = 1, kOut = KEEP_CURRENT ? 4 : 3;   // out: [current,] voltage, threshold + refractory, spikes
+    static constexpr int kVol = kOut - 3, kTheta = kOut - 2, kSpk = kOut - 1;
     static constexpr bool kReverse = false;
+    static constexpr bool kTransforms = true;
     static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
     struct Params {
         const float* in[1];
-        float* out[kOut + 1];
+        float* out[kOut];
         float *cur_last, *vol_last, *th_last, *ref_last;   // [M] values of the last step, or nullptr
         const float *i_decay, *v_decay, *th_decay, *ref_decay, *i_state, *v_state, *th_state, *ref_state;
         int step, base;
         float w, inv_w, spike_scale;
         int64_t npb, n_id, n_vd, n_td, n_rd, n_is, n_vs, n_ts, n_rs;
     };
-    int yc, yv, th, r, mi, mv, mt, mr, th_step, base;
-    float w, inv_w, spike_scale, th_f, ref_f, cur_f, vol_f;
+    int yc, yv, th, r, th_out, r_out, mi, mv, mt, mr, th_step, base;
+    float w, inv_w, spike_scale;
 
     __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
         w = p.w; inv_w = p.inv_w; spike_scale = p.spike_scale; th_step = p.step; base = p.base;
-        yc = yv = th = r = mi = mv = mt = mr = 0;
-        th_f = ref_f = cur_f = vol_f = 0.f;
+        yc = yv = th = r = th_out = r_out = mi = mv = mt = mr = 0;
         if (valid) {
             yc = trunc_i32(p.i_state[p.n_is == 1 ? 0 : m] * w);
             yv = trunc_i32(p.v_state[p.n_vs == 1 ? 0 : m] * w);
@@ -49,39 +53,47 @@ struct AlifFwd {
             mr = 4096 - trunc_i32(p.ref_decay[param_index(m, p.npb, p.n_rd)]);
         }
     }
+    // what the next operator reads of a state: trunc(w * (float(y) / w)); for a power of two the scaling
+    // is exact and only the int -> float32 rounding remains
+    __device__ __forceinline__ int reread(int y) const {
+        const float f = (float)y;
+        return POW2 ? trunc_i32(f) : trunc_i32(w * (f / w));
+    }
+    __device__ __forceinline__ void pre(float4 (&x)[1]) const { x[0] = to_state(x[0], w); }
     __device__ __forceinline__ void step(const float (&x)[1], float (&o)[kOut]) {
-        yc = rs0_12(yc, mi) + trunc_i32(w * x[0]);
-        const float cf = (float)yc;
-        const float cur = POW2 ? cf * inv_w : cf / w;
-        yv = rs0_12(yv, mv) + trunc_i32(w * cur);               // the voltage op reads the float32 current
-        const float vf = (float)yv;
-        const float vol = POW2 ? vf * inv_w : vf / w;
+        yc = rs0_12(yc, mi) + __float_as_int(x[0]);
+        yv = rs0_12(yv, mv) + reread(yc);                       // the voltage op reads the float32 current
         r = rs0_12(r, mr);
         th = rs0_12(th - base, mt) + base;
-        const float thf = (float)th, rf = (float)r;
-        th_f = POW2 ? thf * inv_w : thf / w;
-        ref_f = POW2 ? rf * inv_w : rf / w;
-        const bool fired = trunc_i32(w * vol) >= th + r;        // the threshold op reads the float32 voltage
+        th_out = th; r_out = r;
+        const bool fired = reread(yv) >= th + r;                // the threshold op reads the float32 voltage
         r += fired ? 2 * th : 0;
         th += fired ? th_step : 0;
-        if (KEEP_CURRENT) o[0] = cur;
-        cur_f = cur;
-        vol_f = vol;
-        o[kVol] = vol;
-        o[kTheta] = th_f + ref_f;
+        if (KEEP_CURRENT) o[0] = __int_as_float(yc);
+        o[kVol] = __int_as_float(yv);
+        o[kTheta] = __int_as_float(th_out);
+        o[kSpk] = __int_as_float(r_out);
     }
     __device__ __forceinline__ float spike(float vol, float theta) const {
         const float h = (vol >= theta) ? 1.0f : 0.0f;
         return GRADED ? (h * vol) / spike_scale : h;
     }
-    __device__ __forceinline__ float4 derive(const float4 (&y)[kOut]) const {
-        return make_float4(spike(y[kVol].x, y[kTheta].x), spike(y[kVol].y, y[kTheta].y),
-                           spike(y[kVol].z, y[kTheta].z), spike(y[kVol].w, y[kTheta].w));
+    __device__ __forceinline__ void post(float4 (&y)[kOut]) const {
+        if (KEEP_CURRENT) y[0] = from_state<POW2>(y[0], w, inv_w);
+        const float4 vol = from_state<POW2>(y[kVol], w, inv_w);
+        const float4 thf = from_state<POW2>(y[kTheta], w, inv_w), rf = from_state<POW2>(y[kSpk], w, inv_w);
+        const float4 theta = make_float4(thf.x + rf.x, thf.y + rf.y, thf.z + rf.z, thf.w + rf.w);
+        y[kVol] = vol;
+        y[kTheta] = theta;
+        y[kSpk] = make_float4(spike(vol.x, theta.x), spike(vol.y, theta.y), spike(vol.z, theta.z), spike(vol.w, theta.w));
     }
     __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
-        if (valid && p.th_last) { p.th_last[m] = th_f; p.ref_last[m] = ref_f; }
-        if (valid && p.cur_last) p.cur_last[m] = cur_f;
-        if (valid && p.vol_last) p.vol_last[m] = vol_f;
+        if (valid && p.th_last) {
+            p.th_last[m] = from_state<POW2>(__int_as_float(th_out), w, inv_w);
+            p.ref_last[m] = from_state<POW2>(__int_as_float(r_out), w, inv_w);
+        }
+        if (valid && p.cur_last) p.cur_last[m] = from_state<POW2>(__int_as_float(yc), w, inv_w);
+        if (valid && p.vol_last) p.vol_last[m] = from_state<POW2>(__int_as_float(yv), w, inv_w);
     }
 };
 
