@@ -6,6 +6,7 @@ operator raises when handed a tensor that is not float32 on a GPU.
 """
 import ctypes
 import os
+import threading
 
 import torch
 
@@ -15,6 +16,7 @@ LIB_PATH = os.environ.get('SLAYER_HIP_LIB') or os.path.join(_HERE, 'libslayer_hi
 ABI_VERSION = 1
 
 _lib = None
+_lib_lock = threading.Lock()       # forward runs on the user thread, backward on an autograd thread
 
 _P = ctypes.c_void_p
 _I64 = ctypes.c_int64
@@ -70,19 +72,22 @@ def lib():
     which has the same soname as the one the library was linked against, is the
     single runtime in the process)."""
     global _lib
-    if _lib is None:
-        if not os.path.exists(LIB_PATH):
-            raise RuntimeError(
-                f'{LIB_PATH} is missing: build it with `make -C lava-dl_amd/csrc` '
-                '(hipcc, gfx950). There is no fallback implementation.')
-        handle = ctypes.CDLL(LIB_PATH)
-        for name, (res, args) in _SIGNATURES.items():
-            fn = getattr(handle, name)
-            fn.restype = res
-            fn.argtypes = args
-        if handle.slayer_abi_version() != ABI_VERSION:
-            raise RuntimeError('libslayer_hip.so ABI version mismatch; rebuild the library')
-        _lib = handle
+    if _lib is not None:
+        return _lib
+    with _lib_lock:
+        if _lib is None:
+            if not os.path.exists(LIB_PATH):
+                raise RuntimeError(
+                    f'{LIB_PATH} is missing: build it with `make -C lava-dl_amd/csrc` '
+                    '(hipcc, gfx950). There is no fallback implementation.')
+            handle = ctypes.CDLL(LIB_PATH)
+            for name, (res, args) in _SIGNATURES.items():
+                fn = getattr(handle, name)
+                fn.restype = res
+                fn.argtypes = args
+            if handle.slayer_abi_version() != ABI_VERSION:
+                raise RuntimeError('libslayer_hip.so ABI version mismatch; rebuild the library')
+            _lib = handle
     return _lib
 
 
