@@ -126,6 +126,13 @@ def raise_on_mismatch(what, fast, check):
                         f'{check[tuple(first)].item()!r} (a 32-bit state overflow shows up like this)')
 
 
+def wants_grad(*tensors):
+    """True when a backward pass could reach one of the tensors: otherwise the operators call their
+    kernels directly and skip the autograd node (a few microseconds per call, which is most of a
+    call on a tensor of one time step)."""
+    return torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
+
+
 def ptr(t):
     return None if t is None else t.data_ptr()
 

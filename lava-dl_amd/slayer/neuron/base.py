@@ -136,16 +136,22 @@ class Neuron(torch.nn.Module):
         elif input.shape[1:-1] != self.shape:
             raise AssertionError(f'Input tensor shape ({input.shape}) does not match with '
                                  f'Neuron shape ({self.shape}).')
+        buffers = self._buffers
         for name, init in self._state_init.items():
-            state = getattr(self, name)
+            state = buffers[name]
             if state.shape[0] != input.shape[0]:            # new batch size: start from the initial value
                 value = float(init() if callable(init) else init)
-                state = torch.full(input.shape[:-1], value, dtype=state.dtype, device=state.device)
+                buffers[name] = state = torch.full(input.shape[:-1], value, dtype=state.dtype, device=state.device)
             if state.shape[1:] != self.shape:               # still the one-element buffer: broadcast it
-                state = state * torch.ones(input.shape[:-1], dtype=state.dtype, device=state.device)
-            setattr(self, name, state)
+                buffers[name] = state * torch.ones(input.shape[:-1], dtype=state.dtype, device=state.device)
         if self.requires_grad:
             self.clamp()
+
+    def _carry(self, **states):
+        """Store the states to carry into the next call (registered buffers; written directly, the
+        generic attribute path of torch.nn.Module costs several microseconds per state)."""
+        for name, value in states.items():
+            self._buffers[name] = value
 
     def _q(self, name):
         """Integer-valued decay with a straight-through gradient."""

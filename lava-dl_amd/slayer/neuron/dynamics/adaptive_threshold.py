@@ -21,6 +21,8 @@ def dynamics(input, ref_state, ref_decay, th_state, th_decay, th_scale, th0, w_s
     (threshold, refractory) : tensors shaped like ``input`` (values before the
     spike update of each step).
     """
+    if not debug and not N.wants_grad(input, ref_state, ref_decay, th_state, th_decay):
+        return _fwd(input, ref_state, ref_decay, th_state, th_decay, th_scale, th0, w_scale)   # skip the autograd node
     _ATHDynamics.DEBUG = debug
     return _ATHDynamics.apply(input, ref_state, ref_decay, th_state, th_decay, th_scale, th0, w_scale)
 

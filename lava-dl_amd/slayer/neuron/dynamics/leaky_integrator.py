@@ -36,14 +36,15 @@ def dynamics(input, decay, state, w_scale, threshold=None, debug=False):
     """
     if threshold is None:
         threshold = -1
+    if not debug and not N.wants_grad(input, decay):
+        return _fwd(input, decay, state, threshold, w_scale)     # skip the autograd node
     _LIDynamics.DEBUG = debug
     return _LIDynamics.apply(input, decay, state, threshold, w_scale)
 
 
 def persistent_state(state, spike):
     """State to carry to the next call when the last step spiked (reset to 0)."""
-    spike = (spike > 0).to(state.dtype)
-    return state * (1 - spike)
+    return state * (spike > 0).logical_not()      # = state * (1 - (spike > 0)): a zero with the state's sign where it spiked
 
 
 def _fwd(input, decay, state, threshold, w_scale, entry='slayer_li_fwd'):

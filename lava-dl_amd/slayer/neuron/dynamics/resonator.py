@@ -22,6 +22,9 @@ def dynamics(real_input, imag_input, sin_decay, cos_decay, real_state, imag_stat
     """
     if threshold is None:
         threshold = -1
+    if not debug and not N.wants_grad(real_input, imag_input, sin_decay, cos_decay):
+        return _fwd(real_input, imag_input, sin_decay, cos_decay, real_state, imag_state,
+                    threshold, w_scale)                                  # skip the autograd node
     _ResDynamics.DEBUG = debug
     return _ResDynamics.apply(real_input, imag_input, sin_decay, cos_decay,
                               real_state, imag_state, threshold, w_scale)

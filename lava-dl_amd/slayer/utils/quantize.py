@@ -28,8 +28,8 @@ def quantize(input, step=1, mode=MODE.ROUND):
     if mode not in (MODE.ROUND, MODE.FLOOR):
         raise ValueError(f'{mode=} is not recognized.')
     if not (torch.is_grad_enabled() and input.requires_grad):      # nothing to pass a gradient to
-        scaled = input / step
-        return (torch.floor(scaled) if mode == MODE.FLOOR else torch.round(scaled)) * step
+        snap = torch.floor if mode == MODE.FLOOR else torch.round
+        return snap(input) if step == 1 else snap(input / step) * step
     return _StraightThrough.apply(input, step, mode == MODE.FLOOR)
 
 
