@@ -24,6 +24,7 @@ template <bool POW2, bool GRADED, bool KEEP_CURRENT>
 struct AlifFwd {
     static constexpr int kIn = 1, kOut = KEEP_CURRENT ? 4 : 3;   // out: [current,] voltage, threshold + refractory, spikes
     static constexpr int kVol = kOut - 3, kTheta = kOut - 2, kSpk = kOut - 1;
+    static constexpr int kCopyWaves = 2;
     static constexpr bool kReverse = false;
     static constexpr bool kTransforms = true;
     static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;

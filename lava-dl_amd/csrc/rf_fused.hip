@@ -21,6 +21,7 @@ struct RfFwd {
     static constexpr int kIn = 2, kOut = 3;          // out: real, imag, spikes
     static constexpr bool kReverse = false;
     static constexpr bool kTransforms = true;
+    static constexpr int kCopyWaves = 2;
     static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
     struct Params {
         const float* in[2];
