@@ -1,6 +1,6 @@
 """Benchmark of the SLAYER neuron-dynamics hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cuba|cuba_fused|cuba_fused_lean|cuba_inference|cuba_fwd_small|alif|alif_fused|alif_fused_lean|rf|rf_fused|rf_fused_lean|rf_inference|synapse|synapse_fused]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cuba|cuba_fused|cuba_fused_lean|cuba_inference|cuba_fwd_small|alif|alif_fused|alif_fused_lean|rf|rf_fused|rf_fused_lean|rf_inference|synapse|synapse_fused|synapse_delay_grad]
 
 A step is one pass of the workload's op sequence over one batch of synthetic input that is already
 resident in HBM (outputs come from torch's caching allocator inside the timed region).  The default
@@ -481,7 +481,30 @@ class SynapseFused(Synapse):
         return spk, g_x
 
 
-WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fused_lean': CubaFusedLean, 'cuba_inference': CubaInference, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'alif_fused': AlifFused, 'alif_fused_lean': AlifFusedLean, 'rf': Rf, 'rf_fused': RfFused, 'rf_fused_lean': RfFusedLean, 'rf_inference': RfInference, 'synapse': Synapse, 'synapse_fused': SynapseFused}
+class SynapseDelayGrad(SynapseFused):
+    name = 'SLAYER synapse stack with a learnable delay (conv K=64 -> Delay -> fused CUBA) fwd+bwd incl. the delay gradient'
+    ops = [('conv', 'conv_kernel', 8), ('shift', 'shift_kernel', 8), ('cuba_fwd', 'stream_kernel<CubaFwd>', 12),
+           ('cuba_bwd', 'stream_kernel<CubaBwd>', 12), ('delay_bwd', 'delay_bwd_kernel', 12), ('corr', 'conv_kernel<corr>', 8)]
+
+    def step(self, t):
+        import importlib
+        D = importlib.import_module('lava_dl_amd.slayer.axon.delay')
+        with t('conv'):
+            y = self.conv.fwd(self.x, self.filt, 1)
+        with t('shift'):
+            z = self.shift(y, self.delay, 1)
+        with t('cuba_fwd'):
+            _, vol, spk = self.F._fwd(z, self.d_i, self.d_v, self.zero, self.zero, 64, 1.25, False, 1, True)
+        with t('cuba_bwd'):
+            g_z, _, _ = self.F._bwd(self.g, vol, None, self.d_i, self.d_v, 1.25, 1.0, 1.0, False, False)
+        with t('delay_bwd'):
+            g_y, g_delay = D._delay_bwd(g_z, z, self.delay, 1)
+        with t('corr'):
+            g_x = self.conv.bwd(g_y, self.filt, 1)
+        return spk, g_x, g_delay
+
+
+WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fused_lean': CubaFusedLean, 'cuba_inference': CubaInference, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'alif_fused': AlifFused, 'alif_fused_lean': AlifFusedLean, 'rf': Rf, 'rf_fused': RfFused, 'rf_fused_lean': RfFusedLean, 'rf_inference': RfInference, 'synapse': Synapse, 'synapse_fused': SynapseFused, 'synapse_delay_grad': SynapseDelayGrad}
 
 
 def cpu_baseline(job, budget_s=20.0):

@@ -188,6 +188,16 @@ int slayer_cspike_bwd(float *grad_re, float *grad_im, const float *grad_spikes,
 int slayer_shift(float *out, const float *in, const float *lut, int64_t scalar_steps,
                  float sampling_time, int64_t M, int64_t neurons_per_batch, int64_t T, void *stream);
 
+/* Backward of the learnable axonal delay, _delayFunction.backward (axon/delay.py:201-221: conv with
+ * [-1, 1] / Ts, product, sum, shift -- four passes) in one: grad_in[m][t] = grad_out[m][t + k_m] with k_m as
+ * in slayer_shift (lut == NULL: scalar_steps), and, when grad_sum is not NULL,
+ * grad_sum[j] = sum over the batch and time of grad_out * ((-1/Ts) out[t] + (1/Ts) out[t-1]) for the
+ * neurons_per_batch neurons of a batch element (the caller scales by Ts and grad_scale as the reference does).
+ * workspace: M + 64 * neurons_per_batch floats, only read and written when grad_sum is wanted. */
+int slayer_delay_bwd(float *grad_in, float *grad_sum, const float *grad_out, const float *out,
+                     const float *lut, int64_t scalar_steps, float sampling_time, float *workspace,
+                     int64_t M, int64_t neurons_per_batch, int64_t T, void *stream);
+
 /* ---- temporal filter ---------------------------------------------------------------------- */
 
 /* Replaces conv fwd (utils/filter/conv.cu:80-125): out[m][t] = Ts * sum_{i<K, t-i>=0} filt[i] * in[m][t-i]. */

@@ -39,6 +39,7 @@ _SIGNATURES = {
     'slayer_cspike_fwd': (_INT, [_P, _P, _P, _P, _I64, _F, _P, _I64, _F, _INT, _F, _I64, _I64, _P]),
     'slayer_cspike_bwd': (_INT, [_P, _P, _P, _P, _P, _P, _I64, _F, _F, _F, _INT, _I64, _P]),
     'slayer_shift': (_INT, [_P, _P, _P, _I64, _F, _I64, _I64, _I64, _P]),
+    'slayer_delay_bwd': (_INT, [_P, _P, _P, _P, _P, _I64, _F, _P, _I64, _I64, _I64, _P]),
     'slayer_conv': (_INT, [_P, _P, _P, _I64, _F, _I64, _I64, _P]),
     'slayer_corr': (_INT, [_P, _P, _P, _I64, _F, _I64, _I64, _P]),
     'slayer_apth_fwd': (_INT, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _INT,

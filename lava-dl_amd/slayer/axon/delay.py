@@ -6,6 +6,7 @@ the reference).
 import numpy as np
 import torch
 
+from .. import _native as N
 from ..utils.time import shift
 from ..utils.filter import conv
 
@@ -95,9 +96,33 @@ class _delayFunction(torch.autograd.Function):
     def backward(ctx, grad_output):
         output, delay_val = ctx.saved_tensors
         ts = ctx.sampling_time
+        if delay_val.numel() > 1 and grad_output.numel() > 0:
+            grad_input, grad_sum = _delay_bwd(grad_output, output, delay_val, ts)
+            return grad_input, grad_sum * ts * ctx.grad_scale, None, None
+        # one delay for everything (shift() then divides in double precision), or nothing to do
         # d output / d delay is minus the time derivative: conv with [-1, 1] / Ts gives x[t-1] - x[t]
         diff_filter = torch.tensor([-1, 1], dtype=grad_output.dtype, device=grad_output.device) / ts
         output_diff = conv(output, diff_filter, 1)
         grad_delay = torch.sum(grad_output * output_diff, [0, -1], keepdim=True) \
             .reshape(grad_output.shape[1:-1]) * ts
         return shift(grad_output, -delay_val, ts), grad_delay * ctx.grad_scale, None, None
+
+
+def _delay_bwd(grad_output, output, delay_val, sampling_time):
+    """(grad_input, sum over batch and time of grad_output * d output / d delay) in one pass over
+    grad_output and output (slayer_delay_bwd) instead of filter, product, sum and shift."""
+    dev = N.require_gpu(grad_output, output)
+    grad_output, output = grad_output.contiguous(), output.contiguous()
+    M, T = N.rows_and_steps(grad_output)
+    npb = N.neurons_per_batch(grad_output)
+    if delay_val.numel() != npb:
+        raise RuntimeError(f'delay has {delay_val.numel()} elements, expected one per neuron ({npb})')
+    lut = delay_val.detach().to(device=dev, dtype=torch.float32).contiguous()
+    grad_input = torch.empty_like(grad_output)
+    grad_sum = torch.empty(npb, dtype=torch.float32, device=dev)
+    workspace = torch.empty(M + 64 * npb, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        N.check(N.lib().slayer_delay_bwd(
+            N.ptr(grad_input), N.ptr(grad_sum), N.ptr(grad_output), N.ptr(output), N.ptr(lut), 0,
+            float(sampling_time), N.ptr(workspace), M, npb, T, N.stream_handle()))
+    return grad_input, grad_sum.reshape(grad_output.shape[1:-1])

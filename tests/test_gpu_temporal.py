@@ -133,6 +133,53 @@ def test_delay_module(slayer):
     assert_exact(slayer.axon.delay(x.to(dev())), O.shift(x, 1), 'delay()')
 
 
+@pytest.mark.parametrize('shape,ts', [((2, 5, 3, 40), 1), ((3, 7, 37), 1), ((2, 6, 1000), 1), ((4, 9, 4, 4, 300), 2),
+                                      ((1, 3, 3), 1), ((2, 64, 1), 1), ((5, 130, 516), 0.5)])
+def test_delay_backward_kernel(slayer, shape, ts):
+    """slayer_delay_bwd against the reference's four-step backward (filter, product, sum, shift): rows longer
+    than one pass of a wave, T % 4 != 0, sampling times other than 1, shifts that empty a row, fractional and
+    negative delays."""
+    import importlib
+    D = importlib.import_module('lava_dl_amd.slayer.axon.delay')      # the package attribute is the function
+    gen = torch.Generator().manual_seed(seed_of('delay bwd', shape, ts))
+    spatial = shape[1:-1]
+    y = torch.rand(shape, generator=gen)
+    g = torch.randn(shape, generator=gen)
+    d = torch.rand(spatial, generator=gen) * 24 * ts - 2 * ts          # a few negative ones
+    d.view(-1)[0] = 0.0
+    d.view(-1)[-1] = (shape[-1] + 5) * ts                               # shifts the whole row out
+    if d.numel() > 3:
+        d.view(-1)[1] = 4 * ts                                          # aligned shift
+    ref_gi, ref_gd = O.delay_bwd(g, y, d, grad_scale=1.0, sampling_time=ts)
+    gi, gsum = D._delay_bwd(g.to(dev()), y.to(dev()), d.to(dev()), ts)
+    assert_exact(gi, ref_gi, f'delay grad_input {shape}')
+    assert_rel(gsum * ts, ref_gd, f'delay grad_delay {shape}', rel=1e-4)
+    # misaligned views take the dword path and must agree with the aligned run
+    if shape[-1] % 4 == 0:
+        flat = torch.zeros(g.numel() + 1, device=dev())
+        flat[1:] = g.to(dev()).flatten()
+        gi2, gsum2 = D._delay_bwd(flat[1:].reshape(shape), y.to(dev()), d.to(dev()), ts)
+        assert torch.equal(gi2, gi) and torch.equal(gsum2, gsum)
+
+
+def test_delay_backward_entry_point_scalar_shift_and_no_sum(slayer):
+    """C ABI directly: lut == NULL moves every row by scalar_steps; grad_sum == NULL skips the sums."""
+    from lava_dl_amd.slayer import _native as N
+    gen = torch.Generator().manual_seed(71)
+    g = torch.randn(3, 10, 64, generator=gen)
+    y = torch.rand(3, 10, 64, generator=gen)
+    gg, yg = g.to(dev()), y.to(dev())
+    for steps in (0, 5, -3, 64, 1000):
+        out = torch.full_like(gg, float('nan'))
+        N.check(N.lib().slayer_delay_bwd(N.ptr(out), None, N.ptr(gg), N.ptr(yg), None, steps, 1.0, None,
+                                         30, 10, 64, N.stream_handle()))
+        assert_exact(out, O.shift(g, -steps), f'delay_bwd scalar shift {steps}')
+    assert N.lib().slayer_delay_bwd(N.ptr(out), N.ptr(out), N.ptr(gg), N.ptr(yg), None, 0, 1.0, None,
+                                    30, 10, 64, N.stream_handle()) != 0           # sums wanted, no workspace
+    assert N.lib().slayer_delay_bwd(N.ptr(out), None, N.ptr(gg), N.ptr(yg), None, 0, 0.0, None,
+                                    30, 10, 64, N.stream_handle()) != 0           # sampling time 0
+
+
 # --------------------------------------------------------------------------------- sigma-delta
 @pytest.mark.parametrize('shape', [(3, 6, 200), (2, 3, 5, 7, 37), (4, 70, 129), (1, 5, 3), (4, 9000, 64)])
 @pytest.mark.parametrize('cum', [False, True])
