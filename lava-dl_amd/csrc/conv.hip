@@ -95,6 +95,123 @@ __global__ __launch_bounds__(kWave) void conv_kernel(float* __restrict__ out, co
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Matrix-core form for 8 < K <= 128 (T % 4 == 0, 16-byte aligned tensors).  A tile of 16 output steps of 16
+// rows is a [16 x (16 + KPAD)] Toeplitz matrix of taps times the [(16 + KPAD) x 16] window of inputs:
+// v_mfma_f32_16x16x4_f32 with D[i][j] = output step i of row j, four input samples per instruction.  With
+// K = 64 the window is 80 samples, so 64 of 80 multiply-adds are useful (the FMA form above issues 82
+// instructions per 64 useful FMAs at half the rate).  Lane l works for row l % 16 and quad l / 16: it loads
+// the 4 samples [16 g + 4 (l / 16), +4) of window group g straight from memory (a float4), which are exactly
+// the B operands of the group's four instructions (sample 4 k + r of a group goes to summation slot k of
+// instruction r), keeps the Toeplitz operands of all groups in registers (they do not depend on the tile),
+// and receives 4 consecutive output steps of its row (a float4 store).  Stepping to the next tile moves
+// every window group down by one, so a tile costs one new load per lane; no LDS, no barrier.
+typedef float mfma_f4 __attribute__((ext_vector_type(4)));
+
+template <int KPAD, bool CORR>
+__global__ __launch_bounds__(kWave) void conv_mfma_kernel(float* __restrict__ out, const float* __restrict__ in,
+                                                          const float* __restrict__ filt, int K, float ts,
+                                                          int64_t M, int T, int span, unsigned spans_per_row) {
+    constexpr int G = KPAD / 16 + 1;        // window groups of 16 samples per tile
+    constexpr int RING = KPAD <= 64 ? 8 : 16;
+    const int lane = threadIdx.x;
+    const int j = lane & 15, kq = lane >> 4;
+    const int64_t rowgroup = blockIdx.x / spans_per_row;
+    const int tbeg = (int)(blockIdx.x - rowgroup * spans_per_row) * span;
+    const int tend = tbeg + span < T ? tbeg + span : T;
+    const int64_t m0 = rowgroup * 16;
+    const int rows = (int)((M - m0) < 16 ? (M - m0) : 16);
+    // raw buffer accesses over the wave's rows: a lane that must not touch memory (row beyond the tensor,
+    // step outside [0, T)) gets an out-of-range offset, reads zeros and has its store dropped; no branch
+    // surrounds a memory instruction, so the loads issued ahead stay in flight across the loop's waits
+    const unsigned wave_bytes = (unsigned)rows * (unsigned)T * 4u;
+    const __amdgpu_buffer_rsrc_t src = make_rsrc(in + m0 * (int64_t)T, wave_bytes);
+    const __amdgpu_buffer_rsrc_t dst = make_rsrc(out + m0 * (int64_t)T, wave_bytes);
+    const bool row_ok = j < rows;
+    const int row_off = j * T * 4;
+
+    // Toeplitz operands: lane (output step i = l % 16, slot kq) of instruction (g, r) holds the tap that
+    // links output step i with window sample 16 g + 4 kq + r
+    float a[G][4];
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int idx = CORR ? (16 * g + 4 * kq + r) - j : j + KPAD - (16 * g + 4 * kq + r);
+            a[g][r] = (idx >= 0 && idx < K) ? filt[idx] : 0.0f;
+        }
+
+    // window group g of the tile at t0 starts at step t0 - KPAD + 16 g (conv) or t0 + 16 g (corr)
+    auto load = [&](int step) -> float4 {
+        const bool ok = row_ok && (unsigned)step < (unsigned)T;
+        return buf_load4<false>(src, ok ? row_off + step * 4 : kOutOfRange);
+    };
+    // Window groups live in a ring of RING registers (absolute group q of the span, starting at step
+    // first + 16 q, sits in slot q % RING): tile n reads groups n .. n + G - 1 and then refills the slot of
+    // group n, which no later tile needs, with group n + RING -- P = RING - G tiles before its first use.
+    // The loop body is RING tiles, so every slot index is a compile-time constant.
+    const int first = (CORR ? tbeg : tbeg - KPAD) + 4 * kq;
+    float4 x[RING];
+    // each load is preceded by a store that falls out of range (dropped by the hardware): the loop is then
+    // entered in the state its back edge leaves, and the wait at its top can leave the youngest loads in
+    // flight instead of draining everything
+#pragma unroll
+    for (int q = 0; q < RING; ++q) {
+        buf_store4<false>(dst, kOutOfRange + 16 * q, make_float4(0.f, 0.f, 0.f, 0.f));
+        x[q] = load(first + 16 * q);
+    }
+
+    for (int t0 = tbeg; t0 < tend; t0 += 16 * RING) {
+#pragma unroll
+        for (int u = 0; u < RING; ++u) {
+            // two accumulators: consecutive instructions do not wait for each other's result
+            mfma_f4 acc = {0.0f, 0.0f, 0.0f, 0.0f}, acc2 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const float4 xv = x[(u + g) % RING];
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][0], xv.x, acc, 0, 0, 0);
+                acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][1], xv.y, acc2, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][2], xv.z, acc, 0, 0, 0);
+                acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][3], xv.w, acc2, 0, 0, 0);
+            }
+            acc += acc2;
+            // tiles past the end of the span (the last pass of the loop may hold some) store nothing
+            const int t = t0 + 16 * u + 4 * kq;
+            buf_store4<false>(dst, (row_ok && t < tend) ? row_off + t * 4 : kOutOfRange,
+                              make_float4(acc[0] * ts, acc[1] * ts, acc[2] * ts, acc[3] * ts));
+            x[u] = load(first + (t0 - tbeg) + 16 * (u + RING));
+        }
+    }
+}
+
+template <bool CORR>
+static int conv_mfma_launch(float* out, const float* in, const float* filt, int K, float ts, int64_t M, int64_t T,
+                            hipStream_t stream) {
+    const int64_t rowgroups = (M + 15) / 16;
+    // about four waves per SIMD on 256 compute units when the rows alone do not provide them; a span is a
+    // whole number of loop passes (RING tiles of 16 outputs) and is preceded by KPAD samples of warm-up
+    const int64_t pass = 16 * (K <= 64 ? 8 : 16);
+    int64_t spans = (4096 + rowgroups - 1) / rowgroups;
+    const int64_t max_spans = (T + pass - 1) / pass;
+    if (spans > max_spans) spans = max_spans;
+    if (spans < 1) spans = 1;
+    const int64_t span = (((T + spans - 1) / spans) + pass - 1) / pass * pass;
+    spans = (T + span - 1) / span;
+    const int64_t blocks = rowgroups * spans;
+    if (blocks > 0x7fffffffLL) return SLAYER_ERANGE;
+    // No non-temporal accesses here: a load or store covers 64 bytes per row, half a cache line, and the caches
+    // put the halves together (measured: non-temporal accesses cost 25-85 % on large tensors).
+#define SLAYER_CONV_MFMA(KP)                                                                                      \
+    hipLaunchKernelGGL((conv_mfma_kernel<KP, CORR>), dim3((unsigned)blocks), dim3(kWave), 0, stream, out, in, filt, \
+                       K, ts, M, (int)T, (int)span, (unsigned)spans)
+    if (K <= 16) SLAYER_CONV_MFMA(16);
+    else if (K <= 32) SLAYER_CONV_MFMA(32);
+    else if (K <= 64) SLAYER_CONV_MFMA(64);
+    else SLAYER_CONV_MFMA(128);
+#undef SLAYER_CONV_MFMA
+    return (int)hipGetLastError();
+}
+
 template <bool CORR>
 static int conv_launch(float* out, const float* in, const float* filt, int64_t K, float ts,
                        int64_t M, int64_t T, hipStream_t stream) {
@@ -103,6 +220,8 @@ static int conv_launch(float* out, const float* in, const float* filt, int64_t K
     if (!out || !in || !filt) return SLAYER_ENULL;
     if (K < 1) return SLAYER_EINVAL;
     if (K > kMaxTaps) return SLAYER_ERANGE;
+    if (K > 8 && K <= 128 && T % 4 == 0 && T <= (1 << 22) && aligned16(out) && aligned16(in))
+        return conv_mfma_launch<CORR>(out, in, filt, (int)K, ts, M, T, stream);
     const unsigned segs = (unsigned)((T + kSeg - 1) / kSeg);
     const int64_t blocks = M * (int64_t)segs;
     if (blocks > 0x7fffffffLL) return SLAYER_ERANGE;

@@ -100,6 +100,34 @@ def test_conv_corr(slayer, shape, K):
     assert np.allclose(y, np.convolve(row, f.double().numpy())[:row.size], rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize('shape,K', [((16, 64), 9), ((5, 3, 16), 16), ((37, 132), 17), ((3, 700, 48), 32), ((2, 9, 1000), 33),
+                                     ((64, 256, 100), 64), ((1, 20, 2048), 64), ((130, 4), 64), ((50, 260), 65),
+                                     ((7, 11, 300), 100), ((33, 520), 128), ((33, 520), 129), ((4, 12), 40)])
+def test_conv_corr_matrix_core_path(slayer, shape, K):
+    """Tap counts either side of every padded size of the matrix-core kernel (16, 32, 64, 128) and of its
+    limits (8 < K <= 128), row counts that are not multiples of 16, rows shorter than a tile and than the
+    filter, rows split into several spans, and a signed filter; float64 numpy.convolve as the judge."""
+    gen = torch.Generator().manual_seed(seed_of('mfma conv', shape, K))
+    x = torch.randn(shape, generator=gen)
+    f = torch.randn(K, generator=gen)
+    T = shape[-1]
+    rows = x.reshape(-1, T).double().numpy()
+    fd = f.double().numpy()
+    for ts in (1, 0.25):
+        y = slayer.utils.filter.conv(x.to(dev()), f.to(dev()), ts).reshape(-1, T).cpu().double().numpy()
+        z = slayer.utils.filter.corr(x.to(dev()), f.to(dev()), ts).reshape(-1, T).cpu().double().numpy()
+        scale = ts * np.abs(fd).sum() * np.abs(rows).max()
+        for r in (0, rows.shape[0] // 2, rows.shape[0] - 1):
+            want = ts * np.convolve(rows[r], fd)[:T]
+            assert np.abs(y[r] - want).max() <= 1e-5 * scale, (shape, K, r)
+            want = ts * np.convolve(rows[r][::-1], fd)[:T][::-1]
+            assert np.abs(z[r] - want).max() <= 1e-5 * scale, (shape, K, r)
+    # non-negative data (no cancellation): the elementwise tolerance against the oracle holds as well
+    xp, fp = x.abs(), f.abs()
+    assert_rel(slayer.utils.filter.conv(xp.to(dev()), fp.to(dev()), 1), O.conv_fwd(xp, fp, 1), f'conv {shape} K={K}')
+    assert_rel(slayer.utils.filter.corr(xp.to(dev()), fp.to(dev()), 1), O.conv_bwd(xp, fp, 1), f'corr {shape} K={K}')
+
+
 def test_conv_autograd_is_corr(slayer):
     gen = torch.Generator().manual_seed(61)
     x = torch.rand((3, 6, 90), generator=gen)
