@@ -52,8 +52,8 @@ inline int fire_above_scaled(float thr, float w, bool pow2) {
         return (pow2 ? f * inv_w : f / w) < thr;
     };
     long long lo = -2147483648LL, hi = 2147483647LL;
-    if (!below(lo)) return (int)lo;          // every state fires except the most negative one
-    if (below(hi) || !(thr == thr)) return (int)hi;
+    if (!(thr == thr) || below(hi)) return (int)hi;      // NaN or beyond every state: never fires
+    if (!below(lo)) return (int)lo;                      // every state fires except the most negative one
     while (hi - lo > 1) {
         const long long mid = lo + (hi - lo) / 2;
         if (below(mid)) lo = mid; else hi = mid;

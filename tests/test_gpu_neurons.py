@@ -256,6 +256,39 @@ def test_fused_rf_equals_the_operator_chain(slayer, shape, w, graded):
     assert torch.equal(c[0].grad, a[0].grad) and torch.equal(c[1].grad, a[1].grad), 'lean input gradients differ'
 
 
+@pytest.mark.parametrize('w', [64, 100, 4096, 3])
+@pytest.mark.parametrize('graded', [False, True])
+def test_fused_rf_spike_decision_on_integer_states(slayer, w, graded):
+    """The fused forward decides the spike on the integer states.  No rotation (sin 0, cos 4096): the real part
+    walks through every integer around threshold * w_scale while the imaginary part alternates in sign, for
+    thresholds that are and are not multiples of 1 / w_scale, negative, zero, beyond the int range, NaN."""
+    D = slayer.neuron.dynamics
+    T = 64
+    steps = torch.arange(T)
+    for thr in (0.7, 1.0, 70 / w, (70 + 0.5) / w, -0.3, 0.0, 1e12, -1e12, float('nan')):
+        centre = 0 if thr != thr or abs(thr) > 1e6 else int(round(thr * w))
+        # row n: real state centre - 8 + n after step 0, then constant; imag -1, +1, -1, ... (units of 1 / w)
+        xr = torch.zeros(16, 1, T)
+        xr[:, 0, 0] = (centre - 8 + torch.arange(16)).float() / w
+        xi = torch.zeros(16, 1, T)
+        xi[:, 0, 0] = -1.0 / w
+        xi[:, 0, 1:] = torch.where(steps[1:] % 2 == 1, 2.0, -2.0) / w      # +2, -2, +2, ...: the sign flips every step
+        sin, cos = torch.tensor([0.0]), torch.tensor([4096.0])
+        zero = torch.zeros(1)
+        args = [t.to(dev()) for t in (xr, xi, sin, cos, zero, zero)]
+        for last in (-1.0, 0.0, 1.0):
+            lastt = torch.full((16, 1), last, device=dev())
+            re, im = D.resonator.dynamics(*args, w)
+            spk = slayer.spike.complex.Spike.apply(re, im, thr, 0.5, 10.0, graded, lastt, 2)
+            f_re, f_im, f_spk = D.rf_fused.dynamics(*args, lastt, w, thr, 0.5, 10.0, graded, 2)
+            assert torch.equal(f_re, re) and torch.equal(f_im, im)
+            assert torch.equal(f_spk, spk), (w, thr, last, graded)
+            _, _, i_spk = D.rf_fused.spikes(*args, lastt, w, thr, graded, 2)
+            assert torch.equal(i_spk, spk), (w, thr, last, graded)
+        if thr == thr and abs(thr) < 1e6:
+            assert 0 < float((spk != 0).float().mean()) < 1, 'both outcomes must occur'
+
+
 def test_rf_neuron_forward_uses_fused_path_with_same_results(slayer):
     gen = torch.Generator().manual_seed(105)
     shape = (3, 12, 150)
