@@ -497,3 +497,60 @@ def test_fused_cuba_under_graph_capture_replays(slayer):
         assert float(want[0].sum()) > 0
         for i, (a, b) in enumerate(zip(got, want)):
             assert torch.equal(a, b), f'replay {k}: output {i} differs from the eager result'
+
+
+@pytest.mark.parametrize('w', [4096, 1000])
+def test_fused_blocks_equal_the_chains_beyond_float32_integers(slayer, w):
+    from tests.util import seed_of
+    """Barely any decay and a biased input: the integer states pass 2**24, where the int -> float32 conversion at
+    every operator boundary rounds.  The fused CUBA / ALIF / RF blocks make the same round trips, so traces,
+    spikes and final states still equal the operator chains bit for bit (full, lean and inference forms)."""
+    gen = torch.Generator().manual_seed(seed_of('beyond 2**24', w))
+    D = slayer.neuron.dynamics
+    shape = (2, 24, 800)
+    C = shape[1]
+    x = (0.2 + 0.3 * torch.rand(shape, generator=gen)).to(dev())
+    zero = torch.zeros(1, device=dev())
+    d_i = torch.randint(0, 3, (C,), generator=gen).float().to(dev())
+    d_v = torch.randint(0, 3, (C,), generator=gen).float().to(dev())
+    # CUBA: threshold far up, so the voltage resets from states beyond 2**24
+    thr = 2.0e4
+    cur = D.leaky_integrator.dynamics(x, d_i, zero, w)
+    vol = D.leaky_integrator.dynamics(cur, d_v, zero, w, thr)
+    spk = slayer.spike.Spike.apply(vol, thr, 1.0, 1.0, False, 0, 1)
+    assert float(vol.abs().max()) * w > 2 ** 24 and 0 < float(spk.sum()) < spk.numel() / 2
+    f_cur, f_vol, f_spk = D.cuba_fused.dynamics(x, d_i, d_v, zero, zero, w, thr, 1.0, 1.0, False, 1)
+    assert torch.equal(f_cur, cur) and torch.equal(f_vol, vol) and torch.equal(f_spk, spk), 'CUBA'
+    l_cur, l_vol, l_spk = D.cuba_fused.dynamics(x, d_i, d_v, zero, zero, w, thr, 1.0, 1.0, False, 1, keep_current=False)
+    assert torch.equal(l_cur, cur[..., -1]) and torch.equal(l_vol, vol) and torch.equal(l_spk, spk), 'CUBA lean'
+    i_cur, i_vol, i_spk = D.cuba_fused.spikes(x, d_i, d_v, zero, zero, w, thr, False, 1)
+    assert torch.equal(i_cur, cur[..., -1]) and torch.equal(i_vol, vol[..., -1]) and torch.equal(i_spk, spk), 'CUBA inference'
+    # ALIF: no reset at all, the voltage keeps growing; threshold and refractory follow it
+    d_th = torch.randint(0, 50, (C,), generator=gen).float().to(dev())
+    d_ref = torch.randint(0, 50, (C,), generator=gen).float().to(dev())
+    one = torch.ones(1, device=dev())
+    step, base = 3.0e3, 1.0e3
+    vol2 = D.leaky_integrator.dynamics(cur, d_v, zero, w)
+    th, ref = D.adaptive_threshold.dynamics(vol2, zero, d_ref, one * base, d_th, step, base, w)
+    spk2 = slayer.spike.Spike.apply(vol2, th + ref, 1.0, 1.0, False, 0, 1)
+    assert float(vol2.abs().max()) * w > 2 ** 24 and float((th + ref).abs().max()) * w > 2 ** 24
+    assert 0 < float(spk2.sum()) < spk2.numel()
+    f = D.alif_fused.dynamics(x, d_i, d_v, d_th, d_ref, zero, zero, one * base, zero, step, base, w, 1.0, 1.0, False, 1)
+    assert torch.equal(f[0], cur) and torch.equal(f[1], vol2) and torch.equal(f[2], th + ref), 'ALIF traces'
+    assert torch.equal(f[3], spk2) and torch.equal(f[4], th[..., -1]) and torch.equal(f[5], ref[..., -1]), 'ALIF'
+    s = D.alif_fused.spikes(x, d_i, d_v, d_th, d_ref, zero, zero, one * base, zero, step, base, w, False, 1)
+    assert torch.equal(s[3], spk2) and torch.equal(s[4], th[..., -1]) and torch.equal(s[5], ref[..., -1]), 'ALIF inference'
+    # RF: slow rotation with a gain just below one, biased input on both parts
+    ph = torch.linspace(0.002, 0.02, C)
+    sin, cos = (4095 * torch.sin(ph)).round().to(dev()), (4095 * torch.cos(ph)).round().to(dev())
+    x = 100 * x
+    square = torch.where(torch.arange(shape[-1]) % 100 < 50, 1.0, -1.0)       # the imaginary part swings through zero
+    xi = (1500 * torch.rand(shape, generator=gen) * square).to(dev())
+    re, im = D.resonator.dynamics(x, xi, sin, cos, zero, zero, w)
+    thr_rf = 5.0e3
+    spk3 = slayer.spike.complex.Spike.apply(re, im, thr_rf, 0.5, 10.0, False, 0, 1)
+    assert float(re.abs().max()) * w > 2 ** 24 and 0 < float(spk3.sum()) < spk3.numel()
+    f_re, f_im, f_spk3 = D.rf_fused.dynamics(x, xi, sin, cos, zero, zero, zero, w, thr_rf, 0.5, 10.0, False, 1)
+    assert torch.equal(f_re, re) and torch.equal(f_im, im) and torch.equal(f_spk3, spk3), 'RF'
+    r_last, i_last, i_spk3 = D.rf_fused.spikes(x, xi, sin, cos, zero, zero, zero, w, thr_rf, False, 1)
+    assert torch.equal(r_last, re[..., -1]) and torch.equal(i_last, im[..., -1]) and torch.equal(i_spk3, spk3), 'RF inference'
