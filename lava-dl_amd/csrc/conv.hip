@@ -106,6 +106,9 @@ __global__ __launch_bounds__(kWave) void conv_kernel(float* __restrict__ out, co
 // instruction r), keeps the Toeplitz operands of all groups in registers (they do not depend on the tile),
 // and receives 4 consecutive output steps of its row (a float4 store).  Stepping to the next tile moves
 // every window group down by one, so a tile costs one new load per lane; no LDS, no barrier.
+// Window samples outside a filter's support meet a zero tap instead of being skipped, so an Inf or NaN in the
+// input also reaches the up to 16 + KPAD - K neighbouring outputs whose window holds it (0 * Inf); finite
+// inputs, the only ones this path sees, give the same sums.
 typedef float mfma_f4 __attribute__((ext_vector_type(4)));
 
 template <int KPAD, bool CORR>
