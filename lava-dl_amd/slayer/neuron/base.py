@@ -46,13 +46,23 @@ class Neuron(torch.nn.Module):
         self.persistent_state = persistent_state
         self.requires_grad = requires_grad
         self.graded_spike = graded_spike
-        self.norm = norm() if norm is not None else None
+        self.norm = self._make_norm(norm)
         self.drop = dropout
         self.debug = False
         self.shape = None
         self.num_neurons = None
         self._ranges = {}
         self._state_init = {}
+
+    def _make_norm(self, norm):
+        """Instantiate a normalisation; one that quantises what it subtracts (``pre_hook_fx``) uses this
+        neuron's weight quantiser for it (neuron/base.py:127-141 in the reference)."""
+        if norm is None:
+            return None
+        instance = norm()
+        if hasattr(instance, 'pre_hook_fx'):
+            instance.pre_hook_fx = self.quantize_8bit
+        return instance
 
     # ------------------------------------------------------------------ parameters
     @property

@@ -33,8 +33,8 @@ class ResonatorNeuron(_Base):
                  graded_spike=False, log_init=True, extra_decays=None, extra_states=None):
         super().__init__(threshold, tau_grad, scale_grad, scale, None, dropout, shared_param,
                          persistent_state, requires_grad, graded_spike)
-        self.real_norm = norm() if norm is not None else None
-        self.imag_norm = norm() if norm is not None else None
+        self.real_norm = self._make_norm(norm)
+        self.imag_norm = self._make_norm(norm)
         self.log_init = log_init
 
         def check(p):

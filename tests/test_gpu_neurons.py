@@ -554,3 +554,24 @@ def test_fused_blocks_equal_the_chains_beyond_float32_integers(slayer, w):
     assert torch.equal(f_re, re) and torch.equal(f_im, im) and torch.equal(f_spk3, spk3), 'RF'
     r_last, i_last, i_spk3 = D.rf_fused.spikes(x, xi, sin, cos, zero, zero, zero, w, thr_rf, False, 1)
     assert torch.equal(r_last, re[..., -1]) and torch.equal(i_last, im[..., -1]) and torch.equal(i_spk3, spk3), 'RF inference'
+
+
+def test_cuba_neuron_with_a_norm_takes_the_operator_chain(slayer):
+    """A normalisation sits between current and voltage, so the fused block cannot be used: forward must be
+    current -> norm (with the neuron's quantiser hooked in) -> voltage with reset -> spike."""
+    gen = torch.Generator().manual_seed(310)
+    x = sparse_input(gen, (4, 10, 120), p=0.3, amp=2.0).to(dev())
+    n = slayer.neuron.cuba.Neuron(1.0, 0.25, 0.05, norm=slayer.neuron.norm.MeanOnlyBatchNorm).to(dev())
+    n.eval()
+    n.norm.running_mean = (torch.rand(10, generator=gen) * 0.4).to(dev())
+    spk = n(x)
+    D = slayer.neuron.dynamics
+    zero = torch.zeros(1, device=dev())
+    cur = D.leaky_integrator.dynamics(x, torch.tensor([1024.0], device=dev()), zero, 4096)
+    shift = n.quantize_8bit(n.norm.running_mean).reshape(1, -1, 1)
+    assert float(shift.abs().max()) > 0 and torch.equal(shift * 32, torch.round(shift * 32))     # steps of 2 / 64
+    vol = D.leaky_integrator.dynamics(cur - shift, torch.tensor([205.0], device=dev()), zero, 4096, 1.0 + 0.01 / 4096)
+    want = slayer.spike.Spike.apply(vol, 1.0 + 0.01 / 4096, 100.0, 0.1, False, 0, 1)
+    assert 0 < float(want.sum()) < want.numel()
+    assert torch.equal(spk, want)
+    assert torch.equal(n.norm.bias, -n.quantize_8bit(n.norm.running_mean, descale=True))

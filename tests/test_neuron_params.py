@@ -122,3 +122,72 @@ def test_small_utilities():
         def value():
             return 42
     assert Handle.value == 42
+
+
+def test_mean_only_batch_norm():
+    """Batch statistics while training, running mean otherwise; hand-computed expectations
+    (neuron/norm.py:9-95 in the reference)."""
+    norm = N.norm.MeanOnlyBatchNorm(momentum=0.25)
+    x = torch.arange(2 * 3 * 4, dtype=torch.float32).reshape(2, 3, 4)
+    mean = torch.tensor([7.5, 11.5, 15.5])                     # per feature over batch and time
+    norm.train()
+    assert torch.allclose(norm(x), x - mean.reshape(1, 3, 1))
+    assert norm.num_features == 3 and torch.allclose(norm.running_mean, 0.25 * mean)
+    norm.eval()
+    assert torch.allclose(norm(x), x - 0.25 * mean.reshape(1, 3, 1))
+    assert torch.allclose(norm.running_mean, 0.25 * mean)      # no update outside training
+    norm.train()
+    norm.update = False
+    assert torch.allclose(norm(x), x - 0.25 * mean.reshape(1, 3, 1))
+    y5 = N.norm.MeanOnlyBatchNorm()(torch.ones(2, 3, 2, 2, 5))
+    assert y5.shape == (2, 3, 2, 2, 5) and float(y5.abs().max()) == 0.0
+    with pytest.raises(AssertionError):
+        N.norm.MeanOnlyBatchNorm()(torch.ones(1, 2, 1, 1, 1, 3))
+
+
+def test_weight_scale_batch_norm():
+    norm = N.norm.WgtScaleBatchNorm(momentum=0.5, weight_exp_bits=3)
+    gen = torch.Generator().manual_seed(5)
+    x = 5.0 * torch.randn(4, 6, 50, generator=gen) + 2.0
+    norm.train()
+    y = norm(x)
+    mean = x.transpose(0, 1).reshape(6, -1).mean(dim=1)
+    var = x.var(unbiased=False)
+    scale = 2.0 ** float(torch.ceil(torch.log2(torch.sqrt(var + 1e-5))).clamp(-3, 3))
+    assert scale == 8.0                                         # std ~ 5 rounds up to 2**3
+    assert torch.allclose(y, (x - mean.reshape(1, 6, 1)) / scale, atol=1e-6)
+    n = x.numel() / 6
+    assert torch.allclose(norm.running_var, 0.5 * var * n / (n + 1))
+    assert torch.allclose(norm.running_mean, 0.5 * mean)
+    assert float(norm.weight_exp) == float(torch.ceil(torch.log2(torch.sqrt(norm.running_var + 1e-5))))
+    assert float(norm.std(torch.tensor([1.0e6]))) == 8.0 and float(norm.std(torch.tensor([1.0e-9]))) == 0.125
+    norm.eval()
+    y = norm(x)
+    assert torch.allclose(y, (x - 0.5 * mean.reshape(1, 6, 1)) / float(norm.std(norm.running_var)), atol=1e-6)
+
+
+def test_neuron_hooks_its_quantiser_into_the_norm():
+    n = N.cuba.Neuron(1.0, 0.25, 0.03, norm=N.norm.MeanOnlyBatchNorm)
+    assert n.norm.pre_hook_fx == n.quantize_8bit
+    n.norm.running_mean = torch.tensor([0.26, -0.51])
+    assert torch.equal(n.norm.bias, -torch.tensor([0.25, -0.5]) * 64)      # steps of 2 / 64, descaled
+    r = N.rf.Neuron(1.0, 10, 0.1, norm=N.norm.WgtScaleBatchNorm)
+    assert r.norm is None and r.real_norm.pre_hook_fx == r.quantize_8bit and r.imag_norm is not r.real_norm
+
+    class Plain(torch.nn.Module):
+        def forward(self, x):
+            return x
+    assert isinstance(N.cuba.Neuron(1.0, 0.25, 0.03, norm=Plain).norm, Plain)
+
+
+def test_neuron_dropout_drops_whole_neurons():
+    drop = N.Dropout(0.5)
+    torch.manual_seed(0)
+    x = torch.ones(8, 4, 5, 20)
+    y = drop(x)
+    assert y.shape == x.shape
+    per_neuron = y.reshape(8 * 4 * 5, 20)
+    assert bool(((per_neuron == 0).all(dim=1) | (per_neuron == 2).all(dim=1)).all())      # constant over time
+    assert 0 < float((per_neuron[:, 0] == 0).float().mean()) < 1
+    drop.eval()
+    assert torch.equal(drop(x), x)
