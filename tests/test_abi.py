@@ -54,6 +54,18 @@ def test_argument_validation_happens_before_any_launch():
     assert L.slayer_shift(one, one, None, 1, 1.0, 8, 3, 8, None) == EINVAL
     assert L.slayer_spike_fwd(one, one, one, 3, 0.0, 0, 1.0, 8, None) == EINVAL             # 3 thresholds for 8 samples
     assert L.slayer_ath_fwd(one, one, one, one, one, one, one, 1 << 40, 0, 64, 8, 4, 1, 1, 1, 1, 8, None) == ERANGE
+    # delay backward: sampling time 0, rows not a multiple of the neurons per batch, sums wanted without workspace
+    assert L.slayer_delay_bwd(one, None, one, one, None, 1, 0.0, None, 8, 4, 8, None) == EINVAL
+    assert L.slayer_delay_bwd(one, None, one, one, None, 1, 1.0, None, 10, 4, 8, None) == EINVAL
+    assert L.slayer_delay_bwd(one, one, one, one, one, 0, 1.0, None, 8, 4, 8, None) == ENULL
+    # fused resonate-and-fire forward: the integer spike decision needs a positive scale
+    rf_tail = (1.0, 0, 1.0)
+    assert L.slayer_rf_fwd(one, one, one, None, None, one, one, one, one, one, one, one, *rf_tail, 0,
+                           8, 4, 1, 1, 1, 1, 8, None) == EINVAL
+    assert L.slayer_rf_fwd(one, one, one, None, None, one, one, one, one, one, one, one, *rf_tail, -64,
+                           8, 4, 1, 1, 1, 1, 8, None) == EINVAL
+    assert L.slayer_rf_fwd(one, None, one, None, None, one, one, one, one, one, one, one, *rf_tail, 64,
+                           8, 4, 1, 1, 1, 1, 8, None) == ENULL                               # real without imag trace
 
 
 def test_operators_refuse_cpu_tensors():
