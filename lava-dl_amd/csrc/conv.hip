@@ -167,17 +167,15 @@ __global__ __launch_bounds__(kWave) void conv_mfma_kernel(float* __restrict__ ou
     for (int t0 = tbeg; t0 < tend; t0 += 16 * RING) {
 #pragma unroll
         for (int u = 0; u < RING; ++u) {
-            // two accumulators: consecutive instructions do not wait for each other's result
-            mfma_f4 acc = {0.0f, 0.0f, 0.0f, 0.0f}, acc2 = {0.0f, 0.0f, 0.0f, 0.0f};
+            mfma_f4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int g = 0; g < G; ++g) {
                 const float4 xv = x[(u + g) % RING];
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][0], xv.x, acc, 0, 0, 0);
-                acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][1], xv.y, acc2, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][1], xv.y, acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][2], xv.z, acc, 0, 0, 0);
-                acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][3], xv.w, acc2, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][3], xv.w, acc, 0, 0, 0);
             }
-            acc += acc2;
             // tiles past the end of the span (the last pass of the loop may hold some) store nothing
             const int t = t0 + 16 * u + 4 * kq;
             buf_store4<false>(dst, (row_ok && t < tend) ? row_off + t * 4 : kOutOfRange,
