@@ -126,11 +126,10 @@ class Neuron(_Base):
         if self.persistent_state:
             with torch.no_grad():
                 last = spike[..., -1]
-                self.current_state = current_last.clone()
-                self.voltage_state = voltage_last.clone()
-                self.refractory_state = adaptive_threshold.persistent_ref_state(ref_last, last, th_last).detach().clone()
-                self.threshold_state = adaptive_threshold.persistent_th_state(
-                    th_last, last, self.threshold_step).detach().clone()
+                self._carry(current_state=current_last, voltage_state=voltage_last,
+                            refractory_state=adaptive_threshold.persistent_ref_state(ref_last, last, th_last).detach(),
+                            threshold_state=adaptive_threshold.persistent_th_state(
+                                th_last, last, self.threshold_step).detach())
         if self.drop is not None:
             spike = self.drop(spike)
         return spike

@@ -159,9 +159,10 @@ class Neuron(torch.nn.Module):
 
     def _carry(self, **states):
         """Store the states to carry into the next call (registered buffers; written directly, the
-        generic attribute path of torch.nn.Module costs several microseconds per state)."""
+        generic attribute path of torch.nn.Module costs several microseconds per state).  A slice of a
+        trace is copied so that the trace can be freed; a tensor of its own is kept as it is."""
         for name, value in states.items():
-            self._buffers[name] = value
+            self._buffers[name] = value.clone() if value._is_view() else value
 
     def _q(self, name):
         """Integer-valued decay with a straight-through gradient."""

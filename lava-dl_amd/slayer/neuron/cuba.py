@@ -101,7 +101,7 @@ class Neuron(_Base):
             voltage_last = voltage[..., -1]
         if self.persistent_state:
             with torch.no_grad():               # the product below is a new tensor; slices of a trace are copied
-                self._carry(current_state=current_last.clone() if current_last._is_view() else current_last,
+                self._carry(current_state=current_last,
                             voltage_state=leaky_integrator.persistent_state(voltage_last, spike[..., -1]).detach())
         if self.drop is not None:
             spike = self.drop(spike)

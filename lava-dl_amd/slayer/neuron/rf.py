@@ -192,8 +192,7 @@ class Neuron(ResonatorNeuron):
             real_last, imag_last = real[..., -1], imag[..., -1]
         if self.persistent_state:
             with torch.no_grad():
-                self.real_state = real_last.clone()
-                self.imag_state = imag_last.clone()
+                self._carry(real_state=real_last, imag_state=imag_last)
         if self.drop is not None:
             spike = self.drop(spike)
         return spike
