@@ -17,8 +17,10 @@ Pin status (see tests/test_oracle_*.py):
                                   vectors computed by the reference's CPU branch
                                   (tests/golden/make_reference_vectors.py)
   li_fwd beyond 2**24             the same vectors (float32 reset compare)
-  ath_fwd                         scalar spec + closed forms + leak invariants
-  apth_fwd, adres_fwd             scalar spec; identity with the pinned pieces they are made of
+  ath_fwd                         vectors of the reference's alif.Neuron (tests/golden/make_reference_neuron_vectors.py)
+                                  + scalar spec + closed forms + leak invariants
+  apth_fwd, adres_fwd             vectors of the reference's adrf.Neuron / adrf_iz.Neuron (same script) + scalar spec;
+                                  identity with the pinned pieces they are made of
                                   (ath recurrences + complex spike condition; res_fwd + ath_fwd on imag)
   li_bwd, res_bwd                 torch autograd through a float IIR + scipy.signal.lfilter (float64)
   spike_bwd, cspike_bwd           closed forms evaluated in float64

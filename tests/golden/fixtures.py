@@ -87,3 +87,29 @@ def reference_big_state_vectors():
                         cos=torch.tensor(z[f'res{k}_cos']), re=state(z[f'res{k}_re']), im=state(z[f'res{k}_im'])))
         k += 1
     return li, res
+
+
+def reference_neuron_vectors():
+    """Vectors written by make_reference_neuron_vectors.py from the reference's own neuron classes (alif, adrf,
+    adrf_iz, sigma_delta; CPU branch, persistent state, two consecutive calls).  Returns a list of dicts:
+    name, module, kwargs, inputs [call] (tensor or (real, imag)), outputs [call], states [call] {name: tensor},
+    params {name: tensor}."""
+    import json
+    z = np.load(os.path.join(HERE, 'reference_neuron_vectors.npz'))
+    names = sorted({k.split('/')[0] for k in z.files})
+    cases = []
+    for name in names:
+        pick = {k[len(name) + 1:]: z[k] for k in z.files if k.startswith(name + '/')}
+        case = dict(name=name, module=str(pick['module']), kwargs=json.loads(str(pick['kwargs'])),
+                    inputs=[], outputs=[], states=[], params={})
+        for call in (0, 1):
+            if f'in{call}' in pick:
+                case['inputs'].append(torch.tensor(pick[f'in{call}']))
+            else:
+                case['inputs'].append((torch.tensor(pick[f'in{call}_real']), torch.tensor(pick[f'in{call}_imag'])))
+            case['outputs'].append(torch.tensor(pick[f'out{call}']))
+            case['states'].append({k.split('/', 1)[1]: torch.tensor(v) for k, v in pick.items()
+                                   if k.startswith(f'state{call}/')})
+        case['params'] = {k.split('/', 1)[1]: torch.tensor(v) for k, v in pick.items() if k.startswith('param/')}
+        cases.append(case)
+    return cases

@@ -133,3 +133,49 @@ def test_sigma_delta_neuron_matches_oracle_chain_and_split(slayer, cum_error):
     m = slayer.neuron.sigma_delta.Neuron(0.25, torch.relu, cum_error=cum_error, persistent_state=True).to(dev())
     parts = torch.cat([m(x[..., :k].to(dev())), m(x[..., k:].to(dev()))], dim=-1)
     assert torch.equal(parts, out), 'sigma_delta output differs after the split'
+
+
+def _reference_neuron_cases():
+    from tests.golden import fixtures as G
+    return G.reference_neuron_vectors()
+
+
+@pytest.mark.parametrize('case', _reference_neuron_cases(), ids=lambda c: c['name'])
+def test_neurons_against_vectors_of_the_reference_classes(slayer, case):
+    """alif / adrf / adrf_iz / sigma_delta neurons against outputs of the reference's own classes
+    (tests/golden/make_reference_neuron_vectors.py): same constructor arguments and parameters, two consecutive
+    calls with persistent state; spikes (graded values included) and every carried state must be equal."""
+    module = getattr(slayer.neuron, case['module'])
+    kwargs = dict(case['kwargs'], persistent_state=True)
+    if 'activation' in kwargs:
+        kwargs['activation'] = {'relu': torch.relu}[kwargs['activation']]
+    neuron = module.Neuron(**kwargs).to(dev())
+    first = case['inputs'][0]
+    gpu = (lambda x: tuple(t.to(dev()) for t in x) if isinstance(x, tuple) else x.to(dev()))
+    if hasattr(neuron, '_prepare'):
+        neuron._prepare(first[0].to(dev()) if isinstance(first, tuple) else first.to(dev()))
+    with torch.no_grad():
+        for pname, value in case['params'].items():
+            owner = neuron
+            *path, leaf = pname.split('.')
+            for part in path:
+                owner = getattr(owner, part)
+            getattr(owner, leaf).data = value.to(dev()).reshape(getattr(owner, leaf).shape
+                                                                if getattr(owner, leaf).numel() == value.numel()
+                                                                else value.shape)
+        for call in (0, 1):
+            out = neuron(gpu(case['inputs'][call]))
+            want = case['outputs'][call]
+            assert float((want != 0).float().mean()) > 0.02
+            assert_exact(out, want, f"{case['name']} output of call {call}")
+            for sname, value in case['states'][call].items():
+                owner = neuron
+                *path, leaf = sname.split('.')
+                for part in path:
+                    owner = getattr(owner, part)
+                if case['module'] == 'sigma_delta':
+                    # the running sum of arbitrary floats: torch.cumsum groups the additions differently on every
+                    # backend (sequential here), the last bits of the carried sums may differ
+                    assert_rel(getattr(owner, leaf), value, f"{case['name']} {sname} after call {call}", rel=1e-5)
+                else:
+                    assert_exact(getattr(owner, leaf), value, f"{case['name']} {sname} after call {call}")

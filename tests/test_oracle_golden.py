@@ -2,6 +2,7 @@
 (tests/lava/lib/dl/netx/test_blocks.py:180-332 in the reference tree), plus
 mutations showing that each fixture is sensitive to the rule it pins."""
 import numpy as np
+import pytest
 import torch
 
 from oracle import slayer_oracle as O
@@ -119,3 +120,85 @@ def test_resonator_threshold_mode_beyond_float32_integers_matches_reference_vect
         re, im = O.res_fwd(case['xr'], case['xi'], case['sin'], case['cos'], zero, zero, G.W_SCALE, case['threshold'])
         assert torch.equal(re, case['re']), case['threshold']
         assert torch.equal(im, case['im']), case['threshold']
+
+
+def _neuron_case(name):
+    return next(c for c in G.reference_neuron_vectors() if c['name'] == name)
+
+
+def _per_channel(v):
+    return v.round()              # the neurons hand the dynamics rounded decays (quantize)
+
+
+@pytest.mark.parametrize('name', ['alif_shared', 'alif_graded_channel'])
+def test_oracle_chain_equals_the_reference_alif_neuron(name):
+    """First call (initial states) of the reference's alif.Neuron, from tests/golden/reference_neuron_vectors.npz:
+    li_fwd -> li_fwd -> ath_fwd -> spike_fwd composed the way neuron/alif.py:499-525,557-591 does, plus the
+    states it carries over."""
+    c = _neuron_case(name)
+    k, p, x = c['kwargs'], c['params'], c['inputs'][0]
+    w = k.get('scale', 64)
+    s = w * 64
+    thr = int(k['threshold'] * w) / w
+    step = int(k['threshold_step'] * w) / w
+    zero = torch.tensor([0.0])
+    cur = O.li_fwd(x, _per_channel(p['current_decay']), zero, s)
+    vol = O.li_fwd(cur, _per_channel(p['voltage_decay']), zero, s)
+    th, ref = O.ath_fwd(vol, zero, _per_channel(p['refractory_decay']), torch.tensor([thr]),
+                        _per_channel(p['threshold_decay']), step, thr, s)
+    spk = O.spike_fwd(vol, th + ref, graded=k.get('graded_spike', False), scale=1)
+    assert torch.equal(spk, c['outputs'][0])
+    st = c['states'][0]
+    assert torch.equal(cur[..., -1], st['current_state']) and torch.equal(vol[..., -1], st['voltage_state'])
+    last = spk[..., -1]
+    assert torch.equal(O.ath_persistent_ref_state(ref[..., -1], last, th[..., -1]), st['refractory_state'])
+    assert torch.equal(O.ath_persistent_th_state(th[..., -1], last, step), st['threshold_state'])
+
+
+@pytest.mark.parametrize('name', ['adrf_shared', 'adrf_channel', 'adrf_iz_shared', 'adrf_iz_graded'])
+def test_oracle_chain_equals_the_reference_adaptive_resonators(name):
+    """First call of adrf.Neuron (res_fwd -> apth_fwd -> complex spike, neuron/adrf.py:583-660) and of
+    adrf_iz.Neuron (adres_fwd -> spike, neuron/adrf_iz.py:574-645): pins apth_fwd and adres_fwd to outputs of the
+    reference itself."""
+    c = _neuron_case(name)
+    k, p = c['kwargs'], c['params']
+    xr, xi = c['inputs'][0]
+    w = k.get('scale', 64)
+    s = w * 64
+    thr = int(k['threshold'] * w) / w
+    step = int(k['threshold_step'] * w) / w
+    zero = torch.tensor([0.0])
+    sin, cos = _per_channel(p['sin_decay']), _per_channel(p['cos_decay'])
+    d_th, d_ref = _per_channel(p['threshold_decay']), _per_channel(p['refractory_decay'])
+    graded = k.get('graded_spike', False)
+    st = c['states'][0]
+    if c['module'] == 'adrf':
+        re, im = O.res_fwd(xr, xi, sin, cos, zero, zero, s)
+        th, ref = O.apth_fwd(re, im, zero, zero, d_ref, torch.tensor([thr]), d_th, step, thr, s)
+        spk = O.cspike_fwd(re, im, th + ref, 0.0, graded=graded, scale=1)
+    else:
+        re, im, th, ref = O.adres_fwd(xr, xi, sin, cos, d_ref, d_th, zero, zero, zero, torch.tensor([thr]), step, thr, s)
+        spk = O.spike_fwd(im, th + ref, graded=graded, scale=1)
+    assert float((spk != 0).float().mean()) > 0.02
+    assert torch.equal(spk, c['outputs'][0])
+    assert torch.equal(re[..., -1], st['real_state']) and torch.equal(im[..., -1], st['imag_state'])
+
+
+def test_oracle_chain_equals_the_reference_sigma_delta_neuron():
+    """sigma_delta.Neuron (neuron/sigma_delta.py:171-219): running sum -> activation -> delta encoder, both
+    calls (the second starts from the carried sums and residuals)."""
+    c = _neuron_case('sigma_delta_relu')
+    thr = c['params']['delta.threshold']
+    pre_sigma = None
+    pre = res = err = torch.zeros(c['inputs'][0].shape[:-1])
+    for call in (0, 1):
+        dend = O.sigma_fwd(c['inputs'][call], pre_sigma)
+        act = torch.relu(dend)
+        out, _, res, err = O.delta_fwd(act, thr, pre, res, err)
+        out = O.quantize_floor(out, 1 / 4096)            # Delta.forward floors its events to the state grid (64 * 64)
+        assert float((out != 0).float().mean()) > 0.05
+        assert torch.equal(out, c['outputs'][call]), call
+        pre_sigma, pre = dend[..., -1], act[..., -1]
+        st = c['states'][call]
+        assert torch.allclose(pre_sigma, st['sigma.pre_state'], rtol=1e-5, atol=1e-6)      # summation order
+        assert torch.allclose(res, st['delta.residual_state'], rtol=1e-4, atol=1e-5)
