@@ -44,6 +44,22 @@ class _Null:
         return False
 
 
+class _Section:
+    def __init__(self, timers, name):
+        self.timers, self.name = timers, name
+
+    def __enter__(self):
+        self.a = torch.cuda.Event(enable_timing=True)
+        self.b = torch.cuda.Event(enable_timing=True)
+        self.a.record()
+        return self
+
+    def __exit__(self, *exc):
+        self.b.record()
+        self.timers.events.setdefault(self.name, []).append((self.a, self.b))
+        return False
+
+
 class Timers:
     """Per-op device time from events recorded on the stream the kernels are launched on
     (torch's current stream)."""
@@ -52,23 +68,17 @@ class Timers:
         self.events = {}
 
     def section(self, name):
-        timers = self
+        return _Section(self, name)
 
-        class _S:
-            def __enter__(self):
-                self.a = torch.cuda.Event(enable_timing=True)
-                self.b = torch.cuda.Event(enable_timing=True)
-                self.a.record()
-                return self
-
-            def __exit__(self, *a):
-                self.b.record()
-                timers.events.setdefault(name, []).append((self.a, self.b))
-                return False
-        return _S()
-
-    def mean_ms(self):
-        return {k: sum(a.elapsed_time(b) for a, b in v) / len(v) for k, v in self.events.items()}
+    def median_ms(self):
+        """Median over the passes: an interval between two events also contains whatever kept the host from
+        launching in time (an allocator or interpreter pause shows up as tens of milliseconds in one pass)."""
+        out = {}
+        for k, v in self.events.items():
+            times = sorted(a.elapsed_time(b) for a, b in v)
+            n = len(times)
+            out[k] = times[n // 2] if n % 2 else 0.5 * (times[n // 2 - 1] + times[n // 2])
+        return out
 
 
 class Workload:
@@ -584,7 +594,7 @@ def main():
     for _ in range(max(3, a.steps // 2)):
         job.step(timers.section)
     torch.cuda.synchronize()
-    op_ms = timers.mean_ms()
+    op_ms = timers.median_ms()
     per_op = []
     for name, kernel, bpn in job.ops:
         gbs = nt * bpn / (op_ms[name] * 1e-3) / 1e9

@@ -18,6 +18,7 @@ struct AthFwd {
         int64_t npb, n_rd, n_td, n_rs, n_ts;
     };
     static constexpr bool kTransforms = true;    // integer tiles, see to_state / from_state
+    static constexpr int kCopyWaves = 2;
     int th, r, mt, mr, th_step, base;
     float w, inv_w;
 

@@ -32,6 +32,7 @@ struct CubaFwd {
         int64_t npb, n_id, n_vd, n_is, n_vs;
     };
     static constexpr bool kTransforms = true;        // integer tiles, see to_state / from_state
+    static constexpr int kCopyWaves = 2;
     int yc, yv, yv_out, mi, mv, fire_above;
     float w, inv_w, spike_thr, spike_scale;
 

@@ -23,6 +23,7 @@ struct LiFwd {
     // on its way into LDS, the state is converted and scaled back on its way out, and the
     // sequential loop is left with the recurrence alone.
     static constexpr bool kTransforms = true;
+    static constexpr int kCopyWaves = 2;
     int y, mult, fire_above;
     float w, inv_w;
 
