@@ -93,7 +93,7 @@ def reference_neuron_vectors():
     """Vectors written by make_reference_neuron_vectors.py from the reference's own neuron classes (alif, adrf,
     adrf_iz, sigma_delta; CPU branch, persistent state, two consecutive calls).  Returns a list of dicts:
     name, module, kwargs, inputs [call] (tensor or (real, imag)), outputs [call], states [call] {name: tensor},
-    params {name: tensor}."""
+    params {name: tensor}, grad_out and grad_in (list: one entry per input tensor of the first call)."""
     import json
     z = np.load(os.path.join(HERE, 'reference_neuron_vectors.npz'))
     names = sorted({k.split('/')[0] for k in z.files})
@@ -111,5 +111,8 @@ def reference_neuron_vectors():
             case['states'].append({k.split('/', 1)[1]: torch.tensor(v) for k, v in pick.items()
                                    if k.startswith(f'state{call}/')})
         case['params'] = {k.split('/', 1)[1]: torch.tensor(v) for k, v in pick.items() if k.startswith('param/')}
+        # gradient of sum(output * grad_out) with respect to the first input (no carried state)
+        case['grad_out'] = torch.tensor(pick['grad_out'])
+        case['grad_in'] = [torch.tensor(pick[f'grad_in{i}']) for i in (0, 1) if f'grad_in{i}' in pick]
         cases.append(case)
     return cases

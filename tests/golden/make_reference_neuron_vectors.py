@@ -13,7 +13,9 @@ Only the CPU branch is exercised.  No bytecode is written.
 
 Every case: a neuron with persistent state is built from the recorded keyword arguments, called on two
 consecutive inputs (the second call starts from the carried state), and its outputs and carried states are stored.
-Per-channel parameters are drawn at random by the neuron on its first call and are stored as well.
+Per-channel parameters are drawn at random by the neuron on its first call and are stored as well.  A second
+neuron with the same parameters and no carried state runs the first input again with autograd on, and the
+gradient of sum(output * g) with respect to the input(s) is stored together with g.
 """
 import importlib
 import json
@@ -106,6 +108,24 @@ def main():
                 out[f'{name}/state{call}/{sname}'] = state.detach().numpy().copy()
         for pname, prm in neuron.named_parameters(recurse=True):
             out[f'{name}/param/{pname}'] = prm.detach().numpy().copy()
+        # gradients: a fresh neuron without carried state and with the same parameters, first input again
+        torch.manual_seed(5200 + k)
+        fresh = mods[module].Neuron(**dict(build, persistent_state=False))
+        g = torch.randn(SHAPE, generator=gen)
+        if is_complex:
+            leaves = [torch.tensor(out[f'{name}/in0_real']).requires_grad_(),
+                      torch.tensor(out[f'{name}/in0_imag']).requires_grad_()]
+            y = fresh.spike(*fresh.dynamics(tuple(leaves))) if module == 'adrf_iz' else fresh(tuple(leaves))
+        else:
+            leaves = [torch.tensor(out[f'{name}/in0']).requires_grad_()]
+            y = fresh(leaves[0])
+        for pname, prm in fresh.named_parameters(recurse=True):
+            assert np.array_equal(prm.detach().numpy(), out[f'{name}/param/{pname}']), pname
+        assert np.array_equal(y.detach().numpy(), out[f'{name}/out0'])
+        y.backward(g)
+        out[f'{name}/grad_out'] = g.numpy()
+        for i, leaf in enumerate(leaves):
+            out[f'{name}/grad_in{i}'] = leaf.grad.numpy()
         print(name, 'events per call', [float((out[f'{name}/out{c}'] != 0).mean()) for c in (0, 1)])
     path = os.path.join(DST, 'reference_neuron_vectors.npz')
     np.savez_compressed(path, **out)

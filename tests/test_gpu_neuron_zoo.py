@@ -179,3 +179,37 @@ def test_neurons_against_vectors_of_the_reference_classes(slayer, case):
                     assert_rel(getattr(owner, leaf), value, f"{case['name']} {sname} after call {call}", rel=1e-5)
                 else:
                     assert_exact(getattr(owner, leaf), value, f"{case['name']} {sname} after call {call}")
+
+
+def _with_parameters(neuron, case, first):
+    if hasattr(neuron, '_prepare'):
+        neuron._prepare(first[0] if isinstance(first, tuple) else first)
+    with torch.no_grad():
+        for pname, value in case['params'].items():
+            owner = neuron
+            *path, leaf = pname.split('.')
+            for part in path:
+                owner = getattr(owner, part)
+            prm = getattr(owner, leaf)
+            prm.data = value.to(dev()).reshape(prm.shape if prm.numel() == value.numel() else value.shape)
+    return neuron
+
+
+@pytest.mark.parametrize('case', _reference_neuron_cases(), ids=lambda c: c['name'])
+def test_neuron_gradients_against_vectors_of_the_reference_classes(slayer, case):
+    """Input gradients of the same neurons (surrogate constants, which tensors the gradient flows through):
+    d sum(output * g) / d input from the reference's own autograd, within 1e-5 relative."""
+    module = getattr(slayer.neuron, case['module'])
+    kwargs = dict(case['kwargs'])
+    if 'activation' in kwargs:
+        kwargs['activation'] = {'relu': torch.relu}[kwargs['activation']]
+    neuron = module.Neuron(**kwargs).to(dev())
+    first = case['inputs'][0]
+    leaves = [t.to(dev()).requires_grad_() for t in (first if isinstance(first, tuple) else (first,))]
+    _with_parameters(neuron, case, tuple(leaves) if len(leaves) == 2 else leaves[0])
+    out = neuron(tuple(leaves) if len(leaves) == 2 else leaves[0])
+    assert_exact(out, case['outputs'][0], f"{case['name']} output")
+    out.backward(case['grad_out'].to(dev()))
+    for i, want in enumerate(case['grad_in']):
+        assert float(want.abs().max()) > 0
+        assert_rel(leaves[i].grad, want, f"{case['name']} gradient of input {i}")
