@@ -12,6 +12,7 @@ whole-job neuron-timesteps/s, per-kernel roofline and the CPU baseline (the torc
 timed on this box's host cores).
 """
 import argparse
+import gc
 import json
 import math
 import os
@@ -583,11 +584,14 @@ def main():
     for _ in range(a.warmup):
         job.step(null)
     torch.cuda.synchronize()
+    gc.collect()
+    gc.disable()                 # a collection of the interpreter's cyclic garbage would stall the launches for milliseconds
     t0 = time.perf_counter()
     for _ in range(a.steps):
         job.step(null)
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / a.steps
+    gc.enable()
 
     # per-kernel device time (separate pass so the event records do not perturb the headline number)
     timers = Timers()
