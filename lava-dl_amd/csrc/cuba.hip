@@ -103,7 +103,7 @@ struct CubaBwd {
         }
     }
     // The surrogate does not depend on the recurrence, so it is evaluated on the way into LDS (by all
-    // 64 lanes, or by the copy wave of the multi-wave kernel) and takes the place of the incoming gradient.
+    // 64 lanes, or by the copy waves of the multi-wave kernel) and takes the place of the incoming gradient.
     static constexpr bool kTransforms = true;
     static constexpr int kCopyWaves = 4;
     __device__ __forceinline__ float surrogate(float g, float v) const {

@@ -130,7 +130,7 @@ struct TileGeom {
 //     elementwise maps (wave-uniform members only) applied to the input quads on their way into LDS
 //     and to the output quads on their way out, so that work that does not belong to the
 //     sequential dependency chain (scaling, int <-> float conversion) is done by all 64 lanes in
-//     the copy phases, or by the copy wave of the two-wave kernel;
+//     the copy phases, or by the copy waves of the multi-wave kernel;
 //   optionally static constexpr int kDerived = 1 and
 //     __device__ float4 derive(const float4 (&y)[kOut]) const;   (uses wave-uniform members only)
 //     an extra output, Params::out[kOut], that is an elementwise function of the other outputs of
@@ -615,7 +615,7 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 constexpr int64_t kAlways = (int64_t)1 << 62;
 
-// Rows per workgroup of the two-wave kernel: 64 unless the Op says otherwise (kDuoRows).
+// Rows per workgroup of the multi-wave kernel: 64 unless the Op says otherwise (kDuoRows).
 template <class Op, class = void>
 struct DuoRows { static constexpr int value = 64; };
 template <class Op>
@@ -669,7 +669,7 @@ int launch_stream_rows(const typename Op::Params& prm, int64_t M, int64_t T, boo
 //  * dwordx4 path when T and every pointer allow it, else the dword fallback;
 //  * non-temporal global accesses when the tensors are too large to be reused out of the
 //    last-level cache;
-//  * while every workgroup of the two-wave kernel is resident at once, run time is set by the
+//  * while every workgroup of the multi-wave kernel is resident at once, run time is set by the
 //    latency of the sequential wave and that kernel is 10-40% faster (all 64 lanes hold a row);
 //  * beyond that the one-wave kernel, with the rows per wave the Op asks for (kRows32Below,
 //    kRows16Below): integer forward recurrences and backward passes with an exp per step keep all
