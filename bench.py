@@ -568,7 +568,8 @@ def main():
     a = ap.parse_args()
     if a.gpus != 1:
         raise SystemExit('bench.py measures one GPU: this hot path has no multi-GPU component '
-                         '(neurons are independent; DESIGN.md says how it would shard). Use --gpus 1.')
+                         '(neurons are independent, so it would shard along the batch axis with one small all-reduce of the '
+                         'parameter gradients). Use --gpus 1.')
     assert torch.cuda.is_available(), 'bench.py needs a GPU'
     dev = torch.device('cuda:0')
     torch.cuda.set_device(dev)
