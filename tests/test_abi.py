@@ -104,3 +104,25 @@ def test_right_shift_to_zero():
     assert slayer.utils.int_utils.right_shift_to_zero(x, 12).tolist() == [-2, -1, -1, 0, 0, 0, 0, 0, 1, 1]
     with pytest.raises(Exception):
         slayer.utils.right_shift_to_zero(torch.zeros(2), 12)
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    """Without the built library there is nothing to fall back to: the first use raises and says how to build it
+    (checked in a fresh interpreter so that the loaded library of this process is not disturbed)."""
+    import subprocess
+    import sys
+    code = (
+        'import sys, torch\n'
+        f'sys.path.insert(0, {ROOT!r})\n'
+        'import lava_dl_amd.slayer as slayer\n'
+        'from lava_dl_amd.slayer import _native\n'
+        'try:\n'
+        '    _native.lib()\n'
+        'except RuntimeError as e:\n'
+        '    print("RAISED", e)\n'
+        'else:\n'
+        '    print("LOADED")\n')
+    env = dict(os.environ, SLAYER_HIP_LIB=str(tmp_path / 'libslayer_hip.so'))
+    run = subprocess.run([sys.executable, '-c', code], env=env, capture_output=True, text=True, timeout=300)
+    assert 'RAISED' in run.stdout and 'is missing' in run.stdout and 'no fallback' in run.stdout.lower(), \
+        run.stdout + run.stderr
