@@ -195,6 +195,12 @@ __device__ __forceinline__ void buf_store4(__amdgpu_buffer_rsrc_t r, int byte_of
 // piece, and the eight lanes that cover the line store it whole with one instruction.  Only the
 // lines shared with neighbouring workgroups are still written in pieces.
 //
+// Ownership rule.  A wave completes a shared line only when both rows that meet in it belong to
+// the passes this wave owns.  Copy waves that share a tile run without a barrier among themselves
+// (one fills a tile buffer with the next chunk right after it has copied the previous chunk out),
+// so a quad taken from a row of another wave could already have been overwritten; at the edge of a
+// wave's row range the line is therefore written in two pieces, as at the edge of a workgroup.
+//
 // Interior chunks (every column of every row inside [0, T), no shared line) run a branch-free
 // recurrence loop; only the first and the last one or two chunks take the predicated path.
 // Everything a wave needs to move the tiles of its R rows between global memory and LDS: buffer
@@ -216,11 +222,15 @@ struct Copier {
     float4 stage[NI][kPasses];               // prefetched inputs
     float4 keep[NO][kPasses];                // first-produced pieces of shared lines, one quad per pass
     int rows, T, crow, cq, interior_end, first_pass;
+    int row_lo, row_hi;                      // rows [row_lo, row_hi) of the tile are copied by this wave
     bool route;
 
     __device__ __forceinline__ void init(const typename Op::Params& prm, int64_t m0, int rows_, int T_, int lane,
                                          unsigned base_f, int first_pass_ = 0) {
         rows = rows_; T = T_; first_pass = first_pass_;
+        row_lo = first_pass * G::kRowsPerPass;
+        row_hi = (first_pass + kPasses) * G::kRowsPerPass;
+        if (row_hi > rows) row_hi = rows;
         const unsigned wave_bytes = (unsigned)rows * (unsigned)T * 4u;
 #pragma unroll
         for (int i = 0; i < NI; ++i)         // an input the caller does not have: every load falls out of range, reads 0
@@ -309,14 +319,16 @@ struct Copier {
                 const int a_next = (a + T) & 31;                   // phase of row r+1
                 const int tail_pos = (a + T) & ~31;                // window position of row r's partial last line
                 const int prev_tail_pos = (((a - T) & 31) + T) & ~31;   // the same for row r-1
-                // the pieces of a line shared with a neighbouring row of this wave
-                const bool own_head = route && r >= 1 && r < rows && a != 0 && cq < 8 && 4 * cq >= a;
-                const bool own_tail = route && valid && r + 1 < rows && 4 * cq + chunk * TC >= tail_pos;
+                // the pieces of a line shared with a neighbouring row that this wave copies too
+                const bool prev_mine = r > row_lo && r < row_hi;       // row r-1 is one of this wave's rows
+                const bool next_mine = r + 1 < row_hi;                 // row r+1 is one of this wave's rows
+                const bool own_head = route && prev_mine && a != 0 && cq < 8 && 4 * cq >= a;
+                const bool own_tail = route && valid && next_mine && 4 * cq + chunk * TC >= tail_pos;
                 bool take, release;
                 int idx;                                           // tile position of the quad to take
                 if (Op::kReverse) {
                     // slot cq of row r's first line, before the row starts: tail of row r-1
-                    const bool slot = route && r >= 1 && r < rows && a != 0 && cq < 8 && 4 * cq < a;
+                    const bool slot = route && prev_mine && a != 0 && cq < 8 && 4 * cq < a;
                     const int kp = prev_tail_pos / TC;
                     take = slot && chunk == kp;
                     release = slot && chunk == 0;
@@ -326,7 +338,7 @@ struct Copier {
                     // slot j of row r's last line, past the end of the row: head of row r+1
                     const int kt = tail_pos / TC;
                     const int j = cq - (tail_pos - kt * TC) / 4;
-                    const bool slot = route && r + 1 < rows && a_next != 0 && j >= 0 && j < 8 && 4 * j >= a_next;
+                    const bool slot = route && next_mine && a_next != 0 && j >= 0 && j < 8 && 4 * j >= a_next;
                     take = slot && chunk == 0;
                     release = slot && chunk == kt;
                     idx = (r + 1) * G::kPitch + 4 * j;
