@@ -42,6 +42,7 @@ extern "C" {
 #define SLAYER_EINVAL   (-1)   /* inconsistent sizes (M, T, neurons_per_batch, num_params, ...) */
 #define SLAYER_ENULL    (-2)   /* a required pointer is NULL */
 #define SLAYER_ERANGE   (-3)   /* a size exceeds what the kernels index (M*T >= 2^40, T >= 2^31, K > 4096 ...) */
+#define SLAYER_ESCRATCH (-4)   /* a size exceeds the library's built-in scratch buffer (slayer_li_bwd_static) */
 
 int slayer_abi_version(void);
 
@@ -71,6 +72,20 @@ int slayer_li_bwd(float *grad_in, float *grad_decay, const float *grad_out, cons
                   const float *decay, float *workspace,
                   int64_t M, int64_t neurons_per_batch, int64_t num_decays,
                   int64_t T, void *stream);
+
+/* slayer_li_bwd for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): same arguments without `workspace`, same kernels, same
+ * results bit for bit.  It has no counterpart in the reference.  The scratch is a buffer built into the
+ * library (5 MiB of device memory per GPU, held until the process ends); the call allocates and frees
+ * nothing.  Limits: M <= SLAYER_LI_BWD_STATIC_MAX_ROWS and num_decays <= SLAYER_LI_BWD_STATIC_MAX_DECAYS,
+ * else SLAYER_ESCRATCH is returned and nothing is launched.  All calls on one GPU share the one buffer:
+ * calls that overlap on the same GPU (different streams, or threads) race; serialise them. */
+#define SLAYER_LI_BWD_STATIC_MAX_ROWS   (1 << 20)
+#define SLAYER_LI_BWD_STATIC_MAX_DECAYS 4096
+int slayer_li_bwd_static(float *grad_in, float *grad_decay, const float *grad_out, const float *out,
+                         const float *decay,
+                         int64_t M, int64_t neurons_per_batch, int64_t num_decays,
+                         int64_t T, void *stream);
 
 /* ---- adaptive threshold + refractory ---------------------------------------------------- */
 

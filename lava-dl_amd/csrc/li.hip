@@ -1,6 +1,7 @@
 // Leaky integrator: forward fixed-point recurrence and reverse-time gradient.
 #include "common.h"
 #include "tile.h"
+#include <mutex>
 
 namespace slayer {
 
@@ -148,6 +149,34 @@ int launch_reduce_param_grad(float* grad, const float* partial, float* scratch, 
     return (int)hipGetLastError();
 }
 
+// Scratch of the entry point that allocates nothing (slayer_li_bwd_static): per-neuron partial sums for
+// up to kStaticMaxRows neurons followed by kRedMaxSplit slice sums for each of up to kStaticMaxDecays
+// decays.  5 MiB of device memory on every GPU the library runs on, held until the process ends.
+constexpr int64_t kStaticMaxRows = SLAYER_LI_BWD_STATIC_MAX_ROWS;
+constexpr int64_t kStaticMaxDecays = SLAYER_LI_BWD_STATIC_MAX_DECAYS;
+static __device__ __align__(256) float scratch[kStaticMaxRows + kRedMaxSplit * kStaticMaxDecays];
+
+// Device address of `scratch` on the current device (in host code the array's name is only a
+// stand-in for the symbol, not an address a kernel could use).  Every GPU holds its own copy, so the
+// address is looked up once per device, with that device current.
+static int static_scratch(float** out) {
+    constexpr int kMaxDevices = 64;
+    static float* ptrs[kMaxDevices] = {nullptr};
+    static std::mutex lock;
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev)) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return SLAYER_ERANGE;
+    std::lock_guard<std::mutex> guard(lock);
+    if (!ptrs[dev]) {
+        float* p = nullptr;
+        if (hipError_t e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch))) return (int)e;
+        if (!p) return (int)hipErrorInvalidSymbol;
+        ptrs[dev] = p;
+    }
+    *out = ptrs[dev];
+    return 0;
+}
+
 }  // namespace slayer
 
 using namespace slayer;
@@ -191,4 +220,16 @@ extern "C" int slayer_li_bwd(float* grad_in, float* grad_decay, const float* gra
                                         (hipStream_t)stream);
     }
     return 0;
+}
+
+extern "C" int slayer_li_bwd_static(float* grad_in, float* grad_decay, const float* grad_out, const float* out,
+                                    const float* decay, int64_t M, int64_t neurons_per_batch, int64_t num_decays,
+                                    int64_t T, void* stream) {
+    if (M > kStaticMaxRows || num_decays > kStaticMaxDecays) return SLAYER_ESCRATCH;
+    float* ws = nullptr;
+    if (grad_decay && M > 0)
+        if (int e = static_scratch(&ws)) return e;
+    // Nothing in the scratch has to start at zero: the streaming kernel writes the partial sum of every
+    // row before the reduction reads it, and the reduction writes every slice sum before it adds them.
+    return slayer_li_bwd(grad_in, grad_decay, grad_out, out, decay, ws, M, neurons_per_batch, num_decays, T, stream);
 }

@@ -29,6 +29,7 @@ _SIGNATURES = {
     'slayer_error_string': (ctypes.c_char_p, [_INT]),
     'slayer_li_fwd': (_INT, [_P, _P, _P, _P, _D, _INT, _I64, _I64, _I64, _I64, _I64, _P]),
     'slayer_li_bwd': (_INT, [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _P]),
+    'slayer_li_bwd_static': (_INT, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _P]),
     'slayer_ath_fwd': (_INT, [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _INT,
                               _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P]),
     'slayer_res_fwd': (_INT, [_P, _P, _P, _P, _P, _P, _P, _P, _D, _INT,

@@ -48,6 +48,10 @@ def test_argument_validation_happens_before_any_launch():
     assert L.slayer_li_fwd(one, one, one, one, 1.0, 64, 8, 4, 1, 1, 1 << 31, None) == ERANGE
     assert L.slayer_li_fwd(one, one, one, one, 1.0, 64, 0, 4, 1, 1, 8, None) == 0          # empty is fine
     assert L.slayer_li_bwd(one, one, one, one, one, None, 8, 4, 1, 8, None) == ENULL       # grad wanted, no workspace
+    # the allocation-free form refuses what its built-in scratch cannot hold
+    assert L.slayer_li_bwd_static(one, one, one, one, one, (1 << 20) + 64, 64, 1, 8, None) == -4
+    assert L.slayer_li_bwd_static(one, one, one, one, one, 8192, 8192, 8192, 8, None) == -4
+    assert b'scratch' in L.slayer_error_string(-4)
     assert L.slayer_res_bwd(one, one, one, None, one, one, one, one, one, one, one, 8, 4, 1, 8, None) == ENULL
     assert L.slayer_conv(one, one, one, 0, 1.0, 8, 8, None) == EINVAL
     assert L.slayer_conv(one, one, one, 5000, 1.0, 8, 8, None) == ERANGE
