@@ -1,6 +1,6 @@
 """Benchmark of the SLAYER neuron-dynamics hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cuba|cuba_fused|cuba_fused_lean|cuba_inference|cuba_fwd_small|alif|alif_fused|alif_fused_lean|rf|rf_fused|rf_fused_lean|rf_inference|synapse|synapse_fused|synapse_delay_grad]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cuba|cuba_fused|cuba_fused_lean|cuba_inference|cuba_fwd_small|alif|alif_fused|alif_fused_lean|rf|rf_fused|rf_fused_lean|rf_inference|synapse|synapse_fused|synapse_folded|synapse_delay_grad]
 
 A step is one pass of the workload's op sequence over one batch of synthetic input that is already
 resident in HBM (outputs come from torch's caching allocator inside the timed region).  The default
@@ -504,6 +504,32 @@ class SynapseFused(Synapse):
         return spk, g_x
 
 
+class SynapseFolded(SynapseFused):
+    name = ('SLAYER synapse stack (conv K=64 -> per-channel shift -> CUBA) fwd+bwd, the shift folded into the fused '
+            'CUBA kernels (read of the input, store of its gradient)')
+    ops = [('conv', 'conv_kernel', 8), ('cuba_fwd', 'stream_kernel<CubaFwd>', 12),
+           ('cuba_bwd', 'stream_kernel<CubaBwd>', 12), ('corr', 'conv_kernel<corr>', 8)]
+
+    def __init__(self, dev):
+        super().__init__(dev)
+        from lava_dl_amd.slayer.neuron.dynamics import delays
+        self.D = delays
+        self.delays = delays.Delays(input_shift=self.delay)
+
+    def step(self, t):
+        with t('conv'):
+            y = self.conv.fwd(self.x, self.filt, 1)
+        with t('cuba_fwd'):
+            _, vol, spk = self.F._fwd(y, self.d_i, self.d_v, self.zero, self.zero, 64, 1.25, False, 1, True,
+                                      folded=self.D.fold(self.delays, y))
+        with t('cuba_bwd'):
+            g_y, _, _ = self.F._bwd(self.g, vol, None, self.d_i, self.d_v, 1.25, 1.0, 1.0, False, False,
+                                    folded=self.D.fold(self.delays, self.g, forward=False))
+        with t('corr'):
+            g_x = self.conv.bwd(g_y, self.filt, 1)
+        return spk, g_x
+
+
 class SynapseDelayGrad(SynapseFused):
     name = 'SLAYER synapse stack with a learnable delay (conv K=64 -> Delay -> fused CUBA) fwd+bwd incl. the delay gradient'
     ops = [('conv', 'conv_kernel', 8), ('shift', 'shift_kernel', 8), ('cuba_fwd', 'stream_kernel<CubaFwd>', 12),
@@ -527,7 +553,7 @@ class SynapseDelayGrad(SynapseFused):
         return spk, g_x, g_delay
 
 
-WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fused_lean': CubaFusedLean, 'cuba_inference': CubaInference, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'alif_fused': AlifFused, 'alif_fused_lean': AlifFusedLean, 'rf': Rf, 'rf_fused': RfFused, 'rf_fused_lean': RfFusedLean, 'rf_inference': RfInference, 'synapse': Synapse, 'synapse_fused': SynapseFused, 'synapse_delay_grad': SynapseDelayGrad}
+WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fused_lean': CubaFusedLean, 'cuba_inference': CubaInference, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'alif_fused': AlifFused, 'alif_fused_lean': AlifFusedLean, 'rf': Rf, 'rf_fused': RfFused, 'rf_fused_lean': RfFusedLean, 'rf_inference': RfInference, 'synapse': Synapse, 'synapse_fused': SynapseFused, 'synapse_folded': SynapseFolded, 'synapse_delay_grad': SynapseDelayGrad}
 
 
 def cpu_baseline(job, budget_s=20.0):

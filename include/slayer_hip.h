@@ -37,7 +37,7 @@
 extern "C" {
 #endif
 
-#define SLAYER_ABI_VERSION 1
+#define SLAYER_ABI_VERSION 2
 
 #define SLAYER_EINVAL   (-1)   /* inconsistent sizes (M, T, neurons_per_batch, num_params, ...) */
 #define SLAYER_ENULL    (-2)   /* a required pointer is NULL */
@@ -45,6 +45,30 @@ extern "C" {
 #define SLAYER_ESCRATCH (-4)   /* a size exceeds the library's built-in scratch buffer (slayer_li_bwd_static) */
 
 int slayer_abi_version(void);
+
+/* Axonal delays folded into a fused neuron block (slayer_cuba_fwd/bwd, slayer_alif_fwd/bwd, slayer_rf_fwd/bwd),
+ * so that the shift before a neuron and the delay after it (block/base.py:15-39,549-553: step_delay, then the
+ * learnable axon/delay.py Delay; utils/time/shift.py:94-143 for the shift itself) cost no pass over the
+ * tensor of their own.  A host structure; the tables are device pointers.
+ *   forward : the neuron sees x[t] = in[t - kin] (zero where t - kin is outside [0, T)) and its spikes
+ *             leave as spike_out[t + kout] = s[t]; spike_out[kout - 1] = out_head[m] when out_head is given
+ *             (the last spike of the previous call: step_delay with persistent state), every other position
+ *             no spike reaches is 0.  State traces (current, voltage, ...) are stored unshifted.
+ *   backward: pass the same structure; grad_spikes is taken as the gradient of the delayed spikes and read as
+ *             g[t] = grad_spikes[t + kout], grad_in is stored as the gradient of `in`: grad_in[t - kin].
+ *   kin  = in_steps  + trunc(in_shift [m % neurons_per_batch] / sampling_time)   (any sign)
+ *   kout = out_steps + trunc(out_delay[m % neurons_per_batch] / sampling_time)   (any sign)
+ * as slayer_shift computes them.  Passing NULL instead of a structure means no delays at all. */
+typedef struct slayer_delays {
+    const float *in_shift;   /* neurons_per_batch floats in time units, or NULL */
+    const float *out_delay;  /* neurons_per_batch floats in time units, or NULL */
+    const float *out_head;   /* M floats, or NULL; forward only */
+    float *spike_last;       /* M floats, or NULL; forward only: receives s[T-1], the spike of the last step, which
+                              * a delayed spike tensor no longer holds (step_delay's buffer, persistent state) */
+    int64_t in_steps;        /* whole steps added to every neuron's input shift */
+    int64_t out_steps;       /* whole steps added to every neuron's output delay (step_delay: 1) */
+    float sampling_time;     /* divides the table entries; must not be 0 when a table is given */
+} slayer_delays;
 
 /* Text for a return code of this library (hipGetErrorString for positive codes). */
 const char *slayer_error_string(int code);
@@ -208,7 +232,9 @@ int slayer_shift(float *out, const float *in, const float *lut, int64_t scalar_s
  * in slayer_shift (lut == NULL: scalar_steps), and, when grad_sum is not NULL,
  * grad_sum[j] = sum over the batch and time of grad_out * ((-1/Ts) out[t] + (1/Ts) out[t-1]) for the
  * neurons_per_batch neurons of a batch element (the caller scales by Ts and grad_scale as the reference does).
- * workspace: M + 64 * neurons_per_batch floats, only read and written when grad_sum is wanted. */
+ * workspace: M + 64 * neurons_per_batch floats, only read and written when grad_sum is wanted.
+ * grad_in may be NULL when only the sums are wanted (a fused block's backward pass reads the gradient
+ * back through the delay itself): 8 instead of 12 bytes per neuron-timestep. */
 int slayer_delay_bwd(float *grad_in, float *grad_sum, const float *grad_out, const float *out,
                      const float *lut, int64_t scalar_steps, float sampling_time, float *workspace,
                      int64_t M, int64_t neurons_per_batch, int64_t T, void *stream);
@@ -277,7 +303,8 @@ int slayer_cuba_fwd(float *cur_out, float *vol_out, float *spk_out, float *cur_l
                     const float *i_state, const float *v_state,
                     double thr_scaled, float spike_threshold, int graded, float spike_scale, int w_scale,
                     int64_t M, int64_t neurons_per_batch, int64_t num_i_decays, int64_t num_v_decays,
-                    int64_t num_i_states, int64_t num_v_states, int64_t T, void *stream);
+                    int64_t num_i_states, int64_t num_v_states, int64_t T,
+                    const slayer_delays *delays, void *stream);
 
 /* Backward of the above = slayer_spike_bwd -> slayer_li_bwd (voltage) -> slayer_li_bwd (current) in
  * one launch (16 instead of 36 bytes per neuron-timestep); grad_in is bit-identical to the chain.
@@ -288,7 +315,7 @@ int slayer_cuba_bwd(float *grad_in, float *grad_i_decay, float *grad_v_decay,
                     const float *i_decay, const float *v_decay,
                     float spike_threshold, float tau_rho, float scale_rho, int graded, float *workspace,
                     int64_t M, int64_t neurons_per_batch, int64_t num_i_decays, int64_t num_v_decays,
-                    int64_t T, void *stream);
+                    int64_t T, const slayer_delays *delays, void *stream);
 
 /* ---- fused resonate-and-fire neuron ------------------------------------------------------------- */
 
@@ -306,7 +333,7 @@ int slayer_rf_fwd(float *re_out, float *im_out, float *spk_out, float *re_last_o
                   float spike_threshold, int graded, float spike_scale, int w_scale,
                   int64_t M, int64_t neurons_per_batch, int64_t num_decays,
                   int64_t num_re_states, int64_t num_im_states, int64_t num_last,
-                  int64_t T, void *stream);
+                  int64_t T, const slayer_delays *delays, void *stream);
 
 /* Backward of the above = slayer_cspike_bwd -> slayer_res_bwd in one launch (20 instead of 44 bytes
  * per neuron-timestep); the input gradients are bit-identical to the chain.  grad_sin / grad_cos may
@@ -315,7 +342,7 @@ int slayer_rf_bwd(float *g_re_in, float *g_im_in, float *grad_sin, float *grad_c
                   const float *grad_spikes, const float *re, const float *im,
                   const float *sin_decay, const float *cos_decay,
                   float spike_threshold, float tau_rho, float scale_rho, int graded, float *workspace,
-                  int64_t M, int64_t neurons_per_batch, int64_t num_decays, int64_t T, void *stream);
+                  int64_t M, int64_t neurons_per_batch, int64_t num_decays, int64_t T, const slayer_delays *delays, void *stream);
 
 /* ---- fused adaptive-threshold LIF neuron ---------------------------------------------------- */
 
@@ -338,7 +365,7 @@ int slayer_alif_fwd(float *cur_out, float *vol_out, float *theta_out, float *spk
                     int64_t M, int64_t neurons_per_batch,
                     int64_t num_i_decays, int64_t num_v_decays, int64_t num_th_decays, int64_t num_ref_decays,
                     int64_t num_i_states, int64_t num_v_states, int64_t num_th_states, int64_t num_ref_states,
-                    int64_t T, void *stream);
+                    int64_t T, const slayer_delays *delays, void *stream);
 
 /* Backward of the above = slayer_spike_bwd with a threshold tensor -> slayer_li_bwd twice, in one launch
  * (20 instead of 40 bytes per neuron-timestep); grad_in is bit-identical to the chain.  grad_i_decay /
@@ -349,7 +376,7 @@ int slayer_alif_bwd(float *grad_in, float *grad_i_decay, float *grad_v_decay,
                     const float *i_decay, const float *v_decay,
                     float tau_rho, float scale_rho, int graded, float *workspace,
                     int64_t M, int64_t neurons_per_batch, int64_t num_i_decays, int64_t num_v_decays,
-                    int64_t T, void *stream);
+                    int64_t T, const slayer_delays *delays, void *stream);
 
 /* ---- recurrent CUBA layer --------------------------------------------------------------------- */
 

@@ -20,11 +20,13 @@ int launch_zero_fill(float* p, int64_t n, hipStream_t stream);          // li.hi
 // refractory state leave the sequential loop as integers in four tiles and become current, voltage,
 // threshold + refractory and spikes on the way out (the tile of the refractory state carries the spikes
 // to memory).
-template <bool POW2, bool GRADED, bool KEEP_CURRENT>
+// SHIFT: the input is read through an axonal delay and the spikes are stored through one (see Shifts).
+template <bool POW2, bool GRADED, bool KEEP_CURRENT, bool SHIFT = false>
 struct AlifFwd {
     static constexpr int kIn = 1, kOut = KEEP_CURRENT ? 4 : 3;   // out: [current,] voltage, threshold + refractory, spikes
     static constexpr int kVol = kOut - 3, kTheta = kOut - 2, kSpk = kOut - 1;
-    static constexpr int kCopyWaves = 2;
+    static constexpr unsigned kShiftIn = SHIFT ? 1u : 0u, kShiftOut = SHIFT ? (1u << kSpk) : 0u;
+    static constexpr int kCopyWaves = SHIFT ? 4 : 2;     // the shifted copies cost the copy waves more instructions
     static constexpr bool kReverse = false;
     static constexpr bool kTransforms = true;
     static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
@@ -36,6 +38,7 @@ struct AlifFwd {
         int step, base;
         float w, inv_w, spike_scale;
         int64_t npb, n_id, n_vd, n_td, n_rd, n_is, n_vs, n_ts, n_rs;
+        Shifts shifts;
     };
     int yc, yv, th, r, th_out, r_out, mi, mv, mt, mr, th_step, base;
     float w, inv_w, spike_scale;
@@ -95,14 +98,22 @@ struct AlifFwd {
         }
         if (valid && p.cur_last) p.cur_last[m] = from_state<POW2>(__int_as_float(yc), w, inv_w);
         if (valid && p.vol_last) p.vol_last[m] = from_state<POW2>(__int_as_float(yv), w, inv_w);
+        if (SHIFT && valid && p.shifts.last) {
+            const float thf = from_state<POW2>(__int_as_float(th_out), w, inv_w);
+            const float rf = from_state<POW2>(__int_as_float(r_out), w, inv_w);
+            p.shifts.last[m] = spike(from_state<POW2>(__int_as_float(yv), w, inv_w), thf + rf);
+        }
     }
 };
 
 // DECAY_GRAD = false drops the saved current and both decay-gradient sums (16 instead of 20 bytes).
-template <bool GRADED, bool DECAY_GRAD>
+// SHIFT: the gradient of the spikes is read back through the output delay, the gradient of the input is stored
+// back through the input shift.
+template <bool GRADED, bool DECAY_GRAD, bool SHIFT = false>
 struct AlifBwd {
     static constexpr int kIn = DECAY_GRAD ? 4 : 3, kOut = 1;   // in: grad of spikes, voltage, threshold + refractory[, current]
     static constexpr bool kReverse = true;
+    static constexpr unsigned kShiftIn = SHIFT ? 1u : 0u, kShiftOut = SHIFT ? 1u : 0u;
     static constexpr int64_t kRows32Below = 4096, kRows16Below = 4096;     // exp per step: keep all lanes busy
     struct Params {
         const float* in[kIn];
@@ -111,6 +122,7 @@ struct AlifBwd {
         float *partial_i, *partial_v;                // per-neuron decay gradients, or nullptr
         float tau, rho;
         int64_t npb, n_id, n_vd;
+        Shifts shifts;
     };
     float ai, av, gc, gx, acc_i, acc_v, tau, rho, lead;
 
@@ -126,7 +138,7 @@ struct AlifBwd {
     // The surrogate does not depend on the recurrence, so it is evaluated on the way into LDS (by all
     // 64 lanes, or by the copy waves of the multi-wave kernel) and takes the place of the incoming gradient.
     static constexpr bool kTransforms = true;
-    static constexpr int kCopyWaves = 4;
+    static constexpr int kCopyWaves = SHIFT ? 8 : 4;
     __device__ __forceinline__ float surrogate(float g, float v, float theta) const {
         const float d = v - theta;
         return GRADED ? (rho * expf(fminf(d, 0.0f) / tau)) * g : (lead * expf(-fabsf(d) / tau)) * g;
@@ -164,8 +176,9 @@ extern "C" int slayer_alif_fwd(float* cur_out, float* vol_out, float* theta_out,
                                int64_t M, int64_t neurons_per_batch,
                                int64_t num_i_decays, int64_t num_v_decays, int64_t num_th_decays, int64_t num_ref_decays,
                                int64_t num_i_states, int64_t num_v_states, int64_t num_th_states, int64_t num_ref_states,
-                               int64_t T, void* stream) {
+                               int64_t T, const slayer_delays* delays, void* stream) {
     if (int e = check_rows(M, T)) return e;
+    if (int e = check_delays(delays, M, neurons_per_batch)) return e;
     if (M == 0 || T == 0) return 0;
     if (!spk_out || !in || !i_decay || !v_decay || !th_decay || !ref_decay ||
         !i_state || !v_state || !th_state || !ref_state)
@@ -184,20 +197,27 @@ extern "C" int slayer_alif_fwd(float* cur_out, float* vol_out, float* theta_out,
 #define SLAYER_ALIF_ARGS cur_last_out, vol_last_out, th_last_out, ref_last_out, i_decay, v_decay, th_decay, ref_decay, i_state,       \
                          v_state, th_state, ref_state, (int)th_step_scaled, (int)th0_scaled, w, 1.0f / w,         \
                          spike_scale, neurons_per_batch, num_i_decays, num_v_decays, num_th_decays,               \
-                         num_ref_decays, num_i_states, num_v_states, num_th_states, num_ref_states
-#define SLAYER_ALIF(P, G)                                                                                         \
+                         num_ref_decays, num_i_states, num_v_states, num_th_states, num_ref_states, sh
+    const Shifts sh = forward_shifts(delays, neurons_per_batch);
+#define SLAYER_ALIF_S(P, G, S)                                                                                    \
     do {                                                                                                          \
         if (cur_out) {                                                                                            \
-            AlifFwd<P, G, true>::Params p{{in}, {cur_out, vol_out, theta_out, spk_out}, SLAYER_ALIF_ARGS};          \
-            return launch_stream<AlifFwd<P, G, true>>(p, M, T, st);                                               \
+            AlifFwd<P, G, true, S>::Params p{{in}, {cur_out, vol_out, theta_out, spk_out}, SLAYER_ALIF_ARGS};     \
+            return launch_stream<AlifFwd<P, G, true, S>>(p, M, T, st);                                            \
         }                                                                                                         \
-        AlifFwd<P, G, false>::Params p{{in}, {vol_out, theta_out, spk_out}, SLAYER_ALIF_ARGS};                      \
-        return launch_stream<AlifFwd<P, G, false>>(p, M, T, st);                                                  \
+        AlifFwd<P, G, false, S>::Params p{{in}, {vol_out, theta_out, spk_out}, SLAYER_ALIF_ARGS};                 \
+        return launch_stream<AlifFwd<P, G, false, S>>(p, M, T, st);                                               \
+    } while (0)
+#define SLAYER_ALIF(P, G)                                                                                         \
+    do {                                                                                                          \
+        if (delays) SLAYER_ALIF_S(P, G, true);                                                                    \
+        SLAYER_ALIF_S(P, G, false);                                                                               \
     } while (0)
     if (is_pow2(w_scale)) { if (graded) SLAYER_ALIF(true, true); else SLAYER_ALIF(true, false); }
     if (graded) SLAYER_ALIF(false, true);
     SLAYER_ALIF(false, false);
 #undef SLAYER_ALIF
+#undef SLAYER_ALIF_S
 #undef SLAYER_ALIF_ARGS
 }
 
@@ -206,8 +226,9 @@ extern "C" int slayer_alif_bwd(float* grad_in, float* grad_i_decay, float* grad_
                                const float* i_decay, const float* v_decay,
                                float tau_rho, float scale_rho, int graded, float* workspace,
                                int64_t M, int64_t neurons_per_batch, int64_t num_i_decays, int64_t num_v_decays,
-                               int64_t T, void* stream) {
+                               int64_t T, const slayer_delays* delays, void* stream) {
     if (int e = check_rows(M, T)) return e;
+    if (int e = check_delays(delays, M, neurons_per_batch)) return e;
     const int64_t mm = M > 0 ? M : neurons_per_batch;
     if (int e = check_params(mm, neurons_per_batch, num_i_decays)) return e;
     if (int e = check_params(mm, neurons_per_batch, num_v_decays)) return e;
@@ -218,22 +239,28 @@ extern "C" int slayer_alif_bwd(float* grad_in, float* grad_i_decay, float* grad_
     if (M > 0 && T > 0) {
         if (!grad_in || !grad_spikes || !voltage || !theta || !i_decay || !v_decay || (want && !current))
             return SLAYER_ENULL;
-#define SLAYER_ALIF_BWD(G)                                                                                        \
+        const Shifts sh = backward_shifts(delays, neurons_per_batch);
+#define SLAYER_ALIF_BWD_S(G, S)                                                                                   \
     do {                                                                                                          \
         if (want) {                                                                                               \
-            AlifBwd<G, true>::Params p{{grad_spikes, voltage, theta, current}, {grad_in}, i_decay, v_decay,         \
-                                       workspace, workspace + M, tau_rho, scale_rho, neurons_per_batch,           \
-                                       num_i_decays, num_v_decays};                                               \
-            if (int e = launch_stream<AlifBwd<G, true>>(p, M, T, st)) return e;                                   \
+            AlifBwd<G, true, S>::Params p{{grad_spikes, voltage, theta, current}, {grad_in}, i_decay, v_decay,    \
+                                          workspace, workspace + M, tau_rho, scale_rho, neurons_per_batch,        \
+                                          num_i_decays, num_v_decays, sh};                                        \
+            if (int e = launch_stream<AlifBwd<G, true, S>>(p, M, T, st)) return e;                                \
         } else {                                                                                                  \
-            AlifBwd<G, false>::Params p{{grad_spikes, voltage, theta}, {grad_in}, i_decay, v_decay, nullptr,        \
-                                        nullptr, tau_rho, scale_rho, neurons_per_batch, num_i_decays,             \
-                                        num_v_decays};                                                            \
-            if (int e = launch_stream<AlifBwd<G, false>>(p, M, T, st)) return e;                                  \
+            AlifBwd<G, false, S>::Params p{{grad_spikes, voltage, theta}, {grad_in}, i_decay, v_decay, nullptr,   \
+                                           nullptr, tau_rho, scale_rho, neurons_per_batch, num_i_decays,          \
+                                           num_v_decays, sh};                                                     \
+            if (int e = launch_stream<AlifBwd<G, false, S>>(p, M, T, st)) return e;                               \
         }                                                                                                         \
+    } while (0)
+#define SLAYER_ALIF_BWD(G)                                                                                        \
+    do {                                                                                                          \
+        if (delays) SLAYER_ALIF_BWD_S(G, true); else SLAYER_ALIF_BWD_S(G, false);                                 \
     } while (0)
         if (graded) SLAYER_ALIF_BWD(true); else SLAYER_ALIF_BWD(false);
 #undef SLAYER_ALIF_BWD
+#undef SLAYER_ALIF_BWD_S
     }
     if (want) {
         if (M == 0 || T == 0) {

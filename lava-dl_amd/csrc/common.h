@@ -27,4 +27,14 @@ inline int check_states(int64_t M, int64_t n) { return (n == 1 || n == M) ? 0 : 
 
 inline bool is_pow2(int w) { return w > 0 && (w & (w - 1)) == 0; }
 
+// Delays folded into a fused block: per-neuron tables need a batch to map onto and a sampling time to
+// divide by; the scalar parts must fit the 32-bit step counts of the kernels (a shift of T steps already
+// empties a row, so anything beyond +-2^30 is equivalent to it).
+inline int check_delays(const slayer_delays* d, int64_t M, int64_t npb) {
+    if (!d) return 0;
+    if (npb <= 0 || (M > 0 && M % npb != 0)) return SLAYER_EINVAL;
+    if ((d->in_shift || d->out_delay) && !(d->sampling_time != 0.0f)) return SLAYER_EINVAL;
+    return 0;
+}
+
 }  // namespace slayer

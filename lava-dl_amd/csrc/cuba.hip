@@ -15,11 +15,13 @@ int launch_zero_fill(float* p, int64_t n, hipStream_t stream);          // li.hi
 
 // KEEP_CURRENT = false leaves the current trace out (a caller that wants no decay gradient does not
 // need it): 12 instead of 16 bytes per neuron-timestep.
-template <bool POW2, bool GRADED, bool KEEP_CURRENT>
+// SHIFT: the input is read through an axonal delay and the spikes are stored through one (see Shifts).
+template <bool POW2, bool GRADED, bool KEEP_CURRENT, bool SHIFT = false>
 struct CubaFwd {
     static constexpr int kIn = 1, kOut = KEEP_CURRENT ? 2 : 1;     // out: [current,] voltage
     static constexpr int kVol = kOut - 1;
     static constexpr int kDerived = 1;               // spikes: a function of the voltage alone
+    static constexpr unsigned kShiftIn = SHIFT ? 1u : 0u, kShiftOut = SHIFT ? (1u << kOut) : 0u;
     static constexpr bool kReverse = false;
     static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
     struct Params {
@@ -30,9 +32,10 @@ struct CubaFwd {
         float w, inv_w, spike_thr, spike_scale;
         int fire_above;                              // voltage reset when the state exceeds this
         int64_t npb, n_id, n_vd, n_is, n_vs;
+        Shifts shifts;
     };
     static constexpr bool kTransforms = true;        // integer tiles, see to_state / from_state
-    static constexpr int kCopyWaves = 2;
+    static constexpr int kCopyWaves = SHIFT ? 4 : 2;     // the shifted copies cost the copy waves more instructions
     int yc, yv, yv_out, mi, mv, fire_above;
     float w, inv_w, spike_thr, spike_scale;
 
@@ -73,15 +76,19 @@ struct CubaFwd {
     __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
         if (valid && p.cur_last) p.cur_last[m] = from_state<POW2>(__int_as_float(yc), w, inv_w);
         if (valid && p.vol_last) p.vol_last[m] = from_state<POW2>(__int_as_float(yv_out), w, inv_w);
+        if (SHIFT && valid && p.shifts.last) p.shifts.last[m] = spike(from_state<POW2>(__int_as_float(yv_out), w, inv_w));
     }
 };
 
 // DECAY_GRAD = false drops the saved current and both decay-gradient sums: 12 instead of 16 bytes
 // per neuron-timestep.
-template <bool GRADED, bool DECAY_GRAD>
+// SHIFT: the gradient of the spikes is read back through the output delay and the gradient of the input is
+// stored back through the input shift (the forward pass's Shifts with the sides swapped and the signs flipped).
+template <bool GRADED, bool DECAY_GRAD, bool SHIFT = false>
 struct CubaBwd {
     static constexpr int kIn = DECAY_GRAD ? 3 : 2, kOut = 1;   // in: grad of spikes, saved voltage[, saved current]
     static constexpr bool kReverse = true;
+    static constexpr unsigned kShiftIn = SHIFT ? 1u : 0u, kShiftOut = SHIFT ? 1u : 0u;
     static constexpr int64_t kRows32Below = 4096, kRows16Below = 4096;     // exp per step: keep all lanes busy
     struct Params {
         const float* in[kIn];
@@ -90,6 +97,7 @@ struct CubaBwd {
         float *partial_i, *partial_v;                // per-neuron decay gradients (DECAY_GRAD only)
         float spike_thr, tau, rho;
         int64_t npb, n_id, n_vd;
+        Shifts shifts;
     };
     float ai, av, gc, gx, acc_i, acc_v, spike_thr, tau, rho, lead;
 
@@ -105,7 +113,7 @@ struct CubaBwd {
     // The surrogate does not depend on the recurrence, so it is evaluated on the way into LDS (by all
     // 64 lanes, or by the copy waves of the multi-wave kernel) and takes the place of the incoming gradient.
     static constexpr bool kTransforms = true;
-    static constexpr int kCopyWaves = 4;
+    static constexpr int kCopyWaves = 8;
     __device__ __forceinline__ float surrogate(float g, float v) const {
         const float d = v - spike_thr;
         return GRADED ? (rho * expf(fminf(d, 0.0f) / tau)) * g : (lead * expf(-fabsf(d) / tau)) * g;
@@ -140,8 +148,10 @@ extern "C" int slayer_cuba_fwd(float* cur_out, float* vol_out, float* spk_out, f
                                const float* i_state, const float* v_state,
                                double thr_scaled, float spike_threshold, int graded, float spike_scale, int w_scale,
                                int64_t M, int64_t neurons_per_batch, int64_t num_i_decays, int64_t num_v_decays,
-                               int64_t num_i_states, int64_t num_v_states, int64_t T, void* stream) {
+                               int64_t num_i_states, int64_t num_v_states, int64_t T,
+                               const slayer_delays* delays, void* stream) {
     if (int e = check_rows(M, T)) return e;
+    if (int e = check_delays(delays, M, neurons_per_batch)) return e;
     if (M == 0 || T == 0) return 0;
     if (!spk_out || !in || !i_decay || !v_decay || !i_state || !v_state) return SLAYER_ENULL;
     if (int e = check_params(M, neurons_per_batch, num_i_decays)) return e;
@@ -152,26 +162,32 @@ extern "C" int slayer_cuba_fwd(float* cur_out, float* vol_out, float* spk_out, f
     const float w = (float)w_scale;
     const int fa = fire_above(thr_scaled > 0 ? (float)thr_scaled : __builtin_inff());
     hipStream_t st = (hipStream_t)stream;
-#define SLAYER_CUBA(P, G)                                                                                        \
+    const Shifts sh = forward_shifts(delays, neurons_per_batch);
+#define SLAYER_CUBA_S(P, G, S)                                                                                   \
     do {                                                                                                         \
         if (cur_out) {                                                                                           \
-            CubaFwd<P, G, true>::Params p{{in}, {cur_out, vol_out, spk_out}, cur_last_out, vol_last_out, i_decay,    \
-                                          v_decay, i_state, v_state, w, 1.0f / w, spike_threshold, spike_scale,  \
-                                          fa,                                                                    \
-                                          neurons_per_batch, num_i_decays, num_v_decays, num_i_states,           \
-                                          num_v_states};                                                         \
-            return launch_stream<CubaFwd<P, G, true>>(p, M, T, st);                                              \
+            CubaFwd<P, G, true, S>::Params p{{in}, {cur_out, vol_out, spk_out}, cur_last_out, vol_last_out,      \
+                                             i_decay, v_decay, i_state, v_state, w, 1.0f / w, spike_threshold,   \
+                                             spike_scale, fa, neurons_per_batch, num_i_decays, num_v_decays,     \
+                                             num_i_states, num_v_states, sh};                                    \
+            return launch_stream<CubaFwd<P, G, true, S>>(p, M, T, st);                                           \
         }                                                                                                        \
-        CubaFwd<P, G, false>::Params p{{in}, {vol_out, spk_out}, cur_last_out, vol_last_out, i_decay, v_decay,    \
-                                       i_state, v_state, w, 1.0f / w, spike_threshold, spike_scale, fa,          \
-                                       neurons_per_batch, num_i_decays, num_v_decays, num_i_states,              \
-                                       num_v_states};                                                            \
-        return launch_stream<CubaFwd<P, G, false>>(p, M, T, st);                                                 \
+        CubaFwd<P, G, false, S>::Params p{{in}, {vol_out, spk_out}, cur_last_out, vol_last_out, i_decay,         \
+                                          v_decay, i_state, v_state, w, 1.0f / w, spike_threshold, spike_scale,  \
+                                          fa, neurons_per_batch, num_i_decays, num_v_decays, num_i_states,       \
+                                          num_v_states, sh};                                                     \
+        return launch_stream<CubaFwd<P, G, false, S>>(p, M, T, st);                                              \
+    } while (0)
+#define SLAYER_CUBA(P, G)                                                                                        \
+    do {                                                                                                         \
+        if (delays) SLAYER_CUBA_S(P, G, true);                                                                   \
+        SLAYER_CUBA_S(P, G, false);                                                                              \
     } while (0)
     if (is_pow2(w_scale)) { if (graded) SLAYER_CUBA(true, true); else SLAYER_CUBA(true, false); }
     if (graded) SLAYER_CUBA(false, true);
     SLAYER_CUBA(false, false);
 #undef SLAYER_CUBA
+#undef SLAYER_CUBA_S
 }
 
 extern "C" int slayer_cuba_bwd(float* grad_in, float* grad_i_decay, float* grad_v_decay,
@@ -179,8 +195,9 @@ extern "C" int slayer_cuba_bwd(float* grad_in, float* grad_i_decay, float* grad_
                                const float* i_decay, const float* v_decay,
                                float spike_threshold, float tau_rho, float scale_rho, int graded, float* workspace,
                                int64_t M, int64_t neurons_per_batch, int64_t num_i_decays, int64_t num_v_decays,
-                               int64_t T, void* stream) {
+                               int64_t T, const slayer_delays* delays, void* stream) {
     if (int e = check_rows(M, T)) return e;
+    if (int e = check_delays(delays, M, neurons_per_batch)) return e;
     const int64_t mm = M > 0 ? M : neurons_per_batch;
     if (int e = check_params(mm, neurons_per_batch, num_i_decays)) return e;
     if (int e = check_params(mm, neurons_per_batch, num_v_decays)) return e;
@@ -190,22 +207,28 @@ extern "C" int slayer_cuba_bwd(float* grad_in, float* grad_i_decay, float* grad_
     hipStream_t st = (hipStream_t)stream;
     if (M > 0 && T > 0) {
         if (!grad_in || !grad_spikes || !voltage || !i_decay || !v_decay || (want && !current)) return SLAYER_ENULL;
-#define SLAYER_CUBA_BWD(G)                                                                                       \
+        const Shifts sh = backward_shifts(delays, neurons_per_batch);
+#define SLAYER_CUBA_BWD_S(G, S)                                                                                  \
     do {                                                                                                         \
         if (want) {                                                                                              \
-            CubaBwd<G, true>::Params p{{grad_spikes, voltage, current}, {grad_in}, i_decay, v_decay, workspace,   \
-                                       workspace + M, spike_threshold, tau_rho, scale_rho, neurons_per_batch,    \
-                                       num_i_decays, num_v_decays};                                              \
-            if (int e = launch_stream<CubaBwd<G, true>>(p, M, T, st)) return e;                                  \
+            CubaBwd<G, true, S>::Params p{{grad_spikes, voltage, current}, {grad_in}, i_decay, v_decay,          \
+                                          workspace, workspace + M, spike_threshold, tau_rho, scale_rho,         \
+                                          neurons_per_batch, num_i_decays, num_v_decays, sh};                    \
+            if (int e = launch_stream<CubaBwd<G, true, S>>(p, M, T, st)) return e;                               \
         } else {                                                                                                 \
-            CubaBwd<G, false>::Params p{{grad_spikes, voltage}, {grad_in}, i_decay, v_decay, nullptr, nullptr,    \
-                                        spike_threshold, tau_rho, scale_rho, neurons_per_batch, num_i_decays,    \
-                                        num_v_decays};                                                           \
-            if (int e = launch_stream<CubaBwd<G, false>>(p, M, T, st)) return e;                                 \
+            CubaBwd<G, false, S>::Params p{{grad_spikes, voltage}, {grad_in}, i_decay, v_decay, nullptr,         \
+                                           nullptr, spike_threshold, tau_rho, scale_rho, neurons_per_batch,      \
+                                           num_i_decays, num_v_decays, sh};                                      \
+            if (int e = launch_stream<CubaBwd<G, false, S>>(p, M, T, st)) return e;                              \
         }                                                                                                        \
+    } while (0)
+#define SLAYER_CUBA_BWD(G)                                                                                       \
+    do {                                                                                                         \
+        if (delays) SLAYER_CUBA_BWD_S(G, true); else SLAYER_CUBA_BWD_S(G, false);                                \
     } while (0)
         if (graded) SLAYER_CUBA_BWD(true); else SLAYER_CUBA_BWD(false);
 #undef SLAYER_CUBA_BWD
+#undef SLAYER_CUBA_BWD_S
     }
     if (want) {
         if (M == 0 || T == 0) {

@@ -16,12 +16,14 @@ int launch_zero_fill(float* p, int64_t n, hipStream_t stream);          // li.hi
 // loop as integers together with the spike decision (taken on the integers: real part above the largest
 // state whose output value is still below the threshold, previous imaginary state negative, new one not),
 // and become output values and spikes on the way out.
-template <bool POW2, bool GRADED>
+// SHIFT: both inputs are read through an axonal delay and the spikes are stored through one (see Shifts).
+template <bool POW2, bool GRADED, bool SHIFT = false>
 struct RfFwd {
     static constexpr int kIn = 2, kOut = 3;          // out: real, imag, spikes
     static constexpr bool kReverse = false;
+    static constexpr unsigned kShiftIn = SHIFT ? 3u : 0u, kShiftOut = SHIFT ? 4u : 0u;
     static constexpr bool kTransforms = true;
-    static constexpr int kCopyWaves = 2;
+    static constexpr int kCopyWaves = SHIFT ? 4 : 2;     // the shifted copies cost the copy waves more instructions
     static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
     struct Params {
         const float* in[2];
@@ -31,13 +33,14 @@ struct RfFwd {
         float w, inv_w, spike_scale;
         int fire_above;                             // a real state above this is at or over the spike threshold
         int64_t npb, nd, n_rs, n_is, n_last;
+        Shifts shifts;
     };
-    int re, im, im_prev, s, c, fire_above;
+    int re, im, im_prev, s, c, fire_above, fired_last;
     float w, inv_w, spike_scale;
 
     __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
         w = p.w; inv_w = p.inv_w; spike_scale = p.spike_scale; fire_above = p.fire_above;
-        re = im = im_prev = s = c = 0;
+        re = im = im_prev = s = c = fired_last = 0;
         if (valid) {
             re = trunc_i32(p.re_state[p.n_rs == 1 ? 0 : m] * w);
             im = trunc_i32(p.im_state[p.n_is == 1 ? 0 : m] * w);
@@ -56,6 +59,7 @@ struct RfFwd {
         const int im_n = rs0_12(s, re) + rs0_12(c, im) + __float_as_int(x[1]);
         const bool fired = (re_n > fire_above) & (im_prev < 0) & (im_n >= 0);
         re = re_n; im = im_n; im_prev = im_n;
+        if (SHIFT) fired_last = fired ? 1 : 0;
         o[0] = __int_as_float(re_n);
         o[1] = __int_as_float(im_n);
         o[2] = __int_as_float(fired ? 1 : 0);
@@ -77,6 +81,8 @@ struct RfFwd {
             p.re_last[m] = from_state<POW2>(__int_as_float(re), w, inv_w);
             p.im_last[m] = from_state<POW2>(__int_as_float(im), w, inv_w);
         }
+        if (SHIFT && valid && p.shifts.last)
+            p.shifts.last[m] = spike(from_state<POW2>(__int_as_float(re), w, inv_w), __int_as_float(fired_last));
     }
 };
 
@@ -84,13 +90,16 @@ struct RfFwd {
 // the copy waves of the multi-wave kernel) and the sequential wave keeps only the rotation: without decay
 // gradients its two results take the places of real and imag; with them real and imag are still needed for
 // the partial sums, so a fourth input slot without a tensor behind it receives the second result.
-template <bool GRADED, bool DECAY_GRAD, bool STAGED>
+// SHIFT: the gradient of the spikes is read back through the output delay, both input gradients are stored
+// back through the input shift.
+template <bool GRADED, bool DECAY_GRAD, bool STAGED, bool SHIFT = false>
 struct RfBwd {
     static_assert(DECAY_GRAD || STAGED, "without decay gradients the surrogate is always staged");
+    static constexpr unsigned kShiftIn = SHIFT ? 1u : 0u, kShiftOut = SHIFT ? 3u : 0u;
     static constexpr int kIn = (DECAY_GRAD && STAGED) ? 4 : 3;     // grad of spikes, saved real, saved imag[, free slot]
     static constexpr int kOut = 2;
     static constexpr bool kTransforms = STAGED;
-    static constexpr int kCopyWaves = STAGED ? 4 : 1;
+    static constexpr int kCopyWaves = STAGED ? (SHIFT ? 8 : 4) : 1;
     static constexpr bool kReverse = true;
     static constexpr int64_t kRows32Below = 4096, kRows16Below = 4096;     // exp per step: keep all lanes busy
     struct Params {
@@ -100,6 +109,7 @@ struct RfBwd {
         float *partial_sin, *partial_cos;
         float spike_thr, tau, rho;
         int64_t npb, nd;
+        Shifts shifts;
     };
     float c, s, gr, gi, acc_s, acc_c, thr, tau, rho, half_over_tau, two_tau, neg_rho_over_tau;
 
@@ -173,8 +183,9 @@ extern "C" int slayer_rf_fwd(float* re_out, float* im_out, float* spk_out, float
                              float spike_threshold, int graded, float spike_scale, int w_scale,
                              int64_t M, int64_t neurons_per_batch, int64_t num_decays,
                              int64_t num_re_states, int64_t num_im_states, int64_t num_last,
-                             int64_t T, void* stream) {
+                             int64_t T, const slayer_delays* delays, void* stream) {
     if (int e = check_rows(M, T)) return e;
+    if (int e = check_delays(delays, M, neurons_per_batch)) return e;
     if (M == 0 || T == 0) return 0;
     if (!spk_out || !re_in || !im_in || !sin_decay || !cos_decay || !re_state || !im_state || !imag_last)
         return SLAYER_ENULL;
@@ -187,26 +198,34 @@ extern "C" int slayer_rf_fwd(float* re_out, float* im_out, float* spk_out, float
     const float w = (float)w_scale;
     const int fire = fire_above_scaled(spike_threshold, w, is_pow2(w_scale));
     hipStream_t st = (hipStream_t)stream;
+    const Shifts sh = forward_shifts(delays, neurons_per_batch);
+#define SLAYER_RF_S(P, G, S)                                                                                     \
+    do {                                                                                                         \
+        RfFwd<P, G, S>::Params p{{re_in, im_in}, {re_out, im_out, spk_out}, re_last_out, im_last_out, sin_decay, \
+                                 cos_decay, re_state, im_state, imag_last, w, 1.0f / w, spike_scale, fire,       \
+                                 neurons_per_batch, num_decays, num_re_states, num_im_states, num_last, sh};     \
+        return launch_stream<RfFwd<P, G, S>>(p, M, T, st);                                                       \
+    } while (0)
 #define SLAYER_RF(P, G)                                                                                          \
     do {                                                                                                         \
-        RfFwd<P, G>::Params p{{re_in, im_in}, {re_out, im_out, spk_out}, re_last_out, im_last_out, sin_decay, cos_decay, re_state,   \
-                              im_state, imag_last, w, 1.0f / w, spike_scale, fire, neurons_per_batch,              \
-                              num_decays,                                                                          \
-                              num_re_states, num_im_states, num_last};                                             \
-        return launch_stream<RfFwd<P, G>>(p, M, T, st);                                                            \
+        if (delays) SLAYER_RF_S(P, G, true);                                                                     \
+        SLAYER_RF_S(P, G, false);                                                                                \
     } while (0)
     if (is_pow2(w_scale)) { if (graded) SLAYER_RF(true, true); else SLAYER_RF(true, false); }
     if (graded) SLAYER_RF(false, true);
     SLAYER_RF(false, false);
 #undef SLAYER_RF
+#undef SLAYER_RF_S
 }
 
 extern "C" int slayer_rf_bwd(float* g_re_in, float* g_im_in, float* grad_sin, float* grad_cos,
                              const float* grad_spikes, const float* re, const float* im,
                              const float* sin_decay, const float* cos_decay,
                              float spike_threshold, float tau_rho, float scale_rho, int graded, float* workspace,
-                             int64_t M, int64_t neurons_per_batch, int64_t num_decays, int64_t T, void* stream) {
+                             int64_t M, int64_t neurons_per_batch, int64_t num_decays, int64_t T,
+                             const slayer_delays* delays, void* stream) {
     if (int e = check_rows(M, T)) return e;
+    if (int e = check_delays(delays, M, neurons_per_batch)) return e;
     if (int e = check_params(M > 0 ? M : neurons_per_batch, neurons_per_batch, num_decays)) return e;
     if ((grad_sin == nullptr) != (grad_cos == nullptr)) return SLAYER_ENULL;
     const bool want = grad_sin != nullptr;
@@ -214,16 +233,21 @@ extern "C" int slayer_rf_bwd(float* g_re_in, float* g_im_in, float* grad_sin, fl
     hipStream_t st = (hipStream_t)stream;
     if (M > 0 && T > 0) {
         if (!g_re_in || !g_im_in || !grad_spikes || !re || !im || !sin_decay || !cos_decay) return SLAYER_ENULL;
-#define SLAYER_RF_BWD(G, D, S)                                                                                    \
+        const Shifts sh = backward_shifts(delays, neurons_per_batch);
+#define SLAYER_RF_BWD_H(G, D, S, H)                                                                               \
     do {                                                                                                          \
-        using Op = RfBwd<G, D, S>;                                                                                \
+        using Op = RfBwd<G, D, S, H>;                                                                             \
         Op::Params p{{grad_spikes, re, im}, {g_re_in, g_im_in}, sin_decay, cos_decay,                             \
                      want ? workspace : nullptr, want ? workspace + M : nullptr,                                  \
-                     spike_threshold, tau_rho, scale_rho, neurons_per_batch, num_decays};                         \
+                     spike_threshold, tau_rho, scale_rho, neurons_per_batch, num_decays, sh};                     \
         if (!S || stream_fits_multiwave<Op>(p, M, T)) {                                                           \
             if (int e = launch_stream<Op>(p, M, T, st)) return e;                                                 \
             done = true;                                                                                          \
         }                                                                                                         \
+    } while (0)
+#define SLAYER_RF_BWD(G, D, S)                                                                                    \
+    do {                                                                                                          \
+        if (delays) SLAYER_RF_BWD_H(G, D, S, true); else SLAYER_RF_BWD_H(G, D, S, false);                         \
     } while (0)
         // The staged forms pay off in the multi-wave kernel (three times faster there); the one-wave kernel
         // gains nothing from the split, so large tensors take the unstaged form (partial sums dropped when
@@ -233,6 +257,7 @@ extern "C" int slayer_rf_bwd(float* g_re_in, float* g_im_in, float* grad_sin, fl
         else { if (want) SLAYER_RF_BWD(false, true, true); else SLAYER_RF_BWD(false, false, true); }
         if (!done) { if (graded) SLAYER_RF_BWD(true, true, false); else SLAYER_RF_BWD(false, true, false); }
 #undef SLAYER_RF_BWD
+#undef SLAYER_RF_BWD_H
     }
     if (want) {
         if (M == 0 || T == 0) {

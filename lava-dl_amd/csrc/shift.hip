@@ -72,7 +72,9 @@ __global__ __launch_bounds__(256) void delay_bwd_kernel(float* __restrict__ grad
             if (t + 2 < T) { gv.z = g[t + 2]; yv.z = y[t + 2]; }
             if (t + 3 < T) { gv.w = g[t + 3]; yv.w = y[t + 3]; }
         }
-        if (VEC4 && (k & 3) == 0) {
+        if (!grad_in) {
+            // sums only: the shifted copy of the gradient is not wanted
+        } else if (VEC4 && (k & 3) == 0) {
             if (s >= 0 && s < T) sv = *reinterpret_cast<const float4*>(g + s);
         } else {
             if (s + 0 >= 0 && s + 0 < T) sv.x = g[s + 0];
@@ -88,7 +90,8 @@ __global__ __launch_bounds__(256) void delay_bwd_kernel(float* __restrict__ grad
             acc = __fmaf_rn(gv.z, f0 * yv.z + f1 * yv.y, acc);
             acc = __fmaf_rn(gv.w, f0 * yv.w + f1 * yv.z, acc);
         }
-        if (VEC4) {
+        if (!grad_in) {
+        } else if (VEC4) {
             *reinterpret_cast<float4*>(dst + t) = sv;
         } else {
             if (t + 0 < T) dst[t + 0] = sv.x;
@@ -145,12 +148,12 @@ extern "C" int slayer_delay_bwd(float* grad_in, float* grad_sum, const float* gr
     if (sampling_time == 0.0f) return SLAYER_EINVAL;
     hipStream_t st = (hipStream_t)stream;
     if (M == 0 || T == 0) return grad_sum ? launch_zero_fill(grad_sum, neurons_per_batch, st) : 0;
-    if (!grad_in || !grad_out || !out) return SLAYER_ENULL;
+    if (!grad_out || !out || (!grad_in && !grad_sum)) return SLAYER_ENULL;
     if (grad_sum && !workspace) return SLAYER_ENULL;
     const int64_t kk = scalar_steps > T ? T : (scalar_steps < -T ? -T : scalar_steps);
     const int64_t blocks = (M + 3) / 4;
     if (blocks > 0x7fffffffLL) return SLAYER_ERANGE;
-    const bool vec = (T % 4 == 0) && aligned16(grad_in) && aligned16(grad_out) && aligned16(out);
+    const bool vec = (T % 4 == 0) && aligned16(grad_in) && aligned16(grad_out) && aligned16(out);   // NULL counts as aligned
     const float f0 = -1.0f / sampling_time, f1 = 1.0f / sampling_time;
     float* partial = grad_sum ? workspace : nullptr;
     if (vec)

@@ -17,6 +17,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include "../../include/slayer_hip.h"
 
 namespace slayer {
 
@@ -153,6 +154,61 @@ struct DerivedCount { static constexpr int value = 0; };
 template <class Op>
 struct DerivedCount<Op, decltype((void)Op::kDerived)> { static constexpr int value = Op::kDerived; };
 
+// Time shifts folded into the copies (an axonal delay on either side of a neuron costs no pass of its own).
+//   static constexpr unsigned kShiftIn  = bit mask over in[]:  input i is read shifted, the recurrence sees
+//                                         x[t] = in[i][t - kin] (zero where t - kin falls outside [0, T));
+//   static constexpr unsigned kShiftOut = bit mask over out[] (bit kOut = the derived output): output o is
+//                                         stored shifted, out[o][t + kout] = y[t]; samples that leave [0, T)
+//                                         are dropped and the positions no sample reaches are filled with
+//                                         zeros (the one just before the first sample with head[m], if given).
+// An Op that sets either carries `Shifts shifts;` in its Params.  kin and kout are per row:
+// steps + trunc(lut[m % npb] / ts), any sign.  Shifted tensors still move 16 bytes per lane and instruction,
+// at dword-aligned addresses (a row's shift need not be a multiple of 4 and differs from row to row); only the
+// quads that straddle an end of their row take extra work.  Everything else is unchanged.
+struct Shifts {
+    const float* in_lut;     // per-neuron input shift in time units, npb entries, or nullptr
+    const float* out_lut;    // per-neuron output shift, npb entries, or nullptr
+    const float* head;       // [M] value of the sample before step 0 of a shifted output (lands at kout - 1), or nullptr
+    float* last;             // [M] receives the shifted output's sample of step T-1 (written by Op::finish), or nullptr
+    int in_steps, out_steps; // scalar parts, in steps
+    int sign;                // +1, or -1 for a backward pass (undoes the forward pass's shifts)
+    float ts;                // sampling time the lut entries are divided by
+    int64_t npb;
+};
+
+template <class Op, class = void>
+struct ShiftInMask { static constexpr unsigned value = 0; };
+template <class Op>
+struct ShiftInMask<Op, decltype((void)Op::kShiftIn)> { static constexpr unsigned value = Op::kShiftIn; };
+template <class Op, class = void>
+struct ShiftOutMask { static constexpr unsigned value = 0; };
+template <class Op>
+struct ShiftOutMask<Op, decltype((void)Op::kShiftOut)> { static constexpr unsigned value = Op::kShiftOut; };
+
+// steps + trunc(lut / ts) with every term held inside [-(T+1), T+1]: a shift of T steps already empties the
+// row, T+1 stands for everything beyond (the sample before the first, `head`, then falls off the row too)
+__host__ __device__ __forceinline__ int clamp_shift(int64_t k, int T) {
+    const int64_t lim = (int64_t)T + 1;
+    return (int)(k > lim ? lim : (k < -lim ? -lim : k));
+}
+__device__ __forceinline__ int row_shift(const float* lut, int steps, float ts, int64_t m, int64_t npb, int T) {
+    int k = clamp_shift(steps, T);
+    if (lut) {
+        const float q = lut[m % npb] / ts;
+        const float lim = (float)T + 1.0f;
+        const int kl = !(q == q) ? 0 : (q >= lim ? T + 1 : (q <= -lim ? -(T + 1) : (int)q));
+        k = clamp_shift((int64_t)k + kl, T);
+    }
+    return k;
+}
+
+__device__ __forceinline__ int in_shift_of(const Shifts& sh, int64_t m, int T) {
+    return sh.sign * row_shift(sh.in_lut, sh.in_steps, sh.ts, m, sh.npb, T);
+}
+__device__ __forceinline__ int out_shift_of(const Shifts& sh, int64_t m, int T) {
+    return sh.sign * row_shift(sh.out_lut, sh.out_steps, sh.ts, m, sh.npb, T);
+}
+
 // ---------------------------------------------------------------------------------------------
 // Buffer addressing.  Global accesses of the dwordx4 path go through raw buffer instructions whose
 // descriptor covers exactly the rows of this wave: a lane that must not touch memory (column
@@ -176,6 +232,15 @@ __device__ __forceinline__ void buf_store4(__amdgpu_buffer_rsrc_t r, int byte_of
     v4u v;
     v.x = __float_as_uint(f.x); v.y = __float_as_uint(f.y); v.z = __float_as_uint(f.z); v.w = __float_as_uint(f.w);
     __builtin_amdgcn_raw_buffer_store_b128(v, r, byte_off, 0, STREAM ? 2 : 0);
+}
+
+template <bool STREAM>
+__device__ __forceinline__ float buf_load1(__amdgpu_buffer_rsrc_t r, int byte_off) {
+    return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, byte_off, 0, STREAM ? 2 : 0));
+}
+template <bool STREAM>
+__device__ __forceinline__ void buf_store1(__amdgpu_buffer_rsrc_t r, int byte_off, float f) {
+    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(f), r, byte_off, 0, STREAM ? 2 : 0);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -215,6 +280,8 @@ struct Copier {
     static constexpr int TC = G::kChunk, NI = Op::kIn, NO = Op::kOut, ND = DerivedCount<Op>::value;
     static constexpr int kPasses = PASSES;
     static_assert(ND == 0 || ND == 1, "at most one derived output");
+    static constexpr unsigned SI = ShiftInMask<Op>::value, SO = ShiftOutMask<Op>::value;
+    static constexpr bool kShifts = SI != 0 || SO != 0;
     using Tiles = float (*)[G::kTileFloats];
 
     __amdgpu_buffer_rsrc_t src[NI], dst[NO + ND];
@@ -223,6 +290,11 @@ struct Copier {
     float4 keep[NO][kPasses];                // first-produced pieces of shared lines, one quad per pass
     int rows, T, crow, cq, interior_end, first_pass;
     int row_lo, row_hi;                      // rows [row_lo, row_hi) of the tile are copied by this wave
+    int kin[kShifts ? kPasses : 1], kout[kShifts ? kPasses : 1];   // shifts of this lane's row in each pass
+    int kout_row;                            // output shift of row `lane` (lane = row), for fill_unreached
+    // wave-uniform: chunks [in_first, in_last] hold only quads whose shifted source lies wholly inside its row,
+    // chunks [out_first, out_last] only quads whose shifted destination does (for every row of this wave)
+    int in_first, in_last, out_first, out_last;
     bool route;
 
     __device__ __forceinline__ void init(const typename Op::Params& prm, int64_t m0, int rows_, int T_, int lane,
@@ -252,6 +324,64 @@ struct Copier {
 #pragma unroll
             for (int o = 0; o < NO; ++o) keep[o][p] = make_float4(0.f, 0.f, 0.f, 0.f);
         }
+        if constexpr (kShifts) {
+            // lane l works out the shifts of row l once (a table look-up with a 64-bit modulo and a division);
+            // the passes pick theirs up from that lane
+            const auto& sh = prm.shifts;
+            const bool mine = lane >= row_lo && lane < row_hi;
+            const int kin_row = (SI != 0 && mine) ? in_shift_of(sh, m0 + lane, T) : 0;
+            kout_row = (SO != 0 && mine) ? out_shift_of(sh, m0 + lane, T) : 0;
+#pragma unroll
+            for (int p = 0; p < kPasses; ++p) {
+                const int r = (first_pass + p) * G::kRowsPerPass + crow;
+                kin[p] = __shfl(kin_row, r);
+                kout[p] = __shfl(kout_row, r);
+            }
+            int in_max = kin_row > 0 ? kin_row : 0, in_min = kin_row < 0 ? kin_row : 0;
+            int out_max = kout_row > 0 ? kout_row : 0, out_min = kout_row < 0 ? kout_row : 0;
+#pragma unroll
+            for (int d = 1; d < kWave; d <<= 1) {
+                int o;
+                o = __shfl_xor(in_max, d); in_max = o > in_max ? o : in_max;
+                o = __shfl_xor(in_min, d); in_min = o < in_min ? o : in_min;
+                o = __shfl_xor(out_max, d); out_max = o > out_max ? o : out_max;
+                o = __shfl_xor(out_min, d); out_min = o < out_min ? o : out_min;
+            }
+            // chunk c holds steps c*TC - 31 .. (c+1)*TC - 1 over all phases; a quad starts at t, its source at
+            // s = t - kin, its destination at u = t + kout; both must lie in [0, T - 4]
+            in_first = (31 + in_max + TC - 1) / TC;
+            in_last = (T + in_min) / TC - 1;
+            out_first = (31 - out_min + TC - 1) / TC;
+            out_last = (T - out_max) / TC - 1;
+            in_first = __builtin_amdgcn_readfirstlane(in_first); in_last = __builtin_amdgcn_readfirstlane(in_last);
+            out_first = __builtin_amdgcn_readfirstlane(out_first); out_last = __builtin_amdgcn_readfirstlane(out_last);
+        }
+    }
+
+    __device__ __forceinline__ bool whole_in(int chunk) const { return chunk >= in_first && chunk <= in_last; }
+    __device__ __forceinline__ bool whole_out(int chunk) const { return chunk >= out_first && chunk <= out_last; }
+
+    // The positions of a shifted output that no sample reaches: [0, kout) for a delay, [T + kout, T) for an
+    // advance.  Row after row of this wave's rows, 64 positions per instruction.
+    __device__ __forceinline__ void fill_unreached(const typename Op::Params& prm, int64_t m0, int lane) const {
+        if constexpr (SO != 0) {
+            const auto& sh = prm.shifts;
+            for (int r = row_lo; r < row_hi; ++r) {
+                const int k = __builtin_amdgcn_readlane(kout_row, r);
+                const int mag = k < 0 ? -k : k;
+                const int len = mag > T ? T : mag;
+                for (int j0 = 0; j0 < len; j0 += kWave) {
+                    const int j = j0 + lane;
+                    const bool ok = j < len;
+                    const int u = k < 0 ? T - len + j : j;
+                    float v = 0.f;
+                    if (ok && sh.head && k > 0 && j == k - 1) v = sh.head[m0 + r];
+#pragma unroll
+                    for (int o = 0; o < NO + ND; ++o)
+                        if (((SO >> o) & 1u) != 0) buf_store1<STREAM>(dst[o], ok ? (r * T + u) * 4 : kOutOfRange, v);
+                }
+            }
+        }
     }
 
     __device__ __forceinline__ bool interior(int chunk) const { return chunk >= 1 && chunk < interior_end; }
@@ -260,23 +390,67 @@ struct Copier {
     __device__ __forceinline__ void fetch_into(float4 (&buf)[NI][kPasses], int chunk) const {
 #pragma unroll
         for (int p = 0; p < kPasses; ++p) {
-            const bool ok = (unsigned)(step0[p] + chunk * TC) < (unsigned)T;
+            const int t = step0[p] + chunk * TC;
+            const bool ok = (unsigned)t < (unsigned)T;
             const int off = ok ? off0[p] + chunk * (TC * 4) : kOutOfRange;
 #pragma unroll
-            for (int i = 0; i < NI; ++i) buf[i][p] = buf_load4<STREAM>(src[i], off);
+            for (int i = 0; i < NI; ++i) {
+                if (((SI >> i) & 1u) != 0) {
+                    // the quad wanted is samples s .. s+3 of the row, s = t - kin (a multiple of 4 only by chance:
+                    // the load is dword-aligned).  One 16-byte load at the nearest position that lies inside
+                    // the row; to_tiles() moves the samples into place when the two differ.
+                    if (whole_in(chunk)) {
+                        buf[i][p] = buf_load4<STREAM>(src[i], ok ? off0[p] + chunk * (TC * 4) - 4 * kin[p] : kOutOfRange);
+                    } else {
+                        const int s = t - kin[p];
+                        const int sc = s < 0 ? 0 : (s > T - 4 ? T - 4 : s);
+                        const bool some = ok && s > -4 && s < T;
+                        buf[i][p] = buf_load4<STREAM>(src[i], some ? off0[p] + 4 * (sc - step0[p]) : kOutOfRange);
+                    }
+                } else {
+                    buf[i][p] = buf_load4<STREAM>(src[i], off);
+                }
+            }
         }
     }
     __device__ __forceinline__ void fetch(int chunk) { fetch_into(stage, chunk); }
 
     // registers -> LDS
-    __device__ __forceinline__ void stage_to_tiles(const Op& op, Tiles tile) const { to_tiles(op, tile, stage); }
-    __device__ __forceinline__ void to_tiles(const Op& op, Tiles tile, const float4 (&buf)[NI][kPasses]) const {
+    // A shifted input whose quad straddles an end of its row was loaded from the nearest position inside the
+    // row: element e of the quad is element e + d of what was loaded, d = wanted - loaded position, or zero.
+    __device__ __forceinline__ float4 place(float4 q, int d) const {
+        const float a[4] = {q.x, q.y, q.z, q.w};
+        float r[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int j = e + d;
+            r[e] = j == 0 ? a[0] : (j == 1 ? a[1] : (j == 2 ? a[2] : (j == 3 ? a[3] : 0.f)));
+        }
+        return make_float4(r[0], r[1], r[2], r[3]);
+    }
+
+    __device__ __forceinline__ void stage_to_tiles(const Op& op, Tiles tile, int chunk) const {
+        to_tiles(op, tile, stage, chunk);
+    }
+    // `chunk` is the chunk `buf` was fetched for
+    __device__ __forceinline__ void to_tiles(const Op& op, Tiles tile, const float4 (&buf)[NI][kPasses],
+                                             int chunk) const {
 #pragma unroll
         for (int p = 0; p < kPasses; ++p) {
             const int r = (first_pass + p) * G::kRowsPerPass + crow;
             float4 x[NI];
 #pragma unroll
             for (int i = 0; i < NI; ++i) x[i] = buf[i][p];
+            if (SI != 0 && !whole_in(chunk)) {
+                const int s = step0[p] + chunk * TC - kin[p];
+                const int sc = s < 0 ? 0 : (s > T - 4 ? T - 4 : s);
+                const int d = (s > -4 && s < T) ? s - sc : 0;
+                if (__any(d != 0)) {                  // rare: only where a row begins or ends
+#pragma unroll
+                    for (int i = 0; i < NI; ++i)
+                        if (((SI >> i) & 1u) != 0) x[i] = place(x[i], d);
+                }
+            }
             if constexpr (HasTransforms<Op>::value) op.pre(x);
 #pragma unroll
             for (int i = 0; i < NI; ++i) *reinterpret_cast<float4*>(&tile[i][r * G::kPitch + 4 * cq]) = x[i];
@@ -291,8 +465,9 @@ struct Copier {
 #pragma unroll
         for (int p = 0; p < kPasses; ++p)
 #pragma unroll
-            for (int o = 0; o < NO + ND; ++o)   // distinct offsets, or the compiler merges them into one store
+            for (int o = 0; o < NO + ND; ++o) { // distinct offsets, or the compiler merges them into one store
                 buf_store4<STREAM>(dst[o], kOutOfRange + 16 * p, make_float4(0.f, 0.f, 0.f, 0.f));
+            }
     }
 
     // LDS -> global.  On edge chunks the line shared by rows r and r+1 is completed before it is
@@ -309,9 +484,9 @@ struct Copier {
             const int r = (first_pass + p) * G::kRowsPerPass + crow;
             const int t = step0[p] + chunk * TC;
             int off = off0[p] + chunk * (TC * 4);
-            float4 v[NO];
+            float4 v[NO], own[NO];                                  // own: this lane's quad, for shifted outputs
 #pragma unroll
-            for (int o = 0; o < NO; ++o) v[o] = *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]);
+            for (int o = 0; o < NO; ++o) own[o] = v[o] = *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]);
             if (!inner) {
                 const int a = 4 * cq - step0[p];                   // phase of row r
                 const bool valid = (unsigned)t < (unsigned)T;
@@ -354,9 +529,48 @@ struct Copier {
                 }
             }
             if constexpr (HasTransforms<Op>::value) op.post(v);
+            // A shifted output leaves from the lane that computed it (no completed lines: its quads do not fall
+            // on line boundaries anyway), sample t + e to position t + e + kout of the row: one dword-aligned
+            // 16-byte store when the whole quad lands inside the row; a quad that straddles an end of the row
+            // (only in the first or last few chunks) leaves sample by sample.
+            const int ubase = off0[p] + chunk * (TC * 4) + (SO != 0 ? 4 * kout[p] : 0);
+            bool whole = true, part = false, any_part = false;
+            const int u = t + (SO != 0 ? kout[p] : 0);
+            if (SO != 0 && !(inner && whole_out(chunk))) {
+                if (inner) {
 #pragma unroll
-            for (int o = 0; o < NO; ++o) buf_store4<STREAM>(dst[o], off, v[o]);
-            if constexpr (ND == 1) buf_store4<STREAM>(dst[NO], off, op.derive(v));
+                    for (int o = 0; o < NO; ++o) own[o] = v[o];
+                } else {
+                    if constexpr (HasTransforms<Op>::value) op.post(own);
+                }
+                const bool t_ok = (unsigned)t < (unsigned)T;
+                whole = t_ok && u >= 0 && u <= T - 4;
+                part = t_ok && !whole && u > -4 && u < T;
+                any_part = __any(part);
+            } else if (SO != 0) {
+#pragma unroll
+                for (int o = 0; o < NO; ++o) own[o] = v[o];
+            }
+            // never streaming: every one of these stores ends in a partial line that the next chunk completes,
+            // so the line has to wait in the cache
+            auto store_shifted = [&](__amdgpu_buffer_rsrc_t d, float4 q) {
+                buf_store4<false>(d, whole ? ubase : kOutOfRange, q);
+                if (any_part) {
+                    const float e[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        buf_store1<false>(d, (part && (unsigned)(u + j) < (unsigned)T) ? ubase + 4 * j : kOutOfRange, e[j]);
+                }
+            };
+#pragma unroll
+            for (int o = 0; o < NO; ++o) {
+                if (((SO >> o) & 1u) != 0) store_shifted(dst[o], own[o]);
+                else buf_store4<STREAM>(dst[o], off, v[o]);
+            }
+            if constexpr (ND == 1) {
+                if constexpr (((SO >> NO) & 1u) != 0) store_shifted(dst[NO], op.derive(own));
+                else buf_store4<STREAM>(dst[NO], off, op.derive(v));
+            }
         }
     }
 };
@@ -437,11 +651,12 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
     Copier<Op, R, STREAM> io;
     io.init(prm, m0, rows, T, lane, base_f);
     io.fetch(Op::kReverse ? nchunks - 1 : 0);
+    io.fill_unreached(prm, m0, lane);
     io.prime_stores();
 
     for (int k = 0; k < nchunks; ++k) {
         const int chunk = Op::kReverse ? nchunks - 1 - k : k;
-        io.stage_to_tiles(op, tile);
+        io.stage_to_tiles(op, tile, chunk);
         __syncthreads();
         io.fetch(Op::kReverse ? chunk - 1 : chunk + 1);
         run_chunk<Op, R, 4>(op, tile, lane, chunk, io.interior(chunk), a_lane, T);
@@ -502,17 +717,18 @@ __global__ __launch_bounds__((1 + NCOPY) * kWave) void stream_kernel_duo(typenam
         io.fetch_into(fetched[0], chunk_of(0));
         io.fetch_into(fetched[1], chunk_of(1));
         io.prime_stores();
-        io.to_tiles(uni, tiles[0], fetched[0]);
+        io.to_tiles(uni, tiles[0], fetched[0], chunk_of(0));
         io.fetch_into(fetched[0], chunk_of(2));
         __syncthreads();                                       // barrier 0
+        io.fill_unreached(prm, m0, lane);                      // while the sequential wave works on chunk 0
         for (int k = 0; k < nloop; k += 2) {
             // wave 0 works on tiles[0] (chunk k); tiles[1] still holds the results of chunk k-1
             io.copy_out(uni, tiles[1], chunk_of(k - 1));
-            io.to_tiles(uni, tiles[1], fetched[1]);            // chunk k+1
+            io.to_tiles(uni, tiles[1], fetched[1], chunk_of(k + 1));
             io.fetch_into(fetched[1], chunk_of(k + 3));
             __syncthreads();                                   // barrier k+1
             io.copy_out(uni, tiles[0], chunk_of(k));
-            io.to_tiles(uni, tiles[0], fetched[0]);            // chunk k+2
+            io.to_tiles(uni, tiles[0], fetched[0], chunk_of(k + 2));
             io.fetch_into(fetched[0], chunk_of(k + 4));
             __syncthreads();                                   // barrier k+2
         }
@@ -541,6 +757,34 @@ __global__ __launch_bounds__(kWave) void stream_kernel_scalar(typename Op::Param
     const int crow = lane / G::kQuads;
     const int cq = lane % G::kQuads;
 
+    constexpr unsigned SI = ShiftInMask<Op>::value, SO = ShiftOutMask<Op>::value;
+    constexpr bool kShifts = SI != 0 || SO != 0;
+    int kin[kShifts ? G::kPasses : 1], kout[kShifts ? G::kPasses : 1];
+    if constexpr (kShifts) {
+        const auto& sh = prm.shifts;
+#pragma unroll
+        for (int p = 0; p < G::kPasses; ++p) {
+            const int r = p * G::kRowsPerPass + crow;
+            kin[p] = (SI != 0 && r < rows) ? in_shift_of(sh, m0 + r, T) : 0;
+            kout[p] = (SO != 0 && r < rows) ? out_shift_of(sh, m0 + r, T) : 0;
+        }
+        if constexpr (SO != 0) {
+            // positions of a shifted output that no sample reaches (see Copier::fill_unreached)
+            for (int r = 0; r < rows; ++r) {
+                const int kr = out_shift_of(sh, m0 + r, T);
+                const int mag = kr < 0 ? -kr : kr;
+                const int len = mag > T ? T : mag;
+                for (int j = lane; j < len; j += kWave) {
+                    const int64_t pos = (int64_t)(m0 + r) * (int64_t)T + (kr < 0 ? T - len + j : j);
+                    const float v = (sh.head && kr > 0 && j == kr - 1) ? sh.head[m0 + r] : 0.f;
+#pragma unroll
+                    for (int o = 0; o < NO + ND; ++o)
+                        if (((SO >> o) & 1u) != 0 && prm.out[o]) prm.out[o][pos] = v;
+                }
+            }
+        }
+    }
+
     for (int k = 0; k < nchunks; ++k) {
         const int chunk = Op::kReverse ? nchunks - 1 - k : k;
         const int t = chunk * TC + 4 * cq;
@@ -553,11 +797,13 @@ __global__ __launch_bounds__(kWave) void stream_kernel_scalar(typename Op::Param
             for (int i = 0; i < NI; ++i) {
                 float4 v = make_float4(0.f, 0.f, 0.f, 0.f);      // zero fill: steps past T-1 must be no-ops
                 if (r < rows && prm.in[i]) {
-                    const float* src = prm.in[i] + off;
-                    if (t + 0 < T) v.x = src[0];
-                    if (t + 1 < T) v.y = src[1];
-                    if (t + 2 < T) v.z = src[2];
-                    if (t + 3 < T) v.w = src[3];
+                    const int ki = ((SI >> i) & 1u) != 0 ? kin[p] : 0;   // sample t + e - ki, if the row has it
+                    const float* src = prm.in[i] + off - ki;
+                    const int s = t - ki;
+                    if (t + 0 < T && (unsigned)(s + 0) < (unsigned)T) v.x = src[0];
+                    if (t + 1 < T && (unsigned)(s + 1) < (unsigned)T) v.y = src[1];
+                    if (t + 2 < T && (unsigned)(s + 2) < (unsigned)T) v.z = src[2];
+                    if (t + 3 < T && (unsigned)(s + 3) < (unsigned)T) v.w = src[3];
                 }
                 x[i] = v;
             }
@@ -610,17 +856,45 @@ __global__ __launch_bounds__(kWave) void stream_kernel_scalar(typename Op::Param
 #pragma unroll
             for (int o = 0; o < NO + ND; ++o) {
                 if (r < rows && prm.out[o]) {
-                    float* d = prm.out[o] + off;
-                    if (t + 0 < T) d[0] = v[o].x;
-                    if (t + 1 < T) d[1] = v[o].y;
-                    if (t + 2 < T) d[2] = v[o].z;
-                    if (t + 3 < T) d[3] = v[o].w;
+                    const int ko = ((SO >> o) & 1u) != 0 ? kout[p] : 0;  // sample t + e goes to t + e + ko
+                    float* d = prm.out[o] + off + ko;
+                    const int u = t + ko;
+                    if (t + 0 < T && (unsigned)(u + 0) < (unsigned)T) d[0] = v[o].x;
+                    if (t + 1 < T && (unsigned)(u + 1) < (unsigned)T) d[1] = v[o].y;
+                    if (t + 2 < T && (unsigned)(u + 2) < (unsigned)T) d[2] = v[o].z;
+                    if (t + 3 < T && (unsigned)(u + 3) < (unsigned)T) d[3] = v[o].w;
                 }
             }
         }
         __syncthreads();
     }
     op.finish(prm, m0 + lane, lane < rows);
+}
+
+// The Shifts of a forward pass (input read through in_shift, designated output stored through out_delay)
+// and of the matching backward pass: the gradient arriving at the delayed output is read back through the
+// output delay, the gradient of the input is stored back through the input shift.
+inline int steps_to_int(int64_t k) {
+    const int64_t lim = (int64_t)1 << 30;
+    return (int)(k > lim ? lim : (k < -lim ? -lim : k));
+}
+inline Shifts forward_shifts(const slayer_delays* d, int64_t npb) {
+    Shifts s{nullptr, nullptr, nullptr, nullptr, 0, 0, 1, 1.0f, npb > 0 ? npb : 1};
+    if (d) {
+        s.in_lut = d->in_shift; s.out_lut = d->out_delay; s.head = d->out_head; s.last = d->spike_last;
+        s.in_steps = steps_to_int(d->in_steps); s.out_steps = steps_to_int(d->out_steps);
+        if (d->sampling_time != 0.0f) s.ts = d->sampling_time;
+    }
+    return s;
+}
+inline Shifts backward_shifts(const slayer_delays* d, int64_t npb) {
+    Shifts s{nullptr, nullptr, nullptr, nullptr, 0, 0, -1, 1.0f, npb > 0 ? npb : 1};
+    if (d) {
+        s.in_lut = d->out_delay; s.out_lut = d->in_shift;
+        s.in_steps = steps_to_int(d->out_steps); s.out_steps = steps_to_int(d->in_steps);
+        if (d->sampling_time != 0.0f) s.ts = d->sampling_time;
+    }
+    return s;
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

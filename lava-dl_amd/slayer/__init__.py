@@ -1,6 +1,6 @@
 """MI355X-native drop-in for the hot path of lava.lib.dl.slayer: neuron
 dynamics, spike functions, time shift and temporal filter, all backed by
 libslayer_hip.so (hand-written HIP for gfx950)."""
-from . import neuron, spike, utils, axon, dendrite
+from . import neuron, spike, utils, axon, dendrite, block
 
-__all__ = ['neuron', 'spike', 'utils', 'axon', 'dendrite']
+__all__ = ['neuron', 'spike', 'utils', 'axon', 'dendrite', 'block']

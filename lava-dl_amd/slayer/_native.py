@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # SLAYER_HIP_LIB points at an alternative build of the same library (e.g. a tuning build)
 LIB_PATH = os.environ.get('SLAYER_HIP_LIB') or os.path.join(_HERE, 'libslayer_hip.so')
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _lib = None
 _lib_lock = threading.Lock()       # forward runs on the user thread, backward on an autograd thread
@@ -23,6 +23,16 @@ _I64 = ctypes.c_int64
 _INT = ctypes.c_int
 _F = ctypes.c_float
 _D = ctypes.c_double
+
+
+
+class Delays(ctypes.Structure):
+    """struct slayer_delays of include/slayer_hip.h (device pointers as integers)."""
+    _fields_ = [('in_shift', _P), ('out_delay', _P), ('out_head', _P), ('spike_last', _P),
+                ('in_steps', _I64), ('out_steps', _I64), ('sampling_time', _F)]
+
+
+_DP = ctypes.POINTER(Delays)
 
 _SIGNATURES = {
     'slayer_abi_version': (_INT, []),
@@ -49,12 +59,12 @@ _SIGNATURES = {
     'slayer_delta_fwd': (_INT, [_P] * 9 + [_INT, _F] + [_I64] * 7 + [_P]),
     'slayer_delta_bwd': (_INT, [_P] * 6 + [_F, _F] + [_I64] * 4 + [_P]),
     'slayer_cumsum': (_INT, [_P, _P, _P, _I64, _INT, _I64, _I64, _P]),
-    'slayer_cuba_fwd': (_INT, [_P] * 10 + [_D, _F, _INT, _F, _INT] + [_I64] * 7 + [_P]),
-    'slayer_cuba_bwd': (_INT, [_P] * 8 + [_F, _F, _F, _INT, _P] + [_I64] * 5 + [_P]),
-    'slayer_rf_fwd': (_INT, [_P] * 12 + [_F, _INT, _F, _INT] + [_I64] * 7 + [_P]),
-    'slayer_rf_bwd': (_INT, [_P] * 9 + [_F, _F, _F, _INT, _P] + [_I64] * 4 + [_P]),
-    'slayer_alif_fwd': (_INT, [_P] * 17 + [_I64, _I64, _INT, _F, _INT] + [_I64] * 11 + [_P]),
-    'slayer_alif_bwd': (_INT, [_P] * 9 + [_F, _F, _INT, _P] + [_I64] * 5 + [_P]),
+    'slayer_cuba_fwd': (_INT, [_P] * 10 + [_D, _F, _INT, _F, _INT] + [_I64] * 7 + [_DP, _P]),
+    'slayer_cuba_bwd': (_INT, [_P] * 8 + [_F, _F, _F, _INT, _P] + [_I64] * 5 + [_DP, _P]),
+    'slayer_rf_fwd': (_INT, [_P] * 12 + [_F, _INT, _F, _INT] + [_I64] * 7 + [_DP, _P]),
+    'slayer_rf_bwd': (_INT, [_P] * 9 + [_F, _F, _F, _INT, _P] + [_I64] * 4 + [_DP, _P]),
+    'slayer_alif_fwd': (_INT, [_P] * 17 + [_I64, _I64, _INT, _F, _INT] + [_I64] * 11 + [_DP, _P]),
+    'slayer_alif_bwd': (_INT, [_P] * 9 + [_F, _F, _INT, _P] + [_I64] * 5 + [_DP, _P]),
     'slayer_cuba_recurrent_fwd': (_INT, [_P] * 10 + [_F, _INT] + [_I64] * 7 + [_P]),
     'slayer_cuba_recurrent_bwd': (_INT, [_P] * 4 + [_F, _F, _F] + [_I64] * 3 + [_P]),
     'slayer_li_fwd_naive': (_INT, [_P, _P, _P, _P, _D, _INT, _I64, _I64, _I64, _I64, _I64, _P]),

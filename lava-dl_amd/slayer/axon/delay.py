@@ -50,7 +50,10 @@ class Delay(torch.nn.Module):
     def shape(self):
         return None if self.init is False else self.delay.shape
 
-    def forward(self, input):
+    def per_neuron(self, input):
+        """The delays as ``forward`` hands them to the shift: one entry per neuron of ``input.shape[1:-1]``
+        (the per-channel parameter repeated over the other neuron axes).  Draws the delays on the first
+        call, clamps them, checks the channel count (axon/delay.py:132-176 in the reference)."""
         if self.init is False:
             if input.dim() <= 2:
                 raise AssertionError(
@@ -64,12 +67,13 @@ class Delay(torch.nn.Module):
                 'Expected input to have same number of channels as delays. '
                 f'Expected {self.shape[0]}, found {input.shape[1]}.')
         if int(np.prod(input.shape[1:-1])) == self.shape[0]:
-            per_neuron = self.delay
-        else:
-            tile = list(input.shape[1:-1])
-            tile[0] = 1
-            per_neuron = self.delay.reshape((-1,) + (1,) * (len(tile) - 1)).repeat(tile)
-        return _delayFunction.apply(input, per_neuron, self.grad_scale, self.sampling_time)
+            return self.delay
+        tile = list(input.shape[1:-1])
+        tile[0] = 1
+        return self.delay.reshape((-1,) + (1,) * (len(tile) - 1)).repeat(tile)
+
+    def forward(self, input):
+        return _delayFunction.apply(input, self.per_neuron(input), self.grad_scale, self.sampling_time)
 
 
 class _delayFunctionNoGradient(torch.autograd.Function):

@@ -4,6 +4,7 @@ import torch
 
 from .base import Neuron as _Base, hardware_decay
 from .dynamics import leaky_integrator, adaptive_threshold, alif_fused
+from .dynamics import delays as D
 from ..spike import Spike
 
 TAU_RHO_MULT = 100
@@ -103,29 +104,35 @@ class Neuron(_Base):
             spike = self.drop(spike)
         return spike
 
-    def forward(self, input):
+    def forward(self, input, delays=None):
         """Spike response.  Without a norm the whole neuron runs as one fused kernel per direction
-        (same bits as ``spike(*dynamics(input)[1:])``)."""
-        if self.norm is not None:
-            _, voltage, threshold, refractory = self.dynamics(input)
-            return self.spike(voltage, threshold, refractory)
+        (same bits as ``spike(*dynamics(input)[1:])``).  ``delays`` and ``debug``: as in ``cuba.Neuron.forward``."""
+        if self.norm is not None or self.debug or (delays and self.drop is not None):
+            _, voltage, threshold, refractory = self.dynamics(D.chain_input(delays, input))
+            spike = self.spike(voltage, threshold, refractory)
+            if delays:
+                self.spike_last = spike[..., -1].detach().clone()
+            return D.chain_output(delays, spike)
         self._prepare(input)
         args = (input, self._q('current_decay'), self._q('voltage_decay'), self._q('threshold_decay'),
                 self._q('refractory_decay'), self.current_state, self.voltage_state, self.threshold_state,
                 self.refractory_state, self.threshold_step, self.threshold, self.s_scale)
-        if not (torch.is_grad_enabled() and (input.requires_grad or self.requires_grad)):
+        if not (torch.is_grad_enabled() and (input.requires_grad or self.requires_grad or D.needs_grad(delays))):
             # nothing to differentiate: only the spikes are written, the last states come per neuron
-            current_last, voltage_last, _, spike, th_last, ref_last = alif_fused.spikes(*args, self.graded_spike, 1)
+            current_last, voltage_last, _, spike, th_last, ref_last, *rest = alif_fused.spikes(
+                *args, self.graded_spike, 1, delays=delays)
         else:
             # without trainable decays the kernel skips the current trace and returns its last step
-            current, voltage, _, spike, th_last, ref_last = alif_fused.dynamics(
+            current, voltage, _, spike, th_last, ref_last, *rest = alif_fused.dynamics(
                 *args, self.tau_rho * TAU_RHO_MULT, self.scale_rho * SCALE_RHO_MULT, self.graded_spike, 1,
-                keep_current=self.requires_grad)
+                keep_current=self.requires_grad, delays=delays)
             current_last = current[..., -1] if self.requires_grad else current
             voltage_last = voltage[..., -1]
+        if delays:
+            self.spike_last = rest[0]
         if self.persistent_state:
             with torch.no_grad():
-                last = spike[..., -1]
+                last = rest[0] if delays else spike[..., -1]
                 self._carry(current_state=current_last, voltage_state=voltage_last,
                             refractory_state=adaptive_threshold.persistent_ref_state(ref_last, last, th_last).detach(),
                             threshold_state=adaptive_threshold.persistent_th_state(

@@ -4,6 +4,7 @@ import torch
 
 from .base import Neuron as _Base, hardware_decay
 from .dynamics import leaky_integrator, cuba_fused
+from .dynamics import delays as D
 from ..spike import Spike
 
 TAU_RHO_MULT = 100      # surrogate-gradient constants of the CUBA family (neuron/cuba.py:20-21)
@@ -79,30 +80,43 @@ class Neuron(_Base):
             spike = self.drop(spike)
         return spike
 
-    def forward(self, input):
+    def forward(self, input, delays=None):
         """Spike response.  Without a normalisation between current and voltage the three steps run
-        as one fused kernel per direction (same bits as ``spike(dynamics(input)[1])``)."""
-        if self.norm is not None:
-            _, voltage = self.dynamics(input)
-            return self.spike(voltage)
+        as one fused kernel per direction (same bits as ``spike(dynamics(input)[1])``).
+
+        ``delays`` (``dynamics.delays.Delays``) folds a shift of the input and the delays that follow the
+        neuron in a block into the same kernels; the result is then the delayed spike tensor and
+        ``self.spike_last`` holds the undelayed spike of the last step.  ``debug=True`` takes the separate
+        operators (whose ``debug`` cross-checks then run) and so does a neuron with dropout and delays."""
+        if self.norm is not None or self.debug or (delays and self.drop is not None):
+            _, voltage = self.dynamics(D.chain_input(delays, input))
+            spike = self.spike(voltage)
+            if delays:
+                self.spike_last = spike[..., -1].detach().clone()
+            return D.chain_output(delays, spike)
         self._prepare(input)
         args = (input, self._q('current_decay'), self._q('voltage_decay'),
                 self.current_state.contiguous(), self.voltage_state.contiguous(), self.s_scale,
                 self.threshold + self.threshold_eps)
-        if not (torch.is_grad_enabled() and (input.requires_grad or self.requires_grad)):
+        spike_last = None
+        if not (torch.is_grad_enabled() and (input.requires_grad or self.requires_grad
+                                             or D.needs_grad(delays))):
             # nothing to differentiate: only the spikes are written, the last current / voltage come per neuron
-            current_last, voltage_last, spike = cuba_fused.spikes(*args, self.graded_spike, 1)
+            current_last, voltage_last, spike, *rest = cuba_fused.spikes(*args, self.graded_spike, 1, delays=delays)
         else:
             # without trainable decays the kernel skips the current trace and returns its last step
-            current, voltage, spike = cuba_fused.dynamics(
+            current, voltage, spike, *rest = cuba_fused.dynamics(
                 *args, self.tau_rho * TAU_RHO_MULT, self.scale_rho * SCALE_RHO_MULT, self.graded_spike, 1,
-                keep_current=self.requires_grad)
+                keep_current=self.requires_grad, delays=delays)
             current_last = current[..., -1] if self.requires_grad else current
             voltage_last = voltage[..., -1]
+        if delays:
+            self.spike_last = spike_last = rest[0]
         if self.persistent_state:
             with torch.no_grad():               # the product below is a new tensor; slices of a trace are copied
+                last = spike_last if delays else spike[..., -1]
                 self._carry(current_state=current_last,
-                            voltage_state=leaky_integrator.persistent_state(voltage_last, spike[..., -1]).detach())
+                            voltage_state=leaky_integrator.persistent_state(voltage_last, last).detach())
         if self.drop is not None:
             spike = self.drop(spike)
         return spike

@@ -5,6 +5,7 @@ import torch
 
 from .base import Neuron as _Base, hardware_decay
 from .dynamics import resonator, rf_fused
+from .dynamics import delays as D
 from ..spike import complex as complex_spike
 from ..utils.quantize import quantize
 
@@ -169,12 +170,16 @@ class Neuron(ResonatorNeuron):
             spike = self.drop(spike)
         return spike
 
-    def forward(self, input):
+    def forward(self, input, delays=None):
         """Spike response to ``(real_input, imag_input)``.  Without input normalisation the dynamics
-        and the spike run as one fused kernel per direction (same bits as ``spike(*dynamics(input))``)."""
-        if self.real_norm is not None or self.imag_norm is not None:
-            real, imag = self.dynamics(input)
-            return self.spike(real, imag)
+        and the spike run as one fused kernel per direction (same bits as ``spike(*dynamics(input))``).
+        ``delays`` (its input shift applies to both inputs) and ``debug``: as in ``cuba.Neuron.forward``."""
+        if self.real_norm is not None or self.imag_norm is not None or self.debug or (delays and self.drop is not None):
+            real, imag = self.dynamics((D.chain_input(delays, input[0]), D.chain_input(delays, input[1])))
+            spike = self.spike(real, imag)
+            if delays:
+                self.spike_last = spike[..., -1].detach().clone()
+            return D.chain_output(delays, spike)
         real_input, imag_input = input
         if real_input.shape != imag_input.shape:
             raise AssertionError(f'Real input tensor shape ({real_input.shape}) does not match '
@@ -182,14 +187,18 @@ class Neuron(ResonatorNeuron):
         self._prepare(real_input)
         args = (real_input, imag_input, quantize(self.sin_decay), quantize(self.cos_decay),
                 self.real_state, self.imag_state, self.imag_state, self.s_scale, self.threshold)
-        needs_grad = real_input.requires_grad or imag_input.requires_grad or self.requires_grad
+        needs_grad = (real_input.requires_grad or imag_input.requires_grad or self.requires_grad
+                      or D.needs_grad(delays))
         if not (torch.is_grad_enabled() and needs_grad):
             # nothing to differentiate: only the spikes are written, the last state comes per neuron
-            real_last, imag_last, spike = rf_fused.spikes(*args, self.graded_spike, 1)
+            real_last, imag_last, spike, *rest = rf_fused.spikes(*args, self.graded_spike, 1, delays=delays)
         else:
-            real, imag, spike = rf_fused.dynamics(*args, self.tau_rho * TAU_RHO_MULT,
-                                                  self.scale_rho * SCALE_RHO_MULT, self.graded_spike, 1)
+            real, imag, spike, *rest = rf_fused.dynamics(*args, self.tau_rho * TAU_RHO_MULT,
+                                                         self.scale_rho * SCALE_RHO_MULT, self.graded_spike, 1,
+                                                         delays=delays)
             real_last, imag_last = real[..., -1], imag[..., -1]
+        if delays:
+            self.spike_last = rest[0]
         if self.persistent_state:
             with torch.no_grad():
                 self._carry(real_state=real_last, imag_state=imag_last)

@@ -39,7 +39,7 @@ int main(void) {
     CHECK(hipMemcpyAsync(d_decay, decay, sizeof(decay), hipMemcpyHostToDevice, stream));
     CHECK(hipMemcpyAsync(d_state, &state, sizeof(float), hipMemcpyHostToDevice, stream));
 
-    if (slayer_abi_version() != 1) { fprintf(stderr, "unexpected ABI version\n"); return 1; }
+    if (slayer_abi_version() != SLAYER_ABI_VERSION) { fprintf(stderr, "unexpected ABI version\n"); return 1; }
     int rc = slayer_li_fwd(d_out, d_in, d_decay, d_state, (double)threshold * W, W, M, C, C, 1, T, (void*)stream);
     if (rc) { fprintf(stderr, "slayer_li_fwd: %s\n", slayer_error_string(rc)); return 1; }
     rc = slayer_spike_fwd(d_spk, d_out, NULL, 0, threshold, 0, 1.0f, (int64_t)M * T, (void*)stream);

@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(handle, n), f'{n} declared in slayer_hip.h but not exported'
     assert sorted(_native.EXPORTS) == names, 'python binding and header disagree'
-    assert _native.lib().slayer_abi_version() == 1
+    assert _native.lib().slayer_abi_version() == 2
     assert b'success' in _native.lib().slayer_error_string(0)
     assert b'inconsistent' in _native.lib().slayer_error_string(-1)
 
@@ -48,6 +48,10 @@ def test_argument_validation_happens_before_any_launch():
     assert L.slayer_li_fwd(one, one, one, one, 1.0, 64, 8, 4, 1, 1, 1 << 31, None) == ERANGE
     assert L.slayer_li_fwd(one, one, one, one, 1.0, 64, 0, 4, 1, 1, 8, None) == 0          # empty is fine
     assert L.slayer_li_bwd(one, one, one, one, one, None, 8, 4, 1, 8, None) == ENULL       # grad wanted, no workspace
+    # delays folded into a fused block: a table needs a sampling time
+    bad = _native.Delays(16, None, None, None, 0, 0, 0.0)
+    assert L.slayer_cuba_fwd(None, one, one, None, None, one, one, one, one, one, 1.0, 1.0, 0, 1.0, 64,
+                             8, 4, 1, 1, 1, 1, 8, ctypes.byref(bad), None) == EINVAL
     # the allocation-free form refuses what its built-in scratch cannot hold
     assert L.slayer_li_bwd_static(one, one, one, one, one, (1 << 20) + 64, 64, 1, 8, None) == -4
     assert L.slayer_li_bwd_static(one, one, one, one, one, 8192, 8192, 8192, 8, None) == -4
@@ -65,11 +69,11 @@ def test_argument_validation_happens_before_any_launch():
     # fused resonate-and-fire forward: the integer spike decision needs a positive scale
     rf_tail = (1.0, 0, 1.0)
     assert L.slayer_rf_fwd(one, one, one, None, None, one, one, one, one, one, one, one, *rf_tail, 0,
-                           8, 4, 1, 1, 1, 1, 8, None) == EINVAL
+                           8, 4, 1, 1, 1, 1, 8, None, None) == EINVAL
     assert L.slayer_rf_fwd(one, one, one, None, None, one, one, one, one, one, one, one, *rf_tail, -64,
-                           8, 4, 1, 1, 1, 1, 8, None) == EINVAL
+                           8, 4, 1, 1, 1, 1, 8, None, None) == EINVAL
     assert L.slayer_rf_fwd(one, None, one, None, None, one, one, one, one, one, one, one, *rf_tail, 64,
-                           8, 4, 1, 1, 1, 1, 8, None) == ENULL                               # real without imag trace
+                           8, 4, 1, 1, 1, 1, 8, None, None) == ENULL                               # real without imag trace
 
 
 def test_operators_refuse_cpu_tensors():
