@@ -177,6 +177,10 @@ static int static_scratch(float** out) {
     return 0;
 }
 
+bool bwd_scan_usable(int64_t M, int64_t npb, int64_t T);   // scan.hip
+int launch_li_bwd_scan(float* grad_in, float* partial, const float* grad_out, const float* out, const float* decay,
+                       int64_t M, int64_t npb, int64_t num_decays, int64_t T, hipStream_t stream);              // scan.hip
+
 }  // namespace slayer
 
 using namespace slayer;
@@ -210,9 +214,15 @@ extern "C" int slayer_li_bwd(float* grad_in, float* grad_decay, const float* gra
     if (grad_decay && !workspace && M > 0) return SLAYER_ENULL;
     if (M > 0 && T > 0) {
         if (!grad_in || !grad_out || !out || !decay) return SLAYER_ENULL;
-        LiBwd::Params p{{grad_out, out}, {grad_in}, decay, grad_decay ? workspace : nullptr,
-                        neurons_per_batch, num_decays};
-        if (int e = launch_stream<LiBwd>(p, M, T, (hipStream_t)stream)) return e;
+        if (bwd_scan_usable(M, neurons_per_batch, T) && aligned16(grad_in) && aligned16(grad_out) && aligned16(out)) {
+            if (int e = launch_li_bwd_scan(grad_in, grad_decay ? workspace : nullptr, grad_out, out, decay, M,
+                                           neurons_per_batch, num_decays, T, (hipStream_t)stream))
+                return e;
+        } else {
+            LiBwd::Params p{{grad_out, out}, {grad_in}, decay, grad_decay ? workspace : nullptr,
+                            neurons_per_batch, num_decays};
+            if (int e = launch_stream<LiBwd>(p, M, T, (hipStream_t)stream)) return e;
+        }
     }
     if (grad_decay) {
         if (M == 0 || T == 0) return launch_zero_fill(grad_decay, num_decays, (hipStream_t)stream);

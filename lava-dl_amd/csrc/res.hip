@@ -151,6 +151,12 @@ struct ResBwd {
     }
 };
 
+bool bwd_scan_usable(int64_t M, int64_t npb, int64_t T);                // scan.hip
+int launch_res_bwd_scan(float* g_re_in, float* g_im_in, float* partial_sin, float* partial_cos, const float* g_re,
+                        const float* g_im, const float* re, const float* im, const float* sin_decay,
+                        const float* cos_decay, int64_t M, int64_t npb, int64_t num_decays, int64_t T,
+                        hipStream_t stream);                            // scan.hip
+
 }  // namespace slayer
 
 using namespace slayer;
@@ -208,10 +214,19 @@ extern "C" int slayer_res_bwd(float* g_re_in, float* g_im_in, float* grad_sin, f
     hipStream_t st = (hipStream_t)stream;
     if (M > 0 && T > 0) {
         if (!g_re_in || !g_im_in || !g_re || !g_im || !re || !im || !sin_decay || !cos_decay) return SLAYER_ENULL;
-        ResBwd::Params p{{g_re, g_im, re, im}, {g_re_in, g_im_in}, sin_decay, cos_decay,
-                         want ? workspace : nullptr, want ? workspace + M : nullptr,
-                         neurons_per_batch, num_decays};
-        if (int e = launch_stream<ResBwd>(p, M, T, st)) return e;
+        if (bwd_scan_usable(M, neurons_per_batch, T) && aligned16(g_re_in) && aligned16(g_im_in) && aligned16(g_re) &&
+            aligned16(g_im) && aligned16(re) && aligned16(im)) {
+            // large tensors: the complex recurrence as a wave scan over a linear stream
+            if (int e = launch_res_bwd_scan(g_re_in, g_im_in, want ? workspace : nullptr, want ? workspace + M : nullptr,
+                                            g_re, g_im, re, im, sin_decay, cos_decay, M, neurons_per_batch,
+                                            num_decays, T, st))
+                return e;
+        } else {
+            ResBwd::Params p{{g_re, g_im, re, im}, {g_re_in, g_im_in}, sin_decay, cos_decay,
+                             want ? workspace : nullptr, want ? workspace + M : nullptr,
+                             neurons_per_batch, num_decays};
+            if (int e = launch_stream<ResBwd>(p, M, T, st)) return e;
+        }
     }
     if (want) {
         if (M == 0 || T == 0) {

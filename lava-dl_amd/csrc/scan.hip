@@ -1,0 +1,568 @@
+// Reverse-time linear recurrences as wave-level scans.
+//
+// The backward pass of a leaky integrator, g[t] = a * g[t+1] + go[t], is linear in g, so it does not have to
+// be walked one step after the other: a lane takes 4 consecutive steps of a row, 64 lanes take 64 consecutive
+// quads of the tensor, and a suffix scan over the lanes of (multiplier, offset) pairs hands every lane the
+// gradient that enters its quad from later times.  Rows end wherever they end among the lanes: the last quad of
+// a row carries multiplier 0, which cuts the chain there.  Memory is read and written as one linear stream
+// (1 KB per tensor and wave-wide access, no LDS transpose, no row-segmented access pattern), which is what the
+// spike kernels reach 0.8 of the HBM peak with; the row-staged engine stays below 0.7.
+//
+// Arithmetic: once a lane knows the gradient that enters its quad it evaluates its 4 steps exactly as the
+// sequential recurrence does (separate multiply and add), so the result differs from the sequential evaluation
+// only through the rounding of that entering value (a few ulp: six combine steps with |a| <= 1).
+#include "common.h"
+#include "tile.h"
+#include <stdlib.h>
+
+namespace slayer {
+
+int launch_reduce_param_grad(float* grad, const float* partial, float* scratch, int64_t M, int64_t npb,
+                             int64_t num_params, hipStream_t stream);   // li.hip
+
+constexpr int kScanWaves = 4;           // waves per workgroup, each with a span of rows of its own
+constexpr int kScanMaxRows = 64;        // rows per wave at most (LDS tables)
+
+// Cross-lane moves as DPP modifiers (they fold into the VALU instruction that consumes them): the value of the
+// lane n below inside a row of 16 lanes (`fill` where there is none), lane 15 / 31 of the rows below for the
+// rows in `rows`, and the lane just below across the whole wave.
+template <int N>
+__device__ __forceinline__ float lane_below_in_row(float v, float fill) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(fill), __float_as_int(v), 0x110 + N, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float row_bcast15(float v, float fill) {      // rows 1 and 3 <- lane 15 of rows 0 and 2
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(fill), __float_as_int(v), 0x142, 0xa, 0xf, false));
+}
+__device__ __forceinline__ float row_bcast31(float v, float fill) {      // rows 2 and 3 <- lane 31
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(fill), __float_as_int(v), 0x143, 0xc, 0xf, false));
+}
+__device__ __forceinline__ float lane_below(float v, float fill) {       // lane l <- lane l - 1, lane 0 <- fill
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(fill), __float_as_int(v), 0x138, 0xf, 0xf, false));
+}
+
+// Inclusive scan over the lanes, lowest lane first, of affine maps c -> B + A * c: afterwards (A, B) of lane l is
+// the composition of the maps of lanes 0 .. l (lane 0 applied first).
+__device__ __forceinline__ void scan_affine(float& A, float& B) {
+#define SLAYER_COMBINE(An, Bn) do { const float an_ = (An), bn_ = (Bn); B = __fmaf_rn(A, bn_, B); A = A * an_; } while (0)
+    SLAYER_COMBINE(lane_below_in_row<1>(A, 1.0f), lane_below_in_row<1>(B, 0.0f));
+    SLAYER_COMBINE(lane_below_in_row<2>(A, 1.0f), lane_below_in_row<2>(B, 0.0f));
+    SLAYER_COMBINE(lane_below_in_row<4>(A, 1.0f), lane_below_in_row<4>(B, 0.0f));
+    SLAYER_COMBINE(lane_below_in_row<8>(A, 1.0f), lane_below_in_row<8>(B, 0.0f));
+    SLAYER_COMBINE(row_bcast15(A, 1.0f), row_bcast15(B, 0.0f));
+    SLAYER_COMBINE(row_bcast31(A, 1.0f), row_bcast31(B, 0.0f));
+#undef SLAYER_COMBINE
+}
+
+// Inclusive sum over the lanes below that belong to the same run: lane l adds lanes l - reach .. l - 1.
+__device__ __forceinline__ float sum_run(float s, int lane, int reach) {
+    const int in_row = lane & 15;
+    float v;
+    v = lane_below_in_row<1>(s, 0.0f); s += reach >= 1 ? v : 0.0f;
+    v = lane_below_in_row<2>(s, 0.0f); s += reach >= 2 ? v : 0.0f;
+    v = lane_below_in_row<4>(s, 0.0f); s += reach >= 4 ? v : 0.0f;
+    v = lane_below_in_row<8>(s, 0.0f); s += reach >= 8 ? v : 0.0f;
+    v = row_bcast15(s, 0.0f); s += reach > in_row ? v : 0.0f;               // the run goes on below this row of 16
+    v = row_bcast31(s, 0.0f); s += reach > (lane & 31) ? v : 0.0f;         // ... and below this half of the wave
+    return s;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Workgroup-level pieces shared by the scan kernels.
+//
+// A workgroup of kScanWaves waves owns `rpg` consecutive rows = one contiguous span of rpg * QR quads and walks it
+// from its end to its start, 64 * kScanWaves quads per pass (so a span is a few passes and the chip as a whole
+// reads and writes memory as one linear stream).  Thread t of a pass holds quad 64 * kScanWaves - 1 - t of the
+// pass: a lower lane and a lower wave are a later time, the scans run upwards.  Within a pass the gradient that
+// leaves lane 63 of a wave enters lane 0 of the next wave: every wave publishes the map of its 64 quads taken
+// together, one barrier, and every wave applies the maps of the waves before it to what the previous pass left.
+constexpr int kScanQuads = kScanWaves * kWave;       // quads per pass
+
+struct ScanSpan {
+    int tid, lane, wv, rows, nq, npass;
+    int64_t row0;
+    __device__ __forceinline__ void init(int64_t M, int QR, int rpg) {
+        tid = threadIdx.x;
+        lane = tid & (kWave - 1);
+        wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+        row0 = (int64_t)blockIdx.x * rpg;
+        rows = (int)((M - row0) < rpg ? (M - row0) : rpg);
+        nq = rows * QR;
+        npass = (nq + kScanQuads - 1) / kScanQuads;
+    }
+    // quad of this thread in the span for the pass that is worked on first (the last one in memory)
+    __device__ __forceinline__ int first_quad() const { return (npass - 1) * kScanQuads + (kScanQuads - 1 - tid); }
+};
+
+// Row and position in the row of a thread's quad, kept up to date from pass to pass.
+struct ScanCursor {
+    int lq, r, pos;
+    __device__ __forceinline__ void init(int lq0, int nq, int QR) {
+        lq = lq0;
+        r = (lq < nq ? lq : nq - 1) / QR;
+        pos = lq - r * QR;                                           // >= QR for a quad past the end of the span
+    }
+    __device__ __forceinline__ void next(int QR) {
+        lq -= kScanQuads;
+        pos -= kScanQuads;
+        while (pos < 0) { pos += QR; --r; }
+        if (r < 0) { r = 0; pos = 0; }                               // before the span: the thread is idle from here on
+    }
+};
+
+// (row0 mod npb) once with scalar 64-bit arithmetic; row rr of the span then uses parameter
+// ((first + rr) mod npb) / per_param, in 32 bits.
+__device__ __forceinline__ unsigned scan_first_in_batch(int64_t row0, unsigned npb) {
+    return (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)((uint64_t)row0 % (uint64_t)npb));
+}
+
+// LDS of one real-valued scan: per pass parity, the map of each wave's 64 quads and what the pass leaves behind.
+struct RealStage {
+    float A[2][kScanWaves], B[2][kScanWaves], carry[2];
+};
+
+// One pass of a real recurrence g[t] = a * g[t+1] + d[t] on this thread's quad d: returns the four results.
+// `ent` receives the gradient that entered the quad (0 at the end of a row).  One workgroup barrier.
+__device__ __forceinline__ float4 real_stage(RealStage& L, const ScanSpan& sp, int parity, float a, float4 d,
+                                             bool active, bool row_end, float& ent) {
+    // the quad by itself (nothing entering): h0 is what leaves it, a^4 what an entering gradient is scaled by
+    const float h3 = d.w;
+    const float h2 = a * h3 + d.z;
+    const float h1 = a * h2 + d.y;
+    const float h0 = a * h1 + d.x;
+    const float a2 = a * a, a3 = a2 * a, a4 = a2 * a2;
+    float A = (active && !row_end) ? a4 : 0.0f;                      // the last quad of a row lets nothing in
+    float B = active ? h0 : 0.0f;
+    scan_affine(A, B);
+    if (sp.lane == kWave - 1) { L.A[parity][sp.wv] = A; L.B[parity][sp.wv] = B; }
+    __syncthreads();
+    // what enters this wave: what the previous pass left, taken through the waves before this one
+    float carry = L.carry[parity];
+#pragma unroll
+    for (int w = 0; w < kScanWaves - 1; ++w)
+        if (w < sp.wv) carry = __fmaf_rn(L.A[parity][w], carry, L.B[parity][w]);
+    const float leaving = __fmaf_rn(A, carry, B);                    // gradient leaving this thread's quad
+    float entering = lane_below(leaving, carry);
+    if (row_end || !active) entering = 0.0f;
+    ent = entering;
+    float4 g;
+    g.w = __fmaf_rn(a, entering, h3);
+    g.z = __fmaf_rn(a2, entering, h2);
+    g.y = __fmaf_rn(a3, entering, h1);
+    g.x = __fmaf_rn(a4, entering, h0);
+    if (sp.tid == kScanQuads - 1) L.carry[parity ^ 1] = g.x;          // the earliest quad of the pass (always inside the span)
+    return g;
+}
+
+// sum_t g[t+1] * y[t] over a quad (g[t+1] of its last step is what entered it)
+__device__ __forceinline__ float next_step_product(float4 g, float entering, float4 y) {
+    return __fmaf_rn(g.y, y.x, __fmaf_rn(g.z, y.y, __fmaf_rn(g.w, y.z, entering * y.w)));
+}
+
+// Adds a quad's contribution to the sum of its row: first over the lanes of this wave that hold the same row (the
+// row's first quad in the wave sits in the highest lane of the run and collects the lanes below), then into the
+// wave's own table, one lane per row.
+__device__ __forceinline__ void add_to_row(float* table, float s, const ScanSpan& sp, const ScanCursor& c, int QR,
+                                           bool active) {
+    if (!active) s = 0.0f;
+    const int reach = active ? QR - 1 - c.pos : 0;                   // quads of the row after this one
+    s = sum_run(s, sp.lane, reach);
+    if (active && (c.pos == 0 || sp.lane == kWave - 1)) table[c.r] += s;
+}
+
+// partial[row] = sum over the waves' tables, in wave order
+__device__ __forceinline__ void store_row_sums(float* partial, const float (*table)[kScanMaxRows], const ScanSpan& sp) {
+    for (int rr = sp.tid; rr < sp.rows; rr += kScanQuads) {
+        float s = table[0][rr];
+#pragma unroll
+        for (int w = 1; w < kScanWaves; ++w) s += table[w][rr];
+        partial[sp.row0 + rr] = s;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Leaky integrator backward.  npb (rows per batch element) and per_param (rows of a batch element that share a
+// parameter; npb when there is one parameter) are 32-bit: the launcher refuses anything larger.
+template <bool PARTIAL, bool STREAM>
+__global__ __launch_bounds__(kScanQuads) void li_bwd_scan_kernel(
+        float* __restrict__ grad_in, float* __restrict__ partial, const float* __restrict__ grad_out,
+        const float* __restrict__ out, const float* __restrict__ decay, int64_t M, int QR, int rpg,
+        unsigned npb, unsigned per_param) {
+    __shared__ float a_tab[kScanMaxRows];
+    __shared__ float row_sum[kScanWaves][kScanMaxRows];
+    __shared__ RealStage stage;
+    ScanSpan sp;
+    sp.init(M, QR, rpg);
+    const int nq = sp.nq;
+    const int64_t base = sp.row0 * (int64_t)QR * 4;                  // first float of the span
+    const unsigned span_bytes = (unsigned)nq * 16u;
+    const __amdgpu_buffer_rsrc_t src_g = make_rsrc(grad_out + base, span_bytes);
+    const __amdgpu_buffer_rsrc_t src_y = make_rsrc(PARTIAL ? out + base : nullptr, PARTIAL ? span_bytes : 0u);
+    const __amdgpu_buffer_rsrc_t dst = make_rsrc(grad_in + base, span_bytes);
+
+    ScanCursor cur;
+    // Four pass buffers: the pass being worked on and the three after it, requested before anything else (a
+    // workgroup lives for a handful of passes: what it reads should be on its way while it sets up).
+    auto fetch_g = [&](int q) { return buf_load4<STREAM>(src_g, (unsigned)q < (unsigned)nq ? q * 16 : kOutOfRange); };
+    auto fetch_y = [&](int q) {
+        return PARTIAL ? buf_load4<STREAM>(src_y, (unsigned)q < (unsigned)nq ? q * 16 : kOutOfRange)
+                       : make_float4(0.f, 0.f, 0.f, 0.f);
+    };
+    const int q0 = sp.first_quad();
+    float4 go0 = fetch_g(q0), y0 = fetch_y(q0);
+    float4 go1 = fetch_g(q0 - kScanQuads), y1 = fetch_y(q0 - kScanQuads);
+    float4 go2 = fetch_g(q0 - 2 * kScanQuads), y2 = fetch_y(q0 - 2 * kScanQuads);
+    float4 go3 = fetch_g(q0 - 3 * kScanQuads), y3 = fetch_y(q0 - 3 * kScanQuads);
+
+    const unsigned first = scan_first_in_batch(sp.row0, npb);
+    for (int rr = sp.tid; rr < sp.rows; rr += kScanQuads)
+        a_tab[rr] = 1.0f - decay[((first + (unsigned)rr) % npb) / per_param] / 4096.0f;
+    if (PARTIAL)
+        for (int rr = sp.lane; rr < sp.rows; rr += kWave) row_sum[sp.wv][rr] = 0.0f;
+    int parity = (sp.npass - 1) & 1;
+    if (sp.tid == 0) stage.carry[parity] = 0.0f;                     // nothing enters the last quad of the span
+    __syncthreads();
+    cur.init(q0, nq, QR);
+
+    // one pass on the quads in (go, y); the buffer is then refilled with the pass four further on
+    auto pass = [&](float4& go, float4& y) {
+        const bool active = cur.lq < nq;
+        const bool row_end = cur.pos == QR - 1;
+        float entering;
+        const float4 g = real_stage(stage, sp, parity, a_tab[cur.r], go, active, row_end, entering);
+        buf_store4<STREAM>(dst, active ? cur.lq * 16 : kOutOfRange, g);
+        if (PARTIAL) add_to_row(row_sum[sp.wv], next_step_product(g, entering, y), sp, cur, QR, active);
+        go = fetch_g(cur.lq - 4 * kScanQuads);
+        y = fetch_y(cur.lq - 4 * kScanQuads);
+        cur.next(QR);
+        parity ^= 1;
+    };
+    for (int left = sp.npass;;) {
+        pass(go0, y0); if (--left == 0) break;
+        pass(go1, y1); if (--left == 0) break;
+        pass(go2, y2); if (--left == 0) break;
+        pass(go3, y3); if (--left == 0) break;
+    }
+    if (PARTIAL) {
+        __syncthreads();
+        store_row_sums(partial, row_sum, sp);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Fused CUBA / ALIF backward: spike surrogate, then the voltage and the current recurrence, each as a scan of its
+// own with the very arithmetic of li_bwd_scan_kernel -- the input gradient is bit-identical to the spike backward
+// kernel followed by two launches of that kernel.  THETA: the spike threshold is a tensor (threshold + refractory
+// of the adaptive neuron), else the scalar spike_thr.
+template <bool GRADED, bool DECAY_GRAD, bool THETA, bool STREAM>
+__global__ __launch_bounds__(kScanQuads) void cuba_bwd_scan_kernel(
+        float* __restrict__ grad_in, float* __restrict__ partial_i, float* __restrict__ partial_v,
+        const float* __restrict__ grad_spikes, const float* __restrict__ voltage, const float* __restrict__ theta,
+        const float* __restrict__ current, const float* __restrict__ i_decay, const float* __restrict__ v_decay,
+        float spike_thr, float tau, float rho, int64_t M, int QR, int rpg,
+        unsigned npb, unsigned per_i, unsigned per_v) {
+    __shared__ float ai_tab[kScanMaxRows], av_tab[kScanMaxRows];
+    __shared__ float sum_i[kScanWaves][kScanMaxRows], sum_v[kScanWaves][kScanMaxRows];
+    __shared__ RealStage stage_v, stage_i;
+    ScanSpan sp;
+    sp.init(M, QR, rpg);
+    const int nq = sp.nq;
+    const int64_t base = sp.row0 * (int64_t)QR * 4;
+    const unsigned span_bytes = (unsigned)nq * 16u;
+    const __amdgpu_buffer_rsrc_t src_g = make_rsrc(grad_spikes + base, span_bytes);
+    const __amdgpu_buffer_rsrc_t src_v = make_rsrc(voltage + base, span_bytes);
+    const __amdgpu_buffer_rsrc_t src_t = make_rsrc(THETA ? theta + base : nullptr, THETA ? span_bytes : 0u);
+    const __amdgpu_buffer_rsrc_t src_c = make_rsrc(DECAY_GRAD ? current + base : nullptr, DECAY_GRAD ? span_bytes : 0u);
+    const __amdgpu_buffer_rsrc_t dst = make_rsrc(grad_in + base, span_bytes);
+    const float lead = (rho / 2.0f) / tau;
+
+    struct Quads { float4 g, v, th, c; };
+    auto fetch = [&](int q) {
+        const int off = (unsigned)q < (unsigned)nq ? q * 16 : kOutOfRange;
+        Quads x;
+        x.g = buf_load4<STREAM>(src_g, off);
+        x.v = buf_load4<STREAM>(src_v, off);
+        x.th = THETA ? buf_load4<STREAM>(src_t, off) : make_float4(0.f, 0.f, 0.f, 0.f);
+        x.c = DECAY_GRAD ? buf_load4<STREAM>(src_c, off) : make_float4(0.f, 0.f, 0.f, 0.f);
+        return x;
+    };
+    // three pass buffers (up to four tensors each): the pass being worked on and the two after it
+    const int q0 = sp.first_quad();
+    Quads b0 = fetch(q0), b1 = fetch(q0 - kScanQuads), b2 = fetch(q0 - 2 * kScanQuads);
+
+    const unsigned first = scan_first_in_batch(sp.row0, npb);
+    for (int rr = sp.tid; rr < sp.rows; rr += kScanQuads) {
+        const unsigned in_batch = (first + (unsigned)rr) % npb;
+        ai_tab[rr] = 1.0f - i_decay[in_batch / per_i] / 4096.0f;
+        av_tab[rr] = 1.0f - v_decay[in_batch / per_v] / 4096.0f;
+    }
+    if (DECAY_GRAD)
+        for (int rr = sp.lane; rr < sp.rows; rr += kWave) { sum_i[sp.wv][rr] = 0.0f; sum_v[sp.wv][rr] = 0.0f; }
+    int parity = (sp.npass - 1) & 1;
+    if (sp.tid == 0) { stage_v.carry[parity] = 0.0f; stage_i.carry[parity] = 0.0f; }
+    __syncthreads();
+    ScanCursor cur;
+    cur.init(q0, nq, QR);
+
+    // the surrogate, expression by expression as the spike backward kernel evaluates it
+    auto surrogate = [&](float g, float v, float th) {
+        const float d = v - (THETA ? th : spike_thr);
+        return GRADED ? (rho * expf(fminf(d, 0.0f) / tau)) * g : (lead * expf(-fabsf(d) / tau)) * g;
+    };
+    auto pass = [&](Quads& x) {
+        const bool active = cur.lq < nq;
+        const bool row_end = cur.pos == QR - 1;
+        const float4 gv = make_float4(surrogate(x.g.x, x.v.x, x.th.x), surrogate(x.g.y, x.v.y, x.th.y),
+                                      surrogate(x.g.z, x.v.z, x.th.z), surrogate(x.g.w, x.v.w, x.th.w));
+        float ent_v, ent_i;
+        const float4 gc = real_stage(stage_v, sp, parity, av_tab[cur.r], gv, active, row_end, ent_v);
+        const float4 gx = real_stage(stage_i, sp, parity, ai_tab[cur.r], gc, active, row_end, ent_i);
+        buf_store4<STREAM>(dst, active ? cur.lq * 16 : kOutOfRange, gx);
+        if (DECAY_GRAD) {
+            add_to_row(sum_v[sp.wv], next_step_product(gc, ent_v, x.v), sp, cur, QR, active);
+            add_to_row(sum_i[sp.wv], next_step_product(gx, ent_i, x.c), sp, cur, QR, active);
+        }
+        x = fetch(cur.lq - 3 * kScanQuads);
+        cur.next(QR);
+        parity ^= 1;
+    };
+    for (int left = sp.npass;;) {
+        pass(b0); if (--left == 0) break;
+        pass(b1); if (--left == 0) break;
+        pass(b2); if (--left == 0) break;
+    }
+    if (DECAY_GRAD) {
+        __syncthreads();
+        store_row_sums(partial_i, sum_i, sp);
+        store_row_sums(partial_v, sum_v, sp);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Resonator backward: z[t] = mu * z[t+1] + g[t] over complex numbers, z = gr + i gi, mu = (c - i s) with
+// c, s = cos_decay / 4096, sin_decay / 4096 (gr[t] = c gr[t+1] + s gi[t+1] + g_re[t],
+// gi[t] = -s gr[t+1] + c gi[t+1] + g_im[t]).  Same structure as the real scan with complex maps.
+struct Cx { float re, im; };
+__device__ __forceinline__ Cx cmul(Cx a, Cx b) {
+    return Cx{__fmaf_rn(a.re, b.re, -(a.im * b.im)), __fmaf_rn(a.re, b.im, a.im * b.re)};
+}
+__device__ __forceinline__ Cx cfma(Cx a, Cx b, Cx c) {            // a * b + c
+    return Cx{__fmaf_rn(a.re, b.re, __fmaf_rn(-a.im, b.im, c.re)), __fmaf_rn(a.re, b.im, __fmaf_rn(a.im, b.re, c.im))};
+}
+
+struct ComplexStage {
+    float Ar[2][kScanWaves], Ai[2][kScanWaves], Br[2][kScanWaves], Bi[2][kScanWaves], cr[2], ci[2];
+};
+
+// inclusive scan over the lanes of complex affine maps z -> B + A * z (see scan_affine)
+__device__ __forceinline__ void scan_affine_complex(Cx& A, Cx& B) {
+#define SLAYER_COMBINE(M) do {                                                                                  \
+        const Cx an_{M(A.re, 1.0f), M(A.im, 0.0f)}, bn_{M(B.re, 0.0f), M(B.im, 0.0f)};                          \
+        B = cfma(A, bn_, B); A = cmul(A, an_); } while (0)
+    SLAYER_COMBINE(lane_below_in_row<1>);
+    SLAYER_COMBINE(lane_below_in_row<2>);
+    SLAYER_COMBINE(lane_below_in_row<4>);
+    SLAYER_COMBINE(lane_below_in_row<8>);
+    SLAYER_COMBINE(row_bcast15);
+    SLAYER_COMBINE(row_bcast31);
+#undef SLAYER_COMBINE
+}
+
+template <bool PARTIAL, bool STREAM>
+__global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
+        float* __restrict__ g_re_in, float* __restrict__ g_im_in, float* __restrict__ partial_sin,
+        float* __restrict__ partial_cos, const float* __restrict__ g_re, const float* __restrict__ g_im,
+        const float* __restrict__ re, const float* __restrict__ im, const float* __restrict__ sin_decay,
+        const float* __restrict__ cos_decay, int64_t M, int QR, int rpg, unsigned npb, unsigned per_param) {
+    __shared__ float c_tab[kScanMaxRows], s_tab[kScanMaxRows];
+    __shared__ float sum_s[kScanWaves][kScanMaxRows], sum_c[kScanWaves][kScanMaxRows];
+    __shared__ ComplexStage L;
+    ScanSpan sp;
+    sp.init(M, QR, rpg);
+    const int nq = sp.nq;
+    const int64_t base = sp.row0 * (int64_t)QR * 4;
+    const unsigned span_bytes = (unsigned)nq * 16u;
+    const __amdgpu_buffer_rsrc_t src_gr = make_rsrc(g_re + base, span_bytes), src_gi = make_rsrc(g_im + base, span_bytes);
+    const __amdgpu_buffer_rsrc_t src_re = make_rsrc(PARTIAL ? re + base : nullptr, PARTIAL ? span_bytes : 0u);
+    const __amdgpu_buffer_rsrc_t src_im = make_rsrc(PARTIAL ? im + base : nullptr, PARTIAL ? span_bytes : 0u);
+    const __amdgpu_buffer_rsrc_t dst_r = make_rsrc(g_re_in + base, span_bytes), dst_i = make_rsrc(g_im_in + base, span_bytes);
+
+    struct Quads { float4 gr, gi, re, im; };
+    auto fetch = [&](int q) {
+        const int off = (unsigned)q < (unsigned)nq ? q * 16 : kOutOfRange;
+        Quads x;
+        x.gr = buf_load4<STREAM>(src_gr, off);
+        x.gi = buf_load4<STREAM>(src_gi, off);
+        x.re = PARTIAL ? buf_load4<STREAM>(src_re, off) : make_float4(0.f, 0.f, 0.f, 0.f);
+        x.im = PARTIAL ? buf_load4<STREAM>(src_im, off) : make_float4(0.f, 0.f, 0.f, 0.f);
+        return x;
+    };
+    const int q0 = sp.first_quad();
+    Quads b0 = fetch(q0), b1 = fetch(q0 - kScanQuads), b2 = fetch(q0 - 2 * kScanQuads);
+
+    const unsigned first = scan_first_in_batch(sp.row0, npb);
+    for (int rr = sp.tid; rr < sp.rows; rr += kScanQuads) {
+        const unsigned j = ((first + (unsigned)rr) % npb) / per_param;
+        c_tab[rr] = cos_decay[j] / 4096.0f;
+        s_tab[rr] = sin_decay[j] / 4096.0f;
+    }
+    if (PARTIAL)
+        for (int rr = sp.lane; rr < sp.rows; rr += kWave) { sum_s[sp.wv][rr] = 0.0f; sum_c[sp.wv][rr] = 0.0f; }
+    int parity = (sp.npass - 1) & 1;
+    if (sp.tid == 0) { L.cr[parity] = 0.0f; L.ci[parity] = 0.0f; }
+    __syncthreads();
+    ScanCursor cur;
+    cur.init(q0, nq, QR);
+
+    auto pass = [&](Quads& x) {
+        const bool active = cur.lq < nq;
+        const bool row_end = cur.pos == QR - 1;
+        const Cx mu{c_tab[cur.r], -s_tab[cur.r]};
+        // the quad by itself
+        const Cx d0{x.gr.x, x.gi.x}, d1{x.gr.y, x.gi.y}, d2{x.gr.z, x.gi.z}, d3{x.gr.w, x.gi.w};
+        const Cx h3 = d3, h2 = cfma(mu, h3, d2), h1 = cfma(mu, h2, d1), h0 = cfma(mu, h1, d0);
+        const Cx mu2 = cmul(mu, mu), mu3 = cmul(mu2, mu), mu4 = cmul(mu2, mu2);
+        const bool open = active && !row_end;
+        Cx A{open ? mu4.re : 0.0f, open ? mu4.im : 0.0f};
+        Cx B{active ? h0.re : 0.0f, active ? h0.im : 0.0f};
+        scan_affine_complex(A, B);
+        if (sp.lane == kWave - 1) {
+            L.Ar[parity][sp.wv] = A.re; L.Ai[parity][sp.wv] = A.im;
+            L.Br[parity][sp.wv] = B.re; L.Bi[parity][sp.wv] = B.im;
+        }
+        __syncthreads();
+        Cx carry{L.cr[parity], L.ci[parity]};
+#pragma unroll
+        for (int w = 0; w < kScanWaves - 1; ++w)
+            if (w < sp.wv) carry = cfma(Cx{L.Ar[parity][w], L.Ai[parity][w]}, carry, Cx{L.Br[parity][w], L.Bi[parity][w]});
+        const Cx leaving = cfma(A, carry, B);
+        Cx ent{lane_below(leaving.re, carry.re), lane_below(leaving.im, carry.im)};
+        if (row_end || !active) ent = Cx{0.0f, 0.0f};
+        const Cx z3 = cfma(mu, ent, h3), z2 = cfma(mu2, ent, h2), z1 = cfma(mu3, ent, h1), z0 = cfma(mu4, ent, h0);
+        const int off = active ? cur.lq * 16 : kOutOfRange;
+        buf_store4<STREAM>(dst_r, off, make_float4(z0.re, z1.re, z2.re, z3.re));
+        buf_store4<STREAM>(dst_i, off, make_float4(z0.im, z1.im, z2.im, z3.im));
+        if (sp.tid == kScanQuads - 1) { L.cr[parity ^ 1] = z0.re; L.ci[parity ^ 1] = z0.im; }
+        if (PARTIAL) {
+            // grad_sin: sum -gr[t+1] im[t] + gi[t+1] re[t];  grad_cos: sum gr[t+1] re[t] + gi[t+1] im[t]
+            const float4 nr = make_float4(z1.re, z2.re, z3.re, ent.re), ni = make_float4(z1.im, z2.im, z3.im, ent.im);
+            float ss = 0.0f, sc = 0.0f;
+            ss = __fmaf_rn(ni.w, x.re.w, __fmaf_rn(-nr.w, x.im.w, ss)); sc = __fmaf_rn(ni.w, x.im.w, __fmaf_rn(nr.w, x.re.w, sc));
+            ss = __fmaf_rn(ni.z, x.re.z, __fmaf_rn(-nr.z, x.im.z, ss)); sc = __fmaf_rn(ni.z, x.im.z, __fmaf_rn(nr.z, x.re.z, sc));
+            ss = __fmaf_rn(ni.y, x.re.y, __fmaf_rn(-nr.y, x.im.y, ss)); sc = __fmaf_rn(ni.y, x.im.y, __fmaf_rn(nr.y, x.re.y, sc));
+            ss = __fmaf_rn(ni.x, x.re.x, __fmaf_rn(-nr.x, x.im.x, ss)); sc = __fmaf_rn(ni.x, x.im.x, __fmaf_rn(nr.x, x.re.x, sc));
+            add_to_row(sum_s[sp.wv], ss, sp, cur, QR, active);
+            add_to_row(sum_c[sp.wv], sc, sp, cur, QR, active);
+        }
+        x = fetch(cur.lq - 3 * kScanQuads);
+        cur.next(QR);
+        parity ^= 1;
+    };
+    for (int left = sp.npass;;) {
+        pass(b0); if (--left == 0) break;
+        pass(b1); if (--left == 0) break;
+        pass(b2); if (--left == 0) break;
+    }
+    if (PARTIAL) {
+        __syncthreads();
+        store_row_sums(partial_sin, sum_s, sp);
+        store_row_sums(partial_cos, sum_c, sp);
+    }
+}
+
+// Rows per workgroup: the fewest rows whose bytes are a whole number of 128-byte lines (so that no line is
+// shared between two workgroups), repeated until the span is at least two passes long; at most kScanMaxRows.
+inline int scan_rows_per_group(int64_t M, int64_t T) {
+    int64_t unit = 32;                                   // rows * T must be a multiple of 32 floats
+    for (int64_t t = T; (t & 1) == 0 && unit > 1; t >>= 1) unit >>= 1;
+    if (unit > kScanMaxRows) unit = 1;
+    int64_t r = unit;
+    const int64_t want = 2 * kScanWaves * kWave * 4;     // floats in two passes
+    while (r * T < want && r + unit <= kScanMaxRows) r += unit;
+    if (r < 1) r = 1;
+    if (r > kScanMaxRows) r = kScanMaxRows;
+    if (r > M) r = M;
+    return (int)r;
+}
+
+// Tensors of at least this many elements take the scan (smaller ones keep the sequential kernel, whose
+// grad_in is bit-identical to a step-by-step evaluation).  SLAYER_BWD_SCAN_MIN overrides it (tuning).
+int64_t bwd_scan_min_elements() {
+    static const int64_t v = [] {
+        const char* e = getenv("SLAYER_BWD_SCAN_MIN");
+        return e ? (int64_t)atoll(e) : (int64_t)1 << 20;
+    }();
+    return v;
+}
+
+// True when the scan kernels can run a problem of this shape: whole quads, spans addressable with 32 bits,
+// 32-bit row arithmetic, large enough (the callers also check that every tensor is 16-byte aligned).
+bool bwd_scan_usable(int64_t M, int64_t npb, int64_t T) {
+    if (M <= 0 || T <= 0 || (T % 4) != 0 || T > (1 << 22) || M * T < bwd_scan_min_elements()) return false;
+    return npb > 0 && npb < ((int64_t)1 << 31);
+}
+
+struct ScanGrid { dim3 grid; int rpg, QR; bool streaming, ok; };
+static ScanGrid scan_grid(int64_t M, int64_t T) {
+    ScanGrid g;
+    g.rpg = scan_rows_per_group(M, T);
+    const int64_t blocks = (M + g.rpg - 1) / g.rpg;
+    g.ok = blocks <= 0x7fffffffLL;
+    g.grid = dim3((unsigned)blocks);
+    g.QR = (int)(T / 4);
+    g.streaming = stream_is_large(M, T);
+    return g;
+}
+static unsigned rows_per_param(int64_t npb, int64_t n) { return (unsigned)(n > 1 ? npb / n : npb); }
+
+int launch_li_bwd_scan(float* grad_in, float* partial, const float* grad_out, const float* out, const float* decay,
+                       int64_t M, int64_t npb, int64_t num_decays, int64_t T, hipStream_t stream) {
+    const ScanGrid g = scan_grid(M, T);
+    if (!g.ok) return SLAYER_ERANGE;
+#define SLAYER_SCAN(P, S)                                                                                        \
+    hipLaunchKernelGGL((li_bwd_scan_kernel<P, S>), g.grid, dim3(kScanQuads), 0, stream, grad_in, partial, grad_out, \
+                       out, decay, M, g.QR, g.rpg, (unsigned)npb, rows_per_param(npb, num_decays))
+    if (partial) { if (g.streaming) SLAYER_SCAN(true, true); else SLAYER_SCAN(true, false); }
+    else { if (g.streaming) SLAYER_SCAN(false, true); else SLAYER_SCAN(false, false); }
+#undef SLAYER_SCAN
+    return (int)hipGetLastError();
+}
+
+// theta == nullptr: CUBA (scalar spike threshold); else ALIF.  partial_i / partial_v both or neither.
+int launch_cuba_bwd_scan(float* grad_in, float* partial_i, float* partial_v, const float* grad_spikes,
+                         const float* voltage, const float* theta, const float* current, const float* i_decay,
+                         const float* v_decay, float spike_thr, float tau, float rho, bool graded,
+                         int64_t M, int64_t npb, int64_t n_id, int64_t n_vd, int64_t T, hipStream_t stream) {
+    const ScanGrid g = scan_grid(M, T);
+    if (!g.ok) return SLAYER_ERANGE;
+#define SLAYER_SCAN(G, D, TH, S)                                                                                 \
+    hipLaunchKernelGGL((cuba_bwd_scan_kernel<G, D, TH, S>), g.grid, dim3(kScanQuads), 0, stream, grad_in, partial_i, \
+                       partial_v, grad_spikes, voltage, theta, current, i_decay, v_decay, spike_thr, tau, rho, M, \
+                       g.QR, g.rpg, (unsigned)npb, rows_per_param(npb, n_id), rows_per_param(npb, n_vd))
+#define SLAYER_SCAN_S(G, D, TH) do { if (g.streaming) SLAYER_SCAN(G, D, TH, true); else SLAYER_SCAN(G, D, TH, false); } while (0)
+#define SLAYER_SCAN_T(G, D) do { if (theta) SLAYER_SCAN_S(G, D, true); else SLAYER_SCAN_S(G, D, false); } while (0)
+    const bool want = partial_i != nullptr;
+    if (graded) { if (want) SLAYER_SCAN_T(true, true); else SLAYER_SCAN_T(true, false); }
+    else { if (want) SLAYER_SCAN_T(false, true); else SLAYER_SCAN_T(false, false); }
+#undef SLAYER_SCAN_T
+#undef SLAYER_SCAN_S
+#undef SLAYER_SCAN
+    return (int)hipGetLastError();
+}
+
+int launch_res_bwd_scan(float* g_re_in, float* g_im_in, float* partial_sin, float* partial_cos, const float* g_re,
+                        const float* g_im, const float* re, const float* im, const float* sin_decay,
+                        const float* cos_decay, int64_t M, int64_t npb, int64_t num_decays, int64_t T,
+                        hipStream_t stream) {
+    const ScanGrid g = scan_grid(M, T);
+    if (!g.ok) return SLAYER_ERANGE;
+#define SLAYER_SCAN(P, S)                                                                                        \
+    hipLaunchKernelGGL((res_bwd_scan_kernel<P, S>), g.grid, dim3(kScanQuads), 0, stream, g_re_in, g_im_in,          \
+                       partial_sin, partial_cos, g_re, g_im, re, im, sin_decay, cos_decay, M, g.QR, g.rpg,       \
+                       (unsigned)npb, rows_per_param(npb, num_decays))
+    if (partial_sin) { if (g.streaming) SLAYER_SCAN(true, true); else SLAYER_SCAN(true, false); }
+    else { if (g.streaming) SLAYER_SCAN(false, true); else SLAYER_SCAN(false, false); }
+#undef SLAYER_SCAN
+    return (int)hipGetLastError();
+}
+
+}  // namespace slayer

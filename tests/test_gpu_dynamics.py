@@ -7,7 +7,7 @@ import torch
 
 from oracle import slayer_oracle as O
 from tests.golden import fixtures as G
-from tests.util import seed_of, dev, sparse_input, assert_exact, assert_rel
+from tests.util import assert_exact, assert_rel, assert_same_gradient, assert_scale, dev, seed_of, sparse_input, SCAN_MIN
 
 pytestmark = pytest.mark.gpu
 
@@ -80,7 +80,7 @@ def test_all_tile_geometries(slayer, M_per_batch):
     from lava_dl_amd.slayer.neuron.dynamics import leaky_integrator as L, resonator as R
     gi, gd = L._bwd(g.to(dev()), out, d1g)
     r_gi, r_gd = O.li_bwd(g, ref, d1)
-    assert_exact(gi, r_gi, 'li_bwd grad_input')
+    (assert_exact if gi.numel() < SCAN_MIN else assert_scale)(gi, r_gi, 'li_bwd grad_input')
     assert_rel(gd, r_gd, 'li_bwd grad_decay', rel=1e-4)
     th, rf = D.adaptive_threshold.dynamics(xg, zg, d1g, og, d2g, 0.5, 1.0, 64)
     r_th, r_rf = O.ath_fwd(x, zero, d1, one, d2, 0.5, 1.0, 64)
@@ -94,8 +94,9 @@ def test_all_tile_geometries(slayer, M_per_batch):
     assert_exact(im, r_im, 'res imag')
     got = R._bwd(g.to(dev()), xg, re, im, sin.to(dev()), cos.to(dev()))
     want = O.res_bwd(g, x, r_re, r_im, sin, cos)
-    assert_exact(got[0], want[0], 'res_bwd grad_real')
-    assert_exact(got[1], want[1], 'res_bwd grad_imag')
+    close = assert_exact if got[0].numel() < SCAN_MIN else assert_scale
+    close(got[0], want[0], 'res_bwd grad_real')
+    close(got[1], want[1], 'res_bwd grad_imag')
     assert_rel(got[2], want[2], 'res_bwd grad_sin', rel=1e-4)
     assert_rel(got[3], want[3], 'res_bwd grad_cos', rel=1e-4)
 

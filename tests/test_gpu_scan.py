@@ -1,0 +1,131 @@
+"""The float backward recurrences as wave scans (csrc/scan.hip: tensors of 2^20 elements and more) against the
+oracle's step-by-step loops (neuron/dynamics/leaky_integrator.py:234-259, resonator.py:379-467 in the reference)
+and against the one-thread-per-neuron GPU kernels; the fused CUBA / ALIF backward scans against the chain of
+spike backward + two leaky-integrator scans, bit for bit."""
+import pytest
+import torch
+
+from oracle import slayer_oracle as O
+from tests.util import dev, sparse_input, assert_rel, assert_scale, seed_of, SCAN_MIN
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope='module')
+def slayer():
+    import lava_dl_amd.slayer as s
+    return s
+
+
+# (shape, number of decays): rows of one quad, rows shorter / longer than a wave and than a pass, row counts that
+# do not fill the last workgroup, rows that are a whole number of lines and rows that are not, per-neuron decays
+SHAPES = [((262144 + 3, 1, 4), 1), ((3, 43691, 8), 43691), ((5, 1024, 300), 1024), ((2, 4099, 128), 4099),
+          ((7, 161, 1000), 161), ((3, 43, 8196), 43), ((1, 2, 524288), 2), ((2, 16, 33, 31, 76), 16)]
+
+
+@pytest.mark.parametrize('shape,nd', SHAPES)
+def test_li_bwd_scan_against_oracle_and_sequential_kernel(slayer, shape, nd):
+    L = slayer.neuron.dynamics.leaky_integrator
+    gen = torch.Generator().manual_seed(seed_of('li-scan', shape))
+    numel = 1
+    for s in shape:
+        numel *= s
+    assert numel >= SCAN_MIN
+    g = torch.randn(shape, generator=gen)
+    y = torch.randn(shape, generator=gen) * 2
+    d = torch.randint(0, 4097, (nd,), generator=gen).float()
+    d[0] = 0.0                                     # a pure integrator: the longest carries
+    if nd > 1:
+        d[1] = 4096.0                              # nothing carried at all
+    gi, gd = L._bwd(g.to(dev()), y.to(dev()), d.to(dev()))
+    seq = L._bwd_naive(g.to(dev()), d.to(dev()))
+    assert_scale(gi, seq.cpu(), 'scan vs step-by-step kernel')
+    # the oracle on slabs of rows (whole tensor when it is small enough for the python loop over time)
+    rows = g.reshape(-1, shape[-1])
+    M = rows.shape[0]
+    npb = M // shape[0]
+    pick = torch.unique(torch.cat([torch.arange(0, min(M, 40)), torch.arange(max(M - 40, 0), M),
+                                   torch.randint(0, M, (60,), generator=gen)]))
+    idx = ((pick % npb) // (npb // nd)) if nd > 1 else torch.zeros_like(pick)
+    a = (1 - d[idx] / 4096).reshape(-1, 1)
+    go, ref = rows[pick], torch.zeros(len(pick), shape[-1])
+    acc = torch.zeros(len(pick), 1)
+    for t in range(shape[-1] - 1, -1, -1):
+        acc = a * acc + go[:, t:t + 1]
+        ref[:, t:t + 1] = acc
+    assert_scale(gi.reshape(-1, shape[-1])[pick.to(dev())], ref, 'scan vs step-by-step recurrence (float32)')
+    # decay gradient in float64 from the sequential result
+    prod = seq.double().cpu()[..., 1:] * y.double()[..., :-1]
+    want = prod.sum().reshape(1) if nd == 1 else prod.reshape(shape[0], nd, -1).sum(dim=(0, 2))
+    assert_rel(gd, want.float(), 'grad_decay', rel=1e-4)
+
+
+def test_li_bwd_scan_whole_tensor_against_oracle(slayer):
+    L = slayer.neuron.dynamics.leaky_integrator
+    shape = (4, 16, 64, 300)
+    gen = torch.Generator().manual_seed(77)
+    g, y = torch.randn(shape, generator=gen), torch.randn(shape, generator=gen)
+    d = torch.randint(0, 4096, (16,), generator=gen).float()
+    gi, gd = L._bwd(g.to(dev()), y.to(dev()), d.to(dev()))
+    r_gi, r_gd = O.li_bwd(g, y, d)
+    assert_scale(gi, r_gi, 'grad_input vs oracle')
+    assert_rel(gd, r_gd, 'grad_decay vs oracle', rel=1e-4)
+
+
+@pytest.mark.parametrize('shape,nd', [((3, 700, 520), 700), ((2, 16, 40, 32, 28), 16), ((9, 128, 1000), 1)])
+def test_res_bwd_scan_against_oracle(slayer, shape, nd):
+    R = slayer.neuron.dynamics.resonator
+    gen = torch.Generator().manual_seed(seed_of('res-scan', shape))
+    g_re, g_im = torch.randn(shape, generator=gen), torch.randn(shape, generator=gen)
+    re, im = torch.randn(shape, generator=gen), torch.randn(shape, generator=gen)
+    decay = torch.randint(40, 4096, (nd,), generator=gen).float()
+    phi = 2 * 3.141592653589793 * torch.rand(nd, generator=gen)
+    sin, cos = ((4096 - decay) * torch.sin(phi)).round(), ((4096 - decay) * torch.cos(phi)).round()
+    to = lambda t: t.to(dev())
+    got = R._bwd(to(g_re), to(g_im), to(re), to(im), to(sin), to(cos))
+    n = min(shape[0], 2)
+    want = O.res_bwd(g_re[:n], g_im[:n], re[:n], im[:n], sin, cos)
+    assert_scale(got[0][:n], want[0], 'grad real')
+    assert_scale(got[1][:n], want[1], 'grad imag')
+    seq = R._bwd_naive(to(g_re), to(g_im), to(sin), to(cos)) if hasattr(R, '_bwd_naive') else None
+    if seq is not None:
+        assert_scale(got[0], seq[0].cpu(), 'grad real vs step-by-step kernel')
+        assert_scale(got[1], seq[1].cpu(), 'grad imag vs step-by-step kernel')
+        gr, gi = seq[0].double().cpu(), seq[1].double().cpu()
+        s_sum = (-gr[..., 1:] * im.double()[..., :-1] + gi[..., 1:] * re.double()[..., :-1])
+        c_sum = (gr[..., 1:] * re.double()[..., :-1] + gi[..., 1:] * im.double()[..., :-1])
+        red = (lambda p: p.sum().reshape(1)) if nd == 1 else (lambda p: p.reshape(shape[0], nd, -1).sum(dim=(0, 2)))
+        assert_rel(got[2], red(s_sum).float(), 'grad sin', rel=1e-4)
+        assert_rel(got[3], red(c_sum).float(), 'grad cos', rel=1e-4)
+
+
+@pytest.mark.parametrize('shape', [(5, 1024, 300), (2, 16, 33, 31, 76), (3, 43, 8196)])
+@pytest.mark.parametrize('graded', [False, True])
+@pytest.mark.parametrize('kind', ['cuba', 'alif'])
+def test_fused_backward_scans_equal_the_chain_of_scans_bit_for_bit(slayer, shape, graded, kind):
+    """Same arithmetic, same spans: spike backward + leaky-integrator scan (voltage) + leaky-integrator scan
+    (current) and the one fused kernel give the same input gradient, every bit."""
+    D = slayer.neuron.dynamics
+    S = slayer.spike.spike
+    gen = torch.Generator().manual_seed(seed_of('fused-scan', shape, graded, kind))
+    C = shape[1]
+    g = torch.randn(shape, generator=gen).to(dev())
+    vol = (torch.randn(shape, generator=gen) * 1.5).to(dev())
+    cur = torch.randn(shape, generator=gen).to(dev())
+    theta = (1 + torch.rand(shape, generator=gen)).to(dev())
+    di = torch.randint(0, 4097, (C,), generator=gen).float().to(dev())
+    dv = torch.randint(0, 4097, (C,), generator=gen).float().to(dev())
+    thr, tau, rho = 1.0, 0.7, 1.3
+    for need in (True, False):
+        if kind == 'cuba':
+            gx, g_i, g_v = D.cuba_fused._bwd(g, vol, cur if need else None, di, dv, thr, tau, rho, graded, need)
+            gv = S._bwd(g, vol, None, thr, tau, rho, graded)
+        else:
+            gx, g_i, g_v = D.alif_fused._bwd(g, vol, theta, cur if need else None, di, dv, tau, rho, graded, need)
+            gv = S._bwd(g, vol, theta, 0.0, tau, rho, graded)
+        gc, r_gv = D.leaky_integrator._bwd(gv, vol, dv, need)
+        r_gx, r_gi = D.leaky_integrator._bwd(gc, cur, di, need)
+        assert torch.equal(gx, r_gx), f'{kind} fused scan differs from the chain (decay gradients: {need})'
+        if need:
+            assert_rel(g_i, r_gi.cpu(), 'grad current decay', rel=1e-4)
+            assert_rel(g_v, r_gv.cpu(), 'grad voltage decay', rel=1e-4)

@@ -44,3 +44,29 @@ def assert_rel(gpu, ref, what='', rel=REL):
         i = int(torch.argmax(err - tol))
         raise AssertionError(f'{what}: elementwise tolerance exceeded at flat index {i}: '
                              f'gpu={g.flatten()[i].item()!r} ref={r.flatten()[i].item()!r}')
+
+
+SCAN_MIN = 1 << 20   # float backward recurrences run as wave scans from this many elements on (csrc/scan.hip)
+
+
+def assert_scale(gpu, ref, what='', rel=REL):
+    """max |gpu - ref| <= rel * max |ref|: the bar for float gradients that went through a scan (its rounding
+    differs from a step-by-step evaluation by a few ulp of the largest terms, not of each result)."""
+    g = gpu.detach().cpu().double()
+    r = ref.detach().cpu().double()
+    assert g.shape == r.shape, (what, g.shape, r.shape)
+    if r.numel() == 0:
+        return
+    scale = float(r.abs().max())
+    err = float((g - r).abs().max())
+    if err > rel * scale:
+        raise AssertionError(f'{what}: max abs err {err:.3e} > {rel} * {scale:.3e}')
+
+
+def assert_same_gradient(a, b, what=''):
+    """Two evaluations of the same float gradient on the GPU: bit-identical while both are step-by-step
+    (small tensors), within 1e-5 of the scale once the scan kernels take over."""
+    if a.numel() < SCAN_MIN:
+        assert torch.equal(a, b), what
+    else:
+        assert_scale(a, b, what)
