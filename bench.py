@@ -27,12 +27,6 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch divided by algorithmic bytes, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# script scaled by a plain copy of known size (profiles/cuba_fwd_bwd_32x16x32x32x300.md).
-MEASURED_TRAFFIC_FACTOR = {'stream_kernel<LiFwd>': 1.037, 'stream_kernel<LiBwd>': 1.058,
-                           'spike_fwd_kernel': 1.000, 'spike_bwd_kernel': 1.000}
-
-
 def _events(gen, shape, p, amp=1.0):
     return (torch.rand(shape, generator=gen) < p).float() * torch.randn(shape, generator=gen) * amp
 
@@ -120,7 +114,7 @@ class Cuba(Workload):
     shape = (32, 16, 32, 32, 300)
     ops = [('li_fwd_current', 'stream_kernel<LiFwd>', 8), ('li_fwd_voltage', 'stream_kernel<LiFwd>', 8),
            ('spike_fwd', 'spike_fwd_kernel', 8), ('spike_bwd', 'spike_bwd_kernel', 12),
-           ('li_bwd_voltage', 'stream_kernel<LiBwd>', 12), ('li_bwd_current', 'stream_kernel<LiBwd>', 12)]
+           ('li_bwd_voltage', 'li_bwd_scan_kernel', 12), ('li_bwd_current', 'li_bwd_scan_kernel', 12)]
     w, thr = 64, 1.0
     note = 'w_scale=64, per-channel decays uniform over [0,4096), threshold 1.0, input Bernoulli(0.02) x N(0,0.5)'
 
@@ -156,20 +150,26 @@ class Cuba(Workload):
         L = self.L
         cur = L._fwd(self.x, self.d_i, self.zero, -1, self.w)
         if op == 'li_bwd_current':
-            return lambda: L._bwd(self.g, cur, self.d_i, False)
+            return lambda: L._bwd(self.g, cur, self.d_i, False, True)
         vol = L._fwd(cur, self.d_v, self.zero, self.thr, self.w)
-        return lambda: L._bwd(self.g, vol, self.d_v, False)
+        return lambda: L._bwd(self.g, vol, self.d_v, False, True)
 
-    def cpu_step(self, n):
+    def cpu_step(self, n, sl=None):
+        """The oracle on batch[:n] (channels `sl` when given); returns (spikes, grad of the input)."""
         from oracle import slayer_oracle as O
         c, zero = self.cpu, torch.tensor([0.0])
-        x, g = c['x'][:n], c['g'][:n]
-        cur = O.li_fwd(x, c['d_i'], zero, self.w)
-        vol = O.li_fwd(cur, c['d_v'], zero, self.w, self.thr)
-        O.spike_fwd(vol, self.thr)
+        x, g, d_i, d_v = c['x'][:n], c['g'][:n], c['d_i'], c['d_v']
+        if sl is not None:
+            x, g, d_i, d_v = x[:, sl], g[:, sl], d_i[sl], d_v[sl]
+        cur = O.li_fwd(x, d_i, zero, self.w)
+        vol = O.li_fwd(cur, d_v, zero, self.w, self.thr)
+        spk = O.spike_fwd(vol, self.thr)
         g_vol = O.spike_bwd(g, vol, self.thr, 1.0, 1.0)
-        g_cur, _ = O.li_bwd(g_vol, vol, c['d_v'])
-        O.li_bwd(g_cur, cur, c['d_i'])
+        g_cur, _ = O.li_bwd(g_vol, vol, d_v)
+        g_x, _ = O.li_bwd(g_cur, cur, d_i)
+        return spk, g_x
+
+    parity_slab = (1, slice(3, 5))      # batch[:1], two channels
 
 
 class CubaFused(Cuba):
@@ -240,10 +240,13 @@ class CubaFwdSmall(Workload):
             vol = self.L._fwd(cur, self.d_v, self.zero, 1.25, 64)
         return vol
 
-    def cpu_step(self, n):
+    def cpu_step(self, n, sl=None):
         from oracle import slayer_oracle as O
         c, zero = self.cpu, torch.tensor([0.0])
-        O.li_fwd(O.li_fwd(c['x'][:n], c['d_i'], zero, 64), c['d_v'], zero, 64, 1.25)
+        x = c['x'][:n] if sl is None else c['x'][:n, sl]
+        return O.li_fwd(O.li_fwd(x, c['d_i'], zero, 64), c['d_v'], zero, 64, 1.25), None
+
+    parity_slab = (4, slice(0, 128))    # the whole tensor
 
 
 class Alif(Workload):
@@ -282,18 +285,24 @@ class Alif(Workload):
             g_x, _ = L._bwd(g_cur, cur, self.d_i)
         return spk, g_x
 
-    def cpu_step(self, n):
+    def cpu_step(self, n, sl=None):
         from oracle import slayer_oracle as O
         c, zero, one = self.cpu, torch.tensor([0.0]), torch.tensor([1.0])
         x, g = c['x'][:n], c['g'][:n]
-        cur = O.li_fwd(x, c['d_i'], zero, 64)
-        vol = O.li_fwd(cur, c['d_v'], zero, 64)
-        th, ref = O.ath_fwd(vol, zero, c['d_ref'], one, c['d_th'], 0.5, 1.0, 64)
+        d_i, d_v, d_ref, d_th = c['d_i'], c['d_v'], c['d_ref'], c['d_th']
+        if sl is not None:
+            x, g, d_i, d_v, d_ref, d_th = x[:, sl], g[:, sl], d_i[sl], d_v[sl], d_ref[sl], d_th[sl]
+        cur = O.li_fwd(x, d_i, zero, 64)
+        vol = O.li_fwd(cur, d_v, zero, 64)
+        th, ref = O.ath_fwd(vol, zero, d_ref, one, d_th, 0.5, 1.0, 64)
         theta = th + ref
-        O.spike_fwd(vol, theta)
+        spk = O.spike_fwd(vol, theta)
         g_vol = O.spike_bwd(g, vol, theta, 1.0, 1.0)
-        g_cur, _ = O.li_bwd(g_vol, vol, c['d_v'])
-        O.li_bwd(g_cur, cur, c['d_i'])
+        g_cur, _ = O.li_bwd(g_vol, vol, d_v)
+        g_x, _ = O.li_bwd(g_cur, cur, d_i)
+        return spk, g_x
+
+    parity_slab = (1, slice(100, 132))
 
 
 class AlifFused(Alif):
@@ -366,13 +375,19 @@ class Rf(Workload):
             out = R._bwd(g_re, g_im, re, im, self.sin, self.cos)
         return spk, out
 
-    def cpu_step(self, n):
+    def cpu_step(self, n, sl=None):
         from oracle import slayer_oracle as O
         c, zero = self.cpu, torch.tensor([0.0])
-        re, im = O.res_fwd(c['xr'][:n], c['xi'][:n], c['sin'], c['cos'], zero, zero, 64)
-        O.cspike_fwd(re, im, 1.0, 0.0)
-        g_re, g_im = O.cspike_bwd(c['g'][:n], re, im, 1.0, 0.5, 10.0)
-        O.res_bwd(g_re, g_im, re, im, c['sin'], c['cos'])
+        xr, xi, g, sin, cos = c['xr'][:n], c['xi'][:n], c['g'][:n], c['sin'], c['cos']
+        if sl is not None:
+            xr, xi, g, sin, cos = xr[:, sl], xi[:, sl], g[:, sl], sin[sl], cos[sl]
+        re, im = O.res_fwd(xr, xi, sin, cos, zero, zero, 64)
+        spk = O.cspike_fwd(re, im, 1.0, 0.0)
+        g_re, g_im = O.cspike_bwd(g, re, im, 1.0, 0.5, 10.0)
+        out = O.res_bwd(g_re, g_im, re, im, sin, cos)
+        return spk, out[0]
+
+    parity_slab = (1, slice(500, 516))
 
 
 class RfFused(Rf):
@@ -464,18 +479,23 @@ class Synapse(Workload):
             g_x = self.conv.bwd(g_y, self.filt, 1)
         return spk, g_x
 
-    def cpu_step(self, n):
+    def cpu_step(self, n, sl=None):
         from oracle import slayer_oracle as O
         c, zero = self.cpu, torch.tensor([0.0])
-        y = O.conv_fwd(c['x'][:n], c['filt'], 1)
-        z = O.shift(y, c['delay'], 1)
+        x, g, delay = c['x'][:n], c['g'][:n], c['delay']
+        if sl is not None:
+            x, g, delay = x[:, sl], g[:, sl], delay[sl]
+        y = O.conv_fwd(x, c['filt'], 1)
+        z = O.shift(y, delay, 1)
         cur = O.li_fwd(z, c['d_i'], zero, 64)
         vol = O.li_fwd(cur, c['d_v'], zero, 64, 1.25)
-        O.spike_fwd(vol, 1.25)
-        g_vol = O.spike_bwd(c['g'][:n], vol, 1.25, 1.0, 1.0)
+        spk = O.spike_fwd(vol, 1.25)
+        g_vol = O.spike_bwd(g, vol, 1.25, 1.0, 1.0)
         g_cur, _ = O.li_bwd(g_vol, vol, c['d_v'])
         g_z, _ = O.li_bwd(g_cur, cur, c['d_i'])
-        O.conv_bwd(O.shift(g_z, -c['delay'], 1), c['filt'], 1)
+        return spk, O.conv_bwd(O.shift(g_z, -delay, 1), c['filt'], 1)
+
+    parity_slab = (1, slice(64, 96))
 
 
 class SynapseFused(Synapse):
@@ -581,6 +601,100 @@ def cpu_baseline(job, budget_s=20.0):
                        f'os.cpu_count()={os.cpu_count()}')
 
 
+def _first_two(out):
+    """(spikes or final trace, input gradient or None) of a workload's step() result."""
+    if torch.is_tensor(out):
+        return out, None
+    spk, grad = out[0], (out[1] if len(out) > 1 else None)
+    if isinstance(grad, (tuple, list)):
+        grad = grad[0]
+    return spk, grad
+
+
+def parity(job):
+    """One step on the GPU against the oracle on a slab of the same tensors (outside every timed region):
+    forward results bit for bit, the input gradient within 1e-5 of its largest magnitude."""
+    n, sl = job.parity_slab
+    spk, grad = _first_two(job.step(lambda name: _Null()))
+    torch.cuda.synchronize()
+    r_spk, r_grad = job.cpu_step(n, sl)
+    got = spk[:n, sl].cpu()
+    if got.shape != r_spk.shape or not torch.equal(got, r_spk):
+        bad = int((got != r_spk).sum()) if got.shape == r_spk.shape else -1
+        raise SystemExit(f'parity FAILED for {job.name}: {bad} forward samples differ from the oracle')
+    info = {'forward': f'bit-exact on batch[:{n}], channels {sl.start}:{sl.stop} ({r_spk.numel()} samples, '
+                       f'{int((r_spk != 0).sum())} non-zero)'}
+    if grad is not None and r_grad is not None:
+        g = grad[:n, sl].cpu().double()
+        err = float((g - r_grad.double()).abs().max())
+        scale = float(r_grad.abs().max())
+        if not err <= 1e-5 * scale:
+            raise SystemExit(f'parity FAILED for {job.name}: input gradient off by {err:.3e} (scale {scale:.3e})')
+        info['grad_input'] = f'max abs err {err:.2e} of scale {scale:.2e}'
+    return info
+
+
+def timed_median(job, iters, warmup):
+    """Median over `iters` whole steps, each between two events on the launch stream."""
+    null = lambda name: _Null()
+    for _ in range(warmup):
+        job.step(null)
+    torch.cuda.synchronize()
+    pairs = []
+    for _ in range(iters):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        job.step(null)
+        b.record()
+        pairs.append((a, b))
+    torch.cuda.synchronize()
+    times = sorted(a.elapsed_time(b) for a, b in pairs)
+    return times[len(times) // 2]
+
+
+# The other benchmark configurations, reported next to the headline in `other_configs` (unfused = the op
+# sequence of the configuration, then the fused forms with their own smaller byte counts).
+OTHER = ['cuba_fwd_small', 'cuba_fused', 'cuba_fused_lean', 'alif', 'alif_fused', 'alif_fused_lean', 'rf', 'rf_fused',
+         'synapse', 'synapse_fused', 'synapse_folded']
+
+
+def other_configs(dev, iters):
+    rows = []
+    for name in OTHER:
+        job = WORKLOADS[name](dev)
+        ok = parity(job)
+        ms = timed_median(job, iters, 20)
+        bpn = job.bytes_per_nt()
+        rows.append({'workload': name, 'shape': list(job.shape), 'bytes_per_nt': bpn, 'ms_per_step': round(ms, 4),
+                     'neuron_timesteps_per_s': job.nt / (ms * 1e-3),
+                     'frac': round(job.nt * bpn / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                     'timing': f'median of {iters} event-timed steps after 20 warm-up steps', 'parity': 'ok',
+                     'parity_detail': ok})
+        del job
+        gc.collect()
+        torch.cuda.empty_cache()
+    return rows
+
+
+def traffic_factor(kernel):
+    """HBM bytes per launch / algorithmic bytes for `kernel` from profiles/traffic_factors.txt (rocprofv3 --pmc
+    FETCH_SIZE and WRITE_SIZE runs of this script, scaled by a plain copy of known size), or None when the file
+    was measured on other kernel sources than the ones in the tree."""
+    import hashlib
+    path = os.path.join(ROOT, 'profiles', 'traffic_factors.txt')
+    if not os.path.exists(path):
+        return None, 'no profiles/traffic_factors.txt'
+    rec = json.load(open(path))
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, 'lava-dl_amd', 'csrc')
+    for f in sorted(os.listdir(csrc)):
+        if f.endswith(('.hip', '.h')):
+            h.update(open(os.path.join(csrc, f), 'rb').read())
+    if h.hexdigest()[:16] != rec.get('csrc_sha16'):
+        return None, f"stale: measured at csrc {rec.get('csrc_sha16')} ({rec.get('commit')}), tree is {h.hexdigest()[:16]}"
+    return rec['factors'].get(kernel), f"measured at commit {rec.get('commit')} (csrc {rec.get('csrc_sha16')})"
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -588,6 +702,8 @@ def main():
     ap.add_argument('--warmup', type=int, default=5)
     ap.add_argument('--workload', default='cuba', choices=sorted(WORKLOADS))
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--no-other-configs', action='store_true')
+    ap.add_argument('--iters', type=int, default=100, help='event-timed iterations behind every median')
     ap.add_argument('--calibration-copies', type=int, default=0,
                     help='also run N plain device copies of one input tensor (a kernel of known traffic, '
                          'used to scale hardware byte counters when profiling)')
@@ -607,6 +723,7 @@ def main():
         torch.empty_like(first).copy_(first)
     nt = job.nt
     null = lambda name: _Null()
+    parity_info = parity(job)        # before any timing; raises when the GPU path and the oracle disagree
 
     for _ in range(a.warmup):
         job.step(null)
@@ -618,11 +735,12 @@ def main():
         job.step(null)
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / a.steps
+    median_ms = timed_median(job, a.iters, 20)
     gc.enable()
 
     # per-kernel device time (separate pass so the event records do not perturb the headline number)
     timers = Timers()
-    for _ in range(max(3, a.steps // 2)):
+    for _ in range(a.iters):
         job.step(timers.section)
     torch.cuda.synchronize()
     op_ms = timers.median_ms()
@@ -634,7 +752,7 @@ def main():
     dom = dict(max(per_op, key=lambda r: r['ms']))
     launch = job.kernel_only(dom['op']) if hasattr(job, 'kernel_only') else None
     if launch is not None:      # the op is more than one launch: time its main kernel by itself
-        n = max(5, a.steps)
+        n = a.iters
         launch()
         begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         begin.record()                      # on the stream the kernel is launched on (torch's current stream)
@@ -647,7 +765,7 @@ def main():
         dom['achieved_GBps'], dom['frac'] = round(gbs, 1), round(gbs / HBM_PEAK_GBS, 4)
     total_bpn = job.bytes_per_nt()
     value = nt / (ms_per_step * 1e-3)
-    factor = MEASURED_TRAFFIC_FACTOR.get(dom['kernel']) if a.workload == 'cuba' else None
+    factor, factor_note = traffic_factor(dom['kernel'])
 
     out = {
         'metric': 'neuron-timesteps/sec fwd+bwd (CUBA) + % of MI355X HBM peak, 1 GPU',
@@ -656,13 +774,23 @@ def main():
         'dtype': 'int32 fixed-point state (fwd) / f32 (bwd), f32 tensors', 'data': 'synthetic',
         'config': {'workload': f'{job.name} {list(job.shape)}; {job.note}', 'bytes_per_nt': total_bpn},
         'hbm_frac_whole_step': value * total_bpn / 1e9 / HBM_PEAK_GBS,
+        'median_ms_per_step': round(median_ms, 4),
+        'median_note': f'median of {a.iters} event-timed steps after 20 warm-up steps',
+        'parity': 'ok', 'parity_detail': parity_info,
         'roofline': {'bound': 'hbm', 'kernel': dom['kernel'], 'op': dom['op'],
                      'achieved': dom['achieved_GBps'], 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
                      'frac': dom['frac'], 'kernel_ms': dom['ms'],
                      'traffic': nt * dom['bytes_per_nt'] * factor if factor else None,
-                     'traffic_unit': 'bytes per launch (rocprofv3 FETCH_SIZE x2 + WRITE_SIZE, see profiles/)'},
+                     'traffic_unit': 'bytes per launch (rocprofv3 FETCH_SIZE x2 + WRITE_SIZE, see profiles/)',
+                     'traffic_note': factor_note},
         'per_op': per_op,
     }
+    if not a.no_other_configs and a.workload == 'cuba':
+        del job
+        gc.collect()
+        torch.cuda.empty_cache()
+        out['other_configs'] = other_configs(dev, a.iters)
+        job = WORKLOADS[a.workload](dev) if not a.no_cpu_baseline else None
     if not a.no_cpu_baseline:
         out['cpu_baseline'] = cpu_baseline(job)
     print(json.dumps(out))

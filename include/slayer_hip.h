@@ -91,7 +91,8 @@ int slayer_li_fwd(float *out, const float *in, const float *decay, const float *
  * grad_decay[j] = sum over the neurons that use decay j of sum_t grad_in[t+1] * out[t].
  * grad_decay (num_decays floats) may be NULL to skip the parameter gradient.
  * workspace: M + 64 * num_decays floats of scratch (per-neuron partial sums, then slice sums),
- * required iff grad_decay != NULL; its contents on return are unspecified. */
+ * required iff grad_decay != NULL; its contents on return are unspecified.  Given without grad_decay it
+ * receives the per-neuron sums (workspace[m] = sum_t grad_in[m][t+1] * out[m][t]) and nothing is reduced. */
 int slayer_li_bwd(float *grad_in, float *grad_decay, const float *grad_out, const float *out,
                   const float *decay, float *workspace,
                   int64_t M, int64_t neurons_per_batch, int64_t num_decays,

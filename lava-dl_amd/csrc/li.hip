@@ -215,11 +215,11 @@ extern "C" int slayer_li_bwd(float* grad_in, float* grad_decay, const float* gra
     if (M > 0 && T > 0) {
         if (!grad_in || !grad_out || !out || !decay) return SLAYER_ENULL;
         if (bwd_scan_usable(M, neurons_per_batch, T) && aligned16(grad_in) && aligned16(grad_out) && aligned16(out)) {
-            if (int e = launch_li_bwd_scan(grad_in, grad_decay ? workspace : nullptr, grad_out, out, decay, M,
+            if (int e = launch_li_bwd_scan(grad_in, workspace, grad_out, out, decay, M,
                                            neurons_per_batch, num_decays, T, (hipStream_t)stream))
                 return e;
         } else {
-            LiBwd::Params p{{grad_out, out}, {grad_in}, decay, grad_decay ? workspace : nullptr,
+            LiBwd::Params p{{grad_out, out}, {grad_in}, decay, workspace,
                             neurons_per_batch, num_decays};
             if (int e = launch_stream<LiBwd>(p, M, T, (hipStream_t)stream)) return e;
         }

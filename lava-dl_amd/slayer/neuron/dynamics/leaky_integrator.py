@@ -62,7 +62,9 @@ def _fwd(input, decay, state, threshold, w_scale, entry='slayer_li_fwd'):
     return output
 
 
-def _bwd(grad_output, output, decay, need_decay_grad=True):
+def _bwd(grad_output, output, decay, need_decay_grad=True, per_neuron_sums=False):
+    """(grad_input, grad_decay).  ``per_neuron_sums`` (without ``need_decay_grad``) returns the per-neuron sums
+    the decay gradient is reduced from in place of it: the main kernel alone, no reduction launches."""
     dev = N.require_gpu(grad_output, output, decay)
     grad_output, output, decay = grad_output.contiguous(), output.contiguous(), decay.contiguous()
     M, T = N.rows_and_steps(grad_output)
@@ -70,12 +72,13 @@ def _bwd(grad_output, output, decay, need_decay_grad=True):
     grad_decay = workspace = None
     if need_decay_grad:
         grad_decay = torch.empty(decay.numel(), dtype=torch.float32, device=dev)
+    if need_decay_grad or per_neuron_sums:
         workspace = torch.empty(M + 64 * decay.numel(), dtype=torch.float32, device=dev)
     with torch.cuda.device(dev):
         N.check(N.lib().slayer_li_bwd(
             N.ptr(grad_input), N.ptr(grad_decay), N.ptr(grad_output), N.ptr(output), N.ptr(decay),
             N.ptr(workspace), M, N.neurons_per_batch(grad_output), decay.numel(), T, N.stream_handle()))
-    return grad_input, grad_decay
+    return grad_input, (workspace[:M] if per_neuron_sums and not need_decay_grad else grad_decay)
 
 
 def _bwd_naive(grad_output, decay):
