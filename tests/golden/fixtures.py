@@ -116,3 +116,15 @@ def reference_neuron_vectors():
         case['grad_in'] = [torch.tensor(pick[f'grad_in{i}']) for i in (0, 1) if f'grad_in{i}' in pick]
         cases.append(case)
     return cases
+
+
+def reference_delay_vectors():
+    """Vectors written by make_reference_delay_vectors.py from the reference's own `axon.Delay` module (forward,
+    gradient of the input, gradient of the delays) and per-neuron `shift` at sampling times other than 1 (CPU branch).
+    Returns {case name: {key: tensor}}."""
+    z = np.load(os.path.join(HERE, 'reference_delay_vectors.npz'))
+    cases = {}
+    for k in z.files:
+        name, key = k.split('/', 1)
+        cases.setdefault(name, {})[key] = torch.tensor(z[k])
+    return cases

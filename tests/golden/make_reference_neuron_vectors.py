@@ -1,11 +1,12 @@
-"""Input/output vectors of the reference's neuron classes that no fixture of the reference pins:
-alif, adrf, adrf_iz and sigma_delta (the CUBA, RF and RF_IZ neurons are pinned by the netx fixtures).
+"""Input/output vectors of the reference's neuron classes: alif, adrf, adrf_iz and sigma_delta, which no fixture
+of the reference pins, and cuba, rf and rf_iz, whose dynamics the netx fixtures pin but whose class-level behaviour
+(surrogate constants, carried states over two calls, graded spikes, per-channel parameters) they do not.
 
 Run in the build container only (it reads /root/reference, which never travels):
 
     python tests/golden/make_reference_neuron_vectors.py
 
-What is imported: `neuron/{base,alif,adrf,adrf_iz,sigma_delta}.py` of the reference and what they import
+What is imported: `neuron/{base,cuba,alif,rf,rf_iz,adrf,adrf_iz,sigma_delta}.py` of the reference and what they import
 (`neuron/dynamics/*.py`, `spike/`, `axon/`, `dendrite/`, `utils/{quantize,int_utils,utils}.py`, `utils/time/`,
 `utils/filter/`, `jitconfig.py`), under empty stand-in packages for `slayer`, `slayer.utils`, `slayer.neuron` and
 `slayer.neuron.dynamics`, so that the package `__init__` files that pull in h5py / matplotlib / lava do not run.
@@ -48,7 +49,7 @@ def load_reference_neurons():
     quantize = importlib.import_module('lava.lib.dl.slayer.utils.quantize')
     utils.quantize, utils.QUANTIZE_MODE = quantize.quantize, quantize.MODE       # what utils/__init__.py re-exports
     return {name: importlib.import_module('lava.lib.dl.slayer.neuron.' + name)
-            for name in ('alif', 'adrf', 'adrf_iz', 'sigma_delta')}
+            for name in ('alif', 'adrf', 'adrf_iz', 'sigma_delta', 'cuba', 'rf', 'rf_iz')}
 
 
 def events(gen, shape, p, amp):
@@ -74,6 +75,13 @@ CASES = [
     ('sigma_delta_relu', 'sigma_delta', dict(threshold=0.1, activation='relu'), False, (0.5, 0.3)),
     # cum_error=True is left out: that branch of the reference (axon/delta.py:39, `1 - (bool tensor)`) raises
     # under the installed torch
+    ('cuba_shared', 'cuba', dict(threshold=0.5, current_decay=0.25, voltage_decay=0.1), False, (0.3, 1.0)),
+    ('cuba_graded_channel', 'cuba', dict(threshold=0.6, current_decay=[0.1, 0.4], voltage_decay=[0.05, 0.2],
+                                         shared_param=False, graded_spike=True, scale=32), False, (0.4, 1.5)),
+    ('rf_shared', 'rf', dict(threshold=0.4, period=8, decay=0.08), True, (0.4, 1.0)),
+    ('rf_channel', 'rf', dict(threshold=0.5, period=[5, 20], decay=[0.02, 0.2], shared_param=False), True, (0.4, 1.0)),
+    ('rf_iz_shared', 'rf_iz', dict(threshold=0.4, period=8, decay=0.08), True, (0.4, 1.0)),
+    ('rf_iz_graded', 'rf_iz', dict(threshold=0.5, period=12, decay=0.05, graded_spike=True), True, (0.5, 1.2)),
 ]
 ACTIVATIONS = {'relu': torch.relu}
 SHAPE = (3, 6, 48)

@@ -202,3 +202,32 @@ def test_oracle_chain_equals_the_reference_sigma_delta_neuron():
         st = c['states'][call]
         assert torch.allclose(pre_sigma, st['sigma.pre_state'], rtol=1e-5, atol=1e-6)      # summation order
         assert torch.allclose(res, st['delta.residual_state'], rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize('name', ['delay_nct', 'delay_nchwt', 'delay_ts2'])
+def test_oracle_delay_against_the_reference_delay_module(name):
+    """tests/golden/reference_delay_vectors.npz: the reference's own axon.Delay (CPU branch).  Its per-neuron shift
+    divides by the sampling time twice (utils/time/shift.py:82,56), so its result for a delay d is the oracle's (one
+    division, like the CUDA kernel) for d / Ts; at Ts = 1 the two coincide."""
+    c = G.reference_delay_vectors()[name]
+    ts, _, grad_scale = (float(v) for v in c['cfg'])
+    d = c['delay'] / ts
+    if c['in'].dim() > 3:
+        tile = list(c['in'].shape[1:-1])
+        tile[0] = 1
+        d = d.reshape((-1,) + (1,) * (len(tile) - 1)).repeat(tile)
+    assert torch.equal(O.delay_fwd(c['in'], d, ts), c['out'])
+    g_in, g_d = O.delay_bwd(c['grad_out'], c['out'], d, grad_scale, ts)
+    assert torch.equal(g_in, c['grad_in'])
+    if c['in'].dim() == 3:
+        assert torch.allclose(g_d, c['grad_delay'], rtol=1e-5, atol=1e-5)
+    # a wrong sign of the shift back, or a shift of the output instead of the gradient, fails
+    assert not torch.equal(O.shift(c['grad_out'], d, ts), c['grad_in'])
+
+
+@pytest.mark.parametrize('name', ['shift_ts2', 'shift_ts_half'])
+def test_oracle_shift_against_the_reference_at_other_sampling_times(name):
+    c = G.reference_delay_vectors()[name]
+    ts = float(c['ts'])
+    assert torch.equal(O.shift(c['in'], c['shift'] / ts, ts), c['out'])
+    assert not torch.equal(O.shift(c['in'], c['shift'], ts), c['out'])     # one division is a different result
