@@ -1,6 +1,6 @@
 """Benchmark of the SLAYER neuron-dynamics hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cuba|cuba_fused|cuba_fused_lean|cuba_inference|cuba_fwd_small|alif|alif_fused|alif_fused_lean|rf|rf_fused|rf_fused_lean|rf_inference|synapse|synapse_fused|synapse_folded|synapse_delay_grad]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cuba|cuba_fused|cuba_fused_lean|cuba_inference|cuba_fwd_small|alif|alif_fused|alif_fused_lean|rf|rf_fused|rf_fused_lean|rf_inference|synapse|synapse_fused|synapse_folded|synapse_delay_grad|dense_synapse]
 
 A step is one pass of the workload's op sequence over one batch of synthetic input that is already
 resident in HBM (outputs come from torch's caching allocator inside the timed region).  The default
@@ -573,7 +573,46 @@ class SynapseDelayGrad(SynapseFused):
         return spk, g_x, g_delay
 
 
-WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fused_lean': CubaFusedLean, 'cuba_inference': CubaInference, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'alif_fused': AlifFused, 'alif_fused_lean': AlifFusedLean, 'rf': Rf, 'rf_fused': RfFused, 'rf_fused_lean': RfFusedLean, 'rf_inference': RfInference, 'synapse': Synapse, 'synapse_fused': SynapseFused, 'synapse_folded': SynapseFolded, 'synapse_delay_grad': SynapseDelayGrad}
+class DenseSynapse(Workload):
+    """Dense synapse (the reference's 1x1x1 conv3d over [N, C, 1, 1, T], synapse/layer.py:144-175, written as the
+    batched GEMM it is) feeding the fused CUBA kernel, forward only: the kernel list of this workload shows what runs
+    between the GEMM and the neuron.  (`F.conv3d` itself goes through MIOpen here, which transposes to channels-last
+    and back around its kernel; `torch.matmul` does not.)"""
+    name = 'Dense synapse (batched GEMM) -> fused CUBA neuron, forward'
+    shape = (32, 256, 1500)
+    ops = [('dense_gemm', 'torch.matmul (GEMM, outside this library)', 8), ('cuba_fwd', 'stream_kernel<CubaFwd>', 8)]
+    note = '256 -> 256 neurons, input Bernoulli(0.03), weights N(0, 0.3) on the 2/64 grid, CUBA decays 1024/128, threshold 1.25'
+
+    def __init__(self, dev):
+        super().__init__(dev, 1005)
+        from lava_dl_amd.slayer.neuron.dynamics import cuba_fused
+        self.F = cuba_fused
+        g = self.gen
+        self.put(s=(torch.rand(self.shape, generator=g) < 0.03).float(),
+                 wgt=(torch.randn(256, 256, generator=g) * 0.3 * 32).round() / 32,
+                 d_i=torch.tensor([1024.0]), d_v=torch.tensor([128.0]))
+
+    def step(self, t):
+        with t('dense_gemm'):
+            z = torch.matmul(self.wgt, self.s)           # [256, C] @ [N, C, T] -> [N, 256, T], time innermost
+        with t('cuba_fwd'):
+            out = self.F._fwd(z, self.d_i, self.d_v, self.zero, self.zero, 64, 1.25, False, 1, True, True)
+        return out[2]
+
+    def cpu_step(self, n, sl=None):
+        from oracle import slayer_oracle as O
+        c, zero = self.cpu, torch.tensor([0.0])
+        z = torch.matmul(c['wgt'], c['s'][:n])
+        if sl is not None:
+            z = z[:, sl]
+        cur = O.li_fwd(z, c['d_i'], zero, 64)
+        vol = O.li_fwd(cur, c['d_v'], zero, 64, 1.25)
+        return O.spike_fwd(vol, 1.25), None
+
+    parity_slab = (1, slice(32, 64))
+
+
+WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fused_lean': CubaFusedLean, 'cuba_inference': CubaInference, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'alif_fused': AlifFused, 'alif_fused_lean': AlifFusedLean, 'rf': Rf, 'rf_fused': RfFused, 'rf_fused_lean': RfFusedLean, 'rf_inference': RfInference, 'synapse': Synapse, 'synapse_fused': SynapseFused, 'synapse_folded': SynapseFolded, 'synapse_delay_grad': SynapseDelayGrad, 'dense_synapse': DenseSynapse}
 
 
 def cpu_baseline(job, budget_s=20.0):

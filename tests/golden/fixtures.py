@@ -34,6 +34,17 @@ def dense_lif():
                 expected=_unpack(z['out_bits'], T)[:, 1:])
 
 
+def dense_lif_block():
+    """The same dense LIF block before its synapse: dict(spikes=[1,200,T] 0/1 input, weight=[256,200] synaptic
+    weights in units of the state scale (integer weight * 64 / 4096), then as dense_lif())."""
+    z = np.load(os.path.join(HERE, 'netx_dense_lif.npz'))
+    T = int(z['num_steps'])
+    fx = dense_lif()
+    fx['spikes'] = torch.tensor(_unpack(z['in_bits'], T), dtype=torch.float32).reshape(1, -1, T)
+    fx['weight'] = torch.tensor(z['weight'].astype(np.float64) * 64 / W_SCALE, dtype=torch.float32)
+    return fx
+
+
 def complex_dense_rf():
     """RF dense block: vth=25, period=11, alpha=0.05 (no reset, phase spike)."""
     z = np.load(os.path.join(HERE, 'netx_complex_dense_rf.npz'))

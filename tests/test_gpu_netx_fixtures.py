@@ -85,3 +85,41 @@ def test_rf_neuron_forward_on_the_complex_dense_fixture(slayer, form):
         assert torch.isfinite(xr.grad).all() and torch.isfinite(xi.grad).all()
     got = spk[0].detach().cpu().numpy().astype(np.int64)[:, :fx['expected'].shape[1]]
     assert int((got != fx['expected']).sum()) == 0 and got.sum() > 40000
+
+
+def test_dense_synapse_output_feeds_the_fused_neuron_without_a_layout_pass(slayer):
+    """The reference's Dense synapse is a 1x1x1 `conv3d` over [N, C_in, 1, 1, T] (synapse/layer.py:144-175), i.e. the
+    batched GEMM weight @ x over [N, C_in, T].  Its output [N, C_out, T] is contiguous with time innermost, which is
+    the layout the kernels take: the fused neuron kernel receives the GEMM's own buffer (no transpose, no copy in
+    between).  Checked on the dense LIF block of the netx fixture, synapse included, for both ways of writing it."""
+    import torch.nn.functional as F
+    from lava_dl_amd.slayer.neuron.dynamics import cuba_fused
+    fx = G.dense_lif_block()
+    s, w = fx['spikes'].to(dev()), fx['weight'].to(dev())
+    z_conv = F.conv3d(s.reshape(1, s.shape[1], 1, 1, -1), w.reshape(w.shape[0], w.shape[1], 1, 1, 1))
+    z_mm = torch.matmul(w, s)
+    assert z_conv.is_contiguous() and z_conv.shape == (1, 256, 1, 1, s.shape[-1])
+    assert z_mm.is_contiguous() and z_mm.shape == (1, 256, s.shape[-1])
+    assert torch.equal(z_mm.cpu(), fx['x']), 'synaptic input differs from weight @ spikes'
+    assert torch.equal(z_conv.reshape(z_mm.shape), z_mm)
+    library = cuba_fused.N.lib()
+    seen = []
+
+    class Spy:
+        def __getattr__(self, name):
+            fn = getattr(library, name)
+            if name != 'slayer_cuba_fwd':
+                return fn
+            return lambda *a: (seen.append(a[5]), fn(*a))[1]         # a[5]: the input pointer handed to the kernel
+    real_lib = cuba_fused.N.lib
+    cuba_fused.N.lib = lambda: Spy()
+    try:
+        for z in (z_mm, z_conv):
+            n = _cuba(slayer, fx, trainable=False)
+            with torch.no_grad():
+                spk = n(z)
+            got = spk.reshape(256, -1).cpu().numpy().astype(np.int64)[:, :fx['expected'].shape[1]]
+            assert int((got != fx['expected']).sum()) == 0 and got.sum() == 1826
+    finally:
+        cuba_fused.N.lib = real_lib
+    assert seen == [z_mm.data_ptr(), z_conv.data_ptr()], 'the kernel did not read the GEMM output in place'
