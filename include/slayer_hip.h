@@ -37,7 +37,7 @@
 extern "C" {
 #endif
 
-#define SLAYER_ABI_VERSION 2
+#define SLAYER_ABI_VERSION 3
 
 #define SLAYER_EINVAL   (-1)   /* inconsistent sizes (M, T, neurons_per_batch, num_params, ...) */
 #define SLAYER_ENULL    (-2)   /* a required pointer is NULL */
@@ -379,32 +379,55 @@ int slayer_alif_bwd(float *grad_in, float *grad_i_decay, float *grad_v_decay,
                     int64_t M, int64_t neurons_per_batch, int64_t num_i_decays, int64_t num_v_decays,
                     int64_t T, const slayer_delays *delays, void *stream);
 
-/* ---- recurrent CUBA layer --------------------------------------------------------------------- */
+/* ---- recurrent layer (CUBA or ALIF neurons) ---------------------------------------------------- */
 
-/* The time loop of utils/recurrent.py:45-81 (CustomRecurrent.forward) for a CUBA neuron with binary
- * spikes, in one launch:  feedback[t] = R s[t-1],  s[t] = neuron(z[t] + feedback[t]),  s[-1] = 0.
+/* The time loop of utils/recurrent.py:45-81 (CustomRecurrent.forward) for a CUBA neuron
+ * (neuron/cuba.py:356-421 called one step at a time), in one launch:
+ *   feedback[t] = R s[t-1],  s[t] = neuron(z[t] + feedback[t]),  s[-1] = 0.
  * z, spk_out, vol_out: [N][C][T]; rec_t = R^T followed by a row of zeros, [C + 1][C] (row j = the
  * weights from neuron j; the kernel pads its spike lists with the index of the zero row);
  * decays [1] or [C]; states [1] or [N*C] are the neuron's persistent current / voltage before the
  * first step.  vol_out is the voltage trace the backward pass needs; cur_last_out / vol_last_out
- * ([N*C]) are the current and the (un-reset) voltage of the last step.  C <= 1024.
+ * ([N*C]) are the current and the (un-reset) voltage of the last step.  graded != 0: a spike carries
+ * voltage / spike_scale instead of 1 (spike/spike.py:77-87), into spk_out and into the feedback.
+ * C <= 1024.
  * Equal to calling the neuron one step at a time (the state between two calls makes the same float32
  * round trip) whenever the feedback sums are exact in float32, e.g. with quantised weights. */
 int slayer_cuba_recurrent_fwd(float *spk_out, float *vol_out, float *cur_last_out, float *vol_last_out,
                               const float *z, const float *rec_t,
                               const float *i_decay, const float *v_decay,
                               const float *i_state, const float *v_state,
-                              float spike_threshold, int w_scale,
+                              float spike_threshold, int graded, float spike_scale, int w_scale,
                               int64_t N, int64_t C, int64_t num_i_decays, int64_t num_v_decays,
                               int64_t num_i_states, int64_t num_v_states, int64_t T, void *stream);
 
+/* The same loop for an ALIF neuron (neuron/alif.py:383-623 called one step at a time): a step decays the
+ * refractory state and the threshold (towards th0), spikes where voltage >= threshold + refractory, and hands
+ * threshold + spike * th_step, refractory + 2 * spike * threshold and the voltage (no reset) to the next step
+ * as float32 (neuron/dynamics/adaptive_threshold.py:133-172).  theta_out [N][C][T] receives threshold +
+ * refractory of every step (the backward pass needs it); th_last_out / ref_last_out ([N*C]) the decayed
+ * threshold and refractory state of the last step, before that step's spike is added.  th_step is the
+ * neuron's threshold step in state units (float), th0_scaled = base threshold * w_scale.  Otherwise as above. */
+int slayer_alif_recurrent_fwd(float *spk_out, float *vol_out, float *theta_out,
+                              float *cur_last_out, float *vol_last_out, float *th_last_out, float *ref_last_out,
+                              const float *z, const float *rec_t,
+                              const float *i_decay, const float *v_decay, const float *th_decay, const float *ref_decay,
+                              const float *i_state, const float *v_state, const float *th_state, const float *ref_state,
+                              float th_step, int64_t th0_scaled, int graded, float spike_scale, int w_scale,
+                              int64_t N, int64_t C,
+                              int64_t num_i_decays, int64_t num_v_decays, int64_t num_th_decays, int64_t num_ref_decays,
+                              int64_t num_i_states, int64_t num_v_states, int64_t num_th_states, int64_t num_ref_states,
+                              int64_t T, void *stream);
+
 /* Backward of the loop as utils/recurrent.py:83-112 differentiates it (the carried neuron state is a
  * constant, a step contributes its spike surrogate, the gradient reaches step t-1 through R):
- * grad_z[t] = surrogate(voltage[t]) * (grad_spikes[t] + (grad_z[t+1] R));  rec = R, [C][C].
+ * grad_z[t] = surrogate(voltage[t] - threshold[t]) * (grad_spikes[t] + (grad_z[t+1] R));  rec = R, [C][C].
+ * theta: [N][C][T] thresholds of an ALIF layer (theta_out above), or NULL for the constant spike_threshold.
+ * graded selects the surrogate of graded spikes (spike/spike.py:7-19,113-126).
  * The gradient of R is the product grad_z[:, :, 1:] x spikes[:, :, :-1] and is left to the caller. */
-int slayer_cuba_recurrent_bwd(float *grad_z, const float *grad_spikes, const float *voltage, const float *rec,
-                              float spike_threshold, float tau_rho, float scale_rho,
-                              int64_t N, int64_t C, int64_t T, void *stream);
+int slayer_recurrent_bwd(float *grad_z, const float *grad_spikes, const float *voltage, const float *theta,
+                         const float *rec, float spike_threshold, float tau_rho, float scale_rho, int graded,
+                         int64_t N, int64_t C, int64_t T, void *stream);
 
 /* ---- cross-check implementations (debug mode) ------------------------------------------------ */
 

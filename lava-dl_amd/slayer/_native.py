@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # SLAYER_HIP_LIB points at an alternative build of the same library (e.g. a tuning build)
 LIB_PATH = os.environ.get('SLAYER_HIP_LIB') or os.path.join(_HERE, 'libslayer_hip.so')
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _lib = None
 _lib_lock = threading.Lock()       # forward runs on the user thread, backward on an autograd thread
@@ -65,8 +65,9 @@ _SIGNATURES = {
     'slayer_rf_bwd': (_INT, [_P] * 9 + [_F, _F, _F, _INT, _P] + [_I64] * 4 + [_DP, _P]),
     'slayer_alif_fwd': (_INT, [_P] * 17 + [_I64, _I64, _INT, _F, _INT] + [_I64] * 11 + [_DP, _P]),
     'slayer_alif_bwd': (_INT, [_P] * 9 + [_F, _F, _INT, _P] + [_I64] * 5 + [_DP, _P]),
-    'slayer_cuba_recurrent_fwd': (_INT, [_P] * 10 + [_F, _INT] + [_I64] * 7 + [_P]),
-    'slayer_cuba_recurrent_bwd': (_INT, [_P] * 4 + [_F, _F, _F] + [_I64] * 3 + [_P]),
+    'slayer_cuba_recurrent_fwd': (_INT, [_P] * 10 + [_F, _INT, _F, _INT] + [_I64] * 7 + [_P]),
+    'slayer_alif_recurrent_fwd': (_INT, [_P] * 17 + [_F, _I64, _INT, _F, _INT] + [_I64] * 11 + [_P]),
+    'slayer_recurrent_bwd': (_INT, [_P] * 5 + [_F, _F, _F, _INT] + [_I64] * 3 + [_P]),
     'slayer_li_fwd_naive': (_INT, [_P, _P, _P, _P, _D, _INT, _I64, _I64, _I64, _I64, _I64, _P]),
     'slayer_li_bwd_naive': (_INT, [_P, _P, _P, _I64, _I64, _I64, _I64, _P]),
     'slayer_ath_fwd_naive': (_INT, [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _INT,

@@ -1,8 +1,9 @@
 """Recurrent spiking layer: ``s[t] = neuron(z[t] + R s[t-1])``.
 
 Interface of lava.lib.dl.slayer.utils.recurrent (utils/recurrent.py:7-112 in the reference).
-For a CUBA neuron with binary spikes on the GPU the whole time loop is one kernel launch per
-direction (slayer_cuba_recurrent_fwd / _bwd); any other neuron runs the reference's loop of
+For a CUBA or an ALIF neuron on the GPU (binary or graded spikes, up to 1024 neurons per sample) the
+whole time loop is one kernel launch per direction (slayer_cuba_recurrent_fwd /
+slayer_alif_recurrent_fwd / slayer_recurrent_bwd); any other neuron runs the reference's loop of
 one-step neuron calls.
 """
 import torch
@@ -42,10 +43,9 @@ def custom_recurrent_ground_truth_2(z, neuron, recurrent_synapse):
 
 
 def _fusable(z, neuron):
-    from ..neuron import cuba
-    return (type(neuron) is cuba.Neuron and z.is_cuda and z.dim() == 3 and z.dtype == torch.float32
-            and neuron.norm is None and neuron.drop is None and not neuron.graded_spike
-            and neuron.persistent_state and z.shape[1] <= 1024)
+    from ..neuron import alif, cuba
+    return (type(neuron) in (cuba.Neuron, alif.Neuron) and z.is_cuda and z.dim() == 3 and z.dtype == torch.float32
+            and neuron.norm is None and neuron.drop is None and neuron.persistent_state and z.shape[1] <= 1024)
 
 
 def custom_recurrent(z, neuron, recurrent_synapse):
@@ -55,7 +55,7 @@ def custom_recurrent(z, neuron, recurrent_synapse):
     neuron carries from one step to the next is treated as a constant."""
     recurrent_mat = _recurrent_matrix(recurrent_synapse)
     if _fusable(z, neuron):
-        return _FusedCubaRecurrent.apply(z, neuron, recurrent_mat)
+        return _FusedRecurrent.apply(z, neuron, recurrent_mat)
     return CustomRecurrent.apply(z, neuron, recurrent_mat)
 
 
@@ -101,46 +101,67 @@ def _weight_gradient(grad_z, x):
     return torch.matmul(grad_output, spikes_in)
 
 
-class _FusedCubaRecurrent(torch.autograd.Function):
+class _FusedRecurrent(torch.autograd.Function):
+    """The whole time loop of a CUBA or an ALIF layer as one launch per direction."""
+
     @staticmethod
     def forward(ctx, z, neuron, recurrent_mat):
-        from ..neuron import cuba
-        from ..neuron.dynamics import leaky_integrator
+        from ..neuron import alif, cuba
+        from ..neuron.dynamics import adaptive_threshold, leaky_integrator
         dev = N.require_gpu(z)
         z = z.detach().contiguous()
         neuron._prepare(z)
         n, c, t = z.shape
         rec = recurrent_mat.detach().to(dev).float().contiguous()
         rec_t = torch.cat([rec.transpose(0, 1), rec.new_zeros(1, c)], dim=0).contiguous()   # + the zero row
-        i_decay = neuron._q('current_decay').detach().contiguous()
-        v_decay = neuron._q('voltage_decay').detach().contiguous()
-        i_state, v_state = neuron.current_state.contiguous(), neuron.voltage_state.contiguous()
+        is_alif = type(neuron) is alif.Neuron
+        names = ('current', 'voltage') + (('threshold', 'refractory') if is_alif else ())
+        decays = [neuron._q(f'{k}_decay').detach().contiguous() for k in names]
+        states = [getattr(neuron, f'{k}_state').contiguous() for k in names]
         spk, vol = torch.empty_like(z), torch.empty_like(z)
-        cur_last, vol_last = torch.empty_like(i_state), torch.empty_like(v_state)
-        threshold = neuron.threshold + neuron.threshold_eps
+        theta = torch.empty_like(z) if is_alif else None
+        last = [torch.empty_like(s) for s in states]
+        graded = 1 if neuron.graded_spike else 0
         with torch.cuda.device(dev):
-            N.check(N.lib().slayer_cuba_recurrent_fwd(
-                N.ptr(spk), N.ptr(vol), N.ptr(cur_last), N.ptr(vol_last), N.ptr(z), N.ptr(rec_t),
-                N.ptr(i_decay), N.ptr(v_decay), N.ptr(i_state), N.ptr(v_state),
-                float(threshold), int(neuron.s_scale), n, c, i_decay.numel(), v_decay.numel(),
-                i_state.numel(), v_state.numel(), t, N.stream_handle()))
-        neuron.current_state = cur_last
-        neuron.voltage_state = leaky_integrator.persistent_state(vol_last, spk[..., -1]).detach().clone()
-        ctx.save_for_backward(vol, spk, rec)
-        ctx.cfg = (float(threshold), float(neuron.tau_rho * cuba.TAU_RHO_MULT),
-                   float(neuron.scale_rho * cuba.SCALE_RHO_MULT))
+            if is_alif:
+                threshold = 0.0
+                N.check(N.lib().slayer_alif_recurrent_fwd(
+                    N.ptr(spk), N.ptr(vol), N.ptr(theta), *[N.ptr(x) for x in last], N.ptr(z), N.ptr(rec_t),
+                    *[N.ptr(d) for d in decays], *[N.ptr(s) for s in states],
+                    float(neuron.threshold_step), int(neuron.threshold * neuron.s_scale), graded, 1.0,
+                    int(neuron.s_scale), n, c, *[d.numel() for d in decays], *[s.numel() for s in states], t,
+                    N.stream_handle()))
+            else:
+                threshold = neuron.threshold + neuron.threshold_eps
+                N.check(N.lib().slayer_cuba_recurrent_fwd(
+                    N.ptr(spk), N.ptr(vol), *[N.ptr(x) for x in last], N.ptr(z), N.ptr(rec_t),
+                    *[N.ptr(d) for d in decays], *[N.ptr(s) for s in states],
+                    float(threshold), graded, 1.0, int(neuron.s_scale), n, c,
+                    *[d.numel() for d in decays], *[s.numel() for s in states], t, N.stream_handle()))
+        neuron.current_state = last[0]
+        if is_alif:
+            neuron.voltage_state = last[1]
+            neuron.refractory_state = adaptive_threshold.persistent_ref_state(last[3], spk[..., -1], last[2]).detach()
+            neuron.threshold_state = adaptive_threshold.persistent_th_state(
+                last[2], spk[..., -1], neuron.threshold_step).detach()
+        else:
+            neuron.voltage_state = leaky_integrator.persistent_state(last[1], spk[..., -1]).detach().clone()
+        mult = alif if is_alif else cuba
+        ctx.save_for_backward(vol, spk, rec, *([theta] if is_alif else []))
+        ctx.cfg = (float(threshold), float(neuron.tau_rho * mult.TAU_RHO_MULT),
+                   float(neuron.scale_rho * mult.SCALE_RHO_MULT), graded)
         return spk
 
     @staticmethod
     def backward(ctx, grad_x):
-        vol, spk, rec = ctx.saved_tensors
-        threshold, tau_rho, scale_rho = ctx.cfg
+        vol, spk, rec, *theta = ctx.saved_tensors
+        threshold, tau_rho, scale_rho, graded = ctx.cfg
         dev = N.require_gpu(grad_x)
         grad_x = grad_x.contiguous()
         n, c, t = grad_x.shape
         grad_z = torch.empty_like(grad_x)
         with torch.cuda.device(dev):
-            N.check(N.lib().slayer_cuba_recurrent_bwd(
-                N.ptr(grad_z), N.ptr(grad_x), N.ptr(vol), N.ptr(rec), threshold, tau_rho, scale_rho,
-                n, c, t, N.stream_handle()))
+            N.check(N.lib().slayer_recurrent_bwd(
+                N.ptr(grad_z), N.ptr(grad_x), N.ptr(vol), N.ptr(theta[0]) if theta else None, N.ptr(rec),
+                threshold, tau_rho, scale_rho, graded, n, c, t, N.stream_handle()))
         return grad_z, None, _weight_gradient(grad_z, spk)

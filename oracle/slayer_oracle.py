@@ -509,11 +509,12 @@ def sigma_fwd(x, pre_state=None):
 
 
 # --------------------------------------------------------------------------- recurrent layer
-def recurrent_cuba_fwd(z, rec, i_decay, v_decay, i_state, v_state, w_scale, threshold):
+def recurrent_cuba_fwd(z, rec, i_decay, v_decay, i_state, v_state, w_scale, threshold, graded=False):
     """Recurrent CUBA layer, S/utils/recurrent.py:45-81 with the CUBA neuron called one step at a
     time (S/neuron/cuba.py:356-421, persistent state): feedback = s[t-1] @ R^T, the neuron's current
     and voltage LI run one step each from the carried float32 states, a spike resets the carried
-    voltage.  z: [N, C, T]; rec = R [C, C].  Returns (spikes, voltage, current_state, voltage_state)."""
+    voltage; a graded spike carries the voltage (scale 1, S/neuron/cuba.py:403-409).
+    z: [N, C, T]; rec = R [C, C].  Returns (spikes, voltage, current_state, voltage_state)."""
     spikes = torch.zeros_like(z)
     voltage = torch.zeros_like(z)
     cur_state = _full_state(i_state, z[..., :1])
@@ -524,7 +525,7 @@ def recurrent_cuba_fwd(z, rec, i_decay, v_decay, i_state, v_state, w_scale, thre
         dend = (z[..., t] + torch.matmul(s, rec_t)).unsqueeze(-1)
         cur = li_fwd(dend, i_decay, cur_state, w_scale)
         vol = li_fwd(cur, v_decay, vol_state, w_scale, threshold)
-        spk = spike_fwd(vol, threshold)
+        spk = spike_fwd(vol, threshold, graded, 1)
         cur_state = cur[..., -1]
         vol_state = li_persistent_state(vol[..., -1], spk[..., -1])
         s = spk[..., 0]
@@ -533,15 +534,43 @@ def recurrent_cuba_fwd(z, rec, i_decay, v_decay, i_state, v_state, w_scale, thre
     return spikes, voltage, cur_state, vol_state
 
 
-def recurrent_cuba_bwd(grad_x, spikes, voltage, rec, threshold, tau_rho, scale_rho):
+def recurrent_alif_fwd(z, rec, decays, states, th_step, th0, w_scale, graded=False):
+    """Recurrent ALIF layer: the same loop with the ALIF neuron called one step at a time
+    (S/neuron/alif.py:383-623, persistent state).  decays / states = (current, voltage, threshold,
+    refractory).  The voltage is not reset; a spike adds th_step to the carried threshold and twice the
+    threshold to the carried refractory state (DYN/adaptive_threshold.py:133-172).
+    Returns (spikes, voltage, theta = threshold + refractory, states after the last step)."""
+    spikes, voltage, theta = torch.zeros_like(z), torch.zeros_like(z), torch.zeros_like(z)
+    cur_state, vol_state, th_state, ref_state = (_full_state(x, z[..., :1]) for x in states)
+    s = torch.zeros(z.shape[:-1])
+    rec_t = rec.transpose(0, 1)
+    for t in range(z.shape[-1]):
+        dend = (z[..., t] + torch.matmul(s, rec_t)).unsqueeze(-1)
+        cur = li_fwd(dend, decays[0], cur_state, w_scale)
+        vol = li_fwd(cur, decays[1], vol_state, w_scale)
+        th, ref = ath_fwd(vol, ref_state, decays[3], th_state, decays[2], th_step, th0, w_scale)
+        spk = spike_fwd(vol, th + ref, graded, 1)
+        cur_state, vol_state = cur[..., -1], vol[..., -1]
+        ref_state = ath_persistent_ref_state(ref[..., -1], spk[..., -1], th[..., -1])
+        th_state = ath_persistent_th_state(th[..., -1], spk[..., -1], th_step)
+        s = spk[..., 0]
+        spikes[..., t] = s
+        voltage[..., t] = vol[..., 0]
+        theta[..., t] = (th + ref)[..., 0]
+    return spikes, voltage, theta, (cur_state, vol_state, th_state, ref_state)
+
+
+def recurrent_cuba_bwd(grad_x, spikes, voltage, rec, threshold, tau_rho, scale_rho, graded=False):
     """S/utils/recurrent.py:83-112: the carried neuron state is a constant, so a step contributes the
     spike surrogate (the two one-step LI backward passes are identities); the gradient reaches step
-    t-1 through R.  Returns (grad_z, grad_R)."""
+    t-1 through R.  threshold: a number, or for an ALIF layer the tensor threshold + refractory of
+    every step.  Returns (grad_z, grad_R)."""
     grad_z = torch.zeros_like(grad_x)
     carry = torch.zeros(grad_x.shape[:-1])
     for t in range(grad_x.shape[-1] - 1, -1, -1):
         gs = carry + grad_x[..., t]
-        gd = spike_bwd(gs.unsqueeze(-1), voltage[..., t:t + 1], threshold, tau_rho, scale_rho)[..., 0]
+        th = threshold[..., t:t + 1] if torch.is_tensor(threshold) and threshold.dim() > 0 else threshold
+        gd = spike_bwd(gs.unsqueeze(-1), voltage[..., t:t + 1], th, tau_rho, scale_rho, graded)[..., 0]
         grad_z[..., t] = gd
         carry = torch.matmul(gd, rec)
     grad_out = grad_z[..., 1:].transpose(0, 1).reshape(grad_z.shape[1], -1)

@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(handle, n), f'{n} declared in slayer_hip.h but not exported'
     assert sorted(_native.EXPORTS) == names, 'python binding and header disagree'
-    assert _native.lib().slayer_abi_version() == 2
+    assert _native.lib().slayer_abi_version() == _native.ABI_VERSION == 3
     assert b'success' in _native.lib().slayer_error_string(0)
     assert b'inconsistent' in _native.lib().slayer_error_string(-1)
 
