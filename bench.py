@@ -709,6 +709,16 @@ def other_configs(dev, iters):
                      'frac': round(job.nt * bpn / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                      'timing': f'median of {iters} event-timed steps after 20 warm-up steps', 'parity': 'ok',
                      'parity_detail': ok})
+        if job.nt < (1 << 20):
+            # latency-bound: host time per call matters as much as the kernels; wall clock over many steps
+            null = lambda name: _Null()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(2000):
+                job.step(null)
+            torch.cuda.synchronize()
+            rows[-1]['us_per_step_event_timed'] = round(ms * 1e3, 2)
+            rows[-1]['us_per_step_wall_clock'] = round((time.perf_counter() - t0) / 2000 * 1e6, 2)
         del job
         gc.collect()
         torch.cuda.empty_cache()

@@ -286,6 +286,11 @@ int slayer_cumsum(float *out, const float *in, const float *state, int64_t num_s
 
 /* ---- fused CUBA neuron -------------------------------------------------------------------------- */
 
+/* Decays of the fused neuron entry points (slayer_cuba_*, slayer_alif_*, slayer_*_recurrent_fwd): the neuron
+ * classes hand their kernels quantize(decay) (neuron/cuba.py:356-374, utils/quantize.py:18-26,52-81: torch.round, i.e. to nearest,
+ * ties to even); these entry points do that rounding themselves, so a caller may pass the parameter as it is.
+ * The operator entry points (slayer_li_fwd, slayer_ath_fwd, ...) truncate like the kernels they replace. */
+
 /* No single counterpart in the reference: one launch for what cuba.Neuron.forward does with three
  * (neuron/cuba.py:356-374 + :401-410 = leaky_integrator.dynamics, leaky_integrator.dynamics with
  * threshold, Spike.forward).  Bit-identical to slayer_li_fwd -> slayer_li_fwd -> slayer_spike_fwd

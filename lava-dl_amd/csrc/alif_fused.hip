@@ -56,10 +56,10 @@ struct AlifFwd {
             yv = trunc_i32(p.v_state[p.n_vs == 1 ? 0 : m] * w);
             th = trunc_i32(p.th_state[p.n_ts == 1 ? 0 : m] * w);
             r = trunc_i32(p.ref_state[p.n_rs == 1 ? 0 : m] * w);
-            mi = 4096 - trunc_i32(p.i_decay[param_index(m, p.npb, p.n_id)]);
-            mv = 4096 - trunc_i32(p.v_decay[param_index(m, p.npb, p.n_vd)]);
-            mt = 4096 - trunc_i32(p.th_decay[param_index(m, p.npb, p.n_td)]);
-            mr = 4096 - trunc_i32(p.ref_decay[param_index(m, p.npb, p.n_rd)]);
+            mi = 4096 - trunc_i32(rintf(p.i_decay[param_index(m, p.npb, p.n_id)]));
+            mv = 4096 - trunc_i32(rintf(p.v_decay[param_index(m, p.npb, p.n_vd)]));
+            mt = 4096 - trunc_i32(rintf(p.th_decay[param_index(m, p.npb, p.n_td)]));
+            mr = 4096 - trunc_i32(rintf(p.ref_decay[param_index(m, p.npb, p.n_rd)]));
         }
     }
     // what the next operator reads of a state: trunc(w * (float(y) / w)); for a power of two the scaling
@@ -136,8 +136,8 @@ struct AlifBwd {
         lead = (rho / 2.0f) / tau;
         ai = av = gc = gx = acc_i = acc_v = 0.f;
         if (valid) {
-            ai = 1.0f - p.i_decay[param_index(m, p.npb, p.n_id)] / 4096.0f;
-            av = 1.0f - p.v_decay[param_index(m, p.npb, p.n_vd)] / 4096.0f;
+            ai = 1.0f - rintf(p.i_decay[param_index(m, p.npb, p.n_id)]) / 4096.0f;
+            av = 1.0f - rintf(p.v_decay[param_index(m, p.npb, p.n_vd)]) / 4096.0f;
         }
     }
     // The surrogate does not depend on the recurrence, so it is evaluated on the way into LDS (by all

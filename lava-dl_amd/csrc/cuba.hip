@@ -51,8 +51,8 @@ struct CubaFwd {
         if (valid) {
             yc = trunc_i32(p.i_state[p.n_is == 1 ? 0 : m] * w);
             yv = trunc_i32(p.v_state[p.n_vs == 1 ? 0 : m] * w);
-            mi = 4096 - trunc_i32(p.i_decay[param_index(m, p.npb, p.n_id)]);
-            mv = 4096 - trunc_i32(p.v_decay[param_index(m, p.npb, p.n_vd)]);
+            mi = 4096 - trunc_i32(rintf(p.i_decay[param_index(m, p.npb, p.n_id)]));
+            mv = 4096 - trunc_i32(rintf(p.v_decay[param_index(m, p.npb, p.n_vd)]));
         }
     }
     __device__ __forceinline__ void pre(float4 (&x)[1]) const { x[0] = to_state(x[0], w); }
@@ -111,8 +111,8 @@ struct CubaBwd {
         lead = (rho / 2.0f) / tau;
         ai = av = gc = gx = acc_i = acc_v = 0.f;
         if (valid) {
-            ai = 1.0f - p.i_decay[param_index(m, p.npb, p.n_id)] / 4096.0f;
-            av = 1.0f - p.v_decay[param_index(m, p.npb, p.n_vd)] / 4096.0f;
+            ai = 1.0f - rintf(p.i_decay[param_index(m, p.npb, p.n_id)]) / 4096.0f;
+            av = 1.0f - rintf(p.v_decay[param_index(m, p.npb, p.n_vd)]) / 4096.0f;
         }
     }
     // The surrogate does not depend on the recurrence, so it is evaluated on the way into LDS (by all

@@ -57,13 +57,13 @@ __global__ __launch_bounds__(kMaxRecurrent) void recurrent_fwd_kernel(const Recu
     if (live) {
         yc = trunc_i32(p.i_state[p.n_is == 1 ? 0 : m] * w);
         yv = trunc_i32(p.v_state[p.n_vs == 1 ? 0 : m] * w);
-        mi = 4096 - trunc_i32(p.i_decay[param_index(m, C, p.n_id)]);
-        mv = 4096 - trunc_i32(p.v_decay[param_index(m, C, p.n_vd)]);
+        mi = 4096 - trunc_i32(rintf(p.i_decay[param_index(m, C, p.n_id)]));
+        mv = 4096 - trunc_i32(rintf(p.v_decay[param_index(m, C, p.n_vd)]));
         if (ALIF) {
             th = trunc_i32(p.th_state[p.n_ts == 1 ? 0 : m] * w);
             r = trunc_i32(p.ref_state[p.n_rs == 1 ? 0 : m] * w);
-            mt = 4096 - trunc_i32(p.th_decay[param_index(m, C, p.n_td)]);
-            mr = 4096 - trunc_i32(p.ref_decay[param_index(m, C, p.n_rd)]);
+            mt = 4096 - trunc_i32(rintf(p.th_decay[param_index(m, C, p.n_td)]));
+            mr = 4096 - trunc_i32(rintf(p.ref_decay[param_index(m, C, p.n_rd)]));
         }
     }
     float cur = 0.f, vol = 0.f, thf = 0.f, rf = 0.f;

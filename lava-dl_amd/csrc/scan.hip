@@ -292,8 +292,8 @@ __global__ __launch_bounds__(kScanQuads) void cuba_bwd_scan_kernel(
     const unsigned first = scan_first_in_batch(sp.row0, npb);
     for (int rr = sp.tid; rr < sp.rows; rr += kScanQuads) {
         const unsigned in_batch = (first + (unsigned)rr) % npb;
-        ai_tab[rr] = 1.0f - i_decay[in_batch / per_i] / 4096.0f;
-        av_tab[rr] = 1.0f - v_decay[in_batch / per_v] / 4096.0f;
+        ai_tab[rr] = 1.0f - rintf(i_decay[in_batch / per_i]) / 4096.0f;
+        av_tab[rr] = 1.0f - rintf(v_decay[in_batch / per_v]) / 4096.0f;
     }
     if (DECAY_GRAD)
         for (int rr = sp.lane; rr < sp.rows; rr += kWave) { sum_i[sp.wv][rr] = 0.0f; sum_v[sp.wv][rr] = 0.0f; }

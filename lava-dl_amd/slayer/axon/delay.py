@@ -125,7 +125,7 @@ def _delay_bwd(grad_output, output, delay_val, sampling_time):
     grad_input = torch.empty_like(grad_output)
     grad_sum = torch.empty(npb, dtype=torch.float32, device=dev)
     workspace = torch.empty(M + 64 * npb, dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_delay_bwd(
             N.ptr(grad_input), N.ptr(grad_sum), N.ptr(grad_output), N.ptr(output), N.ptr(lut), 0,
             float(sampling_time), N.ptr(workspace), M, npb, T, N.stream_handle()))

@@ -18,7 +18,7 @@ def _fwd(input, threshold, pre_state, residual_state, error_state, cum_error, qu
     output, delta_input = torch.empty_like(input), torch.empty_like(input)
     residual_out = torch.empty(input.shape[:-1], dtype=input.dtype, device=dev)
     error_out = torch.empty(input.shape[:-1], dtype=input.dtype, device=dev)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_delta_fwd(
             N.ptr(output), N.ptr(delta_input), N.ptr(residual_out), N.ptr(error_out),
             N.ptr(input), N.ptr(threshold), N.ptr(pre_state), N.ptr(residual_state), N.ptr(error_state),
@@ -37,7 +37,7 @@ def _bwd(grad_output, delta_input, threshold, tau_grad, scale_grad, need_thresho
     if need_threshold_grad:
         grad_threshold = torch.empty(threshold.numel(), dtype=torch.float32, device=dev)
         workspace = torch.empty(M + 64 * threshold.numel(), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_delta_bwd(
             N.ptr(grad_input), N.ptr(grad_threshold), N.ptr(grad_output), N.ptr(delta_input), N.ptr(threshold),
             N.ptr(workspace), float(tau_grad), float(scale_grad),

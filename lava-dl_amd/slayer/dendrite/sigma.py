@@ -16,7 +16,7 @@ def _cumsum(input, state=None, reverse=False):
     state = None if state is None else state.contiguous()
     M, T = N.rows_and_steps(input)
     output = torch.empty_like(input)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_cumsum(N.ptr(output), N.ptr(input), N.ptr(state),
                                       0 if state is None else state.numel(), 1 if reverse else 0,
                                       M, T, N.stream_handle()))

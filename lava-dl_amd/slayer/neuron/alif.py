@@ -114,8 +114,8 @@ class Neuron(_Base):
                 self.spike_last = spike[..., -1].detach().clone()
             return D.chain_output(delays, spike)
         self._prepare(input)
-        args = (input, self._q('current_decay'), self._q('voltage_decay'), self._q('threshold_decay'),
-                self._q('refractory_decay'), self.current_state, self.voltage_state, self.threshold_state,
+        args = (input, self._q('current_decay', True), self._q('voltage_decay', True), self._q('threshold_decay', True),
+                self._q('refractory_decay', True), self.current_state, self.voltage_state, self.threshold_state,
                 self.refractory_state, self.threshold_step, self.threshold, self.s_scale)
         if not (torch.is_grad_enabled() and (input.requires_grad or self.requires_grad or D.needs_grad(delays))):
             # nothing to differentiate: only the spikes are written, the last states come per neuron

@@ -164,6 +164,11 @@ class Neuron(torch.nn.Module):
         for name, value in states.items():
             self._buffers[name] = value.clone() if value._is_view() else value
 
-    def _q(self, name):
-        """Integer-valued decay with a straight-through gradient."""
-        return quantize(getattr(self, name))
+    def _q(self, name, fused=False):
+        """Integer-valued decay with a straight-through gradient.  ``fused``: for a fused neuron kernel, which
+        rounds the decays itself (to nearest, ties to even, as ``quantize`` does); the parameter goes in as it is
+        unless a gradient has to reach it, which saves the rounding launch."""
+        param = getattr(self, name)
+        if fused and not (torch.is_grad_enabled() and param.requires_grad):
+            return param
+        return quantize(param)

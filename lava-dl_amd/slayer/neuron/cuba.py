@@ -95,7 +95,7 @@ class Neuron(_Base):
                 self.spike_last = spike[..., -1].detach().clone()
             return D.chain_output(delays, spike)
         self._prepare(input)
-        args = (input, self._q('current_decay'), self._q('voltage_decay'),
+        args = (input, self._q('current_decay', True), self._q('voltage_decay', True),
                 self.current_state.contiguous(), self.voltage_state.contiguous(), self.s_scale,
                 self.threshold + self.threshold_eps)
         spike_last = None

@@ -36,7 +36,7 @@ def _fwd(re_input, im_input, im_state, ref_state, ref_decay, th_state, th_decay,
         if s.numel() not in (1, M):
             raise RuntimeError(f'{name} has {s.numel()} elements, expected 1 or {M}')
     threshold, refractory = torch.empty_like(re_input), torch.empty_like(re_input)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_apth_fwd(
             N.ptr(threshold), N.ptr(refractory), N.ptr(re_input), N.ptr(im_input),
             N.ptr(im_state), N.ptr(ref_state), N.ptr(ref_decay), N.ptr(th_state), N.ptr(th_decay),

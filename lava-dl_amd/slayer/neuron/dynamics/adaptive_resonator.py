@@ -42,7 +42,7 @@ def _fwd(real_input, imag_input, sin_decay, cos_decay, ref_decay, th_decay,
         if s.numel() not in (1, M):
             raise RuntimeError(f'{name} has {s.numel()} elements, expected 1 or {M}')
     outs = [torch.empty_like(real_input) for _ in range(4)]
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_adres_fwd(
             *[N.ptr(o) for o in outs], N.ptr(real_input), N.ptr(imag_input),
             N.ptr(sin_decay), N.ptr(cos_decay), N.ptr(ref_decay), N.ptr(th_decay),

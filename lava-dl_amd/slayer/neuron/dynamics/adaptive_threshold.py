@@ -50,7 +50,7 @@ def _fwd(input, ref_state, ref_decay, th_state, th_decay, th_scale, th0, w_scale
             raise RuntimeError(f'{name} has {s.numel()} elements, expected 1 or {M}')
     threshold = torch.empty_like(input)
     refractory = torch.empty_like(input)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(getattr(N.lib(), entry)(
             N.ptr(threshold), N.ptr(refractory), N.ptr(input),
             N.ptr(ref_state), N.ptr(ref_decay), N.ptr(th_state), N.ptr(th_decay),

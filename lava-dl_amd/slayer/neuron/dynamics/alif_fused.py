@@ -73,7 +73,7 @@ def _fwd(input, decays, states, threshold_step, threshold_base, w_scale, graded,
     if want_last:
         th_last = torch.empty(input.shape[:-1], dtype=input.dtype, device=dev)
         ref_last = torch.empty(input.shape[:-1], dtype=input.dtype, device=dev)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_alif_fwd(
             N.ptr(cur), N.ptr(vol), N.ptr(theta), N.ptr(spk), N.ptr(cur_last), N.ptr(vol_last), N.ptr(th_last),
             N.ptr(ref_last),
@@ -99,7 +99,7 @@ def _bwd(grad_spikes, vol, theta, cur, i_decay, v_decay, tau_rho, scale_rho, gra
         g_i = torch.empty(i_decay.numel(), dtype=torch.float32, device=dev)
         g_v = torch.empty(v_decay.numel(), dtype=torch.float32, device=dev)
         workspace = torch.empty(2 * M + 64 * (i_decay.numel() + v_decay.numel()), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_alif_bwd(
             N.ptr(grad_input), N.ptr(g_i), N.ptr(g_v), N.ptr(grad_spikes), N.ptr(vol), N.ptr(theta), N.ptr(cur),
             N.ptr(i_decay), N.ptr(v_decay), float(tau_rho), float(scale_rho), 1 if graded else 0, N.ptr(workspace),

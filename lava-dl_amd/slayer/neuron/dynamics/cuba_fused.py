@@ -65,7 +65,7 @@ def _fwd(input, i_decay, v_decay, i_state, v_state, w_scale, threshold, graded, 
     cur = None if lean else torch.empty_like(input)
     cur_last = torch.empty(input.shape[:-1], dtype=input.dtype, device=dev) if lean else None
     vol_last = torch.empty(input.shape[:-1], dtype=input.dtype, device=dev) if spikes_only else None
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_cuba_fwd(
             N.ptr(cur), N.ptr(vol), N.ptr(spk), N.ptr(cur_last), N.ptr(vol_last), N.ptr(input),
             N.ptr(i_decay), N.ptr(v_decay),
@@ -90,7 +90,7 @@ def _bwd(grad_spikes, vol, cur, i_decay, v_decay, threshold, tau_rho, scale_rho,
         g_i = torch.empty(i_decay.numel(), dtype=torch.float32, device=dev)
         g_v = torch.empty(v_decay.numel(), dtype=torch.float32, device=dev)
         workspace = torch.empty(2 * M + 64 * (i_decay.numel() + v_decay.numel()), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_cuba_bwd(
             N.ptr(grad_input), N.ptr(g_i), N.ptr(g_v), N.ptr(grad_spikes), N.ptr(vol), N.ptr(cur),
             N.ptr(i_decay), N.ptr(v_decay), float(threshold), float(tau_rho), float(scale_rho),

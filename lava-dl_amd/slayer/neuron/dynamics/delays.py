@@ -116,7 +116,7 @@ def output_delay_gradient(delays, grad_spikes, spikes):
     ts = delays.sampling_time
     grad_sum = torch.empty(npb, dtype=torch.float32, device=dev)
     workspace = torch.empty(M + 64 * npb, dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_delay_bwd(None, N.ptr(grad_sum), N.ptr(grad_spikes), N.ptr(spikes), None, 0,
                                          float(ts), N.ptr(workspace), M, npb, T, N.stream_handle()))
     grad = grad_sum * ts * delays.grad_scale

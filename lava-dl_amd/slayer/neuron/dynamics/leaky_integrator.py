@@ -54,7 +54,7 @@ def _fwd(input, decay, state, threshold, w_scale, entry='slayer_li_fwd'):
     if state.numel() not in (1, M):
         raise RuntimeError(f'state has {state.numel()} elements, expected 1 or {M}')
     output = torch.empty_like(input)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(getattr(N.lib(), entry)(
             N.ptr(output), N.ptr(input), N.ptr(decay), N.ptr(state),
             float(threshold * w_scale), int(w_scale),
@@ -74,7 +74,7 @@ def _bwd(grad_output, output, decay, need_decay_grad=True, per_neuron_sums=False
         grad_decay = torch.empty(decay.numel(), dtype=torch.float32, device=dev)
     if need_decay_grad or per_neuron_sums:
         workspace = torch.empty(M + 64 * decay.numel(), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_li_bwd(
             N.ptr(grad_input), N.ptr(grad_decay), N.ptr(grad_output), N.ptr(output), N.ptr(decay),
             N.ptr(workspace), M, N.neurons_per_batch(grad_output), decay.numel(), T, N.stream_handle()))
@@ -86,7 +86,7 @@ def _bwd_naive(grad_output, decay):
     grad_output, decay = grad_output.contiguous(), decay.contiguous()
     M, T = N.rows_and_steps(grad_output)
     grad_input = torch.empty_like(grad_output)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_li_bwd_naive(
             N.ptr(grad_input), N.ptr(grad_output), N.ptr(decay), M, N.neurons_per_batch(grad_output),
             decay.numel(), T, N.stream_handle()))

@@ -58,7 +58,7 @@ def _fwd(real_input, imag_input, sin_decay, cos_decay, real_state, imag_state, t
             raise RuntimeError(f'{name} has {s.numel()} elements, expected 1 or {M}')
     real = torch.empty_like(real_input)
     imag = torch.empty_like(imag_input)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(getattr(N.lib(), entry)(
             N.ptr(real), N.ptr(imag), N.ptr(real_input), N.ptr(imag_input),
             N.ptr(sin_decay), N.ptr(cos_decay), N.ptr(real_state), N.ptr(imag_state),
@@ -80,7 +80,7 @@ def _bwd(grad_real, grad_imag, real, imag, sin_decay, cos_decay, need_decay_grad
         g_sin = torch.empty(sin_decay.numel(), dtype=torch.float32, device=dev)
         g_cos = torch.empty(cos_decay.numel(), dtype=torch.float32, device=dev)
         workspace = torch.empty(2 * M + 128 * sin_decay.numel(), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_res_bwd(
             N.ptr(g_re_in), N.ptr(g_im_in), N.ptr(g_sin), N.ptr(g_cos),
             N.ptr(grad_real), N.ptr(grad_imag), N.ptr(real), N.ptr(imag),
@@ -94,7 +94,7 @@ def _bwd_naive(grad_real, grad_imag, sin_decay, cos_decay):
     grad_real, grad_imag = grad_real.contiguous(), grad_imag.contiguous()
     M, T = N.rows_and_steps(grad_real)
     g_re_in, g_im_in = torch.empty_like(grad_real), torch.empty_like(grad_imag)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_res_bwd_naive(
             N.ptr(g_re_in), N.ptr(g_im_in), N.ptr(grad_real), N.ptr(grad_imag),
             N.ptr(sin_decay.contiguous()), N.ptr(cos_decay.contiguous()),

@@ -57,7 +57,7 @@ def _fwd(real_input, imag_input, sin_decay, cos_decay, real_state, imag_state, i
         re_last, im_last = (torch.empty(real_input.shape[:-1], dtype=real_input.dtype, device=dev) for _ in range(2))
     else:
         real, imag = torch.empty_like(real_input), torch.empty_like(real_input)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_rf_fwd(
             N.ptr(real), N.ptr(imag), N.ptr(spk), N.ptr(re_last), N.ptr(im_last), N.ptr(real_input),
             N.ptr(imag_input),
@@ -79,7 +79,7 @@ def _bwd(grad_spikes, real, imag, sin_decay, cos_decay, threshold, tau_rho, scal
         g_sin = torch.empty(sin_decay.numel(), dtype=torch.float32, device=dev)
         g_cos = torch.empty(cos_decay.numel(), dtype=torch.float32, device=dev)
         workspace = torch.empty(2 * M + 128 * sin_decay.numel(), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_rf_bwd(
             N.ptr(g_re), N.ptr(g_im), N.ptr(g_sin), N.ptr(g_cos), N.ptr(grad_spikes), N.ptr(real), N.ptr(imag),
             N.ptr(sin_decay), N.ptr(cos_decay), float(threshold), float(tau_rho), float(scale_rho),

@@ -26,7 +26,7 @@ def _fwd(real, imag, th, th_value, last, last_value, graded, scale):
         raise RuntimeError(f'real/imag shapes differ: {real.shape} vs {imag.shape}')
     M, T = N.rows_and_steps(real)
     spikes = torch.empty_like(real)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_cspike_fwd(
             N.ptr(spikes), N.ptr(real), N.ptr(imag), N.ptr(th), 0 if th is None else th.numel(), th_value,
             N.ptr(last), 0 if last is None else last.numel(), last_value,
@@ -39,7 +39,7 @@ def _bwd(grad_out, real, imag, th, th_value, tau_rho, scale_rho, graded):
     grad_out = grad_out.contiguous()
     g_re = torch.empty_like(real)
     g_im = torch.empty_like(imag)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_cspike_bwd(
             N.ptr(g_re), N.ptr(g_im), N.ptr(grad_out), N.ptr(real), N.ptr(imag), N.ptr(th),
             0 if th is None else th.numel(), th_value,

@@ -23,7 +23,7 @@ def split_threshold(threshold, like):
 def _fwd(voltage, th, th_value, graded, scale):
     dev = N.require_gpu(voltage)
     spikes = torch.empty_like(voltage)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_spike_fwd(
             N.ptr(spikes), N.ptr(voltage), N.ptr(th), 0 if th is None else th.numel(), th_value,
             1 if graded else 0, float(scale), voltage.numel(), N.stream_handle()))
@@ -34,7 +34,7 @@ def _bwd(grad_spikes, voltage, th, th_value, tau_rho, scale_rho, graded):
     dev = N.require_gpu(grad_spikes, voltage)
     grad_spikes = grad_spikes.contiguous()
     grad_voltage = torch.empty_like(voltage)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_spike_bwd(
             N.ptr(grad_voltage), N.ptr(grad_spikes), N.ptr(voltage), N.ptr(th),
             0 if th is None else th.numel(), th_value,

@@ -15,7 +15,7 @@ def _run(entry, input, filter, sampling_time):
     input, filter = input.contiguous(), filter.contiguous()
     M, T = N.rows_and_steps(input)
     output = torch.empty_like(input)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(getattr(N.lib(), entry)(
             N.ptr(output), N.ptr(input), N.ptr(filter), filter.numel(), float(sampling_time),
             M, T, N.stream_handle()))

@@ -116,13 +116,13 @@ class _FusedRecurrent(torch.autograd.Function):
         rec_t = torch.cat([rec.transpose(0, 1), rec.new_zeros(1, c)], dim=0).contiguous()   # + the zero row
         is_alif = type(neuron) is alif.Neuron
         names = ('current', 'voltage') + (('threshold', 'refractory') if is_alif else ())
-        decays = [neuron._q(f'{k}_decay').detach().contiguous() for k in names]
+        decays = [neuron._q(f'{k}_decay', True).detach().contiguous() for k in names]
         states = [getattr(neuron, f'{k}_state').contiguous() for k in names]
         spk, vol = torch.empty_like(z), torch.empty_like(z)
         theta = torch.empty_like(z) if is_alif else None
         last = [torch.empty_like(s) for s in states]
         graded = 1 if neuron.graded_spike else 0
-        with torch.cuda.device(dev):
+        with N.device_guard(dev):
             if is_alif:
                 threshold = 0.0
                 N.check(N.lib().slayer_alif_recurrent_fwd(
@@ -160,7 +160,7 @@ class _FusedRecurrent(torch.autograd.Function):
         grad_x = grad_x.contiguous()
         n, c, t = grad_x.shape
         grad_z = torch.empty_like(grad_x)
-        with torch.cuda.device(dev):
+        with N.device_guard(dev):
             N.check(N.lib().slayer_recurrent_bwd(
                 N.ptr(grad_z), N.ptr(grad_x), N.ptr(vol), N.ptr(theta[0]) if theta else None, N.ptr(rec),
                 threshold, tau_rho, scale_rho, graded, n, c, t, N.stream_handle()))

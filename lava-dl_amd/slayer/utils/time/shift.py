@@ -35,7 +35,7 @@ def shift(input, shift_val, sampling_time=1):
         if torch.is_tensor(shift_val):
             shift_val = shift_val.item()
         lut, steps, npb = None, int(shift_val / sampling_time), max(M, 1)
-    with torch.cuda.device(dev):
+    with N.device_guard(dev):
         N.check(N.lib().slayer_shift(
             N.ptr(output), N.ptr(input), N.ptr(lut), steps, float(sampling_time),
             M, npb, T, N.stream_handle()))

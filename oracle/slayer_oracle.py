@@ -29,6 +29,9 @@ Pin status (see tests/test_oracle_*.py):
   delay_bwd                       finite-difference identity on the conv([-1,1]) form
   delta_fwd / delta_bwd, sigma    hand-computed sequences, reconstruction invariant |x - sigma(delta(x))| < threshold,
                                   float64 closed forms of the threshold gradient, numpy.cumsum
+  recurrent_cuba_fwd/_bwd,        no reference fixture; without feedback = the pinned operators over the whole sequence,
+  recurrent_alif_fwd              hand-computed cases (delay and orientation of R, graded value, threshold / refractory
+                                  jump), backward = float64 autograd through an independently written unrolled graph
 """
 
 import numpy as np

@@ -577,3 +577,42 @@ def test_cuba_neuron_with_a_norm_takes_the_operator_chain(slayer):
     assert 0 < float(want.sum()) < want.numel()
     assert torch.equal(spk, want)
     assert torch.equal(n.norm.bias, -n.quantize_8bit(n.norm.running_mean, descale=True))
+
+
+@pytest.mark.parametrize('kind', ['cuba', 'alif'])
+@pytest.mark.parametrize('trained', [False, True])
+def test_fused_neurons_round_their_decays_like_the_quantizer(slayer, kind, trained):
+    """Decays that are not integers, halves among them (round-half-even): the fused kernels take the parameters
+    as they are and round them themselves; the operator chain gets quantize(decay) from the neuron class."""
+    gen = torch.Generator().manual_seed(991)
+    x = sparse_input(gen, (3, 4, 7, 120), p=0.3, amp=1.5).to(dev())
+    decays = [[1000.5, 1001.5, 409.6, 37.49], [300.5, 12.5, 2047.51, 0.4]]
+    if kind == 'cuba':
+        mk = lambda: slayer.neuron.cuba.Neuron(1.0, [0.2, 0.4], [0.1, 0.3], shared_param=False, requires_grad=trained,
+                                               persistent_state=True).to(dev())
+    else:
+        mk = lambda: slayer.neuron.alif.Neuron(1.0, 0.5, [0.2, 0.4], [0.1, 0.3], [0.1, 0.3], [0.2, 0.4],
+                                               shared_param=False, requires_grad=trained,
+                                               persistent_state=True).to(dev())
+    a, b = mk(), mk()
+    a._prepare(x)
+    b._prepare(x)
+    for n in (a, b):
+        with torch.no_grad():
+            n.current_decay.copy_(torch.tensor(decays[0]))
+            n.voltage_decay.copy_(torch.tensor(decays[1]))
+            if kind == 'alif':
+                n.threshold_decay.copy_(torch.tensor([100.5, 101.5, 77.7, 3.2]))
+                n.refractory_decay.copy_(torch.tensor([600.5, 601.5, 15.5, 900.49]))
+    for grad in (False, True):
+        xa, xb = x.clone().requires_grad_(grad), x.clone().requires_grad_(grad)
+        with torch.set_grad_enabled(grad):
+            sa = a(xa)                                                   # fused
+            sb = b.spike(*b.dynamics(xb)[1:])                            # separate operators
+        assert float(sa.detach().sum()) > 0
+        assert torch.equal(sa.detach(), sb.detach()), f'spikes differ (grad={grad})'
+        assert torch.equal(a.voltage_state, b.voltage_state) and torch.equal(a.current_state, b.current_state)
+        if grad:
+            sa.sum().backward()
+            sb.sum().backward()
+            assert_same_gradient(xa.grad, xb.grad, 'input gradient')
