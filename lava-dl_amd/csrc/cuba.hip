@@ -29,6 +29,7 @@ struct CubaFwd {
     static constexpr unsigned kShiftIn = SHIFT ? 1u : 0u, kShiftOut = SHIFT ? (1u << kOut) : 0u;
     static constexpr bool kReverse = false;
     static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
+    static constexpr bool kLongPiecesOnAliasedRows = true;
     struct Params {
         const float* in[1];
         float* out[kOut + 1];

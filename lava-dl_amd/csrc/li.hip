@@ -11,6 +11,7 @@ struct LiFwd {
     static constexpr int kIn = 1, kOut = 1;
     static constexpr bool kReverse = false;
     static constexpr int64_t kRows32Below = 32768, kRows16Below = 8192;
+    static constexpr bool kLongPiecesOnAliasedRows = true;
     struct Params {
         const float* in[1];
         float* out[1];

@@ -138,6 +138,7 @@ struct TileGeom {
 //     the same step: it is computed while a quad is copied out and needs neither an LDS tile nor
 //     boundary registers
 //   static constexpr int64_t kRows32Below, kRows16Below;   (rows-per-wave policy, see launch_stream)
+//   static constexpr bool kLongPiecesOnAliasedRows;        (optional, see row_stride_aliases)
 //   struct Params { const float* in[kIn]; float* out[kOut]; ... };   (a null out[] entry is not stored, a null
 //     in[] entry other than in[0] reads as zeros: a slot for pre() to fill)
 //   __device__ void init(const Params&, int64_t m, bool valid);
@@ -981,6 +982,24 @@ bool stream_fits_multiwave(const typename Op::Params& prm, int64_t M, int64_t T)
     return (M + RD - 1) / RD <= (int64_t)per_cu * compute_units();
 }
 
+// Rows a multiple of 2 KB apart (or within 64 bytes of one: T = 512, 1024, 2048, also 500) put the same columns
+// of every row on few memory channels, and a wave-wide access that touches eight rows (128-byte pieces) is served
+// by them one after the other: a plain copy in that pattern drops from 5.0 to 3.6 TB/s at T = 1024
+// (microbench/row_tile_copy.hip).  512-byte pieces of two rows per access (16 rows per wave) do not suffer;
+// Ops whose recurrence is light enough to run on 16 lanes per wave ask for them (kLongPiecesOnAliasedRows:
+// LI forward 311 -> 265 us, fused CUBA forward 616 -> 542 us at [2400,64,1024]; the adaptive-threshold and
+// resonator recurrences lose more on the idle lanes than they gain).
+inline bool row_stride_aliases(int64_t T) {
+    const int64_t r = (T * 4) % 2048;
+    return T >= 384 && (r <= 64 || r >= 2048 - 64);
+}
+template <class Op, class = void>
+struct LongPiecesOnAliasedRows { static constexpr bool value = false; };
+template <class Op>
+struct LongPiecesOnAliasedRows<Op, decltype((void)Op::kLongPiecesOnAliasedRows)> {
+    static constexpr bool value = Op::kLongPiecesOnAliasedRows;
+};
+
 template <class Op>
 int launch_stream(const typename Op::Params& prm, int64_t M, int64_t T, hipStream_t stream) {
     if (M == 0 || T == 0) return 0;
@@ -996,7 +1015,8 @@ int launch_stream(const typename Op::Params& prm, int64_t M, int64_t T, hipStrea
             hipLaunchKernelGGL((stream_kernel_duo<Op, RD, false, NC>), grid, block, 0, stream, prm, M, (int)T);
         return (int)hipGetLastError();
     }
-    if (M < Op::kRows16Below) return launch_stream_rows<Op, 16>(prm, M, T, vec, streaming, stream);
+    if (M < Op::kRows16Below || (LongPiecesOnAliasedRows<Op>::value && row_stride_aliases(T)))
+        return launch_stream_rows<Op, 16>(prm, M, T, vec, streaming, stream);
     if constexpr (Op::kRows16Below < kAlways && Op::kRows16Below < Op::kRows32Below)
         if (M < Op::kRows32Below) return launch_stream_rows<Op, 32>(prm, M, T, vec, streaming, stream);
     if constexpr (Op::kRows32Below < kAlways)

@@ -247,3 +247,33 @@ def test_tensors_beyond_four_gib(slayer, C, T):
     assert torch.equal(f_cur, cur) and torch.equal(f_vol, vol) and torch.equal(f_spk, spk)
     del f_cur, f_vol, f_spk, cur, vol, spk, x
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize('T', [512, 1024, 500])
+def test_rows_a_power_of_two_apart_take_long_pieces_with_the_same_results(slayer, T):
+    """Tensors too large for the all-resident kernel whose rows are (nearly) a multiple of 2 KB apart: LI forward
+    and the fused CUBA forward switch to 16 rows per wave there.  Oracle on a slab of rows, the fused kernel against
+    the chain of operators over the whole tensor, and the split-in-time invariance."""
+    M0 = 160 * 1024 * 1024 // T                        # 640 MB per tensor: far more rows than stay resident
+    shape = (M0 // 64, 64, T)
+    D = slayer.neuron.dynamics
+    L = D.leaky_integrator
+    x = gpu_events(shape, 0.05, 1.0, 70 + T)
+    gen = torch.Generator().manual_seed(71)
+    d_i = torch.randint(0, 4096, (64,), generator=gen).float()
+    d_v = torch.randint(0, 4096, (64,), generator=gen).float()
+    zero = torch.zeros(1, device=dev())
+    cur = L._fwd(x, d_i.to(dev()), zero, -1, 4096)
+    vol = L._fwd(cur, d_v.to(dev()), zero, 1.25, 4096)
+    f_cur, f_vol, f_spk = D.cuba_fused._fwd(x, d_i.to(dev()), d_v.to(dev()), zero, zero, 4096, 1.25, False, 1)
+    assert torch.equal(f_cur, cur) and torch.equal(f_vol, vol)
+    assert torch.equal(f_spk, (vol >= 1.25).float()) and float(f_spk.sum()) > 1000
+    sl = (slice(None, None, shape[0] // 3), slice(None, None, 7))
+    r_cur = O.li_fwd(x[sl].cpu(), d_i[::7], torch.tensor([0.0]), 4096)
+    r_vol = O.li_fwd(r_cur, d_v[::7], torch.tensor([0.0]), 4096, 1.25)
+    assert_exact(cur[sl], r_cur, 'current slab')
+    assert_exact(vol[sl], r_vol, 'voltage slab')
+    k = T // 2 + 4
+    c1 = L._fwd(x[..., :k].contiguous(), d_i.to(dev()), zero, -1, 4096)
+    c2 = L._fwd(x[..., k:].contiguous(), d_i.to(dev()), c1[..., -1].contiguous(), -1, 4096)
+    assert torch.equal(torch.cat([c1, c2], -1), cur)
