@@ -96,91 +96,153 @@ __global__ __launch_bounds__(kWave) void conv_kernel(float* __restrict__ out, co
 }
 
 // ---------------------------------------------------------------------------------------------
-// Matrix-core form for 8 < K <= 128 (T % 4 == 0, 16-byte aligned tensors).  A tile of 16 output steps of 16
-// rows is a [16 x (16 + KPAD)] Toeplitz matrix of taps times the [(16 + KPAD) x 16] window of inputs:
-// v_mfma_f32_16x16x4_f32 with D[i][j] = output step i of row j, four input samples per instruction.  With
-// K = 64 the window is 80 samples, so 64 of 80 multiply-adds are useful (the FMA form above issues 82
-// instructions per 64 useful FMAs at half the rate).  Lane l works for row l % 16 and quad l / 16: it loads
-// the 4 samples [16 g + 4 (l / 16), +4) of window group g straight from memory (a float4), which are exactly
-// the B operands of the group's four instructions (sample 4 k + r of a group goes to summation slot k of
-// instruction r), keeps the Toeplitz operands of all groups in registers (they do not depend on the tile),
-// and receives 4 consecutive output steps of its row (a float4 store).  Stepping to the next tile moves
-// every window group down by one, so a tile costs one new load per lane; no LDS, no barrier.
+// Matrix-core form for 8 < K <= 128 (T % 4 == 0, T >= 16, 16-byte aligned tensors).  The tensor is walked as one
+// flat stream of M * T samples in tiles of 256 consecutive samples, each seen as 16 blocks of 16 output steps:
+// D[i][n] = output 16 n + i of the tile is the [16 x (16 + KPAD)] Toeplitz matrix of taps times the
+// [(16 + KPAD) x 16] matrix whose column n is the window of block n (v_mfma_f32_16x16x4_f32, four window samples
+// per instruction).  With K = 64 the window is 80 samples, so 64 of 80 multiply-adds are useful (the FMA form
+// above issues 82 instructions per 64 useful FMAs at half the rate).  The window of block n, shifted by 16
+// samples, is the window of block n + 1: the B operands of all window groups are the same 256 (+ KPAD) samples,
+// read at different offsets.  So a tile costs one wave-wide load of 1 KB of consecutive bytes (lane l: samples
+// [4 l, 4 l + 4) of the tile), kept in an LDS ring of four tiles, and one wave-wide store that covers the tile's
+// 1 KB (lane (kq, n) of the result holds the outputs 16 n + 4 kq .. + 3; passing the result through LDS to store
+// in lane order as well changes nothing): whole 128-byte lines in both directions, every input byte fetched once
+// (plus one tile per wave for the window of its first or last tile).
+// In the ring a tile is stored quad-transposed (quad 4 n + kq at slot 16 kq + n), which makes the operand reads
+// (lane (kq, n) reads slot 16 kq + n + g of group g, spilling into the neighbouring tile) conflict-free.
+// The Toeplitz operands do not depend on the tile and stay in registers (4 per window group).
+//
+// Rows: a block's window must not see the neighbouring row.  Every lane masks the window quads of its block that
+// lie outside the row of the block (it reads a quad of zeros instead; rows are whole quads).  A block that holds
+// the end of one row and the start of the next (T % 16 != 0) needs both views: such a tile is multiplied twice,
+// once with every block seeing the row of its first output and once the row of its last output, and every output
+// quad takes the result of its own row.
 // Window samples outside a filter's support meet a zero tap instead of being skipped, so an Inf or NaN in the
-// input also reaches the up to 16 + KPAD - K neighbouring outputs whose window holds it (0 * Inf); finite
-// inputs, the only ones this path sees, give the same sums.
+// input also reaches the up to 16 + KPAD - K neighbouring outputs of its row whose window holds it (0 * Inf);
+// finite inputs, the only ones this path sees, give the same sums.
 typedef float mfma_f4 __attribute__((ext_vector_type(4)));
+
+constexpr int kConvTile = 256;             // samples per tile
+constexpr int kConvRing = 4;               // tiles in the LDS ring = tiles per loop pass
 
 template <int KPAD, bool CORR>
 __global__ __launch_bounds__(kWave) void conv_mfma_kernel(float* __restrict__ out, const float* __restrict__ in,
                                                           const float* __restrict__ filt, int K, float ts,
-                                                          int64_t M, int T, int span, unsigned spans_per_row) {
-    constexpr int G = KPAD / 16 + 1;        // window groups of 16 samples per tile
-    constexpr int RING = KPAD <= 64 ? 8 : 16;
+                                                          int64_t total, int T, int tiles_per_wave) {
+    constexpr int G = KPAD / 16 + 1;        // window groups of 16 samples per block
+    constexpr int kZero = kConvRing * 64;   // ring slot that holds a quad of zeros
+    __shared__ __attribute__((aligned(16))) float4 ring[kConvRing * 64 + 1];
     const int lane = threadIdx.x;
-    const int j = lane & 15, kq = lane >> 4;
-    const int64_t rowgroup = blockIdx.x / spans_per_row;
-    const int tbeg = (int)(blockIdx.x - rowgroup * spans_per_row) * span;
-    const int tend = tbeg + span < T ? tbeg + span : T;
-    const int64_t m0 = rowgroup * 16;
-    const int rows = (int)((M - m0) < 16 ? (M - m0) : 16);
-    // raw buffer accesses over the wave's rows: a lane that must not touch memory (row beyond the tensor,
-    // step outside [0, T)) gets an out-of-range offset, reads zeros and has its store dropped; no branch
-    // surrounds a memory instruction, so the loads issued ahead stay in flight across the loop's waits
-    const unsigned wave_bytes = (unsigned)rows * (unsigned)T * 4u;
-    const __amdgpu_buffer_rsrc_t src = make_rsrc(in + m0 * (int64_t)T, wave_bytes);
-    const __amdgpu_buffer_rsrc_t dst = make_rsrc(out + m0 * (int64_t)T, wave_bytes);
-    const bool row_ok = j < rows;
-    const int row_off = j * T * 4;
+    const int n = lane & 15, kq = lane >> 4;
+    // this wave's tiles: samples [first, last) of the flat tensor; its accesses are relative to the row that
+    // holds `first`, through a descriptor that ends with the tensor
+    const int64_t first = (int64_t)blockIdx.x * tiles_per_wave * kConvTile;
+    const int64_t rest = total - first;
+    const int mine = (int)(rest < (int64_t)tiles_per_wave * kConvTile ? rest : (int64_t)tiles_per_wave * kConvTile);
+    const int64_t row0 = first / T;
+    const int lead = (int)(first - row0 * T);                 // samples of row0 in front of `first`
+    // offsets below are relative to `origin`, one tile in front of `first` (the conv window reaches back)
+    const int64_t origin = first - kConvTile;
+    const int64_t avail = total - origin;                     // samples from origin to the end of the tensor
+    const int bound = (int)(avail < (int64_t)(tiles_per_wave + 2) * kConvTile ? avail
+                                                                              : (int64_t)(tiles_per_wave + 2) * kConvTile);
+    const __amdgpu_buffer_rsrc_t src = make_rsrc(in + origin, (unsigned)bound * 4u);
+    const __amdgpu_buffer_rsrc_t dst = make_rsrc(out + origin, (unsigned)bound * 4u);
+    const int floor0 = origin < 0 ? kConvTile : 0;            // nothing in front of the tensor
+    if (lane == 0) ring[kZero] = make_float4(0.f, 0.f, 0.f, 0.f);
 
-    // Toeplitz operands: lane (output step i = l % 16, slot kq) of instruction (g, r) holds the tap that
-    // links output step i with window sample 16 g + 4 kq + r
+    // Toeplitz operands: lane (output step i = l % 16 of a block, slot kq) of instruction (g, r) holds the tap
+    // that links output step i with window sample 16 g + 4 kq + r
     float a[G][4];
 #pragma unroll
     for (int g = 0; g < G; ++g)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int idx = CORR ? (16 * g + 4 * kq + r) - j : j + KPAD - (16 * g + 4 * kq + r);
+            const int idx = CORR ? (16 * g + 4 * kq + r) - n : n + KPAD - (16 * g + 4 * kq + r);
             a[g][r] = (idx >= 0 && idx < K) ? filt[idx] : 0.0f;
         }
 
-    // window group g of the tile at t0 starts at step t0 - KPAD + 16 g (conv) or t0 + 16 g (corr)
-    auto load = [&](int step) -> float4 {
-        const bool ok = row_ok && (unsigned)step < (unsigned)T;
-        return buf_load4<false>(src, ok ? row_off + step * 4 : kOutOfRange);
+    // Ring slot (in quads) of the operand of group g, relative to the ring position of the tile being computed:
+    // the window of block n starts KPAD samples before the block (conv) or with it (corr), so group g is block
+    // b = n + g - KPAD / 16 (conv) or n + g (corr) of the tile, or of its neighbour when b leaves [0, 16).
+    int opnd[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const int b = n + g - (CORR ? 0 : KPAD / 16);
+        const int tile = b < 0 ? -1 : (b >= 16 ? 1 : 0);
+        opnd[g] = ((tile * 64 + 16 * kq + (b - 16 * tile)) + kConvRing * 64) & (kConvRing * 64 - 1);
+    }
+    const int wslot = 16 * (lane & 3) + (lane >> 2);       // where this lane's loaded quad goes within a tile
+    // sample (relative to `first`) of the first window quad of this lane: group g adds 16 g
+    const int wq = 16 * n + 4 * kq - (CORR ? 0 : KPAD);
+
+    // Step s writes tile w0 + s into the ring (w0 = -1: the conv window reaches back into the previous tile;
+    // corr reaches forward, so its tile s is written one step before tile s - 1 is computed) and computes tile
+    // s - 1.  Loads run kConvRing steps ahead of their ring write, in registers.
+    constexpr int w0 = CORR ? 0 : -1;
+    const int lend = kConvTile + mine + (CORR ? kConvTile : 0);   // relative to origin: last sample a tile may read
+    auto load = [&](int tile) -> float4 {
+        const int t = (tile + 1) * kConvTile + 4 * lane;          // relative to origin
+        return buf_load4<false>(src, (t >= floor0 && t < lend) ? t * 4 : kOutOfRange);
     };
-    // Window groups live in a ring of RING registers (absolute group q of the span, starting at step
-    // first + 16 q, sits in slot q % RING): tile n reads groups n .. n + G - 1 and then refills the slot of
-    // group n, which no later tile needs, with group n + RING -- P = RING - G tiles before its first use.
-    // The loop body is RING tiles, so every slot index is a compile-time constant.
-    const int first = (CORR ? tbeg : tbeg - KPAD) + 4 * kq;
-    float4 x[RING];
+    float4 stage[kConvRing];
     // each load is preceded by a store that falls out of range (dropped by the hardware): the loop is then
     // entered in the state its back edge leaves, and the wait at its top can leave the youngest loads in
     // flight instead of draining everything
 #pragma unroll
-    for (int q = 0; q < RING; ++q) {
-        buf_store4<false>(dst, kOutOfRange + 16 * q, make_float4(0.f, 0.f, 0.f, 0.f));
-        x[q] = load(first + 16 * q);
+    for (int u = 0; u < kConvRing; ++u) {
+        buf_store4<false>(dst, kOutOfRange + 16 * u, make_float4(0.f, 0.f, 0.f, 0.f));
+        stage[u] = load(w0 + u);
     }
-
-    for (int t0 = tbeg; t0 < tend; t0 += 16 * RING) {
+    const int steps = (mine + kConvTile - 1) / kConvTile + 1;
+    for (int s0 = 0; s0 < steps; s0 += kConvRing) {
 #pragma unroll
-        for (int u = 0; u < RING; ++u) {
+        for (int u = 0; u < kConvRing; ++u) {
+            // ring position of tile w0 + s is (s & 3) = u: s0 is a multiple of the ring length
+            ring[u * 64 + wslot] = stage[u];
+            stage[u] = load(w0 + s0 + u + kConvRing);
+            // tile s - 1 sits at ring position (u - 1 - w0) & 3
+            const int here = ((u - 1 - w0 + kConvRing) & (kConvRing - 1)) * 64;
+            // the first step computes no tile and the last pass may hold steps past the end of the wave's tiles:
+            // they skip the matrix work (a wave-uniform branch without memory instructions inside) and store
+            // out of range
+            const int tile0 = (s0 + u - 1) * kConvTile;               // relative to `first`
             mfma_f4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (s0 + u >= 1 && tile0 < mine) {
+                // rows of the first and the last output of this lane's block, as sample ranges relative to `first`
+                const int o0 = tile0 + 16 * n + lead;                 // relative to the start of row0
+                const int ra = o0 / T;
+                const int lo_a = ra * T - lead, rb_more = (o0 - ra * T + 15 >= T) ? T : 0;
+                auto multiply = [&](mfma_f4 d, int g, int lo) -> mfma_f4 {
+                    const int q = tile0 + wq + 16 * g;                // first sample of the quad
+                    const bool ok = q >= lo && q < lo + T;
+                    const float4 xv = ring[ok ? ((here + opnd[g]) & (kConvRing * 64 - 1)) : kZero];
+                    d = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][0], xv.x, d, 0, 0, 0);
+                    d = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][1], xv.y, d, 0, 0, 0);
+                    d = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][2], xv.z, d, 0, 0, 0);
+                    return __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][3], xv.w, d, 0, 0, 0);
+                };
+                // every block sees the row of its first output (conv) or of its last output (corr) ...
+                const int lo_full = lo_a + (CORR ? rb_more : 0);
 #pragma unroll
-            for (int g = 0; g < G; ++g) {
-                const float4 xv = x[(u + g) % RING];
-                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][0], xv.x, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][1], xv.y, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][2], xv.z, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][3], xv.w, acc, 0, 0, 0);
+                for (int g = 0; g < G; ++g) acc = multiply(acc, g, lo_full);
+                // ... and the outputs of a block's other row take their own view.  They are the last outputs
+                // of the previous row (corr) or the first ones of the next row (conv), and inside their row their
+                // window holds samples of this block only: one window group, the block itself.
+                if (__any(rb_more != 0)) {
+                    mfma_f4 other = {0.0f, 0.0f, 0.0f, 0.0f};
+                    other = multiply(other, CORR ? 0 : G - 1, lo_a + (CORR ? 0 : rb_more));
+                    const bool in_next = (tile0 + 16 * n + 4 * kq) >= lo_a + T;      // this lane's output quad
+                    const bool take = rb_more != 0 && in_next != CORR;
+                    acc[0] = take ? other[0] : acc[0];
+                    acc[1] = take ? other[1] : acc[1];
+                    acc[2] = take ? other[2] : acc[2];
+                    acc[3] = take ? other[3] : acc[3];
+                }
             }
-            // tiles past the end of the span (the last pass of the loop may hold some) store nothing
-            const int t = t0 + 16 * u + 4 * kq;
-            buf_store4<false>(dst, (row_ok && t < tend) ? row_off + t * 4 : kOutOfRange,
+            const int t = tile0 + 16 * n + 4 * kq;
+            buf_store4<false>(dst, (s0 + u >= 1 && t < mine) ? (t + kConvTile) * 4 : kOutOfRange,
                               make_float4(acc[0] * ts, acc[1] * ts, acc[2] * ts, acc[3] * ts));
-            x[u] = load(first + (t0 - tbeg) + 16 * (u + RING));
         }
     }
 }
@@ -188,23 +250,18 @@ __global__ __launch_bounds__(kWave) void conv_mfma_kernel(float* __restrict__ ou
 template <bool CORR>
 static int conv_mfma_launch(float* out, const float* in, const float* filt, int K, float ts, int64_t M, int64_t T,
                             hipStream_t stream) {
-    const int64_t rowgroups = (M + 15) / 16;
-    // about four waves per SIMD on 256 compute units when the rows alone do not provide them; a span is a
-    // whole number of loop passes (RING tiles of 16 outputs) and is preceded by KPAD samples of warm-up
-    const int64_t pass = 16 * (K <= 64 ? 8 : 16);
-    int64_t spans = (4096 + rowgroups - 1) / rowgroups;
-    const int64_t max_spans = (T + pass - 1) / pass;
-    if (spans > max_spans) spans = max_spans;
-    if (spans < 1) spans = 1;
-    const int64_t span = (((T + spans - 1) / spans) + pass - 1) / pass * pass;
-    spans = (T + span - 1) / span;
-    const int64_t blocks = rowgroups * spans;
+    // about eight thousand waves (four per SIMD on 256 compute units, twice over), each a whole number of loop
+    // passes of consecutive tiles; every wave reads one tile more than it writes
+    const int64_t total = M * T;
+    const int64_t tiles = (total + kConvTile - 1) / kConvTile;
+    int64_t per_wave = (tiles / 8192 + kConvRing - 1) / kConvRing * kConvRing;
+    if (per_wave < kConvRing) per_wave = kConvRing;
+    if (per_wave > 64) per_wave = 64;
+    const int64_t blocks = (tiles + per_wave - 1) / per_wave;
     if (blocks > 0x7fffffffLL) return SLAYER_ERANGE;
-    // No non-temporal accesses here: a load or store covers 64 bytes per row, half a cache line, and the caches
-    // put the halves together (measured: non-temporal accesses cost 25-85 % on large tensors).
 #define SLAYER_CONV_MFMA(KP)                                                                                      \
     hipLaunchKernelGGL((conv_mfma_kernel<KP, CORR>), dim3((unsigned)blocks), dim3(kWave), 0, stream, out, in, filt, \
-                       K, ts, M, (int)T, (int)span, (unsigned)spans)
+                       K, ts, total, (int)T, (int)per_wave)
     if (K <= 16) SLAYER_CONV_MFMA(16);
     else if (K <= 32) SLAYER_CONV_MFMA(32);
     else if (K <= 64) SLAYER_CONV_MFMA(64);
@@ -221,7 +278,7 @@ static int conv_launch(float* out, const float* in, const float* filt, int64_t K
     if (!out || !in || !filt) return SLAYER_ENULL;
     if (K < 1) return SLAYER_EINVAL;
     if (K > kMaxTaps) return SLAYER_ERANGE;
-    if (K > 8 && K <= 128 && T % 4 == 0 && T <= (1 << 22) && aligned16(out) && aligned16(in))
+    if (K > 8 && K <= 128 && T % 4 == 0 && T >= 16 && T <= (1 << 22) && aligned16(out) && aligned16(in))
         return conv_mfma_launch<CORR>(out, in, filt, (int)K, ts, M, T, stream);
     const unsigned segs = (unsigned)((T + kSeg - 1) / kSeg);
     const int64_t blocks = M * (int64_t)segs;

@@ -102,30 +102,61 @@ def test_conv_corr(slayer, shape, K):
 
 @pytest.mark.parametrize('shape,K', [((16, 64), 9), ((5, 3, 16), 16), ((37, 132), 17), ((3, 700, 48), 32), ((2, 9, 1000), 33),
                                      ((64, 256, 100), 64), ((1, 20, 2048), 64), ((130, 4), 64), ((50, 260), 65),
-                                     ((7, 11, 300), 100), ((33, 520), 128), ((33, 520), 129), ((4, 12), 40)])
+                                     ((7, 11, 300), 100), ((33, 520), 128), ((33, 520), 129), ((4, 12), 40),
+                                     ((50, 16), 64), ((40, 20), 17), ((700, 36), 128), ((33, 148), 100),
+                                     ((4000, 300), 64), ((3, 5, 1500), 64), ((5, 2, 4096), 9), ((1, 1, 16), 16),
+                                     ((2, 1021, 256), 33), ((300, 1028), 16)])
 def test_conv_corr_matrix_core_path(slayer, shape, K):
-    """Tap counts either side of every padded size of the matrix-core kernel (16, 32, 64, 128) and of its
-    limits (8 < K <= 128), row counts that are not multiples of 16, rows shorter than a tile and than the
-    filter, rows split into several spans, and a signed filter; float64 numpy.convolve as the judge."""
+    """The matrix-core kernel walks the tensor as one stream of 256-sample tiles.  Tap counts either side of every
+    padded size (16, 32, 64, 128) and of the kernel's limits (8 < K <= 128, T >= 16); rows shorter than a block, a
+    tile or the filter (several rows in one window), rows that end inside a 16-sample block (T % 16 != 0: the
+    two-view tiles) and on one, tensors of one tile and of thousands (several waves, each starting mid-row), a
+    signed filter.  Every row against scipy.signal.lfilter in float64."""
+    from scipy.signal import lfilter
     gen = torch.Generator().manual_seed(seed_of('mfma conv', shape, K))
     x = torch.randn(shape, generator=gen)
     f = torch.randn(K, generator=gen)
     T = shape[-1]
     rows = x.reshape(-1, T).double().numpy()
     fd = f.double().numpy()
+    conv_ref = lfilter(fd, [1.0], rows, axis=-1)
+    corr_ref = lfilter(fd, [1.0], rows[:, ::-1], axis=-1)[:, ::-1]
+    assert np.allclose(conv_ref[0], np.convolve(rows[0], fd)[:T]) and \
+        np.allclose(corr_ref[-1], np.convolve(rows[-1][::-1], fd)[:T][::-1])
     for ts in (1, 0.25):
         y = slayer.utils.filter.conv(x.to(dev()), f.to(dev()), ts).reshape(-1, T).cpu().double().numpy()
         z = slayer.utils.filter.corr(x.to(dev()), f.to(dev()), ts).reshape(-1, T).cpu().double().numpy()
         scale = ts * np.abs(fd).sum() * np.abs(rows).max()
-        for r in (0, rows.shape[0] // 2, rows.shape[0] - 1):
-            want = ts * np.convolve(rows[r], fd)[:T]
-            assert np.abs(y[r] - want).max() <= 1e-5 * scale, (shape, K, r)
-            want = ts * np.convolve(rows[r][::-1], fd)[:T][::-1]
-            assert np.abs(z[r] - want).max() <= 1e-5 * scale, (shape, K, r)
+        assert np.abs(y - ts * conv_ref).max() <= 1e-5 * scale, (shape, K, 'conv')
+        assert np.abs(z - ts * corr_ref).max() <= 1e-5 * scale, (shape, K, 'corr')
     # non-negative data (no cancellation): the elementwise tolerance against the oracle holds as well
     xp, fp = x.abs(), f.abs()
     assert_rel(slayer.utils.filter.conv(xp.to(dev()), fp.to(dev()), 1), O.conv_fwd(xp, fp, 1), f'conv {shape} K={K}')
     assert_rel(slayer.utils.filter.corr(xp.to(dev()), fp.to(dev()), 1), O.conv_bwd(xp, fp, 1), f'corr {shape} K={K}')
+
+
+@pytest.mark.parametrize('T,K', [(300, 64), (304, 16), (20, 100), (1500, 33)])
+def test_conv_rows_do_not_see_each_other(slayer, T, K):
+    """A row's window is cut at the row: an Inf at the end (start) of one row leaves every other row finite and
+    unchanged in conv (corr); inside its own row it arrives where the filter carries it."""
+    gen = torch.Generator().manual_seed(seed_of('rows', T, K))
+    M = 97
+    x = torch.randn(M, T, generator=gen)
+    f = torch.randn(K, generator=gen)
+    base_c = slayer.utils.filter.conv(x.to(dev()), f.to(dev()), 1).cpu()
+    base_r = slayer.utils.filter.corr(x.to(dev()), f.to(dev()), 1).cpu()
+    for r in (0, 41, M - 1):
+        bad = x.clone()
+        bad[r, T - 1] = float('inf')
+        y = slayer.utils.filter.conv(bad.to(dev()), f.to(dev()), 1).cpu()
+        others = [i for i in range(M) if i != r]
+        assert torch.equal(y[others], base_c[others]), f'conv: row {r} leaked'
+        assert not torch.isfinite(y[r, T - 1])
+        bad = x.clone()
+        bad[r, 0] = float('inf')
+        z = slayer.utils.filter.corr(bad.to(dev()), f.to(dev()), 1).cpu()
+        assert torch.equal(z[others], base_r[others]), f'corr: row {r} leaked'
+        assert not torch.isfinite(z[r, 0])
 
 
 def test_conv_autograd_is_corr(slayer):
