@@ -367,12 +367,38 @@ __device__ __forceinline__ void scan_affine_complex(Cx& A, Cx& B) {
 #undef SLAYER_COMBINE
 }
 
-template <bool PARTIAL, bool STREAM>
+// SURR = 0: g_re / g_im are the incoming gradients of the two states (resonator backward).
+// SURR = 1 (binary spikes) / 2 (graded): the fused resonate-and-fire backward -- g_re holds the gradient of the
+// spikes, g_im is not read, and the gradients of the states come from the complex spike surrogate of the saved
+// states, evaluated as the quads arrive (same expression order as cspike_bwd_kernel, so the result equals the
+// chain surrogate -> resonator scan bit for bit); re / im are then read whether or not the sums are wanted.
+struct SpikeSurrogate { float thr, tau, rho; };
+
+template <int SURR>
+__device__ __forceinline__ void complex_spike_surrogate(const SpikeSurrogate& k, float g, float r, float i,
+                                                        float& g_re, float& g_im) {
+    const float half_over_tau = (1.0f / 2.0f) / k.tau;
+    const float two_tau = 2.0f * k.tau;
+    const float neg_rho_over_tau = (-k.rho) / k.tau;
+    float d_re;
+    if (SURR == 2) d_re = expf(-fmaxf(k.thr - r, 0.0f) / k.tau);
+    else d_re = half_over_tau * expf(-fabsf(r - k.thr) / k.tau);
+    const float d_im = half_over_tau * expf(-fabsf(i) / k.tau);
+    const float dr = r - k.thr;
+    const float sg_r = dr > 0.0f ? 1.0f : (dr < 0.0f ? -1.0f : (dr == 0.0f ? 0.0f : dr));
+    const float sg_i = i > 0.0f ? 1.0f : (i < 0.0f ? -1.0f : (i == 0.0f ? 0.0f : i));
+    const float step_re = 0.5f * (1.0f + sg_r * (1.0f - two_tau * d_re));
+    g_re = g * ((k.rho * d_re) * d_im);
+    g_im = g * (((neg_rho_over_tau * sg_i) * d_im) * step_re);
+}
+
+template <bool PARTIAL, bool STREAM, int SURR>
 __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
         float* __restrict__ g_re_in, float* __restrict__ g_im_in, float* __restrict__ partial_sin,
         float* __restrict__ partial_cos, const float* __restrict__ g_re, const float* __restrict__ g_im,
         const float* __restrict__ re, const float* __restrict__ im, const float* __restrict__ sin_decay,
-        const float* __restrict__ cos_decay, int64_t M, int QR, int rpg, unsigned npb, unsigned per_param) {
+        const float* __restrict__ cos_decay, SpikeSurrogate surr, int64_t M, int QR, int rpg, unsigned npb,
+        unsigned per_param) {
     __shared__ float c_tab[kScanMaxRows], s_tab[kScanMaxRows];
     __shared__ float sum_s[kScanWaves][kScanMaxRows], sum_c[kScanWaves][kScanMaxRows];
     __shared__ ComplexStage L;
@@ -381,9 +407,11 @@ __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
     const int nq = sp.nq;
     const int64_t base = sp.row0 * (int64_t)QR * 4;
     const unsigned span_bytes = (unsigned)nq * 16u;
-    const __amdgpu_buffer_rsrc_t src_gr = make_rsrc(g_re + base, span_bytes), src_gi = make_rsrc(g_im + base, span_bytes);
-    const __amdgpu_buffer_rsrc_t src_re = make_rsrc(PARTIAL ? re + base : nullptr, PARTIAL ? span_bytes : 0u);
-    const __amdgpu_buffer_rsrc_t src_im = make_rsrc(PARTIAL ? im + base : nullptr, PARTIAL ? span_bytes : 0u);
+    constexpr bool kStates = PARTIAL || SURR != 0;          // the saved states are read
+    const __amdgpu_buffer_rsrc_t src_gr = make_rsrc(g_re + base, span_bytes);
+    const __amdgpu_buffer_rsrc_t src_gi = make_rsrc(SURR == 0 ? g_im + base : nullptr, SURR == 0 ? span_bytes : 0u);
+    const __amdgpu_buffer_rsrc_t src_re = make_rsrc(kStates ? re + base : nullptr, kStates ? span_bytes : 0u);
+    const __amdgpu_buffer_rsrc_t src_im = make_rsrc(kStates ? im + base : nullptr, kStates ? span_bytes : 0u);
     const __amdgpu_buffer_rsrc_t dst_r = make_rsrc(g_re_in + base, span_bytes), dst_i = make_rsrc(g_im_in + base, span_bytes);
 
     struct Quads { float4 gr, gi, re, im; };
@@ -391,9 +419,9 @@ __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
         const int off = (unsigned)q < (unsigned)nq ? q * 16 : kOutOfRange;
         Quads x;
         x.gr = buf_load4<STREAM>(src_gr, off);
-        x.gi = buf_load4<STREAM>(src_gi, off);
-        x.re = PARTIAL ? buf_load4<STREAM>(src_re, off) : make_float4(0.f, 0.f, 0.f, 0.f);
-        x.im = PARTIAL ? buf_load4<STREAM>(src_im, off) : make_float4(0.f, 0.f, 0.f, 0.f);
+        x.gi = SURR == 0 ? buf_load4<STREAM>(src_gi, off) : make_float4(0.f, 0.f, 0.f, 0.f);
+        x.re = kStates ? buf_load4<STREAM>(src_re, off) : make_float4(0.f, 0.f, 0.f, 0.f);
+        x.im = kStates ? buf_load4<STREAM>(src_im, off) : make_float4(0.f, 0.f, 0.f, 0.f);
         return x;
     };
     const int q0 = sp.first_quad();
@@ -417,6 +445,13 @@ __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
         const bool active = cur.lq < nq;
         const bool row_end = cur.pos == QR - 1;
         const Cx mu{c_tab[cur.r], -s_tab[cur.r]};
+        if (SURR != 0) {                   // quads outside the span hold zeros: their gradient is zero too
+            const float4 g = x.gr;
+            complex_spike_surrogate<SURR>(surr, g.x, x.re.x, x.im.x, x.gr.x, x.gi.x);
+            complex_spike_surrogate<SURR>(surr, g.y, x.re.y, x.im.y, x.gr.y, x.gi.y);
+            complex_spike_surrogate<SURR>(surr, g.z, x.re.z, x.im.z, x.gr.z, x.gi.z);
+            complex_spike_surrogate<SURR>(surr, g.w, x.re.w, x.im.w, x.gr.w, x.gi.w);
+        }
         // the quad by itself
         const Cx d0{x.gr.x, x.gi.x}, d1{x.gr.y, x.gi.y}, d2{x.gr.z, x.gi.z}, d3{x.gr.w, x.gi.w};
         const Cx h3 = d3, h2 = cfma(mu, h3, d2), h1 = cfma(mu, h2, d1), h0 = cfma(mu, h1, d0);
@@ -549,18 +584,26 @@ int launch_cuba_bwd_scan(float* grad_in, float* partial_i, float* partial_v, con
     return (int)hipGetLastError();
 }
 
+// surrogate: 0 = g_re / g_im are the gradients of the states; 1 / 2 = g_re is the gradient of binary / graded
+// spikes (g_im unused) and spike_thr, tau, rho parametrise the complex spike surrogate.
 int launch_res_bwd_scan(float* g_re_in, float* g_im_in, float* partial_sin, float* partial_cos, const float* g_re,
                         const float* g_im, const float* re, const float* im, const float* sin_decay,
-                        const float* cos_decay, int64_t M, int64_t npb, int64_t num_decays, int64_t T,
-                        hipStream_t stream) {
+                        const float* cos_decay, int surrogate, float spike_thr, float tau, float rho, int64_t M,
+                        int64_t npb, int64_t num_decays, int64_t T, hipStream_t stream) {
     const ScanGrid g = scan_grid(M, T);
     if (!g.ok) return SLAYER_ERANGE;
-#define SLAYER_SCAN(P, S)                                                                                        \
-    hipLaunchKernelGGL((res_bwd_scan_kernel<P, S>), g.grid, dim3(kScanQuads), 0, stream, g_re_in, g_im_in,          \
-                       partial_sin, partial_cos, g_re, g_im, re, im, sin_decay, cos_decay, M, g.QR, g.rpg,       \
+    const SpikeSurrogate k{spike_thr, tau, rho};
+#define SLAYER_SCAN(P, S, U)                                                                                     \
+    hipLaunchKernelGGL((res_bwd_scan_kernel<P, S, U>), g.grid, dim3(kScanQuads), 0, stream, g_re_in, g_im_in,       \
+                       partial_sin, partial_cos, g_re, g_im, re, im, sin_decay, cos_decay, k, M, g.QR, g.rpg,    \
                        (unsigned)npb, rows_per_param(npb, num_decays))
-    if (partial_sin) { if (g.streaming) SLAYER_SCAN(true, true); else SLAYER_SCAN(true, false); }
-    else { if (g.streaming) SLAYER_SCAN(false, true); else SLAYER_SCAN(false, false); }
+#define SLAYER_SCAN_S(P, U) do { if (g.streaming) SLAYER_SCAN(P, true, U); else SLAYER_SCAN(P, false, U); } while (0)
+#define SLAYER_SCAN_P(U) do { if (partial_sin) SLAYER_SCAN_S(true, U); else SLAYER_SCAN_S(false, U); } while (0)
+    if (surrogate == 0) SLAYER_SCAN_P(0);
+    else if (surrogate == 1) SLAYER_SCAN_P(1);
+    else SLAYER_SCAN_P(2);
+#undef SLAYER_SCAN_P
+#undef SLAYER_SCAN_S
 #undef SLAYER_SCAN
     return (int)hipGetLastError();
 }

@@ -129,3 +129,35 @@ def test_fused_backward_scans_equal_the_chain_of_scans_bit_for_bit(slayer, shape
         if need:
             assert_rel(g_i, r_gi.cpu(), 'grad current decay', rel=1e-4)
             assert_rel(g_v, r_gv.cpu(), 'grad voltage decay', rel=1e-4)
+
+
+@pytest.mark.parametrize('shape', [(5, 1024, 300), (2, 16, 33, 31, 76), (3, 43, 8196)])
+@pytest.mark.parametrize('graded', [False, True])
+def test_fused_rf_backward_scan_equals_the_chain_of_scans_bit_for_bit(slayer, shape, graded):
+    """Complex spike surrogate + resonator backward scan in one kernel against the two operators in a row (same
+    arithmetic, same spans), and the surrogate + oracle loop on a slab."""
+    D = slayer.neuron.dynamics
+    C = slayer.spike.complex
+    gen = torch.Generator().manual_seed(seed_of('rf-scan', shape, graded))
+    n = shape[1]
+    g = torch.randn(shape, generator=gen).to(dev())
+    re = (torch.randn(shape, generator=gen) * 1.5).to(dev())
+    im = torch.randn(shape, generator=gen).to(dev())
+    decay = torch.randint(40, 4096, (n,), generator=gen).float()
+    phi = 2 * 3.141592653589793 * torch.rand(n, generator=gen)
+    sin = ((4096 - decay) * torch.sin(phi)).round().to(dev())
+    cos = ((4096 - decay) * torch.cos(phi)).round().to(dev())
+    thr, tau, rho = 1.0, 0.7, 1.3
+    for need in (True, False):
+        g_re, g_im, g_sin, g_cos = D.rf_fused._bwd(g, re, im, sin, cos, thr, tau, rho, graded, need)
+        s_re, s_im = C._bwd(g, re, im, None, thr, tau, rho, graded)
+        r_re, r_im, r_sin, r_cos = D.resonator._bwd(s_re, s_im, re, im, sin, cos, need)
+        assert torch.equal(g_re, r_re) and torch.equal(g_im, r_im), f'fused RF scan differs from the chain ({need})'
+        if need:
+            assert_rel(g_sin, r_sin.cpu(), 'grad sin', rel=1e-4)
+            assert_rel(g_cos, r_cos.cpu(), 'grad cos', rel=1e-4)
+    k = min(shape[0], 2)
+    o_re, o_im = O.cspike_bwd(g[:k].cpu(), re[:k].cpu(), im[:k].cpu(), thr, tau, rho, graded)
+    want = O.res_bwd(o_re, o_im, re[:k].cpu(), im[:k].cpu(), sin.cpu(), cos.cpu())
+    assert_scale(g_re[:k], want[0], 'grad real vs oracle')
+    assert_scale(g_im[:k], want[1], 'grad imag vs oracle')
