@@ -64,7 +64,12 @@ class _corr(torch.autograd.Function):
 
 def conv(input, filter, sampling_time=1):
     """Convolution in time; the last axis of ``input`` is time, ``filter`` is
-    flattened to 1-D.  Output has the shape of ``input``."""
+    flattened to 1-D.  Output has the shape of ``input``.
+
+    Two deviations from the reference: filters longer than 4096 taps raise (the reference accepts any
+    length), and for filters of 9 to 128 taps a non-finite input sample also makes the few neighbouring
+    outputs of its row NaN whose window holds it beyond the filter's support (the matrix-core kernel
+    multiplies those samples by zero taps instead of skipping them); finite inputs give the same sums."""
     if input.dim() == 1:
         input = input.reshape(1, -1)
     return _conv.apply(input, filter.flatten(), sampling_time)

@@ -52,7 +52,14 @@ def custom_recurrent(z, neuron, recurrent_synapse):
     """Spikes of the recurrent layer for the dendrite input ``z`` ([N, C, T]).  The neuron must keep
     its state between calls (``persistent_state=True``); its state after the call is that of the
     last step.  Gradients reach ``z`` and the recurrent weights; as in the reference, the state the
-    neuron carries from one step to the next is treated as a constant."""
+    neuron carries from one step to the next is treated as a constant.
+
+    The one-launch kernel adds the feedback row by row in the order the neurons fired, 16 at a time, where
+    the reference's loop calls ``torch.matmul``.  The two sums are the same bits whenever every partial sum
+    is exactly representable in float32, which holds for quantised recurrent weights (multiples of a power
+    of two of moderate size, what the synapse's ``pre_hook_fx`` quantiser produces).  With unquantised
+    weights the sums can differ in the last bit and a dendrite value within that distance of the threshold
+    may spike in one and not in the other; no fixture of the reference pins that case."""
     recurrent_mat = _recurrent_matrix(recurrent_synapse)
     if _fusable(z, neuron):
         return _FusedRecurrent.apply(z, neuron, recurrent_mat)
