@@ -9,6 +9,7 @@ struct AthFwd {
     static constexpr int kIn = 1, kOut = 2;      // out: threshold trace, refractory trace
     static constexpr bool kReverse = false;
     static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
+    static constexpr bool kMultiwaveWhenLarge = true;
     struct Params {
         const float* in[1];
         float* out[2];

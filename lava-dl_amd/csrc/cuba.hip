@@ -30,6 +30,7 @@ struct CubaFwd {
     static constexpr bool kReverse = false;
     static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
     static constexpr bool kLongPiecesOnAliasedRows = true;
+    static constexpr bool kMultiwaveWhenLarge = !SHIFT;
     struct Params {
         const float* in[1];
         float* out[kOut + 1];

@@ -12,6 +12,7 @@ struct LiFwd {
     static constexpr bool kReverse = false;
     static constexpr int64_t kRows32Below = 32768, kRows16Below = 8192;
     static constexpr bool kLongPiecesOnAliasedRows = true;
+    static constexpr bool kMultiwaveWhenLarge = true;
     struct Params {
         const float* in[1];
         float* out[1];

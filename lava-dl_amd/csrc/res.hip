@@ -13,6 +13,7 @@ struct ResFwd {
     static constexpr int kIn = 2, kOut = 2;
     static constexpr bool kReverse = false;
     static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
+    static constexpr bool kMultiwaveWhenLarge = true;
     struct Params {
         const float* in[2];
         float* out[2];

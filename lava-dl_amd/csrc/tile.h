@@ -1000,19 +1000,62 @@ struct LongPiecesOnAliasedRows<Op, decltype((void)Op::kLongPiecesOnAliasedRows)>
     static constexpr bool value = Op::kLongPiecesOnAliasedRows;
 };
 
+// Ops that also take the multi-wave kernel when their workgroups outnumber the compute units' slots
+// (kMultiwaveWhenLarge): the integer forward recurrences, whose one-wave kernel does copies and recurrence
+// one after the other in the same wave.  Measured on [4,16,8192,300] / [4,16,2048,1000] / [4,16,1024,2000]
+// tensors against the one-wave kernel: LI 262 -> 248 / 216 -> 212 / 220 -> 217 us, fused CUBA 542 -> 496 /
+// 454 -> 436 / 453 -> 451, adaptive threshold 396 -> 377 / 336 -> 326 / 340 -> 339, resonator 525 -> 515 /
+// 446 -> 436 / 466 -> 467, fused RF 700 -> 653 / 621 -> 584 / 609 -> 603, fused ALIF 698 -> 681 / 608 -> 583 /
+// 611 -> 598.
+template <class Op, class = void>
+struct MultiwaveWhenLarge { static constexpr bool value = false; };
+template <class Op>
+struct MultiwaveWhenLarge<Op, decltype((void)Op::kMultiwaveWhenLarge)> {
+    static constexpr bool value = Op::kMultiwaveWhenLarge;
+};
+
+// Workgroups of the multi-wave kernel a compute unit should hold when they come in several rounds: the fewer
+// rows the chip works on at a time, the closer together its memory accesses fall (a plain copy in this access
+// pattern gains 10-20 % when the rows in flight drop from all of the tensor to a tenth of it), but a
+// workgroup spends its first microseconds waiting for its first tiles and others must cover for it.
+constexpr int kGroupsPerCuWhenLarge = 4;
+
+// Dynamic LDS (unused by the kernel) that holds a kernel with `static_lds` bytes to `groups` workgroups per CU.
+inline unsigned lds_pad_for(int groups, size_t static_lds) {
+    const size_t lds_per_cu = 160 * 1024, want = lds_per_cu / (size_t)(groups + 1) + 256;   // too much for groups + 1
+    if (static_lds >= want) return 0;
+    const size_t pad = want - static_lds;
+    return (unsigned)(pad > 60 * 1024 ? 60 * 1024 : pad);
+}
+template <class Op, int R, bool STREAM>
+unsigned duo_pad_when_large() {
+    static const unsigned pad = [] {
+        hipFuncAttributes a;
+        if (hipFuncGetAttributes(&a, (const void*)stream_kernel_duo<Op, R, STREAM, CopyWaves<Op>::value>) != hipSuccess)
+            return 0u;
+        return lds_pad_for(kGroupsPerCuWhenLarge, a.sharedSizeBytes);
+    }();
+    return pad;
+}
+
 template <class Op>
 int launch_stream(const typename Op::Params& prm, int64_t M, int64_t T, hipStream_t stream) {
     if (M == 0 || T == 0) return 0;
     const bool vec = stream_vectorizes<Op>(prm, T);
     const bool streaming = stream_is_large(M, T);
-    if (stream_fits_multiwave<Op>(prm, M, T)) {
+    const bool resident = stream_fits_multiwave<Op>(prm, M, T);
+    const bool long_pieces = LongPiecesOnAliasedRows<Op>::value && row_stride_aliases(T);
+    if (resident || (vec && MultiwaveWhenLarge<Op>::value && !long_pieces)) {
         constexpr int RD = DuoRows<Op>::value;
         constexpr int NC = CopyWaves<Op>::value;
         const dim3 grid((unsigned)((M + RD - 1) / RD)), block((1 + NC) * kWave);
-        if (streaming)
-            hipLaunchKernelGGL((stream_kernel_duo<Op, RD, true, NC>), grid, block, 0, stream, prm, M, (int)T);
-        else
-            hipLaunchKernelGGL((stream_kernel_duo<Op, RD, false, NC>), grid, block, 0, stream, prm, M, (int)T);
+        if (streaming) {
+            const unsigned pad = resident ? 0u : duo_pad_when_large<Op, RD, true>();
+            hipLaunchKernelGGL((stream_kernel_duo<Op, RD, true, NC>), grid, block, pad, stream, prm, M, (int)T);
+        } else {
+            const unsigned pad = resident ? 0u : duo_pad_when_large<Op, RD, false>();
+            hipLaunchKernelGGL((stream_kernel_duo<Op, RD, false, NC>), grid, block, pad, stream, prm, M, (int)T);
+        }
         return (int)hipGetLastError();
     }
     if (M < Op::kRows16Below || (LongPiecesOnAliasedRows<Op>::value && row_stride_aliases(T)))
