@@ -84,6 +84,78 @@ struct AlifFwd {
         o[kTheta] = __int_as_float(th_out);
         o[kSpk] = __int_as_float(r_out);
     }
+    // The same step as two Ops for the staged multi-wave kernel: current and voltage recurrences, and the
+    // threshold / refractory recurrences reading the voltage out of its tile one chunk later.
+    static constexpr int kStages = 2;
+    struct Stage0 {
+        static constexpr int kIn = 1, kOut = KEEP_CURRENT ? 2 : 1;
+        static constexpr bool kReverse = false, kTileMapped = true;
+        static constexpr int in_tile(int) { return 0; }
+        static constexpr int out_tile(int o) { return o; }       // [current,] voltage: tiles 0 .. kVol
+        int yc, yv, mi, mv;
+        float w, inv_w;
+        __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
+            w = p.w; inv_w = p.inv_w; yc = yv = mi = mv = 0;
+            if (valid) {
+                yc = trunc_i32(p.i_state[p.n_is == 1 ? 0 : m] * w);
+                yv = trunc_i32(p.v_state[p.n_vs == 1 ? 0 : m] * w);
+                mi = 4096 - trunc_i32(rintf(p.i_decay[param_index(m, p.npb, p.n_id)]));
+                mv = 4096 - trunc_i32(rintf(p.v_decay[param_index(m, p.npb, p.n_vd)]));
+            }
+        }
+        __device__ __forceinline__ void step(const float (&x)[1], float (&o)[kOut]) {
+            yc = rs0_12(yc, mi) + __float_as_int(x[0]);
+            const float cf = (float)yc;
+            yv = rs0_12(yv, mv) + (POW2 ? trunc_i32(cf) : trunc_i32(w * (cf / w)));
+            if (KEEP_CURRENT) o[0] = __int_as_float(yc);
+            o[kVol] = __int_as_float(yv);
+        }
+        __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
+            if (valid && p.cur_last) p.cur_last[m] = from_state<POW2>(__int_as_float(yc), w, inv_w);
+            if (valid && p.vol_last) p.vol_last[m] = from_state<POW2>(__int_as_float(yv), w, inv_w);
+        }
+    };
+    struct Stage1 {
+        static constexpr int kIn = 1, kOut = 2;
+        static constexpr bool kReverse = false, kTileMapped = true;
+        static constexpr int in_tile(int) { return kVol; }
+        static constexpr int out_tile(int o) { return kTheta + o; }   // threshold, refractory state
+        int th, r, th_out, r_out, yv_last, mt, mr, th_step, base;
+        float w, inv_w, spike_scale;
+        __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
+            w = p.w; inv_w = p.inv_w; spike_scale = p.spike_scale; th_step = p.step; base = p.base;
+            th = r = th_out = r_out = yv_last = mt = mr = 0;
+            if (valid) {
+                th = trunc_i32(p.th_state[p.n_ts == 1 ? 0 : m] * w);
+                r = trunc_i32(p.ref_state[p.n_rs == 1 ? 0 : m] * w);
+                yv_last = trunc_i32(p.v_state[p.n_vs == 1 ? 0 : m] * w);
+                mt = 4096 - trunc_i32(rintf(p.th_decay[param_index(m, p.npb, p.n_td)]));
+                mr = 4096 - trunc_i32(rintf(p.ref_decay[param_index(m, p.npb, p.n_rd)]));
+            }
+        }
+        __device__ __forceinline__ void step(const float (&x)[1], float (&o)[2]) {
+            const int yv = __float_as_int(x[0]);
+            const float vf = (float)yv;
+            r = rs0_12(r, mr);
+            th = rs0_12(th - base, mt) + base;
+            th_out = th; r_out = r; yv_last = yv;
+            const bool fired = (POW2 ? trunc_i32(vf) : trunc_i32(w * (vf / w))) >= th + r;
+            r += fired ? 2 * th : 0;
+            th += fired ? th_step : 0;
+            o[0] = __int_as_float(th_out);
+            o[1] = __int_as_float(r_out);
+        }
+        __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
+            const float thf = from_state<POW2>(__int_as_float(th_out), w, inv_w);
+            const float rf = from_state<POW2>(__int_as_float(r_out), w, inv_w);
+            if (valid && p.th_last) { p.th_last[m] = thf; p.ref_last[m] = rf; }
+            if (SHIFT && valid && p.shifts.last) {
+                const float vol = from_state<POW2>(__int_as_float(yv_last), w, inv_w);
+                const float h = (vol >= thf + rf) ? 1.0f : 0.0f;
+                p.shifts.last[m] = GRADED ? (h * vol) / spike_scale : h;
+            }
+        }
+    };
     __device__ __forceinline__ float spike(float vol, float theta) const {
         const float h = (vol >= theta) ? 1.0f : 0.0f;
         return GRADED ? (h * vol) / spike_scale : h;

@@ -73,6 +73,63 @@ struct CubaFwd {
         if (KEEP_CURRENT) o[0] = __int_as_float(yc);
         o[kVol] = __int_as_float(yn);
     }
+    // The same step as two Ops for the staged multi-wave kernel: the current recurrence, and the voltage
+    // recurrence reading the current out of its tile one chunk later.
+    static constexpr int kStages = 2;
+    static constexpr bool kStagedWhenLarge = !SHIFT;
+    struct Stage0 {
+        static constexpr int kIn = 1, kOut = 1;
+        static constexpr bool kReverse = false, kTileMapped = true;
+        static constexpr int in_tile(int) { return 0; }
+        static constexpr int out_tile(int) { return 0; }         // the current replaces the input in place
+        int yc, mi;
+        float w, inv_w;
+        __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
+            w = p.w; inv_w = p.inv_w; yc = mi = 0;
+            if (valid) {
+                yc = trunc_i32(p.i_state[p.n_is == 1 ? 0 : m] * w);
+                mi = 4096 - trunc_i32(rintf(p.i_decay[param_index(m, p.npb, p.n_id)]));
+            }
+        }
+        __device__ __forceinline__ void step(const float (&x)[1], float (&o)[1]) {
+            yc = rs0_12(yc, mi) + __float_as_int(x[0]);
+            o[0] = __int_as_float(yc);
+        }
+        __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
+            if (valid && p.cur_last) p.cur_last[m] = from_state<POW2>(__int_as_float(yc), w, inv_w);
+        }
+    };
+    struct Stage1 {
+        static constexpr int kIn = 1, kOut = 1;
+        static constexpr bool kReverse = false, kTileMapped = true;
+        static constexpr int in_tile(int) { return 0; }
+        static constexpr int out_tile(int) { return kVol; }      // without a current trace: in place
+        int yv, yv_out, mv, fire_above;
+        float w, inv_w, spike_thr, spike_scale;
+        __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
+            w = p.w; inv_w = p.inv_w; fire_above = p.fire_above; spike_thr = p.spike_thr; spike_scale = p.spike_scale;
+            yv = yv_out = mv = 0;
+            if (valid) {
+                yv = trunc_i32(p.v_state[p.n_vs == 1 ? 0 : m] * w);
+                mv = 4096 - trunc_i32(rintf(p.v_decay[param_index(m, p.npb, p.n_vd)]));
+            }
+        }
+        __device__ __forceinline__ void step(const float (&x)[1], float (&o)[1]) {
+            const float cf = (float)__float_as_int(x[0]);
+            const int yn = rs0_12(yv, mv) + (POW2 ? trunc_i32(cf) : trunc_i32(w * (cf / w)));
+            yv = (yn > fire_above) ? 0 : yn;
+            yv_out = yn;
+            o[0] = __int_as_float(yn);
+        }
+        __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
+            const float vol = from_state<POW2>(__int_as_float(yv_out), w, inv_w);
+            if (valid && p.vol_last) p.vol_last[m] = vol;
+            if (SHIFT && valid && p.shifts.last) {
+                const float h = (vol >= spike_thr) ? 1.0f : 0.0f;
+                p.shifts.last[m] = GRADED ? (h * vol) / spike_scale : h;
+            }
+        }
+    };
     __device__ __forceinline__ float spike(float vol) const {
         const float h = (vol >= spike_thr) ? 1.0f : 0.0f;
         return GRADED ? (h * vol) / spike_scale : h;

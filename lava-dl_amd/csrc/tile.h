@@ -17,6 +17,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 #include "../../include/slayer_hip.h"
 
 namespace slayer {
@@ -589,6 +590,19 @@ __device__ __forceinline__ int chunk_count(int a_lane, bool valid, int T) {
     return last + 1;
 }
 
+// Which tile an Op's i-th input / o-th output lives in: its own index, unless the Op is one stage of a
+// staged Op (kTileMapped) and names the tiles of the whole Op it reads and writes.
+template <class Op, class = void>
+struct TileMap {
+    static constexpr int in(int i) { return i; }
+    static constexpr int out(int o) { return o; }
+};
+template <class Op>
+struct TileMap<Op, decltype((void)Op::kTileMapped)> {
+    static constexpr int in(int i) { return Op::in_tile(i); }
+    static constexpr int out(int o) { return Op::out_tile(o); }
+};
+
 // The sequential part: lane = neuron, one chunk of the tiles in place.
 template <class Op, int R, int UNROLL, int S = kTileSamples>
 __device__ __forceinline__ void run_chunk(Op& op, float (*tile)[TileGeom<R, S>::kTileFloats], int lane, int chunk,
@@ -599,7 +613,7 @@ __device__ __forceinline__ void run_chunk(Op& op, float (*tile)[TileGeom<R, S>::
         float xin[NI][4], yout[NO][4];
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
-            const float4 v = *reinterpret_cast<const float4*>(&tile[i][lane * G::kPitch + 4 * qq]);
+            const float4 v = *reinterpret_cast<const float4*>(&tile[TileMap<Op>::in(i)][lane * G::kPitch + 4 * qq]);
             xin[i][0] = v.x; xin[i][1] = v.y; xin[i][2] = v.z; xin[i][3] = v.w;
         }
 #pragma unroll
@@ -614,7 +628,7 @@ __device__ __forceinline__ void run_chunk(Op& op, float (*tile)[TileGeom<R, S>::
         }
 #pragma unroll
         for (int o = 0; o < NO; ++o)
-            *reinterpret_cast<float4*>(&tile[o][lane * G::kPitch + 4 * qq]) =
+            *reinterpret_cast<float4*>(&tile[TileMap<Op>::out(o)][lane * G::kPitch + 4 * qq]) =
                 make_float4(yout[o][0], yout[o][1], yout[o][2], yout[o][3]);
     };
     if (inner) {
@@ -734,6 +748,81 @@ __global__ __launch_bounds__((1 + NCOPY) * kWave) void stream_kernel_duo(typenam
             __syncthreads();                                   // barrier k+2
         }
         io.copy_out(uni, tiles[1], chunk_of(nloop - 1));
+    }
+}
+
+// The multi-wave kernel for an Op whose step is a chain of two recurrences, the second reading what the
+// first produced (kStages = 2, Stage0 / Stage1: Ops of their own that name the tiles they read and write).
+// The two recurrences run in two waves, the second one chunk behind the first, so a step of the workgroup
+// costs the longer of the two instead of their sum; that is what bounds the kernel while all workgroups are
+// resident.  Three sets of tiles rotate:
+//   period j (between barriers j and j+1): wave 0 runs stage 0 on chunk j in tiles[j % 3], wave 1 runs stage 1
+//   on chunk j-1 in tiles[(j-1) % 3], the copy waves store chunk j-2 from tiles[(j+1) % 3], refill them with
+//   chunk j+1 and issue the loads of chunk j+4 (three chunks of loads in flight).
+// Every wave passes the same number of barriers; chunk numbers outside [0, nchunks) name no chunk.
+template <class Op, int R, bool STREAM, int NCOPY>
+__global__ __launch_bounds__((2 + NCOPY) * kWave) void stream_kernel_staged(typename Op::Params prm, int64_t M, int T) {
+    using G = TileGeom<R>;
+    constexpr int TC = G::kChunk;
+    constexpr int NI = Op::kIn, NO = Op::kOut, NT = NI > NO ? NI : NO;
+    constexpr int PASSES = G::kPasses / NCOPY;
+    static_assert(PASSES * NCOPY == G::kPasses, "copy waves share the passes evenly");
+    static_assert(Op::kStages == 2 && !Op::kReverse, "two forward stages");
+    __shared__ __attribute__((aligned(16))) float tiles[3][NT][G::kTileFloats];
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int role = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));   // wave-uniform
+    const int64_t m0 = (int64_t)blockIdx.x * R;
+    const int rows = (int)((M - m0) < R ? (M - m0) : R);
+    const unsigned base_f = (unsigned)(reinterpret_cast<uintptr_t>(prm.in[0]) >> 2);
+    const int a_lane = (int)((base_f + (unsigned)(m0 + lane) * (unsigned)T) & 31u);
+    const int nchunks = chunk_count<TC>(a_lane, lane < rows, T);
+    const int periods = (nchunks + 2 + 2) / 3 * 3;          // the last chunk leaves in period nchunks + 1
+    const int interior_end = (T & ~31) / TC;
+
+    auto sequential = [&](auto& stage, int lag) {
+        stage.init(prm, m0 + lane, lane < rows);
+        for (int j = 0; j < periods; j += 3) {
+#pragma unroll
+            for (int h = 0; h < 3; ++h) {
+                const int chunk = j + h - lag;
+                __syncthreads();                               // barrier j+h
+                if (chunk >= 0 && chunk < nchunks)
+                    run_chunk<typename std::remove_reference<decltype(stage)>::type, R, 4>(
+                        stage, tiles[(h + 3 - lag) % 3], lane, chunk, chunk >= 1 && chunk < interior_end, a_lane, T);
+            }
+        }
+        __syncthreads();                                       // barrier `periods`
+        stage.finish(prm, m0 + lane, lane < rows);
+    };
+    if (role == 0) {
+        typename Op::Stage0 st;
+        sequential(st, 0);
+    } else if (role == 1) {
+        typename Op::Stage1 st;
+        sequential(st, 1);
+    } else {
+        Op uni;                                                // wave-uniform members only (pre, post, derive)
+        uni.init(prm, 0, false);
+        Copier<Op, R, STREAM, PASSES> io;
+        io.init(prm, m0, rows, T, lane, base_f, (role - 2) * PASSES);
+        float4 fetched[3][NI][PASSES];
+#pragma unroll
+        for (int d = 0; d < 3; ++d) io.fetch_into(fetched[d], d);
+        io.prime_stores();
+        io.to_tiles(uni, tiles[0], fetched[0], 0);
+        io.fetch_into(fetched[0], 3);
+        __syncthreads();                                       // barrier 0
+        io.fill_unreached(prm, m0, lane);                      // while the first wave works on chunk 0
+        for (int j = 0; j < periods; j += 3) {
+#pragma unroll
+            for (int h = 0; h < 3; ++h) {
+                io.copy_out(uni, tiles[(h + 1) % 3], j + h - 2);
+                io.to_tiles(uni, tiles[(h + 1) % 3], fetched[(h + 1) % 3], j + h + 1);
+                io.fetch_into(fetched[(h + 1) % 3], j + h + 4);
+                __syncthreads();                               // barrier j+h+1
+            }
+        }
     }
 }
 
@@ -1038,13 +1127,69 @@ unsigned duo_pad_when_large() {
     return pad;
 }
 
+// Ops made of two chained recurrences (kStages = 2) run them in two waves while every workgroup of that
+// kernel is resident.
+template <class Op, class = void>
+struct StageCount { static constexpr int value = 1; };
+template <class Op>
+struct StageCount<Op, decltype((void)Op::kStages)> { static constexpr int value = Op::kStages; };
+
+template <class Op, bool STREAM>
+int staged_groups_per_cu() {
+    static const int n = [] {
+        int v = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&v, stream_kernel_staged<Op, 64, STREAM, CopyWaves<Op>::value>,
+                                                         (2 + CopyWaves<Op>::value) * kWave, 0) != hipSuccess)
+            v = 0;
+        return v;
+    }();
+    return n;
+}
+
+// Staged Ops that keep the staged kernel when its workgroups come in several rounds (kStagedWhenLarge).
+template <class Op, class = void>
+struct StagedWhenLarge { static constexpr bool value = false; };
+template <class Op>
+struct StagedWhenLarge<Op, decltype((void)Op::kStagedWhenLarge)> { static constexpr bool value = Op::kStagedWhenLarge; };
+
+// (fused CUBA forward, [4,16,8192,300] / [4,16,2048,1000] / [4,16,1024,2000]: 518 -> 494 / 452 -> 437 / 448 -> 443 us
+// against the two-wave form; the fused ALIF forward, whose nine to twelve tiles leave room for one workgroup per
+// compute unit, loses a quarter at T = 300 and stays with the two-wave form.)
+constexpr int kStagedGroupsPerCuWhenLarge = 3;
+template <class Op, bool STREAM>
+unsigned staged_pad_when_large() {
+    static const unsigned pad = [] {
+        hipFuncAttributes a;
+        if (hipFuncGetAttributes(&a, (const void*)stream_kernel_staged<Op, 64, STREAM, CopyWaves<Op>::value>) != hipSuccess)
+            return 0u;
+        return lds_pad_for(kStagedGroupsPerCuWhenLarge, a.sharedSizeBytes);
+    }();
+    return pad;
+}
+
 template <class Op>
 int launch_stream(const typename Op::Params& prm, int64_t M, int64_t T, hipStream_t stream) {
     if (M == 0 || T == 0) return 0;
     const bool vec = stream_vectorizes<Op>(prm, T);
     const bool streaming = stream_is_large(M, T);
-    const bool resident = stream_fits_multiwave<Op>(prm, M, T);
     const bool long_pieces = LongPiecesOnAliasedRows<Op>::value && row_stride_aliases(T);
+    if constexpr (StageCount<Op>::value == 2) {
+        const int per_cu = streaming ? staged_groups_per_cu<Op, true>() : staged_groups_per_cu<Op, false>();
+        const bool fits = (M + 63) / 64 <= (int64_t)per_cu * compute_units();
+        if (vec && per_cu > 0 && (fits || (StagedWhenLarge<Op>::value && !long_pieces))) {
+            constexpr int NC = CopyWaves<Op>::value;
+            const dim3 grid((unsigned)((M + 63) / 64)), block((2 + NC) * kWave);
+            if (streaming) {
+                const unsigned pad = fits ? 0u : staged_pad_when_large<Op, true>();
+                hipLaunchKernelGGL((stream_kernel_staged<Op, 64, true, NC>), grid, block, pad, stream, prm, M, (int)T);
+            } else {
+                const unsigned pad = fits ? 0u : staged_pad_when_large<Op, false>();
+                hipLaunchKernelGGL((stream_kernel_staged<Op, 64, false, NC>), grid, block, pad, stream, prm, M, (int)T);
+            }
+            return (int)hipGetLastError();
+        }
+    }
+    const bool resident = stream_fits_multiwave<Op>(prm, M, T);
     if (resident || (vec && MultiwaveWhenLarge<Op>::value && !long_pieces)) {
         constexpr int RD = DuoRows<Op>::value;
         constexpr int NC = CopyWaves<Op>::value;
