@@ -16,7 +16,8 @@ bool bwd_scan_usable(int64_t M, int64_t npb, int64_t T);                // scan.
 int launch_cuba_bwd_scan(float* grad_in, float* partial_i, float* partial_v, const float* grad_spikes,
                          const float* voltage, const float* theta, const float* current, const float* i_decay,
                          const float* v_decay, float spike_thr, float tau, float rho, bool graded,
-                         int64_t M, int64_t npb, int64_t n_id, int64_t n_vd, int64_t T, hipStream_t stream);   // scan.hip
+                         int64_t M, int64_t npb, int64_t n_id, int64_t n_vd, int64_t T, const Shifts* shifts,
+                         hipStream_t stream);   // scan.hip
 
 // KEEP_CURRENT = false leaves the current trace out (a caller that wants no decay gradient does not
 // need it): 12 instead of 16 bytes per neuron-timestep.
@@ -271,16 +272,16 @@ extern "C" int slayer_cuba_bwd(float* grad_in, float* grad_i_decay, float* grad_
     hipStream_t st = (hipStream_t)stream;
     if (M > 0 && T > 0) {
         if (!grad_in || !grad_spikes || !voltage || !i_decay || !v_decay || (want && !current)) return SLAYER_ENULL;
-        // large tensors without folded delays: the two recurrences as wave scans over a linear stream
-        if (!delays && bwd_scan_usable(M, neurons_per_batch, T) && aligned16(grad_in) && aligned16(grad_spikes) &&
+        const Shifts sh = backward_shifts(delays, neurons_per_batch);
+        // large tensors: the two recurrences as wave scans over a linear stream
+        if (bwd_scan_usable(M, neurons_per_batch, T) && aligned16(grad_in) && aligned16(grad_spikes) &&
             aligned16(voltage) && aligned16(current)) {
             if (int e = launch_cuba_bwd_scan(grad_in, want ? workspace : nullptr, want ? workspace + M : nullptr,
                                              grad_spikes, voltage, nullptr, want ? current : nullptr, i_decay, v_decay,
                                              spike_threshold, tau_rho, scale_rho, graded != 0, M, neurons_per_batch,
-                                             num_i_decays, num_v_decays, T, st))
+                                             num_i_decays, num_v_decays, T, delays ? &sh : nullptr, st))
                 return e;
         } else {
-        const Shifts sh = backward_shifts(delays, neurons_per_batch);
 #define SLAYER_CUBA_BWD_S(G, S)                                                                                  \
     do {                                                                                                         \
         if (want) {                                                                                              \

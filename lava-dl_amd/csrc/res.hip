@@ -156,7 +156,8 @@ bool bwd_scan_usable(int64_t M, int64_t npb, int64_t T);                // scan.
 int launch_res_bwd_scan(float* g_re_in, float* g_im_in, float* partial_sin, float* partial_cos, const float* g_re,
                         const float* g_im, const float* re, const float* im, const float* sin_decay,
                         const float* cos_decay, int surrogate, float spike_thr, float tau, float rho, int64_t M,
-                        int64_t npb, int64_t num_decays, int64_t T, hipStream_t stream);       // scan.hip
+                        int64_t npb, int64_t num_decays, int64_t T, const Shifts* shifts,
+                        hipStream_t stream);       // scan.hip
 
 }  // namespace slayer
 
@@ -220,7 +221,7 @@ extern "C" int slayer_res_bwd(float* g_re_in, float* g_im_in, float* grad_sin, f
             // large tensors: the complex recurrence as a wave scan over a linear stream
             if (int e = launch_res_bwd_scan(g_re_in, g_im_in, want ? workspace : nullptr, want ? workspace + M : nullptr,
                                             g_re, g_im, re, im, sin_decay, cos_decay, 0, 0.0f, 1.0f, 0.0f, M,
-                                            neurons_per_batch, num_decays, T, st))
+                                            neurons_per_batch, num_decays, T, nullptr, st))
                 return e;
         } else {
             ResBwd::Params p{{g_re, g_im, re, im}, {g_re_in, g_im_in}, sin_decay, cos_decay,

@@ -177,7 +177,8 @@ bool bwd_scan_usable(int64_t M, int64_t npb, int64_t T);                // scan.
 int launch_res_bwd_scan(float* g_re_in, float* g_im_in, float* partial_sin, float* partial_cos, const float* g_re,
                         const float* g_im, const float* re, const float* im, const float* sin_decay,
                         const float* cos_decay, int surrogate, float spike_thr, float tau, float rho, int64_t M,
-                        int64_t npb, int64_t num_decays, int64_t T, hipStream_t stream);       // scan.hip
+                        int64_t npb, int64_t num_decays, int64_t T, const Shifts* shifts,
+                        hipStream_t stream);       // scan.hip
 
 }  // namespace slayer
 
@@ -260,13 +261,13 @@ extern "C" int slayer_rf_bwd(float* g_re_in, float* g_im_in, float* grad_sin, fl
         // gains nothing from the split, so large tensors take the unstaged form (partial sums dropped when
         // the decay gradients are not wanted).
         bool done = false;
-        if (!delays && bwd_scan_usable(M, neurons_per_batch, T) && aligned16(g_re_in) && aligned16(g_im_in) &&
+        if (bwd_scan_usable(M, neurons_per_batch, T) && aligned16(g_re_in) && aligned16(g_im_in) &&
             aligned16(grad_spikes) && aligned16(re) && aligned16(im)) {
             // large tensors: surrogate + complex recurrence as a wave scan over a linear stream
             if (int e = launch_res_bwd_scan(g_re_in, g_im_in, want ? workspace : nullptr, want ? workspace + M : nullptr,
                                             grad_spikes, nullptr, re, im, sin_decay, cos_decay, graded ? 2 : 1,
                                             spike_threshold, tau_rho, scale_rho, M, neurons_per_batch, num_decays,
-                                            T, st))
+                                            T, delays ? &sh : nullptr, st))
                 return e;
             done = true;
         }

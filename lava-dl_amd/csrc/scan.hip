@@ -180,6 +180,72 @@ __device__ __forceinline__ void store_row_sums(float* partial, const float (*tab
 }
 
 // ---------------------------------------------------------------------------------------------
+// Axonal delays folded into a scan (see Shifts in tile.h): the tensor named as shifted input is read as
+// x[t] = in[t - kin], the outputs are stored as out[t + kout], row by row.  A lane's quad of four steps then sits at
+// a dword-aligned address of its row, or straddles an end of the row.
+struct ScanShiftTables { int kin[kScanMaxRows], kout[kScanMaxRows]; };
+
+__device__ __forceinline__ void scan_shift_tables(ScanShiftTables& tab, const Shifts& sh, const ScanSpan& sp, int T) {
+    for (int rr = sp.tid; rr < sp.rows; rr += kScanQuads) {
+        tab.kin[rr] = in_shift_of(sh, sp.row0 + rr, T);
+        tab.kout[rr] = out_shift_of(sh, sp.row0 + rr, T);
+    }
+}
+
+// element e of the result is element e + d of q, zero outside it
+__device__ __forceinline__ float4 scan_place(float4 q, int d) {
+    const float a[4] = {q.x, q.y, q.z, q.w};
+    float r[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int j = e + d;
+        r[e] = j == 0 ? a[0] : (j == 1 ? a[1] : (j == 2 ? a[2] : (j == 3 ? a[3] : 0.f)));
+    }
+    return make_float4(r[0], r[1], r[2], r[3]);
+}
+
+// The quad of steps 4*pos .. 4*pos+3 of row r read through the shift k: one 16-byte load at the nearest position
+// inside the row (out of range when no sample of the quad exists); `d` is what scan_place() needs afterwards.
+__device__ __forceinline__ float4 scan_load_shifted(__amdgpu_buffer_rsrc_t src, bool in_span, int r, int pos, int k,
+                                                    int T, int& d) {
+    const int s = 4 * pos - k;
+    const int sc = s < 0 ? 0 : (s > T - 4 ? T - 4 : s);
+    const bool some = in_span && s > -4 && s < T;
+    d = some ? s - sc : 0;
+    return buf_load4<false>(src, some ? (r * T + sc) * 4 : kOutOfRange);
+}
+
+// The quad of steps 4*pos .. of row r stored through the shift k (sample t lands at t + k; samples that leave the
+// row are dropped): one 16-byte store when the whole quad lands inside the row, else sample by sample.  Never
+// streaming: a shifted quad ends in a partial line that a neighbouring quad completes.
+__device__ __forceinline__ void scan_store_shifted(__amdgpu_buffer_rsrc_t dst, bool active, int r, int pos, int k,
+                                                   int T, float4 v) {
+    const int u = 4 * pos + k;
+    const bool whole = active && u >= 0 && u <= T - 4;
+    const bool part = active && !whole && u > -4 && u < T;
+    const int base = (r * T + u) * 4;
+    buf_store4<false>(dst, whole ? base : kOutOfRange, v);
+    if (__any(part)) {
+        const float e[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            buf_store1<false>(dst, (part && (unsigned)(u + j) < (unsigned)T) ? base + 4 * j : kOutOfRange, e[j]);
+    }
+}
+
+// Zeros at the positions of a shifted output that no sample reaches: [0, k) for k > 0, [T + k, T) for k < 0.
+__device__ __forceinline__ void scan_fill_unreached(__amdgpu_buffer_rsrc_t dst, const int* kout, const ScanSpan& sp,
+                                                    int T) {
+    for (int rr = 0; rr < sp.rows; ++rr) {
+        const int k = kout[rr];
+        const int mag = k < 0 ? -k : k;
+        const int len = mag > T ? T : mag;
+        for (int j = sp.tid; j < len; j += kScanQuads)
+            buf_store1<false>(dst, (rr * T + (k < 0 ? T - len + j : j)) * 4, 0.0f);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // Leaky integrator backward.  npb (rows per batch element) and per_param (rows of a batch element that share a
 // parameter; npb when there is one parameter) are 32-bit: the launcher refuses anything larger.
 template <bool PARTIAL, bool STREAM>
@@ -253,19 +319,21 @@ __global__ __launch_bounds__(kScanQuads) void li_bwd_scan_kernel(
 // own with the very arithmetic of li_bwd_scan_kernel -- the input gradient is bit-identical to the spike backward
 // kernel followed by two launches of that kernel.  THETA: the spike threshold is a tensor (threshold + refractory
 // of the adaptive neuron), else the scalar spike_thr.
-template <bool GRADED, bool DECAY_GRAD, bool THETA, bool STREAM>
+template <bool GRADED, bool DECAY_GRAD, bool THETA, bool STREAM, bool SHIFT = false>
 __global__ __launch_bounds__(kScanQuads) void cuba_bwd_scan_kernel(
         float* __restrict__ grad_in, float* __restrict__ partial_i, float* __restrict__ partial_v,
         const float* __restrict__ grad_spikes, const float* __restrict__ voltage, const float* __restrict__ theta,
         const float* __restrict__ current, const float* __restrict__ i_decay, const float* __restrict__ v_decay,
         float spike_thr, float tau, float rho, int64_t M, int QR, int rpg,
-        unsigned npb, unsigned per_i, unsigned per_v) {
+        unsigned npb, unsigned per_i, unsigned per_v, Shifts shifts) {
     __shared__ float ai_tab[kScanMaxRows], av_tab[kScanMaxRows];
     __shared__ float sum_i[kScanWaves][kScanMaxRows], sum_v[kScanWaves][kScanMaxRows];
     __shared__ RealStage stage_v, stage_i;
+    __shared__ ScanShiftTables shift_tab;
     ScanSpan sp;
     sp.init(M, QR, rpg);
     const int nq = sp.nq;
+    const int T = 4 * QR;
     const int64_t base = sp.row0 * (int64_t)QR * 4;
     const unsigned span_bytes = (unsigned)nq * 16u;
     const __amdgpu_buffer_rsrc_t src_g = make_rsrc(grad_spikes + base, span_bytes);
@@ -275,19 +343,32 @@ __global__ __launch_bounds__(kScanQuads) void cuba_bwd_scan_kernel(
     const __amdgpu_buffer_rsrc_t dst = make_rsrc(grad_in + base, span_bytes);
     const float lead = (rho / 2.0f) / tau;
 
-    struct Quads { float4 g, v, th, c; };
-    auto fetch = [&](int q) {
+    struct Quads { float4 g, v, th, c; int dg; };
+    // the saved traces (never shifted), then the gradient of the spikes (read through the output delay when SHIFT)
+    auto fetch_saved = [&](Quads& x, int q) {
         const int off = (unsigned)q < (unsigned)nq ? q * 16 : kOutOfRange;
-        Quads x;
-        x.g = buf_load4<STREAM>(src_g, off);
         x.v = buf_load4<STREAM>(src_v, off);
         x.th = THETA ? buf_load4<STREAM>(src_t, off) : make_float4(0.f, 0.f, 0.f, 0.f);
         x.c = DECAY_GRAD ? buf_load4<STREAM>(src_c, off) : make_float4(0.f, 0.f, 0.f, 0.f);
-        return x;
+    };
+    auto fetch_grad = [&](Quads& x, int q, const ScanCursor& at) {
+        if (SHIFT) {
+            x.g = scan_load_shifted(src_g, (unsigned)q < (unsigned)nq, at.r, at.pos, shift_tab.kin[at.r], T, x.dg);
+        } else {
+            x.g = buf_load4<STREAM>(src_g, (unsigned)q < (unsigned)nq ? q * 16 : kOutOfRange);
+            x.dg = 0;
+        }
     };
     // three pass buffers (up to four tensors each): the pass being worked on and the two after it
     const int q0 = sp.first_quad();
-    Quads b0 = fetch(q0), b1 = fetch(q0 - kScanQuads), b2 = fetch(q0 - 2 * kScanQuads);
+    Quads b0, b1, b2;
+    fetch_saved(b0, q0); fetch_saved(b1, q0 - kScanQuads); fetch_saved(b2, q0 - 2 * kScanQuads);
+    ScanCursor cur, ahead;                           // ahead: the quad of this thread in the pass fetched next
+    cur.init(q0, nq, QR);
+    ahead = cur;
+    if (!SHIFT) {
+        fetch_grad(b0, q0, ahead); fetch_grad(b1, q0 - kScanQuads, ahead); fetch_grad(b2, q0 - 2 * kScanQuads, ahead);
+    }
 
     const unsigned first = scan_first_in_batch(sp.row0, npb);
     for (int rr = sp.tid; rr < sp.rows; rr += kScanQuads) {
@@ -295,13 +376,18 @@ __global__ __launch_bounds__(kScanQuads) void cuba_bwd_scan_kernel(
         ai_tab[rr] = 1.0f - rintf(i_decay[in_batch / per_i]) / 4096.0f;
         av_tab[rr] = 1.0f - rintf(v_decay[in_batch / per_v]) / 4096.0f;
     }
+    if (SHIFT) scan_shift_tables(shift_tab, shifts, sp, T);
     if (DECAY_GRAD)
         for (int rr = sp.lane; rr < sp.rows; rr += kWave) { sum_i[sp.wv][rr] = 0.0f; sum_v[sp.wv][rr] = 0.0f; }
     int parity = (sp.npass - 1) & 1;
     if (sp.tid == 0) { stage_v.carry[parity] = 0.0f; stage_i.carry[parity] = 0.0f; }
     __syncthreads();
-    ScanCursor cur;
-    cur.init(q0, nq, QR);
+    if (SHIFT) {                                     // the shifts are known now
+        fetch_grad(b0, ahead.lq, ahead); ahead.next(QR);
+        fetch_grad(b1, ahead.lq, ahead); ahead.next(QR);
+        fetch_grad(b2, ahead.lq, ahead); ahead.next(QR);
+        scan_fill_unreached(dst, shift_tab.kout, sp, T);
+    }
 
     // the surrogate, expression by expression as the spike backward kernel evaluates it
     auto surrogate = [&](float g, float v, float th) {
@@ -311,17 +397,21 @@ __global__ __launch_bounds__(kScanQuads) void cuba_bwd_scan_kernel(
     auto pass = [&](Quads& x) {
         const bool active = cur.lq < nq;
         const bool row_end = cur.pos == QR - 1;
+        if (SHIFT && __any(x.dg != 0)) x.g = scan_place(x.g, x.dg);      // rare: only where a row begins or ends
         const float4 gv = make_float4(surrogate(x.g.x, x.v.x, x.th.x), surrogate(x.g.y, x.v.y, x.th.y),
                                       surrogate(x.g.z, x.v.z, x.th.z), surrogate(x.g.w, x.v.w, x.th.w));
         float ent_v, ent_i;
         const float4 gc = real_stage(stage_v, sp, parity, av_tab[cur.r], gv, active, row_end, ent_v);
         const float4 gx = real_stage(stage_i, sp, parity, ai_tab[cur.r], gc, active, row_end, ent_i);
-        buf_store4<STREAM>(dst, active ? cur.lq * 16 : kOutOfRange, gx);
+        if (SHIFT) scan_store_shifted(dst, active, cur.r, cur.pos, shift_tab.kout[cur.r], T, gx);
+        else buf_store4<STREAM>(dst, active ? cur.lq * 16 : kOutOfRange, gx);
         if (DECAY_GRAD) {
             add_to_row(sum_v[sp.wv], next_step_product(gc, ent_v, x.v), sp, cur, QR, active);
             add_to_row(sum_i[sp.wv], next_step_product(gx, ent_i, x.c), sp, cur, QR, active);
         }
-        x = fetch(cur.lq - 3 * kScanQuads);
+        fetch_saved(x, cur.lq - 3 * kScanQuads);
+        if (SHIFT) { fetch_grad(x, ahead.lq, ahead); ahead.next(QR); }
+        else fetch_grad(x, cur.lq - 3 * kScanQuads, ahead);
         cur.next(QR);
         parity ^= 1;
     };
@@ -392,19 +482,22 @@ __device__ __forceinline__ void complex_spike_surrogate(const SpikeSurrogate& k,
     g_im = g * (((neg_rho_over_tau * sg_i) * d_im) * step_re);
 }
 
-template <bool PARTIAL, bool STREAM, int SURR>
+template <bool PARTIAL, bool STREAM, int SURR, bool SHIFT = false>
 __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
         float* __restrict__ g_re_in, float* __restrict__ g_im_in, float* __restrict__ partial_sin,
         float* __restrict__ partial_cos, const float* __restrict__ g_re, const float* __restrict__ g_im,
         const float* __restrict__ re, const float* __restrict__ im, const float* __restrict__ sin_decay,
         const float* __restrict__ cos_decay, SpikeSurrogate surr, int64_t M, int QR, int rpg, unsigned npb,
-        unsigned per_param) {
+        unsigned per_param, Shifts shifts) {
+    static_assert(!SHIFT || SURR != 0, "delays are folded into the fused resonate-and-fire form only");
     __shared__ float c_tab[kScanMaxRows], s_tab[kScanMaxRows];
     __shared__ float sum_s[kScanWaves][kScanMaxRows], sum_c[kScanWaves][kScanMaxRows];
     __shared__ ComplexStage L;
+    __shared__ ScanShiftTables shift_tab;
     ScanSpan sp;
     sp.init(M, QR, rpg);
     const int nq = sp.nq;
+    const int T = 4 * QR;
     const int64_t base = sp.row0 * (int64_t)QR * 4;
     const unsigned span_bytes = (unsigned)nq * 16u;
     constexpr bool kStates = PARTIAL || SURR != 0;          // the saved states are read
@@ -414,18 +507,31 @@ __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
     const __amdgpu_buffer_rsrc_t src_im = make_rsrc(kStates ? im + base : nullptr, kStates ? span_bytes : 0u);
     const __amdgpu_buffer_rsrc_t dst_r = make_rsrc(g_re_in + base, span_bytes), dst_i = make_rsrc(g_im_in + base, span_bytes);
 
-    struct Quads { float4 gr, gi, re, im; };
-    auto fetch = [&](int q) {
+    struct Quads { float4 gr, gi, re, im; int dg; };
+    // the tensors that are never shifted, then the incoming gradient (read through the output delay when SHIFT)
+    auto fetch_saved = [&](Quads& x, int q) {
         const int off = (unsigned)q < (unsigned)nq ? q * 16 : kOutOfRange;
-        Quads x;
-        x.gr = buf_load4<STREAM>(src_gr, off);
         x.gi = SURR == 0 ? buf_load4<STREAM>(src_gi, off) : make_float4(0.f, 0.f, 0.f, 0.f);
         x.re = kStates ? buf_load4<STREAM>(src_re, off) : make_float4(0.f, 0.f, 0.f, 0.f);
         x.im = kStates ? buf_load4<STREAM>(src_im, off) : make_float4(0.f, 0.f, 0.f, 0.f);
-        return x;
+    };
+    auto fetch_grad = [&](Quads& x, int q, const ScanCursor& at) {
+        if (SHIFT) {
+            x.gr = scan_load_shifted(src_gr, (unsigned)q < (unsigned)nq, at.r, at.pos, shift_tab.kin[at.r], T, x.dg);
+        } else {
+            x.gr = buf_load4<STREAM>(src_gr, (unsigned)q < (unsigned)nq ? q * 16 : kOutOfRange);
+            x.dg = 0;
+        }
     };
     const int q0 = sp.first_quad();
-    Quads b0 = fetch(q0), b1 = fetch(q0 - kScanQuads), b2 = fetch(q0 - 2 * kScanQuads);
+    Quads b0, b1, b2;
+    fetch_saved(b0, q0); fetch_saved(b1, q0 - kScanQuads); fetch_saved(b2, q0 - 2 * kScanQuads);
+    ScanCursor cur, ahead;                           // ahead: the quad of this thread in the pass fetched next
+    cur.init(q0, nq, QR);
+    ahead = cur;
+    if (!SHIFT) {
+        fetch_grad(b0, q0, ahead); fetch_grad(b1, q0 - kScanQuads, ahead); fetch_grad(b2, q0 - 2 * kScanQuads, ahead);
+    }
 
     const unsigned first = scan_first_in_batch(sp.row0, npb);
     for (int rr = sp.tid; rr < sp.rows; rr += kScanQuads) {
@@ -433,18 +539,25 @@ __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
         c_tab[rr] = cos_decay[j] / 4096.0f;
         s_tab[rr] = sin_decay[j] / 4096.0f;
     }
+    if (SHIFT) scan_shift_tables(shift_tab, shifts, sp, T);
     if (PARTIAL)
         for (int rr = sp.lane; rr < sp.rows; rr += kWave) { sum_s[sp.wv][rr] = 0.0f; sum_c[sp.wv][rr] = 0.0f; }
     int parity = (sp.npass - 1) & 1;
     if (sp.tid == 0) { L.cr[parity] = 0.0f; L.ci[parity] = 0.0f; }
     __syncthreads();
-    ScanCursor cur;
-    cur.init(q0, nq, QR);
+    if (SHIFT) {                                     // the shifts are known now
+        fetch_grad(b0, ahead.lq, ahead); ahead.next(QR);
+        fetch_grad(b1, ahead.lq, ahead); ahead.next(QR);
+        fetch_grad(b2, ahead.lq, ahead); ahead.next(QR);
+        scan_fill_unreached(dst_r, shift_tab.kout, sp, T);
+        scan_fill_unreached(dst_i, shift_tab.kout, sp, T);
+    }
 
     auto pass = [&](Quads& x) {
         const bool active = cur.lq < nq;
         const bool row_end = cur.pos == QR - 1;
         const Cx mu{c_tab[cur.r], -s_tab[cur.r]};
+        if (SHIFT && __any(x.dg != 0)) x.gr = scan_place(x.gr, x.dg);    // rare: only where a row begins or ends
         if (SURR != 0) {                   // quads outside the span hold zeros: their gradient is zero too
             const float4 g = x.gr;
             complex_spike_surrogate<SURR>(surr, g.x, x.re.x, x.im.x, x.gr.x, x.gi.x);
@@ -473,9 +586,15 @@ __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
         Cx ent{lane_below(leaving.re, carry.re), lane_below(leaving.im, carry.im)};
         if (row_end || !active) ent = Cx{0.0f, 0.0f};
         const Cx z3 = cfma(mu, ent, h3), z2 = cfma(mu2, ent, h2), z1 = cfma(mu3, ent, h1), z0 = cfma(mu4, ent, h0);
-        const int off = active ? cur.lq * 16 : kOutOfRange;
-        buf_store4<STREAM>(dst_r, off, make_float4(z0.re, z1.re, z2.re, z3.re));
-        buf_store4<STREAM>(dst_i, off, make_float4(z0.im, z1.im, z2.im, z3.im));
+        if (SHIFT) {
+            const int k = shift_tab.kout[cur.r];
+            scan_store_shifted(dst_r, active, cur.r, cur.pos, k, T, make_float4(z0.re, z1.re, z2.re, z3.re));
+            scan_store_shifted(dst_i, active, cur.r, cur.pos, k, T, make_float4(z0.im, z1.im, z2.im, z3.im));
+        } else {
+            const int off = active ? cur.lq * 16 : kOutOfRange;
+            buf_store4<STREAM>(dst_r, off, make_float4(z0.re, z1.re, z2.re, z3.re));
+            buf_store4<STREAM>(dst_i, off, make_float4(z0.im, z1.im, z2.im, z3.im));
+        }
         if (sp.tid == kScanQuads - 1) { L.cr[parity ^ 1] = z0.re; L.ci[parity ^ 1] = z0.im; }
         if (PARTIAL) {
             // grad_sin: sum -gr[t+1] im[t] + gi[t+1] re[t];  grad_cos: sum gr[t+1] re[t] + gi[t+1] im[t]
@@ -488,7 +607,9 @@ __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
             add_to_row(sum_s[sp.wv], ss, sp, cur, QR, active);
             add_to_row(sum_c[sp.wv], sc, sp, cur, QR, active);
         }
-        x = fetch(cur.lq - 3 * kScanQuads);
+        fetch_saved(x, cur.lq - 3 * kScanQuads);
+        if (SHIFT) { fetch_grad(x, ahead.lq, ahead); ahead.next(QR); }
+        else fetch_grad(x, cur.lq - 3 * kScanQuads, ahead);
         cur.next(QR);
         parity ^= 1;
     };
@@ -563,23 +684,30 @@ int launch_li_bwd_scan(float* grad_in, float* partial, const float* grad_out, co
 }
 
 // theta == nullptr: CUBA (scalar spike threshold); else ALIF.  partial_i / partial_v both or neither.
+// shifts: the backward pass's Shifts when axonal delays are folded in (the gradient of the spikes is read back
+// through the output delay, the input gradient stored back through the input shift), else nullptr.
 int launch_cuba_bwd_scan(float* grad_in, float* partial_i, float* partial_v, const float* grad_spikes,
                          const float* voltage, const float* theta, const float* current, const float* i_decay,
                          const float* v_decay, float spike_thr, float tau, float rho, bool graded,
-                         int64_t M, int64_t npb, int64_t n_id, int64_t n_vd, int64_t T, hipStream_t stream) {
+                         int64_t M, int64_t npb, int64_t n_id, int64_t n_vd, int64_t T, const Shifts* shifts,
+                         hipStream_t stream) {
     const ScanGrid g = scan_grid(M, T);
     if (!g.ok) return SLAYER_ERANGE;
-#define SLAYER_SCAN(G, D, TH, S)                                                                                 \
-    hipLaunchKernelGGL((cuba_bwd_scan_kernel<G, D, TH, S>), g.grid, dim3(kScanQuads), 0, stream, grad_in, partial_i, \
-                       partial_v, grad_spikes, voltage, theta, current, i_decay, v_decay, spike_thr, tau, rho, M, \
-                       g.QR, g.rpg, (unsigned)npb, rows_per_param(npb, n_id), rows_per_param(npb, n_vd))
-#define SLAYER_SCAN_S(G, D, TH) do { if (g.streaming) SLAYER_SCAN(G, D, TH, true); else SLAYER_SCAN(G, D, TH, false); } while (0)
+    const Shifts sh = shifts ? *shifts : Shifts{nullptr, nullptr, nullptr, nullptr, 0, 0, 1, 1.0f, 1};
+#define SLAYER_SCAN(G, D, TH, S, SH)                                                                             \
+    hipLaunchKernelGGL((cuba_bwd_scan_kernel<G, D, TH, S, SH>), g.grid, dim3(kScanQuads), 0, stream, grad_in,    \
+                       partial_i, partial_v, grad_spikes, voltage, theta, current, i_decay, v_decay, spike_thr,  \
+                       tau, rho, M, g.QR, g.rpg, (unsigned)npb, rows_per_param(npb, n_id),                       \
+                       rows_per_param(npb, n_vd), sh)
+#define SLAYER_SCAN_H(G, D, TH, S) do { if (shifts) SLAYER_SCAN(G, D, TH, S, true); else SLAYER_SCAN(G, D, TH, S, false); } while (0)
+#define SLAYER_SCAN_S(G, D, TH) do { if (g.streaming) SLAYER_SCAN_H(G, D, TH, true); else SLAYER_SCAN_H(G, D, TH, false); } while (0)
 #define SLAYER_SCAN_T(G, D) do { if (theta) SLAYER_SCAN_S(G, D, true); else SLAYER_SCAN_S(G, D, false); } while (0)
     const bool want = partial_i != nullptr;
     if (graded) { if (want) SLAYER_SCAN_T(true, true); else SLAYER_SCAN_T(true, false); }
     else { if (want) SLAYER_SCAN_T(false, true); else SLAYER_SCAN_T(false, false); }
 #undef SLAYER_SCAN_T
 #undef SLAYER_SCAN_S
+#undef SLAYER_SCAN_H
 #undef SLAYER_SCAN
     return (int)hipGetLastError();
 }
@@ -589,19 +717,21 @@ int launch_cuba_bwd_scan(float* grad_in, float* partial_i, float* partial_v, con
 int launch_res_bwd_scan(float* g_re_in, float* g_im_in, float* partial_sin, float* partial_cos, const float* g_re,
                         const float* g_im, const float* re, const float* im, const float* sin_decay,
                         const float* cos_decay, int surrogate, float spike_thr, float tau, float rho, int64_t M,
-                        int64_t npb, int64_t num_decays, int64_t T, hipStream_t stream) {
+                        int64_t npb, int64_t num_decays, int64_t T, const Shifts* shifts, hipStream_t stream) {
     const ScanGrid g = scan_grid(M, T);
     if (!g.ok) return SLAYER_ERANGE;
+    if (shifts && surrogate == 0) return SLAYER_EINVAL;      // delays belong to the fused resonate-and-fire form
     const SpikeSurrogate k{spike_thr, tau, rho};
-#define SLAYER_SCAN(P, S, U)                                                                                     \
-    hipLaunchKernelGGL((res_bwd_scan_kernel<P, S, U>), g.grid, dim3(kScanQuads), 0, stream, g_re_in, g_im_in,       \
+    const Shifts sh = shifts ? *shifts : Shifts{nullptr, nullptr, nullptr, nullptr, 0, 0, 1, 1.0f, 1};
+#define SLAYER_SCAN(P, S, U, SH)                                                                                 \
+    hipLaunchKernelGGL((res_bwd_scan_kernel<P, S, U, SH>), g.grid, dim3(kScanQuads), 0, stream, g_re_in, g_im_in,  \
                        partial_sin, partial_cos, g_re, g_im, re, im, sin_decay, cos_decay, k, M, g.QR, g.rpg,    \
-                       (unsigned)npb, rows_per_param(npb, num_decays))
-#define SLAYER_SCAN_S(P, U) do { if (g.streaming) SLAYER_SCAN(P, true, U); else SLAYER_SCAN(P, false, U); } while (0)
-#define SLAYER_SCAN_P(U) do { if (partial_sin) SLAYER_SCAN_S(true, U); else SLAYER_SCAN_S(false, U); } while (0)
-    if (surrogate == 0) SLAYER_SCAN_P(0);
-    else if (surrogate == 1) SLAYER_SCAN_P(1);
-    else SLAYER_SCAN_P(2);
+                       (unsigned)npb, rows_per_param(npb, num_decays), sh)
+#define SLAYER_SCAN_S(P, U, SH) do { if (g.streaming) SLAYER_SCAN(P, true, U, SH); else SLAYER_SCAN(P, false, U, SH); } while (0)
+#define SLAYER_SCAN_P(U, SH) do { if (partial_sin) SLAYER_SCAN_S(true, U, SH); else SLAYER_SCAN_S(false, U, SH); } while (0)
+    if (surrogate == 0) SLAYER_SCAN_P(0, false);
+    else if (surrogate == 1) { if (shifts) SLAYER_SCAN_P(1, true); else SLAYER_SCAN_P(1, false); }
+    else { if (shifts) SLAYER_SCAN_P(2, true); else SLAYER_SCAN_P(2, false); }
 #undef SLAYER_SCAN_P
 #undef SLAYER_SCAN_S
 #undef SLAYER_SCAN
