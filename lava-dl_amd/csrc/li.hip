@@ -6,7 +6,9 @@
 namespace slayer {
 
 // ---------------------------------------------------------------------------------- forward
-template <bool POW2>
+// RESET = false: no threshold was given, the reset decision is left out of the step (a third of its
+// instructions: what a step costs is what bounds the kernel while few neurons keep the chip busy).
+template <bool POW2, bool RESET = true>
 struct LiFwd {
     static constexpr int kIn = 1, kOut = 1;
     static constexpr bool kReverse = false;
@@ -43,7 +45,7 @@ struct LiFwd {
     __device__ __forceinline__ void step(const float (&x)[1], float (&o)[1]) {
         const int yn = rs0_12(y, mult) + __float_as_int(x[0]);
         o[0] = __int_as_float(yn);
-        y = (yn > fire_above) ? 0 : yn;              // (float)yn >= threshold, decided on the integer
+        y = (RESET && yn > fire_above) ? 0 : yn;     // (float)yn >= threshold, decided on the integer
     }
     __device__ __forceinline__ void finish(const Params&, int64_t, bool) {}
 };
@@ -199,12 +201,16 @@ extern "C" int slayer_li_fwd(float* out, const float* in, const float* decay, co
     if (w_scale == 0) return SLAYER_EINVAL;
     const float w = (float)w_scale;
     const int fa = fire_above(thr_scaled > 0 ? (float)thr_scaled : __builtin_inff());
-    if (is_pow2(w_scale)) {
-        LiFwd<true>::Params p{{in}, {out}, decay, state, w, 1.0f / w, fa, neurons_per_batch, num_decays, num_states};
-        return launch_stream<LiFwd<true>>(p, M, T, (hipStream_t)stream);
-    }
-    LiFwd<false>::Params p{{in}, {out}, decay, state, w, 1.0f / w, fa, neurons_per_batch, num_decays, num_states};
-    return launch_stream<LiFwd<false>>(p, M, T, (hipStream_t)stream);
+#define SLAYER_LI_FWD(P, R)                                                                                       \
+    do {                                                                                                          \
+        LiFwd<P, R>::Params p{{in}, {out}, decay, state, w, 1.0f / w, fa, neurons_per_batch, num_decays, num_states}; \
+        return launch_stream<LiFwd<P, R>>(p, M, T, (hipStream_t)stream);                                          \
+    } while (0)
+    const bool reset = thr_scaled > 0;
+    if (is_pow2(w_scale)) { if (reset) SLAYER_LI_FWD(true, true); else SLAYER_LI_FWD(true, false); }
+    if (reset) SLAYER_LI_FWD(false, true);
+    SLAYER_LI_FWD(false, false);
+#undef SLAYER_LI_FWD
 }
 
 extern "C" int slayer_li_bwd(float* grad_in, float* grad_decay, const float* grad_out, const float* out,
