@@ -36,7 +36,7 @@ struct AlifFwd {
     static constexpr bool kReverse = false;
     static constexpr bool kTransforms = true;
     static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
-    static constexpr bool kMultiwaveWhenLarge = !SHIFT;
+    static constexpr bool kMultiwaveWhenLarge = true;
     struct Params {
         const float* in[1];
         float* out[kOut];

@@ -31,7 +31,7 @@ struct CubaFwd {
     static constexpr bool kReverse = false;
     static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
     static constexpr bool kLongPiecesOnAliasedRows = true;
-    static constexpr bool kMultiwaveWhenLarge = !SHIFT;
+    static constexpr bool kMultiwaveWhenLarge = true;
     struct Params {
         const float* in[1];
         float* out[kOut + 1];
@@ -43,7 +43,7 @@ struct CubaFwd {
         Shifts shifts;
     };
     static constexpr bool kTransforms = true;        // integer tiles, see to_state / from_state
-    static constexpr int kCopyWaves = SHIFT ? 4 : 2;     // the shifted copies cost the copy waves more instructions
+    static constexpr int kCopyWaves = SHIFT ? 8 : 2;     // the shifted copies cost the copy waves more instructions
     int yc, yv, yv_out, mi, mv, fire_above;
     float w, inv_w, spike_thr, spike_scale;
 
@@ -75,14 +75,16 @@ struct CubaFwd {
         o[kVol] = __int_as_float(yn);
     }
     // The same step as two Ops for the staged multi-wave kernel: the current recurrence, and the voltage
-    // recurrence reading the current out of its tile one chunk later.
+    // recurrence one chunk later.  What the voltage op reads of the current (the float32 round trip) is worked
+    // out by the first wave and left in the voltage tile, where the second wave replaces it with the voltage:
+    // that evens out the two steps (8 and 9 instructions instead of 6 and 11).
     static constexpr int kStages = 2;
-    static constexpr bool kStagedWhenLarge = !SHIFT;
+    static constexpr bool kStagedWhenLarge = true;
     struct Stage0 {
-        static constexpr int kIn = 1, kOut = 1;
+        static constexpr int kIn = 1, kOut = KEEP_CURRENT ? 2 : 1;
         static constexpr bool kReverse = false, kTileMapped = true;
         static constexpr int in_tile(int) { return 0; }
-        static constexpr int out_tile(int) { return 0; }         // the current replaces the input in place
+        static constexpr int out_tile(int o) { return o; }       // [current,] what the voltage op reads of it
         int yc, mi;
         float w, inv_w;
         __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
@@ -92,9 +94,11 @@ struct CubaFwd {
                 mi = 4096 - trunc_i32(rintf(p.i_decay[param_index(m, p.npb, p.n_id)]));
             }
         }
-        __device__ __forceinline__ void step(const float (&x)[1], float (&o)[1]) {
+        __device__ __forceinline__ void step(const float (&x)[1], float (&o)[kOut]) {
             yc = rs0_12(yc, mi) + __float_as_int(x[0]);
-            o[0] = __int_as_float(yc);
+            const float cf = (float)yc;
+            if (KEEP_CURRENT) o[0] = __int_as_float(yc);
+            o[kVol] = __int_as_float(POW2 ? trunc_i32(cf) : trunc_i32(w * (cf / w)));
         }
         __device__ __forceinline__ void finish(const Params& p, int64_t m, bool valid) {
             if (valid && p.cur_last) p.cur_last[m] = from_state<POW2>(__int_as_float(yc), w, inv_w);
@@ -103,8 +107,8 @@ struct CubaFwd {
     struct Stage1 {
         static constexpr int kIn = 1, kOut = 1;
         static constexpr bool kReverse = false, kTileMapped = true;
-        static constexpr int in_tile(int) { return 0; }
-        static constexpr int out_tile(int) { return kVol; }      // without a current trace: in place
+        static constexpr int in_tile(int) { return kVol; }
+        static constexpr int out_tile(int) { return kVol; }      // in place
         int yv, yv_out, mv, fire_above;
         float w, inv_w, spike_thr, spike_scale;
         __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
@@ -116,8 +120,7 @@ struct CubaFwd {
             }
         }
         __device__ __forceinline__ void step(const float (&x)[1], float (&o)[1]) {
-            const float cf = (float)__float_as_int(x[0]);
-            const int yn = rs0_12(yv, mv) + (POW2 ? trunc_i32(cf) : trunc_i32(w * (cf / w)));
+            const int yn = rs0_12(yv, mv) + __float_as_int(x[0]);
             yv = (yn > fire_above) ? 0 : yn;
             yv_out = yn;
             o[0] = __int_as_float(yn);

@@ -25,7 +25,7 @@ struct RfFwd {
     static constexpr bool kTransforms = true;
     static constexpr int kCopyWaves = SHIFT ? 4 : 2;     // the shifted copies cost the copy waves more instructions
     static constexpr int64_t kRows32Below = 32768, kRows16Below = 32768;
-    static constexpr bool kMultiwaveWhenLarge = !SHIFT;
+    static constexpr bool kMultiwaveWhenLarge = true;
     struct Params {
         const float* in[2];
         float* out[3];

@@ -277,6 +277,24 @@ def test_rf_fused_with_delays(slayer, geom, form):
     assert_exact(res_f[3], r_spk_u[..., -1], 'last spike vs oracle')
 
 
+# More workgroups than the chip holds at once (131 072 rows): the multi-wave kernels then run in several rounds, held
+# to a few workgroups per compute unit, with the delays folded in.
+GEOM_ROUNDS = ((32, 4096, 128), 'table', 'table', 1, True)
+
+
+@pytest.mark.parametrize('form', ['full', 'lean'])
+def test_cuba_fused_with_delays_in_several_rounds(slayer, form):
+    test_cuba_fused_with_delays(slayer, GEOM_ROUNDS, form, False)
+
+
+def test_alif_fused_with_delays_in_several_rounds(slayer):
+    test_alif_fused_with_delays(slayer, GEOM_ROUNDS, 'full')
+
+
+def test_rf_fused_with_delays_in_several_rounds(slayer):
+    test_rf_fused_with_delays(slayer, GEOM_ROUNDS, 'train')
+
+
 class _Block:
     """What block.neuron_delay needs of a block: neuron, delay_shift, delay (and its own delay_buffer)."""
 
