@@ -203,11 +203,12 @@ struct AlifBwd {
         int64_t npb, n_id, n_vd;
         Shifts shifts;
     };
-    float ai, av, gc, gx, acc_i, acc_v, tau, rho, lead;
+    float ai, av, gc, gx, acc_i, acc_v, tau, rho, lead, inv_tau;
 
     __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
         tau = p.tau; rho = p.rho;
         lead = (rho / 2.0f) / tau;
+        inv_tau = 1.0f / tau;
         ai = av = gc = gx = acc_i = acc_v = 0.f;
         if (valid) {
             ai = 1.0f - rintf(p.i_decay[param_index(m, p.npb, p.n_id)]) / 4096.0f;
@@ -220,7 +221,7 @@ struct AlifBwd {
     static constexpr int kCopyWaves = SHIFT ? 8 : 4;
     __device__ __forceinline__ float surrogate(float g, float v, float theta) const {
         const float d = v - theta;
-        return GRADED ? (rho * expf(fminf(d, 0.0f) / tau)) * g : (lead * expf(-fabsf(d) / tau)) * g;
+        return GRADED ? (rho * expf(fminf(d, 0.0f) * inv_tau)) * g : (lead * expf(-fabsf(d) * inv_tau)) * g;
     }
     __device__ __forceinline__ void pre(float4 (&x)[kIn]) const {
         x[0] = make_float4(surrogate(x[0].x, x[1].x, x[2].x), surrogate(x[0].y, x[1].y, x[2].y),

@@ -196,6 +196,7 @@ __global__ __launch_bounds__(kMaxRecurrent) void recurrent_bwd_kernel(
     const float* trow = THETA ? theta + m * (int64_t)T : nullptr;
     float* orow = grad_z + m * (int64_t)T;
     const float lead = (rho / 2.0f) / tau;
+    const float inv_tau = 1.0f / tau;
     float carry = 0.f;
     float4 gq = make_float4(0.f, 0.f, 0.f, 0.f), vq = gq, oq = gq, tq = gq;
 
@@ -217,7 +218,7 @@ __global__ __launch_bounds__(kMaxRecurrent) void recurrent_bwd_kernel(
         }
         const float gs = carry + g;
         const float d = v - th;
-        const float factor = GRADED ? rho * expf(fminf(d, 0.0f) / tau) : lead * expf(-fabsf(d) / tau);
+        const float factor = GRADED ? rho * expf(fminf(d, 0.0f) * inv_tau) : lead * expf(-fabsf(d) * inv_tau);
         const float gd = live ? factor * gs : 0.f;
         if (VEC4) {
             if ((t & 3) == 3) oq.w = gd;

@@ -112,11 +112,12 @@ struct RfBwd {
         int64_t npb, nd;
         Shifts shifts;
     };
-    float c, s, gr, gi, acc_s, acc_c, thr, tau, rho, half_over_tau, two_tau, neg_rho_over_tau;
+    float c, s, gr, gi, acc_s, acc_c, thr, tau, rho, half_over_tau, two_tau, neg_rho_over_tau, inv_tau;
 
     __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
         thr = p.spike_thr; tau = p.tau; rho = p.rho;
         half_over_tau = (1.0f / 2.0f) / tau;
+        inv_tau = 1.0f / tau;
         two_tau = 2.0f * tau;
         neg_rho_over_tau = (-rho) / tau;
         c = s = gr = gi = acc_s = acc_c = 0.f;
@@ -129,9 +130,9 @@ struct RfBwd {
     // complex spike surrogate (same expression order as the stand-alone kernel)
     __device__ __forceinline__ void surrogate(float g, float r, float i, float& g_re, float& g_im) const {
         float d_re;
-        if (GRADED) d_re = expf(-fmaxf(thr - r, 0.0f) / tau);
-        else d_re = half_over_tau * expf(-fabsf(r - thr) / tau);
-        const float d_im = half_over_tau * expf(-fabsf(i) / tau);
+        if (GRADED) d_re = expf(-fmaxf(thr - r, 0.0f) * inv_tau);
+        else d_re = half_over_tau * expf(-fabsf(r - thr) * inv_tau);
+        const float d_im = half_over_tau * expf(-fabsf(i) * inv_tau);
         const float dr = r - thr;
         const float sg_r = dr > 0.0f ? 1.0f : (dr < 0.0f ? -1.0f : (dr == 0.0f ? 0.0f : dr));
         const float sg_i = i > 0.0f ? 1.0f : (i < 0.0f ? -1.0f : (i == 0.0f ? 0.0f : i));

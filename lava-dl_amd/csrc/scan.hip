@@ -342,6 +342,7 @@ __global__ __launch_bounds__(kScanQuads) void cuba_bwd_scan_kernel(
     const __amdgpu_buffer_rsrc_t src_c = make_rsrc(DECAY_GRAD ? current + base : nullptr, DECAY_GRAD ? span_bytes : 0u);
     const __amdgpu_buffer_rsrc_t dst = make_rsrc(grad_in + base, span_bytes);
     const float lead = (rho / 2.0f) / tau;
+    const float inv_tau = 1.0f / tau;
 
     struct Quads { float4 g, v, th, c; int dg; };
     // the saved traces (never shifted), then the gradient of the spikes (read through the output delay when SHIFT)
@@ -394,7 +395,7 @@ __global__ __launch_bounds__(kScanQuads) void cuba_bwd_scan_kernel(
     // the surrogate, expression by expression as the spike backward kernel evaluates it
     auto surrogate = [&](float g, float v, float th) {
         const float d = v - (THETA ? th : spike_thr);
-        return GRADED ? (rho * expf(fminf(d, 0.0f) / tau)) * g : (lead * expf(-fabsf(d) / tau)) * g;
+        return GRADED ? (rho * expf(fminf(d, 0.0f) * inv_tau)) * g : (lead * expf(-fabsf(d) * inv_tau)) * g;
     };
     auto pass = [&](Quads& x) {
         const bool active = cur.lq < nq;
@@ -472,12 +473,13 @@ template <int SURR>
 __device__ __forceinline__ void complex_spike_surrogate(const SpikeSurrogate& k, float g, float r, float i,
                                                         float& g_re, float& g_im) {
     const float half_over_tau = (1.0f / 2.0f) / k.tau;
+    const float inv_tau = 1.0f / k.tau;
     const float two_tau = 2.0f * k.tau;
     const float neg_rho_over_tau = (-k.rho) / k.tau;
     float d_re;
-    if (SURR == 2) d_re = expf(-fmaxf(k.thr - r, 0.0f) / k.tau);
-    else d_re = half_over_tau * expf(-fabsf(r - k.thr) / k.tau);
-    const float d_im = half_over_tau * expf(-fabsf(i) / k.tau);
+    if (SURR == 2) d_re = expf(-fmaxf(k.thr - r, 0.0f) * inv_tau);
+    else d_re = half_over_tau * expf(-fabsf(r - k.thr) * inv_tau);
+    const float d_im = half_over_tau * expf(-fabsf(i) * inv_tau);
     const float dr = r - k.thr;
     const float sg_r = dr > 0.0f ? 1.0f : (dr < 0.0f ? -1.0f : (dr == 0.0f ? 0.0f : dr));
     const float sg_i = i > 0.0f ? 1.0f : (i < 0.0f ? -1.0f : (i == 0.0f ? 0.0f : i));

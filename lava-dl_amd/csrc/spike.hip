@@ -51,10 +51,16 @@ __global__ __launch_bounds__(kEltBlock) void spike_bwd_kernel(float* __restrict_
                                                               float th0, float tau, float rho, int64_t n, int64_t nq) {
     if (!TENSOR_TH && th) th0 = th[0];
     const float lead = (rho / 2.0f) / tau;       // scale_rho / 2 / tau_rho, left to right
+    // The exponent is (v - threshold) * (1 / tau) where the reference divides by tau: at most an ulp and a half
+    // apart in the exponent (identical for tau = 1), far inside the 1e-5 bar of the float gradients, and it takes
+    // the ten instructions of a correctly rounded division out of every sample -- which is what held the fused
+    // backward scans below their memory rate.  Every kernel that evaluates a surrogate does the same, so fused
+    // and unfused paths stay bit-identical to each other.
+    const float inv_tau = 1.0f / tau;
     auto f = [&](float x, float t, float g) -> float {
         const float d = x - t;
-        if (GRADED) return (rho * expf(fminf(d, 0.0f) / tau)) * g;
-        return (lead * expf(-fabsf(d) / tau)) * g;
+        if (GRADED) return (rho * expf(fminf(d, 0.0f) * inv_tau)) * g;
+        return (lead * expf(-fabsf(d) * inv_tau)) * g;
     };
     const int64_t k = (int64_t)blockIdx.x * kEltBlock + threadIdx.x;
     if (k < nq) {
@@ -113,14 +119,15 @@ __global__ __launch_bounds__(kEltBlock) void cspike_bwd_kernel(float* __restrict
                                                                float rho, int64_t n, int64_t nq) {
     if (!TENSOR_TH && th) th0 = th[0];
     const float half_over_tau = (1.0f / 2.0f) / tau;   // 1 / 2 / tau_rho
+    const float inv_tau = 1.0f / tau;
     const float two_tau = 2.0f * tau;
     const float neg_rho_over_tau = (-rho) / tau;
     auto sign = [](float x) -> float { return x > 0.0f ? 1.0f : (x < 0.0f ? -1.0f : (x == 0.0f ? 0.0f : x)); };
     auto f = [&](float r, float i, float t, float g, float& o_re, float& o_im) {
         float d_re;
-        if (GRADED) d_re = expf(-fmaxf(t - r, 0.0f) / tau);
-        else d_re = half_over_tau * expf(-fabsf(r - t) / tau);
-        const float d_im = half_over_tau * expf(-fabsf(i) / tau);
+        if (GRADED) d_re = expf(-fmaxf(t - r, 0.0f) * inv_tau);
+        else d_re = half_over_tau * expf(-fabsf(r - t) * inv_tau);
+        const float d_im = half_over_tau * expf(-fabsf(i) * inv_tau);
         const float step_re = 0.5f * (1.0f + sign(r - t) * (1.0f - two_tau * d_re));
         o_re = g * ((rho * d_re) * d_im);
         o_im = g * (((neg_rho_over_tau * sign(i)) * d_im) * step_re);
