@@ -8,12 +8,9 @@ namespace slayer {
 // consecutive quads of a row, so loads and stores are contiguous along time.
 // VEC4: T % 4 == 0 and 16-byte aligned bases -> dwordx4 stores, and one dwordx4 load per quad whose
 // source lies wholly inside the row, at a dword-aligned address when the row's shift is not a multiple of 4
-// (the quads that straddle an end of the row load sample by sample).
-typedef float quad_align4 __attribute__((ext_vector_type(4), aligned(4)));
-__device__ __forceinline__ float4 load_quad_dword_aligned(const float* p) {
-    const quad_align4 v = *reinterpret_cast<const quad_align4*>(p);
-    return make_float4(v.x, v.y, v.z, v.w);
-}
+// (the quads that straddle an end of the row load sample by sample).  Without VEC4 the stores are 16 bytes at
+// dword-aligned addresses too, except for a row's last, partial quad.
+
 template <bool VEC4>
 __global__ __launch_bounds__(256) void shift_kernel(float* __restrict__ out, const float* __restrict__ in,
                                                     const float* __restrict__ lut, int scalar_steps, float ts,
@@ -33,7 +30,7 @@ __global__ __launch_bounds__(256) void shift_kernel(float* __restrict__ out, con
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
     if (VEC4 && (k & 3) == 0) {
         if (s >= 0 && s < T) v = *reinterpret_cast<const float4*>(row + s);
-    } else if (VEC4 && s >= 0 && s + 3 < T) {
+    } else if (s >= 0 && s + 3 < T) {
         v = load_quad_dword_aligned(row + s);
     } else {
         if (s + 0 >= 0 && s + 0 < T) v.x = row[s + 0];
@@ -43,6 +40,8 @@ __global__ __launch_bounds__(256) void shift_kernel(float* __restrict__ out, con
     }
     if (VEC4) {
         *reinterpret_cast<float4*>(dst) = v;
+    } else if (t + 3 < T) {
+        store_quad_dword_aligned(dst, v);
     } else {
         if (t + 0 < T) dst[0] = v.x;
         if (t + 1 < T) dst[1] = v.y;

@@ -100,6 +100,19 @@ __device__ __forceinline__ void store4(float* p, float4 v, bool streaming) {
     }
 }
 
+// 16-byte accesses at addresses that are only dword-aligned (rows of a length that is not a multiple of 4, or
+// shifted by such a count): the hardware takes them, the type tells the compiler not to assume more.
+typedef float quad_align4 __attribute__((ext_vector_type(4), aligned(4)));
+__device__ __forceinline__ float4 load_quad_dword_aligned(const float* p) {
+    const quad_align4 v = *reinterpret_cast<const quad_align4*>(p);
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void store_quad_dword_aligned(float* p, float4 f) {
+    quad_align4 v;
+    v.x = f.x; v.y = f.y; v.z = f.z; v.w = f.w;
+    *reinterpret_cast<quad_align4*>(p) = v;
+}
+
 // float32 -> int32 toward zero; out-of-range values saturate (v_cvt_i32_f32).
 __device__ __forceinline__ int trunc_i32(float x) { return (int)x; }
 
@@ -890,10 +903,14 @@ __global__ __launch_bounds__(kWave) void stream_kernel_scalar(typename Op::Param
                     const int ki = ((SI >> i) & 1u) != 0 ? kin[p] : 0;   // sample t + e - ki, if the row has it
                     const float* src = prm.in[i] + off - ki;
                     const int s = t - ki;
-                    if (t + 0 < T && (unsigned)(s + 0) < (unsigned)T) v.x = src[0];
-                    if (t + 1 < T && (unsigned)(s + 1) < (unsigned)T) v.y = src[1];
-                    if (t + 2 < T && (unsigned)(s + 2) < (unsigned)T) v.z = src[2];
-                    if (t + 3 < T && (unsigned)(s + 3) < (unsigned)T) v.w = src[3];
+                    if (t + 3 < T && s >= 0 && s + 3 < T) {
+                        v = load_quad_dword_aligned(src);        // the whole quad exists: one 16-byte access
+                    } else {
+                        if (t + 0 < T && (unsigned)(s + 0) < (unsigned)T) v.x = src[0];
+                        if (t + 1 < T && (unsigned)(s + 1) < (unsigned)T) v.y = src[1];
+                        if (t + 2 < T && (unsigned)(s + 2) < (unsigned)T) v.z = src[2];
+                        if (t + 3 < T && (unsigned)(s + 3) < (unsigned)T) v.w = src[3];
+                    }
                 }
                 x[i] = v;
             }
@@ -949,10 +966,14 @@ __global__ __launch_bounds__(kWave) void stream_kernel_scalar(typename Op::Param
                     const int ko = ((SO >> o) & 1u) != 0 ? kout[p] : 0;  // sample t + e goes to t + e + ko
                     float* d = prm.out[o] + off + ko;
                     const int u = t + ko;
-                    if (t + 0 < T && (unsigned)(u + 0) < (unsigned)T) d[0] = v[o].x;
-                    if (t + 1 < T && (unsigned)(u + 1) < (unsigned)T) d[1] = v[o].y;
-                    if (t + 2 < T && (unsigned)(u + 2) < (unsigned)T) d[2] = v[o].z;
-                    if (t + 3 < T && (unsigned)(u + 3) < (unsigned)T) d[3] = v[o].w;
+                    if (t + 3 < T && u >= 0 && u + 3 < T) {
+                        store_quad_dword_aligned(d, v[o]);       // the whole quad lands inside the row
+                    } else {
+                        if (t + 0 < T && (unsigned)(u + 0) < (unsigned)T) d[0] = v[o].x;
+                        if (t + 1 < T && (unsigned)(u + 1) < (unsigned)T) d[1] = v[o].y;
+                        if (t + 2 < T && (unsigned)(u + 2) < (unsigned)T) d[2] = v[o].z;
+                        if (t + 3 < T && (unsigned)(u + 3) < (unsigned)T) d[3] = v[o].w;
+                    }
                 }
             }
         }
