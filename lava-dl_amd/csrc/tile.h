@@ -191,6 +191,14 @@ struct Shifts {
     int64_t npb;
 };
 
+// prm.shifts, or no shifts at all for an Op whose Params carry none
+template <class P, class = void>
+struct ShiftsOf { static __host__ __device__ __forceinline__ Shifts get(const P&) { return Shifts{nullptr, nullptr, nullptr, nullptr, 0, 0, 1, 1.0f, 1}; } };
+template <class P>
+struct ShiftsOf<P, decltype((void)sizeof(((P*)nullptr)->shifts))> {
+    static __host__ __device__ __forceinline__ const Shifts& get(const P& p) { return p.shifts; }
+};
+
 template <class Op, class = void>
 struct ShiftInMask { static constexpr unsigned value = 0; };
 template <class Op>
@@ -289,14 +297,22 @@ __device__ __forceinline__ void buf_store1(__amdgpu_buffer_rsrc_t r, int byte_of
 //
 // A wave can share the job with others: it then owns PASSES of the G::kPasses wave-wide accesses
 // that cover a tile, starting at pass first_pass.
-template <class Op, int R, bool STREAM, int PASSES = TileGeom<R>::kPasses, int S = kTileSamples>
+//
+// UNAL: rows that are not whole quads (T % 4 != 0, or base pointers that are only dword-aligned).  Tile columns
+// are still laid on 128-byte lines by the row phases, so quads sit on 16-byte boundaries of memory, but a row
+// may now begin and end inside a quad.  Every tensor then takes the path of the shifted ones (with a shift of
+// zero unless it really is shifted): 16-byte accesses where the whole quad lies inside the row, the quads that
+// straddle an end of the row loaded from the nearest position inside it and stored sample by sample, no line
+// completion; the recurrence skips the steps of such a quad that lie outside the row.
+template <class Op, int R, bool STREAM, int PASSES = TileGeom<R>::kPasses, int S = kTileSamples, bool UNAL = false>
 struct Copier {
     using G = TileGeom<R, S>;
     static constexpr int TC = G::kChunk, NI = Op::kIn, NO = Op::kOut, ND = DerivedCount<Op>::value;
     static constexpr int kPasses = PASSES;
     static_assert(ND == 0 || ND == 1, "at most one derived output");
-    static constexpr unsigned SI = ShiftInMask<Op>::value, SO = ShiftOutMask<Op>::value;
-    static constexpr bool kShifts = SI != 0 || SO != 0;
+    static constexpr unsigned SI = ShiftInMask<Op>::value, SO = ShiftOutMask<Op>::value;     // really shifted
+    static constexpr unsigned AI = UNAL ? (1u << NI) - 1u : SI, AO = UNAL ? (1u << (NO + ND)) - 1u : SO;   // careful path
+    static constexpr bool kShifts = AI != 0 || AO != 0;
     using Tiles = float (*)[G::kTileFloats];
 
     __amdgpu_buffer_rsrc_t src[NI], dst[NO + ND];
@@ -330,7 +346,7 @@ struct Copier {
         // chunks [1, interior_end) hold only valid columns and touch no shared line, for every phase
         interior_end = (T & ~31) / TC;
         // rows shorter than a line could start and end inside the same line; they keep direct stores
-        route = T >= 32;
+        route = T >= 32 && !UNAL;
 #pragma unroll
         for (int p = 0; p < kPasses; ++p) {
             const int r = (first_pass + p) * G::kRowsPerPass + crow;
@@ -342,7 +358,7 @@ struct Copier {
         if constexpr (kShifts) {
             // lane l works out the shifts of row l once (a table look-up with a 64-bit modulo and a division);
             // the passes pick theirs up from that lane
-            const auto& sh = prm.shifts;
+            const Shifts sh = ShiftsOf<typename Op::Params>::get(prm);
             const bool mine = lane >= row_lo && lane < row_hi;
             const int kin_row = (SI != 0 && mine) ? in_shift_of(sh, m0 + lane, T) : 0;
             kout_row = (SO != 0 && mine) ? out_shift_of(sh, m0 + lane, T) : 0;
@@ -380,7 +396,7 @@ struct Copier {
     // advance.  Row after row of this wave's rows, 64 positions per instruction.
     __device__ __forceinline__ void fill_unreached(const typename Op::Params& prm, int64_t m0, int lane) const {
         if constexpr (SO != 0) {
-            const auto& sh = prm.shifts;
+            const Shifts sh = ShiftsOf<typename Op::Params>::get(prm);
             for (int r = row_lo; r < row_hi; ++r) {
                 const int k = __builtin_amdgcn_readlane(kout_row, r);
                 const int mag = k < 0 ? -k : k;
@@ -406,18 +422,19 @@ struct Copier {
 #pragma unroll
         for (int p = 0; p < kPasses; ++p) {
             const int t = step0[p] + chunk * TC;
-            const bool ok = (unsigned)t < (unsigned)T;
+            const bool ok = UNAL ? (t > -4 && t < T) : (unsigned)t < (unsigned)T;   // some step of the quad is in the row
             const int off = ok ? off0[p] + chunk * (TC * 4) : kOutOfRange;
 #pragma unroll
             for (int i = 0; i < NI; ++i) {
-                if (((SI >> i) & 1u) != 0) {
+                if (((AI >> i) & 1u) != 0) {
                     // the quad wanted is samples s .. s+3 of the row, s = t - kin (a multiple of 4 only by chance:
                     // the load is dword-aligned).  One 16-byte load at the nearest position that lies inside
                     // the row; to_tiles() moves the samples into place when the two differ.
+                    const int ki = ((SI >> i) & 1u) != 0 ? kin[p] : 0;
                     if (whole_in(chunk)) {
-                        buf[i][p] = buf_load4<STREAM>(src[i], ok ? off0[p] + chunk * (TC * 4) - 4 * kin[p] : kOutOfRange);
+                        buf[i][p] = buf_load4<STREAM>(src[i], ok ? off0[p] + chunk * (TC * 4) - 4 * ki : kOutOfRange);
                     } else {
-                        const int s = t - kin[p];
+                        const int s = t - ki;
                         const int sc = s < 0 ? 0 : (s > T - 4 ? T - 4 : s);
                         const bool some = ok && s > -4 && s < T;
                         buf[i][p] = buf_load4<STREAM>(src[i], some ? off0[p] + 4 * (sc - step0[p]) : kOutOfRange);
@@ -456,14 +473,19 @@ struct Copier {
             float4 x[NI];
 #pragma unroll
             for (int i = 0; i < NI; ++i) x[i] = buf[i][p];
-            if (SI != 0 && !whole_in(chunk)) {
-                const int s = step0[p] + chunk * TC - kin[p];
-                const int sc = s < 0 ? 0 : (s > T - 4 ? T - 4 : s);
-                const int d = (s > -4 && s < T) ? s - sc : 0;
-                if (__any(d != 0)) {                  // rare: only where a row begins or ends
+            if (AI != 0 && !whole_in(chunk)) {
+                auto offset_of = [&](int ki) {        // wanted minus loaded position of a quad read through shift ki
+                    const int s = step0[p] + chunk * TC - ki;
+                    const int sc = s < 0 ? 0 : (s > T - 4 ? T - 4 : s);
+                    return (s > -4 && s < T) ? s - sc : 0;
+                };
+                const int d = offset_of(SI != 0 ? kin[p] : 0), d0 = (UNAL && SI != AI) ? offset_of(0) : 0;
+                if (__any((d | d0) != 0)) {           // rare: only where a row begins or ends
 #pragma unroll
-                    for (int i = 0; i < NI; ++i)
+                    for (int i = 0; i < NI; ++i) {
                         if (((SI >> i) & 1u) != 0) x[i] = place(x[i], d);
+                        else if (((AI >> i) & 1u) != 0) x[i] = place(x[i], d0);
+                    }
                 }
             }
             if constexpr (HasTransforms<Op>::value) op.pre(x);
@@ -548,42 +570,47 @@ struct Copier {
             // on line boundaries anyway), sample t + e to position t + e + kout of the row: one dword-aligned
             // 16-byte store when the whole quad lands inside the row; a quad that straddles an end of the row
             // (only in the first or last few chunks) leaves sample by sample.
-            const int ubase = off0[p] + chunk * (TC * 4) + (SO != 0 ? 4 * kout[p] : 0);
-            bool whole = true, part = false, any_part = false;
-            const int u = t + (SO != 0 ? kout[p] : 0);
-            if (SO != 0 && !(inner && whole_out(chunk))) {
+            const bool careful = AO != 0 && !(inner && whole_out(chunk));   // a quad of this chunk may straddle an end of its row
+            if (careful) {
                 if (inner) {
 #pragma unroll
                     for (int o = 0; o < NO; ++o) own[o] = v[o];
                 } else {
                     if constexpr (HasTransforms<Op>::value) op.post(own);
                 }
-                const bool t_ok = (unsigned)t < (unsigned)T;
-                whole = t_ok && u >= 0 && u <= T - 4;
-                part = t_ok && !whole && u > -4 && u < T;
-                any_part = __any(part);
-            } else if (SO != 0) {
+            } else if (AO != 0) {
 #pragma unroll
                 for (int o = 0; o < NO; ++o) own[o] = v[o];
             }
-            // never streaming: every one of these stores ends in a partial line that the next chunk completes,
-            // so the line has to wait in the cache
-            auto store_shifted = [&](__amdgpu_buffer_rsrc_t d, float4 q) {
-                buf_store4<false>(d, whole ? ubase : kOutOfRange, q);
-                if (any_part) {
+            const bool t_some = UNAL ? (t > -4 && t < T) : (unsigned)t < (unsigned)T;
+            const bool t_whole = t >= 0 && t <= T - 4;
+            // Sample t + e of the quad goes to position t + e + ko of the row.  A really shifted tensor is never
+            // stored with the streaming hint: each of its stores ends in a partial line that the next chunk
+            // completes, so the line has to wait in the cache.
+            auto store_through = [&](__amdgpu_buffer_rsrc_t d, float4 q, int ko, bool shifted) {
+                const int ubase = off0[p] + chunk * (TC * 4) + 4 * ko;
+                const int u = t + ko;
+                const bool whole = !careful || (t_some && t_whole && u >= 0 && u <= T - 4);
+                const bool part = careful && t_some && !whole && u > -4 && u < T;
+                if (shifted || !STREAM) buf_store4<false>(d, whole ? ubase : kOutOfRange, q);
+                else buf_store4<true>(d, whole ? ubase : kOutOfRange, q);
+                if (careful && __any(part)) {
                     const float e[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
-                        buf_store1<false>(d, (part && (unsigned)(u + j) < (unsigned)T) ? ubase + 4 * j : kOutOfRange, e[j]);
+                        buf_store1<false>(d, (part && (unsigned)(t + j) < (unsigned)T && (unsigned)(u + j) < (unsigned)T)
+                                                 ? ubase + 4 * j : kOutOfRange, e[j]);
                 }
             };
 #pragma unroll
             for (int o = 0; o < NO; ++o) {
-                if (((SO >> o) & 1u) != 0) store_shifted(dst[o], own[o]);
+                if (((SO >> o) & 1u) != 0) store_through(dst[o], own[o], kout[p], true);
+                else if (((AO >> o) & 1u) != 0) store_through(dst[o], own[o], 0, false);
                 else buf_store4<STREAM>(dst[o], off, v[o]);
             }
             if constexpr (ND == 1) {
-                if constexpr (((SO >> NO) & 1u) != 0) store_shifted(dst[NO], op.derive(own));
+                if constexpr (((SO >> NO) & 1u) != 0) store_through(dst[NO], op.derive(own), kout[p], true);
+                else if constexpr (((AO >> NO) & 1u) != 0) store_through(dst[NO], op.derive(own), 0, false);
                 else buf_store4<STREAM>(dst[NO], off, op.derive(v));
             }
         }
@@ -617,7 +644,9 @@ struct TileMap<Op, decltype((void)Op::kTileMapped)> {
 };
 
 // The sequential part: lane = neuron, one chunk of the tiles in place.
-template <class Op, int R, int UNROLL, int S = kTileSamples>
+// EXACT: rows may begin and end inside a quad (see Copier, UNAL); on the edge chunks the steps of a quad that lie
+// outside the row are then skipped one by one.
+template <class Op, int R, int UNROLL, int S = kTileSamples, bool EXACT = false>
 __device__ __forceinline__ void run_chunk(Op& op, float (*tile)[TileGeom<R, S>::kTileFloats], int lane, int chunk,
                                           bool inner, int a_lane, int T) {
     using G = TileGeom<R, S>;
@@ -649,11 +678,45 @@ __device__ __forceinline__ void run_chunk(Op& op, float (*tile)[TileGeom<R, S>::
 #pragma unroll UNROLL
             for (int q = 0; q < G::kQuads; ++q) run_quad(Op::kReverse ? G::kQuads - 1 - q : q);
         }
-    } else {
+    } else if (!EXACT) {
         const int tl = chunk * G::kChunk - a_lane;       // step held by column 0 of this lane's row
         for (int q = 0; q < G::kQuads; ++q) {
             const int qq = Op::kReverse ? G::kQuads - 1 - q : q;
             if (lane < R && (unsigned)(tl + 4 * qq) < (unsigned)T) run_quad(qq);
+        }
+    } else {
+        const int tl = chunk * G::kChunk - a_lane;
+        for (int q = 0; q < G::kQuads; ++q) {
+            const int qq = Op::kReverse ? G::kQuads - 1 - q : q;
+            const int t0 = tl + 4 * qq;                  // step of the quad's first column
+            if (lane < R && t0 > -4 && t0 < T) {
+                if (t0 >= 0 && t0 <= T - 4) {
+                    run_quad(qq);
+                } else {
+                    float xin[NI][4], yout[NO][4];
+#pragma unroll
+                    for (int i = 0; i < NI; ++i) {
+                        const float4 v = *reinterpret_cast<const float4*>(&tile[TileMap<Op>::in(i)][lane * G::kPitch + 4 * qq]);
+                        xin[i][0] = v.x; xin[i][1] = v.y; xin[i][2] = v.z; xin[i][3] = v.w;
+                    }
+#pragma unroll
+                    for (int st = 0; st < 4; ++st) {
+                        const int ss = Op::kReverse ? 3 - st : st;
+                        float x[NI], y[NO];
+#pragma unroll
+                        for (int i = 0; i < NI; ++i) x[i] = xin[i][ss];
+#pragma unroll
+                        for (int o = 0; o < NO; ++o) y[o] = 0.f;
+                        if ((unsigned)(t0 + ss) < (unsigned)T) op.step(x, y);    // steps outside the row leave the state alone
+#pragma unroll
+                        for (int o = 0; o < NO; ++o) yout[o][ss] = y[o];
+                    }
+#pragma unroll
+                    for (int o = 0; o < NO; ++o)
+                        *reinterpret_cast<float4*>(&tile[TileMap<Op>::out(o)][lane * G::kPitch + 4 * qq]) =
+                            make_float4(yout[o][0], yout[o][1], yout[o][2], yout[o][3]);
+                }
+            }
         }
     }
 }
@@ -704,7 +767,7 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
 // A chunk is a few hundred nanoseconds of recurrence, less than a trip to memory, so the copy
 // waves keep the loads of two chunks in flight (chunk j waits in fetched[j & 1]).  All waves run
 // an even number of chunks; a surplus chunk lies outside every row and neither computes nor stores.
-template <class Op, int R, bool STREAM, int NCOPY, int S = kTileSamples>
+template <class Op, int R, bool STREAM, int NCOPY, int S = kTileSamples, bool UNAL = false>
 __global__ __launch_bounds__((1 + NCOPY) * kWave) void stream_kernel_duo(typename Op::Params prm, int64_t M, int T) {
     using G = TileGeom<R, S>;
     constexpr int TC = G::kChunk;
@@ -732,14 +795,14 @@ __global__ __launch_bounds__((1 + NCOPY) * kWave) void stream_kernel_duo(typenam
             const int chunk = chunk_of(k);
             __syncthreads();                                   // barrier k
             if (k < nchunks)
-                run_chunk<Op, R, 4, S>(op, tiles[k & 1], lane, chunk, chunk >= 1 && chunk < interior_end, a_lane, T);
+                run_chunk<Op, R, 4, S, UNAL>(op, tiles[k & 1], lane, chunk, chunk >= 1 && chunk < interior_end, a_lane, T);
         }
         __syncthreads();                                       // barrier nloop
         op.finish(prm, m0 + lane, lane < rows);
     } else {
         Op uni;                                                // wave-uniform members only (pre, post, derive)
         uni.init(prm, 0, false);
-        Copier<Op, R, STREAM, PASSES, S> io;
+        Copier<Op, R, STREAM, PASSES, S, UNAL> io;
         io.init(prm, m0, rows, T, lane, base_f, (role - 1) * PASSES);
         float4 fetched[2][NI][PASSES];
         io.fetch_into(fetched[0], chunk_of(0));
@@ -773,7 +836,7 @@ __global__ __launch_bounds__((1 + NCOPY) * kWave) void stream_kernel_duo(typenam
 //   on chunk j-1 in tiles[(j-1) % 3], the copy waves store chunk j-2 from tiles[(j+1) % 3], refill them with
 //   chunk j+1 and issue the loads of chunk j+4 (three chunks of loads in flight).
 // Every wave passes the same number of barriers; chunk numbers outside [0, nchunks) name no chunk.
-template <class Op, int R, bool STREAM, int NCOPY>
+template <class Op, int R, bool STREAM, int NCOPY, bool UNAL = false>
 __global__ __launch_bounds__((2 + NCOPY) * kWave) void stream_kernel_staged(typename Op::Params prm, int64_t M, int T) {
     using G = TileGeom<R>;
     constexpr int TC = G::kChunk;
@@ -801,7 +864,7 @@ __global__ __launch_bounds__((2 + NCOPY) * kWave) void stream_kernel_staged(type
                 const int chunk = j + h - lag;
                 __syncthreads();                               // barrier j+h
                 if (chunk >= 0 && chunk < nchunks)
-                    run_chunk<typename std::remove_reference<decltype(stage)>::type, R, 4>(
+                    run_chunk<typename std::remove_reference<decltype(stage)>::type, R, 4, kTileSamples, UNAL>(
                         stage, tiles[(h + 3 - lag) % 3], lane, chunk, chunk >= 1 && chunk < interior_end, a_lane, T);
             }
         }
@@ -817,7 +880,7 @@ __global__ __launch_bounds__((2 + NCOPY) * kWave) void stream_kernel_staged(type
     } else {
         Op uni;                                                // wave-uniform members only (pre, post, derive)
         uni.init(prm, 0, false);
-        Copier<Op, R, STREAM, PASSES> io;
+        Copier<Op, R, STREAM, PASSES, kTileSamples, UNAL> io;
         io.init(prm, m0, rows, T, lane, base_f, (role - 2) * PASSES);
         float4 fetched[3][NI][PASSES];
 #pragma unroll
@@ -840,8 +903,9 @@ __global__ __launch_bounds__((2 + NCOPY) * kWave) void stream_kernel_staged(type
 }
 
 // ---------------------------------------------------------------------------------------------
-// Fallback for T % 4 != 0 or bases that are not 16-byte aligned: same tiling, dword accesses,
-// no phase and no boundary buffer.  Bit-exact, not tuned.
+// Last resort for rows shorter than a quad (T < 4) or longer than 2^22 steps: same tiling, no phase, no prefetch,
+// no boundary handling.  Bit-exact, not tuned.  (Rows that are merely not whole quads -- T % 4 != 0, bases that
+// are only dword-aligned -- take the multi-wave kernels in their UNAL form.)
 template <class Op, int R>
 __global__ __launch_bounds__(kWave) void stream_kernel_scalar(typename Op::Params prm, int64_t M, int T) {
     using G = TileGeom<R>;
@@ -1026,11 +1090,11 @@ template <class Op>
 struct CopyWaves<Op, decltype((void)Op::kCopyWaves)> { static constexpr int value = Op::kCopyWaves; };
 
 // Workgroups of the multi-wave kernel that one compute unit holds at a time (LDS and registers).
-template <class Op, int R, bool STREAM>
+template <class Op, int R, bool STREAM, bool UNAL = false>
 int duo_groups_per_cu() {
     static const int n = [] {
         int v = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&v, stream_kernel_duo<Op, R, STREAM, CopyWaves<Op>::value>,
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&v, stream_kernel_duo<Op, R, STREAM, CopyWaves<Op>::value, kTileSamples, UNAL>,
                                                          (1 + CopyWaves<Op>::value) * kWave, 0) != hipSuccess)
             v = 0;
         return v;
@@ -1137,11 +1201,11 @@ inline unsigned lds_pad_for(int groups, size_t static_lds) {
     const size_t pad = want - static_lds;
     return (unsigned)(pad > 60 * 1024 ? 60 * 1024 : pad);
 }
-template <class Op, int R, bool STREAM>
+template <class Op, int R, bool STREAM, bool UNAL = false>
 unsigned duo_pad_when_large() {
     static const unsigned pad = [] {
         hipFuncAttributes a;
-        if (hipFuncGetAttributes(&a, (const void*)stream_kernel_duo<Op, R, STREAM, CopyWaves<Op>::value>) != hipSuccess)
+        if (hipFuncGetAttributes(&a, (const void*)stream_kernel_duo<Op, R, STREAM, CopyWaves<Op>::value, kTileSamples, UNAL>) != hipSuccess)
             return 0u;
         return lds_pad_for(kGroupsPerCuWhenLarge, a.sharedSizeBytes);
     }();
@@ -1155,11 +1219,11 @@ struct StageCount { static constexpr int value = 1; };
 template <class Op>
 struct StageCount<Op, decltype((void)Op::kStages)> { static constexpr int value = Op::kStages; };
 
-template <class Op, bool STREAM>
+template <class Op, bool STREAM, bool UNAL = false>
 int staged_groups_per_cu() {
     static const int n = [] {
         int v = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&v, stream_kernel_staged<Op, 64, STREAM, CopyWaves<Op>::value>,
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&v, stream_kernel_staged<Op, 64, STREAM, CopyWaves<Op>::value, UNAL>,
                                                          (2 + CopyWaves<Op>::value) * kWave, 0) != hipSuccess)
             v = 0;
         return v;
@@ -1177,15 +1241,40 @@ struct StagedWhenLarge<Op, decltype((void)Op::kStagedWhenLarge)> { static conste
 // against the two-wave form; the fused ALIF forward, whose nine to twelve tiles leave room for one workgroup per
 // compute unit, loses a quarter at T = 300 and stays with the two-wave form.)
 constexpr int kStagedGroupsPerCuWhenLarge = 3;
-template <class Op, bool STREAM>
+template <class Op, bool STREAM, bool UNAL = false>
 unsigned staged_pad_when_large() {
     static const unsigned pad = [] {
         hipFuncAttributes a;
-        if (hipFuncGetAttributes(&a, (const void*)stream_kernel_staged<Op, 64, STREAM, CopyWaves<Op>::value>) != hipSuccess)
+        if (hipFuncGetAttributes(&a, (const void*)stream_kernel_staged<Op, 64, STREAM, CopyWaves<Op>::value, UNAL>) != hipSuccess)
             return 0u;
         return lds_pad_for(kStagedGroupsPerCuWhenLarge, a.sharedSizeBytes);
     }();
     return pad;
+}
+
+// Rows that are not whole quads (T % 4 != 0 or bases that are only dword-aligned): the multi-wave kernels in their
+// UNAL form, at every size (the one-wave kernels have no such form; rows shorter than a quad or longer than 2^22
+// steps stay with the dword kernel).
+template <class Op, bool STREAM>
+int launch_stream_unaligned(const typename Op::Params& prm, int64_t M, int64_t T, hipStream_t stream) {
+    constexpr int NC = CopyWaves<Op>::value;
+    if constexpr (StageCount<Op>::value == 2) {
+        const int per_cu = staged_groups_per_cu<Op, STREAM, true>();
+        const bool fits = (M + 63) / 64 <= (int64_t)per_cu * compute_units();
+        if (per_cu > 0 && (fits || StagedWhenLarge<Op>::value)) {
+            const dim3 grid((unsigned)((M + 63) / 64)), block((2 + NC) * kWave);
+            const unsigned pad = fits ? 0u : staged_pad_when_large<Op, STREAM, true>();
+            hipLaunchKernelGGL((stream_kernel_staged<Op, 64, STREAM, NC, true>), grid, block, pad, stream, prm, M, (int)T);
+            return (int)hipGetLastError();
+        }
+    }
+    constexpr int RD = DuoRows<Op>::value;
+    const int64_t groups = (M + RD - 1) / RD;
+    const bool resident = groups <= (int64_t)duo_groups_per_cu<Op, RD, STREAM, true>() * compute_units();
+    const dim3 grid((unsigned)groups), block((1 + NC) * kWave);
+    const unsigned pad = resident ? 0u : duo_pad_when_large<Op, RD, STREAM, true>();
+    hipLaunchKernelGGL((stream_kernel_duo<Op, RD, STREAM, NC, kTileSamples, true>), grid, block, pad, stream, prm, M, (int)T);
+    return (int)hipGetLastError();
 }
 
 template <class Op>
@@ -1193,6 +1282,9 @@ int launch_stream(const typename Op::Params& prm, int64_t M, int64_t T, hipStrea
     if (M == 0 || T == 0) return 0;
     const bool vec = stream_vectorizes<Op>(prm, T);
     const bool streaming = stream_is_large(M, T);
+    if (!vec && T >= 4 && T <= (1 << 22))
+        return streaming ? launch_stream_unaligned<Op, true>(prm, M, T, stream)
+                         : launch_stream_unaligned<Op, false>(prm, M, T, stream);
     const bool long_pieces = LongPiecesOnAliasedRows<Op>::value && row_stride_aliases(T);
     if constexpr (StageCount<Op>::value == 2) {
         const int per_cu = streaming ? staged_groups_per_cu<Op, true>() : staged_groups_per_cu<Op, false>();

@@ -70,6 +70,30 @@ def test_li_and_res_against_the_independent_kernels(slayer, N, C, H, T, offset):
         D.resonator.dynamics(x.detach(), x2.detach(), sin.detach(), cos.detach(), state, zero, 64, 0.8, debug=True)
 
 
+# Rows that are not whole quads (T % 4 != 0) or that start at addresses that are only dword-aligned: the multi-wave
+# kernels' form for them (csrc/tile.h, UNAL), where a row may begin and end inside a 16-byte quad.
+def _unaligned_cases():
+    rng = np.random.default_rng(4242)
+    cases = []
+    for T in [5, 6, 7, 9, 13, 30, 31, 33, 34, 35, 61, 63, 65, 66, 95, 97, 127, 130, 131, 301, 302, 303, 1001]:
+        N, C, H = int(rng.integers(1, 4)), int(rng.integers(1, 40)), int(rng.integers(1, 12))
+        cases.append((N, C, H, T, int(rng.integers(0, 4))))
+    cases.append((2, 600, 130, 37, 1))      # more workgroups than the chip holds at once
+    cases.append((3, 400, 110, 64, 3))      # whole quads in length, dword-aligned start
+    return cases
+
+
+@pytest.mark.parametrize('N,C,H,T,offset', _unaligned_cases())
+def test_rows_that_are_not_whole_quads(slayer, N, C, H, T, offset):
+    test_li_and_res_against_the_independent_kernels(slayer, N, C, H, T, offset)
+
+
+@pytest.mark.parametrize('N,C,H,T,offset', _unaligned_cases()[::3])
+@pytest.mark.parametrize('graded', [False, True])
+def test_fused_blocks_on_rows_that_are_not_whole_quads(slayer, N, C, H, T, offset, graded):
+    test_fused_blocks_against_the_operator_chains(slayer, N, C, H, T, offset, 64, graded)
+
+
 def _fused_cases():
     rng = np.random.default_rng(977)
     cases = []
