@@ -903,9 +903,10 @@ __global__ __launch_bounds__((2 + NCOPY) * kWave) void stream_kernel_staged(type
 }
 
 // ---------------------------------------------------------------------------------------------
-// Last resort for rows shorter than a quad (T < 4) or longer than 2^22 steps: same tiling, no phase, no prefetch,
-// no boundary handling.  Bit-exact, not tuned.  (Rows that are merely not whole quads -- T % 4 != 0, bases that
-// are only dword-aligned -- take the multi-wave kernels in their UNAL form.)
+// Rows that are not whole quads (T % 4 != 0, bases that are only dword-aligned) and are short (fewer than
+// kUnalignedMinSteps steps; longer ones take the multi-wave kernels in their UNAL form) or longer than 2^22 steps:
+// same tiling, 16-byte accesses at dword-aligned addresses for whole quads, no phase, no prefetch, no boundary
+// handling.  Bit-exact.
 template <class Op, int R>
 __global__ __launch_bounds__(kWave) void stream_kernel_scalar(typename Op::Params prm, int64_t M, int T) {
     using G = TileGeom<R>;
@@ -1253,8 +1254,13 @@ unsigned staged_pad_when_large() {
 }
 
 // Rows that are not whole quads (T % 4 != 0 or bases that are only dword-aligned): the multi-wave kernels in their
-// UNAL form, at every size (the one-wave kernels have no such form; rows shorter than a quad or longer than 2^22
+// UNAL form, at every neuron count (the one-wave kernels have no such form; short rows and rows longer than 2^22
 // steps stay with the dword kernel).
+// On short rows every chunk is an edge chunk and the sample-by-sample handling of the straddling quads outweighs
+// what prefetch and overlap bring: measured against the dword kernel, 131 072 rows of 37 / 65 steps lose (fused CUBA
+// fwd 36 -> 100 us, 54 -> 100 us), 65 536 rows of 129 steps are even, 32 768 rows of 301 steps win (81 -> 56 us).
+constexpr int64_t kUnalignedMinSteps = 256;
+
 template <class Op, bool STREAM>
 int launch_stream_unaligned(const typename Op::Params& prm, int64_t M, int64_t T, hipStream_t stream) {
     constexpr int NC = CopyWaves<Op>::value;
@@ -1282,7 +1288,7 @@ int launch_stream(const typename Op::Params& prm, int64_t M, int64_t T, hipStrea
     if (M == 0 || T == 0) return 0;
     const bool vec = stream_vectorizes<Op>(prm, T);
     const bool streaming = stream_is_large(M, T);
-    if (!vec && T >= 4 && T <= (1 << 22))
+    if (!vec && T >= kUnalignedMinSteps && T <= (1 << 22))
         return streaming ? launch_stream_unaligned<Op, true>(prm, M, T, stream)
                          : launch_stream_unaligned<Op, false>(prm, M, T, stream);
     const bool long_pieces = LongPiecesOnAliasedRows<Op>::value && row_stride_aliases(T);

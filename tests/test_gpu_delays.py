@@ -66,7 +66,9 @@ GEOMS = [((2, 5, 64), 'table', 'table', 1, True),
          ((1, 130, 300), 'scalar', 'table', 1, False),
          ((2, 9, 40), None, None, 1, True),                # step_delay alone
          ((2, 9, 40), 'table', None, 0, False),            # input shift alone
-         ((4, 33, 20), 'table', 'table', 2, False)]        # rows shorter than a line
+         ((4, 33, 20), 'table', 'table', 2, False),        # rows shorter than a line
+         ((2, 70, 301), 'table', 'table', 1, True),        # T % 4 != 0, long rows: multi-wave kernels, every tensor
+         ((1, 130, 258), 'scalar', 'table', 1, False)]     # on the careful path next to the really shifted ones
 
 
 # Tensors of 2^20 elements and more: the backward passes run as wave scans, with the delays folded into the scans'

@@ -75,11 +75,16 @@ def test_li_and_res_against_the_independent_kernels(slayer, N, C, H, T, offset):
 def _unaligned_cases():
     rng = np.random.default_rng(4242)
     cases = []
-    for T in [5, 6, 7, 9, 13, 30, 31, 33, 34, 35, 61, 63, 65, 66, 95, 97, 127, 130, 131, 301, 302, 303, 1001]:
+    # rows of 256 steps and more take the multi-wave form, shorter ones the dword kernel
+    for T in [5, 6, 7, 9, 13, 30, 31, 33, 34, 35, 61, 63, 65, 66, 95, 97, 127, 130, 131, 255, 257, 258, 259, 261, 287, 289,
+              301, 302, 303, 319, 321, 350, 450, 1001]:
         N, C, H = int(rng.integers(1, 4)), int(rng.integers(1, 40)), int(rng.integers(1, 12))
         cases.append((N, C, H, T, int(rng.integers(0, 4))))
-    cases.append((2, 600, 130, 37, 1))      # more workgroups than the chip holds at once
-    cases.append((3, 400, 110, 64, 3))      # whole quads in length, dword-aligned start
+    for T, offset in [(256, 1), (300, 2), (320, 3), (1000, 1)]:       # whole quads in length, dword-aligned start
+        cases.append((2, int(rng.integers(1, 40)), int(rng.integers(1, 12)), T, offset))
+    cases.append((2, 600, 130, 37, 1))      # more workgroups than the chip holds at once: dword kernel
+    cases.append((2, 300, 130, 257, 1))     # ... multi-wave form
+    cases.append((3, 400, 110, 64, 3))
     return cases
 
 
