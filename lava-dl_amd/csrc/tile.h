@@ -1195,6 +1195,11 @@ struct MultiwaveWhenLarge<Op, decltype((void)Op::kMultiwaveWhenLarge)> {
 // workgroup spends its first microseconds waiting for its first tiles and others must cover for it.
 constexpr int kGroupsPerCuWhenLarge = 4;
 
+// Rows of a chunk or two are all prologue for a workgroup of several waves: below 128 steps the one-wave kernels
+// stay (1 M rows of 16 steps: LI fwd 42 us one-wave, 74 us multi-wave; fused CUBA fwd 72 / 155; 512 K rows of
+// 32 steps: 36 / 46 and 52 / 88; at 64 steps even to 25 % behind, from 128 steps on 3-15 % ahead).
+constexpr int64_t kMultiwaveWhenLargeMinSteps = 128;
+
 // Dynamic LDS (unused by the kernel) that holds a kernel with `static_lds` bytes to `groups` workgroups per CU.
 inline unsigned lds_pad_for(int groups, size_t static_lds) {
     const size_t lds_per_cu = 160 * 1024, want = lds_per_cu / (size_t)(groups + 1) + 256;   // too much for groups + 1
@@ -1295,7 +1300,7 @@ int launch_stream(const typename Op::Params& prm, int64_t M, int64_t T, hipStrea
     if constexpr (StageCount<Op>::value == 2) {
         const int per_cu = streaming ? staged_groups_per_cu<Op, true>() : staged_groups_per_cu<Op, false>();
         const bool fits = (M + 63) / 64 <= (int64_t)per_cu * compute_units();
-        if (vec && per_cu > 0 && (fits || (StagedWhenLarge<Op>::value && !long_pieces))) {
+        if (vec && per_cu > 0 && (fits || (StagedWhenLarge<Op>::value && !long_pieces && T >= kMultiwaveWhenLargeMinSteps))) {
             constexpr int NC = CopyWaves<Op>::value;
             const dim3 grid((unsigned)((M + 63) / 64)), block((2 + NC) * kWave);
             if (streaming) {
@@ -1309,7 +1314,7 @@ int launch_stream(const typename Op::Params& prm, int64_t M, int64_t T, hipStrea
         }
     }
     const bool resident = stream_fits_multiwave<Op>(prm, M, T);
-    if (resident || (vec && MultiwaveWhenLarge<Op>::value && !long_pieces)) {
+    if (resident || (vec && MultiwaveWhenLarge<Op>::value && !long_pieces && T >= kMultiwaveWhenLargeMinSteps)) {
         constexpr int RD = DuoRows<Op>::value;
         constexpr int NC = CopyWaves<Op>::value;
         const dim3 grid((unsigned)((M + RD - 1) / RD)), block((1 + NC) * kWave);
