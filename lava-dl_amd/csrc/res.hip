@@ -120,6 +120,7 @@ struct AdResFwd {
 struct ResBwd {
     static constexpr int kIn = 4, kOut = 2;      // in: g_re, g_im, saved re, saved im
     static constexpr bool kReverse = true;
+    static constexpr int kCopyWaves = 2;
     static constexpr int64_t kRows32Below = kAlways, kRows16Below = 16384;
     struct Params {
         const float* in[4];
