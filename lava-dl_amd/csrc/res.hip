@@ -71,6 +71,7 @@ struct AdResFwd {
     static constexpr int kIn = 2, kOut = 4;      // out: real, imag, threshold, refractory
     static constexpr bool kReverse = false;
     static constexpr int64_t kRows32Below = kAlways, kRows16Below = 16384;
+    static constexpr bool kMultiwaveWhenLarge = true;
     struct Params {
         const float* in[2];
         float* out[4];
