@@ -233,6 +233,22 @@ __device__ __forceinline__ void scan_store_shifted(__amdgpu_buffer_rsrc_t dst, b
     }
 }
 
+// Rows of any length (T >= 4 floats, not a whole number of quads): a row is walked as ceil(T / 4) quads, the last
+// of which holds T mod 4 steps followed by steps that do not exist.  Its 16-byte load sits at T - 4, so the wanted
+// samples arrive in the upper elements: scan_tail_place() moves them down by `dd` = 4 - T mod 4 (uniform) and
+// zeroes the rest, after which the steps that do not exist behave as steps with zero input behind the row's end.
+__device__ __forceinline__ float4 scan_load_row(__amdgpu_buffer_rsrc_t src, bool in_span, int r, int pos, int T) {
+    const int s = 4 * pos;
+    return buf_load4<false>(src, in_span ? (r * T + (s > T - 4 ? T - 4 : s)) * 4 : kOutOfRange);
+}
+__device__ __forceinline__ float4 scan_tail_place(float4 q, int dd, bool row_end) {
+    float4 p = q;
+    if (dd == 1) p = make_float4(q.y, q.z, q.w, 0.f);
+    else if (dd == 2) p = make_float4(q.z, q.w, 0.f, 0.f);
+    else if (dd == 3) p = make_float4(q.w, 0.f, 0.f, 0.f);
+    return row_end ? p : q;
+}
+
 // Zeros at the positions of a shifted output that no sample reaches: [0, k) for k > 0, [T + k, T) for k < 0.
 __device__ __forceinline__ void scan_fill_unreached(__amdgpu_buffer_rsrc_t dst, const int* kout, const ScanSpan& sp,
                                                     int T) {
@@ -248,10 +264,11 @@ __device__ __forceinline__ void scan_fill_unreached(__amdgpu_buffer_rsrc_t dst, 
 // ---------------------------------------------------------------------------------------------
 // Leaky integrator backward.  npb (rows per batch element) and per_param (rows of a batch element that share a
 // parameter; npb when there is one parameter) are 32-bit: the launcher refuses anything larger.
-template <bool PARTIAL, bool STREAM>
+// ANYT: rows of any length T >= 4 (see scan_load_row); else T = 4 * QR and the span is read as one flat stream.
+template <bool PARTIAL, bool STREAM, bool ANYT = false>
 __global__ __launch_bounds__(kScanQuads) void li_bwd_scan_kernel(
         float* __restrict__ grad_in, float* __restrict__ partial, const float* __restrict__ grad_out,
-        const float* __restrict__ out, const float* __restrict__ decay, int64_t M, int QR, int rpg,
+        const float* __restrict__ out, const float* __restrict__ decay, int64_t M, int T, int QR, int rpg,
         unsigned npb, unsigned per_param) {
     __shared__ float a_tab[kScanMaxRows];
     __shared__ float row_sum[kScanWaves][kScanMaxRows];
@@ -259,25 +276,34 @@ __global__ __launch_bounds__(kScanQuads) void li_bwd_scan_kernel(
     ScanSpan sp;
     sp.init(M, QR, rpg);
     const int nq = sp.nq;
-    const int64_t base = sp.row0 * (int64_t)QR * 4;                  // first float of the span
-    const unsigned span_bytes = (unsigned)nq * 16u;
+    const int64_t base = sp.row0 * (int64_t)T;                       // first float of the span
+    const unsigned span_bytes = (unsigned)(sp.rows * T) * 4u;
+    const int dd = (4 - (T & 3)) & 3;
     const __amdgpu_buffer_rsrc_t src_g = make_rsrc(grad_out + base, span_bytes);
     const __amdgpu_buffer_rsrc_t src_y = make_rsrc(PARTIAL ? out + base : nullptr, PARTIAL ? span_bytes : 0u);
     const __amdgpu_buffer_rsrc_t dst = make_rsrc(grad_in + base, span_bytes);
 
-    ScanCursor cur;
+    ScanCursor cur, ahead;                           // ahead: the quad of this thread in the pass fetched next
     // Four pass buffers: the pass being worked on and the three after it, requested before anything else (a
     // workgroup lives for a handful of passes: what it reads should be on its way while it sets up).
-    auto fetch_g = [&](int q) { return buf_load4<STREAM>(src_g, (unsigned)q < (unsigned)nq ? q * 16 : kOutOfRange); };
-    auto fetch_y = [&](int q) {
-        return PARTIAL ? buf_load4<STREAM>(src_y, (unsigned)q < (unsigned)nq ? q * 16 : kOutOfRange)
-                       : make_float4(0.f, 0.f, 0.f, 0.f);
+    auto fetch = [&](float4& go, float4& y, int q) {
+        const bool in_span = (unsigned)q < (unsigned)nq;
+        if (ANYT) {
+            go = scan_load_row(src_g, in_span, ahead.r, ahead.pos, T);
+            y = PARTIAL ? scan_load_row(src_y, in_span, ahead.r, ahead.pos, T) : make_float4(0.f, 0.f, 0.f, 0.f);
+            ahead.next(QR);
+        } else {
+            go = buf_load4<STREAM>(src_g, in_span ? q * 16 : kOutOfRange);
+            y = PARTIAL ? buf_load4<STREAM>(src_y, in_span ? q * 16 : kOutOfRange) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
     };
     const int q0 = sp.first_quad();
-    float4 go0 = fetch_g(q0), y0 = fetch_y(q0);
-    float4 go1 = fetch_g(q0 - kScanQuads), y1 = fetch_y(q0 - kScanQuads);
-    float4 go2 = fetch_g(q0 - 2 * kScanQuads), y2 = fetch_y(q0 - 2 * kScanQuads);
-    float4 go3 = fetch_g(q0 - 3 * kScanQuads), y3 = fetch_y(q0 - 3 * kScanQuads);
+    if (ANYT) { cur.init(q0, nq, QR); ahead = cur; }
+    float4 go0, y0, go1, y1, go2, y2, go3, y3;
+    fetch(go0, y0, q0);
+    fetch(go1, y1, q0 - kScanQuads);
+    fetch(go2, y2, q0 - 2 * kScanQuads);
+    fetch(go3, y3, q0 - 3 * kScanQuads);
 
     const unsigned first = scan_first_in_batch(sp.row0, npb);
     for (int rr = sp.tid; rr < sp.rows; rr += kScanQuads)
@@ -287,18 +313,22 @@ __global__ __launch_bounds__(kScanQuads) void li_bwd_scan_kernel(
     int parity = (sp.npass - 1) & 1;
     if (sp.tid == 0) stage.carry[parity] = 0.0f;                     // nothing enters the last quad of the span
     __syncthreads();
-    cur.init(q0, nq, QR);
+    if (!ANYT) cur.init(q0, nq, QR);
 
     // one pass on the quads in (go, y); the buffer is then refilled with the pass four further on
     auto pass = [&](float4& go, float4& y) {
         const bool active = cur.lq < nq;
         const bool row_end = cur.pos == QR - 1;
+        if (ANYT && dd != 0) {
+            go = scan_tail_place(go, dd, row_end);
+            if (PARTIAL) y = scan_tail_place(y, dd, row_end);
+        }
         float entering;
         const float4 g = real_stage(stage, sp, parity, a_tab[cur.r], go, active, row_end, entering);
-        buf_store4<STREAM>(dst, active ? cur.lq * 16 : kOutOfRange, g);
+        if (ANYT) scan_store_shifted(dst, active, cur.r, cur.pos, 0, T, g);
+        else buf_store4<STREAM>(dst, active ? cur.lq * 16 : kOutOfRange, g);
         if (PARTIAL) add_to_row(row_sum[sp.wv], next_step_product(g, entering, y), sp, cur, QR, active);
-        go = fetch_g(cur.lq - 4 * kScanQuads);
-        y = fetch_y(cur.lq - 4 * kScanQuads);
+        fetch(go, y, cur.lq - 4 * kScanQuads);
         cur.next(QR);
         parity ^= 1;
     };
@@ -319,13 +349,14 @@ __global__ __launch_bounds__(kScanQuads) void li_bwd_scan_kernel(
 // own with the very arithmetic of li_bwd_scan_kernel -- the input gradient is bit-identical to the spike backward
 // kernel followed by two launches of that kernel.  THETA: the spike threshold is a tensor (threshold + refractory
 // of the adaptive neuron), else the scalar spike_thr.
-template <bool GRADED, bool DECAY_GRAD, bool THETA, bool STREAM, bool SHIFT = false, int NBUF = 3>
+template <bool GRADED, bool DECAY_GRAD, bool THETA, bool STREAM, int MODE = 0, int NBUF = 3>
 __global__ __launch_bounds__(kScanQuads) void cuba_bwd_scan_kernel(
         float* __restrict__ grad_in, float* __restrict__ partial_i, float* __restrict__ partial_v,
         const float* __restrict__ grad_spikes, const float* __restrict__ voltage, const float* __restrict__ theta,
         const float* __restrict__ current, const float* __restrict__ i_decay, const float* __restrict__ v_decay,
-        float spike_thr, float tau, float rho, int64_t M, int QR, int rpg,
+        float spike_thr, float tau, float rho, int64_t M, int T, int QR, int rpg,
         unsigned npb, unsigned per_i, unsigned per_v, Shifts shifts) {
+    constexpr bool SHIFT = MODE != 0, ANYT = MODE == 2;
     __shared__ float ai_tab[kScanMaxRows], av_tab[kScanMaxRows];
     __shared__ float sum_i[kScanWaves][kScanMaxRows], sum_v[kScanWaves][kScanMaxRows];
     __shared__ RealStage stage_v, stage_i;
@@ -333,9 +364,9 @@ __global__ __launch_bounds__(kScanQuads) void cuba_bwd_scan_kernel(
     ScanSpan sp;
     sp.init(M, QR, rpg);
     const int nq = sp.nq;
-    const int T = 4 * QR;
-    const int64_t base = sp.row0 * (int64_t)QR * 4;
-    const unsigned span_bytes = (unsigned)nq * 16u;
+    const int64_t base = sp.row0 * (int64_t)T;
+    const unsigned span_bytes = (unsigned)(sp.rows * T) * 4u;
+    const int dd = (4 - (T & 3)) & 3;
     const __amdgpu_buffer_rsrc_t src_g = make_rsrc(grad_spikes + base, span_bytes);
     const __amdgpu_buffer_rsrc_t src_v = make_rsrc(voltage + base, span_bytes);
     const __amdgpu_buffer_rsrc_t src_t = make_rsrc(THETA ? theta + base : nullptr, THETA ? span_bytes : 0u);
@@ -346,11 +377,19 @@ __global__ __launch_bounds__(kScanQuads) void cuba_bwd_scan_kernel(
 
     struct Quads { float4 g, v, th, c; int dg; };
     // the saved traces (never shifted), then the gradient of the spikes (read through the output delay when SHIFT)
-    auto fetch_saved = [&](Quads& x, int q) {
-        const int off = (unsigned)q < (unsigned)nq ? q * 16 : kOutOfRange;
-        x.v = buf_load4<STREAM>(src_v, off);
-        x.th = THETA ? buf_load4<STREAM>(src_t, off) : make_float4(0.f, 0.f, 0.f, 0.f);
-        x.c = DECAY_GRAD ? buf_load4<STREAM>(src_c, off) : make_float4(0.f, 0.f, 0.f, 0.f);
+    auto fetch_saved = [&](Quads& x, int q, const ScanCursor& at) {
+        const bool in_span = (unsigned)q < (unsigned)nq;
+        const float4 none = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (ANYT) {
+            x.v = scan_load_row(src_v, in_span, at.r, at.pos, T);
+            x.th = THETA ? scan_load_row(src_t, in_span, at.r, at.pos, T) : none;
+            x.c = DECAY_GRAD ? scan_load_row(src_c, in_span, at.r, at.pos, T) : none;
+        } else {
+            const int off = in_span ? q * 16 : kOutOfRange;
+            x.v = buf_load4<STREAM>(src_v, off);
+            x.th = THETA ? buf_load4<STREAM>(src_t, off) : none;
+            x.c = DECAY_GRAD ? buf_load4<STREAM>(src_c, off) : none;
+        }
     };
     auto fetch_grad = [&](Quads& x, int q, const ScanCursor& at) {
         if (SHIFT) {
@@ -364,10 +403,17 @@ __global__ __launch_bounds__(kScanQuads) void cuba_bwd_scan_kernel(
     // three passes are requested whole with three buffers; longer spans gain 7-8 % from a fourth)
     const int q0 = sp.first_quad();
     Quads b[NBUF];
-#pragma unroll
-    for (int h = 0; h < NBUF; ++h) fetch_saved(b[h], q0 - h * kScanQuads);
     ScanCursor cur, ahead;                           // ahead: the quad of this thread in the pass fetched next
-    cur.init(q0, nq, QR);
+    if (ANYT) {
+        cur.init(q0, nq, QR);
+        ahead = cur;
+#pragma unroll
+        for (int h = 0; h < NBUF; ++h) { fetch_saved(b[h], ahead.lq, ahead); ahead.next(QR); }
+    } else {
+#pragma unroll
+        for (int h = 0; h < NBUF; ++h) fetch_saved(b[h], q0 - h * kScanQuads, ahead);
+        cur.init(q0, nq, QR);
+    }
     ahead = cur;
     if (!SHIFT) {
 #pragma unroll
@@ -401,6 +447,11 @@ __global__ __launch_bounds__(kScanQuads) void cuba_bwd_scan_kernel(
         const bool active = cur.lq < nq;
         const bool row_end = cur.pos == QR - 1;
         if (SHIFT && __any(x.dg != 0)) x.g = scan_place(x.g, x.dg);      // rare: only where a row begins or ends
+        if (ANYT && dd != 0) {
+            x.v = scan_tail_place(x.v, dd, row_end);
+            if (THETA) x.th = scan_tail_place(x.th, dd, row_end);
+            if (DECAY_GRAD) x.c = scan_tail_place(x.c, dd, row_end);
+        }
         const float4 gv = make_float4(surrogate(x.g.x, x.v.x, x.th.x), surrogate(x.g.y, x.v.y, x.th.y),
                                       surrogate(x.g.z, x.v.z, x.th.z), surrogate(x.g.w, x.v.w, x.th.w));
         float ent_v, ent_i;
@@ -412,7 +463,7 @@ __global__ __launch_bounds__(kScanQuads) void cuba_bwd_scan_kernel(
             add_to_row(sum_v[sp.wv], next_step_product(gc, ent_v, x.v), sp, cur, QR, active);
             add_to_row(sum_i[sp.wv], next_step_product(gx, ent_i, x.c), sp, cur, QR, active);
         }
-        fetch_saved(x, cur.lq - NBUF * kScanQuads);
+        fetch_saved(x, cur.lq - NBUF * kScanQuads, ahead);
         if (SHIFT) { fetch_grad(x, ahead.lq, ahead); ahead.next(QR); }
         else fetch_grad(x, cur.lq - NBUF * kScanQuads, ahead);
         cur.next(QR);
@@ -488,14 +539,15 @@ __device__ __forceinline__ void complex_spike_surrogate(const SpikeSurrogate& k,
     g_im = g * (((neg_rho_over_tau * sg_i) * d_im) * step_re);
 }
 
-template <bool PARTIAL, bool STREAM, int SURR, bool SHIFT = false, int NBUF = 3>
+template <bool PARTIAL, bool STREAM, int SURR, int MODE = 0, int NBUF = 3>
 __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
         float* __restrict__ g_re_in, float* __restrict__ g_im_in, float* __restrict__ partial_sin,
         float* __restrict__ partial_cos, const float* __restrict__ g_re, const float* __restrict__ g_im,
         const float* __restrict__ re, const float* __restrict__ im, const float* __restrict__ sin_decay,
-        const float* __restrict__ cos_decay, SpikeSurrogate surr, int64_t M, int QR, int rpg, unsigned npb,
+        const float* __restrict__ cos_decay, SpikeSurrogate surr, int64_t M, int T, int QR, int rpg, unsigned npb,
         unsigned per_param, Shifts shifts) {
-    static_assert(!SHIFT || SURR != 0, "delays are folded into the fused resonate-and-fire form only");
+    constexpr bool SHIFT = MODE != 0, ANYT = MODE == 2;
+    static_assert(MODE != 1 || SURR != 0, "delays are folded into the fused resonate-and-fire form only");
     __shared__ float c_tab[kScanMaxRows], s_tab[kScanMaxRows];
     __shared__ float sum_s[kScanWaves][kScanMaxRows], sum_c[kScanWaves][kScanMaxRows];
     __shared__ ComplexStage L;
@@ -503,9 +555,9 @@ __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
     ScanSpan sp;
     sp.init(M, QR, rpg);
     const int nq = sp.nq;
-    const int T = 4 * QR;
-    const int64_t base = sp.row0 * (int64_t)QR * 4;
-    const unsigned span_bytes = (unsigned)nq * 16u;
+    const int64_t base = sp.row0 * (int64_t)T;
+    const unsigned span_bytes = (unsigned)(sp.rows * T) * 4u;
+    const int dd = (4 - (T & 3)) & 3;
     constexpr bool kStates = PARTIAL || SURR != 0;          // the saved states are read
     const __amdgpu_buffer_rsrc_t src_gr = make_rsrc(g_re + base, span_bytes);
     const __amdgpu_buffer_rsrc_t src_gi = make_rsrc(SURR == 0 ? g_im + base : nullptr, SURR == 0 ? span_bytes : 0u);
@@ -515,11 +567,19 @@ __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
 
     struct Quads { float4 gr, gi, re, im; int dg; };
     // the tensors that are never shifted, then the incoming gradient (read through the output delay when SHIFT)
-    auto fetch_saved = [&](Quads& x, int q) {
-        const int off = (unsigned)q < (unsigned)nq ? q * 16 : kOutOfRange;
-        x.gi = SURR == 0 ? buf_load4<STREAM>(src_gi, off) : make_float4(0.f, 0.f, 0.f, 0.f);
-        x.re = kStates ? buf_load4<STREAM>(src_re, off) : make_float4(0.f, 0.f, 0.f, 0.f);
-        x.im = kStates ? buf_load4<STREAM>(src_im, off) : make_float4(0.f, 0.f, 0.f, 0.f);
+    auto fetch_saved = [&](Quads& x, int q, const ScanCursor& at) {
+        const bool in_span = (unsigned)q < (unsigned)nq;
+        const float4 none = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (ANYT) {
+            x.gi = SURR == 0 ? scan_load_row(src_gi, in_span, at.r, at.pos, T) : none;
+            x.re = kStates ? scan_load_row(src_re, in_span, at.r, at.pos, T) : none;
+            x.im = kStates ? scan_load_row(src_im, in_span, at.r, at.pos, T) : none;
+        } else {
+            const int off = in_span ? q * 16 : kOutOfRange;
+            x.gi = SURR == 0 ? buf_load4<STREAM>(src_gi, off) : none;
+            x.re = kStates ? buf_load4<STREAM>(src_re, off) : none;
+            x.im = kStates ? buf_load4<STREAM>(src_im, off) : none;
+        }
     };
     auto fetch_grad = [&](Quads& x, int q, const ScanCursor& at) {
         if (SHIFT) {
@@ -531,10 +591,17 @@ __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
     };
     const int q0 = sp.first_quad();
     Quads b[NBUF];
-#pragma unroll
-    for (int h = 0; h < NBUF; ++h) fetch_saved(b[h], q0 - h * kScanQuads);
     ScanCursor cur, ahead;                           // ahead: the quad of this thread in the pass fetched next
-    cur.init(q0, nq, QR);
+    if (ANYT) {
+        cur.init(q0, nq, QR);
+        ahead = cur;
+#pragma unroll
+        for (int h = 0; h < NBUF; ++h) { fetch_saved(b[h], ahead.lq, ahead); ahead.next(QR); }
+    } else {
+#pragma unroll
+        for (int h = 0; h < NBUF; ++h) fetch_saved(b[h], q0 - h * kScanQuads, ahead);
+        cur.init(q0, nq, QR);
+    }
     ahead = cur;
     if (!SHIFT) {
 #pragma unroll
@@ -565,6 +632,10 @@ __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
         const bool row_end = cur.pos == QR - 1;
         const Cx mu{c_tab[cur.r], -s_tab[cur.r]};
         if (SHIFT && __any(x.dg != 0)) x.gr = scan_place(x.gr, x.dg);    // rare: only where a row begins or ends
+        if (ANYT && dd != 0) {
+            if (SURR == 0) x.gi = scan_tail_place(x.gi, dd, row_end);
+            if (kStates) { x.re = scan_tail_place(x.re, dd, row_end); x.im = scan_tail_place(x.im, dd, row_end); }
+        }
         if (SURR != 0) {                   // quads outside the span hold zeros: their gradient is zero too
             const float4 g = x.gr;
             complex_spike_surrogate<SURR>(surr, g.x, x.re.x, x.im.x, x.gr.x, x.gi.x);
@@ -614,7 +685,7 @@ __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
             add_to_row(sum_s[sp.wv], ss, sp, cur, QR, active);
             add_to_row(sum_c[sp.wv], sc, sp, cur, QR, active);
         }
-        fetch_saved(x, cur.lq - NBUF * kScanQuads);
+        fetch_saved(x, cur.lq - NBUF * kScanQuads, ahead);
         if (SHIFT) { fetch_grad(x, ahead.lq, ahead); ahead.next(QR); }
         else fetch_grad(x, cur.lq - NBUF * kScanQuads, ahead);
         cur.next(QR);
@@ -659,21 +730,26 @@ int64_t bwd_scan_min_elements() {
     return v;
 }
 
-// True when the scan kernels can run a problem of this shape: whole quads, spans addressable with 32 bits,
-// 32-bit row arithmetic, large enough (the callers also check that every tensor is 16-byte aligned).
+// True when the scan kernels can run a problem of this shape: spans addressable with 32 bits, 32-bit row
+// arithmetic, large enough (the callers also check that every tensor is 16-byte aligned).  Rows that are not a
+// whole number of quads take the any-length form of the kernels, from kScanAnyLengthMinSteps steps on (a short
+// row is mostly its partial last quad).
+constexpr int64_t kScanAnyLengthMinSteps = 64;
 bool bwd_scan_usable(int64_t M, int64_t npb, int64_t T) {
-    if (M <= 0 || T <= 0 || (T % 4) != 0 || T > (1 << 22) || M * T < bwd_scan_min_elements()) return false;
+    if (M <= 0 || T < 4 || T > (1 << 22) || M * T < bwd_scan_min_elements()) return false;
+    if ((T % 4) != 0 && T < kScanAnyLengthMinSteps) return false;
     return npb > 0 && npb < ((int64_t)1 << 31);
 }
 
-struct ScanGrid { dim3 grid; int rpg, QR, passes; bool streaming, ok; };   // passes: of a full span
+struct ScanGrid { dim3 grid; int rpg, QR, passes; bool streaming, ok, any_length; };   // passes: of a full span
 static ScanGrid scan_grid(int64_t M, int64_t T) {
     ScanGrid g;
     g.rpg = scan_rows_per_group(M, T);
     const int64_t blocks = (M + g.rpg - 1) / g.rpg;
     g.ok = blocks <= 0x7fffffffLL;
     g.grid = dim3((unsigned)blocks);
-    g.QR = (int)(T / 4);
+    g.QR = (int)((T + 3) / 4);
+    g.any_length = (T % 4) != 0;
     g.passes = (int)(((int64_t)g.rpg * g.QR + kScanQuads - 1) / kScanQuads);
     g.streaming = stream_is_large(M, T);
     return g;
@@ -684,11 +760,12 @@ int launch_li_bwd_scan(float* grad_in, float* partial, const float* grad_out, co
                        int64_t M, int64_t npb, int64_t num_decays, int64_t T, hipStream_t stream) {
     const ScanGrid g = scan_grid(M, T);
     if (!g.ok) return SLAYER_ERANGE;
-#define SLAYER_SCAN(P, S)                                                                                        \
-    hipLaunchKernelGGL((li_bwd_scan_kernel<P, S>), g.grid, dim3(kScanQuads), 0, stream, grad_in, partial, grad_out, \
-                       out, decay, M, g.QR, g.rpg, (unsigned)npb, rows_per_param(npb, num_decays))
-    if (partial) { if (g.streaming) SLAYER_SCAN(true, true); else SLAYER_SCAN(true, false); }
-    else { if (g.streaming) SLAYER_SCAN(false, true); else SLAYER_SCAN(false, false); }
+#define SLAYER_SCAN(P, S, A)                                                                                     \
+    hipLaunchKernelGGL((li_bwd_scan_kernel<P, S, A>), g.grid, dim3(kScanQuads), 0, stream, grad_in, partial,     \
+                       grad_out, out, decay, M, (int)T, g.QR, g.rpg, (unsigned)npb, rows_per_param(npb, num_decays))
+    if (g.any_length) { if (partial) SLAYER_SCAN(true, false, true); else SLAYER_SCAN(false, false, true); }
+    else if (partial) { if (g.streaming) SLAYER_SCAN(true, true, false); else SLAYER_SCAN(true, false, false); }
+    else { if (g.streaming) SLAYER_SCAN(false, true, false); else SLAYER_SCAN(false, false, false); }
 #undef SLAYER_SCAN
     return (int)hipGetLastError();
 }
@@ -707,11 +784,11 @@ int launch_cuba_bwd_scan(float* grad_in, float* partial_i, float* partial_v, con
 #define SLAYER_SCAN_N(G, D, TH, S, SH, NB)                                                                       \
     hipLaunchKernelGGL((cuba_bwd_scan_kernel<G, D, TH, S, SH, NB>), g.grid, dim3(kScanQuads), 0, stream, grad_in, \
                        partial_i, partial_v, grad_spikes, voltage, theta, current, i_decay, v_decay, spike_thr,  \
-                       tau, rho, M, g.QR, g.rpg, (unsigned)npb, rows_per_param(npb, n_id),                       \
+                       tau, rho, M, (int)T, g.QR, g.rpg, (unsigned)npb, rows_per_param(npb, n_id),               \
                        rows_per_param(npb, n_vd), sh)
 #define SLAYER_SCAN(G, D, TH, S, SH) do { if (g.passes > 3) SLAYER_SCAN_N(G, D, TH, S, SH, 4); else SLAYER_SCAN_N(G, D, TH, S, SH, 3); } while (0)
-#define SLAYER_SCAN_H(G, D, TH, S) do { if (shifts) SLAYER_SCAN(G, D, TH, S, true); else SLAYER_SCAN(G, D, TH, S, false); } while (0)
-#define SLAYER_SCAN_S(G, D, TH) do { if (g.streaming) SLAYER_SCAN_H(G, D, TH, true); else SLAYER_SCAN_H(G, D, TH, false); } while (0)
+#define SLAYER_SCAN_H(G, D, TH, S) do { if (shifts) SLAYER_SCAN(G, D, TH, S, 1); else SLAYER_SCAN(G, D, TH, S, 0); } while (0)
+#define SLAYER_SCAN_S(G, D, TH) do { if (g.any_length) SLAYER_SCAN(G, D, TH, false, 2); else if (g.streaming) SLAYER_SCAN_H(G, D, TH, true); else SLAYER_SCAN_H(G, D, TH, false); } while (0)
 #define SLAYER_SCAN_T(G, D) do { if (theta) SLAYER_SCAN_S(G, D, true); else SLAYER_SCAN_S(G, D, false); } while (0)
     const bool want = partial_i != nullptr;
     if (graded) { if (want) SLAYER_SCAN_T(true, true); else SLAYER_SCAN_T(true, false); }
@@ -737,14 +814,15 @@ int launch_res_bwd_scan(float* g_re_in, float* g_im_in, float* partial_sin, floa
     const Shifts sh = shifts ? *shifts : Shifts{nullptr, nullptr, nullptr, nullptr, 0, 0, 1, 1.0f, 1};
 #define SLAYER_SCAN_N(P, S, U, SH, NB)                                                                           \
     hipLaunchKernelGGL((res_bwd_scan_kernel<P, S, U, SH, NB>), g.grid, dim3(kScanQuads), 0, stream, g_re_in, g_im_in, \
-                       partial_sin, partial_cos, g_re, g_im, re, im, sin_decay, cos_decay, k, M, g.QR, g.rpg,    \
+                       partial_sin, partial_cos, g_re, g_im, re, im, sin_decay, cos_decay, k, M, (int)T, g.QR,   \
+                       g.rpg,                                                                                    \
                        (unsigned)npb, rows_per_param(npb, num_decays), sh)
 #define SLAYER_SCAN(P, S, U, SH) do { if (g.passes > 3) SLAYER_SCAN_N(P, S, U, SH, 4); else SLAYER_SCAN_N(P, S, U, SH, 3); } while (0)
-#define SLAYER_SCAN_S(P, U, SH) do { if (g.streaming) SLAYER_SCAN(P, true, U, SH); else SLAYER_SCAN(P, false, U, SH); } while (0)
+#define SLAYER_SCAN_S(P, U, SH) do { if (g.any_length) SLAYER_SCAN(P, false, U, 2); else if (g.streaming) SLAYER_SCAN(P, true, U, SH); else SLAYER_SCAN(P, false, U, SH); } while (0)
 #define SLAYER_SCAN_P(U, SH) do { if (partial_sin) SLAYER_SCAN_S(true, U, SH); else SLAYER_SCAN_S(false, U, SH); } while (0)
-    if (surrogate == 0) SLAYER_SCAN_P(0, false);
-    else if (surrogate == 1) { if (shifts) SLAYER_SCAN_P(1, true); else SLAYER_SCAN_P(1, false); }
-    else { if (shifts) SLAYER_SCAN_P(2, true); else SLAYER_SCAN_P(2, false); }
+    if (surrogate == 0) SLAYER_SCAN_P(0, 0);
+    else if (surrogate == 1) { if (shifts) SLAYER_SCAN_P(1, 1); else SLAYER_SCAN_P(1, 0); }
+    else { if (shifts) SLAYER_SCAN_P(2, 1); else SLAYER_SCAN_P(2, 0); }
 #undef SLAYER_SCAN_P
 #undef SLAYER_SCAN_S
 #undef SLAYER_SCAN

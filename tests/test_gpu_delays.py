@@ -77,7 +77,9 @@ GEOMS = [((2, 5, 64), 'table', 'table', 1, True),
 GEOMS_SCAN = [((4, 300, 900), 'table', 'table', 1, True),          # T % 32 != 0
               ((2, 16, 6, 7, 800), 'table', 'table', 0, False),    # NCHWT, per-neuron tables
               ((8, 450, 300), 'scalar', 'table', 1, False),        # short rows: spans of 8 rows
-              ((2, 260, 2048), 'table', None, 2, False)]           # rows a power of two long
+              ((2, 260, 2048), 'table', None, 2, False),           # rows a power of two long
+              ((4, 300, 901), 'table', 'table', 1, True),          # rows that are not whole quads
+              ((8, 450, 302), 'scalar', 'table', 1, False)]
 
 
 def _same_gradient(a, b, what):

@@ -20,7 +20,10 @@ def slayer():
 # (shape, number of decays): rows of one quad, rows shorter / longer than a wave and than a pass, row counts that
 # do not fill the last workgroup, rows that are a whole number of lines and rows that are not, per-neuron decays
 SHAPES = [((262144 + 3, 1, 4), 1), ((3, 43691, 8), 43691), ((5, 1024, 300), 1024), ((2, 4099, 128), 4099),
-          ((7, 161, 1000), 161), ((3, 43, 8196), 43), ((1, 2, 524288), 2), ((2, 16, 33, 31, 76), 16)]
+          ((7, 161, 1000), 161), ((3, 43, 8196), 43), ((1, 2, 524288), 2), ((2, 16, 33, 31, 76), 16),
+          # rows that are not a whole number of quads (T % 4 = 1, 2, 3): the any-length form of the scans
+          ((5, 1024, 301), 1024), ((7, 161, 1002), 161), ((3, 43, 8195), 43), ((2, 4099, 129), 4099),
+          ((4, 4100, 67), 4100), ((1, 3, 400001), 3)]
 
 
 @pytest.mark.parametrize('shape,nd', SHAPES)
@@ -72,7 +75,8 @@ def test_li_bwd_scan_whole_tensor_against_oracle(slayer):
     assert_rel(gd, r_gd, 'grad_decay vs oracle', rel=1e-4)
 
 
-@pytest.mark.parametrize('shape,nd', [((3, 700, 520), 700), ((2, 16, 40, 32, 28), 16), ((9, 128, 1000), 1)])
+@pytest.mark.parametrize('shape,nd', [((3, 700, 520), 700), ((2, 16, 40, 32, 28), 16), ((9, 128, 1000), 1),
+                                      ((3, 700, 521), 700), ((9, 128, 1003), 1), ((6, 300, 602), 300)])
 def test_res_bwd_scan_against_oracle(slayer, shape, nd):
     R = slayer.neuron.dynamics.resonator
     gen = torch.Generator().manual_seed(seed_of('res-scan', shape))
@@ -99,7 +103,8 @@ def test_res_bwd_scan_against_oracle(slayer, shape, nd):
         assert_rel(got[3], red(c_sum).float(), 'grad cos', rel=1e-4)
 
 
-@pytest.mark.parametrize('shape', [(5, 1024, 300), (2, 16, 33, 31, 76), (3, 43, 8196)])
+@pytest.mark.parametrize('shape', [(5, 1024, 300), (2, 16, 33, 31, 76), (3, 43, 8196),
+                                   (5, 1024, 301), (3, 43, 8194), (4, 2100, 127)])
 @pytest.mark.parametrize('graded', [False, True])
 @pytest.mark.parametrize('kind', ['cuba', 'alif'])
 def test_fused_backward_scans_equal_the_chain_of_scans_bit_for_bit(slayer, shape, graded, kind):
@@ -131,7 +136,8 @@ def test_fused_backward_scans_equal_the_chain_of_scans_bit_for_bit(slayer, shape
             assert_rel(g_v, r_gv.cpu(), 'grad voltage decay', rel=1e-4)
 
 
-@pytest.mark.parametrize('shape', [(5, 1024, 300), (2, 16, 33, 31, 76), (3, 43, 8196)])
+@pytest.mark.parametrize('shape', [(5, 1024, 300), (2, 16, 33, 31, 76), (3, 43, 8196),
+                                   (5, 1024, 301), (3, 43, 8194), (4, 2100, 127)])
 @pytest.mark.parametrize('graded', [False, True])
 def test_fused_rf_backward_scan_equals_the_chain_of_scans_bit_for_bit(slayer, shape, graded):
     """Complex spike surrogate + resonator backward scan in one kernel against the two operators in a row (same
