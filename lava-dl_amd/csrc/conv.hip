@@ -96,7 +96,7 @@ __global__ __launch_bounds__(kWave) void conv_kernel(float* __restrict__ out, co
 }
 
 // ---------------------------------------------------------------------------------------------
-// Matrix-core form for 8 < K <= 128 (T % 4 == 0, T >= 16, 16-byte aligned tensors).  The tensor is walked as one
+// Matrix-core form for 8 < K <= 128 (T >= 16, M * T a whole number of quads, 16-byte aligned tensors).  The tensor is walked as one
 // flat stream of M * T samples in tiles of 256 consecutive samples, each seen as 16 blocks of 16 output steps:
 // D[i][n] = output 16 n + i of the tile is the [16 x (16 + KPAD)] Toeplitz matrix of taps times the
 // [(16 + KPAD) x 16] matrix whose column n is the window of block n (v_mfma_f32_16x16x4_f32, four window samples
@@ -113,7 +113,9 @@ __global__ __launch_bounds__(kWave) void conv_kernel(float* __restrict__ out, co
 // The Toeplitz operands do not depend on the tile and stay in registers (4 per window group).
 //
 // Rows: a block's window must not see the neighbouring row.  Every lane masks the window quads of its block that
-// lie outside the row of the block (it reads a quad of zeros instead; rows are whole quads).  A block that holds
+// lie outside the row of the block (it reads a quad of zeros instead).  Where rows are not whole quads (ANYT: T % 4
+// != 0) a row begins or ends inside a quad: the samples of such a quad that belong to the other row are replaced by
+// zeros one by one, and an output quad that straddles two rows takes each output from its own row's view.  A block that holds
 // the end of one row and the start of the next (T % 16 != 0) needs both views: such a tile is multiplied twice,
 // once with every block seeing the row of its first output and once the row of its last output, and every output
 // quad takes the result of its own row.
@@ -125,7 +127,7 @@ typedef float mfma_f4 __attribute__((ext_vector_type(4)));
 constexpr int kConvTile = 256;             // samples per tile
 constexpr int kConvRing = 4;               // tiles in the LDS ring = tiles per loop pass
 
-template <int KPAD, bool CORR>
+template <int KPAD, bool CORR, bool ANYT = false>
 __global__ __launch_bounds__(kWave) void conv_mfma_kernel(float* __restrict__ out, const float* __restrict__ in,
                                                           const float* __restrict__ filt, int K, float ts,
                                                           int64_t total, int T, int tiles_per_wave) {
@@ -215,8 +217,15 @@ __global__ __launch_bounds__(kWave) void conv_mfma_kernel(float* __restrict__ ou
                 const int lo_a = ra * T - lead, rb_more = (o0 - ra * T + 15 >= T) ? T : 0;
                 auto multiply = [&](mfma_f4 d, int g, int lo) -> mfma_f4 {
                     const int q = tile0 + wq + 16 * g;                // first sample of the quad
-                    const bool ok = q >= lo && q < lo + T;
-                    const float4 xv = ring[ok ? ((here + opnd[g]) & (kConvRing * 64 - 1)) : kZero];
+                    const bool ok = ANYT ? (q + 3 >= lo && q < lo + T) : (q >= lo && q < lo + T);
+                    float4 xv = ring[ok ? ((here + opnd[g]) & (kConvRing * 64 - 1)) : kZero];
+                    if (ANYT) {                                       // a row may begin or end inside the quad
+                        const unsigned rel = (unsigned)(q - lo);
+                        xv.x = rel < (unsigned)T ? xv.x : 0.0f;
+                        xv.y = rel + 1u < (unsigned)T ? xv.y : 0.0f;
+                        xv.z = rel + 2u < (unsigned)T ? xv.z : 0.0f;
+                        xv.w = rel + 3u < (unsigned)T ? xv.w : 0.0f;
+                    }
                     d = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][0], xv.x, d, 0, 0, 0);
                     d = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][1], xv.y, d, 0, 0, 0);
                     d = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][2], xv.z, d, 0, 0, 0);
@@ -232,12 +241,12 @@ __global__ __launch_bounds__(kWave) void conv_mfma_kernel(float* __restrict__ ou
                 if (__any(rb_more != 0)) {
                     mfma_f4 other = {0.0f, 0.0f, 0.0f, 0.0f};
                     other = multiply(other, CORR ? 0 : G - 1, lo_a + (CORR ? 0 : rb_more));
-                    const bool in_next = (tile0 + 16 * n + 4 * kq) >= lo_a + T;      // this lane's output quad
-                    const bool take = rb_more != 0 && in_next != CORR;
-                    acc[0] = take ? other[0] : acc[0];
-                    acc[1] = take ? other[1] : acc[1];
-                    acc[2] = take ? other[2] : acc[2];
-                    acc[3] = take ? other[3] : acc[3];
+                    const int oq = tile0 + 16 * n + 4 * kq;           // this lane's output quad
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const bool in_next = oq + (ANYT ? j : 0) >= lo_a + T;
+                        acc[j] = (rb_more != 0 && in_next != CORR) ? other[j] : acc[j];
+                    }
                 }
             }
             const int t = tile0 + 16 * n + 4 * kq;
@@ -247,7 +256,7 @@ __global__ __launch_bounds__(kWave) void conv_mfma_kernel(float* __restrict__ ou
     }
 }
 
-template <bool CORR>
+template <bool CORR, bool ANYT>
 static int conv_mfma_launch(float* out, const float* in, const float* filt, int K, float ts, int64_t M, int64_t T,
                             hipStream_t stream) {
     // about eight thousand waves (four per SIMD on 256 compute units, twice over), each a whole number of loop
@@ -260,7 +269,7 @@ static int conv_mfma_launch(float* out, const float* in, const float* filt, int 
     const int64_t blocks = (tiles + per_wave - 1) / per_wave;
     if (blocks > 0x7fffffffLL) return SLAYER_ERANGE;
 #define SLAYER_CONV_MFMA(KP)                                                                                      \
-    hipLaunchKernelGGL((conv_mfma_kernel<KP, CORR>), dim3((unsigned)blocks), dim3(kWave), 0, stream, out, in, filt, \
+    hipLaunchKernelGGL((conv_mfma_kernel<KP, CORR, ANYT>), dim3((unsigned)blocks), dim3(kWave), 0, stream, out, in, filt, \
                        K, ts, total, (int)T, (int)per_wave)
     if (K <= 16) SLAYER_CONV_MFMA(16);
     else if (K <= 32) SLAYER_CONV_MFMA(32);
@@ -278,8 +287,11 @@ static int conv_launch(float* out, const float* in, const float* filt, int64_t K
     if (!out || !in || !filt) return SLAYER_ENULL;
     if (K < 1) return SLAYER_EINVAL;
     if (K > kMaxTaps) return SLAYER_ERANGE;
-    if (K > 8 && K <= 128 && T % 4 == 0 && T >= 16 && T <= (1 << 22) && aligned16(out) && aligned16(in))
-        return conv_mfma_launch<CORR>(out, in, filt, (int)K, ts, M, T, stream);
+    // the matrix kernel walks the tensor as one flat stream of whole quads: rows of any length from 16 steps on, as
+    // long as the tensor as a whole is a whole number of quads
+    if (K > 8 && K <= 128 && (M * T) % 4 == 0 && T >= 16 && T <= (1 << 22) && aligned16(out) && aligned16(in))
+        return T % 4 == 0 ? conv_mfma_launch<CORR, false>(out, in, filt, (int)K, ts, M, T, stream)
+                          : conv_mfma_launch<CORR, true>(out, in, filt, (int)K, ts, M, T, stream);
     const unsigned segs = (unsigned)((T + kSeg - 1) / kSeg);
     const int64_t blocks = M * (int64_t)segs;
     if (blocks > 0x7fffffffLL) return SLAYER_ERANGE;

@@ -105,13 +105,17 @@ def test_conv_corr(slayer, shape, K):
                                      ((7, 11, 300), 100), ((33, 520), 128), ((33, 520), 129), ((4, 12), 40),
                                      ((50, 16), 64), ((40, 20), 17), ((700, 36), 128), ((33, 148), 100),
                                      ((4000, 300), 64), ((3, 5, 1500), 64), ((5, 2, 4096), 9), ((1, 1, 16), 16),
-                                     ((2, 1021, 256), 33), ((300, 1028), 16)])
+                                     ((2, 1021, 256), 33), ((300, 1028), 16),
+                                     # rows that are not whole quads (the tensor as a whole still is)
+                                     ((4, 37, 350), 64), ((8, 301), 64), ((12, 1003), 33), ((64, 250), 16),
+                                     ((4, 5, 18), 9), ((20, 17), 12), ((2, 6, 1450), 100), ((4000, 302), 64),
+                                     ((4, 999, 19), 64), ((2, 2, 4099), 128)])
 def test_conv_corr_matrix_core_path(slayer, shape, K):
     """The matrix-core kernel walks the tensor as one stream of 256-sample tiles.  Tap counts either side of every
     padded size (16, 32, 64, 128) and of the kernel's limits (8 < K <= 128, T >= 16); rows shorter than a block, a
     tile or the filter (several rows in one window), rows that end inside a 16-sample block (T % 16 != 0: the
-    two-view tiles) and on one, tensors of one tile and of thousands (several waves, each starting mid-row), a
-    signed filter.  Every row against scipy.signal.lfilter in float64."""
+    two-view tiles) and on one, tensors of one tile and of thousands (several waves, each starting mid-row), rows
+    that begin and end inside a quad (T % 4 != 0), a signed filter.  Every row against scipy.signal.lfilter in float64."""
     from scipy.signal import lfilter
     gen = torch.Generator().manual_seed(seed_of('mfma conv', shape, K))
     x = torch.randn(shape, generator=gen)
@@ -135,12 +139,12 @@ def test_conv_corr_matrix_core_path(slayer, shape, K):
     assert_rel(slayer.utils.filter.corr(xp.to(dev()), fp.to(dev()), 1), O.conv_bwd(xp, fp, 1), f'corr {shape} K={K}')
 
 
-@pytest.mark.parametrize('T,K', [(300, 64), (304, 16), (20, 100), (1500, 33)])
+@pytest.mark.parametrize('T,K', [(300, 64), (304, 16), (20, 100), (1500, 33), (301, 64), (350, 16), (19, 100), (1003, 33)])
 def test_conv_rows_do_not_see_each_other(slayer, T, K):
     """A row's window is cut at the row: an Inf at the end (start) of one row leaves every other row finite and
     unchanged in conv (corr); inside its own row it arrives where the filter carries it."""
     gen = torch.Generator().manual_seed(seed_of('rows', T, K))
-    M = 97
+    M = 97 if T % 4 == 0 else 100          # the matrix kernel wants the tensor as a whole in whole quads
     x = torch.randn(M, T, generator=gen)
     f = torch.randn(K, generator=gen)
     base_c = slayer.utils.filter.conv(x.to(dev()), f.to(dev()), 1).cpu()
