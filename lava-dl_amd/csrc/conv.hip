@@ -123,9 +123,41 @@ __global__ __launch_bounds__(kWave) void conv_kernel(float* __restrict__ out, co
 // input also reaches the up to 16 + KPAD - K neighbouring outputs of its row whose window holds it (0 * Inf);
 // finite inputs, the only ones this path sees, give the same sums.
 typedef float mfma_f4 __attribute__((ext_vector_type(4)));
+typedef __bf16 mfma_bf8 __attribute__((ext_vector_type(8)));
 
 constexpr int kConvTile = 256;             // samples per tile
 constexpr int kConvRing = 4;               // tiles in the LDS ring = tiles per loop pass
+
+// A float as the sum of three bfloat16 numbers, each the rounding to nearest of what the parts before it leave
+// (|second| <= 2^-9, |third| <= 2^-18 of the value, what the three leave out <= 2^-27), four floats at a time:
+// part t of the quad as four bfloat16 in two dwords.
+struct SplitQuad { uint2 part[3]; };
+typedef __bf16 conv_bf2 __attribute__((ext_vector_type(2)));
+typedef float conv_f2 __attribute__((ext_vector_type(2)));
+// two floats rounded to bfloat16 in one dword; a and b become what the rounding left
+__device__ __forceinline__ unsigned round_pair(float& a, float& b) {
+    const conv_bf2 h = __builtin_convertvector(conv_f2{a, b}, conv_bf2);
+    const conv_f2 back = __builtin_convertvector(h, conv_f2);
+    a -= back.x;
+    b -= back.y;
+    return __builtin_bit_cast(unsigned, h);
+}
+__device__ __forceinline__ SplitQuad split_quad(float4 v) {
+    SplitQuad q;
+#pragma unroll
+    for (int t = 0; t < 3; ++t) {
+        q.part[t].x = round_pair(v.x, v.y);
+        q.part[t].y = round_pair(v.z, v.w);
+    }
+    return q;
+}
+// d += A * B over 32 window samples (two quads per lane).  An odd last group is paired with zeros rather than given
+// to the 16-sample instruction: that instruction, fed the accumulator of a 32-sample one, returned half of the
+// accumulator without the products of the instruction before it on this toolchain.
+__device__ __forceinline__ mfma_f4 mfma_pair(uint2 a0, uint2 a1, uint2 b0, uint2 b1, mfma_f4 d) {
+    const uint4 a = make_uint4(a0.x, a0.y, a1.x, a1.y), b = make_uint4(b0.x, b0.y, b1.x, b1.y);
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mfma_bf8, a), __builtin_bit_cast(mfma_bf8, b), d, 0, 0, 0);
+}
 
 template <int KPAD, bool CORR, bool ANYT = false>
 __global__ __launch_bounds__(kWave) void conv_mfma_kernel(float* __restrict__ out, const float* __restrict__ in,
@@ -256,6 +288,197 @@ __global__ __launch_bounds__(kWave) void conv_mfma_kernel(float* __restrict__ ou
     }
 }
 
+// The same kernel for more than 32 taps, where the float instruction (one pass of the matrix pipe per 4 window
+// samples) is what bounds it: every tap and every sample is split into three bfloat16 parts that add up to it
+// to within 2^-27 (each part the rounding to nearest of what the parts before it leave), and the products of the
+// parts are taken with the bfloat16 instruction (one pass per 32 window samples: two window groups at a time) --
+// part i of the taps with part j of the samples for i + j <= 2, six products, each exact, summed in float32.  What
+// is left out (i + j >= 3 and the remainders) is below 2^-25 of a product: less than the rounding of a float sum.
+// The parts are made once per sample on the way into the ring (three planes of four bfloat16 per quad).
+// A part that is zero in every lane of a tile and its neighbour (wave-uniform: spikes, small
+// integers, anything of at most 8 significant bits has no second and third part) is left out together with its
+// products, which then are exactly zero: such inputs cost three products instead of six.
+// Measured against the float form (conv on 3 % spikes / corr on normal random data, us): [524288,300] K = 64
+// 293 / 307 -> 265 / 306, K = 128 464 / 469 -> 310 / 422; [65536,2000] K = 64 245 / 255 -> 221 / 241, K = 128
+// 350 / 361 -> 228 / 316; [8192,1500] K = 64 36 / 30 -> 32 / 31.  Up to 32 taps the float form is as fast or
+// faster (memory-bound; the split costs about 25 vector instructions per quad) and stays.
+template <int KPAD, bool CORR, bool ANYT = false>
+__global__ __launch_bounds__(kWave) void conv_mfma_split_kernel(float* __restrict__ out, const float* __restrict__ in,
+                                                          const float* __restrict__ filt, int K, float ts,
+                                                          int64_t total, int T, int tiles_per_wave) {
+    constexpr int G = KPAD / 16 + 1;        // window groups of 16 samples per block
+    constexpr int kZero = kConvRing * 64;   // ring slot that holds a quad of zeros
+    __shared__ __attribute__((aligned(16))) uint2 ring[3][kConvRing * 64 + 2];
+    const int lane = threadIdx.x;
+    const int n = lane & 15, kq = lane >> 4;
+    // this wave's tiles: samples [first, last) of the flat tensor; its accesses are relative to the row that
+    // holds `first`, through a descriptor that ends with the tensor
+    const int64_t first = (int64_t)blockIdx.x * tiles_per_wave * kConvTile;
+    const int64_t rest = total - first;
+    const int mine = (int)(rest < (int64_t)tiles_per_wave * kConvTile ? rest : (int64_t)tiles_per_wave * kConvTile);
+    const int64_t row0 = first / T;
+    const int lead = (int)(first - row0 * T);                 // samples of row0 in front of `first`
+    // offsets below are relative to `origin`, one tile in front of `first` (the conv window reaches back)
+    const int64_t origin = first - kConvTile;
+    const int64_t avail = total - origin;                     // samples from origin to the end of the tensor
+    const int bound = (int)(avail < (int64_t)(tiles_per_wave + 2) * kConvTile ? avail
+                                                                              : (int64_t)(tiles_per_wave + 2) * kConvTile);
+    const __amdgpu_buffer_rsrc_t src = make_rsrc(in + origin, (unsigned)bound * 4u);
+    const __amdgpu_buffer_rsrc_t dst = make_rsrc(out + origin, (unsigned)bound * 4u);
+    const int floor0 = origin < 0 ? kConvTile : 0;            // nothing in front of the tensor
+    if (lane < 3) ring[lane][kZero] = make_uint2(0u, 0u);
+
+    // Toeplitz operands: lane (output step i = l % 16 of a block, slot kq) of group g holds the taps that link
+    // output step i with window samples 16 g + 4 kq + r, r = 0 .. 3, in three parts
+    SplitQuad a[G];
+    bool a_part[3] = {true, false, false};                    // does any lane hold a non-zero part t of a tap?
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        float tap[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int idx = CORR ? (16 * g + 4 * kq + r) - n : n + KPAD - (16 * g + 4 * kq + r);
+            tap[r] = (idx >= 0 && idx < K) ? filt[idx] : 0.0f;
+        }
+        a[g] = split_quad(make_float4(tap[0], tap[1], tap[2], tap[3]));
+        a_part[1] = a_part[1] || __any((a[g].part[1].x | a[g].part[1].y) != 0u);
+        a_part[2] = a_part[2] || __any((a[g].part[2].x | a[g].part[2].y) != 0u);
+    }
+
+    // Ring slot (in quads) of the operand of group g, relative to the ring position of the tile being computed:
+    // the window of block n starts KPAD samples before the block (conv) or with it (corr), so group g is block
+    // b = n + g - KPAD / 16 (conv) or n + g (corr) of the tile, or of its neighbour when b leaves [0, 16).
+    int opnd[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const int b = n + g - (CORR ? 0 : KPAD / 16);
+        const int tile = b < 0 ? -1 : (b >= 16 ? 1 : 0);
+        opnd[g] = ((tile * 64 + 16 * kq + (b - 16 * tile)) + kConvRing * 64) & (kConvRing * 64 - 1);
+    }
+    const int wslot = 16 * (lane & 3) + (lane >> 2);       // where this lane's loaded quad goes within a tile
+    // sample (relative to `first`) of the first window quad of this lane: group g adds 16 g
+    const int wq = 16 * n + 4 * kq - (CORR ? 0 : KPAD);
+
+    // Step s writes tile w0 + s into the ring (w0 = -1: the conv window reaches back into the previous tile;
+    // corr reaches forward, so its tile s is written one step before tile s - 1 is computed) and computes tile
+    // s - 1.  Loads run kConvRing steps ahead of their ring write, in registers.
+    constexpr int w0 = CORR ? 0 : -1;
+    const int lend = kConvTile + mine + (CORR ? kConvTile : 0);   // relative to origin: last sample a tile may read
+    auto load = [&](int tile) -> float4 {
+        const int t = (tile + 1) * kConvTile + 4 * lane;          // relative to origin
+        return buf_load4<false>(src, (t >= floor0 && t < lend) ? t * 4 : kOutOfRange);
+    };
+    float4 stage[kConvRing];
+    // does the tile at a ring position hold a non-zero second / third part?  (Spikes and other values of at most
+    // eight significant bits do not: their products with those parts are left out.)
+    bool mid_at[kConvRing] = {false, false, false, false}, low_at[kConvRing] = {false, false, false, false};
+    // each load is preceded by a store that falls out of range (dropped by the hardware): the loop is then
+    // entered in the state its back edge leaves, and the wait at its top can leave the youngest loads in
+    // flight instead of draining everything
+#pragma unroll
+    for (int u = 0; u < kConvRing; ++u) {
+        buf_store4<false>(dst, kOutOfRange + 16 * u, make_float4(0.f, 0.f, 0.f, 0.f));
+        stage[u] = load(w0 + u);
+    }
+    const int steps = (mine + kConvTile - 1) / kConvTile + 1;
+    for (int s0 = 0; s0 < steps; s0 += kConvRing) {
+#pragma unroll
+        for (int u = 0; u < kConvRing; ++u) {
+            // ring position of tile w0 + s is (s & 3) = u: s0 is a multiple of the ring length
+            {
+                const SplitQuad q = split_quad(stage[u]);
+                ring[0][u * 64 + wslot] = q.part[0];
+                ring[1][u * 64 + wslot] = q.part[1];
+                ring[2][u * 64 + wslot] = q.part[2];
+                mid_at[u] = __any((q.part[1].x | q.part[1].y) != 0u);
+                low_at[u] = __any((q.part[2].x | q.part[2].y) != 0u);
+            }
+            stage[u] = load(w0 + s0 + u + kConvRing);
+            // tile s - 1 sits at ring position (u - 1 - w0) & 3; its windows reach into the tile before it (conv)
+            // or after it (corr)
+            constexpr int kRingMask = kConvRing - 1;
+            const int at = (u - 1 - w0 + kConvRing) & kRingMask, beside = (at + (CORR ? 1 : kConvRing - 1)) & kRingMask;
+            const int here = at * 64;
+            const bool b_part[3] = {true, mid_at[at] || mid_at[beside], low_at[at] || low_at[beside]};
+            // the first step computes no tile and the last pass may hold steps past the end of the wave's tiles:
+            // they skip the matrix work (a wave-uniform branch without memory instructions inside) and store
+            // out of range
+            const int tile0 = (s0 + u - 1) * kConvTile;               // relative to `first`
+            mfma_f4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (s0 + u >= 1 && tile0 < mine) {
+                // rows of the first and the last output of this lane's block, as sample ranges relative to `first`
+                const int o0 = tile0 + 16 * n + lead;                 // relative to the start of row0
+                const int ra = o0 / T;
+                const int lo_a = ra * T - lead, rb_more = (o0 - ra * T + 15 >= T) ? T : 0;
+                // slot of the window quad of group g as the row [lo, lo + T) sees it, and which of its samples the
+                // row holds (ANYT: a row may begin or end inside the quad), as masks over the two dwords
+                auto slot_of = [&](int g, int lo, uint2& keep) -> int {
+                    const int q = tile0 + wq + 16 * g;                // first sample of the quad
+                    const bool ok = ANYT ? (q + 3 >= lo && q < lo + T) : (q >= lo && q < lo + T);
+                    if (ANYT) {
+                        const unsigned rel = (unsigned)(q - lo);
+                        keep.x = (rel < (unsigned)T ? 0x0000ffffu : 0u) | (rel + 1u < (unsigned)T ? 0xffff0000u : 0u);
+                        keep.y = (rel + 2u < (unsigned)T ? 0x0000ffffu : 0u) | (rel + 3u < (unsigned)T ? 0xffff0000u : 0u);
+                    }
+                    return ok ? ((here + opnd[g]) & (kConvRing * 64 - 1)) : kZero;
+                };
+                // the products of the parts of the taps with the parts of the samples over the window groups [g0, g1)
+                auto multiply = [&](mfma_f4 d, int g0, int g1, int lo) -> mfma_f4 {
+                    int slot[G];
+                    uint2 keep[G];
+#pragma unroll
+                    for (int g = 0; g < G; ++g)
+                        if (g >= g0 && g < g1) slot[g] = slot_of(g, lo, keep[g]);
+                    auto term = [&](mfma_f4 d, int ta, int tb) -> mfma_f4 {
+                        uint2 x[G];
+#pragma unroll
+                        for (int g = 0; g < G; ++g)
+                            if (g >= g0 && g < g1) {
+                                x[g] = ring[tb][slot[g]];
+                                if (ANYT) { x[g].x &= keep[g].x; x[g].y &= keep[g].y; }
+                            }
+#pragma unroll
+                        for (int h = 0; h < (G + 1) / 2; ++h) {            // two groups per instruction
+                            const int g = g0 + 2 * h;
+                            if (g + 1 < g1) d = mfma_pair(a[g].part[ta], a[g + 1].part[ta], x[g], x[g + 1], d);
+                            else if (g < g1) d = mfma_pair(a[g].part[ta], make_uint2(0u, 0u), x[g], make_uint2(0u, 0u), d);
+                        }
+                        return d;
+                    };
+                    // smallest products first; parts that are zero throughout (wave-uniform) are left out.  (Reading
+                    // every part of the samples once and keeping two accumulators is slower at K = 64: 376 -> 395 us
+                    // on 524 288 rows of 300 dense samples.)
+                    if (a_part[2]) d = term(d, 2, 0);
+                    if (a_part[1] && b_part[1]) d = term(d, 1, 1);
+                    if (b_part[2]) d = term(d, 0, 2);
+                    if (a_part[1]) d = term(d, 1, 0);
+                    if (b_part[1]) d = term(d, 0, 1);
+                    return term(d, 0, 0);
+                };
+                // every block sees the row of its first output (conv) or of its last output (corr) ...
+                acc = multiply(acc, 0, G, lo_a + (CORR ? rb_more : 0));
+                // ... and the outputs of a block's other row take their own view.  They are the last outputs
+                // of the previous row (corr) or the first ones of the next row (conv), and inside their row their
+                // window holds samples of this block only: one window group, the block itself.
+                if (__any(rb_more != 0)) {
+                    mfma_f4 other = {0.0f, 0.0f, 0.0f, 0.0f};
+                    constexpr int gb = CORR ? 0 : G - 1;
+                    other = multiply(other, gb, gb + 1, lo_a + (CORR ? 0 : rb_more));
+                    const int oq = tile0 + 16 * n + 4 * kq;           // this lane's output quad
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const bool in_next = oq + (ANYT ? j : 0) >= lo_a + T;
+                        acc[j] = (rb_more != 0 && in_next != CORR) ? other[j] : acc[j];
+                    }
+                }
+            }
+            const int t = tile0 + 16 * n + 4 * kq;
+            buf_store4<false>(dst, (s0 + u >= 1 && t < mine) ? (t + kConvTile) * 4 : kOutOfRange,
+                              make_float4(acc[0] * ts, acc[1] * ts, acc[2] * ts, acc[3] * ts));
+        }
+    }
+}
+
 template <bool CORR, bool ANYT>
 static int conv_mfma_launch(float* out, const float* in, const float* filt, int K, float ts, int64_t M, int64_t T,
                             hipStream_t stream) {
@@ -271,10 +494,15 @@ static int conv_mfma_launch(float* out, const float* in, const float* filt, int 
 #define SLAYER_CONV_MFMA(KP)                                                                                      \
     hipLaunchKernelGGL((conv_mfma_kernel<KP, CORR, ANYT>), dim3((unsigned)blocks), dim3(kWave), 0, stream, out, in, filt, \
                        K, ts, total, (int)T, (int)per_wave)
+#define SLAYER_CONV_MFMA_SPLIT(KP)                                                                                \
+    hipLaunchKernelGGL((conv_mfma_split_kernel<KP, CORR, ANYT>), dim3((unsigned)blocks), dim3(kWave), 0, stream, out, \
+                       in, filt, K, ts, total, (int)T, (int)per_wave)
+    // up to 32 taps the float instructions keep up with memory; beyond that the three-part bfloat16 form is faster
     if (K <= 16) SLAYER_CONV_MFMA(16);
     else if (K <= 32) SLAYER_CONV_MFMA(32);
-    else if (K <= 64) SLAYER_CONV_MFMA(64);
-    else SLAYER_CONV_MFMA(128);
+    else if (K <= 64) SLAYER_CONV_MFMA_SPLIT(64);
+    else SLAYER_CONV_MFMA_SPLIT(128);
+#undef SLAYER_CONV_MFMA_SPLIT
 #undef SLAYER_CONV_MFMA
     return (int)hipGetLastError();
 }

@@ -199,10 +199,15 @@ def test_synapse_stack_full_size(slayer):
     r_gz, _ = O.li_bwd(r_gc, r_cur, d_i)
     r_gx = O.conv_bwd(O.shift(r_gz, -delay, 1), filt, 1)
     assert_scale(xg.grad[sl], r_gx, 'grad through the stack')
-    # adjointness <conv(x), g> == <x, corr(g)> over the whole tensor, in float64
+    # adjointness <conv(x), g> == <x, corr(g)> over the whole tensor, in float64.  Both sides are sums of 12 M terms
+    # of either sign that cancel to about 1e-5 of the sum of their magnitudes; every output carries a float32
+    # rounding error of up to 1e-7 of its value, and the matrix instructions round toward zero on the way (a bias of
+    # about 1e-8 that does not average out), so the bar is 1e-8 of the sum of the magnitudes.  A tap or a step off by
+    # one moves the two sides apart by more than that sum's thousandth.
     lhs = (y.detach().double() * g.double()).sum()
     rhs = (x.double() * slayer.utils.filter.corr(g, filt.to(dev()), 1).double()).sum()
-    assert abs(float(lhs - rhs)) <= 1e-5 * abs(float(lhs))
+    magnitudes = float((y.detach().double().abs() * g.double().abs()).sum())
+    assert abs(float(lhs - rhs)) <= 1e-8 * magnitudes
 
 
 @pytest.mark.parametrize('C,T', [(300000, 1000), (150000, 999)])
