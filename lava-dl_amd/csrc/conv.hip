@@ -482,13 +482,18 @@ __global__ __launch_bounds__(kWave) void conv_mfma_split_kernel(float* __restric
 template <bool CORR, bool ANYT>
 static int conv_mfma_launch(float* out, const float* in, const float* filt, int K, float ts, int64_t M, int64_t T,
                             hipStream_t stream) {
-    // about eight thousand waves (four per SIMD on 256 compute units, twice over), each a whole number of loop
-    // passes of consecutive tiles; every wave reads one tile more than it writes
+    // Tiles per wave (a whole number of loop passes of consecutive tiles; every wave reads one tile more than it
+    // writes): few, so that the waves in flight together walk the tensor as one narrow front -- up to 16 taps, where
+    // a wave's set-up is 8 tap loads, 8 tiles per wave run at 5.7-6.0 TB/s against 4.8 with 64 ([524288,300]
+    // 260 -> 217 us, [65536,2000] 212 -> 182 us) -- but enough to pay for the set-up of the longer filters (20 to
+    // 36 tap loads and their split: 32 tiles, 330 -> 276 us against 8 at K = 64), and no more than leaves about
+    // three thousand waves to a small tensor ([8192,1500], K = 64: 30.1 us with 8 tiles, 27.7 with 12-16, 34.7 with 32).
     const int64_t total = M * T;
     const int64_t tiles = (total + kConvTile - 1) / kConvTile;
-    int64_t per_wave = (tiles / 8192 + kConvRing - 1) / kConvRing * kConvRing;
+    const int64_t cap = K <= 16 ? 8 : 32;
+    int64_t per_wave = (tiles / 3072 + kConvRing - 1) / kConvRing * kConvRing;
     if (per_wave < kConvRing) per_wave = kConvRing;
-    if (per_wave > 64) per_wave = 64;
+    if (per_wave > cap) per_wave = cap;
     const int64_t blocks = (tiles + per_wave - 1) / per_wave;
     if (blocks > 0x7fffffffLL) return SLAYER_ERANGE;
 #define SLAYER_CONV_MFMA(KP)                                                                                      \

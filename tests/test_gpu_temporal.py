@@ -139,6 +139,25 @@ def test_conv_corr_matrix_core_path(slayer, shape, K):
     assert_rel(slayer.utils.filter.corr(xp.to(dev()), fp.to(dev()), 1), O.conv_bwd(xp, fp, 1), f'corr {shape} K={K}')
 
 
+@pytest.mark.parametrize('K', [16, 24, 64, 100])
+@pytest.mark.parametrize('shape', [(8192, 3200), (40000, 302)])
+def test_conv_corr_many_tiles_per_wave(slayer, shape, K):
+    """Tensors of tens of millions of samples, where a wave takes 8 (up to 16 taps) or 32 consecutive tiles: every
+    row against scipy.signal.lfilter in float64."""
+    from scipy.signal import lfilter
+    gen = torch.Generator().manual_seed(seed_of('many tiles', shape, K))
+    M, T = shape
+    x = torch.randn(shape, generator=gen)
+    f = torch.randn(K, generator=gen)
+    rows, fd = x.double().numpy(), f.double().numpy()
+    scale = np.abs(fd).sum() * np.abs(rows).max()
+    y = slayer.utils.filter.conv(x.to(dev()), f.to(dev()), 1).cpu().double().numpy()
+    assert np.abs(y - lfilter(fd, [1.0], rows, axis=-1)).max() <= 1e-5 * scale
+    del y
+    z = slayer.utils.filter.corr(x.to(dev()), f.to(dev()), 1).cpu().double().numpy()
+    assert np.abs(z - lfilter(fd, [1.0], rows[:, ::-1], axis=-1)[:, ::-1]).max() <= 1e-5 * scale
+
+
 @pytest.mark.parametrize('T,K', [(300, 64), (304, 16), (20, 100), (1500, 33), (301, 64), (350, 16), (19, 100), (1003, 33)])
 def test_conv_rows_do_not_see_each_other(slayer, T, K):
     """A row's window is cut at the row: an Inf at the end (start) of one row leaves every other row finite and
