@@ -159,66 +159,85 @@ __device__ __forceinline__ mfma_f4 mfma_pair(uint2 a0, uint2 a1, uint2 b0, uint2
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mfma_bf8, a), __builtin_bit_cast(mfma_bf8, b), d, 0, 0, 0);
 }
 
+// What both matrix kernels share: the tiles of a wave, its addressing and the ring slots of its operands.
+template <int KPAD, bool CORR>
+struct ConvWave {
+    static constexpr int G = KPAD / 16 + 1;        // window groups of 16 samples per block
+    static constexpr int kZero = kConvRing * 64;   // ring slot that holds a quad of zeros
+    // Step s writes tile w0 + s into the ring (w0 = -1: the conv window reaches back into the previous tile;
+    // corr reaches forward, so its tile s is written one step before tile s - 1 is computed) and computes tile
+    // s - 1.  Loads run kConvRing steps ahead of their ring write, in registers.
+    static constexpr int w0 = CORR ? 0 : -1;
+    int lane, n, kq;
+    int mine, lead, floor0, lend, steps, wslot, wq;
+    int opnd[G];
+    __amdgpu_buffer_rsrc_t src, dst;
+
+    __device__ __forceinline__ void init(float* out, const float* in, int64_t total, int T, int tiles_per_wave) {
+        lane = threadIdx.x;
+        n = lane & 15;
+        kq = lane >> 4;
+        // this wave's tiles: samples [first, last) of the flat tensor; its accesses are relative to the row that
+        // holds `first`, through a descriptor that ends with the tensor
+        const int64_t first = (int64_t)blockIdx.x * tiles_per_wave * kConvTile;
+        const int64_t rest = total - first;
+        mine = (int)(rest < (int64_t)tiles_per_wave * kConvTile ? rest : (int64_t)tiles_per_wave * kConvTile);
+        const int64_t row0 = first / T;
+        lead = (int)(first - row0 * T);                 // samples of row0 in front of `first`
+        // offsets below are relative to `origin`, one tile in front of `first` (the conv window reaches back)
+        const int64_t origin = first - kConvTile;
+        const int64_t avail = total - origin;           // samples from origin to the end of the tensor
+        const int bound = (int)(avail < (int64_t)(tiles_per_wave + 2) * kConvTile ? avail
+                                                                                  : (int64_t)(tiles_per_wave + 2) * kConvTile);
+        src = make_rsrc(in + origin, (unsigned)bound * 4u);
+        dst = make_rsrc(out + origin, (unsigned)bound * 4u);
+        floor0 = origin < 0 ? kConvTile : 0;            // nothing in front of the tensor
+        // Ring slot (in quads) of the operand of group g, relative to the ring position of the tile being computed:
+        // the window of block n starts KPAD samples before the block (conv) or with it (corr), so group g is block
+        // b = n + g - KPAD / 16 (conv) or n + g (corr) of the tile, or of its neighbour when b leaves [0, 16).
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const int b = n + g - (CORR ? 0 : KPAD / 16);
+            const int tile = b < 0 ? -1 : (b >= 16 ? 1 : 0);
+            opnd[g] = ((tile * 64 + 16 * kq + (b - 16 * tile)) + kConvRing * 64) & (kConvRing * 64 - 1);
+        }
+        wslot = 16 * (lane & 3) + (lane >> 2);          // where this lane's loaded quad goes within a tile
+        // sample (relative to `first`) of the first window quad of this lane: group g adds 16 g
+        wq = 16 * n + 4 * kq - (CORR ? 0 : KPAD);
+        lend = kConvTile + mine + (CORR ? kConvTile : 0);   // relative to origin: last sample a tile may read
+        steps = (mine + kConvTile - 1) / kConvTile + 1;
+    }
+    // Toeplitz operand: the tap that links output step n of a block with window sample 16 g + 4 kq + r
+    __device__ __forceinline__ float tap(const float* filt, int K, int g, int r) const {
+        const int idx = CORR ? (16 * g + 4 * kq + r) - n : n + KPAD - (16 * g + 4 * kq + r);
+        return (idx >= 0 && idx < K) ? filt[idx] : 0.0f;
+    }
+    // this lane's quad of a tile of the wave (tile -1 / tile count: the neighbours the windows reach into)
+    __device__ __forceinline__ float4 load(int tile) const {
+        const int t = (tile + 1) * kConvTile + 4 * lane;          // relative to origin
+        return buf_load4<false>(src, (t >= floor0 && t < lend) ? t * 4 : kOutOfRange);
+    }
+};
+
 template <int KPAD, bool CORR, bool ANYT = false>
 __global__ __launch_bounds__(kWave) void conv_mfma_kernel(float* __restrict__ out, const float* __restrict__ in,
                                                           const float* __restrict__ filt, int K, float ts,
                                                           int64_t total, int T, int tiles_per_wave) {
-    constexpr int G = KPAD / 16 + 1;        // window groups of 16 samples per block
-    constexpr int kZero = kConvRing * 64;   // ring slot that holds a quad of zeros
+    using W = ConvWave<KPAD, CORR>;
+    constexpr int G = W::G, kZero = W::kZero, w0 = W::w0;
     __shared__ __attribute__((aligned(16))) float4 ring[kConvRing * 64 + 1];
-    const int lane = threadIdx.x;
-    const int n = lane & 15, kq = lane >> 4;
-    // this wave's tiles: samples [first, last) of the flat tensor; its accesses are relative to the row that
-    // holds `first`, through a descriptor that ends with the tensor
-    const int64_t first = (int64_t)blockIdx.x * tiles_per_wave * kConvTile;
-    const int64_t rest = total - first;
-    const int mine = (int)(rest < (int64_t)tiles_per_wave * kConvTile ? rest : (int64_t)tiles_per_wave * kConvTile);
-    const int64_t row0 = first / T;
-    const int lead = (int)(first - row0 * T);                 // samples of row0 in front of `first`
-    // offsets below are relative to `origin`, one tile in front of `first` (the conv window reaches back)
-    const int64_t origin = first - kConvTile;
-    const int64_t avail = total - origin;                     // samples from origin to the end of the tensor
-    const int bound = (int)(avail < (int64_t)(tiles_per_wave + 2) * kConvTile ? avail
-                                                                              : (int64_t)(tiles_per_wave + 2) * kConvTile);
-    const __amdgpu_buffer_rsrc_t src = make_rsrc(in + origin, (unsigned)bound * 4u);
-    const __amdgpu_buffer_rsrc_t dst = make_rsrc(out + origin, (unsigned)bound * 4u);
-    const int floor0 = origin < 0 ? kConvTile : 0;            // nothing in front of the tensor
+    W wv;
+    wv.init(out, in, total, T, tiles_per_wave);
+    const int lane = wv.lane, n = wv.n, kq = wv.kq, mine = wv.mine, lead = wv.lead, wslot = wv.wslot, wq = wv.wq;
+    const int* opnd = wv.opnd;
+    const __amdgpu_buffer_rsrc_t dst = wv.dst;
     if (lane == 0) ring[kZero] = make_float4(0.f, 0.f, 0.f, 0.f);
-
-    // Toeplitz operands: lane (output step i = l % 16 of a block, slot kq) of instruction (g, r) holds the tap
-    // that links output step i with window sample 16 g + 4 kq + r
     float a[G][4];
 #pragma unroll
     for (int g = 0; g < G; ++g)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int idx = CORR ? (16 * g + 4 * kq + r) - n : n + KPAD - (16 * g + 4 * kq + r);
-            a[g][r] = (idx >= 0 && idx < K) ? filt[idx] : 0.0f;
-        }
-
-    // Ring slot (in quads) of the operand of group g, relative to the ring position of the tile being computed:
-    // the window of block n starts KPAD samples before the block (conv) or with it (corr), so group g is block
-    // b = n + g - KPAD / 16 (conv) or n + g (corr) of the tile, or of its neighbour when b leaves [0, 16).
-    int opnd[G];
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-        const int b = n + g - (CORR ? 0 : KPAD / 16);
-        const int tile = b < 0 ? -1 : (b >= 16 ? 1 : 0);
-        opnd[g] = ((tile * 64 + 16 * kq + (b - 16 * tile)) + kConvRing * 64) & (kConvRing * 64 - 1);
-    }
-    const int wslot = 16 * (lane & 3) + (lane >> 2);       // where this lane's loaded quad goes within a tile
-    // sample (relative to `first`) of the first window quad of this lane: group g adds 16 g
-    const int wq = 16 * n + 4 * kq - (CORR ? 0 : KPAD);
-
-    // Step s writes tile w0 + s into the ring (w0 = -1: the conv window reaches back into the previous tile;
-    // corr reaches forward, so its tile s is written one step before tile s - 1 is computed) and computes tile
-    // s - 1.  Loads run kConvRing steps ahead of their ring write, in registers.
-    constexpr int w0 = CORR ? 0 : -1;
-    const int lend = kConvTile + mine + (CORR ? kConvTile : 0);   // relative to origin: last sample a tile may read
-    auto load = [&](int tile) -> float4 {
-        const int t = (tile + 1) * kConvTile + 4 * lane;          // relative to origin
-        return buf_load4<false>(src, (t >= floor0 && t < lend) ? t * 4 : kOutOfRange);
-    };
+        for (int r = 0; r < 4; ++r) a[g][r] = wv.tap(filt, K, g, r);
+    auto load = [&](int tile) -> float4 { return wv.load(tile); };
     float4 stage[kConvRing];
     // each load is preceded by a store that falls out of range (dropped by the hardware): the loop is then
     // entered in the state its back edge leaves, and the wait at its top can leave the youngest loads in
@@ -228,7 +247,7 @@ __global__ __launch_bounds__(kWave) void conv_mfma_kernel(float* __restrict__ ou
         buf_store4<false>(dst, kOutOfRange + 16 * u, make_float4(0.f, 0.f, 0.f, 0.f));
         stage[u] = load(w0 + u);
     }
-    const int steps = (mine + kConvTile - 1) / kConvTile + 1;
+    const int steps = wv.steps;
     for (int s0 = 0; s0 < steps; s0 += kConvRing) {
 #pragma unroll
         for (int u = 0; u < kConvRing; ++u) {
@@ -306,68 +325,25 @@ template <int KPAD, bool CORR, bool ANYT = false>
 __global__ __launch_bounds__(kWave) void conv_mfma_split_kernel(float* __restrict__ out, const float* __restrict__ in,
                                                           const float* __restrict__ filt, int K, float ts,
                                                           int64_t total, int T, int tiles_per_wave) {
-    constexpr int G = KPAD / 16 + 1;        // window groups of 16 samples per block
-    constexpr int kZero = kConvRing * 64;   // ring slot that holds a quad of zeros
+    using W = ConvWave<KPAD, CORR>;
+    constexpr int G = W::G, kZero = W::kZero, w0 = W::w0;
     __shared__ __attribute__((aligned(16))) uint2 ring[3][kConvRing * 64 + 2];
-    const int lane = threadIdx.x;
-    const int n = lane & 15, kq = lane >> 4;
-    // this wave's tiles: samples [first, last) of the flat tensor; its accesses are relative to the row that
-    // holds `first`, through a descriptor that ends with the tensor
-    const int64_t first = (int64_t)blockIdx.x * tiles_per_wave * kConvTile;
-    const int64_t rest = total - first;
-    const int mine = (int)(rest < (int64_t)tiles_per_wave * kConvTile ? rest : (int64_t)tiles_per_wave * kConvTile);
-    const int64_t row0 = first / T;
-    const int lead = (int)(first - row0 * T);                 // samples of row0 in front of `first`
-    // offsets below are relative to `origin`, one tile in front of `first` (the conv window reaches back)
-    const int64_t origin = first - kConvTile;
-    const int64_t avail = total - origin;                     // samples from origin to the end of the tensor
-    const int bound = (int)(avail < (int64_t)(tiles_per_wave + 2) * kConvTile ? avail
-                                                                              : (int64_t)(tiles_per_wave + 2) * kConvTile);
-    const __amdgpu_buffer_rsrc_t src = make_rsrc(in + origin, (unsigned)bound * 4u);
-    const __amdgpu_buffer_rsrc_t dst = make_rsrc(out + origin, (unsigned)bound * 4u);
-    const int floor0 = origin < 0 ? kConvTile : 0;            // nothing in front of the tensor
+    W wv;
+    wv.init(out, in, total, T, tiles_per_wave);
+    const int lane = wv.lane, n = wv.n, kq = wv.kq, mine = wv.mine, lead = wv.lead, wslot = wv.wslot, wq = wv.wq;
+    const int* opnd = wv.opnd;
+    const __amdgpu_buffer_rsrc_t dst = wv.dst;
     if (lane < 3) ring[lane][kZero] = make_uint2(0u, 0u);
-
-    // Toeplitz operands: lane (output step i = l % 16 of a block, slot kq) of group g holds the taps that link
-    // output step i with window samples 16 g + 4 kq + r, r = 0 .. 3, in three parts
+    // the taps in three parts, and whether any lane holds a non-zero second / third part of a tap
     SplitQuad a[G];
-    bool a_part[3] = {true, false, false};                    // does any lane hold a non-zero part t of a tap?
+    bool a_part[3] = {true, false, false};
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-        float tap[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int idx = CORR ? (16 * g + 4 * kq + r) - n : n + KPAD - (16 * g + 4 * kq + r);
-            tap[r] = (idx >= 0 && idx < K) ? filt[idx] : 0.0f;
-        }
-        a[g] = split_quad(make_float4(tap[0], tap[1], tap[2], tap[3]));
+        a[g] = split_quad(make_float4(wv.tap(filt, K, g, 0), wv.tap(filt, K, g, 1), wv.tap(filt, K, g, 2), wv.tap(filt, K, g, 3)));
         a_part[1] = a_part[1] || __any((a[g].part[1].x | a[g].part[1].y) != 0u);
         a_part[2] = a_part[2] || __any((a[g].part[2].x | a[g].part[2].y) != 0u);
     }
-
-    // Ring slot (in quads) of the operand of group g, relative to the ring position of the tile being computed:
-    // the window of block n starts KPAD samples before the block (conv) or with it (corr), so group g is block
-    // b = n + g - KPAD / 16 (conv) or n + g (corr) of the tile, or of its neighbour when b leaves [0, 16).
-    int opnd[G];
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-        const int b = n + g - (CORR ? 0 : KPAD / 16);
-        const int tile = b < 0 ? -1 : (b >= 16 ? 1 : 0);
-        opnd[g] = ((tile * 64 + 16 * kq + (b - 16 * tile)) + kConvRing * 64) & (kConvRing * 64 - 1);
-    }
-    const int wslot = 16 * (lane & 3) + (lane >> 2);       // where this lane's loaded quad goes within a tile
-    // sample (relative to `first`) of the first window quad of this lane: group g adds 16 g
-    const int wq = 16 * n + 4 * kq - (CORR ? 0 : KPAD);
-
-    // Step s writes tile w0 + s into the ring (w0 = -1: the conv window reaches back into the previous tile;
-    // corr reaches forward, so its tile s is written one step before tile s - 1 is computed) and computes tile
-    // s - 1.  Loads run kConvRing steps ahead of their ring write, in registers.
-    constexpr int w0 = CORR ? 0 : -1;
-    const int lend = kConvTile + mine + (CORR ? kConvTile : 0);   // relative to origin: last sample a tile may read
-    auto load = [&](int tile) -> float4 {
-        const int t = (tile + 1) * kConvTile + 4 * lane;          // relative to origin
-        return buf_load4<false>(src, (t >= floor0 && t < lend) ? t * 4 : kOutOfRange);
-    };
+    auto load = [&](int tile) -> float4 { return wv.load(tile); };
     float4 stage[kConvRing];
     // does the tile at a ring position hold a non-zero second / third part?  (Spikes and other values of at most
     // eight significant bits do not: their products with those parts are left out.)
@@ -380,7 +356,7 @@ __global__ __launch_bounds__(kWave) void conv_mfma_split_kernel(float* __restric
         buf_store4<false>(dst, kOutOfRange + 16 * u, make_float4(0.f, 0.f, 0.f, 0.f));
         stage[u] = load(w0 + u);
     }
-    const int steps = (mine + kConvTile - 1) / kConvTile + 1;
+    const int steps = wv.steps;
     for (int s0 = 0; s0 < steps; s0 += kConvRing) {
 #pragma unroll
         for (int u = 0; u < kConvRing; ++u) {
