@@ -317,6 +317,9 @@ __global__ __launch_bounds__(kWave) void conv_mfma_kernel(float* __restrict__ ou
 // A part that is zero in every lane of a tile and its neighbour (wave-uniform: spikes, small
 // integers, anything of at most 8 significant bits has no second and third part) is left out together with its
 // products, which then are exactly zero: such inputs cost three products instead of six.
+// Range: a value beyond the largest bfloat16 (3.3895e38) overflows its first part (NaN); parts below the smallest
+// normal float32 are lost, so a tap or sample below about 3e-33 in magnitude enters with an absolute error of up to
+// 1.2e-38 (3.38e38 * 1e-38 gives 3.3834).
 // Measured against the float form (conv on 3 % spikes / corr on normal random data, us): [524288,300] K = 64
 // 293 / 307 -> 265 / 306, K = 128 464 / 469 -> 310 / 422; [65536,2000] K = 64 245 / 255 -> 221 / 241, K = 128
 // 350 / 361 -> 228 / 316; [8192,1500] K = 64 36 / 30 -> 32 / 31.  Up to 32 taps the float form is as fast or
