@@ -139,6 +139,23 @@ def test_conv_corr_matrix_core_path(slayer, shape, K):
     assert_rel(slayer.utils.filter.corr(xp.to(dev()), fp.to(dev()), 1), O.conv_bwd(xp, fp, 1), f'corr {shape} K={K}')
 
 
+@pytest.mark.parametrize('K', [16, 64, 128])
+@pytest.mark.parametrize('x_scale,f_scale', [(1e-25, 1.0), (1e25, 1e-3), (1.0, 1e-30), (1e-12, 1e-12)])
+def test_conv_corr_small_and_large_magnitudes(slayer, K, x_scale, f_scale):
+    """The bar holds relative to the data's own scale from 1e-30 to 1e25 (beyond 32 taps the operands are split into
+    bfloat16 parts, which keeps full precision while the parts stay normal float32 numbers: down to about 3e-33)."""
+    from scipy.signal import lfilter
+    gen = torch.Generator().manual_seed(seed_of('magnitudes', K, x_scale, f_scale))
+    x = torch.randn(64, 300, generator=gen) * x_scale
+    f = torch.randn(K, generator=gen) * f_scale
+    rows, fd = x.double().numpy(), f.double().numpy()
+    scale = np.abs(fd).sum() * np.abs(rows).max()
+    y = slayer.utils.filter.conv(x.to(dev()), f.to(dev()), 1).cpu().double().numpy()
+    z = slayer.utils.filter.corr(x.to(dev()), f.to(dev()), 1).cpu().double().numpy()
+    assert np.abs(y - lfilter(fd, [1.0], rows, axis=-1)).max() <= 1e-5 * scale
+    assert np.abs(z - lfilter(fd, [1.0], rows[:, ::-1], axis=-1)[:, ::-1]).max() <= 1e-5 * scale
+
+
 @pytest.mark.parametrize('K', [16, 24, 64, 100])
 @pytest.mark.parametrize('shape', [(8192, 3200), (40000, 302)])
 def test_conv_corr_many_tiles_per_wave(slayer, shape, K):
