@@ -242,7 +242,10 @@ int slayer_delay_bwd(float *grad_in, float *grad_sum, const float *grad_out, con
 
 /* ---- temporal filter ---------------------------------------------------------------------- */
 
-/* Replaces conv fwd (utils/filter/conv.cu:80-125): out[m][t] = Ts * sum_{i<K, t-i>=0} filt[i] * in[m][t-i]. */
+/* Replaces conv fwd (utils/filter/conv.cu:80-125): out[m][t] = Ts * sum_{i<K, t-i>=0} filt[i] * in[m][t-i].
+ * K <= 4096 (SLAYER_ERANGE beyond).  float32 throughout; for 32 < K <= 128 the products are formed on the matrix
+ * cores from three bfloat16 parts per operand (each operand to within 2^-27, sums in float32): as close to the
+ * exact sum as float32 multiply-adds, for operands between about 3e-33 and 3.39e38 in magnitude. */
 int slayer_conv(float *out, const float *in, const float *filt, int64_t K, float sampling_time,
                 int64_t M, int64_t T, void *stream);
 
