@@ -1160,7 +1160,7 @@ bool stream_fits_multiwave(const typename Op::Params& prm, int64_t M, int64_t T)
 // Rows a multiple of 2 KB apart (or within 64 bytes of one: T = 512, 1024, 2048, also 500) put the same columns
 // of every row on few memory channels, and a wave-wide access that touches eight rows (128-byte pieces) is served
 // by them one after the other: a plain copy in that pattern drops from 5.0 to 3.6 TB/s at T = 1024
-// (microbench/row_tile_copy.hip).  512-byte pieces of two rows per access (16 rows per wave) do not suffer;
+// (measured with a stand-alone copy program).  512-byte pieces of two rows per access (16 rows per wave) do not suffer;
 // Ops whose recurrence is light enough to run on 16 lanes per wave ask for them (kLongPiecesOnAliasedRows:
 // LI forward 311 -> 265 us, fused CUBA forward 616 -> 542 us at [2400,64,1024]; the adaptive-threshold and
 // resonator recurrences lose more on the idle lanes than they gain).
