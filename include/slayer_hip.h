@@ -25,7 +25,10 @@
  *   - States: num_states == 1 broadcasts one value, otherwise num_states == M.
  *   - Integer states are held in 32 bits with 64-bit products (as the reference
  *     kernels do, leaky_integrator.cu:43,61); results equal the int64 CPU branch
- *     while every state stays inside +-(2^31 - 1).
+ *     (leaky_integrator.py:210-231) while no intermediate leaves 32 bits.  That is
+ *     not left to chance: every forward kernel watches the states it stores and
+ *     raises a process-wide flag (slayer_range_status) when one comes within a
+ *     factor of two of the limit -- before anything can have overflowed.
  */
 #ifndef SLAYER_HIP_H
 #define SLAYER_HIP_H
@@ -37,12 +40,13 @@
 extern "C" {
 #endif
 
-#define SLAYER_ABI_VERSION 3
+#define SLAYER_ABI_VERSION 4
 
 #define SLAYER_EINVAL   (-1)   /* inconsistent sizes (M, T, neurons_per_batch, num_params, ...) */
 #define SLAYER_ENULL    (-2)   /* a required pointer is NULL */
 #define SLAYER_ERANGE   (-3)   /* a size exceeds what the kernels index (M*T >= 2^40, T >= 2^31, K > 4096 ...) */
 #define SLAYER_ESCRATCH (-4)   /* a size exceeds the library's built-in scratch buffer (slayer_li_bwd_static) */
+#define SLAYER_ENOFLAG  (-5)   /* the range flag could not be set up (slayer_range_status) */
 
 int slayer_abi_version(void);
 
@@ -72,6 +76,40 @@ typedef struct slayer_delays {
 
 /* Text for a return code of this library (hipGetErrorString for positive codes). */
 const char *slayer_error_string(int code);
+
+/* ---- range of the 32-bit states -------------------------------------------------------- */
+
+/* The reference's CPU branch holds its fixed-point states in int64 (leaky_integrator.py:213, resonator.py:340), its
+ * CUDA kernels and this library in int32 (leaky_integrator.cu:61 notes the overflow).  Here an overflow cannot pass
+ * unnoticed: every forward entry point (slayer_li_fwd, slayer_ath_fwd, slayer_apth_fwd, slayer_res_fwd,
+ * slayer_adres_fwd, slayer_cuba_fwd, slayer_alif_fwd, slayer_rf_fwd, slayer_*_recurrent_fwd) raises a sticky,
+ * process-wide flag when
+ *   - a state it stores (or is handed as initial state) reaches 2^30 in magnitude (2^29 for the real / imaginary
+ *     states of the resonator family, whose step adds two products; 2^28 for threshold and refractory states, whose
+ *     spike adds the step and twice the threshold), in units of 1 / w_scale, or
+ *   - a decay multiplier (4096 - decay; sin / cos decay) exceeds 8191 in magnitude, or
+ *   - a scaled threshold step, base threshold or reset value is itself beyond the bound of the state it enters.
+ * While the flag is clear, no sum or product of a launch that has completed left 32 bits, and its results are those
+ * of the 64-bit evaluation, bit for bit.  Once it is raised, the results of the launches since it was last clear are
+ * suspect (sums saturate at the int32 limits instead of wrapping); the *_naive entry points evaluate in 64 bits.
+ * The flag is one word of pinned host memory that the kernels write and the host reads in place: reading it costs
+ * no device call and no synchronisation, and tells about every launch that has completed.
+ *
+ * slayer_range_status: *raised (may be NULL) receives 1 when the flag is up, else 0; clear != 0 lowers it.
+ * Returns 0, or SLAYER_ENOFLAG when the word could not be set up (then no kernel reports anything).  The word is set
+ * up by the first call of this function or of any forward entry point, with one hipHostMalloc of 64 bytes: make
+ * that first call outside a stream capture.  Neither function has a counterpart in the reference. */
+int slayer_range_status(int *raised, int clear);
+
+/* Host address of the flag word (non-zero = raised), for polling without a call; NULL when it could not be set up. */
+const volatile unsigned *slayer_range_word(void);
+
+/* 1 when the float backward entry points (slayer_li_bwd, slayer_res_bwd, slayer_cuba_bwd, slayer_alif_bwd,
+ * slayer_rf_bwd) evaluate a tensor of this shape as wave scans (grad_in then equals a step-by-step evaluation to
+ * a few ulp of the largest terms), 0 when they walk it step by step (grad_in bit-identical to it); 16-byte
+ * aligned tensors assumed.  For callers that compare the two, like the reference's debug cross-check
+ * (leaky_integrator.py:168-205). */
+int slayer_bwd_takes_scan(int64_t M, int64_t neurons_per_batch, int64_t T);
 
 /* ---- leaky integrator ---------------------------------------------------------------- */
 
@@ -104,7 +142,11 @@ int slayer_li_bwd(float *grad_in, float *grad_decay, const float *grad_out, cons
  * library (5 MiB of device memory per GPU, held until the process ends); the call allocates and frees
  * nothing.  Limits: M <= SLAYER_LI_BWD_STATIC_MAX_ROWS and num_decays <= SLAYER_LI_BWD_STATIC_MAX_DECAYS,
  * else SLAYER_ESCRATCH is returned and nothing is launched.  All calls on one GPU share the one buffer:
- * calls that overlap on the same GPU (different streams, or threads) race; serialise them. */
+ * calls that overlap on the same GPU (different streams, or threads) race; serialise them.
+ * The first call on a device looks the buffer's address up (hipGetSymbolAddress, which may load the code object):
+ * make that call outside a stream capture, as a warm-up; later calls on that device only launch.
+ * With grad_decay == NULL nothing is summed and the scratch is not touched (slayer_li_bwd given a workspace
+ * without grad_decay would leave the per-neuron sums there; this entry point has no place to hand them out). */
 #define SLAYER_LI_BWD_STATIC_MAX_ROWS   (1 << 20)
 #define SLAYER_LI_BWD_STATIC_MAX_DECAYS 4096
 int slayer_li_bwd_static(float *grad_in, float *grad_decay, const float *grad_out, const float *out,
@@ -245,7 +287,8 @@ int slayer_delay_bwd(float *grad_in, float *grad_sum, const float *grad_out, con
 /* Replaces conv fwd (utils/filter/conv.cu:80-125): out[m][t] = Ts * sum_{i<K, t-i>=0} filt[i] * in[m][t-i].
  * K <= 4096 (SLAYER_ERANGE beyond).  float32 throughout; for 32 < K <= 128 the products are formed on the matrix
  * cores from three bfloat16 parts per operand (each operand to within 2^-27, sums in float32): as close to the
- * exact sum as float32 multiply-adds, for operands between about 3e-33 and 3.39e38 in magnitude. */
+ * exact sum as float32 multiply-adds, for every finite operand of at least about 3e-33 in magnitude (smaller
+ * ones enter with an absolute error of up to 1.2e-38). */
 int slayer_conv(float *out, const float *in, const float *filt, int64_t K, float sampling_time,
                 int64_t M, int64_t T, void *stream);
 

@@ -46,7 +46,10 @@ struct AlifFwd {
         float w, inv_w, spike_scale;
         int64_t npb, n_id, n_vd, n_td, n_rd, n_is, n_vs, n_ts, n_rs;
         Shifts shifts;
+        unsigned* range_flag;
     };
+    static constexpr bool kRangeChecked = true;
+    static constexpr int range_log2(int o) { return o >= kTheta ? 28 : 30; }   // threshold / refractory : current, voltage
     int yc, yv, th, r, th_out, r_out, mi, mv, mt, mr, th_step, base;
     float w, inv_w, spike_scale;
 
@@ -62,6 +65,10 @@ struct AlifFwd {
             mv = 4096 - trunc_i32(rintf(p.v_decay[param_index(m, p.npb, p.n_vd)]));
             mt = 4096 - trunc_i32(rintf(p.th_decay[param_index(m, p.npb, p.n_td)]));
             mr = 4096 - trunc_i32(rintf(p.ref_decay[param_index(m, p.npb, p.n_rd)]));
+            check_multiplier(mi, p.range_flag); check_multiplier(mv, p.range_flag);
+            check_multiplier(mt, p.range_flag); check_multiplier(mr, p.range_flag);
+            check_state(yc, 30, p.range_flag); check_state(yv, 30, p.range_flag);
+            check_state(th, 28, p.range_flag); check_state(r, 28, p.range_flag);
         }
     }
     // what the next operator reads of a state: trunc(w * (float(y) / w)); for a power of two the scaling
@@ -72,8 +79,8 @@ struct AlifFwd {
     }
     __device__ __forceinline__ void pre(float4 (&x)[1]) const { x[0] = to_state(x[0], w); }
     __device__ __forceinline__ void step(const float (&x)[1], float (&o)[kOut]) {
-        yc = rs0_12(yc, mi) + __float_as_int(x[0]);
-        yv = rs0_12(yv, mv) + reread(yc);                       // the voltage op reads the float32 current
+        yc = add_sat(rs0_12(yc, mi), __float_as_int(x[0]));
+        yv = add_sat(rs0_12(yv, mv), reread(yc));               // the voltage op reads the float32 current
         r = rs0_12(r, mr);
         th = rs0_12(th - base, mt) + base;
         th_out = th; r_out = r;
@@ -102,12 +109,14 @@ struct AlifFwd {
                 yv = trunc_i32(p.v_state[p.n_vs == 1 ? 0 : m] * w);
                 mi = 4096 - trunc_i32(rintf(p.i_decay[param_index(m, p.npb, p.n_id)]));
                 mv = 4096 - trunc_i32(rintf(p.v_decay[param_index(m, p.npb, p.n_vd)]));
+                check_multiplier(mi, p.range_flag); check_multiplier(mv, p.range_flag);
+                check_state(yc, 30, p.range_flag); check_state(yv, 30, p.range_flag);
             }
         }
         __device__ __forceinline__ void step(const float (&x)[1], float (&o)[kOut]) {
-            yc = rs0_12(yc, mi) + __float_as_int(x[0]);
+            yc = add_sat(rs0_12(yc, mi), __float_as_int(x[0]));
             const float cf = (float)yc;
-            yv = rs0_12(yv, mv) + (POW2 ? trunc_i32(cf) : trunc_i32(w * (cf / w)));
+            yv = add_sat(rs0_12(yv, mv), POW2 ? trunc_i32(cf) : trunc_i32(w * (cf / w)));
             if (KEEP_CURRENT) o[0] = __int_as_float(yc);
             o[kVol] = __int_as_float(yv);
         }
@@ -132,6 +141,8 @@ struct AlifFwd {
                 yv_last = trunc_i32(p.v_state[p.n_vs == 1 ? 0 : m] * w);
                 mt = 4096 - trunc_i32(rintf(p.th_decay[param_index(m, p.npb, p.n_td)]));
                 mr = 4096 - trunc_i32(rintf(p.ref_decay[param_index(m, p.npb, p.n_rd)]));
+                check_multiplier(mt, p.range_flag); check_multiplier(mr, p.range_flag);
+                check_state(th, 28, p.range_flag); check_state(r, 28, p.range_flag);
             }
         }
         __device__ __forceinline__ void step(const float (&x)[1], float (&o)[2]) {
@@ -277,8 +288,9 @@ extern "C" int slayer_alif_fwd(float* cur_out, float* vol_out, float* theta_out,
 #define SLAYER_ALIF_ARGS cur_last_out, vol_last_out, th_last_out, ref_last_out, i_decay, v_decay, th_decay, ref_decay, i_state,       \
                          v_state, th_state, ref_state, (int)th_step_scaled, (int)th0_scaled, w, 1.0f / w,         \
                          spike_scale, neurons_per_batch, num_i_decays, num_v_decays, num_th_decays,               \
-                         num_ref_decays, num_i_states, num_v_states, num_th_states, num_ref_states, sh
+                         num_ref_decays, num_i_states, num_v_states, num_th_states, num_ref_states, sh, flag
     const Shifts sh = forward_shifts(delays, neurons_per_batch);
+    unsigned* flag = range_flag_for_threshold(th_step_scaled, th0_scaled);
 #define SLAYER_ALIF_S(P, G, S)                                                                                    \
     do {                                                                                                          \
         if (cur_out) {                                                                                            \

@@ -27,6 +27,21 @@ inline int check_states(int64_t M, int64_t n) { return (n == 1 || n == M) ? 0 : 
 
 inline bool is_pow2(int w) { return w > 0 && (w & (w - 1)) == 0; }
 
+// The process-wide range flag of the 32-bit fixed-point states (api.hip): one word of pinned host memory that the
+// kernels can write.  range_flag_device() is the address a kernel stores to (nullptr when the word could not be
+// set up: the kernels then skip the report); range_flag_raise_from_host() sets it from an entry point, for scaled
+// arguments that are already beyond what a state may hold.
+unsigned* range_flag_device();
+void range_flag_raise_from_host();
+// threshold step and base of the adaptive-threshold family: both enter the states, whose bound is 2^28
+inline unsigned* range_flag_for_threshold(int64_t step_scaled, int64_t base_scaled) {
+    unsigned* flag = range_flag_device();
+    const int64_t lim = (int64_t)1 << 28;
+    if (step_scaled >= lim || step_scaled <= -lim || base_scaled >= lim || base_scaled <= -lim)
+        range_flag_raise_from_host();
+    return flag;
+}
+
 // Delays folded into a fused block: per-neuron tables need a batch to map onto and a sampling time to
 // divide by; the scalar parts must fit the 32-bit step counts of the kernels (a shift of T steps already
 // empties a row, so anything beyond +-2^30 is equivalent to it).

@@ -142,10 +142,31 @@ __device__ __forceinline__ unsigned round_pair(float& a, float& b) {
     b -= back.y;
     return __builtin_bit_cast(unsigned, h);
 }
+// A finite float beyond the largest bfloat16 (3.3895e38 .. 3.4028e38) rounds to an infinite first part, and what
+// that leaves is an infinity of the other sign -- which nothing else produces (an infinite or NaN value leaves a
+// NaN), so it marks exactly this case.  Such a value then takes the largest bfloat16 as its first part instead; the
+// parts after it hold the rest as usual.  Rare: a wave-uniform branch that no ordinary tensor enters.
+__device__ __forceinline__ bool is_inf(float x) { return __builtin_isinf(x); }
+__device__ __forceinline__ void clamp_first_part(float orig, float& rest, unsigned& pair, int half) {
+    if (is_inf(rest)) {
+        const unsigned top = (__float_as_uint(orig) >> 16 & 0x8000u) | 0x7f7fu;      // +-3.3895e38 as bfloat16
+        pair = half ? (pair & 0x0000ffffu) | (top << 16) : (pair & 0xffff0000u) | top;
+        rest = orig - __uint_as_float(top << 16);
+    }
+}
 __device__ __forceinline__ SplitQuad split_quad(float4 v) {
     SplitQuad q;
+    const float4 orig = v;
+    q.part[0].x = round_pair(v.x, v.y);
+    q.part[0].y = round_pair(v.z, v.w);
+    if (__any(is_inf(v.x) || is_inf(v.y) || is_inf(v.z) || is_inf(v.w))) {
+        clamp_first_part(orig.x, v.x, q.part[0].x, 0);
+        clamp_first_part(orig.y, v.y, q.part[0].x, 1);
+        clamp_first_part(orig.z, v.z, q.part[0].y, 0);
+        clamp_first_part(orig.w, v.w, q.part[0].y, 1);
+    }
 #pragma unroll
-    for (int t = 0; t < 3; ++t) {
+    for (int t = 1; t < 3; ++t) {
         q.part[t].x = round_pair(v.x, v.y);
         q.part[t].y = round_pair(v.z, v.w);
     }
@@ -317,9 +338,9 @@ __global__ __launch_bounds__(kWave) void conv_mfma_kernel(float* __restrict__ ou
 // A part that is zero in every lane of a tile and its neighbour (wave-uniform: spikes, small
 // integers, anything of at most 8 significant bits has no second and third part) is left out together with its
 // products, which then are exactly zero: such inputs cost three products instead of six.
-// Range: a value beyond the largest bfloat16 (3.3895e38) overflows its first part (NaN); parts below the smallest
-// normal float32 are lost, so a tap or sample below about 3e-33 in magnitude enters with an absolute error of up to
-// 1.2e-38 (3.38e38 * 1e-38 gives 3.3834).
+// Range: a finite value beyond the largest bfloat16 (3.3895e38) takes that as its first part (split_quad), so
+// every finite float32 is covered; parts below the smallest normal float32 are lost, so a tap or sample below about
+// 3e-33 in magnitude enters with an absolute error of up to 1.2e-38 (3.38e38 * 1e-38 gives 3.3834).
 // Measured against the float form (conv on 3 % spikes / corr on normal random data, us): [524288,300] K = 64
 // 293 / 307 -> 265 / 306, K = 128 464 / 469 -> 310 / 422; [65536,2000] K = 64 245 / 255 -> 221 / 241, K = 128
 // 350 / 361 -> 228 / 316; [8192,1500] K = 64 36 / 30 -> 32 / 31.  Up to 32 taps the float form is as fast or

@@ -41,7 +41,10 @@ struct CubaFwd {
         int fire_above;                              // voltage reset when the state exceeds this
         int64_t npb, n_id, n_vd, n_is, n_vs;
         Shifts shifts;
+        unsigned* range_flag;
     };
+    static constexpr bool kRangeChecked = true;
+    static constexpr int range_log2(int) { return 30; }
     static constexpr bool kTransforms = true;        // integer tiles, see to_state / from_state
     static constexpr int kCopyWaves = SHIFT ? 8 : 2;     // the shifted copies cost the copy waves more instructions
     int yc, yv, yv_out, mi, mv, fire_above;
@@ -56,6 +59,8 @@ struct CubaFwd {
             yv = trunc_i32(p.v_state[p.n_vs == 1 ? 0 : m] * w);
             mi = 4096 - trunc_i32(rintf(p.i_decay[param_index(m, p.npb, p.n_id)]));
             mv = 4096 - trunc_i32(rintf(p.v_decay[param_index(m, p.npb, p.n_vd)]));
+            check_multiplier(mi, p.range_flag); check_multiplier(mv, p.range_flag);
+            check_state(yc, 30, p.range_flag); check_state(yv, 30, p.range_flag);
         }
     }
     __device__ __forceinline__ void pre(float4 (&x)[1]) const { x[0] = to_state(x[0], w); }
@@ -64,11 +69,11 @@ struct CubaFwd {
         for (int i = 0; i < kOut; ++i) o[i] = from_state<POW2>(o[i], w, inv_w);
     }
     __device__ __forceinline__ void step(const float (&x)[1], float (&o)[kOut]) {
-        yc = rs0_12(yc, mi) + __float_as_int(x[0]);
+        yc = add_sat(rs0_12(yc, mi), __float_as_int(x[0]));
         // the voltage op reads the float32 current: trunc(w * (float(yc) / w)); for a power of two
         // the scaling is exact and only the int -> float32 rounding remains
         const float cf = (float)yc;
-        const int yn = rs0_12(yv, mv) + (POW2 ? trunc_i32(cf) : trunc_i32(w * (cf / w)));
+        const int yn = add_sat(rs0_12(yv, mv), POW2 ? trunc_i32(cf) : trunc_i32(w * (cf / w)));
         yv = (yn > fire_above) ? 0 : yn;             // float(yn) >= threshold, decided on the integer
         yv_out = yn;
         if (KEEP_CURRENT) o[0] = __int_as_float(yc);
@@ -92,10 +97,11 @@ struct CubaFwd {
             if (valid) {
                 yc = trunc_i32(p.i_state[p.n_is == 1 ? 0 : m] * w);
                 mi = 4096 - trunc_i32(rintf(p.i_decay[param_index(m, p.npb, p.n_id)]));
+                check_multiplier(mi, p.range_flag); check_state(yc, 30, p.range_flag);
             }
         }
         __device__ __forceinline__ void step(const float (&x)[1], float (&o)[kOut]) {
-            yc = rs0_12(yc, mi) + __float_as_int(x[0]);
+            yc = add_sat(rs0_12(yc, mi), __float_as_int(x[0]));
             const float cf = (float)yc;
             if (KEEP_CURRENT) o[0] = __int_as_float(yc);
             o[kVol] = __int_as_float(POW2 ? trunc_i32(cf) : trunc_i32(w * (cf / w)));
@@ -117,10 +123,11 @@ struct CubaFwd {
             if (valid) {
                 yv = trunc_i32(p.v_state[p.n_vs == 1 ? 0 : m] * w);
                 mv = 4096 - trunc_i32(rintf(p.v_decay[param_index(m, p.npb, p.n_vd)]));
+                check_multiplier(mv, p.range_flag); check_state(yv, 30, p.range_flag);
             }
         }
         __device__ __forceinline__ void step(const float (&x)[1], float (&o)[1]) {
-            const int yn = rs0_12(yv, mv) + __float_as_int(x[0]);
+            const int yn = add_sat(rs0_12(yv, mv), __float_as_int(x[0]));
             yv = (yn > fire_above) ? 0 : yn;
             yv_out = yn;
             o[0] = __int_as_float(yn);
@@ -238,13 +245,13 @@ extern "C" int slayer_cuba_fwd(float* cur_out, float* vol_out, float* spk_out, f
             CubaFwd<P, G, true, S>::Params p{{in}, {cur_out, vol_out, spk_out}, cur_last_out, vol_last_out,      \
                                              i_decay, v_decay, i_state, v_state, w, 1.0f / w, spike_threshold,   \
                                              spike_scale, fa, neurons_per_batch, num_i_decays, num_v_decays,     \
-                                             num_i_states, num_v_states, sh};                                    \
+                                             num_i_states, num_v_states, sh, range_flag_device()};               \
             return launch_stream<CubaFwd<P, G, true, S>>(p, M, T, st);                                           \
         }                                                                                                        \
         CubaFwd<P, G, false, S>::Params p{{in}, {vol_out, spk_out}, cur_last_out, vol_last_out, i_decay,         \
                                           v_decay, i_state, v_state, w, 1.0f / w, spike_threshold, spike_scale,  \
                                           fa, neurons_per_batch, num_i_decays, num_v_decays, num_i_states,       \
-                                          num_v_states, sh};                                                     \
+                                          num_v_states, sh, range_flag_device()};                                \
         return launch_stream<CubaFwd<P, G, false, S>>(p, M, T, st);                                              \
     } while (0)
 #define SLAYER_CUBA(P, G)                                                                                        \

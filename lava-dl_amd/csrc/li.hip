@@ -23,7 +23,10 @@ struct LiFwd {
         float w, inv_w;
         int fire_above;               // reset when the state exceeds this (INT_MAX: reset disabled)
         int64_t npb, num_decays, num_states;
+        unsigned* range_flag;         // raised when a state comes within a factor of two of the 32-bit limit
     };
+    static constexpr bool kRangeChecked = true;
+    static constexpr int range_log2(int) { return 30; }
     // The tiles hold integers (bit patterns in float registers): the input is scaled and truncated
     // on its way into LDS, the state is converted and scaled back on its way out, and the
     // sequential loop is left with the recurrence alone.
@@ -38,12 +41,14 @@ struct LiFwd {
         if (valid) {
             y = trunc_i32(p.state[p.num_states == 1 ? 0 : m] * w);
             mult = 4096 - trunc_i32(p.decay[param_index(m, p.npb, p.num_decays)]);
+            check_multiplier(mult, p.range_flag);
+            check_state(y, 30, p.range_flag);
         }
     }
     __device__ __forceinline__ void pre(float4 (&x)[1]) const { x[0] = to_state(x[0], w); }
     __device__ __forceinline__ void post(float4 (&o)[1]) const { o[0] = from_state<POW2>(o[0], w, inv_w); }
     __device__ __forceinline__ void step(const float (&x)[1], float (&o)[1]) {
-        const int yn = rs0_12(y, mult) + __float_as_int(x[0]);
+        const int yn = add_sat(rs0_12(y, mult), __float_as_int(x[0]));
         o[0] = __int_as_float(yn);
         y = (RESET && yn > fire_above) ? 0 : yn;     // (float)yn >= threshold, decided on the integer
     }
@@ -204,7 +209,8 @@ extern "C" int slayer_li_fwd(float* out, const float* in, const float* decay, co
     const int fa = fire_above(thr_scaled > 0 ? (float)thr_scaled : __builtin_inff());
 #define SLAYER_LI_FWD(P, R)                                                                                       \
     do {                                                                                                          \
-        LiFwd<P, R>::Params p{{in}, {out}, decay, state, w, 1.0f / w, fa, neurons_per_batch, num_decays, num_states}; \
+        LiFwd<P, R>::Params p{{in}, {out}, decay, state, w, 1.0f / w, fa, neurons_per_batch, num_decays, num_states, \
+                              range_flag_device()};                                                               \
         return launch_stream<LiFwd<P, R>>(p, M, T, (hipStream_t)stream);                                          \
     } while (0)
     const bool reset = thr_scaled > 0;

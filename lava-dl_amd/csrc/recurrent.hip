@@ -30,6 +30,7 @@ struct RecurrentFwd {
     float w, inv_w, spike_thr, spike_scale, th_step_f;
     int base;
     int C, T;
+    unsigned* range_flag;                                     // see raise_range_flag in tile.h
 };
 
 template <bool ALIF, bool GRADED, bool POW2, bool VEC4>
@@ -54,6 +55,7 @@ __global__ __launch_bounds__(kMaxRecurrent) void recurrent_fwd_kernel(const Recu
     auto from = [&](int y) -> float { const float f = (float)y; return POW2 ? f * inv_w : f / w; };
 
     int yc = 0, yv = 0, th = 0, r = 0, mi = 0, mv = 0, mt = 0, mr = 0;
+    unsigned acc_lif = 0u, acc_th = 0u;                       // range of the states, see range_bits in tile.h
     if (live) {
         yc = trunc_i32(p.i_state[p.n_is == 1 ? 0 : m] * w);
         yv = trunc_i32(p.v_state[p.n_vs == 1 ? 0 : m] * w);
@@ -64,7 +66,11 @@ __global__ __launch_bounds__(kMaxRecurrent) void recurrent_fwd_kernel(const Recu
             r = trunc_i32(p.ref_state[p.n_rs == 1 ? 0 : m] * w);
             mt = 4096 - trunc_i32(rintf(p.th_decay[param_index(m, C, p.n_td)]));
             mr = 4096 - trunc_i32(rintf(p.ref_decay[param_index(m, C, p.n_rd)]));
+            check_multiplier(mt, p.range_flag); check_multiplier(mr, p.range_flag);
         }
+        check_multiplier(mi, p.range_flag); check_multiplier(mv, p.range_flag);
+        acc_lif = ((unsigned)yc + (1u << 30)) | ((unsigned)yv + (1u << 30));
+        acc_th = ((unsigned)th + (1u << 28)) | ((unsigned)r + (1u << 28));
     }
     float cur = 0.f, vol = 0.f, thf = 0.f, rf = 0.f;
     float4 zq = make_float4(0.f, 0.f, 0.f, 0.f), sq = zq, vq = zq, tq = zq;
@@ -107,15 +113,17 @@ __global__ __launch_bounds__(kMaxRecurrent) void recurrent_fwd_kernel(const Recu
         const float dend = zt + fb;
         // one step of every state, each starting from the float32 value the previous call left and
         // handing a float32 value to the next operator
-        yc = rs0_12(yc, mi) + trunc_i32(w * dend);
+        yc = add_sat(rs0_12(yc, mi), trunc_i32(w * dend));
         cur = from(yc);
         yc = trunc_i32(w * cur);
-        const int yn = rs0_12(yv, mv) + yc;
+        const int yn = add_sat(rs0_12(yv, mv), yc);
+        acc_lif |= ((unsigned)yc + (1u << 30)) | ((unsigned)yn + (1u << 30));
         vol = from(yn);
         float theta = p.spike_thr;
         if (ALIF) {
             r = rs0_12(r, mr);
             th = rs0_12(th - p.base, mt) + p.base;
+            acc_th |= ((unsigned)th + (1u << 28)) | ((unsigned)r + (1u << 28));
             thf = from(th);
             rf = from(r);
             theta = thf + rf;
@@ -169,6 +177,7 @@ __global__ __launch_bounds__(kMaxRecurrent) void recurrent_fwd_kernel(const Recu
         }
         __syncthreads();
     }
+    if (live && (range_exceeded(acc_lif, 30) || range_exceeded(acc_th, 28))) raise_range_flag(p.range_flag);
     if (live) {
         p.cur_last[m] = cur;
         p.vol_last[m] = vol;
@@ -306,6 +315,7 @@ extern "C" int slayer_cuba_recurrent_fwd(float* spk_out, float* vol_out, float* 
     p.n_id = num_i_decays; p.n_vd = num_v_decays; p.n_is = num_i_states; p.n_vs = num_v_states;
     p.w = (float)w_scale; p.inv_w = 1.0f / p.w; p.spike_thr = spike_threshold; p.spike_scale = spike_scale;
     p.C = (int)C; p.T = (int)T;
+    p.range_flag = range_flag_device();
     return launch_recurrent_fwd<false>(p, graded, w_scale, N, (hipStream_t)stream);
 }
 
@@ -342,6 +352,7 @@ extern "C" int slayer_alif_recurrent_fwd(float* spk_out, float* vol_out, float* 
     p.w = (float)w_scale; p.inv_w = 1.0f / p.w; p.spike_scale = spike_scale; p.th_step_f = th_step;
     p.base = (int)th0_scaled;
     p.C = (int)C; p.T = (int)T;
+    p.range_flag = range_flag_for_threshold(0, th0_scaled);
     return launch_recurrent_fwd<true>(p, graded, w_scale, N, (hipStream_t)stream);
 }
 

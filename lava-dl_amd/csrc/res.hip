@@ -21,7 +21,10 @@ struct ResFwd {
         float w, inv_w;
         int fire_above, im_reset;                // reset when the imaginary state exceeds fire_above
         int64_t npb, num_decays, n_rs, n_is;
+        unsigned* range_flag;
     };
+    static constexpr bool kRangeChecked = true;
+    static constexpr int range_log2(int) { return 29; }     // two products per step
     static constexpr bool kTransforms = true;    // integer tiles, see to_state / from_state
     int re, im, s, c, fire_above, im_reset;
     float w, inv_w;
@@ -35,6 +38,8 @@ struct ResFwd {
             const int64_t j = param_index(m, p.npb, p.num_decays);
             s = trunc_i32(p.sin_decay[j]);
             c = trunc_i32(p.cos_decay[j]);
+            check_multiplier(s, p.range_flag); check_multiplier(c, p.range_flag);
+            check_state(re, 29, p.range_flag); check_state(im, 29, p.range_flag);
         }
     }
     __device__ __forceinline__ void pre(float4 (&x)[2]) const {
@@ -46,8 +51,8 @@ struct ResFwd {
         o[1] = from_state<POW2>(o[1], w, inv_w);
     }
     __device__ __forceinline__ void step(const float (&x)[2], float (&o)[2]) {
-        const int re_n = rs0_12(c, re) - rs0_12(s, im) + __float_as_int(x[0]);
-        const int im_n = rs0_12(s, re) + rs0_12(c, im) + __float_as_int(x[1]);
+        const int re_n = add_sat(rs0_12(c, re) - rs0_12(s, im), __float_as_int(x[0]));
+        const int im_n = add_sat(rs0_12(s, re) + rs0_12(c, im), __float_as_int(x[1]));
         o[0] = __int_as_float(re_n);
         o[1] = __int_as_float(im_n);
         if (HAS_THR) {
@@ -80,13 +85,16 @@ struct AdResFwd {
         int step, base;
         float w, inv_w;
         int64_t npb, nd, n_rd, n_td, n_res, n_ims, n_rs, n_ts;
+        unsigned* range_flag;
     };
     int re, im, s, c, th, r, mt, mr, th_step, base;
+    unsigned acc_res, acc_th;                    // float tiles: the states are range-checked in the loop
     float w, inv_w;
 
     __device__ __forceinline__ void init(const Params& p, int64_t m, bool valid) {
         w = p.w; inv_w = p.inv_w; th_step = p.step; base = p.base;
         re = im = s = c = th = r = mt = mr = 0;
+        acc_res = acc_th = 0u;
         if (valid) {
             re = trunc_i32(p.re_state[p.n_res == 1 ? 0 : m] * w);
             im = trunc_i32(p.im_state[p.n_ims == 1 ? 0 : m] * w);
@@ -97,13 +105,19 @@ struct AdResFwd {
             c = trunc_i32(p.cos_decay[j]);
             mt = 4096 - trunc_i32(p.th_decay[param_index(m, p.npb, p.n_td)]);
             mr = 4096 - trunc_i32(p.ref_decay[param_index(m, p.npb, p.n_rd)]);
+            check_multiplier(s, p.range_flag); check_multiplier(c, p.range_flag);
+            check_multiplier(mt, p.range_flag); check_multiplier(mr, p.range_flag);
+            check_state(re, 29, p.range_flag); check_state(im, 29, p.range_flag);
+            check_state(th, 28, p.range_flag); check_state(r, 28, p.range_flag);
         }
     }
     __device__ __forceinline__ void step(const float (&x)[2], float (&o)[4]) {
         r = rs0_12(r, mr);
         th = rs0_12(th - base, mt) + base;
-        const int re_n = rs0_12(c, re) - rs0_12(s, im) + trunc_i32(w * x[0]);
-        const int im_n = rs0_12(s, re) + rs0_12(c, im) + trunc_i32(w * x[1]);
+        const int re_n = add_sat(rs0_12(c, re) - rs0_12(s, im), trunc_i32(w * x[0]));
+        const int im_n = add_sat(rs0_12(s, re) + rs0_12(c, im), trunc_i32(w * x[1]));
+        acc_res |= ((unsigned)re_n + (1u << 29)) | ((unsigned)im_n + (1u << 29));
+        acc_th |= ((unsigned)th + (1u << 28)) | ((unsigned)r + (1u << 28));
         const float ref = (float)re_n, imf = (float)im_n, thf = (float)th, rf = (float)r;
         o[0] = POW2 ? ref * inv_w : ref / w;
         o[1] = POW2 ? imf * inv_w : imf / w;
@@ -115,7 +129,9 @@ struct AdResFwd {
         re = re_n;
         im = im_n;
     }
-    __device__ __forceinline__ void finish(const Params&, int64_t, bool) {}
+    __device__ __forceinline__ void finish(const Params& p, int64_t, bool) {
+        if (range_exceeded(acc_res, 29) || range_exceeded(acc_th, 28)) raise_range_flag(p.range_flag);
+    }
 };
 
 struct ResBwd {
@@ -173,7 +189,8 @@ static int res_fwd_launch(float* re_out, float* im_out, const float* re_in, cons
                           hipStream_t stream) {
     using Op = ResFwd<POW2, HAS_THR>;
     typename Op::Params p{{re_in, im_in}, {re_out, im_out}, sin_decay, cos_decay, re_state, im_state,
-                          w, 1.0f / w, fire_above(thr), im_reset, npb, nd, n_rs, n_is};
+                          w, 1.0f / w, fire_above(thr), im_reset, npb, nd, n_rs, n_is, range_flag_device()};
+    if (HAS_THR && (im_reset >= (1 << 29) || im_reset < -(1 << 29))) range_flag_raise_from_host();
     return launch_stream<Op>(p, M, T, stream);
 }
 
@@ -271,18 +288,19 @@ extern "C" int slayer_adres_fwd(float* re_out, float* im_out, float* th_out, flo
     if (w_scale == 0) return SLAYER_EINVAL;
     const int64_t lim = 0x7fffffffLL;
     if (th_step_scaled > lim || th_step_scaled < -lim || th0_scaled > lim || th0_scaled < -lim) return SLAYER_ERANGE;
+    unsigned* flag = range_flag_for_threshold(th_step_scaled, th0_scaled);
     const float w = (float)w_scale;
     hipStream_t st = (hipStream_t)stream;
     if (is_pow2(w_scale)) {
         AdResFwd<true>::Params p{{re_in, im_in}, {re_out, im_out, th_out, ref_out}, sin_decay, cos_decay, ref_decay,
                                  th_decay, re_state, im_state, ref_state, th_state, (int)th_step_scaled,
                                  (int)th0_scaled, w, 1.0f / w, neurons_per_batch, num_decays, num_ref_decays,
-                                 num_th_decays, num_re_states, num_im_states, num_ref_states, num_th_states};
+                                 num_th_decays, num_re_states, num_im_states, num_ref_states, num_th_states, flag};
         return launch_stream<AdResFwd<true>>(p, M, T, st);
     }
     AdResFwd<false>::Params p{{re_in, im_in}, {re_out, im_out, th_out, ref_out}, sin_decay, cos_decay, ref_decay,
                               th_decay, re_state, im_state, ref_state, th_state, (int)th_step_scaled,
                               (int)th0_scaled, w, 1.0f / w, neurons_per_batch, num_decays, num_ref_decays,
-                              num_th_decays, num_re_states, num_im_states, num_ref_states, num_th_states};
+                              num_th_decays, num_re_states, num_im_states, num_ref_states, num_th_states, flag};
     return launch_stream<AdResFwd<false>>(p, M, T, st);
 }

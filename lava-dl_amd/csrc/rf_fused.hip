@@ -35,7 +35,10 @@ struct RfFwd {
         int fire_above;                             // a real state above this is at or over the spike threshold
         int64_t npb, nd, n_rs, n_is, n_last;
         Shifts shifts;
+        unsigned* range_flag;
     };
+    static constexpr bool kRangeChecked = true;
+    static constexpr int range_log2(int o) { return o < 2 ? 29 : 0; }     // real, imag (two products per step); not the spike flags
     int re, im, im_prev, s, c, fire_above, fired_last;
     float w, inv_w, spike_scale;
 
@@ -49,6 +52,8 @@ struct RfFwd {
             s = trunc_i32(p.sin_decay[j]);
             c = trunc_i32(p.cos_decay[j]);
             im_prev = (p.imag_last[p.n_last == 1 ? 0 : m] < 0.0f) ? -1 : 0;      // only its sign matters
+            check_multiplier(s, p.range_flag); check_multiplier(c, p.range_flag);
+            check_state(re, 29, p.range_flag); check_state(im, 29, p.range_flag);
         }
     }
     __device__ __forceinline__ void pre(float4 (&x)[2]) const {
@@ -56,8 +61,8 @@ struct RfFwd {
         x[1] = to_state(x[1], w);
     }
     __device__ __forceinline__ void step(const float (&x)[2], float (&o)[3]) {
-        const int re_n = rs0_12(c, re) - rs0_12(s, im) + __float_as_int(x[0]);
-        const int im_n = rs0_12(s, re) + rs0_12(c, im) + __float_as_int(x[1]);
+        const int re_n = add_sat(rs0_12(c, re) - rs0_12(s, im), __float_as_int(x[0]));
+        const int im_n = add_sat(rs0_12(s, re) + rs0_12(c, im), __float_as_int(x[1]));
         const bool fired = (re_n > fire_above) & (im_prev < 0) & (im_n >= 0);
         re = re_n; im = im_n; im_prev = im_n;
         if (SHIFT) fired_last = fired ? 1 : 0;
@@ -212,7 +217,8 @@ extern "C" int slayer_rf_fwd(float* re_out, float* im_out, float* spk_out, float
     do {                                                                                                         \
         RfFwd<P, G, S>::Params p{{re_in, im_in}, {re_out, im_out, spk_out}, re_last_out, im_last_out, sin_decay, \
                                  cos_decay, re_state, im_state, imag_last, w, 1.0f / w, spike_scale, fire,       \
-                                 neurons_per_batch, num_decays, num_re_states, num_im_states, num_last, sh};     \
+                                 neurons_per_batch, num_decays, num_re_states, num_im_states, num_last, sh,      \
+                                 range_flag_device()};                                                           \
         return launch_stream<RfFwd<P, G, S>>(p, M, T, st);                                                       \
     } while (0)
 #define SLAYER_RF(P, G)                                                                                          \

@@ -40,10 +40,19 @@ __device__ __forceinline__ float lane_below(float v, float fill) {       // lane
     return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(fill), __float_as_int(v), 0x138, 0xf, 0xf, false));
 }
 
+// c -> B + A * c applied to c.  A map with multiplier 0 is a cut (the last quad of a row): it lets nothing in, not
+// even an Inf or a NaN that a later row produced (0 * Inf would be a NaN), so rows stay independent of each other
+// as they are in a step-by-step evaluation.  For finite operands the result is the same bit for bit.
+__device__ __forceinline__ float apply_affine(float A, float c, float B) {
+    const float v = __fmaf_rn(A, c, B);
+    return A == 0.0f ? B : v;
+}
+
 // Inclusive scan over the lanes, lowest lane first, of affine maps c -> B + A * c: afterwards (A, B) of lane l is
 // the composition of the maps of lanes 0 .. l (lane 0 applied first).
 __device__ __forceinline__ void scan_affine(float& A, float& B) {
-#define SLAYER_COMBINE(An, Bn) do { const float an_ = (An), bn_ = (Bn); B = __fmaf_rn(A, bn_, B); A = A * an_; } while (0)
+#define SLAYER_COMBINE(An, Bn) do { const float an_ = (An), bn_ = (Bn); const bool cut_ = A == 0.0f;            \
+        const float b2_ = __fmaf_rn(A, bn_, B), a2_ = A * an_; B = cut_ ? B : b2_; A = cut_ ? 0.0f : a2_; } while (0)
     SLAYER_COMBINE(lane_below_in_row<1>(A, 1.0f), lane_below_in_row<1>(B, 0.0f));
     SLAYER_COMBINE(lane_below_in_row<2>(A, 1.0f), lane_below_in_row<2>(B, 0.0f));
     SLAYER_COMBINE(lane_below_in_row<4>(A, 1.0f), lane_below_in_row<4>(B, 0.0f));
@@ -139,8 +148,8 @@ __device__ __forceinline__ float4 real_stage(RealStage& L, const ScanSpan& sp, i
     float carry = L.carry[parity];
 #pragma unroll
     for (int w = 0; w < kScanWaves - 1; ++w)
-        if (w < sp.wv) carry = __fmaf_rn(L.A[parity][w], carry, L.B[parity][w]);
-    const float leaving = __fmaf_rn(A, carry, B);                    // gradient leaving this thread's quad
+        if (w < sp.wv) carry = apply_affine(L.A[parity][w], carry, L.B[parity][w]);
+    const float leaving = apply_affine(A, carry, B);                 // gradient leaving this thread's quad
     float entering = lane_below(leaving, carry);
     if (row_end || !active) entering = 0.0f;
     ent = entering;
@@ -499,11 +508,21 @@ struct ComplexStage {
     float Ar[2][kScanWaves], Ai[2][kScanWaves], Br[2][kScanWaves], Bi[2][kScanWaves], cr[2], ci[2];
 };
 
+// z -> B + A * z applied to z; a zero multiplier is a cut that lets nothing in (see apply_affine)
+__device__ __forceinline__ Cx apply_affine_complex(Cx A, Cx z, Cx B) {
+    const Cx v = cfma(A, z, B);
+    const bool cut = A.re == 0.0f && A.im == 0.0f;
+    return Cx{cut ? B.re : v.re, cut ? B.im : v.im};
+}
+
 // inclusive scan over the lanes of complex affine maps z -> B + A * z (see scan_affine)
 __device__ __forceinline__ void scan_affine_complex(Cx& A, Cx& B) {
 #define SLAYER_COMBINE(M) do {                                                                                  \
         const Cx an_{M(A.re, 1.0f), M(A.im, 0.0f)}, bn_{M(B.re, 0.0f), M(B.im, 0.0f)};                          \
-        B = cfma(A, bn_, B); A = cmul(A, an_); } while (0)
+        const bool cut_ = A.re == 0.0f && A.im == 0.0f;                                                         \
+        const Cx b2_ = cfma(A, bn_, B), a2_ = cmul(A, an_);                                                     \
+        B = Cx{cut_ ? B.re : b2_.re, cut_ ? B.im : b2_.im};                                                     \
+        A = Cx{cut_ ? 0.0f : a2_.re, cut_ ? 0.0f : a2_.im}; } while (0)
     SLAYER_COMBINE(lane_below_in_row<1>);
     SLAYER_COMBINE(lane_below_in_row<2>);
     SLAYER_COMBINE(lane_below_in_row<4>);
@@ -659,8 +678,8 @@ __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
         Cx carry{L.cr[parity], L.ci[parity]};
 #pragma unroll
         for (int w = 0; w < kScanWaves - 1; ++w)
-            if (w < sp.wv) carry = cfma(Cx{L.Ar[parity][w], L.Ai[parity][w]}, carry, Cx{L.Br[parity][w], L.Bi[parity][w]});
-        const Cx leaving = cfma(A, carry, B);
+            if (w < sp.wv) carry = apply_affine_complex(Cx{L.Ar[parity][w], L.Ai[parity][w]}, carry, Cx{L.Br[parity][w], L.Bi[parity][w]});
+        const Cx leaving = apply_affine_complex(A, carry, B);
         Cx ent{lane_below(leaving.re, carry.re), lane_below(leaving.im, carry.im)};
         if (row_end || !active) ent = Cx{0.0f, 0.0f};
         const Cx z3 = cfma(mu, ent, h3), z2 = cfma(mu2, ent, h2), z1 = cfma(mu3, ent, h1), z0 = cfma(mu4, ent, h0);

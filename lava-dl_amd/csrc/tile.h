@@ -32,6 +32,39 @@ __device__ __forceinline__ int rs0_12(int a, int b) {
     return (int)(((long long)a * (long long)b + bias) >> 12);
 }
 
+// a + b held inside the int32 range (v_add_i32 with clamp: one instruction, as the wrapping add).  The state
+// updates use it so that a sum that leaves the range ends at the limit, where the range check of the copy-out
+// sees it, instead of wrapping to an innocent-looking value.
+__device__ __forceinline__ int add_sat(int a, int b) { return __builtin_elementwise_add_sat(a, b); }
+
+// Range of the 32-bit states.  The kernels follow the reference's 64-bit evaluation bit for bit while no
+// intermediate leaves 32 bits.  That is guaranteed while every stored state stays below a bound that leaves room
+// for one more step (2^30 for a single decayed state plus input, 2^29 for the two-product resonator step, 2^28 for
+// threshold / refractory states, whose spike adds step and twice the threshold) and every decay multiplier is at
+// most 8191 in magnitude: an Op with integer tiles names the bound of each output tile (range_log2), the copy-out
+// tests every value it stores on its way (off the sequential chain), the Op's init tests the multipliers, and
+// either raises the process-wide flag behind Params::range_flag (pinned host memory that the device can write).
+__device__ __forceinline__ void raise_range_flag(unsigned* flag) {
+    if (flag) *reinterpret_cast<volatile unsigned*>(flag) = 1u;
+}
+__device__ __forceinline__ void check_multiplier(int mult, unsigned* flag) {
+    if (mult > 8191 || mult < -8191) raise_range_flag(flag);
+}
+template <class Op, class = void>
+struct RangeChecked { static constexpr bool value = false; };
+template <class Op>
+struct RangeChecked<Op, decltype((void)Op::kRangeChecked)> { static constexpr bool value = Op::kRangeChecked; };
+// accumulates v + 2^L for a quad: a value outside [-2^L, 2^L) sets a bit at or above bit L + 1
+__device__ __forceinline__ unsigned range_bits(float4 q, int log2_bound) {
+    const unsigned b = 1u << log2_bound;
+    return (__float_as_uint(q.x) + b) | (__float_as_uint(q.y) + b) | (__float_as_uint(q.z) + b) | (__float_as_uint(q.w) + b);
+}
+__device__ __forceinline__ bool range_exceeded(unsigned acc, int log2_bound) { return (acc >> (log2_bound + 1)) != 0u; }
+// an initial state (never stored, so never seen by the copy-out) against the bound of its tile
+__device__ __forceinline__ void check_state(int y, int log2_bound, unsigned* flag) {
+    if (range_exceeded((unsigned)y + (1u << log2_bound), log2_bound)) raise_range_flag(flag);
+}
+
 // Largest integer y whose float32 conversion is below thr: (float)y >= thr  <=>  y > fire_above(thr),
 // so a recurrence can take its reset decision on the integer state.  INT_MAX (never fires) for
 // thresholds beyond the int range, NaN or +inf.
@@ -323,6 +356,7 @@ struct Copier {
     int row_lo, row_hi;                      // rows [row_lo, row_hi) of the tile are copied by this wave
     int kin[kShifts ? kPasses : 1], kout[kShifts ? kPasses : 1];   // shifts of this lane's row in each pass
     int kout_row;                            // output shift of row `lane` (lane = row), for fill_unreached
+    unsigned range_acc[RangeChecked<Op>::value ? NO : 1];   // see range_bits
     // wave-uniform: chunks [in_first, in_last] hold only quads whose shifted source lies wholly inside its row,
     // chunks [out_first, out_last] only quads whose shifted destination does (for every row of this wave)
     int in_first, in_last, out_first, out_last;
@@ -331,6 +365,8 @@ struct Copier {
     __device__ __forceinline__ void init(const typename Op::Params& prm, int64_t m0, int rows_, int T_, int lane,
                                          unsigned base_f, int first_pass_ = 0) {
         rows = rows_; T = T_; first_pass = first_pass_;
+#pragma unroll
+        for (int o = 0; o < (RangeChecked<Op>::value ? NO : 1); ++o) range_acc[o] = 0u;
         row_lo = first_pass * G::kRowsPerPass;
         row_hi = (first_pass + kPasses) * G::kRowsPerPass;
         if (row_hi > rows) row_hi = rows;
@@ -507,6 +543,17 @@ struct Copier {
             }
     }
 
+    // Raises the range flag when a state this wave stored came too close to the 32-bit limit (see range_bits).
+    __device__ __forceinline__ void report_range(const typename Op::Params& prm) const {
+        if constexpr (RangeChecked<Op>::value) {
+            bool bad = false;
+#pragma unroll
+            for (int o = 0; o < NO; ++o)
+                if (Op::range_log2(o) != 0) bad = bad || range_exceeded(range_acc[o], Op::range_log2(o));
+            if (bad) raise_range_flag(prm.range_flag);
+        }
+    }
+
     // LDS -> global.  On edge chunks the line shared by rows r and r+1 is completed before it is
     // stored: in a forward pass the lanes that copy the last line of row r fill its slots past
     // the end of the row with the head of row r+1, which they fetched from that row's tile in
@@ -524,6 +571,11 @@ struct Copier {
             float4 v[NO], own[NO];                                  // own: this lane's quad, for shifted outputs
 #pragma unroll
             for (int o = 0; o < NO; ++o) own[o] = v[o] = *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]);
+            if constexpr (RangeChecked<Op>::value) {
+#pragma unroll
+                for (int o = 0; o < NO; ++o)
+                    if (Op::range_log2(o) != 0) range_acc[o] |= range_bits(v[o], Op::range_log2(o));
+            }
             if (!inner) {
                 const int a = 4 * cq - step0[p];                   // phase of row r
                 const bool valid = (unsigned)t < (unsigned)T;
@@ -755,6 +807,7 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
         io.copy_out(op, tile, chunk);
         __syncthreads();
     }
+    io.report_range(prm);
     op.finish(prm, m0 + lane, lane < rows);
 }
 
@@ -824,6 +877,7 @@ __global__ __launch_bounds__((1 + NCOPY) * kWave) void stream_kernel_duo(typenam
             __syncthreads();                                   // barrier k+2
         }
         io.copy_out(uni, tiles[1], chunk_of(nloop - 1));
+        io.report_range(prm);
     }
 }
 
@@ -899,6 +953,7 @@ __global__ __launch_bounds__((2 + NCOPY) * kWave) void stream_kernel_staged(type
                 __syncthreads();                               // barrier j+h+1
             }
         }
+        io.report_range(prm);
     }
 }
 
@@ -1021,6 +1076,12 @@ __global__ __launch_bounds__(kWave) void stream_kernel_scalar(typename Op::Param
             float4 y[NO], v[NO + ND];
 #pragma unroll
             for (int o = 0; o < NO; ++o) y[o] = *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]);
+            if constexpr (RangeChecked<Op>::value) {
+#pragma unroll
+                for (int o = 0; o < NO; ++o)
+                    if (Op::range_log2(o) != 0 && r < rows && range_exceeded(range_bits(y[o], Op::range_log2(o)), Op::range_log2(o)))
+                        raise_range_flag(prm.range_flag);
+            }
             if constexpr (HasTransforms<Op>::value) op.post(y);
 #pragma unroll
             for (int o = 0; o < NO; ++o) v[o] = y[o];

@@ -2,5 +2,7 @@
 dynamics, spike functions, time shift and temporal filter, all backed by
 libslayer_hip.so (hand-written HIP for gfx950)."""
 from . import neuron, spike, utils, axon, dendrite, block
+from ._native import range_check, range_flag, range_policy, clear_range_flag
 
-__all__ = ['neuron', 'spike', 'utils', 'axon', 'dendrite', 'block']
+__all__ = ['neuron', 'spike', 'utils', 'axon', 'dendrite', 'block',
+           'range_check', 'range_flag', 'range_policy', 'clear_range_flag']

@@ -14,7 +14,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # SLAYER_HIP_LIB points at an alternative build of the same library (e.g. a tuning build)
 LIB_PATH = os.environ.get('SLAYER_HIP_LIB') or os.path.join(_HERE, 'libslayer_hip.so')
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _lib = None
 _lib_lock = threading.Lock()       # forward runs on the user thread, backward on an autograd thread
@@ -38,6 +38,9 @@ _DP = ctypes.POINTER(Delays)
 _SIGNATURES = {
     'slayer_abi_version': (_INT, []),
     'slayer_error_string': (ctypes.c_char_p, [_INT]),
+    'slayer_range_status': (_INT, [ctypes.POINTER(_INT), _INT]),
+    'slayer_range_word': (_P, []),
+    'slayer_bwd_takes_scan': (_INT, [_I64, _I64, _I64]),
     'slayer_li_fwd': (_INT, [_P, _P, _P, _P, _D, _INT, _I64, _I64, _I64, _I64, _I64, _P]),
     'slayer_li_bwd': (_INT, [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _P]),
     'slayer_li_bwd_static': (_INT, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _P]),
@@ -109,6 +112,72 @@ def check(code):
     if code != 0:
         msg = lib().slayer_error_string(code).decode()
         raise RuntimeError(f'libslayer_hip call failed ({code}): {msg}')
+    if (_range_word or _find_range_word()).value:
+        _range_raised()
+
+
+# ---- range of the 32-bit fixed-point states -------------------------------------------------------------------
+# The forward kernels raise a flag (one word of pinned host memory, slayer_range_status in include/slayer_hip.h)
+# when a state comes within a factor of two of the int32 limit, where the reference's int64 CPU branch
+# (neuron/dynamics/leaky_integrator.py:213) would simply go on.  Every operator call looks at the word after its
+# launch -- a plain memory read -- so an overflow of a launch that has completed is reported by the next call, and
+# range_check() reports it on demand.
+_range_word = None
+_range_policy = 'raise'
+
+
+def _find_range_word():
+    global _range_word
+    addr = lib().slayer_range_word()
+    if not addr:                      # no device to map the word for: nothing can be launched either
+        return ctypes.c_uint(0)
+    _range_word = ctypes.c_uint.from_address(addr)
+    return _range_word
+
+
+def _range_raised():
+    clear_range_flag()
+    msg = ('a fixed-point state of a slayer kernel came within a factor of two of the 32-bit range (or a decay '
+           'multiplier lies beyond +-8191): results since the last check may differ from a 64-bit evaluation. '
+           'Lower w_scale or the input magnitude, or run with debug=True to compare against the 64-bit kernels.')
+    if _range_policy == 'raise':
+        raise OverflowError(msg)
+    if _range_policy == 'warn':
+        import warnings
+        warnings.warn(msg, RuntimeWarning, stacklevel=3)
+
+
+def range_policy(mode=None):
+    """What a raised range flag does when an operator call or ``range_check`` sees it: ``'raise'`` (default,
+    OverflowError), ``'warn'`` (RuntimeWarning) or ``'ignore'``.  Returns the mode that was set before."""
+    global _range_policy
+    before = _range_policy
+    if mode is not None:
+        if mode not in ('raise', 'warn', 'ignore'):
+            raise ValueError(f'unknown range policy {mode!r}')
+        _range_policy = mode
+    return before
+
+
+def range_flag():
+    """True when a launch that has completed raised the range flag since it was last cleared."""
+    return bool((_range_word or _find_range_word()).value)
+
+
+def clear_range_flag():
+    """Lowers the flag; returns whether it was up."""
+    raised = ctypes.c_int(0)
+    lib().slayer_range_status(ctypes.byref(raised), 1)
+    return bool(raised.value)
+
+
+def range_check(sync=True):
+    """Waits for the device (unless ``sync`` is false) and applies the policy to the flag: the definite answer for
+    everything launched so far."""
+    if sync and torch.cuda.is_available():
+        torch.cuda.synchronize()
+    if range_flag():
+        _range_raised()
 
 
 def require_gpu(*tensors):
@@ -130,10 +199,19 @@ def require_gpu(*tensors):
     return dev
 
 
+def scan_tolerance(grad):
+    """Tolerance of the debug cross-check of a float backward pass on ``grad``: 1e-5 of the largest magnitude when
+    the library evaluates a tensor of this shape as a wave scan (whose rounding differs from a step-by-step
+    evaluation by a few ulp of the largest terms), None -- every bit must agree -- when it walks it step by step."""
+    M, T = rows_and_steps(grad)
+    scan = lib().slayer_bwd_takes_scan(M, neurons_per_batch(grad), T) and grad.data_ptr() % 16 == 0
+    return 1e-5 if scan else None
+
+
 def raise_on_mismatch(what, fast, check, rel=None):
     """debug mode: the streaming kernel and the one-thread-per-neuron kernel must agree, bit for bit for the
-    fixed-point forward passes; float gradients (``rel`` given) within ``rel`` of their largest magnitude (large
-    tensors take a scan whose rounding differs from the step-by-step evaluation by a few ulp)."""
+    fixed-point forward passes and for float gradients that both kernels walk step by step; float gradients that
+    went through a scan (``rel`` given, see ``scan_tolerance``) within ``rel`` of their largest magnitude."""
     if rel is not None:
         scale = float(check.abs().max()) if check.numel() else 0.0
         err = float((fast - check).abs().max()) if check.numel() else 0.0

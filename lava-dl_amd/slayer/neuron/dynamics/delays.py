@@ -27,7 +27,11 @@ class Delays:
         ``axon.Delay`` hands to its shift).  When it requires a gradient it receives the one
         ``axon.Delay`` computes, scaled by ``grad_scale``.
     output_steps : int
-        whole steps added to every neuron's spike delay (``step_delay`` of a block: 1).
+        whole steps added to every neuron's spike delay (``step_delay`` of a block: 1); not negative.  The
+        spikes move by the *sum* ``output_steps + trunc(output_delay / sampling_time)`` of each neuron, in the
+        fused kernels and in the separate operators alike (a negative ``output_delay`` entry next to a positive
+        ``output_steps`` therefore loses no sample in between); an ``output_head`` or a trained
+        ``output_delay`` needs entries that are not negative, as ``axon.Delay`` keeps them.
     output_head : tensor or None
         shaped like the states: the spike that precedes the first one (``step_delay``'s buffer when the
         neuron keeps its state between calls); it lands just before the first spike of this call.
@@ -43,6 +47,8 @@ class Delays:
         self.sampling_time = sampling_time
         self.grad_scale = grad_scale
 
+        if self.output_steps < 0:
+            raise RuntimeError(f'output_steps is a delay in whole steps, it cannot be negative ({self.output_steps})')
         if output_head is not None and self.output_steps != 1:
             raise RuntimeError('output_head is the buffer of a one-step delay: it needs output_steps == 1')
 
@@ -139,6 +145,16 @@ def chain_output(delays, spike):
     from ...axon.delay import delay, _delayFunction
     if not delays:
         return spike
+    if delays.output_steps != 0 and delays.output_delay is not None:
+        od = delays.output_delay if torch.is_tensor(delays.output_delay) else torch.tensor(float(delays.output_delay))
+        if delays.output_head is None and not od.requires_grad:
+            # one shift by the sum, as the fused kernels do: two shifts in a row would drop the samples that
+            # leave the row in between when the two parts have opposite signs
+            steps = delays.output_steps + torch.trunc(od.detach().float() / delays.sampling_time)
+            return delay(spike, steps.to(spike.device) if steps.numel() > 1 else float(steps), 1)
+        if bool((od.detach() < 0).any()):
+            raise RuntimeError('a negative output_delay next to output_steps needs the summed shift, which an '
+                               'output_head or a trained output_delay does not take')
     if delays.output_steps != 0:
         spike = delay(spike, delays.output_steps)
         if delays.output_head is not None:

@@ -114,7 +114,7 @@ class _LIDynamics(torch.autograd.Function):
         grad_input, grad_decay = _bwd(grad_output, output, decay.detach(), need)
         if ctx.debug:
             N.raise_on_mismatch('leaky_integrator backward', grad_input, _bwd_naive(grad_output, decay.detach()),
-                                rel=1e-5)
+                                rel=N.scan_tolerance(grad_output))
         if grad_decay is not None:
             grad_decay = grad_decay.reshape(decay.shape)
         return grad_input, grad_decay, None, None, None

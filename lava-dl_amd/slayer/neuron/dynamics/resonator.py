@@ -134,8 +134,8 @@ class _ResDynamics(torch.autograd.Function):
                                         sin_decay.detach(), cos_decay.detach(), need)
         if ctx.debug:
             c_re, c_im = _bwd_naive(grad_real, grad_imag, sin_decay.detach(), cos_decay.detach())
-            N.raise_on_mismatch('resonator grad real', g_re, c_re, rel=1e-5)
-            N.raise_on_mismatch('resonator grad imag', g_im, c_im, rel=1e-5)
+            N.raise_on_mismatch('resonator grad real', g_re, c_re, rel=N.scan_tolerance(g_re))
+            N.raise_on_mismatch('resonator grad imag', g_im, c_im, rel=N.scan_tolerance(g_im))
         _raise_on_nan(grad_real=grad_real, grad_imag=grad_imag, grad_real_input=g_re,
                       grad_imag_input=g_im, grad_sin_decay=g_sin, grad_cos_decay=g_cos)
         if g_sin is not None:

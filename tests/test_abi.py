@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(handle, n), f'{n} declared in slayer_hip.h but not exported'
     assert sorted(_native.EXPORTS) == names, 'python binding and header disagree'
-    assert _native.lib().slayer_abi_version() == _native.ABI_VERSION == 3
+    assert _native.lib().slayer_abi_version() == _native.ABI_VERSION == 4
     assert b'success' in _native.lib().slayer_error_string(0)
     assert b'inconsistent' in _native.lib().slayer_error_string(-1)
 
@@ -58,6 +58,14 @@ def test_argument_validation_happens_before_any_launch():
     assert b'scratch' in L.slayer_error_string(-4)
     assert L.slayer_res_bwd(one, one, one, None, one, one, one, one, one, one, one, 8, 4, 1, 8, None) == ENULL
     assert L.slayer_conv(one, one, one, 0, 1.0, 8, 8, None) == EINVAL
+    # which float backward passes are wave scans: tensors of 2^20 elements and more, whole quads or rows of 64+ steps
+    assert L.slayer_bwd_takes_scan(4096, 64, 300) == 1 and L.slayer_bwd_takes_scan(4096, 64, 301) == 1
+    assert L.slayer_bwd_takes_scan(512, 64, 300) == 0 and L.slayer_bwd_takes_scan(1 << 20, 64, 3) == 0
+    # the range flag needs a device to map its word for; without one the call says so instead of failing
+    raised = ctypes.c_int(7)
+    code = L.slayer_range_status(ctypes.byref(raised), 0)
+    assert code == (0 if torch.cuda.is_available() else -5)
+    assert b'range flag' in L.slayer_error_string(-5)
     assert L.slayer_conv(one, one, one, 5000, 1.0, 8, 8, None) == ERANGE
     assert L.slayer_shift(one, one, None, 1, 1.0, 8, 3, 8, None) == EINVAL
     assert L.slayer_spike_fwd(one, one, one, 3, 0.0, 0, 1.0, 8, None) == EINVAL             # 3 thresholds for 8 samples

@@ -416,3 +416,27 @@ def test_fused_cuba_with_delays_at_synapse_workload_size(slayer):
         r_gc, _ = O.li_bwd(r_gv, r_vol, vd)
         r_gx, _ = O.li_bwd(r_gc, r_cur, cd)
         assert_rel(xg.grad[b:b + 1, sl], O.shift(r_gx, -in_shift[sl], 1), f'slab {b} grad_input')
+
+
+def test_delay_parts_of_opposite_sign_move_the_spikes_by_their_sum(slayer):
+    """``output_steps`` and a negative ``output_delay`` add up to one shift in the fused kernels; the separate
+    operators (debug, dropout or norm) must not drop the samples that two shifts in a row would push off the
+    row in between: the same ``Neuron.forward(delays=...)`` gives the same spikes either way."""
+    D = slayer.neuron.dynamics.delays
+    gen = torch.Generator().manual_seed(11)
+    x = sparse_input(gen, (2, 6, 64), p=0.4).to(dev())
+    table = torch.tensor([-1.0, 0.0, -2.0, 1.0, -1.0, 3.0])
+    n = slayer.neuron.cuba.Neuron(1.0, 0.25, 0.03).to(dev())
+    plain = n(x)
+    assert float(plain[..., -1].abs().sum()) > 0 or float(plain[..., -2].abs().sum()) > 0
+    fused = n(x, delays=D.Delays(output_delay=table, output_steps=1))
+    n.debug = True
+    chain = n(x, delays=D.Delays(output_delay=table, output_steps=1))
+    assert torch.equal(fused, chain)
+    # rows whose parts cancel are the undelayed spikes, last sample included
+    assert torch.equal(fused[:, 0], plain[:, 0]) and torch.equal(fused[:, 4], plain[:, 4])
+    assert torch.equal(fused[:, 2, :-1], plain[:, 2, 1:])
+    with pytest.raises(RuntimeError):
+        D.Delays(output_steps=-1)
+    with pytest.raises(RuntimeError):
+        D.chain_output(D.Delays(output_delay=table.to(dev()).requires_grad_(), output_steps=1), plain)

@@ -167,3 +167,50 @@ def test_fused_rf_backward_scan_equals_the_chain_of_scans_bit_for_bit(slayer, sh
     want = O.res_bwd(o_re, o_im, re[:k].cpu(), im[:k].cpu(), sin.cpu(), cos.cpu())
     assert_scale(g_re[:k], want[0], 'grad real vs oracle')
     assert_scale(g_im[:k], want[1], 'grad imag vs oracle')
+
+
+@pytest.mark.parametrize('shape', [(5, 1024, 300), (3, 43, 8196), (5, 1024, 301)])
+@pytest.mark.parametrize('bad', [float('nan'), float('inf')])
+def test_a_non_finite_row_does_not_reach_its_neighbours(slayer, shape, bad):
+    """Rows are independent in the step-by-step recurrences (neuron/dynamics/leaky_integrator.py:234-259,
+    resonator.py:379-467 in the reference): a NaN or Inf in the gradient of one row must leave every other row of
+    the scan's span exactly as it is without it -- the cut at a row end lets nothing in, not 0 * Inf either."""
+    D = slayer.neuron.dynamics
+    gen = torch.Generator().manual_seed(seed_of('scan-nonfinite', shape))
+    C, T = shape[1], shape[-1]
+    g = torch.randn(shape, generator=gen)
+    y = torch.randn(shape, generator=gen)
+    cur = torch.randn(shape, generator=gen)
+    d = torch.randint(0, 4097, (C,), generator=gen).float()
+    d2 = torch.randint(0, 4097, (C,), generator=gen).float()
+    rows = g.reshape(-1, T)
+    M = rows.shape[0]
+    victims = [3, M // 2 + 1, M - 2]                     # inside a span, wherever spans happen to begin and end
+    dirty = rows.clone()
+    for i, r in enumerate(victims):
+        dirty[r, (T // 3) * (i + 1) - 1 if i < 2 else T - 1] = bad
+    dirty = dirty.reshape(shape)
+    clean_rows = torch.ones(M, dtype=torch.bool)
+    clean_rows[victims] = False
+    to = lambda t: t.to(dev())
+
+    def untouched(a, b, what):
+        a, b = a.reshape(-1, T)[clean_rows.to(a.device)], b.reshape(-1, T)[clean_rows.to(b.device)]
+        assert bool(torch.isfinite(a).all()), what + ': a clean row became non-finite'
+        assert torch.equal(a, b), what + ': a clean row changed'
+
+    want, _ = D.leaky_integrator._bwd(to(g), to(y), to(d), True)
+    got, _ = D.leaky_integrator._bwd(to(dirty), to(y), to(d), True)
+    untouched(got, want, 'leaky integrator scan')
+    assert not bool(torch.isfinite(got.reshape(-1, T)[victims]).all())
+
+    sin = ((4096 - d.clamp(40, 4095)) * 0.6).round()
+    cos = ((4096 - d.clamp(40, 4095)) * 0.8).round()
+    want = D.resonator._bwd(to(g), to(cur), to(y), to(cur), to(sin), to(cos), True)
+    got = D.resonator._bwd(to(dirty), to(cur), to(y), to(cur), to(sin), to(cos), True)
+    untouched(got[0], want[0], 'resonator scan, real')
+    untouched(got[1], want[1], 'resonator scan, imag')
+
+    want = D.cuba_fused._bwd(to(g), to(y), to(cur), to(d), to(d2), 1.0, 0.7, 1.3, False, True)[0]
+    got = D.cuba_fused._bwd(to(dirty), to(y), to(cur), to(d), to(d2), 1.0, 0.7, 1.3, False, True)[0]
+    untouched(got, want, 'fused CUBA scan')

@@ -156,6 +156,29 @@ def test_conv_corr_small_and_large_magnitudes(slayer, K, x_scale, f_scale):
     assert np.abs(z - lfilter(fd, [1.0], rows[:, ::-1], axis=-1)[:, ::-1]).max() <= 1e-5 * scale
 
 
+@pytest.mark.parametrize('K', [16, 64, 128])
+def test_conv_corr_at_the_top_of_the_float32_range(slayer, K):
+    """Sparse samples of the largest float32 magnitudes (3.3895e38 is the largest bfloat16, 3.4028e38 the largest
+    float32: in between a sample has no nearest bfloat16) and taps of the same magnitudes against unit samples:
+    the results stay finite and meet the bar, as the reference's float32 multiply-adds do
+    (utils/filter/conv.cu:25-78)."""
+    from scipy.signal import lfilter
+    gen = torch.Generator().manual_seed(seed_of('top of range', K))
+    big = torch.tensor([3.3895e38, 3.39e38, 3.40e38, 3.4028234e38, -3.395e38, -3.4028234e38, 1.7e38, 3.38e38])
+    x = torch.zeros(64, 300)
+    pos = torch.randperm(64 * 300, generator=gen)[:400]
+    x.view(-1)[pos] = big[torch.randint(0, len(big), (400,), generator=gen)]
+    f = torch.randn(K, generator=gen) * (0.5 / K)            # sums of overlapping windows stay below the maximum
+    for xs, fs in ((x, f), ((x != 0).float() * 0.125, torch.cat([big, torch.zeros(K - len(big))])[torch.randperm(K, generator=gen)])):
+        rows, fd = xs.double().numpy(), fs.double().numpy()
+        scale = np.abs(fd).sum() * np.abs(rows).max()
+        y = slayer.utils.filter.conv(xs.to(dev()), fs.to(dev()), 1).cpu().double().numpy()
+        z = slayer.utils.filter.corr(xs.to(dev()), fs.to(dev()), 1).cpu().double().numpy()
+        assert np.isfinite(y).all() and np.isfinite(z).all()
+        assert np.abs(y - lfilter(fd, [1.0], rows, axis=-1)).max() <= 1e-5 * scale
+        assert np.abs(z - lfilter(fd, [1.0], rows[:, ::-1], axis=-1)[:, ::-1]).max() <= 1e-5 * scale
+
+
 @pytest.mark.parametrize('K', [16, 24, 64, 100])
 @pytest.mark.parametrize('shape', [(8192, 3200), (40000, 302)])
 def test_conv_corr_many_tiles_per_wave(slayer, shape, K):
