@@ -112,7 +112,7 @@ class Workload:
 class Cuba(Workload):
     name = 'CUBA conv-layer neuron tensor fwd+bwd'
     shape = (32, 16, 32, 32, 300)
-    ops = [('li_fwd_current', 'stream_kernel<LiFwd>', 8), ('li_fwd_voltage', 'stream_kernel<LiFwd>', 8),
+    ops = [('li_fwd_current', 'stream_kernel_duo<LiFwd>', 8), ('li_fwd_voltage', 'stream_kernel_duo<LiFwd>', 8),
            ('spike_fwd', 'spike_fwd_kernel', 8), ('spike_bwd', 'spike_bwd_kernel', 12),
            ('li_bwd_voltage', 'li_bwd_scan_kernel', 12), ('li_bwd_current', 'li_bwd_scan_kernel', 12)]
     w, thr = 64, 1.0
@@ -176,7 +176,7 @@ class CubaFused(Cuba):
     """Same tensor and parameters as `cuba`, run through the fused kernels: the intermediates are written
     (autograd needs them) but never re-read by a separate operator.  Reported against its own byte count."""
     name = 'CUBA conv-layer neuron tensor fwd+bwd, fused kernels'
-    ops = [('cuba_fwd', 'stream_kernel<CubaFwd>', 16), ('cuba_bwd', 'stream_kernel<CubaBwd>', 16)]
+    ops = [('cuba_fwd', 'stream_kernel_staged<CubaFwd>', 16), ('cuba_bwd', 'cuba_bwd_scan_kernel', 16)]
 
     def __init__(self, dev):
         super().__init__(dev)
@@ -193,7 +193,7 @@ class CubaFused(Cuba):
 
 class CubaFusedLean(Cuba):
     name = 'CUBA neuron fwd+bwd, fused kernels without the current trace (no decay gradients)'
-    ops = [('cuba_fwd', 'stream_kernel<CubaFwd>', 12), ('cuba_bwd', 'stream_kernel<CubaBwd>', 12)]
+    ops = [('cuba_fwd', 'stream_kernel_staged<CubaFwd>', 12), ('cuba_bwd', 'cuba_bwd_scan_kernel', 12)]
 
     def __init__(self, dev):
         super().__init__(dev)
@@ -210,7 +210,7 @@ class CubaFusedLean(Cuba):
 
 class CubaInference(Cuba):
     name = 'CUBA neuron forward, spikes only (inference)'
-    ops = [('cuba_fwd', 'stream_kernel<CubaFwd>', 8)]
+    ops = [('cuba_fwd', 'stream_kernel_staged<CubaFwd>', 8)]
 
     def __init__(self, dev):
         super().__init__(dev)
@@ -226,7 +226,7 @@ class CubaInference(Cuba):
 class CubaFwdSmall(Workload):
     name = 'CUBA LIF dynamics forward only (latency-bound: 512 neurons)'
     shape = (4, 128, 200)
-    ops = [('li_fwd_current', 'stream_kernel<LiFwd>', 8), ('li_fwd_voltage', 'stream_kernel<LiFwd>', 8)]
+    ops = [('li_fwd_current', 'stream_kernel_duo<LiFwd>', 8), ('li_fwd_voltage', 'stream_kernel_duo<LiFwd>', 8)]
     note = 'w_scale=64, scalar decays 1024 / 128, threshold 1.25, input Bernoulli(0.05) x N(0,1)'
 
     def __init__(self, dev):
@@ -252,10 +252,10 @@ class CubaFwdSmall(Workload):
 class Alif(Workload):
     name = 'ALIF adaptive-threshold dynamics fwd+bwd'
     shape = (64, 512, 1000)
-    ops = [('li_fwd_current', 'stream_kernel<LiFwd>', 8), ('li_fwd_voltage', 'stream_kernel<LiFwd>', 8),
-           ('ath_fwd', 'stream_kernel<AthFwd>', 12), ('threshold_add', 'torch add (outside the API)', 12),
+    ops = [('li_fwd_current', 'stream_kernel_duo<LiFwd>', 8), ('li_fwd_voltage', 'stream_kernel_duo<LiFwd>', 8),
+           ('ath_fwd', 'stream_kernel_duo<AthFwd>', 12), ('threshold_add', 'torch add (outside the API)', 12),
            ('spike_fwd', 'spike_fwd_kernel', 12), ('spike_bwd', 'spike_bwd_kernel', 16),
-           ('li_bwd_voltage', 'stream_kernel<LiBwd>', 12), ('li_bwd_current', 'stream_kernel<LiBwd>', 12)]
+           ('li_bwd_voltage', 'li_bwd_scan_kernel', 12), ('li_bwd_current', 'li_bwd_scan_kernel', 12)]
     note = 'w_scale=64, four per-channel decay vectors uniform over [0,4096), th0 1.0, step 0.5'
 
     def __init__(self, dev):
@@ -307,7 +307,7 @@ class Alif(Workload):
 
 class AlifFused(Alif):
     name = 'ALIF adaptive-threshold dynamics fwd+bwd, fused kernels'
-    ops = [('alif_fwd', 'stream_kernel<AlifFwd>', 20), ('alif_bwd', 'stream_kernel<AlifBwd>', 20)]
+    ops = [('alif_fwd', 'stream_kernel_duo<AlifFwd>', 20), ('alif_bwd', 'cuba_bwd_scan_kernel<THETA>', 20)]
 
     def __init__(self, dev):
         super().__init__(dev)
@@ -326,7 +326,7 @@ class AlifFused(Alif):
 
 class AlifFusedLean(Alif):
     name = 'ALIF fwd+bwd, fused kernels without the current trace (no decay gradients)'
-    ops = [('alif_fwd', 'stream_kernel<AlifFwd>', 16), ('alif_bwd', 'stream_kernel<AlifBwd>', 16)]
+    ops = [('alif_fwd', 'stream_kernel_duo<AlifFwd>', 16), ('alif_bwd', 'cuba_bwd_scan_kernel<THETA>', 16)]
 
     def __init__(self, dev):
         super().__init__(dev)
@@ -346,8 +346,8 @@ class AlifFusedLean(Alif):
 class Rf(Workload):
     name = 'Resonator (RF) dynamics fwd+bwd'
     shape = (64, 1024, 2000)
-    ops = [('res_fwd', 'stream_kernel<ResFwd>', 16), ('cspike_fwd', 'cspike_fwd_kernel', 12),
-           ('cspike_bwd', 'cspike_bwd_kernel', 20), ('res_bwd', 'stream_kernel<ResBwd>', 24)]
+    ops = [('res_fwd', 'stream_kernel_duo<ResFwd>', 16), ('cspike_fwd', 'cspike_fwd_kernel', 12),
+           ('cspike_bwd', 'cspike_bwd_kernel', 20), ('res_bwd', 'res_bwd_scan_kernel', 24)]
     note = 'w_scale=64, per-channel decay uniform over [0,4096), frequency uniform over [5,50] Hz at 1 ms'
 
     def __init__(self, dev):
@@ -392,7 +392,7 @@ class Rf(Workload):
 
 class RfFused(Rf):
     name = 'Resonator (RF) dynamics fwd+bwd, fused kernels'
-    ops = [('rf_fwd', 'stream_kernel<RfFwd>', 20), ('rf_bwd', 'stream_kernel<RfBwd>', 20)]
+    ops = [('rf_fwd', 'stream_kernel_duo<RfFwd>', 20), ('rf_bwd', 'res_bwd_scan_kernel<SURR>', 20)]
 
     def __init__(self, dev):
         super().__init__(dev)
@@ -422,7 +422,7 @@ class RfFusedLean(RfFused):
 
 class RfInference(Rf):
     name = 'Resonator (RF) neuron forward, spikes only (inference)'
-    ops = [('rf_fwd', 'stream_kernel<RfFwd>', 12)]
+    ops = [('rf_fwd', 'stream_kernel_duo<RfFwd>', 12)]
 
     def __init__(self, dev):
         super().__init__(dev)
@@ -439,11 +439,11 @@ class RfInference(Rf):
 class Synapse(Workload):
     name = 'SLAYER synapse stack (conv K=64 -> per-channel shift -> CUBA) fwd+bwd'
     shape = (32, 256, 1500)
-    ops = [('conv', 'conv_kernel', 8), ('shift', 'shift_kernel', 8),
-           ('li_fwd_current', 'stream_kernel<LiFwd>', 8), ('li_fwd_voltage', 'stream_kernel<LiFwd>', 8),
+    ops = [('conv', 'conv_mfma_split_kernel<64,conv>', 8), ('shift', 'shift_kernel', 8),
+           ('li_fwd_current', 'stream_kernel_duo<LiFwd>', 8), ('li_fwd_voltage', 'stream_kernel_duo<LiFwd>', 8),
            ('spike_fwd', 'spike_fwd_kernel', 8), ('spike_bwd', 'spike_bwd_kernel', 12),
-           ('li_bwd_voltage', 'stream_kernel<LiBwd>', 12), ('li_bwd_current', 'stream_kernel<LiBwd>', 12),
-           ('shift_back', 'shift_kernel', 8), ('corr', 'conv_kernel<corr>', 8)]
+           ('li_bwd_voltage', 'li_bwd_scan_kernel', 12), ('li_bwd_current', 'li_bwd_scan_kernel', 12),
+           ('shift_back', 'shift_kernel', 8), ('corr', 'conv_mfma_split_kernel<64,corr>', 8)]
     note = 'alpha kernel tau 4, K=64, delays uniform over [0,32), CUBA scalar decays 1024/128, threshold 1.25'
 
     def __init__(self, dev):
@@ -500,8 +500,8 @@ class Synapse(Workload):
 
 class SynapseFused(Synapse):
     name = 'SLAYER synapse stack (conv K=64 -> per-channel shift -> CUBA) fwd+bwd, fused CUBA kernels without the current trace'
-    ops = [('conv', 'conv_kernel', 8), ('shift', 'shift_kernel', 8), ('cuba_fwd', 'stream_kernel<CubaFwd>', 12),
-           ('cuba_bwd', 'stream_kernel<CubaBwd>', 12), ('shift_back', 'shift_kernel', 8), ('corr', 'conv_kernel<corr>', 8)]
+    ops = [('conv', 'conv_mfma_split_kernel<64,conv>', 8), ('shift', 'shift_kernel', 8), ('cuba_fwd', 'stream_kernel_staged<CubaFwd>', 12),
+           ('cuba_bwd', 'cuba_bwd_scan_kernel', 12), ('shift_back', 'shift_kernel', 8), ('corr', 'conv_mfma_split_kernel<64,corr>', 8)]
 
     def __init__(self, dev):
         super().__init__(dev)
@@ -527,8 +527,8 @@ class SynapseFused(Synapse):
 class SynapseFolded(SynapseFused):
     name = ('SLAYER synapse stack (conv K=64 -> per-channel shift -> CUBA) fwd+bwd, the shift folded into the fused '
             'CUBA kernels (read of the input, store of its gradient)')
-    ops = [('conv', 'conv_kernel', 8), ('cuba_fwd', 'stream_kernel<CubaFwd>', 12),
-           ('cuba_bwd', 'stream_kernel<CubaBwd>', 12), ('corr', 'conv_kernel<corr>', 8)]
+    ops = [('conv', 'conv_mfma_split_kernel<64,conv>', 8), ('cuba_fwd', 'stream_kernel_staged<CubaFwd>', 12),
+           ('cuba_bwd', 'cuba_bwd_scan_kernel', 12), ('corr', 'conv_mfma_split_kernel<64,corr>', 8)]
 
     def __init__(self, dev):
         super().__init__(dev)
@@ -552,8 +552,8 @@ class SynapseFolded(SynapseFused):
 
 class SynapseDelayGrad(SynapseFused):
     name = 'SLAYER synapse stack with a learnable delay (conv K=64 -> Delay -> fused CUBA) fwd+bwd incl. the delay gradient'
-    ops = [('conv', 'conv_kernel', 8), ('shift', 'shift_kernel', 8), ('cuba_fwd', 'stream_kernel<CubaFwd>', 12),
-           ('cuba_bwd', 'stream_kernel<CubaBwd>', 12), ('delay_bwd', 'delay_bwd_kernel', 12), ('corr', 'conv_kernel<corr>', 8)]
+    ops = [('conv', 'conv_mfma_split_kernel<64,conv>', 8), ('shift', 'shift_kernel', 8), ('cuba_fwd', 'stream_kernel_staged<CubaFwd>', 12),
+           ('cuba_bwd', 'cuba_bwd_scan_kernel', 12), ('delay_bwd', 'delay_bwd_kernel', 12), ('corr', 'conv_mfma_split_kernel<64,corr>', 8)]
 
     def step(self, t):
         import importlib
@@ -580,7 +580,7 @@ class DenseSynapse(Workload):
     and back around its kernel; `torch.matmul` does not.)"""
     name = 'Dense synapse (batched GEMM) -> fused CUBA neuron, forward'
     shape = (32, 256, 1500)
-    ops = [('dense_gemm', 'torch.matmul (GEMM, outside this library)', 8), ('cuba_fwd', 'stream_kernel<CubaFwd>', 8)]
+    ops = [('dense_gemm', 'torch.matmul (GEMM, outside this library)', 8), ('cuba_fwd', 'stream_kernel_staged<CubaFwd>', 8)]
     note = '256 -> 256 neurons, input Bernoulli(0.03), weights N(0, 0.3) on the 2/64 grid, CUBA decays 1024/128, threshold 1.25'
 
     def __init__(self, dev):

@@ -136,6 +136,8 @@ def _find_range_word():
 
 
 def _range_raised():
+    if _range_policy == 'ignore':           # nobody is looking: the flag stays up until someone lowers it
+        return
     clear_range_flag()
     msg = ('a fixed-point state of a slayer kernel came within a factor of two of the 32-bit range (or a decay '
            'multiplier lies beyond +-8191): results since the last check may differ from a 64-bit evaluation. '
@@ -149,7 +151,8 @@ def _range_raised():
 
 def range_policy(mode=None):
     """What a raised range flag does when an operator call or ``range_check`` sees it: ``'raise'`` (default,
-    OverflowError), ``'warn'`` (RuntimeWarning) or ``'ignore'``.  Returns the mode that was set before."""
+    OverflowError), ``'warn'`` (RuntimeWarning) or ``'ignore'`` (nothing happens and the flag stays up until
+    ``clear_range_flag``).  Reporting lowers the flag.  Returns the mode that was set before."""
     global _range_policy
     before = _range_policy
     if mode is not None:

@@ -62,6 +62,14 @@ int main(void) {
             if ((float)y >= threshold * (float)W) y = 0;
         }
     }
+    /* this workload stays far below 2^30: the range flag is down after the launches have completed */
+    int raised = -1;
+    rc = slayer_range_status(&raised, 0);
+    if (rc != 0 || raised != 0 || slayer_range_word() == NULL) {
+        fprintf(stderr, "range flag: status %d (%s), raised %d, word %p\n", rc, slayer_error_string(rc), raised,
+                (const void*)slayer_range_word());
+        ++bad;
+    }
     /* an argument error comes back as a code, nothing is launched */
     if (slayer_li_fwd(d_out, d_in, d_decay, d_state, 1.0, W, M, 4, C, 1, T, (void*)stream) != SLAYER_EINVAL) ++bad;
     hipFree(d_in); hipFree(d_out); hipFree(d_spk); hipFree(d_decay); hipFree(d_state);

@@ -9,7 +9,7 @@ import pytest
 import torch
 
 from oracle import slayer_oracle as O
-from tests.util import assert_exact, assert_rel, assert_same_gradient, assert_scale, dev, SCAN_MIN
+from tests.util import assert_exact, assert_rel, assert_same_gradient, assert_scale, assert_sum, dev, li_bwd_f64, SCAN_MIN
 
 pytestmark = pytest.mark.gpu
 
@@ -114,6 +114,38 @@ def test_alif_full_size(slayer):
                         A.persistent_th_state(t1[..., -1], s1, 0.5).contiguous(), dg['th'], 0.5, 1.0, 64)
     assert torch.equal(torch.cat([t1, t2], -1), th)
     assert torch.equal(torch.cat([r1, r2], -1), ref)
+    del t1, t2, r1, r2
+    # backward at full size (spike/spike.py:10-23, neuron/dynamics/leaky_integrator.py:234-259 in the reference):
+    # surrogate against the tensor threshold, voltage recurrence, current recurrence -- by the three operators and
+    # by the one fused kernel, both against the oracle on the slab, elementwise
+    g = gpu_randn(shape, 23)
+    theta = th + ref
+    S = slayer.spike.spike
+    g_vol = S._bwd(g, vol, theta, 0.0, 1.0, 1.0, False)
+    g_cur, gd_v = D.leaky_integrator._bwd(g_vol, vol, dg['v'], True)
+    g_x, gd_i = D.leaky_integrator._bwd(g_cur, cur, dg['i'], True)
+    f_x, f_gi, f_gv = D.alif_fused._bwd(g, vol, theta, cur, dg['i'], dg['v'], 1.0, 1.0, False, True)
+    assert torch.equal(f_x, g_x), 'fused ALIF backward differs from the operator chain'
+    gs = g[sl].cpu()
+    o_gv = O.spike_bwd(gs, r_vol, r_th + r_ref, 1.0, 1.0)
+    o_gc, _ = O.li_bwd(o_gv, r_vol, d['v'])
+    o_gx, _ = O.li_bwd(o_gc, r_cur, d['i'])
+    assert_rel(g_vol[sl], o_gv, 'spike surrogate slab')
+    assert_scale(g_cur[sl], o_gc, 'voltage gradient slab')
+    assert_scale(g_x[sl], o_gx, 'input gradient slab')
+    # element by element: each recurrence in float64 on the very gradient the kernel read, against the sum of the
+    # magnitudes of the terms that make up the element
+    T = shape[-1]
+    for name, got, fed, dec in (('voltage', g_cur, g_vol, d['v']), ('input', g_x, g_cur, d['i'])):
+        a = (1 - dec / 4096).repeat(2)                   # rows of the slab: 2 batch entries x 512 channels
+        want, mag = li_bwd_f64(fed[sl].reshape(-1, T), a)
+        assert_sum(got[sl].reshape(-1, T), want, mag, f'{name} gradient slab, elementwise')
+    # decay gradients: float64 sums of the GPU's own products, held to 1e-5 of the sum of the terms' magnitudes
+    for name, got, fused, grad_next, trace in (('voltage', gd_v, f_gv, g_cur, vol), ('current', gd_i, f_gi, g_x, cur)):
+        terms = grad_next[..., 1:].double() * trace[..., :-1].double()
+        want, mag = terms.sum(dim=(0, 2)), terms.abs().sum(dim=(0, 2))
+        assert_sum(got, want, mag, f'grad {name} decay')
+        assert_sum(fused, want, mag, f'fused grad {name} decay')
 
 
 def test_rf_full_size(slayer):

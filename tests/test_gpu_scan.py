@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from oracle import slayer_oracle as O
-from tests.util import dev, sparse_input, assert_rel, assert_scale, seed_of, SCAN_MIN
+from tests.util import dev, sparse_input, assert_rel, assert_scale, assert_sum, li_bwd_f64, seed_of, SCAN_MIN
 
 pytestmark = pytest.mark.gpu
 
@@ -57,6 +57,8 @@ def test_li_bwd_scan_against_oracle_and_sequential_kernel(slayer, shape, nd):
         acc = a * acc + go[:, t:t + 1]
         ref[:, t:t + 1] = acc
     assert_scale(gi.reshape(-1, shape[-1])[pick.to(dev())], ref, 'scan vs step-by-step recurrence (float32)')
+    want64, mag64 = li_bwd_f64(go, a.float())          # every element against the magnitudes of its own terms
+    assert_sum(gi.reshape(-1, shape[-1])[pick.to(dev())], want64, mag64, 'scan vs float64 recurrence, elementwise')
     # decay gradient in float64 from the sequential result
     prod = seq.double().cpu()[..., 1:] * y.double()[..., :-1]
     want = prod.sum().reshape(1) if nd == 1 else prod.reshape(shape[0], nd, -1).sum(dim=(0, 2))

@@ -63,6 +63,41 @@ def assert_scale(gpu, ref, what='', rel=REL):
         raise AssertionError(f'{what}: max abs err {err:.3e} > {rel} * {scale:.3e}')
 
 
+def assert_sum(gpu, ref, magnitude, what='', rel=REL):
+    """A parameter gradient is a sum of very many terms of both signs: |gpu - ref| <= rel * (sum of the terms'
+    magnitudes), per parameter.  ``ref`` is the sum and ``magnitude`` the sum of absolute values, both in float64.
+    (Relative to the result itself no summation order, the reference's included, can promise anything once the
+    terms cancel.)"""
+    g = gpu.detach().cpu().double().reshape(-1)
+    r = ref.detach().cpu().double().reshape(-1)
+    m = magnitude.detach().cpu().double().reshape(-1)
+    assert g.shape == r.shape == m.shape, (what, g.shape, r.shape, m.shape)
+    err = (g - r).abs()
+    bad = err > rel * m
+    if bool(bad.any()):
+        i = int(torch.argmax(err / m.clamp_min(1e-300)))
+        raise AssertionError(f'{what}: |{g[i].item()!r} - {r[i].item()!r}| = {err[i].item():.3e} > {rel} * '
+                             f'{m[i].item():.3e} (parameter {i})')
+
+
+def li_bwd_f64(grad_out, a):
+    """g[t] = a g[t+1] + grad_out[t] on rows [R, T] in float64 (neuron/dynamics/leaky_integrator.py:234-259 in the
+    reference, a = 1 - decay / 4096 per row), and next to it the same recurrence on magnitudes,
+    B[t] = |a| B[t+1] + |grad_out[t]|: the sum of the magnitudes of the terms a^k grad_out[t+k] that make up g[t].
+    A float32 evaluation in any order is off by a few ulp of B[t], not of g[t]: where the terms cancel, the bar for
+    an element is rel * B[t] (``assert_sum``), which is rel * |g[t]| wherever they do not."""
+    go = grad_out.detach().cpu().double()
+    a = a.detach().cpu().double().reshape(-1, 1)
+    g, bound = torch.zeros_like(go), torch.zeros_like(go)
+    acc = torch.zeros(go.shape[0], 1, dtype=torch.float64)
+    mag = torch.zeros_like(acc)
+    for t in range(go.shape[1] - 1, -1, -1):
+        acc = a * acc + go[:, t:t + 1]
+        mag = a.abs() * mag + go[:, t:t + 1].abs()
+        g[:, t:t + 1], bound[:, t:t + 1] = acc, mag
+    return g, bound
+
+
 def assert_same_gradient(a, b, what=''):
     """Two evaluations of the same float gradient on the GPU: bit-identical while both are step-by-step
     (small tensors), within 1e-5 of the scale once the scan kernels take over."""
