@@ -573,6 +573,141 @@ class SynapseDelayGrad(SynapseFused):
         return spk, g_x, g_delay
 
 
+class BlockTail(SynapseFused):
+    """The tail of a SLAYER block with a trained axonal delay (block/base.py:549-553, axon/delay.py:178-221 in the
+    reference): fused CUBA neuron -> learnable per-channel Delay, forward and backward including the delay's
+    gradient, by separate operators: the Delay is a shift after the neuron, its backward pass one kernel that
+    shifts the gradient back and sums grad * (out[t-1] - out[t]) / Ts per channel."""
+    name = 'Block tail: fused CUBA -> learnable Delay (separate kernels), fwd+bwd incl. the delay gradient'
+    ops = [('cuba_fwd', 'stream_kernel_staged<CubaFwd>', 8), ('delay', 'shift_kernel', 8),
+           ('delay_bwd', 'delay_bwd_kernel', 12), ('cuba_bwd', 'cuba_bwd_scan_kernel', 12)]
+
+    def __init__(self, dev):
+        super().__init__(dev)
+        import importlib
+        self.AX = importlib.import_module('lava_dl_amd.slayer.axon.delay')
+
+    def step(self, t):
+        with t('cuba_fwd'):
+            _, vol, spk = self.F._fwd(self.x, self.d_i, self.d_v, self.zero, self.zero, 64, 1.25, False, 1, True)
+        with t('delay'):
+            out = self.shift(spk, self.delay, 1)
+        with t('delay_bwd'):
+            g_spk, g_delay = self.AX._delay_bwd(self.g, out, self.delay, 1)
+        with t('cuba_bwd'):
+            g_x, _, _ = self.F._bwd(g_spk, vol, None, self.d_i, self.d_v, 1.25, 1.0, 1.0, False, False)
+        return out, g_x, g_delay
+
+    def cpu_step(self, n, sl=None):
+        from oracle import slayer_oracle as O
+        c, zero = self.cpu, torch.tensor([0.0])
+        x, g, delay = c['x'][:n], c['g'][:n], c['delay']
+        if sl is not None:
+            x, g, delay = x[:, sl], g[:, sl], delay[sl]
+        cur = O.li_fwd(x, c['d_i'], zero, 64)
+        vol = O.li_fwd(cur, c['d_v'], zero, 64, 1.25)
+        out = O.shift(O.spike_fwd(vol, 1.25), delay, 1)
+        g_vol = O.spike_bwd(O.shift(g, -delay, 1), vol, 1.25, 1.0, 1.0)
+        g_cur, _ = O.li_bwd(g_vol, vol, c['d_v'])
+        return out, O.li_bwd(g_cur, cur, c['d_i'])[0]
+
+
+class BlockTailFolded(BlockTail):
+    """The same block tail with the Delay folded into the neuron's two kernels: the forward kernel stores its spikes
+    through the delay, the backward scan reads the gradient back through it and, with the delayed spikes as one more
+    input, leaves the delay gradient's per-row sums on the way.  Same results (spikes and input gradient bit for
+    bit)."""
+    name = 'Block tail: fused CUBA with the learnable Delay folded into its kernels, fwd+bwd incl. the delay gradient'
+    ops = [('cuba_fwd', 'stream_kernel_staged<CubaFwd,SHIFT>', 8), ('cuba_bwd', 'cuba_bwd_scan_kernel<SHIFT,DELAY>', 16)]
+
+    def __init__(self, dev):
+        super().__init__(dev)
+        from lava_dl_amd.slayer.neuron.dynamics import delays
+        self.D = delays
+        self.delays = delays.Delays(output_delay=self.delay)
+
+    def step(self, t):
+        with t('cuba_fwd'):
+            _, vol, out = self.F._fwd(self.x, self.d_i, self.d_v, self.zero, self.zero, 64, 1.25, False, 1, True,
+                                      folded=self.D.fold(self.delays, self.x))
+        with t('cuba_bwd'):
+            folded = self.D.fold(self.delays, self.g, forward=False, delayed_spikes=out)
+            g_x, _, _ = self.F._bwd(self.g, vol, None, self.d_i, self.d_v, 1.25, 1.0, 1.0, False, False, folded=folded)
+            g_delay = folded.grad_sum
+        return out, g_x, g_delay
+
+
+class ConvSynapse(Cuba):
+    """The convolution synapse that produces config[1]'s tensor (synapse/layer.py:297-323 in the reference: F.conv3d
+    with a 3x3x1 kernel on NCHWT spikes), feeding the fused CUBA neuron, forward and backward down to the gradient of
+    the input spikes.  The synapse kernel works on the time-innermost layout as it is; the neuron reads its output in
+    place.  Weights are multiples of 1/64 (quantised, as a SLAYER synapse's are), so the weighted spikes are exact
+    and the forward parity check stays bit for bit.  Bytes per neuron-timestep of the output tensor."""
+    name = 'Conv synapse (3x3, 8 -> 16 channels) -> fused CUBA neuron, fwd+bwd (input gradient)'
+    ops = [('conv_synapse', 'synapse_conv_kernel', 6), ('cuba_fwd', 'stream_kernel_staged<CubaFwd>', 16),
+           ('cuba_bwd', 'cuba_bwd_scan_kernel', 16), ('conv_synapse_bwd', 'synapse_conv_kernel', 6)]
+    note = Cuba.note + '; input spikes Bernoulli(0.05) on 8 channels, weights round(N(0, 0.3) * 64) / 64'
+    in_channels = 8
+
+    def __init__(self, dev):
+        super().__init__(dev)
+        import importlib
+        g = self.gen
+        self.put(s=(torch.rand((self.shape[0], self.in_channels) + self.shape[2:], generator=g) < 0.05).float(),
+                 wgt=(torch.randn(self.shape[1], self.in_channels, 3, 3, 1, generator=g) * 0.3 * 64).round() / 64)
+        self.syn = importlib.import_module('lava_dl_amd.slayer.synapse.layer')
+        self.F = importlib.import_module('lava_dl_amd.slayer.neuron.dynamics.cuba_fused')
+        self.w4 = self.wgt[..., 0].contiguous()
+        self.w4_back = self.wgt[..., 0].flip(2, 3).transpose(0, 1).contiguous()
+
+    def synapse(self, s):
+        return self.syn._launch(s, self.w4, (1, 1), (1, 1), (1, 1))
+
+    def synapse_back(self, g):
+        return self.syn._launch(g, self.w4_back, (1, 1), (1, 1), (1, 1))
+
+    def step(self, t):
+        with t('conv_synapse'):
+            z = self.synapse(self.s)
+        with t('cuba_fwd'):
+            cur, vol, spk = self.F._fwd(z, self.d_i, self.d_v, self.zero, self.zero, self.w, self.thr, False, 1)
+        with t('cuba_bwd'):
+            g_z, _, _ = self.F._bwd(self.g, vol, cur, self.d_i, self.d_v, self.thr, 1.0, 1.0, False)
+        with t('conv_synapse_bwd'):
+            g_s = self.synapse_back(g_z)
+        return spk, g_s
+
+    def cpu_step(self, n, sl=None):
+        from oracle import slayer_oracle as O
+        c, zero = self.cpu, torch.tensor([0.0])
+        s, g, wgt, d_i, d_v = c['s'][:n], c['g'][:n], c['wgt'], c['d_i'], c['d_v']
+        z = O.conv_synapse(s, wgt, (1, 1), (1, 1), (1, 1))
+        cur = O.li_fwd(z, d_i, zero, self.w)
+        vol = O.li_fwd(cur, d_v, zero, self.w, self.thr)
+        spk = O.spike_fwd(vol, self.thr)
+        g_vol = O.spike_bwd(g, vol, self.thr, 1.0, 1.0)
+        g_cur, _ = O.li_bwd(g_vol, vol, d_v)
+        g_z, _ = O.li_bwd(g_cur, cur, d_i)
+        g_s = torch.nn.grad.conv3d_input(s.shape, wgt.double(), g_z.double(), (1, 1, 1), (1, 1, 0)).float()
+        return (spk if sl is None else spk[:, sl]), None if sl is not None else g_s
+
+    parity_slab = (1, slice(0, 16))
+
+
+class ConvSynapseLibrary(ConvSynapse):
+    """The same stack with the reference's own call for the synapse: the library convolution transposes the tensor to
+    channels-last and back around its kernel (three extra passes each way)."""
+    name = 'Conv synapse by F.conv3d (library kernel + layout transposes) -> fused CUBA neuron, fwd+bwd (input gradient)'
+    ops = [('conv_synapse', 'F.conv3d: library conv + batched_transpose x3', 6), ('cuba_fwd', 'stream_kernel_staged<CubaFwd>', 16),
+           ('cuba_bwd', 'cuba_bwd_scan_kernel', 16), ('conv_synapse_bwd', 'conv3d_input: library conv + transposes', 6)]
+
+    def synapse(self, s):
+        return torch.nn.functional.conv3d(s, self.wgt, None, (1, 1, 1), (1, 1, 0))
+
+    def synapse_back(self, g):
+        return torch.nn.grad.conv3d_input(self.s.shape, self.wgt, g, (1, 1, 1), (1, 1, 0))
+
+
 class DenseSynapse(Workload):
     """Dense synapse (the reference's 1x1x1 conv3d over [N, C, 1, 1, T], synapse/layer.py:144-175, written as the
     batched GEMM it is) feeding the fused CUBA kernel, forward only: the kernel list of this workload shows what runs
@@ -612,7 +747,9 @@ class DenseSynapse(Workload):
     parity_slab = (1, slice(32, 64))
 
 
-WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fused_lean': CubaFusedLean, 'cuba_inference': CubaInference, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'alif_fused': AlifFused, 'alif_fused_lean': AlifFusedLean, 'rf': Rf, 'rf_fused': RfFused, 'rf_fused_lean': RfFusedLean, 'rf_inference': RfInference, 'synapse': Synapse, 'synapse_fused': SynapseFused, 'synapse_folded': SynapseFolded, 'synapse_delay_grad': SynapseDelayGrad, 'dense_synapse': DenseSynapse}
+WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fused_lean': CubaFusedLean, 'cuba_inference': CubaInference, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'alif_fused': AlifFused, 'alif_fused_lean': AlifFusedLean, 'rf': Rf, 'rf_fused': RfFused, 'rf_fused_lean': RfFusedLean, 'rf_inference': RfInference, 'synapse': Synapse, 'synapse_fused': SynapseFused, 'synapse_folded': SynapseFolded, 'synapse_delay_grad': SynapseDelayGrad, 'block_tail': BlockTail, 'block_tail_folded': BlockTailFolded,
+             'conv_synapse': ConvSynapse, 'conv_synapse_library': ConvSynapseLibrary,
+             'dense_synapse': DenseSynapse}
 
 
 def cpu_baseline(job, budget_s=20.0):
@@ -694,7 +831,8 @@ def timed_median(job, iters, warmup):
 # The other benchmark configurations, reported next to the headline in `other_configs` (unfused = the op
 # sequence of the configuration, then the fused forms with their own smaller byte counts).
 OTHER = ['cuba_fwd_small', 'cuba_fused', 'cuba_fused_lean', 'alif', 'alif_fused', 'alif_fused_lean', 'rf', 'rf_fused',
-         'synapse', 'synapse_fused', 'synapse_folded']
+         'synapse', 'synapse_fused', 'synapse_folded', 'block_tail', 'block_tail_folded',
+         'conv_synapse', 'conv_synapse_library']
 
 
 def other_configs(dev, iters):

@@ -72,6 +72,14 @@ typedef struct slayer_delays {
     int64_t in_steps;        /* whole steps added to every neuron's input shift */
     int64_t out_steps;       /* whole steps added to every neuron's output delay (step_delay: 1) */
     float sampling_time;     /* divides the table entries; must not be 0 when a table is given */
+    /* backward only, all three or none: the gradient of out_delay as the learnable Delay computes it
+     * (axon/delay.py:201-221): grad_out_delay[j] = sum over the batch and t of
+     * grad_spikes[t] * (delayed_spikes[t-1] - delayed_spikes[t]) / sampling_time for neuron j of a batch element.
+     * Tensors of 2^20 elements and more get it from the backward scan itself, which reads the gradient anyway (one more
+     * tensor read instead of a pass of its own over two); smaller ones from slayer_delay_bwd, launched inside. */
+    const float *delayed_spikes; /* M*T floats: the delayed spike tensor the forward pass stored */
+    float *grad_out_delay;       /* neurons_per_batch floats */
+    float *grad_workspace;       /* M + 64 * neurons_per_batch floats of scratch */
 } slayer_delays;
 
 /* Text for a return code of this library (hipGetErrorString for positive codes). */
@@ -296,6 +304,22 @@ int slayer_conv(float *out, const float *in, const float *filt, int64_t K, float
 int slayer_corr(float *out, const float *in, const float *filt, int64_t K, float sampling_time,
                 int64_t M, int64_t T, void *stream);
 
+/* ---- convolution synapse ------------------------------------------------------------------ */
+
+/* Replaces the F.conv3d call of the convolution synapse (synapse/layer.py:297-323: a kernel of (kh, kw, 1) over
+ * [N, C, H, W, T], no bias, one group) for time-innermost tensors, without leaving that layout:
+ * out[n][co][ho][wo][t] = sum over ci, y, x of weight[co][ci][y][x] *
+ *                         in[n][ci][ho * stride_h + y * dil_h - pad_h][wo * stride_w + x * dil_w - pad_w][t]
+ * (zero outside the image), Ho = (H + 2 pad_h - dil_h (kh - 1) - 1) / stride_h + 1, Wo likewise; weight is
+ * [Co][Ci][kh][kw] (the reference's [Co][Ci][kh][kw][1]).  float32 operands and accumulation on the matrix cores.
+ * The gradient of the input is the same call on the gradient with the weights transposed and flipped.
+ * SLAYER_ERANGE for what the kernel does not take (T not a multiple of 4, tensors not 16-byte aligned, a batch entry of
+ * 2 GiB or more, more than about 860 taps Ci * kh * kw): the caller keeps its library convolution for those. */
+int slayer_conv_synapse(float *out, const float *in, const float *weight,
+                        int64_t N, int64_t Ci, int64_t Co, int64_t H, int64_t W, int64_t T,
+                        int64_t kh, int64_t kw, int64_t stride_h, int64_t stride_w,
+                        int64_t pad_h, int64_t pad_w, int64_t dil_h, int64_t dil_w, void *stream);
+
 /* ---- sigma-delta ---------------------------------------------------------------------------- */
 
 /* _DeltaUnit.forward (axon/delta.py:10-66; a python time loop in the reference, no kernel there):
@@ -479,6 +503,48 @@ int slayer_alif_recurrent_fwd(float *spk_out, float *vol_out, float *theta_out,
 int slayer_recurrent_bwd(float *grad_z, const float *grad_spikes, const float *voltage, const float *theta,
                          const float *rec, float spike_threshold, float tau_rho, float scale_rho, int graded,
                          int64_t N, int64_t C, int64_t T, void *stream);
+
+/* The same loops, one launch per time step: for layers of any width up to 16384 neurons (C a multiple of 4).
+ * A step multiplies the weight matrix with the spikes of the previous step for the whole batch (the matrix is read
+ * once per step, on the matrix cores in float32) and runs one neuron step on the result; the launches follow each
+ * other on `stream`.  Same arguments, results and arithmetic as slayer_cuba_recurrent_fwd / slayer_alif_recurrent_fwd
+ * except: `rec` is R itself, [C][C] (row c = the weights that reach neuron c), 16-byte aligned like the *_last
+ * outputs; the feedback of a step is summed in a fixed order of its own (equal bits whenever the sums are exact in
+ * float32, e.g. quantised weights and binary spikes); `workspace` is device memory of at least
+ * slayer_recurrent_steps_workspace(N, C, T, alif) floats, 16-byte aligned, whose contents are undefined afterwards
+ * (time-major copies of the tensors and the states between two steps).
+ * slayer_recurrent_steps_workspace returns the number of floats (with_theta != 0: an ALIF layer), or a negative
+ * error code for sizes the entry points refuse (SLAYER_ERANGE: C % 4 != 0, C > 16384, N * C >= 2^29). */
+int64_t slayer_recurrent_steps_workspace(int64_t N, int64_t C, int64_t T, int with_theta);
+int slayer_cuba_recurrent_steps_fwd(float *spk_out, float *vol_out, float *cur_last_out, float *vol_last_out,
+                                    const float *z, const float *rec,
+                                    const float *i_decay, const float *v_decay,
+                                    const float *i_state, const float *v_state,
+                                    float spike_threshold, int graded, float spike_scale, int w_scale,
+                                    int64_t N, int64_t C, int64_t num_i_decays, int64_t num_v_decays,
+                                    int64_t num_i_states, int64_t num_v_states, int64_t T,
+                                    float *workspace, int64_t workspace_floats, void *stream);
+int slayer_alif_recurrent_steps_fwd(float *spk_out, float *vol_out, float *theta_out,
+                                    float *cur_last_out, float *vol_last_out, float *th_last_out, float *ref_last_out,
+                                    const float *z, const float *rec,
+                                    const float *i_decay, const float *v_decay, const float *th_decay,
+                                    const float *ref_decay,
+                                    const float *i_state, const float *v_state, const float *th_state,
+                                    const float *ref_state,
+                                    float th_step, int64_t th0_scaled, int graded, float spike_scale, int w_scale,
+                                    int64_t N, int64_t C,
+                                    int64_t num_i_decays, int64_t num_v_decays, int64_t num_th_decays,
+                                    int64_t num_ref_decays,
+                                    int64_t num_i_states, int64_t num_v_states, int64_t num_th_states,
+                                    int64_t num_ref_states,
+                                    int64_t T, float *workspace, int64_t workspace_floats, void *stream);
+
+/* slayer_recurrent_bwd one launch per time step (see above); rec_t = R transposed, [C][C], 16-byte aligned:
+ * row c holds the weights that leave neuron c.  Workspace as above (with_theta = theta != NULL). */
+int slayer_recurrent_steps_bwd(float *grad_z, const float *grad_spikes, const float *voltage, const float *theta,
+                               const float *rec_t, float spike_threshold, float tau_rho, float scale_rho, int graded,
+                               int64_t N, int64_t C, int64_t T,
+                               float *workspace, int64_t workspace_floats, void *stream);
 
 /* ---- cross-check implementations (debug mode) ------------------------------------------------ */
 

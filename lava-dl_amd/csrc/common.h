@@ -49,7 +49,27 @@ inline int check_delays(const slayer_delays* d, int64_t M, int64_t npb) {
     if (!d) return 0;
     if (npb <= 0 || (M > 0 && M % npb != 0)) return SLAYER_EINVAL;
     if ((d->in_shift || d->out_delay) && !(d->sampling_time != 0.0f)) return SLAYER_EINVAL;
+    // the delay gradient of a backward pass: all three of its pointers or none, and a sampling time to divide by
+    const int given = (d->delayed_spikes != nullptr) + (d->grad_out_delay != nullptr) + (d->grad_workspace != nullptr);
+    if (given != 0 && given != 3) return SLAYER_ENULL;
+    if (given == 3 && !(d->sampling_time != 0.0f)) return SLAYER_EINVAL;
     return 0;
+}
+
+// After the main kernel of a fused backward pass: the gradient of the output delay, when the caller asked for it.
+// in_scan: the backward scan has left the per-row sums in grad_workspace; else nothing has been summed yet and the
+// stand-alone kernel does the whole job.  (li.hip, shift.hip)
+int launch_reduce_param_grad(float* grad, const float* partial, float* scratch, int64_t M, int64_t npb,
+                             int64_t num_params, hipStream_t stream);
+int launch_zero_fill(float* p, int64_t n, hipStream_t stream);
+inline int finish_delay_gradient(const slayer_delays* d, const float* grad_spikes, bool in_scan, int64_t M, int64_t npb,
+                                 int64_t T, hipStream_t stream) {
+    if (!d || !d->grad_out_delay) return 0;
+    if (M == 0 || T == 0) return launch_zero_fill(d->grad_out_delay, npb, stream);
+    if (in_scan)
+        return launch_reduce_param_grad(d->grad_out_delay, d->grad_workspace, d->grad_workspace + M, M, npb, npb, stream);
+    return slayer_delay_bwd(nullptr, d->grad_out_delay, grad_spikes, d->delayed_spikes, nullptr, 0, d->sampling_time,
+                            d->grad_workspace, M, npb, T, (void*)stream);
 }
 
 }  // namespace slayer

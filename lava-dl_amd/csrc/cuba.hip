@@ -281,12 +281,14 @@ extern "C" int slayer_cuba_bwd(float* grad_in, float* grad_i_decay, float* grad_
     const bool want = grad_i_decay != nullptr;
     if (want && !workspace && M > 0) return SLAYER_ENULL;
     hipStream_t st = (hipStream_t)stream;
+    bool in_scan = false;
     if (M > 0 && T > 0) {
         if (!grad_in || !grad_spikes || !voltage || !i_decay || !v_decay || (want && !current)) return SLAYER_ENULL;
         const Shifts sh = backward_shifts(delays, neurons_per_batch);
         // large tensors: the two recurrences as wave scans over a linear stream
         if (bwd_scan_usable(M, neurons_per_batch, T) && aligned16(grad_in) && aligned16(grad_spikes) &&
             aligned16(voltage) && aligned16(current)) {
+            in_scan = true;
             if (int e = launch_cuba_bwd_scan(grad_in, want ? workspace : nullptr, want ? workspace + M : nullptr,
                                              grad_spikes, voltage, nullptr, want ? current : nullptr, i_decay, v_decay,
                                              spike_threshold, tau_rho, scale_rho, graded != 0, M, neurons_per_batch,
@@ -316,6 +318,7 @@ extern "C" int slayer_cuba_bwd(float* grad_in, float* grad_i_decay, float* grad_
 #undef SLAYER_CUBA_BWD_S
         }
     }
+    if (int e = finish_delay_gradient(delays, grad_spikes, in_scan, M, neurons_per_batch, T, st)) return e;
     if (want) {
         if (M == 0 || T == 0) {
             if (int e = launch_zero_fill(grad_i_decay, num_i_decays, st)) return e;

@@ -246,6 +246,7 @@ extern "C" int slayer_rf_bwd(float* g_re_in, float* g_im_in, float* grad_sin, fl
     const bool want = grad_sin != nullptr;
     if (want && !workspace && M > 0) return SLAYER_ENULL;
     hipStream_t st = (hipStream_t)stream;
+    bool in_scan = false;
     if (M > 0 && T > 0) {
         if (!g_re_in || !g_im_in || !grad_spikes || !re || !im || !sin_decay || !cos_decay) return SLAYER_ENULL;
         const Shifts sh = backward_shifts(delays, neurons_per_batch);
@@ -277,6 +278,7 @@ extern "C" int slayer_rf_bwd(float* g_re_in, float* g_im_in, float* grad_sin, fl
                                             T, delays ? &sh : nullptr, st))
                 return e;
             done = true;
+            in_scan = true;
         }
         if (done) {}
         else if (graded) { if (want) SLAYER_RF_BWD(true, true, true); else SLAYER_RF_BWD(true, false, true); }
@@ -285,6 +287,7 @@ extern "C" int slayer_rf_bwd(float* g_re_in, float* g_im_in, float* grad_sin, fl
 #undef SLAYER_RF_BWD
 #undef SLAYER_RF_BWD_H
     }
+    if (int e = finish_delay_gradient(delays, grad_spikes, in_scan, M, neurons_per_batch, T, st)) return e;
     if (want) {
         if (M == 0 || T == 0) {
             if (int e = launch_zero_fill(grad_sin, num_decays, st)) return e;

@@ -258,6 +258,12 @@ __device__ __forceinline__ float4 scan_tail_place(float4 q, int dd, bool row_end
     return row_end ? p : q;
 }
 
+// The steps of a row's last quad that do not exist (dd of them) hold nothing: a gradient read through a negative
+// shift finds samples of the row at their positions, which must not enter the recurrence.
+__device__ __forceinline__ float4 scan_tail_mask(float4 q, int dd, bool row_end) {
+    return row_end ? make_float4(q.x, dd >= 3 ? 0.f : q.y, dd >= 2 ? 0.f : q.z, dd >= 1 ? 0.f : q.w) : q;
+}
+
 // Zeros at the positions of a shifted output that no sample reaches: [0, k) for k > 0, [T + k, T) for k < 0.
 __device__ __forceinline__ void scan_fill_unreached(__amdgpu_buffer_rsrc_t dst, const int* kout, const ScanSpan& sp,
                                                     int T) {
@@ -268,6 +274,47 @@ __device__ __forceinline__ void scan_fill_unreached(__amdgpu_buffer_rsrc_t dst, 
         for (int j = sp.tid; j < len; j += kScanQuads)
             buf_store1<false>(dst, (rr * T + (k < 0 ? T - len + j : j)) * 4, 0.0f);
     }
+}
+
+// The gradient of a learnable output delay, folded into a scan that reads the gradient of the delayed spikes anyway
+// (axon/delay.py:201-221 in the reference: sum over t of grad[t] * (out[t-1] - out[t]) / Ts on the delayed tensor).
+// A lane's quad of steps t sits at u = t + kf of the delayed tensors (kf: the forward pass's output shift of the
+// row), so the lanes of a row cover u in [kf, T + kf); the delayed spikes are zero outside that range except for the
+// one sample before it (the head a step delay carries over), so two more terms per row complete the sum: u = kf - 1
+// (taken by the lane of the row's first quad) and u = T + kf (by the lane of its last).  All loads are issued for
+// every lane, out of range where they do not apply.
+struct DelayGradQuads { float4 s; float sp, ag, as, asp, bg, bs, bsp; };
+
+__device__ __forceinline__ float scan_load_at(__amdgpu_buffer_rsrc_t src, bool on, int r, int u, int T) {
+    return buf_load1<false>(src, (on && u >= 0 && u < T) ? (r * T + u) * 4 : kOutOfRange);
+}
+// k: the shift the scan reads the gradient through (minus the forward pass's output shift)
+__device__ __forceinline__ void delay_grad_fetch(DelayGradQuads& d, __amdgpu_buffer_rsrc_t src_g, __amdgpu_buffer_rsrc_t src_s,
+                                                 bool in_span, int r, int pos, int QR, int k, int T) {
+    int unused;
+    d.s = scan_load_shifted(src_s, in_span, r, pos, k, T, unused);
+    const int kf = -k, u0 = 4 * pos + kf;
+    d.sp = scan_load_at(src_s, in_span, r, u0 - 1, T);
+    const bool first = in_span && pos == 0 && kf >= 1, last = in_span && pos == QR - 1 && kf < 0;
+    d.ag = scan_load_at(src_g, first, r, kf - 1, T);
+    d.as = scan_load_at(src_s, first, r, kf - 1, T);
+    d.asp = scan_load_at(src_s, first, r, kf - 2, T);
+    d.bg = scan_load_at(src_g, last, r, T + kf, T);
+    d.bs = scan_load_at(src_s, last, r, T + kf, T);
+    d.bsp = scan_load_at(src_s, last, r, T + kf - 1, T);
+}
+// g: the gradient quad in place (zeros where the row has no sample); place: what scan_place needs for d.s
+__device__ __forceinline__ float delay_grad_terms(DelayGradQuads& d, float4 g, int place, float inv_ts) {
+    if (__any(place != 0)) d.s = scan_place(d.s, place);
+    const float f0 = -inv_ts, f1 = inv_ts;
+    float acc = 0.0f;
+    acc = __fmaf_rn(g.x, f0 * d.s.x + f1 * d.sp, acc);
+    acc = __fmaf_rn(g.y, f0 * d.s.y + f1 * d.s.x, acc);
+    acc = __fmaf_rn(g.z, f0 * d.s.z + f1 * d.s.y, acc);
+    acc = __fmaf_rn(g.w, f0 * d.s.w + f1 * d.s.z, acc);
+    acc = __fmaf_rn(d.ag, f0 * d.as + f1 * d.asp, acc);
+    acc = __fmaf_rn(d.bg, f0 * d.bs + f1 * d.bsp, acc);
+    return acc;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -358,7 +405,8 @@ __global__ __launch_bounds__(kScanQuads) void li_bwd_scan_kernel(
 // own with the very arithmetic of li_bwd_scan_kernel -- the input gradient is bit-identical to the spike backward
 // kernel followed by two launches of that kernel.  THETA: the spike threshold is a tensor (threshold + refractory
 // of the adaptive neuron), else the scalar spike_thr.
-template <bool GRADED, bool DECAY_GRAD, bool THETA, bool STREAM, int MODE = 0, int NBUF = 3>
+// DELAY: also leaves the per-row sums of the output delay's gradient (SHIFT forms only, see delay_grad_fetch).
+template <bool GRADED, bool DECAY_GRAD, bool THETA, bool STREAM, int MODE = 0, int NBUF = 3, bool DELAY = false>
 __global__ __launch_bounds__(kScanQuads) void cuba_bwd_scan_kernel(
         float* __restrict__ grad_in, float* __restrict__ partial_i, float* __restrict__ partial_v,
         const float* __restrict__ grad_spikes, const float* __restrict__ voltage, const float* __restrict__ theta,
@@ -366,8 +414,10 @@ __global__ __launch_bounds__(kScanQuads) void cuba_bwd_scan_kernel(
         float spike_thr, float tau, float rho, int64_t M, int T, int QR, int rpg,
         unsigned npb, unsigned per_i, unsigned per_v, Shifts shifts) {
     constexpr bool SHIFT = MODE != 0, ANYT = MODE == 2;
+    static_assert(!DELAY || SHIFT, "the delay gradient belongs to the forms that read the gradient through a delay");
     __shared__ float ai_tab[kScanMaxRows], av_tab[kScanMaxRows];
     __shared__ float sum_i[kScanWaves][kScanMaxRows], sum_v[kScanWaves][kScanMaxRows];
+    __shared__ float sum_d[DELAY ? kScanWaves : 1][DELAY ? kScanMaxRows : 1];
     __shared__ RealStage stage_v, stage_i;
     __shared__ ScanShiftTables shift_tab;
     ScanSpan sp;
@@ -381,10 +431,11 @@ __global__ __launch_bounds__(kScanQuads) void cuba_bwd_scan_kernel(
     const __amdgpu_buffer_rsrc_t src_t = make_rsrc(THETA ? theta + base : nullptr, THETA ? span_bytes : 0u);
     const __amdgpu_buffer_rsrc_t src_c = make_rsrc(DECAY_GRAD ? current + base : nullptr, DECAY_GRAD ? span_bytes : 0u);
     const __amdgpu_buffer_rsrc_t dst = make_rsrc(grad_in + base, span_bytes);
+    const __amdgpu_buffer_rsrc_t src_s = make_rsrc(DELAY ? shifts.delayed + base : nullptr, DELAY ? span_bytes : 0u);
     const float lead = (rho / 2.0f) / tau;
     const float inv_tau = 1.0f / tau;
 
-    struct Quads { float4 g, v, th, c; int dg; };
+    struct Quads { float4 g, v, th, c; int dg; DelayGradQuads dq; };
     // the saved traces (never shifted), then the gradient of the spikes (read through the output delay when SHIFT)
     auto fetch_saved = [&](Quads& x, int q, const ScanCursor& at) {
         const bool in_span = (unsigned)q < (unsigned)nq;
@@ -403,6 +454,8 @@ __global__ __launch_bounds__(kScanQuads) void cuba_bwd_scan_kernel(
     auto fetch_grad = [&](Quads& x, int q, const ScanCursor& at) {
         if (SHIFT) {
             x.g = scan_load_shifted(src_g, (unsigned)q < (unsigned)nq, at.r, at.pos, shift_tab.kin[at.r], T, x.dg);
+            if (DELAY)
+                delay_grad_fetch(x.dq, src_g, src_s, (unsigned)q < (unsigned)nq, at.r, at.pos, QR, shift_tab.kin[at.r], T);
         } else {
             x.g = buf_load4<STREAM>(src_g, (unsigned)q < (unsigned)nq ? q * 16 : kOutOfRange);
             x.dg = 0;
@@ -438,6 +491,8 @@ __global__ __launch_bounds__(kScanQuads) void cuba_bwd_scan_kernel(
     if (SHIFT) scan_shift_tables(shift_tab, shifts, sp, T);
     if (DECAY_GRAD)
         for (int rr = sp.lane; rr < sp.rows; rr += kWave) { sum_i[sp.wv][rr] = 0.0f; sum_v[sp.wv][rr] = 0.0f; }
+    if (DELAY)
+        for (int rr = sp.lane; rr < sp.rows; rr += kWave) sum_d[sp.wv][rr] = 0.0f;
     int parity = (sp.npass - 1) & 1;
     if (sp.tid == 0) { stage_v.carry[parity] = 0.0f; stage_i.carry[parity] = 0.0f; }
     __syncthreads();
@@ -456,6 +511,8 @@ __global__ __launch_bounds__(kScanQuads) void cuba_bwd_scan_kernel(
         const bool active = cur.lq < nq;
         const bool row_end = cur.pos == QR - 1;
         if (SHIFT && __any(x.dg != 0)) x.g = scan_place(x.g, x.dg);      // rare: only where a row begins or ends
+        if (ANYT && dd != 0) x.g = scan_tail_mask(x.g, dd, row_end);
+        if (DELAY) add_to_row(sum_d[sp.wv], delay_grad_terms(x.dq, x.g, x.dg, 1.0f / shifts.ts), sp, cur, QR, active);
         if (ANYT && dd != 0) {
             x.v = scan_tail_place(x.v, dd, row_end);
             if (THETA) x.th = scan_tail_place(x.th, dd, row_end);
@@ -485,11 +542,12 @@ __global__ __launch_bounds__(kScanQuads) void cuba_bwd_scan_kernel(
         pass(b[2]); if (--left == 0) break;
         if (NBUF == 4) { pass(b[NBUF - 1]); if (--left == 0) break; }
     }
+    if (DECAY_GRAD || DELAY) __syncthreads();
     if (DECAY_GRAD) {
-        __syncthreads();
         store_row_sums(partial_i, sum_i, sp);
         store_row_sums(partial_v, sum_v, sp);
     }
+    if constexpr (DELAY) store_row_sums(shifts.delay_partial, sum_d, sp);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -558,7 +616,7 @@ __device__ __forceinline__ void complex_spike_surrogate(const SpikeSurrogate& k,
     g_im = g * (((neg_rho_over_tau * sg_i) * d_im) * step_re);
 }
 
-template <bool PARTIAL, bool STREAM, int SURR, int MODE = 0, int NBUF = 3>
+template <bool PARTIAL, bool STREAM, int SURR, int MODE = 0, int NBUF = 3, bool DELAY = false>
 __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
         float* __restrict__ g_re_in, float* __restrict__ g_im_in, float* __restrict__ partial_sin,
         float* __restrict__ partial_cos, const float* __restrict__ g_re, const float* __restrict__ g_im,
@@ -567,8 +625,10 @@ __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
         unsigned per_param, Shifts shifts) {
     constexpr bool SHIFT = MODE != 0, ANYT = MODE == 2;
     static_assert(MODE != 1 || SURR != 0, "delays are folded into the fused resonate-and-fire form only");
+    static_assert(!DELAY || (SHIFT && SURR != 0), "the delay gradient belongs to the forms that read the spike gradient through a delay");
     __shared__ float c_tab[kScanMaxRows], s_tab[kScanMaxRows];
     __shared__ float sum_s[kScanWaves][kScanMaxRows], sum_c[kScanWaves][kScanMaxRows];
+    __shared__ float sum_d[DELAY ? kScanWaves : 1][DELAY ? kScanMaxRows : 1];
     __shared__ ComplexStage L;
     __shared__ ScanShiftTables shift_tab;
     ScanSpan sp;
@@ -583,8 +643,9 @@ __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
     const __amdgpu_buffer_rsrc_t src_re = make_rsrc(kStates ? re + base : nullptr, kStates ? span_bytes : 0u);
     const __amdgpu_buffer_rsrc_t src_im = make_rsrc(kStates ? im + base : nullptr, kStates ? span_bytes : 0u);
     const __amdgpu_buffer_rsrc_t dst_r = make_rsrc(g_re_in + base, span_bytes), dst_i = make_rsrc(g_im_in + base, span_bytes);
+    const __amdgpu_buffer_rsrc_t src_d = make_rsrc(DELAY ? shifts.delayed + base : nullptr, DELAY ? span_bytes : 0u);
 
-    struct Quads { float4 gr, gi, re, im; int dg; };
+    struct Quads { float4 gr, gi, re, im; int dg; DelayGradQuads dq; };
     // the tensors that are never shifted, then the incoming gradient (read through the output delay when SHIFT)
     auto fetch_saved = [&](Quads& x, int q, const ScanCursor& at) {
         const bool in_span = (unsigned)q < (unsigned)nq;
@@ -603,6 +664,8 @@ __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
     auto fetch_grad = [&](Quads& x, int q, const ScanCursor& at) {
         if (SHIFT) {
             x.gr = scan_load_shifted(src_gr, (unsigned)q < (unsigned)nq, at.r, at.pos, shift_tab.kin[at.r], T, x.dg);
+            if (DELAY)
+                delay_grad_fetch(x.dq, src_gr, src_d, (unsigned)q < (unsigned)nq, at.r, at.pos, QR, shift_tab.kin[at.r], T);
         } else {
             x.gr = buf_load4<STREAM>(src_gr, (unsigned)q < (unsigned)nq ? q * 16 : kOutOfRange);
             x.dg = 0;
@@ -636,6 +699,8 @@ __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
     if (SHIFT) scan_shift_tables(shift_tab, shifts, sp, T);
     if (PARTIAL)
         for (int rr = sp.lane; rr < sp.rows; rr += kWave) { sum_s[sp.wv][rr] = 0.0f; sum_c[sp.wv][rr] = 0.0f; }
+    if (DELAY)
+        for (int rr = sp.lane; rr < sp.rows; rr += kWave) sum_d[sp.wv][rr] = 0.0f;
     int parity = (sp.npass - 1) & 1;
     if (sp.tid == 0) { L.cr[parity] = 0.0f; L.ci[parity] = 0.0f; }
     __syncthreads();
@@ -651,6 +716,8 @@ __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
         const bool row_end = cur.pos == QR - 1;
         const Cx mu{c_tab[cur.r], -s_tab[cur.r]};
         if (SHIFT && __any(x.dg != 0)) x.gr = scan_place(x.gr, x.dg);    // rare: only where a row begins or ends
+        if (ANYT && dd != 0) x.gr = scan_tail_mask(x.gr, dd, row_end);
+        if (DELAY) add_to_row(sum_d[sp.wv], delay_grad_terms(x.dq, x.gr, x.dg, 1.0f / shifts.ts), sp, cur, QR, active);
         if (ANYT && dd != 0) {
             if (SURR == 0) x.gi = scan_tail_place(x.gi, dd, row_end);
             if (kStates) { x.re = scan_tail_place(x.re, dd, row_end); x.im = scan_tail_place(x.im, dd, row_end); }
@@ -717,11 +784,12 @@ __global__ __launch_bounds__(kScanQuads) void res_bwd_scan_kernel(
         pass(b[2]); if (--left == 0) break;
         if (NBUF == 4) { pass(b[NBUF - 1]); if (--left == 0) break; }
     }
+    if (PARTIAL || DELAY) __syncthreads();
     if (PARTIAL) {
-        __syncthreads();
         store_row_sums(partial_sin, sum_s, sp);
         store_row_sums(partial_cos, sum_c, sp);
     }
+    if constexpr (DELAY) store_row_sums(shifts.delay_partial, sum_d, sp);
 }
 
 // Rows per workgroup: the fewest rows whose bytes are a whole number of 128-byte lines (so that no line is
@@ -800,16 +868,18 @@ int launch_cuba_bwd_scan(float* grad_in, float* partial_i, float* partial_v, con
     const ScanGrid g = scan_grid(M, T);
     if (!g.ok) return SLAYER_ERANGE;
     const Shifts sh = shifts ? *shifts : Shifts{nullptr, nullptr, nullptr, nullptr, 0, 0, 1, 1.0f, 1};
-#define SLAYER_SCAN_N(G, D, TH, S, SH, NB)                                                                       \
-    hipLaunchKernelGGL((cuba_bwd_scan_kernel<G, D, TH, S, SH, NB>), g.grid, dim3(kScanQuads), 0, stream, grad_in, \
+#define SLAYER_SCAN_L(G, D, TH, S, SH, NB, DL)                                                                   \
+    hipLaunchKernelGGL((cuba_bwd_scan_kernel<G, D, TH, S, SH, NB, DL>), g.grid, dim3(kScanQuads), 0, stream, grad_in, \
                        partial_i, partial_v, grad_spikes, voltage, theta, current, i_decay, v_decay, spike_thr,  \
                        tau, rho, M, (int)T, g.QR, g.rpg, (unsigned)npb, rows_per_param(npb, n_id),               \
                        rows_per_param(npb, n_vd), sh)
+#define SLAYER_SCAN_N(G, D, TH, S, SH, NB) do { if (SH != 0 && delay_grad) SLAYER_SCAN_L(G, D, TH, S, SH, NB, (SH != 0)); else SLAYER_SCAN_L(G, D, TH, S, SH, NB, false); } while (0)
 #define SLAYER_SCAN(G, D, TH, S, SH) do { if (g.passes > 3) SLAYER_SCAN_N(G, D, TH, S, SH, 4); else SLAYER_SCAN_N(G, D, TH, S, SH, 3); } while (0)
 #define SLAYER_SCAN_H(G, D, TH, S) do { if (shifts) SLAYER_SCAN(G, D, TH, S, 1); else SLAYER_SCAN(G, D, TH, S, 0); } while (0)
 #define SLAYER_SCAN_S(G, D, TH) do { if (g.any_length) SLAYER_SCAN(G, D, TH, false, 2); else if (g.streaming) SLAYER_SCAN_H(G, D, TH, true); else SLAYER_SCAN_H(G, D, TH, false); } while (0)
 #define SLAYER_SCAN_T(G, D) do { if (theta) SLAYER_SCAN_S(G, D, true); else SLAYER_SCAN_S(G, D, false); } while (0)
     const bool want = partial_i != nullptr;
+    const bool delay_grad = shifts && sh.delayed && sh.delay_partial;
     if (graded) { if (want) SLAYER_SCAN_T(true, true); else SLAYER_SCAN_T(true, false); }
     else { if (want) SLAYER_SCAN_T(false, true); else SLAYER_SCAN_T(false, false); }
 #undef SLAYER_SCAN_T
@@ -817,6 +887,7 @@ int launch_cuba_bwd_scan(float* grad_in, float* partial_i, float* partial_v, con
 #undef SLAYER_SCAN_H
 #undef SLAYER_SCAN
 #undef SLAYER_SCAN_N
+#undef SLAYER_SCAN_L
     return (int)hipGetLastError();
 }
 
@@ -831,11 +902,13 @@ int launch_res_bwd_scan(float* g_re_in, float* g_im_in, float* partial_sin, floa
     if (shifts && surrogate == 0) return SLAYER_EINVAL;      // delays belong to the fused resonate-and-fire form
     const SpikeSurrogate k{spike_thr, tau, rho};
     const Shifts sh = shifts ? *shifts : Shifts{nullptr, nullptr, nullptr, nullptr, 0, 0, 1, 1.0f, 1};
-#define SLAYER_SCAN_N(P, S, U, SH, NB)                                                                           \
-    hipLaunchKernelGGL((res_bwd_scan_kernel<P, S, U, SH, NB>), g.grid, dim3(kScanQuads), 0, stream, g_re_in, g_im_in, \
+    const bool delay_grad = shifts && surrogate != 0 && sh.delayed && sh.delay_partial;
+#define SLAYER_SCAN_L(P, S, U, SH, NB, DL)                                                                       \
+    hipLaunchKernelGGL((res_bwd_scan_kernel<P, S, U, SH, NB, DL>), g.grid, dim3(kScanQuads), 0, stream, g_re_in, g_im_in, \
                        partial_sin, partial_cos, g_re, g_im, re, im, sin_decay, cos_decay, k, M, (int)T, g.QR,   \
                        g.rpg,                                                                                    \
                        (unsigned)npb, rows_per_param(npb, num_decays), sh)
+#define SLAYER_SCAN_N(P, S, U, SH, NB) do { if (SH != 0 && U != 0 && delay_grad) SLAYER_SCAN_L(P, S, U, SH, NB, (SH != 0 && U != 0)); else SLAYER_SCAN_L(P, S, U, SH, NB, false); } while (0)
 #define SLAYER_SCAN(P, S, U, SH) do { if (g.passes > 3) SLAYER_SCAN_N(P, S, U, SH, 4); else SLAYER_SCAN_N(P, S, U, SH, 3); } while (0)
 #define SLAYER_SCAN_S(P, U, SH) do { if (g.any_length) SLAYER_SCAN(P, false, U, 2); else if (g.streaming) SLAYER_SCAN(P, true, U, SH); else SLAYER_SCAN(P, false, U, SH); } while (0)
 #define SLAYER_SCAN_P(U, SH) do { if (partial_sin) SLAYER_SCAN_S(true, U, SH); else SLAYER_SCAN_S(false, U, SH); } while (0)
@@ -846,6 +919,7 @@ int launch_res_bwd_scan(float* g_re_in, float* g_im_in, float* partial_sin, floa
 #undef SLAYER_SCAN_S
 #undef SLAYER_SCAN
 #undef SLAYER_SCAN_N
+#undef SLAYER_SCAN_L
     return (int)hipGetLastError();
 }
 

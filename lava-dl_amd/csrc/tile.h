@@ -17,7 +17,6 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
-#include <stdlib.h>
 #include <type_traits>
 #include "../../include/slayer_hip.h"
 
@@ -51,11 +50,29 @@ __device__ __forceinline__ void raise_range_flag(unsigned* flag) {
 __device__ __forceinline__ void check_multiplier(int mult, unsigned* flag) {
     if (mult > 8191 || mult < -8191) raise_range_flag(flag);
 }
+#ifndef SLAYER_RANGE_CHECK
+#define SLAYER_RANGE_CHECK 1             // 0: a build without the copy-out's range test, to measure what it costs
+#endif
 template <class Op, class = void>
 struct RangeChecked { static constexpr bool value = false; };
 template <class Op>
-struct RangeChecked<Op, decltype((void)Op::kRangeChecked)> { static constexpr bool value = Op::kRangeChecked; };
-// accumulates v + 2^L for a quad: a value outside [-2^L, 2^L) sets a bit at or above bit L + 1
+struct RangeChecked<Op, decltype((void)Op::kRangeChecked)> { static constexpr bool value = Op::kRangeChecked && SLAYER_RANGE_CHECK != 0; };
+// Smallest and largest value seen (integer bit patterns in float registers): two three-way minima / maxima per
+// quad, the cheapest form for the copy waves, whose instruction count is what bounds the kernels on few rows.
+struct RangeSpan {
+    int lo, hi;
+    __device__ __forceinline__ void reset() { lo = 0; hi = 0; }
+    __device__ __forceinline__ void track(float4 q) {
+        const int x = __float_as_int(q.x), y = __float_as_int(q.y), z = __float_as_int(q.z), w = __float_as_int(q.w);
+        hi = max(max(hi, x), y); hi = max(max(hi, z), w);
+        lo = min(min(lo, x), y); lo = min(min(lo, z), w);
+    }
+    __device__ __forceinline__ bool exceeded(int log2_bound) const {
+        return hi >= (1 << log2_bound) || lo < -(1 << log2_bound);
+    }
+};
+// the same test for states that are watched inside a sequential loop: accumulates v + 2^L for a quad; a value
+// outside [-2^L, 2^L) sets a bit at or above bit L + 1
 __device__ __forceinline__ unsigned range_bits(float4 q, int log2_bound) {
     const unsigned b = 1u << log2_bound;
     return (__float_as_uint(q.x) + b) | (__float_as_uint(q.y) + b) | (__float_as_uint(q.z) + b) | (__float_as_uint(q.w) + b);
@@ -223,6 +240,10 @@ struct Shifts {
     int sign;                // +1, or -1 for a backward pass (undoes the forward pass's shifts)
     float ts;                // sampling time the lut entries are divided by
     int64_t npb;
+    // backward scans only: the delayed spikes the forward pass stored and the per-row sums of
+    // grad[t] * (delayed[t-1] - delayed[t]) / ts they leave for the delay gradient, or nullptr
+    const float* delayed;
+    float* delay_partial;
 };
 
 // prm.shifts, or no shifts at all for an Op whose Params carry none
@@ -242,21 +263,22 @@ struct ShiftOutMask { static constexpr unsigned value = 0; };
 template <class Op>
 struct ShiftOutMask<Op, decltype((void)Op::kShiftOut)> { static constexpr unsigned value = Op::kShiftOut; };
 
-// steps + trunc(lut / ts) with every term held inside [-(T+1), T+1]: a shift of T steps already empties the
-// row, T+1 stands for everything beyond (the sample before the first, `head`, then falls off the row too)
+// steps + trunc(lut / ts), the sum held inside [-(T+1), T+1]: a shift of T steps already empties the row, T+1
+// stands for everything beyond (the sample before the first, `head`, then falls off the row too).  The terms are
+// added before the sum is clamped (two large terms of opposite sign leave a small shift); a table entry beyond
+// +-2^30 steps counts as +-2^30.
 __host__ __device__ __forceinline__ int clamp_shift(int64_t k, int T) {
     const int64_t lim = (int64_t)T + 1;
     return (int)(k > lim ? lim : (k < -lim ? -lim : k));
 }
 __device__ __forceinline__ int row_shift(const float* lut, int steps, float ts, int64_t m, int64_t npb, int T) {
-    int k = clamp_shift(steps, T);
+    int64_t k = steps;
     if (lut) {
         const float q = lut[m % npb] / ts;
-        const float lim = (float)T + 1.0f;
-        const int kl = !(q == q) ? 0 : (q >= lim ? T + 1 : (q <= -lim ? -(T + 1) : (int)q));
-        k = clamp_shift((int64_t)k + kl, T);
+        const float lim = 1073741824.0f;
+        k += !(q == q) ? 0 : (q >= lim ? (1 << 30) : (q <= -lim ? -(1 << 30) : (int)q));
     }
-    return k;
+    return clamp_shift(k, T);
 }
 
 __device__ __forceinline__ int in_shift_of(const Shifts& sh, int64_t m, int T) {
@@ -357,7 +379,7 @@ struct Copier {
     int row_lo, row_hi;                      // rows [row_lo, row_hi) of the tile are copied by this wave
     int kin[kShifts ? kPasses : 1], kout[kShifts ? kPasses : 1];   // shifts of this lane's row in each pass
     int kout_row;                            // output shift of row `lane` (lane = row), for fill_unreached
-    unsigned range_acc[RangeChecked<Op>::value ? NO : 1];   // see range_bits
+    RangeSpan range_seen[RangeChecked<Op>::value ? NO : 1];  // of the states this wave stored
     // wave-uniform: chunks [in_first, in_last] hold only quads whose shifted source lies wholly inside its row,
     // chunks [out_first, out_last] only quads whose shifted destination does (for every row of this wave)
     int in_first, in_last, out_first, out_last;
@@ -367,12 +389,17 @@ struct Copier {
                                          unsigned base_f, int first_pass_ = 0) {
         rows = rows_; T = T_; first_pass = first_pass_;
 #pragma unroll
-        for (int o = 0; o < (RangeChecked<Op>::value ? NO : 1); ++o) range_acc[o] = 0u;
+        for (int o = 0; o < (RangeChecked<Op>::value ? NO : 1); ++o) range_seen[o].reset();
         row_lo = first_pass * G::kRowsPerPass;
         row_hi = (first_pass + kPasses) * G::kRowsPerPass;
         if (row_hi > rows) row_hi = rows;
-        rebase_src(prm, m0, rows);
-        rebase_dst(prm, m0, rows);
+        const unsigned wave_bytes = (unsigned)rows * (unsigned)T * 4u;
+#pragma unroll
+        for (int i = 0; i < NI; ++i)         // an input the caller does not have: every load falls out of range, reads 0
+            src[i] = prm.in[i] ? make_rsrc(prm.in[i] + m0 * (int64_t)T, wave_bytes) : make_rsrc(nullptr, 0);
+#pragma unroll
+        for (int o = 0; o < NO + ND; ++o)    // an output the caller does not want: every store falls out of range
+            dst[o] = prm.out[o] ? make_rsrc(prm.out[o] + m0 * (int64_t)T, wave_bytes) : make_rsrc(nullptr, 0);
         crow = lane / G::kQuads;                // row within a pass
         cq = lane % G::kQuads;                  // quad within the row
         // chunks [1, interior_end) hold only valid columns and touch no shared line, for every phase
@@ -419,27 +446,6 @@ struct Copier {
             in_first = __builtin_amdgcn_readfirstlane(in_first); in_last = __builtin_amdgcn_readfirstlane(in_last);
             out_first = __builtin_amdgcn_readfirstlane(out_first); out_last = __builtin_amdgcn_readfirstlane(out_last);
         }
-    }
-
-    // The descriptors of the loads / of the stores moved to the row block that starts at row m0 and has rows_ rows
-    // (0: a block that does not exist, every access falls out of range).  A workgroup that walks several row blocks
-    // loads ahead in the next block while it still stores the previous one, so the two sides move separately.
-    // Everything else a lane knows (phases, offsets within the block, shifts) is the same in every block of a
-    // workgroup: blocks are a whole number of 128-byte lines apart.
-    __device__ __forceinline__ void rebase_src(const typename Op::Params& prm, int64_t m0, int rows_) {
-        const unsigned bytes = (unsigned)rows_ * (unsigned)T * 4u;
-#pragma unroll
-        for (int i = 0; i < NI; ++i)         // an input the caller does not have: every load falls out of range, reads 0
-            src[i] = (prm.in[i] && rows_ > 0) ? make_rsrc(prm.in[i] + m0 * (int64_t)T, bytes) : make_rsrc(nullptr, 0);
-    }
-    __device__ __forceinline__ void rebase_dst(const typename Op::Params& prm, int64_t m0, int rows_) {
-        const unsigned bytes = (unsigned)rows_ * (unsigned)T * 4u;
-#pragma unroll
-        for (int o = 0; o < NO + ND; ++o)    // an output the caller does not want: every store falls out of range
-            dst[o] = (prm.out[o] && rows_ > 0) ? make_rsrc(prm.out[o] + m0 * (int64_t)T, bytes) : make_rsrc(nullptr, 0);
-        rows = rows_;
-        row_hi = (first_pass + kPasses) * G::kRowsPerPass;
-        if (row_hi > rows) row_hi = rows;
     }
 
     __device__ __forceinline__ bool whole_in(int chunk) const { return chunk >= in_first && chunk <= in_last; }
@@ -566,7 +572,7 @@ struct Copier {
             bool bad = false;
 #pragma unroll
             for (int o = 0; o < NO; ++o)
-                if (Op::range_log2(o) != 0) bad = bad || range_exceeded(range_acc[o], Op::range_log2(o));
+                if (Op::range_log2(o) != 0) bad = bad || range_seen[o].exceeded(Op::range_log2(o));
             if (bad) raise_range_flag(prm.range_flag);
         }
     }
@@ -590,11 +596,18 @@ struct Copier {
             for (int o = 0; o < NO; ++o) own[o] = v[o] = *reinterpret_cast<const float4*>(&tile[o][r * G::kPitch + 4 * cq]);
             if constexpr (RangeChecked<Op>::value) {
                 // only quads that hold steps of the row: the tiles of a chunk number that names no chunk (before
-                // the first, after the last) were never filled
-                const bool counted = inner || (UNAL ? (t > -4 && t < T) : (unsigned)t < (unsigned)T);
+                // the first, after the last) were never filled.  Interior chunks hold nothing else.
+                if (inner) {
 #pragma unroll
-                for (int o = 0; o < NO; ++o)
-                    if (Op::range_log2(o) != 0) range_acc[o] |= counted ? range_bits(v[o], Op::range_log2(o)) : 0u;
+                    for (int o = 0; o < NO; ++o)
+                        if (Op::range_log2(o) != 0) range_seen[o].track(v[o]);
+                } else {
+                    const bool counted = UNAL ? (t > -4 && t < T) : (unsigned)t < (unsigned)T;
+                    const float4 none = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+                    for (int o = 0; o < NO; ++o)
+                        if (Op::range_log2(o) != 0) range_seen[o].track(counted ? v[o] : none);
+                }
             }
             if (!inner) {
                 const int a = 4 * cq - step0[p];                   // phase of row r
@@ -840,31 +853,8 @@ __global__ __launch_bounds__(kWave) void stream_kernel(typename Op::Params prm, 
 // A chunk is a few hundred nanoseconds of recurrence, less than a trip to memory, so the copy
 // waves keep the loads of two chunks in flight (chunk j waits in fetched[j & 1]).  All waves run
 // an even number of chunks; a surplus chunk lies outside every row and neither computes nor stores.
-//
-// Several row blocks per workgroup (large tensors).  A workgroup takes the row blocks blockIdx.x,
-// blockIdx.x + gridDim.x, ... (`per_group` of them at most) one after the other, and the chunks of all its blocks
-// form one sequence: while the sequential wave finishes the last chunks of a block the copy waves already load
-// the first chunks of the next one, so a workgroup never waits for memory with nothing to do, few workgroups per
-// compute unit keep it busy, and the chip touches few rows at a time -- which is what its memory system rewards
-// (a plain copy in this access pattern: 5.0 TB/s with 262 144 rows in flight, 5.7 with 32 768).  Row blocks are
-// R * T floats = a whole number of 128-byte lines apart (R a multiple of 32), so phases, chunk counts and every
-// per-lane offset are the same in all blocks of a workgroup; only the buffer descriptors move on.
-constexpr int kNoChunk = -8;             // a chunk number that names no chunk: every access falls out of range
-
-// Position in the chunk sequence of a workgroup: row block i (of `blocks`), k-th chunk of the block in processing
-// order (of `per_block`); positions before the first and after the last block name no chunk.
-struct ChunkCursor {
-    int i, k;
-    __device__ __forceinline__ bool advance(int per_block) {      // true when a new block begins
-        if (++k < per_block) return false;
-        k = 0; ++i;
-        return true;
-    }
-};
-
 template <class Op, int R, bool STREAM, int NCOPY, int S = kTileSamples, bool UNAL = false>
-__global__ __launch_bounds__((1 + NCOPY) * kWave) void stream_kernel_duo(typename Op::Params prm, int64_t M, int T,
-                                                                           int per_group) {
+__global__ __launch_bounds__((1 + NCOPY) * kWave) void stream_kernel_duo(typename Op::Params prm, int64_t M, int T) {
     using G = TileGeom<R, S>;
     constexpr int TC = G::kChunk;
     constexpr int NI = Op::kIn, NO = Op::kOut, NT = NI > NO ? NI : NO;
@@ -874,82 +864,52 @@ __global__ __launch_bounds__((1 + NCOPY) * kWave) void stream_kernel_duo(typenam
 
     const int lane = threadIdx.x & (kWave - 1);
     const int role = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));   // wave-uniform
-    const int64_t nblocks = (M + R - 1) / R;
-    // the row blocks of this workgroup: blockIdx.x + i * gridDim.x for i < blocks
-    const int64_t left = nblocks - (int64_t)blockIdx.x;
-    const int64_t avail = (left + (int64_t)gridDim.x - 1) / (int64_t)gridDim.x;
-    const int blocks = (int)(avail < (int64_t)per_group ? avail : (int64_t)per_group);
-    auto first_row = [&](int i) { return ((int64_t)blockIdx.x + (int64_t)i * (int64_t)gridDim.x) * R; };
-    auto rows_of = [&](int i) {
-        if (i < 0 || i >= blocks) return 0;
-        const int64_t r = M - first_row(i);
-        return (int)(r < R ? r : R);
-    };
-    const int64_t m0 = first_row(0);
-    const int rows = rows_of(0);
+    const int64_t m0 = (int64_t)blockIdx.x * R;
+    const int rows = (int)((M - m0) < R ? (M - m0) : R);
     const unsigned base_f = (unsigned)(reinterpret_cast<uintptr_t>(prm.in[0]) >> 2);
     const int a_lane = (int)((base_f + (unsigned)(m0 + lane) * (unsigned)T) & 31u);
     const int nchunks = chunk_count<TC>(a_lane, lane < rows, T);
     const int nloop = (nchunks + 1) & ~1;
     const int interior_end = (T & ~31) / TC;
-    // k-th chunk of a block in processing order; values outside [0, nchunks) name no chunk
+    // k-th chunk in processing order; values outside [0, nchunks) name no chunk
     auto chunk_of = [&](int k) { return Op::kReverse ? nchunks - 1 - k : k; };
 
     if (role == 0) {
         Op op;
-        for (int i = 0; i < blocks; ++i) {
-            const int64_t mb = first_row(i);
-            const int rows_i = rows_of(i);
-            op.init(prm, mb + lane, lane < rows_i);
-            for (int k = 0; k < nloop; ++k) {
-                const int chunk = chunk_of(k);
-                __syncthreads();                               // barrier i * nloop + k
-                if (k < nchunks)
-                    run_chunk<Op, R, 4, S, UNAL>(op, tiles[k & 1], lane, chunk, chunk >= 1 && chunk < interior_end, a_lane, T);
-            }
-            op.finish(prm, mb + lane, lane < rows_i);
+        op.init(prm, m0 + lane, lane < rows);
+        for (int k = 0; k < nloop; ++k) {
+            const int chunk = chunk_of(k);
+            __syncthreads();                                   // barrier k
+            if (k < nchunks)
+                run_chunk<Op, R, 4, S, UNAL>(op, tiles[k & 1], lane, chunk, chunk >= 1 && chunk < interior_end, a_lane, T);
         }
-        __syncthreads();                                       // barrier blocks * nloop
+        __syncthreads();                                       // barrier nloop
+        op.finish(prm, m0 + lane, lane < rows);
     } else {
         Op uni;                                                // wave-uniform members only (pre, post, derive)
         uni.init(prm, 0, false);
         Copier<Op, R, STREAM, PASSES, S, UNAL> io;
         io.init(prm, m0, rows, T, lane, base_f, (role - 1) * PASSES);
         float4 fetched[2][NI][PASSES];
-        ChunkCursor fe{0, 0}, fi{0, 0}, ou{-1, nloop - 1};     // next chunk to load, to put into tiles, to store
-        auto chunk_at = [&](const ChunkCursor& c) { return (c.i >= 0 && c.i < blocks) ? chunk_of(c.k) : kNoChunk; };
-        auto fetch = [&](float4 (&buf)[NI][PASSES]) {
-            io.fetch_into(buf, chunk_at(fe));
-            if (fe.advance(nloop)) io.rebase_src(prm, first_row(fe.i), rows_of(fe.i));
-        };
-        auto fill = [&](float (*tile)[G::kTileFloats], const float4 (&buf)[NI][PASSES]) {
-            io.to_tiles(uni, tile, buf, chunk_at(fi));
-            fi.advance(nloop);
-        };
-        auto store = [&](float (*tile)[G::kTileFloats]) {
-            io.copy_out(uni, tile, chunk_at(ou));
-            if (ou.advance(nloop)) io.rebase_dst(prm, first_row(ou.i), rows_of(ou.i));
-        };
-        fetch(fetched[0]);
-        fetch(fetched[1]);
+        io.fetch_into(fetched[0], chunk_of(0));
+        io.fetch_into(fetched[1], chunk_of(1));
         io.prime_stores();
-        fill(tiles[0], fetched[0]);
-        fetch(fetched[0]);
+        io.to_tiles(uni, tiles[0], fetched[0], chunk_of(0));
+        io.fetch_into(fetched[0], chunk_of(2));
         __syncthreads();                                       // barrier 0
         io.fill_unreached(prm, m0, lane);                      // while the sequential wave works on chunk 0
-        const int total = blocks * nloop;
-        for (int v = 0; v < total; v += 2) {
-            // wave 0 works on tiles[0] (chunk v of the sequence); tiles[1] still holds the results of chunk v-1
-            store(tiles[1]);
-            fill(tiles[1], fetched[1]);
-            fetch(fetched[1]);
-            __syncthreads();                                   // barrier v+1
-            store(tiles[0]);
-            fill(tiles[0], fetched[0]);
-            fetch(fetched[0]);
-            __syncthreads();                                   // barrier v+2
+        for (int k = 0; k < nloop; k += 2) {
+            // wave 0 works on tiles[0] (chunk k); tiles[1] still holds the results of chunk k-1
+            io.copy_out(uni, tiles[1], chunk_of(k - 1));
+            io.to_tiles(uni, tiles[1], fetched[1], chunk_of(k + 1));
+            io.fetch_into(fetched[1], chunk_of(k + 3));
+            __syncthreads();                                   // barrier k+1
+            io.copy_out(uni, tiles[0], chunk_of(k));
+            io.to_tiles(uni, tiles[0], fetched[0], chunk_of(k + 2));
+            io.fetch_into(fetched[0], chunk_of(k + 4));
+            __syncthreads();                                   // barrier k+2
         }
-        store(tiles[1]);
+        io.copy_out(uni, tiles[1], chunk_of(nloop - 1));
         io.report_range(prm);
     }
 }
@@ -963,11 +923,8 @@ __global__ __launch_bounds__((1 + NCOPY) * kWave) void stream_kernel_duo(typenam
 //   on chunk j-1 in tiles[(j-1) % 3], the copy waves store chunk j-2 from tiles[(j+1) % 3], refill them with
 //   chunk j+1 and issue the loads of chunk j+4 (three chunks of loads in flight).
 // Every wave passes the same number of barriers; chunk numbers outside [0, nchunks) name no chunk.
-// Several row blocks per workgroup as in stream_kernel_duo: the chunks of a block are padded to a multiple of
-// three, so that the tile rotation carries on from block to block, and chunk j above is the j-th of the sequence.
 template <class Op, int R, bool STREAM, int NCOPY, bool UNAL = false>
-__global__ __launch_bounds__((2 + NCOPY) * kWave) void stream_kernel_staged(typename Op::Params prm, int64_t M, int T,
-                                                                              int per_group) {
+__global__ __launch_bounds__((2 + NCOPY) * kWave) void stream_kernel_staged(typename Op::Params prm, int64_t M, int T) {
     using G = TileGeom<R>;
     constexpr int TC = G::kChunk;
     constexpr int NI = Op::kIn, NO = Op::kOut, NT = NI > NO ? NI : NO;
@@ -978,41 +935,28 @@ __global__ __launch_bounds__((2 + NCOPY) * kWave) void stream_kernel_staged(type
 
     const int lane = threadIdx.x & (kWave - 1);
     const int role = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));   // wave-uniform
-    const int64_t nblocks = (M + R - 1) / R;
-    const int64_t left = nblocks - (int64_t)blockIdx.x;
-    const int64_t avail = (left + (int64_t)gridDim.x - 1) / (int64_t)gridDim.x;
-    const int blocks = (int)(avail < (int64_t)per_group ? avail : (int64_t)per_group);
-    auto first_row = [&](int i) { return ((int64_t)blockIdx.x + (int64_t)i * (int64_t)gridDim.x) * R; };
-    auto rows_of = [&](int i) {
-        if (i < 0 || i >= blocks) return 0;
-        const int64_t r = M - first_row(i);
-        return (int)(r < R ? r : R);
-    };
-    const int64_t m0 = first_row(0);
-    const int rows = rows_of(0);
+    const int64_t m0 = (int64_t)blockIdx.x * R;
+    const int rows = (int)((M - m0) < R ? (M - m0) : R);
     const unsigned base_f = (unsigned)(reinterpret_cast<uintptr_t>(prm.in[0]) >> 2);
     const int a_lane = (int)((base_f + (unsigned)(m0 + lane) * (unsigned)T) & 31u);
     const int nchunks = chunk_count<TC>(a_lane, lane < rows, T);
-    const int per_block = blocks > 1 ? (nchunks + 2) / 3 * 3 : nchunks;   // chunks of a block in the sequence, padded
-    const int periods = (blocks * per_block + 2 + 2) / 3 * 3;   // the last chunk leaves two periods after it entered
+    const int periods = (nchunks + 2 + 2) / 3 * 3;          // the last chunk leaves in period nchunks + 1
     const int interior_end = (T & ~31) / TC;
 
     auto sequential = [&](auto& stage, int lag) {
-        ChunkCursor at{lag == 0 ? 0 : -1, lag == 0 ? 0 : per_block - lag};   // the chunk of period 0 is `lag` behind
+        stage.init(prm, m0 + lane, lane < rows);
         for (int j = 0; j < periods; j += 3) {
 #pragma unroll
             for (int h = 0; h < 3; ++h) {
-                const bool real = at.i >= 0 && at.i < blocks;
-                if (real && at.k == 0) stage.init(prm, first_row(at.i) + lane, lane < rows_of(at.i));
+                const int chunk = j + h - lag;
                 __syncthreads();                               // barrier j+h
-                if (real && at.k < nchunks)
+                if (chunk >= 0 && chunk < nchunks)
                     run_chunk<typename std::remove_reference<decltype(stage)>::type, R, 4, kTileSamples, UNAL>(
-                        stage, tiles[(h + 3 - lag) % 3], lane, at.k, at.k >= 1 && at.k < interior_end, a_lane, T);
-                if (real && at.k == per_block - 1) stage.finish(prm, first_row(at.i) + lane, lane < rows_of(at.i));
-                at.advance(per_block);
+                        stage, tiles[(h + 3 - lag) % 3], lane, chunk, chunk >= 1 && chunk < interior_end, a_lane, T);
             }
         }
         __syncthreads();                                       // barrier `periods`
+        stage.finish(prm, m0 + lane, lane < rows);
     };
     if (role == 0) {
         typename Op::Stage0 st;
@@ -1026,33 +970,19 @@ __global__ __launch_bounds__((2 + NCOPY) * kWave) void stream_kernel_staged(type
         Copier<Op, R, STREAM, PASSES, kTileSamples, UNAL> io;
         io.init(prm, m0, rows, T, lane, base_f, (role - 2) * PASSES);
         float4 fetched[3][NI][PASSES];
-        ChunkCursor fe{0, 0}, fi{0, 0}, ou{-1, per_block - 2};  // next chunk to load, to put into tiles, to store
-        auto chunk_at = [&](const ChunkCursor& c) { return (c.i >= 0 && c.i < blocks && c.k < nchunks) ? c.k : kNoChunk; };
-        auto fetch = [&](float4 (&buf)[NI][PASSES]) {
-            io.fetch_into(buf, chunk_at(fe));
-            if (fe.advance(per_block)) io.rebase_src(prm, first_row(fe.i), rows_of(fe.i));
-        };
-        auto fill = [&](float (*tile)[G::kTileFloats], const float4 (&buf)[NI][PASSES]) {
-            io.to_tiles(uni, tile, buf, chunk_at(fi));
-            fi.advance(per_block);
-        };
-        auto store = [&](float (*tile)[G::kTileFloats]) {
-            io.copy_out(uni, tile, chunk_at(ou));
-            if (ou.advance(per_block)) io.rebase_dst(prm, first_row(ou.i), rows_of(ou.i));
-        };
 #pragma unroll
-        for (int d = 0; d < 3; ++d) fetch(fetched[d]);
+        for (int d = 0; d < 3; ++d) io.fetch_into(fetched[d], d);
         io.prime_stores();
-        fill(tiles[0], fetched[0]);
-        fetch(fetched[0]);
+        io.to_tiles(uni, tiles[0], fetched[0], 0);
+        io.fetch_into(fetched[0], 3);
         __syncthreads();                                       // barrier 0
         io.fill_unreached(prm, m0, lane);                      // while the first wave works on chunk 0
         for (int j = 0; j < periods; j += 3) {
 #pragma unroll
             for (int h = 0; h < 3; ++h) {
-                store(tiles[(h + 1) % 3]);                     // chunk j+h-2
-                fill(tiles[(h + 1) % 3], fetched[(h + 1) % 3]);   // chunk j+h+1
-                fetch(fetched[(h + 1) % 3]);                   // chunk j+h+4
+                io.copy_out(uni, tiles[(h + 1) % 3], j + h - 2);
+                io.to_tiles(uni, tiles[(h + 1) % 3], fetched[(h + 1) % 3], j + h + 1);
+                io.fetch_into(fetched[(h + 1) % 3], j + h + 4);
                 __syncthreads();                               // barrier j+h+1
             }
         }
@@ -1234,6 +1164,7 @@ inline Shifts backward_shifts(const slayer_delays* d, int64_t npb) {
         s.in_lut = d->out_delay; s.out_lut = d->in_shift;
         s.in_steps = steps_to_int(d->out_steps); s.out_steps = steps_to_int(d->in_steps);
         if (d->sampling_time != 0.0f) s.ts = d->sampling_time;
+        s.delayed = d->delayed_spikes; s.delay_partial = d->grad_workspace;
     }
     return s;
 }
@@ -1365,30 +1296,6 @@ constexpr int kGroupsPerCuWhenLarge = 4;
 // 32 steps: 36 / 46 and 52 / 88; at 64 steps even to 25 % behind, from 128 steps on 3-15 % ahead).
 constexpr int64_t kMultiwaveWhenLargeMinSteps = 128;
 
-// How the row blocks of a multi-wave launch are shared out.  Resident (every block gets a workgroup of its own
-// that runs at once), or an Op with real shifts (its per-row shift tables differ from block to block): one block
-// per workgroup.  Else as many workgroups as the chip holds at `per_cu` per compute unit, each walking
-// `per_group` blocks.  SLAYER_GROUPS_PER_CU overrides `per_cu` and SLAYER_BLOCKS_PER_GROUP = 1 switches the walk
-// off (tuning).
-struct BlockPlan { int64_t groups; int per_group; int per_cu; };
-inline int tuning_int(const char* name) {
-    const char* e = getenv(name);
-    return e ? atoi(e) : 0;
-}
-template <class Op>
-BlockPlan plan_blocks(int64_t nblocks, bool one_each, int want_per_cu, int fits_per_cu) {
-    static const int env_per_cu = tuning_int("SLAYER_GROUPS_PER_CU"), env_walk = tuning_int("SLAYER_BLOCKS_PER_GROUP");
-    int per_cu = env_per_cu > 0 ? env_per_cu : want_per_cu;
-    if (fits_per_cu > 0 && per_cu > fits_per_cu) per_cu = fits_per_cu;
-    if (per_cu < 1) per_cu = 1;
-    const bool shifted = ShiftInMask<Op>::value != 0 || ShiftOutMask<Op>::value != 0;
-    const int64_t slots = (int64_t)per_cu * compute_units();
-    if (one_each || shifted || env_walk == 1 || slots <= 0 || nblocks <= slots) return BlockPlan{nblocks, 1, per_cu};
-    const int64_t per_group = (nblocks + slots - 1) / slots;
-    if (per_group > 0x3fffffff) return BlockPlan{nblocks, 1, per_cu};
-    return BlockPlan{(nblocks + per_group - 1) / per_group, (int)per_group, per_cu};
-}
-
 // Dynamic LDS (unused by the kernel) that holds a kernel with `static_lds` bytes to `groups` workgroups per CU.
 inline unsigned lds_pad_for(int groups, size_t static_lds) {
     const size_t lds_per_cu = 160 * 1024, want = lds_per_cu / (size_t)(groups + 1) + 256;   // too much for groups + 1
@@ -1397,14 +1304,14 @@ inline unsigned lds_pad_for(int groups, size_t static_lds) {
     return (unsigned)(pad > 60 * 1024 ? 60 * 1024 : pad);
 }
 template <class Op, int R, bool STREAM, bool UNAL = false>
-unsigned duo_pad_when_large(int groups) {
-    static const size_t lds = [] {
+unsigned duo_pad_when_large() {
+    static const unsigned pad = [] {
         hipFuncAttributes a;
         if (hipFuncGetAttributes(&a, (const void*)stream_kernel_duo<Op, R, STREAM, CopyWaves<Op>::value, kTileSamples, UNAL>) != hipSuccess)
-            return (size_t)0;
-        return (size_t)a.sharedSizeBytes;
+            return 0u;
+        return lds_pad_for(kGroupsPerCuWhenLarge, a.sharedSizeBytes);
     }();
-    return lds == 0 ? 0u : lds_pad_for(groups, lds);
+    return pad;
 }
 
 // Ops made of two chained recurrences (kStages = 2) run them in two waves while every workgroup of that
@@ -1437,14 +1344,14 @@ struct StagedWhenLarge<Op, decltype((void)Op::kStagedWhenLarge)> { static conste
 // compute unit, loses a quarter at T = 300 and stays with the two-wave form.)
 constexpr int kStagedGroupsPerCuWhenLarge = 3;
 template <class Op, bool STREAM, bool UNAL = false>
-unsigned staged_pad_when_large(int groups) {
-    static const size_t lds = [] {
+unsigned staged_pad_when_large() {
+    static const unsigned pad = [] {
         hipFuncAttributes a;
         if (hipFuncGetAttributes(&a, (const void*)stream_kernel_staged<Op, 64, STREAM, CopyWaves<Op>::value, UNAL>) != hipSuccess)
-            return (size_t)0;
-        return (size_t)a.sharedSizeBytes;
+            return 0u;
+        return lds_pad_for(kStagedGroupsPerCuWhenLarge, a.sharedSizeBytes);
     }();
-    return lds == 0 ? 0u : lds_pad_for(groups, lds);
+    return pad;
 }
 
 // Rows that are not whole quads (T % 4 != 0 or bases that are only dword-aligned): the multi-wave kernels in their
@@ -1462,23 +1369,18 @@ int launch_stream_unaligned(const typename Op::Params& prm, int64_t M, int64_t T
         const int per_cu = staged_groups_per_cu<Op, STREAM, true>();
         const bool fits = (M + 63) / 64 <= (int64_t)per_cu * compute_units();
         if (per_cu > 0 && (fits || StagedWhenLarge<Op>::value)) {
-            const BlockPlan plan = plan_blocks<Op>((M + 63) / 64, fits, kStagedGroupsPerCuWhenLarge, per_cu);
-            const dim3 grid((unsigned)plan.groups), block((2 + NC) * kWave);
-            const unsigned pad = fits ? 0u : staged_pad_when_large<Op, STREAM, true>(plan.per_cu);
-            hipLaunchKernelGGL((stream_kernel_staged<Op, 64, STREAM, NC, true>), grid, block, pad, stream, prm, M, (int)T,
-                               plan.per_group);
+            const dim3 grid((unsigned)((M + 63) / 64)), block((2 + NC) * kWave);
+            const unsigned pad = fits ? 0u : staged_pad_when_large<Op, STREAM, true>();
+            hipLaunchKernelGGL((stream_kernel_staged<Op, 64, STREAM, NC, true>), grid, block, pad, stream, prm, M, (int)T);
             return (int)hipGetLastError();
         }
     }
     constexpr int RD = DuoRows<Op>::value;
     const int64_t groups = (M + RD - 1) / RD;
-    const int per_cu = duo_groups_per_cu<Op, RD, STREAM, true>();
-    const bool resident = groups <= (int64_t)per_cu * compute_units();
-    const BlockPlan plan = plan_blocks<Op>(groups, resident || RD % 32 != 0, kGroupsPerCuWhenLarge, per_cu);
-    const dim3 grid((unsigned)plan.groups), block((1 + NC) * kWave);
-    const unsigned pad = resident ? 0u : duo_pad_when_large<Op, RD, STREAM, true>(plan.per_cu);
-    hipLaunchKernelGGL((stream_kernel_duo<Op, RD, STREAM, NC, kTileSamples, true>), grid, block, pad, stream, prm, M, (int)T,
-                       plan.per_group);
+    const bool resident = groups <= (int64_t)duo_groups_per_cu<Op, RD, STREAM, true>() * compute_units();
+    const dim3 grid((unsigned)groups), block((1 + NC) * kWave);
+    const unsigned pad = resident ? 0u : duo_pad_when_large<Op, RD, STREAM, true>();
+    hipLaunchKernelGGL((stream_kernel_duo<Op, RD, STREAM, NC, kTileSamples, true>), grid, block, pad, stream, prm, M, (int)T);
     return (int)hipGetLastError();
 }
 
@@ -1494,20 +1396,15 @@ int launch_stream(const typename Op::Params& prm, int64_t M, int64_t T, hipStrea
     if constexpr (StageCount<Op>::value == 2) {
         const int per_cu = streaming ? staged_groups_per_cu<Op, true>() : staged_groups_per_cu<Op, false>();
         const bool fits = (M + 63) / 64 <= (int64_t)per_cu * compute_units();
-        static const int env_staged = tuning_int("SLAYER_STAGED_LARGE");     // tuning: 1 = always, 2 = never
-        const bool when_large = env_staged == 1 || (env_staged != 2 && StagedWhenLarge<Op>::value);
-        if (vec && per_cu > 0 && (fits || (when_large && !long_pieces && T >= kMultiwaveWhenLargeMinSteps))) {
+        if (vec && per_cu > 0 && (fits || (StagedWhenLarge<Op>::value && !long_pieces && T >= kMultiwaveWhenLargeMinSteps))) {
             constexpr int NC = CopyWaves<Op>::value;
-            const BlockPlan plan = plan_blocks<Op>((M + 63) / 64, fits, kStagedGroupsPerCuWhenLarge, per_cu);
-            const dim3 grid((unsigned)plan.groups), block((2 + NC) * kWave);
+            const dim3 grid((unsigned)((M + 63) / 64)), block((2 + NC) * kWave);
             if (streaming) {
-                const unsigned pad = fits ? 0u : staged_pad_when_large<Op, true>(plan.per_cu);
-                hipLaunchKernelGGL((stream_kernel_staged<Op, 64, true, NC>), grid, block, pad, stream, prm, M, (int)T,
-                                   plan.per_group);
+                const unsigned pad = fits ? 0u : staged_pad_when_large<Op, true>();
+                hipLaunchKernelGGL((stream_kernel_staged<Op, 64, true, NC>), grid, block, pad, stream, prm, M, (int)T);
             } else {
-                const unsigned pad = fits ? 0u : staged_pad_when_large<Op, false>(plan.per_cu);
-                hipLaunchKernelGGL((stream_kernel_staged<Op, 64, false, NC>), grid, block, pad, stream, prm, M, (int)T,
-                                   plan.per_group);
+                const unsigned pad = fits ? 0u : staged_pad_when_large<Op, false>();
+                hipLaunchKernelGGL((stream_kernel_staged<Op, 64, false, NC>), grid, block, pad, stream, prm, M, (int)T);
             }
             return (int)hipGetLastError();
         }
@@ -1516,15 +1413,13 @@ int launch_stream(const typename Op::Params& prm, int64_t M, int64_t T, hipStrea
     if (resident || (vec && MultiwaveWhenLarge<Op>::value && !long_pieces && T >= kMultiwaveWhenLargeMinSteps)) {
         constexpr int RD = DuoRows<Op>::value;
         constexpr int NC = CopyWaves<Op>::value;
-        const int per_cu = streaming ? duo_groups_per_cu<Op, RD, true>() : duo_groups_per_cu<Op, RD, false>();
-        const BlockPlan plan = plan_blocks<Op>((M + RD - 1) / RD, resident || RD % 32 != 0, kGroupsPerCuWhenLarge, per_cu);
-        const dim3 grid((unsigned)plan.groups), block((1 + NC) * kWave);
+        const dim3 grid((unsigned)((M + RD - 1) / RD)), block((1 + NC) * kWave);
         if (streaming) {
-            const unsigned pad = resident ? 0u : duo_pad_when_large<Op, RD, true>(plan.per_cu);
-            hipLaunchKernelGGL((stream_kernel_duo<Op, RD, true, NC>), grid, block, pad, stream, prm, M, (int)T, plan.per_group);
+            const unsigned pad = resident ? 0u : duo_pad_when_large<Op, RD, true>();
+            hipLaunchKernelGGL((stream_kernel_duo<Op, RD, true, NC>), grid, block, pad, stream, prm, M, (int)T);
         } else {
-            const unsigned pad = resident ? 0u : duo_pad_when_large<Op, RD, false>(plan.per_cu);
-            hipLaunchKernelGGL((stream_kernel_duo<Op, RD, false, NC>), grid, block, pad, stream, prm, M, (int)T, plan.per_group);
+            const unsigned pad = resident ? 0u : duo_pad_when_large<Op, RD, false>();
+            hipLaunchKernelGGL((stream_kernel_duo<Op, RD, false, NC>), grid, block, pad, stream, prm, M, (int)T);
         }
         return (int)hipGetLastError();
     }

@@ -30,7 +30,8 @@ _D = ctypes.c_double
 class Delays(ctypes.Structure):
     """struct slayer_delays of include/slayer_hip.h (device pointers as integers)."""
     _fields_ = [('in_shift', _P), ('out_delay', _P), ('out_head', _P), ('spike_last', _P),
-                ('in_steps', _I64), ('out_steps', _I64), ('sampling_time', _F)]
+                ('in_steps', _I64), ('out_steps', _I64), ('sampling_time', _F),
+                ('delayed_spikes', _P), ('grad_out_delay', _P), ('grad_workspace', _P)]
 
 
 _DP = ctypes.POINTER(Delays)
@@ -55,6 +56,7 @@ _SIGNATURES = {
     'slayer_cspike_bwd': (_INT, [_P, _P, _P, _P, _P, _P, _I64, _F, _F, _F, _INT, _I64, _P]),
     'slayer_shift': (_INT, [_P, _P, _P, _I64, _F, _I64, _I64, _I64, _P]),
     'slayer_delay_bwd': (_INT, [_P, _P, _P, _P, _P, _I64, _F, _P, _I64, _I64, _I64, _P]),
+    'slayer_conv_synapse': (_INT, [_P, _P, _P] + [_I64] * 14 + [_P]),
     'slayer_conv': (_INT, [_P, _P, _P, _I64, _F, _I64, _I64, _P]),
     'slayer_corr': (_INT, [_P, _P, _P, _I64, _F, _I64, _I64, _P]),
     'slayer_apth_fwd': (_INT, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _INT,
@@ -72,6 +74,10 @@ _SIGNATURES = {
     'slayer_cuba_recurrent_fwd': (_INT, [_P] * 10 + [_F, _INT, _F, _INT] + [_I64] * 7 + [_P]),
     'slayer_alif_recurrent_fwd': (_INT, [_P] * 17 + [_F, _I64, _INT, _F, _INT] + [_I64] * 11 + [_P]),
     'slayer_recurrent_bwd': (_INT, [_P] * 5 + [_F, _F, _F, _INT] + [_I64] * 3 + [_P]),
+    'slayer_recurrent_steps_workspace': (_I64, [_I64, _I64, _I64, _INT]),
+    'slayer_cuba_recurrent_steps_fwd': (_INT, [_P] * 10 + [_F, _INT, _F, _INT] + [_I64] * 7 + [_P, _I64, _P]),
+    'slayer_alif_recurrent_steps_fwd': (_INT, [_P] * 17 + [_F, _I64, _INT, _F, _INT] + [_I64] * 11 + [_P, _I64, _P]),
+    'slayer_recurrent_steps_bwd': (_INT, [_P] * 5 + [_F, _F, _F, _INT] + [_I64] * 3 + [_P, _I64, _P]),
     'slayer_li_fwd_naive': (_INT, [_P, _P, _P, _P, _D, _INT, _I64, _I64, _I64, _I64, _I64, _P]),
     'slayer_li_bwd_naive': (_INT, [_P, _P, _P, _I64, _I64, _I64, _I64, _P]),
     'slayer_ath_fwd_naive': (_INT, [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _INT,

@@ -122,10 +122,11 @@ class _CubaFused(torch.autograd.Function):
         threshold, tau_rho, scale_rho, graded = ctx.cfg
         need = (ctx.needs_input_grad[1] or ctx.needs_input_grad[2]) and cur is not None
         grad_spikes = grad_spikes.contiguous()
+        folded = D.fold(ctx.delays, grad_spikes, forward=False, delayed_spikes=spk) if ctx.delays else None
         g_in, g_i, g_v = _bwd(grad_spikes, vol, cur, i_decay.detach(), v_decay.detach(),
                               threshold, tau_rho, scale_rho, graded, need,
-                              D.fold(ctx.delays, grad_spikes, forward=False) if ctx.delays else None)
+                              folded)
         if g_i is not None:
             g_i, g_v = g_i.reshape(i_decay.shape), g_v.reshape(v_decay.shape)
-        g_delay = D.output_delay_gradient(ctx.delays, grad_spikes, spk) if spk is not None else None
+        g_delay = D.delay_gradient(ctx.delays, folded)
         return (g_in, g_i, g_v) + (None,) * 10 + (g_delay,)

@@ -76,9 +76,10 @@ def _table(value, npb, dev, what):
 
 class Folded:
     """The C structure for one call, the tensors it points into (kept alive with it) and the tensor that
-    receives the last undelayed spike."""
+    receives the last undelayed spike.  A backward call given the delayed spikes of the forward pass also
+    asks for the gradient of the spike delay (``grad_sum``: one entry per neuron, summed over batch and time)."""
 
-    def __init__(self, delays, like, forward):
+    def __init__(self, delays, like, forward, delayed_spikes=None):
         dev = like.device
         npb = N.neurons_per_batch(like)
         ts = delays.sampling_time
@@ -93,42 +94,44 @@ class Folded:
             if delays.output_head is not None:
                 head = delays.output_head.detach().to(device=dev, dtype=torch.float32).expand(like.shape[:-1]) \
                     .contiguous()
-        self.keep = (in_lut, out_lut, head)
+        self.grad_sum = workspace = None
+        if delayed_spikes is not None and not forward:
+            delayed_spikes = delayed_spikes.contiguous()
+            M = delayed_spikes.numel() // max(delayed_spikes.shape[-1], 1)
+            self.grad_sum = torch.empty(npb, dtype=torch.float32, device=dev)
+            workspace = torch.empty(M + 64 * npb, dtype=torch.float32, device=dev)
+        else:
+            delayed_spikes = None
+        self.keep = (in_lut, out_lut, head, delayed_spikes, workspace)
         self.out_lut, self.out_steps = out_lut, out_steps
         self.struct = N.Delays(N.ptr(in_lut), N.ptr(out_lut), N.ptr(head), N.ptr(self.spike_last),
-                               in_steps, out_steps, float(ts))
+                               in_steps, out_steps, float(ts),
+                               N.ptr(delayed_spikes), N.ptr(self.grad_sum), N.ptr(workspace))
 
     @property
     def ref(self):
         return ctypes.byref(self.struct)
 
 
-def fold(delays, like, forward=True):
-    """``Folded`` for a ``Delays`` that folds anything, else None (the kernels then take their plain form)."""
-    return Folded(delays, like, forward) if delays else None
+def fold(delays, like, forward=True, delayed_spikes=None):
+    """``Folded`` for a ``Delays`` that folds anything, else None (the kernels then take their plain form).
+    ``delayed_spikes`` (backward only): the spikes the forward pass stored, when the spike delay is trained."""
+    return Folded(delays, like, forward, delayed_spikes) if delays else None
+
+
+def delay_gradient(delays, folded):
+    """Gradient of ``delays.output_delay`` from what a fused backward call left in ``folded.grad_sum``
+    (axon/delay.py:201-221 in the reference: the sum times the sampling time times ``grad_scale``)."""
+    if folded is None or folded.grad_sum is None:
+        return None
+    grad = folded.grad_sum * delays.sampling_time * delays.grad_scale
+    if delays.output_delay.numel() == 1:
+        grad = grad.sum()
+    return grad.reshape(delays.output_delay.shape)
 
 
 def ref(folded):
     return None if folded is None else folded.ref
-
-
-def output_delay_gradient(delays, grad_spikes, spikes):
-    """Gradient of ``delays.output_delay``: what ``axon.Delay``'s backward pass computes from the delayed
-    spikes and their gradient (axon/delay.py:201-221), sums only (8 bytes per neuron-timestep)."""
-    dev = grad_spikes.device
-    grad_spikes, spikes = grad_spikes.contiguous(), spikes.contiguous()
-    M, T = N.rows_and_steps(grad_spikes)
-    npb = N.neurons_per_batch(grad_spikes)
-    ts = delays.sampling_time
-    grad_sum = torch.empty(npb, dtype=torch.float32, device=dev)
-    workspace = torch.empty(M + 64 * npb, dtype=torch.float32, device=dev)
-    with N.device_guard(dev):
-        N.check(N.lib().slayer_delay_bwd(None, N.ptr(grad_sum), N.ptr(grad_spikes), N.ptr(spikes), None, 0,
-                                         float(ts), N.ptr(workspace), M, npb, T, N.stream_handle()))
-    grad = grad_sum * ts * delays.grad_scale
-    if delays.output_delay.numel() == 1:
-        grad = grad.sum()
-    return grad.reshape(delays.output_delay.shape)
 
 
 def chain_input(delays, input):

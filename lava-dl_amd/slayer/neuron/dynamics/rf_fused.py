@@ -112,12 +112,13 @@ class _RfFused(torch.autograd.Function):
         threshold, tau_rho, scale_rho, graded = ctx.cfg
         need = ctx.needs_input_grad[2] or ctx.needs_input_grad[3]
         grad_spikes = grad_spikes.contiguous()
+        folded = D.fold(ctx.delays, grad_spikes, forward=False, delayed_spikes=spk) if ctx.delays else None
         g_re, g_im, g_sin, g_cos = _bwd(grad_spikes, real, imag, sin_decay.detach(), cos_decay.detach(),
                                         threshold, tau_rho, scale_rho, graded, need,
-                                        D.fold(ctx.delays, grad_spikes, forward=False) if ctx.delays else None)
+                                        folded)
         _res._raise_on_nan(grad_spikes=grad_spikes, grad_real_input=g_re, grad_imag_input=g_im,
                            grad_sin_decay=g_sin, grad_cos_decay=g_cos)
         if g_sin is not None:
             g_sin, g_cos = g_sin.reshape(sin_decay.shape), g_cos.reshape(cos_decay.shape)
-        g_delay = D.output_delay_gradient(ctx.delays, grad_spikes, spk) if spk is not None else None
+        g_delay = D.delay_gradient(ctx.delays, folded)
         return (g_re, g_im, g_sin, g_cos) + (None,) * 10 + (g_delay,)

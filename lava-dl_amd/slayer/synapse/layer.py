@@ -1,0 +1,145 @@
+"""Convolution synapse on time-innermost tensors.
+
+Interface of lava.lib.dl.slayer.synapse.Conv (synapse/layer.py:178-323 in the reference): a spatial convolution
+applied at every time step of an NCHWT tensor.  The reference calls ``F.conv3d`` with a kernel of (kh, kw, 1); the
+library behind it wants channels last and transposes the tensor there and back around its kernel.  Here
+slayer_conv_synapse of libslayer_hip.so computes it where the tensor lies, so the neuron that follows reads the
+result in place.  What the kernel does not take (grouped convolutions, rows that are not whole quads of time steps)
+goes to ``F.conv3d`` as before; the weight gradient always does (``torch.nn.grad.conv3d_weight``).
+"""
+import torch
+import torch.nn.functional as F
+
+from .. import _native as N
+
+_ERANGE = -3
+
+
+def _pair(v, what):
+    if isinstance(v, int):
+        return (v, v)
+    if len(v) == 2:
+        return (int(v[0]), int(v[1]))
+    raise Exception(f'{what} can be either int or tuple of size 2. Found {v}')
+
+
+def _launch(input, weight4, stride, padding, dilation):
+    """out or None (None: outside what the kernel takes).  weight4: [Co, Ci, kh, kw]."""
+    n, ci, h, w, t = input.shape
+    co, _, kh, kw = weight4.shape
+    ho = (h + 2 * padding[0] - dilation[0] * (kh - 1) - 1) // stride[0] + 1
+    wo = (w + 2 * padding[1] - dilation[1] * (kw - 1) - 1) // stride[1] + 1
+    if ho < 1 or wo < 1:
+        raise RuntimeError(f'convolution kernel {kh}x{kw} does not fit an image of {h}x{w}')
+    out = torch.empty((n, co, ho, wo, t), dtype=torch.float32, device=input.device)
+    with N.device_guard(input.device):
+        code = N.lib().slayer_conv_synapse(N.ptr(out), N.ptr(input), N.ptr(weight4), n, ci, co, h, w, t, kh, kw,
+                                           stride[0], stride[1], padding[0], padding[1], dilation[0], dilation[1],
+                                           N.stream_handle())
+    if code == _ERANGE:
+        return None
+    N.check(code)
+    return out
+
+
+class _ConvSynapse(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input, weight, stride, padding, dilation):
+        out = _launch(input, weight.detach()[..., 0].contiguous(), stride, padding, dilation)
+        if out is None:
+            raise RuntimeError('not a shape the kernel takes')       # conv_synapse() checks before it gets here
+        ctx.save_for_backward(input, weight)
+        ctx.cfg = (stride, padding, dilation)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        input, weight = ctx.saved_tensors
+        stride, padding, dilation = ctx.cfg
+        grad_output = grad_output.contiguous()
+        grad_input = grad_weight = None
+        if ctx.needs_input_grad[0]:
+            kh, kw = weight.shape[2], weight.shape[3]
+            if stride == (1, 1):
+                # the same convolution on the gradient, weights transposed and flipped
+                flipped = weight.detach()[..., 0].flip(2, 3).transpose(0, 1).contiguous()
+                back = (dilation[0] * (kh - 1) - padding[0], dilation[1] * (kw - 1) - padding[1])
+                if back[0] >= 0 and back[1] >= 0:
+                    grad_input = _launch(grad_output, flipped, (1, 1), back, dilation)
+            if grad_input is None or grad_input.shape != input.shape:
+                grad_input = torch.nn.grad.conv3d_input(input.shape, weight, grad_output, stride + (1,),
+                                                        padding + (0,), dilation + (1,), 1)
+        if ctx.needs_input_grad[1]:
+            grad_weight = torch.nn.grad.conv3d_weight(input, weight.shape, grad_output, stride + (1,), padding + (0,),
+                                                      dilation + (1,), 1)
+        return grad_input, grad_weight, None, None, None
+
+
+def conv_synapse(input, weight, stride=1, padding=0, dilation=1, groups=1):
+    """``F.conv3d(input, weight, None, stride + (1,), padding + (0,), dilation + (1,), groups)`` for an NCHWT
+    ``input`` and a ``weight`` of [Co, Ci / groups, kh, kw, 1], computed in place of the layout when the kernel
+    takes the shape (one group, float32 on the GPU, T a multiple of 4), by the library call otherwise."""
+    stride, padding, dilation = _pair(stride, 'stride'), _pair(padding, 'padding'), _pair(dilation, 'dilation')
+    takes = (groups == 1 and input.is_cuda and input.dtype == torch.float32 and weight.dtype == torch.float32
+             and input.dim() == 5 and weight.dim() == 5 and weight.shape[-1] == 1 and input.shape[-1] % 4 == 0
+             and input.shape[1] * weight.shape[2] * weight.shape[3] <= 860 and input.numel() > 0
+             and input[0].numel() * 4 < 2 ** 31)
+    if takes:
+        input = input.contiguous()
+        takes = input.data_ptr() % 16 == 0
+    if not takes:
+        return F.conv3d(input, weight, None, stride + (1,), padding + (0,), dilation + (1,), groups)
+    return _ConvSynapse.apply(input, weight, stride, padding, dilation)
+
+
+class Conv(torch.nn.Conv3d):
+    """Convolution synapse layer (synapse/layer.py:178-323 in the reference).
+
+    Parameters
+    ----------
+    in_features, out_features : int
+    kernel_size, stride, padding, dilation : int or (height, width)
+    groups : int
+    weight_scale : int
+        weight initialization scale factor.
+    weight_norm : bool
+        weight normalization (``torch.nn.utils.weight_norm`` over the output channels, as in the reference).
+    pre_hook_fx : callable or None
+        applied to the weight before every forward pass (typically a quantizer).
+    """
+
+    def __init__(self, in_features, out_features, kernel_size, stride=1, padding=0, dilation=1, groups=1,
+                 weight_scale=1, weight_norm=False, pre_hook_fx=None):
+        kernel = _pair(kernel_size, 'kernel_size')
+        self._stride2, self._padding2, self._dilation2 = _pair(stride, 'stride'), _pair(padding, 'padding'), \
+            _pair(dilation, 'dilation')
+        super().__init__(in_features, out_features, kernel + (1,), self._stride2 + (1,), self._padding2 + (0,),
+                         self._dilation2 + (1,), groups, bias=False)
+        if weight_scale != 1:
+            self.weight = torch.nn.Parameter(weight_scale * self.weight)
+        self._pre_hook_fx = pre_hook_fx
+        self.weight_norm_enabled = False
+        self.complex = False
+        if weight_norm is True:
+            self.enable_weight_norm()
+
+    def enable_weight_norm(self):
+        torch.nn.utils.weight_norm(self, name='weight')
+        self.weight_norm_enabled = True
+
+    def disable_weight_norm(self):
+        torch.nn.utils.remove_weight_norm(self, name='weight')
+        self.weight_norm_enabled = False
+
+    @property
+    def pre_hook_fx(self):
+        return self._pre_hook_fx
+
+    @pre_hook_fx.setter
+    def pre_hook_fx(self, fx):
+        self._pre_hook_fx = fx
+
+    def forward(self, input):
+        """Weighted spikes [N, out_features, Ho, Wo, T] for spikes [N, in_features, H, W, T]."""
+        weight = self.weight if self._pre_hook_fx is None else self._pre_hook_fx(self.weight)
+        return conv_synapse(input, weight, self._stride2, self._padding2, self._dilation2, self.groups)

@@ -1,10 +1,11 @@
 """Recurrent spiking layer: ``s[t] = neuron(z[t] + R s[t-1])``.
 
 Interface of lava.lib.dl.slayer.utils.recurrent (utils/recurrent.py:7-112 in the reference).
-For a CUBA or an ALIF neuron on the GPU (binary or graded spikes, up to 1024 neurons per sample) the
-whole time loop is one kernel launch per direction (slayer_cuba_recurrent_fwd /
-slayer_alif_recurrent_fwd / slayer_recurrent_bwd); any other neuron runs the reference's loop of
-one-step neuron calls.
+For a CUBA or an ALIF neuron on the GPU (binary or graded spikes) the time loop runs inside the library: up to
+``ONE_LAUNCH_MAX`` neurons per sample as one kernel launch per direction (slayer_cuba_recurrent_fwd /
+slayer_alif_recurrent_fwd / slayer_recurrent_bwd), wider layers (a multiple of 4 up to 16384 neurons) as one
+launch per time step that multiplies the recurrent matrix with the whole batch (slayer_*_recurrent_steps_*); any
+other neuron runs the reference's loop of one-step neuron calls.
 """
 import torch
 
@@ -42,10 +43,22 @@ def custom_recurrent_ground_truth_2(z, neuron, recurrent_synapse):
     return x
 
 
+ONE_LAUNCH_MAX = 1024       # neurons per sample of the one-launch kernels (one thread per neuron)
+STEPS_MAX = 16384           # ... of the launch-per-step kernels
+
+
+def _by_steps(c):
+    """True for the layer widths that take the launch-per-step kernels."""
+    return c > ONE_LAUNCH_MAX
+
+
 def _fusable(z, neuron):
     from ..neuron import alif, cuba
-    return (type(neuron) in (cuba.Neuron, alif.Neuron) and z.is_cuda and z.dim() == 3 and z.dtype == torch.float32
-            and neuron.norm is None and neuron.drop is None and neuron.persistent_state and z.shape[1] <= 1024)
+    if not (type(neuron) in (cuba.Neuron, alif.Neuron) and z.is_cuda and z.dim() == 3 and z.dtype == torch.float32
+            and neuron.norm is None and neuron.drop is None and neuron.persistent_state):
+        return False
+    c = z.shape[1]
+    return c <= ONE_LAUNCH_MAX or (c % 4 == 0 and c <= STEPS_MAX and z.shape[0] * c < 2 ** 29)
 
 
 def custom_recurrent(z, neuron, recurrent_synapse):
@@ -54,8 +67,9 @@ def custom_recurrent(z, neuron, recurrent_synapse):
     last step.  Gradients reach ``z`` and the recurrent weights; as in the reference, the state the
     neuron carries from one step to the next is treated as a constant.
 
-    The one-launch kernel adds the feedback row by row in the order the neurons fired, 16 at a time, where
-    the reference's loop calls ``torch.matmul``.  The two sums are the same bits whenever every partial sum
+    The one-launch kernel adds the feedback row by row in the order the neurons fired, 16 at a time, the
+    launch-per-step kernels in a fixed order of their own on the matrix cores (float32), where
+    the reference's loop calls ``torch.matmul``.  The sums are the same bits whenever every partial sum
     is exactly representable in float32, which holds for quantised recurrent weights (multiples of a power
     of two of moderate size, what the synapse's ``pre_hook_fx`` quantiser produces).  With unquantised
     weights the sums can differ in the last bit and a dendrite value within that distance of the threshold
@@ -108,8 +122,18 @@ def _weight_gradient(grad_z, x):
     return torch.matmul(grad_output, spikes_in)
 
 
+def _steps_workspace(n, c, t, with_theta, dev):
+    """Scratch memory of a launch-per-step entry point.  The caller holds the tensor until the launches are in the
+    stream; torch's allocator hands its memory to later work of the same stream only."""
+    floats = N.lib().slayer_recurrent_steps_workspace(n, c, t, 1 if with_theta else 0)
+    if floats < 0:
+        N.check(int(floats))
+    return torch.empty(floats, dtype=torch.float32, device=dev)
+
+
 class _FusedRecurrent(torch.autograd.Function):
-    """The whole time loop of a CUBA or an ALIF layer as one launch per direction."""
+    """The whole time loop of a CUBA or an ALIF layer inside the library: one launch per direction, or one per
+    time step for wide layers."""
 
     @staticmethod
     def forward(ctx, z, neuron, recurrent_mat):
@@ -120,7 +144,7 @@ class _FusedRecurrent(torch.autograd.Function):
         neuron._prepare(z)
         n, c, t = z.shape
         rec = recurrent_mat.detach().to(dev).float().contiguous()
-        rec_t = torch.cat([rec.transpose(0, 1), rec.new_zeros(1, c)], dim=0).contiguous()   # + the zero row
+        by_steps = _by_steps(c)
         is_alif = type(neuron) is alif.Neuron
         names = ('current', 'voltage') + (('threshold', 'refractory') if is_alif else ())
         decays = [neuron._q(f'{k}_decay', True).detach().contiguous() for k in names]
@@ -129,22 +153,30 @@ class _FusedRecurrent(torch.autograd.Function):
         theta = torch.empty_like(z) if is_alif else None
         last = [torch.empty_like(s) for s in states]
         graded = 1 if neuron.graded_spike else 0
+        if by_steps:
+            mat, ws = rec, _steps_workspace(n, c, t, is_alif, dev)
+            tail = (N.ptr(ws), ws.numel())
+            entry = 'slayer_alif_recurrent_steps_fwd' if is_alif else 'slayer_cuba_recurrent_steps_fwd'
+        else:
+            mat = torch.cat([rec.transpose(0, 1), rec.new_zeros(1, c)], dim=0).contiguous()   # R^T + the zero row
+            tail = ()
+            entry = 'slayer_alif_recurrent_fwd' if is_alif else 'slayer_cuba_recurrent_fwd'
         with N.device_guard(dev):
             if is_alif:
                 threshold = 0.0
-                N.check(N.lib().slayer_alif_recurrent_fwd(
-                    N.ptr(spk), N.ptr(vol), N.ptr(theta), *[N.ptr(x) for x in last], N.ptr(z), N.ptr(rec_t),
+                N.check(getattr(N.lib(), entry)(
+                    N.ptr(spk), N.ptr(vol), N.ptr(theta), *[N.ptr(x) for x in last], N.ptr(z), N.ptr(mat),
                     *[N.ptr(d) for d in decays], *[N.ptr(s) for s in states],
                     float(neuron.threshold_step), int(neuron.threshold * neuron.s_scale), graded, 1.0,
                     int(neuron.s_scale), n, c, *[d.numel() for d in decays], *[s.numel() for s in states], t,
-                    N.stream_handle()))
+                    *tail, N.stream_handle()))
             else:
                 threshold = neuron.threshold + neuron.threshold_eps
-                N.check(N.lib().slayer_cuba_recurrent_fwd(
-                    N.ptr(spk), N.ptr(vol), *[N.ptr(x) for x in last], N.ptr(z), N.ptr(rec_t),
+                N.check(getattr(N.lib(), entry)(
+                    N.ptr(spk), N.ptr(vol), *[N.ptr(x) for x in last], N.ptr(z), N.ptr(mat),
                     *[N.ptr(d) for d in decays], *[N.ptr(s) for s in states],
                     float(threshold), graded, 1.0, int(neuron.s_scale), n, c,
-                    *[d.numel() for d in decays], *[s.numel() for s in states], t, N.stream_handle()))
+                    *[d.numel() for d in decays], *[s.numel() for s in states], t, *tail, N.stream_handle()))
         neuron.current_state = last[0]
         if is_alif:
             neuron.voltage_state = last[1]
@@ -167,8 +199,16 @@ class _FusedRecurrent(torch.autograd.Function):
         grad_x = grad_x.contiguous()
         n, c, t = grad_x.shape
         grad_z = torch.empty_like(grad_x)
+        th = N.ptr(theta[0]) if theta else None
         with N.device_guard(dev):
-            N.check(N.lib().slayer_recurrent_bwd(
-                N.ptr(grad_z), N.ptr(grad_x), N.ptr(vol), N.ptr(theta[0]) if theta else None, N.ptr(rec),
-                threshold, tau_rho, scale_rho, graded, n, c, t, N.stream_handle()))
+            if _by_steps(c):
+                rec_t = rec.transpose(0, 1).contiguous()
+                ws = _steps_workspace(n, c, t, bool(theta), dev)
+                N.check(N.lib().slayer_recurrent_steps_bwd(
+                    N.ptr(grad_z), N.ptr(grad_x), N.ptr(vol), th, N.ptr(rec_t),
+                    threshold, tau_rho, scale_rho, graded, n, c, t, N.ptr(ws), ws.numel(), N.stream_handle()))
+            else:
+                N.check(N.lib().slayer_recurrent_bwd(
+                    N.ptr(grad_z), N.ptr(grad_x), N.ptr(vol), th, N.ptr(rec),
+                    threshold, tau_rho, scale_rho, graded, n, c, t, N.stream_handle()))
         return grad_z, None, _weight_gradient(grad_z, spk)

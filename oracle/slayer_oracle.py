@@ -511,6 +511,18 @@ def sigma_fwd(x, pre_state=None):
     return out
 
 
+# --------------------------------------------------------------------------- convolution synapse
+def conv_synapse(x, weight, stride=(1, 1), padding=(0, 0), dilation=(1, 1), groups=1):
+    """synapse/layer.py:297-323 in the reference: ``F.conv3d`` of an NCHWT tensor with a weight of
+    [Co, Ci / groups, kh, kw, 1], no bias -- a spatial convolution applied at every time step.  The arithmetic is
+    torch's (a dependency of the reference, torch ^2.9, not its own code): evaluated here in float64 and rounded once,
+    and pinned by a direct evaluation of the defining sum on small cases (tests/test_oracle_spec.py)."""
+    import torch.nn.functional as F
+    out = F.conv3d(x.double(), weight.double(), None, tuple(stride) + (1,), tuple(padding) + (0,),
+                   tuple(dilation) + (1,), groups)
+    return out.float()
+
+
 # --------------------------------------------------------------------------- recurrent layer
 def recurrent_cuba_fwd(z, rec, i_decay, v_decay, i_state, v_state, w_scale, threshold, graded=False):
     """Recurrent CUBA layer, S/utils/recurrent.py:45-81 with the CUBA neuron called one step at a

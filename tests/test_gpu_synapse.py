@@ -1,0 +1,102 @@
+"""The convolution synapse on time-innermost tensors (csrc/synapse.hip, slayer.synapse.Conv) against the oracle's
+float64 evaluation of the reference's call (synapse/layer.py:297-323: F.conv3d with a (kh, kw, 1) kernel on NCHWT),
+every output element to 1e-5 of the sum of the magnitudes of its terms; the input gradient against float64 autograd;
+shapes the kernel does not take go to the library call and give the same result."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import slayer_oracle as O
+from tests.util import assert_sum, dev, seed_of
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope='module')
+def slayer():
+    import lava_dl_amd.slayer as s
+    return s
+
+
+def _check(slayer, shape, co, kernel, stride, padding, dilation, what, backward=True):
+    n, ci, h, w, t = shape
+    gen = torch.Generator().manual_seed(seed_of('conv-synapse', shape, co, kernel, stride, padding, dilation))
+    x = (torch.rand(shape, generator=gen) < 0.3).float() * torch.randn(shape, generator=gen)
+    wt = torch.randn(co, ci, kernel[0], kernel[1], 1, generator=gen)
+    xg = x.to(dev()).requires_grad_(backward)
+    wg = wt.to(dev()).requires_grad_(backward)
+    got = slayer.synapse.conv_synapse(xg, wg, stride, padding, dilation)
+    want = O.conv_synapse(x, wt, stride, padding, dilation)
+    mag = O.conv_synapse(x.abs(), wt.abs(), stride, padding, dilation)
+    assert got.shape == want.shape and got.is_contiguous()
+    assert_sum(got, want.double(), mag.double(), what + ' forward')
+    if backward:
+        g = torch.randn(want.shape, generator=gen)
+        got.backward(g.to(dev()))
+        xd, wd = x.double().requires_grad_(), wt.double().requires_grad_()
+        ref = F.conv3d(xd, wd, None, tuple(stride) + (1,), tuple(padding) + (0,), tuple(dilation) + (1,))
+        ref.backward(g.double())
+        # magnitudes of the terms of both gradients: the same sums over absolute values
+        xa, wa = x.abs().double().requires_grad_(), wt.abs().double().requires_grad_()
+        F.conv3d(xa, wa, None, tuple(stride) + (1,), tuple(padding) + (0,), tuple(dilation) + (1,)).backward(g.abs().double())
+        assert_sum(xg.grad, xd.grad, xa.grad, what + ' grad input')
+        assert_sum(wg.grad, wd.grad, wa.grad, what + ' grad weight', rel=1e-4)      # torch's own kernel, float32 sums
+
+
+@pytest.mark.parametrize('shape,co,kernel,stride,padding,dilation', [
+    ((2, 3, 6, 7, 8), 5, (3, 3), (1, 1), (1, 1), (1, 1)),          # fewer than 16 output channels, one short tile
+    ((2, 8, 9, 9, 64), 16, (3, 3), (1, 1), (1, 1), (1, 1)),         # exactly one tile of 64 steps
+    ((1, 2, 34, 34, 300), 16, (5, 5), (2, 2), (2, 2), (1, 1)),      # stride 2, T = 4 tiles + 44 steps
+    ((2, 4, 12, 10, 100), 40, (3, 2), (1, 2), (0, 1), (2, 1)),      # three blocks of output channels, mixed geometry
+    ((3, 16, 8, 8, 36), 32, (1, 1), (1, 1), (0, 0), (1, 1)),        # 1x1: a dense synapse per pixel
+    ((1, 5, 10, 12, 260), 7, (3, 3), (1, 1), (0, 0), (2, 2)),       # no padding, dilation 2
+])
+def test_conv_synapse_against_the_oracle(slayer, shape, co, kernel, stride, padding, dilation):
+    _check(slayer, shape, co, kernel, stride, padding, dilation, f'{shape} -> {co}')
+
+
+def test_conv_module_mirrors_the_reference_layer(slayer):
+    """slayer.synapse.Conv: same constructor and weight shape as the reference layer, pre_hook_fx applied to the
+    weight, gradients reach weight and input."""
+    gen = torch.Generator().manual_seed(3)
+    syn = slayer.synapse.Conv(3, 6, 3, padding=1, weight_scale=2, pre_hook_fx=lambda w: (w * 8).round() / 8).to(dev())
+    assert tuple(syn.weight.shape) == (6, 3, 3, 3, 1) and syn.bias is None
+    x = (torch.rand(2, 3, 8, 8, 40, generator=gen) < 0.2).float().to(dev()).requires_grad_()
+    y = syn(x)
+    want = O.conv_synapse(x.detach().cpu(), ((syn.weight * 8).round() / 8).detach().cpu(), (1, 1), (1, 1), (1, 1))
+    assert float((y.detach().cpu() - want).abs().max()) <= 1e-5 * float(want.abs().max())
+    y.sum().backward()
+    assert syn.weight.grad is not None and x.grad is not None and x.grad.shape == x.shape
+
+
+def test_shapes_the_kernel_does_not_take_go_to_the_library_call(slayer):
+    gen = torch.Generator().manual_seed(4)
+    x = torch.randn(2, 4, 6, 6, 10, generator=gen).to(dev())                 # T % 4 != 0
+    w = torch.randn(6, 4, 3, 3, 1, generator=gen).to(dev())
+    assert torch.equal(slayer.synapse.conv_synapse(x, w, 1, 1, 1), F.conv3d(x, w, None, (1, 1, 1), (1, 1, 0)))
+    w2 = torch.randn(6, 2, 3, 3, 1, generator=gen).to(dev())                 # two groups
+    x2 = torch.randn(2, 4, 6, 6, 12, generator=gen).to(dev())
+    assert torch.equal(slayer.synapse.conv_synapse(x2, w2, 1, 1, 1, groups=2),
+                       F.conv3d(x2, w2, None, (1, 1, 1), (1, 1, 0), (1, 1, 1), 2))
+
+
+def test_conv_synapse_at_the_size_of_the_benchmark_tensor(slayer):
+    """The synapse that produces config[1]'s tensor: spikes [32, 8, 32, 32, 300] -> [32, 16, 32, 32, 300], 3x3,
+    padding 1.  Slabs against the oracle, the whole tensor against the library call within 1e-5 of the terms'
+    magnitudes, and the fused CUBA neuron reads the result where the kernel left it."""
+    gen = torch.Generator(device=dev()).manual_seed(9)
+    shape = (32, 8, 32, 32, 300)
+    x = (torch.rand(shape, device=dev(), generator=gen) < 0.05).float()
+    w = torch.randn(16, 8, 3, 3, 1, device=dev(), generator=gen) * 0.3
+    z = slayer.synapse.conv_synapse(x, w, 1, 1, 1)
+    assert z.shape == (32, 16, 32, 32, 300) and z.is_contiguous()
+    lib = F.conv3d(x, w, None, (1, 1, 1), (1, 1, 0))
+    mag = F.conv3d(x, w.abs(), None, (1, 1, 1), (1, 1, 0))
+    assert bool(((z - lib).abs() <= 1e-5 * mag + 1e-30).all())
+    for n in (0, 31):
+        want = O.conv_synapse(x[n:n + 1].cpu(), w.cpu(), (1, 1), (1, 1), (1, 1))
+        mg = O.conv_synapse(x[n:n + 1].cpu(), w.abs().cpu(), (1, 1), (1, 1), (1, 1))
+        assert_sum(z[n:n + 1], want.double(), mg.double() + 1e-30, f'batch entry {n}')
+    neuron = slayer.neuron.cuba.Neuron(1.0, 0.25, 0.03).to(dev())
+    spikes = neuron(z)
+    assert spikes.shape == z.shape and 0 < float(spikes.sum()) < spikes.numel()

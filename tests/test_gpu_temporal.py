@@ -250,7 +250,7 @@ def test_delay_module(slayer):
     y.backward(g.to(dev()))
     ref_gi, ref_gd = O.delay_bwd(g, O.delay_fwd(x, per_neuron), per_neuron, grad_scale=2.0)
     assert_exact(xg.grad, ref_gi, 'delay grad_input')
-    assert_rel(mod.delay.grad, ref_gd.sum(dim=1), 'delay grad_delay', rel=1e-4)
+    assert_rel(mod.delay.grad, ref_gd.sum(dim=1), 'delay grad_delay')
     # functional form, default one step
     assert_exact(slayer.axon.delay(x.to(dev())), O.shift(x, 1), 'delay()')
 
@@ -275,7 +275,7 @@ def test_delay_backward_kernel(slayer, shape, ts):
     ref_gi, ref_gd = O.delay_bwd(g, y, d, grad_scale=1.0, sampling_time=ts)
     gi, gsum = D._delay_bwd(g.to(dev()), y.to(dev()), d.to(dev()), ts)
     assert_exact(gi, ref_gi, f'delay grad_input {shape}')
-    assert_rel(gsum * ts, ref_gd, f'delay grad_delay {shape}', rel=1e-4)
+    assert_rel(gsum * ts, ref_gd, f'delay grad_delay {shape}')
     # misaligned views take the dword path and must agree with the aligned run
     if shape[-1] % 4 == 0:
         flat = torch.zeros(g.numel() + 1, device=dev())
@@ -326,7 +326,7 @@ def test_delta_unit_and_sigma(slayer, shape, cum):
         w_in, w_thr = O.delta_bwd(g, r_din, thr, 0.8, 1.5)
         g_in, g_thr = D._bwd(g.to(dev()), din, thr.to(dev()), 0.8, 1.5)
         assert_exact(g_in, w_in, 'delta grad_input')
-        assert_rel(g_thr.reshape(w_thr.shape), w_thr, 'delta grad_threshold', rel=1e-4)
+        assert_rel(g_thr.reshape(w_thr.shape), w_thr, 'delta grad_threshold')
     # running sum: float-mode against torch's cumsum, exact against strictly sequential float32 adds,
     # and exact against torch's cumsum on quantised events (multiples of 1/64 add without rounding)
     assert_rel(SG._cumsum(out), O.sigma_fwd(r_out), 'sigma running sum')
@@ -371,7 +371,7 @@ def test_delta_sigma_modules(slayer):
         w_in, w_thr = O.delta_bwd(g_ev, r_din, thr, 1, 1)
         assert_exact(xg.grad, w_in, 'Delta module grad_input')
         assert enc.threshold.grad.shape == enc.threshold.shape
-        assert_rel(enc.threshold.grad.reshape(w_thr.shape), w_thr, 'Delta module grad_threshold', rel=1e-4)
+        assert_rel(enc.threshold.grad.reshape(w_thr.shape), w_thr, 'Delta module grad_threshold')
     # persistent state: two halves equal one pass
     enc_full = slayer.axon.Delta(0.5).to(dev())
     enc_split = slayer.axon.Delta(0.5, persistent_state=True).to(dev())

@@ -515,3 +515,33 @@ def test_delta_bwd_closed_form():
         term = np.where(sub > 0, -dn * 1.5 * np.exp(-np.abs(sub) / 0.8) / th, -np.sign(dn)) * gn
         want = term.sum() if thr.numel() == 1 else term.sum(axis=(0, 2, 3))
         assert np.allclose(g_thr.numpy().ravel(), np.ravel(want), rtol=1e-5, atol=1e-5)
+
+
+def test_conv_synapse_is_the_defining_sum():
+    """The convolution synapse (synapse/layer.py:297-323 in the reference, torch's conv3d with a (kh, kw, 1) kernel):
+    out[n, co, ho, wo, t] = sum over ci, y, x of w[co, ci, y, x] * in[n, ci, ho * s + y * d - p, wo * s + x * d - p, t],
+    written out as loops on small cases, strides, paddings, dilations and groups included.  A transposed kernel, a
+    swapped stride / dilation or a wrong padding origin fails it."""
+    gen = torch.Generator().manual_seed(5)
+    for (ci, co, h, w, kh, kw, st, pd, dl, gr) in [(3, 4, 5, 6, 3, 3, (1, 1), (1, 1), (1, 1), 1),
+                                                   (2, 4, 7, 5, 2, 3, (2, 1), (0, 2), (1, 2), 1),
+                                                   (4, 6, 6, 6, 3, 2, (1, 2), (2, 0), (2, 1), 2)]:
+        x = torch.randn(2, ci, h, w, 3, generator=gen)
+        wt = torch.randn(co, ci // gr, kh, kw, 1, generator=gen)
+        got = O.conv_synapse(x, wt, st, pd, dl, gr).double()
+        ho = (h + 2 * pd[0] - dl[0] * (kh - 1) - 1) // st[0] + 1
+        wo = (w + 2 * pd[1] - dl[1] * (kw - 1) - 1) // st[1] + 1
+        assert got.shape == (2, co, ho, wo, 3)
+        want = torch.zeros(2, co, ho, wo, 3, dtype=torch.float64)
+        per_in, per_out = ci // gr, co // gr
+        for o in range(co):
+            g0 = (o // per_out) * per_in
+            for c in range(per_in):
+                for y in range(kh):
+                    for xk in range(kw):
+                        for a in range(ho):
+                            for b in range(wo):
+                                yy, xx = a * st[0] + y * dl[0] - pd[0], b * st[1] + xk * dl[1] - pd[1]
+                                if 0 <= yy < h and 0 <= xx < w:
+                                    want[:, o, a, b] += float(wt[o, c, y, xk, 0]) * x[:, g0 + c, yy, xx].double()
+        assert float((got - want).abs().max()) < 1e-5

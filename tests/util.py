@@ -98,6 +98,39 @@ def li_bwd_f64(grad_out, a):
     return g, bound
 
 
+def param_sum_f64(terms, num_params):
+    """(sum, sum of magnitudes) in float64 of ``terms`` [N, C, ..., T'] per parameter, addressed as the kernels
+    address decays: one shared value, one per channel, or one per neuron of a batch element."""
+    t = terms.detach().cpu().double()
+    n = t.shape[0]
+    if num_params == 1:
+        return t.sum().reshape(1), t.abs().sum().reshape(1)
+    per_batch = 1
+    for d in t.shape[1:-1]:
+        per_batch *= d
+    r = t.reshape(n, num_params, (per_batch // num_params) * t.shape[-1])
+    return r.sum(dim=(0, 2)), r.abs().sum(dim=(0, 2))
+
+
+def li_decay_grad_f64(grad_in, out, num_decays):
+    """Decay gradient of the leaky integrator from its input gradient and saved output
+    (neuron/dynamics/leaky_integrator.py:250-257 in the reference): sum of grad_in[t+1] * out[t], with the sum of the
+    terms' magnitudes, both in float64, for ``assert_sum``."""
+    return param_sum_f64(grad_in.detach().cpu().double()[..., 1:] * out.detach().cpu().double()[..., :-1], num_decays)
+
+
+def res_decay_grads_f64(g_re_in, g_im_in, re, im, num_decays):
+    """(sin sum, sin magnitudes, cos sum, cos magnitudes) of the resonator's decay gradients
+    (neuron/dynamics/resonator.py:440-467 in the reference) in float64."""
+    gr, gi = g_re_in.detach().cpu().double()[..., 1:], g_im_in.detach().cpu().double()[..., 1:]
+    r, i = re.detach().cpu().double()[..., :-1], im.detach().cpu().double()[..., :-1]
+    s_sum, _ = param_sum_f64(-gr * i + gi * r, num_decays)
+    c_sum, _ = param_sum_f64(gr * r + gi * i, num_decays)
+    _, mag = param_sum_f64((gr * i).abs() + (gi * r).abs(), num_decays)
+    _, mag_c = param_sum_f64((gr * r).abs() + (gi * i).abs(), num_decays)
+    return s_sum, mag, c_sum, mag_c
+
+
 def assert_same_gradient(a, b, what=''):
     """Two evaluations of the same float gradient on the GPU: bit-identical while both are step-by-step
     (small tensors), within 1e-5 of the scale once the scan kernels take over."""
