@@ -644,8 +644,8 @@ class ConvSynapse(Cuba):
     place.  Weights are multiples of 1/64 (quantised, as a SLAYER synapse's are), so the weighted spikes are exact
     and the forward parity check stays bit for bit.  Bytes per neuron-timestep of the output tensor."""
     name = 'Conv synapse (3x3, 8 -> 16 channels) -> fused CUBA neuron, fwd+bwd (input gradient)'
-    ops = [('conv_synapse', 'synapse_conv_kernel', 6), ('cuba_fwd', 'stream_kernel_staged<CubaFwd>', 16),
-           ('cuba_bwd', 'cuba_bwd_scan_kernel', 16), ('conv_synapse_bwd', 'synapse_conv_kernel', 6)]
+    ops = [('conv_synapse', 'synapse_conv_row_kernel', 6), ('cuba_fwd', 'stream_kernel_staged<CubaFwd>', 16),
+           ('cuba_bwd', 'cuba_bwd_scan_kernel', 16), ('conv_synapse_bwd', 'synapse_conv_row_kernel', 6)]
     note = Cuba.note + '; input spikes Bernoulli(0.05) on 8 channels, weights round(N(0, 0.3) * 64) / 64'
     in_channels = 8
 
@@ -747,9 +747,81 @@ class DenseSynapse(Workload):
     parity_slab = (1, slice(32, 64))
 
 
+class Recurrent(Workload):
+    """A recurrent CUBA layer (utils/recurrent.py:45-112 in the reference: s[t] = neuron(z[t] + R s[t-1]), one neuron
+    call per time step in a Python loop), forward and backward with the gradient of the recurrent weights, through
+    the module interface (custom_recurrent).  2048 neurons take the launch-per-step kernels: a step reads the
+    [C x C] matrix once for the whole batch, so the algorithmic bytes per neuron-timestep are those of the tensors
+    (z, spikes, voltage; gradient, voltage, gradient of z) plus 4 C / N for the matrix."""
+    name = 'Recurrent CUBA layer, 2048 neurons, fwd+bwd (module interface)'
+    shape = (32, 2048, 300)
+    ops = [('recurrent_fwd', 'recurrent_step_fwd_kernel, one launch per time step', 12 + 4 * 2048 // 32),
+           ('recurrent_bwd', 'recurrent_step_bwd_kernel, one launch per time step, + weight-gradient GEMM', 12 + 4 * 2048 // 32)]
+    note = ('CUBA decays 0.25 / 0.25, threshold 1.25, z ~ 1.5 N(0,1), weights N(0, 0.6) * 6 / sqrt(C) quantised to '
+            '8 bits (the synapse pre-hook), about 40 % of the neurons spike per step')
+    generic_loop = False
+
+    def __init__(self, dev):
+        super().__init__(dev, 1011)
+        import importlib
+        slayer = importlib.import_module('lava_dl_amd.slayer')
+        self.Rm = slayer.utils.recurrent
+        g = self.gen
+        n, c, t = self.shape
+        self.neuron = slayer.neuron.cuba.Neuron(threshold=1.25, current_decay=0.25, voltage_decay=0.25,
+                                                persistent_state=True).to(dev)
+        self.put(z=torch.randn(self.shape, generator=g) * 1.5, g=torch.rand(self.shape, generator=g),
+                 wgt=torch.randn(c, c, generator=g) * 0.6 * 6.0 / c ** 0.5)
+        self.z.requires_grad_()
+
+        class _Synapse:
+            pass
+        self.syn = _Synapse()
+        self.syn.weight = self.wgt.reshape(c, c, 1, 1, 1).requires_grad_()
+        self.syn.pre_hook_fx = self.neuron.quantize_8bit
+
+    def step(self, t):
+        R, neuron = self.Rm, self.neuron
+        for k in ('current_state', 'voltage_state'):          # every step starts from the initial state
+            neuron._buffers[k] = self.zero
+        self.z.grad = None
+        self.syn.weight.grad = None
+        with t('recurrent_fwd'):
+            if self.generic_loop:
+                out = R.CustomRecurrent.apply(self.z, neuron, R._recurrent_matrix(self.syn))
+            else:
+                out = R.custom_recurrent(self.z, neuron, self.syn)
+        with t('recurrent_bwd'):
+            out.backward(self.g)
+        return out.detach(), self.z.grad
+
+    def cpu_step(self, n, sl=None):
+        from oracle import slayer_oracle as O
+        c = self.cpu
+        neuron = self.neuron
+        rec = neuron.quantize_8bit(c['wgt'])
+        d_i, d_v = neuron.current_decay.detach().round().cpu(), neuron.voltage_decay.detach().round().cpu()
+        thr = neuron.threshold + neuron.threshold_eps
+        zero = torch.tensor([0.0])
+        spk, vol, _, _ = O.recurrent_cuba_fwd(c['z'][:n], rec, d_i, d_v, zero, zero, int(neuron.s_scale), thr)
+        g_z, _ = O.recurrent_cuba_bwd(c['g'][:n], spk, vol, rec, thr, neuron.tau_rho * 100, neuron.scale_rho * 0.1)
+        return spk[:, sl], g_z[:, sl]
+
+    parity_slab = (1, slice(0, 2048))
+
+
+class RecurrentLoop(Recurrent):
+    """The same layer through the reference's loop of one-step neuron calls (CustomRecurrent, the path layers take
+    that the kernels do not cover)."""
+    name = 'Recurrent CUBA layer, 2048 neurons, fwd+bwd: loop of one-step neuron calls'
+    ops = [('recurrent_fwd', 'a dozen launches per time step (one-step neuron calls + torch.matmul)', 12 + 4 * 2048 // 32),
+           ('recurrent_bwd', 'autograd of every step + torch.matmul', 12 + 4 * 2048 // 32)]
+    generic_loop = True
+
+
 WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fused_lean': CubaFusedLean, 'cuba_inference': CubaInference, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'alif_fused': AlifFused, 'alif_fused_lean': AlifFusedLean, 'rf': Rf, 'rf_fused': RfFused, 'rf_fused_lean': RfFusedLean, 'rf_inference': RfInference, 'synapse': Synapse, 'synapse_fused': SynapseFused, 'synapse_folded': SynapseFolded, 'synapse_delay_grad': SynapseDelayGrad, 'block_tail': BlockTail, 'block_tail_folded': BlockTailFolded,
              'conv_synapse': ConvSynapse, 'conv_synapse_library': ConvSynapseLibrary,
-             'dense_synapse': DenseSynapse}
+             'dense_synapse': DenseSynapse, 'recurrent': Recurrent, 'recurrent_loop': RecurrentLoop}
 
 
 def cpu_baseline(job, budget_s=20.0):
@@ -832,7 +904,7 @@ def timed_median(job, iters, warmup):
 # sequence of the configuration, then the fused forms with their own smaller byte counts).
 OTHER = ['cuba_fwd_small', 'cuba_fused', 'cuba_fused_lean', 'alif', 'alif_fused', 'alif_fused_lean', 'rf', 'rf_fused',
          'synapse', 'synapse_fused', 'synapse_folded', 'block_tail', 'block_tail_folded',
-         'conv_synapse', 'conv_synapse_library']
+         'conv_synapse', 'conv_synapse_library', 'recurrent', 'recurrent_loop']
 
 
 def other_configs(dev, iters):

@@ -508,11 +508,12 @@ int slayer_recurrent_bwd(float *grad_z, const float *grad_spikes, const float *v
  * A step multiplies the weight matrix with the spikes of the previous step for the whole batch (the matrix is read
  * once per step, on the matrix cores in float32) and runs one neuron step on the result; the launches follow each
  * other on `stream`.  Same arguments, results and arithmetic as slayer_cuba_recurrent_fwd / slayer_alif_recurrent_fwd
- * except: `rec` is R itself, [C][C] (row c = the weights that reach neuron c), 16-byte aligned like the *_last
- * outputs; the feedback of a step is summed in a fixed order of its own (equal bits whenever the sums are exact in
+ * except: `rec` is R itself, [C][C] (row c = the weights that reach neuron c); the *_last outputs are 16-byte
+ * aligned; the feedback of a step is summed in a fixed order of its own (equal bits whenever the sums are exact in
  * float32, e.g. quantised weights and binary spikes); `workspace` is device memory of at least
  * slayer_recurrent_steps_workspace(N, C, T, alif) floats, 16-byte aligned, whose contents are undefined afterwards
- * (time-major copies of the tensors and the states between two steps).
+ * (time-major copies of the tensors, the weight matrix in the order the matrix cores read it, the states and the
+ * spikes that one step hands to the next).
  * slayer_recurrent_steps_workspace returns the number of floats (with_theta != 0: an ALIF layer), or a negative
  * error code for sizes the entry points refuse (SLAYER_ERANGE: C % 4 != 0, C > 16384, N * C >= 2^29). */
 int64_t slayer_recurrent_steps_workspace(int64_t N, int64_t C, int64_t T, int with_theta);
@@ -539,10 +540,10 @@ int slayer_alif_recurrent_steps_fwd(float *spk_out, float *vol_out, float *theta
                                     int64_t num_ref_states,
                                     int64_t T, float *workspace, int64_t workspace_floats, void *stream);
 
-/* slayer_recurrent_bwd one launch per time step (see above); rec_t = R transposed, [C][C], 16-byte aligned:
- * row c holds the weights that leave neuron c.  Workspace as above (with_theta = theta != NULL). */
+/* slayer_recurrent_bwd one launch per time step (see above); rec = R, [C][C], as for slayer_recurrent_bwd.
+ * Workspace as above (with_theta = theta != NULL). */
 int slayer_recurrent_steps_bwd(float *grad_z, const float *grad_spikes, const float *voltage, const float *theta,
-                               const float *rec_t, float spike_threshold, float tau_rho, float scale_rho, int graded,
+                               const float *rec, float spike_threshold, float tau_rho, float scale_rho, int graded,
                                int64_t N, int64_t C, int64_t T,
                                float *workspace, int64_t workspace_floats, void *stream);
 

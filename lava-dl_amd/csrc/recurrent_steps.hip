@@ -5,13 +5,19 @@
 //
 // A step is one product of the [C x C] weight matrix with the [N x C] spikes of the previous step -- the matrix
 // is read once per step for the whole batch -- followed by one neuron step of every (sample, neuron).  A workgroup
-// owns 16 neurons for up to 64 samples: its eight waves each take an eighth of the sum over the presynaptic
+// owns 16 neurons for up to 64 samples: its four waves each take a quarter of the sum over the presynaptic
 // neurons on the matrix cores (v_mfma_f32_16x16x4_f32: float32 operands and accumulation; the products of a 0/1
 // spike are exact, and so is every partial sum of quantised weights), the partial sums meet in LDS, and the first
 // waves run the neuron step on the result: lane (q, j) of a 16 x 16 result tile holds neurons 4q .. 4q+3 of sample
 // j, a quad of neighbouring floats in every time-major tensor.  The launches of consecutive steps follow each
 // other in the stream; what a step hands to the next lies in memory: the spikes (the slab of the time-major spike
 // tensor just written) and the integer states.
+//
+// Both operands of the product are read in the order the matrix cores want them: the weight matrix is re-packed
+// once per call (pack_weights_kernel: per tile of 16 neurons and block of 16 k, the 64 quads of the 64 lanes one
+// after the other -- a wave-wide load is one contiguous kilobyte instead of sixteen rows a power of two apart), and
+// a step leaves its spikes in the same order next to the time-major slab (the quad a lane of the neuron step holds
+// is the quad the same lane of the next step's product loads).
 //
 // The tensors of the interface are [N, C, T] with time innermost; a step touches one sample of every row.  The
 // input is therefore copied to a time-major workspace ([T][N][C]) once, the steps read and write slabs of
@@ -26,8 +32,14 @@
 
 namespace slayer {
 
-constexpr int kStepWaves = 8;            // waves per workgroup: each takes an eighth of the sum over k
-constexpr int kStepUnroll = 4;           // blocks of 16 k a wave keeps in flight
+#ifndef SLAYER_STEP_WAVES
+#define SLAYER_STEP_WAVES 4
+#endif
+#ifndef SLAYER_STEP_QUADS
+#define SLAYER_STEP_QUADS 16
+#endif
+constexpr int kStepWaves = SLAYER_STEP_WAVES;   // waves per workgroup: each takes its share of the sum over k
+constexpr int kStepQuads = SLAYER_STEP_QUADS;   // operand quads (weights and activations) a lane keeps in flight
 constexpr int kStepMaxC = 16384;         // 32-bit byte offsets into the weight matrix
 
 typedef float step_f4 __attribute__((ext_vector_type(4)));
@@ -59,34 +71,48 @@ __global__ __launch_bounds__(256) void time_major_kernel(float* __restrict__ dst
     }
 }
 
+// Packed operands.  Weights: wp[tile][kb][lane] (float4) = w[16 tile + j][16 kb + 4 kk .. + 3] for lane = 16 kk + j,
+// zero beyond the matrix.  Activations: ap[kb][s][lane] (float4) = act[16 s + j][16 kb + 4 kk .. + 3], zero beyond
+// the batch and the layer; S = sample tiles, a multiple of the tiles a workgroup takes.
+template <bool TRANSPOSED>
+__global__ __launch_bounds__(kWave) void pack_weights_kernel(float4* __restrict__ wp, const float* __restrict__ w, int C,
+                                                             int KB) {
+    const int lane = threadIdx.x, kk = lane >> 4, j = lane & 15;
+    const int kb = blockIdx.x, tile = blockIdx.y;
+    const int row = 16 * tile + j, k = 16 * kb + 4 * kk;
+    float v[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const bool ok = row < C && k + e < C;
+        v[e] = ok ? (TRANSPOSED ? w[(int64_t)(k + e) * C + row] : w[(int64_t)row * C + k + e]) : 0.f;
+    }
+    wp[((int64_t)tile * KB + kb) * kWave + lane] = make_float4(v[0], v[1], v[2], v[3]);
+}
+
 // sum over k of w[c0 + 4q + i][k] * act[n0 + 16 s + j][k] for this thread's (s, q, j) = (tid / 64, lane / 16,
-// lane % 16), i = 0 .. 3: valid in the threads tid < 64 NT, after one workgroup barrier.  Lane (kk, j) of a wave
-// loads k = kb + 4 kk .. + 3 of weight row c0 + j and of sample row n0 + 16 s + j; element e of the two quads are
-// the operands of one matrix product, so a block of 16 k is four of them.
+// lane % 16), i = 0 .. 3: valid in the threads tid < 64 NT, after one workgroup barrier.  Element e of a lane's two
+// quads are the operands of one matrix product, so a block of 16 k is four of them; wave v takes blocks v, v + 4, ...
 template <int NT>
-__device__ __forceinline__ float4 step_product(const float* __restrict__ w, const float* __restrict__ act, int N,
-                                               int C, int n0, int c0, float4 (*red)[NT][kWave]) {
+__device__ __forceinline__ float4 step_product(const float4* __restrict__ wp, const float4* __restrict__ ap, int KB,
+                                               int S, int s0, float4 (*red)[NT][kWave]) {
+    constexpr int kStepUnroll = kStepQuads / (1 + NT) < 2 ? 2 : kStepQuads / (1 + NT);
     const int tid = threadIdx.x, lane = tid & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int kk = lane >> 4, j = lane & 15;
-    const int w_rows = (C - c0) < 16 ? (C - c0) : 16;
-    const int a_rows = (N - n0) < 16 * NT ? (N - n0) : 16 * NT;
-    const __amdgpu_buffer_rsrc_t wr = make_rsrc(w + (int64_t)c0 * C, (unsigned)(w_rows * C * 4));
-    const __amdgpu_buffer_rsrc_t ar = make_rsrc(act + (int64_t)n0 * C, (unsigned)(a_rows * C * 4));
-    const bool w_ok = j < w_rows;
     step_f4 acc[NT][2];
 #pragma unroll
     for (int s = 0; s < NT; ++s) acc[s][0] = acc[s][1] = step_f4{0.f, 0.f, 0.f, 0.f};
-    for (int kb = wave * 16; kb < C; kb += kStepWaves * 16 * kStepUnroll) {
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int kb0 = wave; kb0 < KB; kb0 += kStepWaves * kStepUnroll) {
         float4 wq[kStepUnroll], aq[kStepUnroll][NT];
 #pragma unroll
         for (int u = 0; u < kStepUnroll; ++u) {
-            const int k = kb + u * (kStepWaves * 16) + 4 * kk;
-            const bool ok = k < C;                                       // C is a whole number of quads
-            wq[u] = buf_load4<false>(wr, (ok && w_ok) ? (j * C + k) * 4 : kOutOfRange);
+            const int kb = kb0 + u * kStepWaves;
+            const bool ok = kb < KB;                                     // the same for the whole wave
+            const int at = ok ? kb : kb0;
+            wq[u] = wp[(int64_t)at * kWave + lane];
+            if (!ok) wq[u] = zero;
 #pragma unroll
-            for (int s = 0; s < NT; ++s)
-                aq[u][s] = buf_load4<false>(ar, (ok && 16 * s + j < a_rows) ? ((16 * s + j) * C + k) * 4 : kOutOfRange);
+            for (int s = 0; s < NT; ++s) aq[u][s] = ap[((int64_t)at * S + s0 + s) * kWave + lane];
         }
 #pragma unroll
         for (int u = 0; u < kStepUnroll; ++u) {
@@ -104,7 +130,7 @@ __device__ __forceinline__ float4 step_product(const float* __restrict__ w, cons
         red[wave][s][lane] = make_float4(acc[s][0][0] + acc[s][1][0], acc[s][0][1] + acc[s][1][1],
                                          acc[s][0][2] + acc[s][1][2], acc[s][0][3] + acc[s][1][3]);
     __syncthreads();
-    float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 sum = zero;
     if (tid < NT * kWave) {
         const int s = tid >> 6;
 #pragma unroll
@@ -121,7 +147,9 @@ struct StepFwd {
     const float* z_t;                                         // [T][N][C]
     int* carried;                                             // [4][N][C]: current, voltage, threshold, refractory
     float *cur_last, *vol_last, *th_last, *ref_last;          // [N*C]; th / ref: ALIF only
-    const float* rec;                                         // [C][C]
+    const float4* rec_packed;                                 // see pack_weights_kernel
+    float4* spk_packed;                                       // two buffers of [KB][S][64] quads, written in turn
+    int KB, S;                                                // blocks of 16 neurons, sample tiles
     const float *i_decay, *v_decay, *th_decay, *ref_decay, *i_state, *v_state, *th_state, *ref_state;
     int64_t n_id, n_vd, n_td, n_rd, n_is, n_vs, n_ts, n_rs;
     float w, inv_w, spike_thr, spike_scale, th_step_f;
@@ -139,69 +167,87 @@ __global__ __launch_bounds__(kStepWaves * kWave) void recurrent_step_fwd_kernel(
     const int C = p.C, N = p.N;
     const int c0 = blockIdx.x * 16, n0 = blockIdx.y * 16 * NT;
     const int64_t slab = (int64_t)N * C;
-    float4 fb = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (t > 0) fb = step_product<NT>(p.rec, p.spk_t + (t - 1) * slab, N, C, n0, c0, red);
-    const int tid = threadIdx.x;
-    if (tid >= NT * kWave) return;
-    const int lane = tid & (kWave - 1);
+    const int s0 = blockIdx.y * NT;
+    const int64_t packed = (int64_t)p.KB * p.S * kWave;       // quads of one buffer of packed spikes
+    const int tid = threadIdx.x, lane = tid & (kWave - 1);
+    const bool worker = tid < NT * kWave;                     // the threads that run the neuron step
     const int n = n0 + 16 * (tid >> 6) + (lane & 15), c = c0 + 4 * (lane >> 4);
-    if (n >= N || c >= C) return;
-    const int64_t m = (int64_t)n * C + c;                     // first of this thread's four neurons
+    const bool valid = worker && n < N && c < C;
+    const int64_t m = valid ? (int64_t)n * C + c : 0;         // first of this thread's four neurons
     const float w = p.w, inv_w = p.inv_w;
     auto from = [&](int y) -> float { const float f = (float)y; return POW2 ? f * inv_w : f / w; };
-    const float4 z4 = *reinterpret_cast<const float4*>(p.z_t + t * slab + m);
-    const float zs[4] = {z4.x, z4.y, z4.z, z4.w}, fbs[4] = {fb.x, fb.y, fb.z, fb.w};
-    int yc[4], yv[4], th[4] = {0, 0, 0, 0}, r[4] = {0, 0, 0, 0};
-    if (t == 0) {
+    // what the neuron step reads is on its way while the product runs
+    float4 z4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    int yc[4] = {0, 0, 0, 0}, yv[4] = {0, 0, 0, 0}, th[4] = {0, 0, 0, 0}, r[4] = {0, 0, 0, 0};
+    int mi[4] = {0, 0, 0, 0}, mv[4] = {0, 0, 0, 0}, mt[4] = {0, 0, 0, 0}, mr[4] = {0, 0, 0, 0};
+    if (valid) {
+        z4 = *reinterpret_cast<const float4*>(p.z_t + t * slab + m);
+        if (t == 0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            yc[i] = trunc_i32(p.i_state[p.n_is == 1 ? 0 : m + i] * w);
-            yv[i] = trunc_i32(p.v_state[p.n_vs == 1 ? 0 : m + i] * w);
+            for (int i = 0; i < 4; ++i) {
+                yc[i] = trunc_i32(p.i_state[p.n_is == 1 ? 0 : m + i] * w);
+                yv[i] = trunc_i32(p.v_state[p.n_vs == 1 ? 0 : m + i] * w);
+                if (ALIF) {
+                    th[i] = trunc_i32(p.th_state[p.n_ts == 1 ? 0 : m + i] * w);
+                    r[i] = trunc_i32(p.ref_state[p.n_rs == 1 ? 0 : m + i] * w);
+                }
+            }
+        } else {
+            const int4 a = *reinterpret_cast<const int4*>(p.carried + m);
+            const int4 b = *reinterpret_cast<const int4*>(p.carried + slab + m);
+            yc[0] = a.x; yc[1] = a.y; yc[2] = a.z; yc[3] = a.w;
+            yv[0] = b.x; yv[1] = b.y; yv[2] = b.z; yv[3] = b.w;
             if (ALIF) {
-                th[i] = trunc_i32(p.th_state[p.n_ts == 1 ? 0 : m + i] * w);
-                r[i] = trunc_i32(p.ref_state[p.n_rs == 1 ? 0 : m + i] * w);
+                const int4 d = *reinterpret_cast<const int4*>(p.carried + 2 * slab + m);
+                const int4 e = *reinterpret_cast<const int4*>(p.carried + 3 * slab + m);
+                th[0] = d.x; th[1] = d.y; th[2] = d.z; th[3] = d.w;
+                r[0] = e.x; r[1] = e.y; r[2] = e.z; r[3] = e.w;
             }
         }
-    } else {
-        const int4 a = *reinterpret_cast<const int4*>(p.carried + m);
-        const int4 b = *reinterpret_cast<const int4*>(p.carried + slab + m);
-        yc[0] = a.x; yc[1] = a.y; yc[2] = a.z; yc[3] = a.w;
-        yv[0] = b.x; yv[1] = b.y; yv[2] = b.z; yv[3] = b.w;
-        if (ALIF) {
-            const int4 d = *reinterpret_cast<const int4*>(p.carried + 2 * slab + m);
-            const int4 e = *reinterpret_cast<const int4*>(p.carried + 3 * slab + m);
-            th[0] = d.x; th[1] = d.y; th[2] = d.z; th[3] = d.w;
-            r[0] = e.x; r[1] = e.y; r[2] = e.z; r[3] = e.w;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            // one decay for the layer or one per neuron (neuron c + i of its sample)
+            mi[i] = 4096 - trunc_i32(rintf(p.i_decay[p.n_id == 1 ? 0 : c + i]));
+            mv[i] = 4096 - trunc_i32(rintf(p.v_decay[p.n_vd == 1 ? 0 : c + i]));
+            if (ALIF) {
+                mt[i] = 4096 - trunc_i32(rintf(p.th_decay[p.n_td == 1 ? 0 : c + i]));
+                mr[i] = 4096 - trunc_i32(rintf(p.ref_decay[p.n_rd == 1 ? 0 : c + i]));
+            }
         }
     }
+    float4 fb = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (t > 0)
+        fb = step_product<NT>(p.rec_packed + (int64_t)blockIdx.x * p.KB * kWave, p.spk_packed + ((t - 1) & 1) * packed,
+                              p.KB, p.S, s0, red);
+    if (!worker) return;
+    // where the next step's product finds this thread's four spikes
+    float4* hand_on = p.spk_packed + (t & 1) * packed + ((int64_t)blockIdx.x * p.S + s0 + (tid >> 6)) * kWave + lane;
+    if (!valid) {
+        *hand_on = make_float4(0.f, 0.f, 0.f, 0.f);
+        return;
+    }
+    const float zs[4] = {z4.x, z4.y, z4.z, z4.w}, fbs[4] = {fb.x, fb.y, fb.z, fb.w};
     unsigned acc_lif = 0u, acc_th = 0u;                       // range of the states, see range_bits in tile.h
     float so[4], vo[4], to[4], co[4], tho[4], ro[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int mi = 4096 - trunc_i32(rintf(p.i_decay[param_index(m + i, C, p.n_id)]));
-        const int mv = 4096 - trunc_i32(rintf(p.v_decay[param_index(m + i, C, p.n_vd)]));
-        int mt = 0, mr = 0;
-        if (ALIF) {
-            mt = 4096 - trunc_i32(rintf(p.th_decay[param_index(m + i, C, p.n_td)]));
-            mr = 4096 - trunc_i32(rintf(p.ref_decay[param_index(m + i, C, p.n_rd)]));
-        }
         if (t == 0) {
-            check_multiplier(mi, p.range_flag); check_multiplier(mv, p.range_flag);
-            if (ALIF) { check_multiplier(mt, p.range_flag); check_multiplier(mr, p.range_flag); }
+            check_multiplier(mi[i], p.range_flag); check_multiplier(mv[i], p.range_flag);
+            if (ALIF) { check_multiplier(mt[i], p.range_flag); check_multiplier(mr[i], p.range_flag); }
             acc_lif |= ((unsigned)yc[i] + (1u << 30)) | ((unsigned)yv[i] + (1u << 30));
             acc_th |= ((unsigned)th[i] + (1u << 28)) | ((unsigned)r[i] + (1u << 28));
         }
         const float dend = zs[i] + fbs[i];
-        yc[i] = add_sat(rs0_12(yc[i], mi), trunc_i32(w * dend));
+        yc[i] = add_sat(rs0_12(yc[i], mi[i]), trunc_i32(w * dend));
         const float cur = from(yc[i]);
         yc[i] = trunc_i32(w * cur);
-        const int yn = add_sat(rs0_12(yv[i], mv), yc[i]);
+        const int yn = add_sat(rs0_12(yv[i], mv[i]), yc[i]);
         acc_lif |= ((unsigned)yc[i] + (1u << 30)) | ((unsigned)yn + (1u << 30));
         const float vol = from(yn);
         float theta = p.spike_thr, thf = 0.f, rf = 0.f;
         if (ALIF) {
-            r[i] = rs0_12(r[i], mr);
-            th[i] = rs0_12(th[i] - p.base, mt) + p.base;
+            r[i] = rs0_12(r[i], mr[i]);
+            th[i] = rs0_12(th[i] - p.base, mt[i]) + p.base;
             acc_th |= ((unsigned)th[i] + (1u << 28)) | ((unsigned)r[i] + (1u << 28));
             thf = from(th[i]);
             rf = from(r[i]);
@@ -221,6 +267,7 @@ __global__ __launch_bounds__(kStepWaves * kWave) void recurrent_step_fwd_kernel(
     }
     if (range_exceeded(acc_lif, 30) || range_exceeded(acc_th, 28)) raise_range_flag(p.range_flag);
     *reinterpret_cast<float4*>(p.spk_t + t * slab + m) = make_float4(so[0], so[1], so[2], so[3]);
+    *hand_on = make_float4(so[0], so[1], so[2], so[3]);
     *reinterpret_cast<float4*>(p.vol_t + t * slab + m) = make_float4(vo[0], vo[1], vo[2], vo[3]);
     if (ALIF) *reinterpret_cast<float4*>(p.theta_t + t * slab + m) = make_float4(to[0], to[1], to[2], to[3]);
     if (t == p.T - 1) {
@@ -243,7 +290,9 @@ __global__ __launch_bounds__(kStepWaves * kWave) void recurrent_step_fwd_kernel(
 struct StepBwd {
     float* gz_t;                                              // [T][N][C]: gradient of the dendrite input
     const float *g_t, *v_t, *theta_t;                         // [T][N][C]; theta: ALIF only
-    const float* rec_t;                                       // [C][C]: the weight matrix transposed
+    const float4* rec_packed;                                 // the transposed matrix, see pack_weights_kernel
+    float4* gz_packed;                                        // two buffers of [KB][S][64] quads, written in turn
+    int KB, S;
     float spike_thr, tau, rho;
     int N, C, T;
 };
@@ -254,18 +303,31 @@ __global__ __launch_bounds__(kStepWaves * kWave) void recurrent_step_bwd_kernel(
     const int C = p.C, N = p.N;
     const int c0 = blockIdx.x * 16, n0 = blockIdx.y * 16 * NT;
     const int64_t slab = (int64_t)N * C;
-    float4 carry = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (t < p.T - 1) carry = step_product<NT>(p.rec_t, p.gz_t + (t + 1) * slab, N, C, n0, c0, red);
-    const int tid = threadIdx.x;
-    if (tid >= NT * kWave) return;
-    const int lane = tid & (kWave - 1);
+    const int s0 = blockIdx.y * NT;
+    const int64_t packed = (int64_t)p.KB * p.S * kWave;
+    const int tid = threadIdx.x, lane = tid & (kWave - 1);
+    const bool worker = tid < NT * kWave;
     const int n = n0 + 16 * (tid >> 6) + (lane & 15), c = c0 + 4 * (lane >> 4);
-    if (n >= N || c >= C) return;
-    const int64_t at = t * slab + (int64_t)n * C + c;
-    const float4 g4 = *reinterpret_cast<const float4*>(p.g_t + at);
-    const float4 v4 = *reinterpret_cast<const float4*>(p.v_t + at);
+    const bool valid = worker && n < N && c < C;
+    const int64_t at = valid ? t * slab + (int64_t)n * C + c : 0;
+    // what the step reads is on its way while the product runs
+    float4 g4 = make_float4(0.f, 0.f, 0.f, 0.f), v4 = g4;
     float4 th4 = make_float4(p.spike_thr, p.spike_thr, p.spike_thr, p.spike_thr);
-    if (THETA) th4 = *reinterpret_cast<const float4*>(p.theta_t + at);
+    if (valid) {
+        g4 = *reinterpret_cast<const float4*>(p.g_t + at);
+        v4 = *reinterpret_cast<const float4*>(p.v_t + at);
+        if (THETA) th4 = *reinterpret_cast<const float4*>(p.theta_t + at);
+    }
+    float4 carry = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (t < p.T - 1)
+        carry = step_product<NT>(p.rec_packed + (int64_t)blockIdx.x * p.KB * kWave, p.gz_packed + ((t + 1) & 1) * packed,
+                                 p.KB, p.S, s0, red);
+    if (!worker) return;
+    float4* hand_on = p.gz_packed + (t & 1) * packed + ((int64_t)blockIdx.x * p.S + s0 + (tid >> 6)) * kWave + lane;
+    if (!valid) {
+        *hand_on = make_float4(0.f, 0.f, 0.f, 0.f);
+        return;
+    }
     const float lead = (p.rho / 2.0f) / p.tau, inv_tau = 1.0f / p.tau;
     auto one = [&](float cy, float g, float v, float th) -> float {
         const float gs = cy + g;
@@ -273,8 +335,10 @@ __global__ __launch_bounds__(kStepWaves * kWave) void recurrent_step_bwd_kernel(
         const float factor = GRADED ? p.rho * expf(fminf(d, 0.0f) * inv_tau) : lead * expf(-fabsf(d) * inv_tau);
         return factor * gs;
     };
-    *reinterpret_cast<float4*>(p.gz_t + at) = make_float4(one(carry.x, g4.x, v4.x, th4.x), one(carry.y, g4.y, v4.y, th4.y),
-                                                          one(carry.z, g4.z, v4.z, th4.z), one(carry.w, g4.w, v4.w, th4.w));
+    const float4 gd = make_float4(one(carry.x, g4.x, v4.x, th4.x), one(carry.y, g4.y, v4.y, th4.y),
+                                  one(carry.z, g4.z, v4.z, th4.z), one(carry.w, g4.w, v4.w, th4.w));
+    *reinterpret_cast<float4*>(p.gz_t + at) = gd;
+    *hand_on = gd;
 }
 
 }  // namespace slayer
@@ -292,8 +356,46 @@ int check_step_sizes(int64_t N, int64_t C, int64_t T) {
     return 0;
 }
 
+// sample tiles per workgroup (1, 2 or 4): one while that still leaves the chip with no more than one workgroup per
+// compute unit (the workgroups of one neuron tile share their weights through the L2), more for larger problems
+int step_sample_tiles(int64_t N, int64_t C) {
+    const int64_t tiles = (N + 15) / 16, KB = (C + 15) / 16;
+    int nt = 1;
+    while (nt < 4 && nt < tiles && KB * ((tiles + nt - 1) / nt) > 256) nt *= 2;
+    return nt;
+}
+
+// what the workspace holds: the time-major tensors, the states between two steps, the packed weights and two
+// buffers of packed activations
+struct StepLayout {
+    int64_t nct, carried, KB, S, weights, packed;             // floats, except KB (blocks of 16) and S (sample tiles)
+    int64_t total(int tensors) const { return tensors * nct + carried + weights + 2 * packed; }
+};
+StepLayout step_layout(int64_t N, int64_t C, int64_t T) {
+    StepLayout l;
+    const int nt = step_sample_tiles(N, C);
+    l.nct = N * C * T;
+    l.carried = 4 * N * C;
+    l.KB = (C + 15) / 16;
+    l.S = (N + 16 * nt - 1) / (16 * nt) * nt;
+    l.weights = l.KB * l.KB * 256;
+    l.packed = l.KB * l.S * 256;
+    return l;
+}
+
 int64_t step_workspace_floats(int64_t N, int64_t C, int64_t T, int with_theta) {
-    return (3 + (with_theta ? 1 : 0)) * N * C * T + 4 * N * C;
+    return step_layout(N, C, T).total(3 + (with_theta ? 1 : 0));
+}
+
+void launch_pack_weights(float* packed, const float* w, int64_t C, bool transposed, hipStream_t st) {
+    const int KB = (int)((C + 15) / 16);
+    const dim3 grid((unsigned)KB, (unsigned)KB);
+    if (transposed)
+        hipLaunchKernelGGL((pack_weights_kernel<true>), grid, dim3(kWave), 0, st, reinterpret_cast<float4*>(packed), w,
+                           (int)C, KB);
+    else
+        hipLaunchKernelGGL((pack_weights_kernel<false>), grid, dim3(kWave), 0, st, reinterpret_cast<float4*>(packed), w,
+                           (int)C, KB);
 }
 
 void launch_time_major(float* dst, const float* src, int64_t M, int64_t T, bool to_time_major, hipStream_t st) {
@@ -305,12 +407,9 @@ void launch_time_major(float* dst, const float* src, int64_t M, int64_t T, bool 
         hipLaunchKernelGGL((time_major_kernel<false>), grid, dim3(256), 0, st, dst, src, M, (int)T);
 }
 
-// sample tiles per workgroup: as many as the batch needs, up to four
-int step_sample_tiles(int64_t N) { return N <= 16 ? 1 : (N <= 32 ? 2 : 4); }
-
 template <bool ALIF>
 int launch_step_fwd(StepFwd p, int graded, int w_scale, hipStream_t st) {
-    const int nt = step_sample_tiles(p.N);
+    const int nt = step_sample_tiles(p.N, p.C);
     const dim3 grid((unsigned)((p.C + 15) / 16), (unsigned)((p.N + 16 * nt - 1) / (16 * nt)));
     const dim3 block(kStepWaves * kWave);
     const bool pow2 = is_pow2(w_scale);
@@ -330,11 +429,14 @@ int launch_step_fwd(StepFwd p, int graded, int w_scale, hipStream_t st) {
 
 // common part of the two forward entry points: copies in, the steps, copies out
 template <bool ALIF>
-int run_steps_fwd(StepFwd p, float* spk, float* vol, float* theta, const float* z, int graded, int w_scale,
+int run_steps_fwd(StepFwd p, float* spk, float* vol, float* theta, const float* z, const float* rec, int graded, int w_scale,
                   float* workspace, int64_t workspace_floats, hipStream_t st) {
-    const int64_t N = p.N, C = p.C, T = p.T, nct = N * C * T;
-    if (workspace_floats < step_workspace_floats(N, C, T, ALIF ? 1 : 0)) return SLAYER_ERANGE;
-    if (!aligned16(workspace) || !aligned16(p.rec) || !aligned16(p.cur_last) || !aligned16(p.vol_last) ||
+    const int64_t N = p.N, C = p.C, T = p.T;
+    const StepLayout l = step_layout(N, C, T);
+    const int64_t nct = l.nct;
+    const int tensors = 3 + (ALIF ? 1 : 0);
+    if (workspace_floats < l.total(tensors)) return SLAYER_ERANGE;
+    if (!aligned16(workspace) || !aligned16(p.cur_last) || !aligned16(p.vol_last) ||
         (ALIF && (!aligned16(p.th_last) || !aligned16(p.ref_last))))
         return SLAYER_ERANGE;
     float* zt = workspace;
@@ -342,7 +444,12 @@ int run_steps_fwd(StepFwd p, float* spk, float* vol, float* theta, const float* 
     p.spk_t = workspace + nct;
     p.vol_t = workspace + 2 * nct;
     p.theta_t = ALIF ? workspace + 3 * nct : nullptr;
-    p.carried = reinterpret_cast<int*>(workspace + (3 + (ALIF ? 1 : 0)) * nct);
+    p.carried = reinterpret_cast<int*>(workspace + tensors * nct);
+    float* wp = workspace + tensors * nct + l.carried;
+    p.rec_packed = reinterpret_cast<const float4*>(wp);
+    p.spk_packed = reinterpret_cast<float4*>(wp + l.weights);
+    p.KB = (int)l.KB; p.S = (int)l.S;
+    launch_pack_weights(wp, rec, C, false, st);
     launch_time_major(zt, z, N * C, T, true, st);
     if (int e = launch_step_fwd<ALIF>(p, graded, w_scale, st)) return e;
     launch_time_major(spk, p.spk_t, N * C, T, false, st);
@@ -371,21 +478,20 @@ extern "C" int slayer_cuba_recurrent_steps_fwd(float* spk_out, float* vol_out, f
     if (!spk_out || !vol_out || !cur_last_out || !vol_last_out || !z || !rec || !i_decay || !v_decay || !i_state ||
         !v_state || !workspace)
         return SLAYER_ENULL;
-    if (int e = check_params(N * C, C, num_i_decays)) return e;
-    if (int e = check_params(N * C, C, num_v_decays)) return e;
+    for (int64_t n : {num_i_decays, num_v_decays})
+        if (n != 1 && n != C) return SLAYER_EINVAL;
     if (int e = check_states(N * C, num_i_states)) return e;
     if (int e = check_states(N * C, num_v_states)) return e;
     if (w_scale == 0 || (graded && spike_scale == 0.0f)) return SLAYER_EINVAL;
     StepFwd p{};
     p.cur_last = cur_last_out; p.vol_last = vol_last_out;
-    p.rec = rec;
     p.i_decay = i_decay; p.v_decay = v_decay; p.i_state = i_state; p.v_state = v_state;
     p.n_id = num_i_decays; p.n_vd = num_v_decays; p.n_is = num_i_states; p.n_vs = num_v_states;
     p.w = (float)w_scale; p.inv_w = 1.0f / (float)w_scale;
     p.spike_thr = spike_threshold; p.spike_scale = spike_scale;
     p.N = (int)N; p.C = (int)C; p.T = (int)T;
     p.range_flag = range_flag_device();
-    return run_steps_fwd<false>(p, spk_out, vol_out, nullptr, z, graded, w_scale, workspace, workspace_floats,
+    return run_steps_fwd<false>(p, spk_out, vol_out, nullptr, z, rec, graded, w_scale, workspace, workspace_floats,
                                 (hipStream_t)stream);
 }
 
@@ -408,14 +514,13 @@ extern "C" int slayer_alif_recurrent_steps_fwd(float* spk_out, float* vol_out, f
         !workspace)
         return SLAYER_ENULL;
     for (int64_t n : {num_i_decays, num_v_decays, num_th_decays, num_ref_decays})
-        if (int e = check_params(N * C, C, n)) return e;
+        if (n != 1 && n != C) return SLAYER_EINVAL;
     for (int64_t n : {num_i_states, num_v_states, num_th_states, num_ref_states})
         if (int e = check_states(N * C, n)) return e;
     if (w_scale == 0 || (graded && spike_scale == 0.0f)) return SLAYER_EINVAL;
     if (th0_scaled > 0x7fffffffLL || th0_scaled < -0x7fffffffLL) return SLAYER_ERANGE;
     StepFwd p{};
     p.cur_last = cur_last_out; p.vol_last = vol_last_out; p.th_last = th_last_out; p.ref_last = ref_last_out;
-    p.rec = rec;
     p.i_decay = i_decay; p.v_decay = v_decay; p.th_decay = th_decay; p.ref_decay = ref_decay;
     p.i_state = i_state; p.v_state = v_state; p.th_state = th_state; p.ref_state = ref_state;
     p.n_id = num_i_decays; p.n_vd = num_v_decays; p.n_td = num_th_decays; p.n_rd = num_ref_decays;
@@ -425,33 +530,40 @@ extern "C" int slayer_alif_recurrent_steps_fwd(float* spk_out, float* vol_out, f
     p.base = (int)th0_scaled;
     p.N = (int)N; p.C = (int)C; p.T = (int)T;
     p.range_flag = range_flag_for_threshold(0, th0_scaled);
-    return run_steps_fwd<true>(p, spk_out, vol_out, theta_out, z, graded, w_scale, workspace, workspace_floats,
+    return run_steps_fwd<true>(p, spk_out, vol_out, theta_out, z, rec, graded, w_scale, workspace, workspace_floats,
                                (hipStream_t)stream);
 }
 
 extern "C" int slayer_recurrent_steps_bwd(float* grad_z, const float* grad_spikes, const float* voltage,
-                                          const float* theta, const float* rec_t, float spike_threshold,
+                                          const float* theta, const float* rec, float spike_threshold,
                                           float tau_rho, float scale_rho, int graded, int64_t N, int64_t C, int64_t T,
                                           float* workspace, int64_t workspace_floats, void* stream) {
     if (int e = check_step_sizes(N, C, T)) return e;
     if (N == 0 || C == 0 || T == 0) return 0;
-    if (!grad_z || !grad_spikes || !voltage || !rec_t || !workspace) return SLAYER_ENULL;
-    if (workspace_floats < step_workspace_floats(N, C, T, theta ? 1 : 0)) return SLAYER_ERANGE;
-    if (!aligned16(workspace) || !aligned16(rec_t)) return SLAYER_ERANGE;
+    if (!grad_z || !grad_spikes || !voltage || !rec || !workspace) return SLAYER_ENULL;
+    const StepLayout l = step_layout(N, C, T);
+    const int tensors = 3 + (theta ? 1 : 0);
+    if (workspace_floats < l.total(tensors)) return SLAYER_ERANGE;
+    if (!aligned16(workspace)) return SLAYER_ERANGE;
     hipStream_t st = (hipStream_t)stream;
-    const int64_t nct = N * C * T;
+    const int64_t nct = l.nct;
     float* g_t = workspace;
     float* v_t = workspace + nct;
     float* gz_t = workspace + 2 * nct;
     float* th_t = theta ? workspace + 3 * nct : nullptr;
+    float* wp = workspace + tensors * nct + l.carried;
+    launch_pack_weights(wp, rec, C, true, st);
     launch_time_major(g_t, grad_spikes, N * C, T, true, st);
     launch_time_major(v_t, voltage, N * C, T, true, st);
     if (theta) launch_time_major(th_t, theta, N * C, T, true, st);
     StepBwd p{};
-    p.gz_t = gz_t; p.g_t = g_t; p.v_t = v_t; p.theta_t = th_t; p.rec_t = rec_t;
+    p.gz_t = gz_t; p.g_t = g_t; p.v_t = v_t; p.theta_t = th_t;
+    p.rec_packed = reinterpret_cast<const float4*>(wp);
+    p.gz_packed = reinterpret_cast<float4*>(wp + l.weights);
+    p.KB = (int)l.KB; p.S = (int)l.S;
     p.spike_thr = spike_threshold; p.tau = tau_rho; p.rho = scale_rho;
     p.N = (int)N; p.C = (int)C; p.T = (int)T;
-    const int nt = step_sample_tiles(N);
+    const int nt = step_sample_tiles(N, C);
     const dim3 grid((unsigned)((C + 15) / 16), (unsigned)((N + 16 * nt - 1) / (16 * nt)));
     const dim3 block(kStepWaves * kWave);
     for (int t = (int)T - 1; t >= 0; --t) {

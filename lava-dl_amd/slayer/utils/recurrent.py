@@ -1,11 +1,11 @@
 """Recurrent spiking layer: ``s[t] = neuron(z[t] + R s[t-1])``.
 
 Interface of lava.lib.dl.slayer.utils.recurrent (utils/recurrent.py:7-112 in the reference).
-For a CUBA or an ALIF neuron on the GPU (binary or graded spikes) the time loop runs inside the library: up to
-``ONE_LAUNCH_MAX`` neurons per sample as one kernel launch per direction (slayer_cuba_recurrent_fwd /
-slayer_alif_recurrent_fwd / slayer_recurrent_bwd), wider layers (a multiple of 4 up to 16384 neurons) as one
-launch per time step that multiplies the recurrent matrix with the whole batch (slayer_*_recurrent_steps_*); any
-other neuron runs the reference's loop of one-step neuron calls.
+For a CUBA or an ALIF neuron on the GPU (binary or graded spikes) the time loop runs inside the library: narrow
+layers (and widths up to ``ONE_LAUNCH_MAX`` that are not a multiple of 4) as one kernel launch per direction
+(slayer_cuba_recurrent_fwd / slayer_alif_recurrent_fwd / slayer_recurrent_bwd), layers from ``STEPS_FROM`` neurons
+on (a multiple of 4 up to 16384) as one launch per time step that multiplies the recurrent matrix with the whole
+batch (slayer_*_recurrent_steps_*); any other neuron runs the reference's loop of one-step neuron calls.
 """
 import torch
 
@@ -44,12 +44,13 @@ def custom_recurrent_ground_truth_2(z, neuron, recurrent_synapse):
 
 
 ONE_LAUNCH_MAX = 1024       # neurons per sample of the one-launch kernels (one thread per neuron)
-STEPS_MAX = 16384           # ... of the launch-per-step kernels
+STEPS_MAX = 16384           # ... of the launch-per-step kernels (whole quads of neurons)
+STEPS_FROM = 256            # width from which a launch per step is the faster form (measured at [32, C, 300])
 
 
 def _by_steps(c):
     """True for the layer widths that take the launch-per-step kernels."""
-    return c > ONE_LAUNCH_MAX
+    return c % 4 == 0 and c <= STEPS_MAX and (c >= STEPS_FROM or c > ONE_LAUNCH_MAX)
 
 
 def _fusable(z, neuron):
@@ -58,7 +59,7 @@ def _fusable(z, neuron):
             and neuron.norm is None and neuron.drop is None and neuron.persistent_state):
         return False
     c = z.shape[1]
-    return c <= ONE_LAUNCH_MAX or (c % 4 == 0 and c <= STEPS_MAX and z.shape[0] * c < 2 ** 29)
+    return c <= ONE_LAUNCH_MAX or (_by_steps(c) and z.shape[0] * c < 2 ** 29)
 
 
 def custom_recurrent(z, neuron, recurrent_synapse):
@@ -202,10 +203,9 @@ class _FusedRecurrent(torch.autograd.Function):
         th = N.ptr(theta[0]) if theta else None
         with N.device_guard(dev):
             if _by_steps(c):
-                rec_t = rec.transpose(0, 1).contiguous()
                 ws = _steps_workspace(n, c, t, bool(theta), dev)
                 N.check(N.lib().slayer_recurrent_steps_bwd(
-                    N.ptr(grad_z), N.ptr(grad_x), N.ptr(vol), th, N.ptr(rec_t),
+                    N.ptr(grad_z), N.ptr(grad_x), N.ptr(vol), th, N.ptr(rec),
                     threshold, tau_rho, scale_rho, graded, n, c, t, N.ptr(ws), ws.numel(), N.stream_handle()))
             else:
                 N.check(N.lib().slayer_recurrent_bwd(

@@ -17,6 +17,13 @@ def slayer():
     return s
 
 
+@pytest.fixture(autouse=True)
+def one_launch(slayer, monkeypatch):
+    """The tests of this file are about the one-launch kernels: widths that would take a launch per step
+    (tests/test_gpu_recurrent_steps.py) stay on them."""
+    monkeypatch.setattr(slayer.utils.recurrent, 'STEPS_FROM', 10 ** 9)
+
+
 class _Dense(torch.nn.Module):
     """Stand-in for the dense synapse the layer is used with: weight [C_out, C_in, 1, 1, 1], optional pre-hook."""
 

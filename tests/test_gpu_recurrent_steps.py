@@ -27,7 +27,7 @@ def by_steps(slayer, monkeypatch):
     def counted(*a):
         calls.append(a)
         return plain(*a)
-    monkeypatch.setattr(R, 'ONE_LAUNCH_MAX', 0)
+    monkeypatch.setattr(R, 'STEPS_FROM', 0)
     monkeypatch.setattr(R, '_steps_workspace', counted)
     yield calls
     assert calls, 'the launch-per-step path was not taken'
@@ -67,8 +67,8 @@ def test_the_two_kernel_paths_agree(slayer, monkeypatch, kind):
     z = (torch.randn(n, c, t, generator=gen) * 1.5).to(dev())
     g = torch.rand(n, c, t, generator=gen).to(dev())
     results = []
-    for limit in (1024, 0):
-        monkeypatch.setattr(R, 'ONE_LAUNCH_MAX', limit)
+    for first in (10 ** 9, 0):
+        monkeypatch.setattr(R, 'STEPS_FROM', first)
         neuron = base._alif(slayer) if kind == 'alif' else base._neuron(slayer)
         syn = base._Dense(c, torch.Generator().manual_seed(5)).to(dev())
         with torch.no_grad():
@@ -124,13 +124,15 @@ def test_wide_layers_match_the_oracle_and_the_generic_loop(slayer, n, c, t):
 def test_sizes_the_step_kernels_refuse(slayer):
     from lava_dl_amd.slayer import _native as N
     lib = N.lib()
-    assert lib.slayer_recurrent_steps_workspace(2, 2048, 10, 0) == 3 * 2 * 2048 * 10 + 4 * 2 * 2048
-    assert lib.slayer_recurrent_steps_workspace(2, 2048, 10, 1) == 4 * 2 * 2048 * 10 + 4 * 2 * 2048
+    base_floats = 4 * 2 * 2048 + 2048 * 2048 + 2 * 2048 * 16            # states, packed weights, packed spikes twice
+    assert lib.slayer_recurrent_steps_workspace(2, 2048, 10, 0) == 3 * 2 * 2048 * 10 + base_floats
+    assert lib.slayer_recurrent_steps_workspace(2, 2048, 10, 1) == 4 * 2 * 2048 * 10 + base_floats
     assert lib.slayer_recurrent_steps_workspace(2, 2050, 10, 0) == -3          # not whole quads of neurons
     assert lib.slayer_recurrent_steps_workspace(2, 16388, 10, 0) == -3
     R = slayer.utils.recurrent
     z = torch.zeros(2, 1030, 4, device=dev())
     assert not R._fusable(z, base._neuron(slayer)) and R._fusable(z[:, :1028].contiguous(), base._neuron(slayer))
+    assert R._by_steps(256) and R._by_steps(1028) and not R._by_steps(252) and not R._by_steps(258)
     # a workspace that is too small is refused before anything is launched
     ws = torch.empty(16, device=dev())
     t = torch.zeros(2 * 1028 * 4, device=dev())
