@@ -551,26 +551,50 @@ class SynapseFolded(SynapseFused):
 
 
 class SynapseDelayGrad(SynapseFused):
-    name = 'SLAYER synapse stack with a learnable delay (conv K=64 -> Delay -> fused CUBA) fwd+bwd incl. the delay gradient'
-    ops = [('conv', 'conv_mfma_split_kernel<64,conv>', 8), ('shift', 'shift_kernel', 8), ('cuba_fwd', 'stream_kernel_staged<CubaFwd>', 12),
-           ('cuba_bwd', 'cuba_bwd_scan_kernel', 12), ('delay_bwd', 'delay_bwd_kernel', 12), ('corr', 'conv_mfma_split_kernel<64,corr>', 8)]
+    """Synaptic filter -> CUBA neuron -> learnable per-channel Delay, the order of a SLAYER block (block/base.py:549-553
+    in the reference: the Delay follows the neuron), forward and backward including the delay's gradient
+    (axon/delay.py:201-221).  The Delay is folded into the neuron's two kernels: the forward kernel stores its spikes
+    through the delay, the backward scan reads the gradient back through it and sums grad * (out[t-1] - out[t]) / Ts
+    per row on the way.  `block_tail` is the neuron + Delay part of this stack with separate kernels."""
+    name = ('SLAYER synapse stack with a learnable delay (conv K=64 -> fused CUBA -> Delay, the Delay folded into the '
+            'neuron kernels) fwd+bwd incl. the delay gradient')
+    ops = [('conv', 'conv_mfma_split_kernel<64,conv>', 8), ('cuba_fwd', 'stream_kernel_staged<CubaFwd,SHIFT>', 12),
+           ('cuba_bwd', 'cuba_bwd_scan_kernel<SHIFT,DELAY>', 16), ('corr', 'conv_mfma_split_kernel<64,corr>', 8)]
+
+    def __init__(self, dev):
+        super().__init__(dev)
+        from lava_dl_amd.slayer.neuron.dynamics import delays
+        self.D = delays
+        self.delays = delays.Delays(output_delay=self.delay)
 
     def step(self, t):
-        import importlib
-        D = importlib.import_module('lava_dl_amd.slayer.axon.delay')
         with t('conv'):
             y = self.conv.fwd(self.x, self.filt, 1)
-        with t('shift'):
-            z = self.shift(y, self.delay, 1)
         with t('cuba_fwd'):
-            _, vol, spk = self.F._fwd(z, self.d_i, self.d_v, self.zero, self.zero, 64, 1.25, False, 1, True)
+            _, vol, out = self.F._fwd(y, self.d_i, self.d_v, self.zero, self.zero, 64, 1.25, False, 1, True,
+                                      folded=self.D.fold(self.delays, y))
         with t('cuba_bwd'):
-            g_z, _, _ = self.F._bwd(self.g, vol, None, self.d_i, self.d_v, 1.25, 1.0, 1.0, False, False)
-        with t('delay_bwd'):
-            g_y, g_delay = D._delay_bwd(g_z, z, self.delay, 1)
+            folded = self.D.fold(self.delays, self.g, forward=False, delayed_spikes=out)
+            g_y, _, _ = self.F._bwd(self.g, vol, None, self.d_i, self.d_v, 1.25, 1.0, 1.0, False, False, folded=folded)
+            g_delay = folded.grad_sum
         with t('corr'):
             g_x = self.conv.bwd(g_y, self.filt, 1)
-        return spk, g_x, g_delay
+        return out, g_x, g_delay
+
+    def cpu_step(self, n, sl=None):
+        from oracle import slayer_oracle as O
+        c, zero = self.cpu, torch.tensor([0.0])
+        x, g, delay = c['x'][:n], c['g'][:n], c['delay']
+        if sl is not None:
+            x, g, delay = x[:, sl], g[:, sl], delay[sl]
+        y = O.conv_fwd(x, c['filt'], 1)
+        cur = O.li_fwd(y, c['d_i'], zero, 64)
+        vol = O.li_fwd(cur, c['d_v'], zero, 64, 1.25)
+        out = O.shift(O.spike_fwd(vol, 1.25), delay, 1)
+        g_vol = O.spike_bwd(O.shift(g, -delay, 1), vol, 1.25, 1.0, 1.0)
+        g_cur, _ = O.li_bwd(g_vol, vol, c['d_v'])
+        g_y, _ = O.li_bwd(g_cur, cur, c['d_i'])
+        return out, O.conv_bwd(g_y, c['filt'], 1)
 
 
 class BlockTail(SynapseFused):
@@ -903,7 +927,7 @@ def timed_median(job, iters, warmup):
 # The other benchmark configurations, reported next to the headline in `other_configs` (unfused = the op
 # sequence of the configuration, then the fused forms with their own smaller byte counts).
 OTHER = ['cuba_fwd_small', 'cuba_fused', 'cuba_fused_lean', 'alif', 'alif_fused', 'alif_fused_lean', 'rf', 'rf_fused',
-         'synapse', 'synapse_fused', 'synapse_folded', 'block_tail', 'block_tail_folded',
+         'synapse', 'synapse_fused', 'synapse_folded', 'synapse_delay_grad', 'block_tail', 'block_tail_folded',
          'conv_synapse', 'conv_synapse_library', 'recurrent', 'recurrent_loop']
 
 
@@ -950,7 +974,7 @@ def other_configs(dev, iters):
 def traffic_factor(kernel):
     """HBM bytes per launch / algorithmic bytes for `kernel` from profiles/traffic_factors.txt (rocprofv3 --pmc
     FETCH_SIZE and WRITE_SIZE runs of this script, scaled by a plain copy of known size), or None when the file
-    was measured on other kernel sources than the ones in the tree."""
+    was measured on other sources of those kernels (the files it lists) than the ones in the tree."""
     import hashlib
     path = os.path.join(ROOT, 'profiles', 'traffic_factors.txt')
     if not os.path.exists(path):
@@ -958,9 +982,8 @@ def traffic_factor(kernel):
     rec = json.load(open(path))
     h = hashlib.sha256()
     csrc = os.path.join(ROOT, 'lava-dl_amd', 'csrc')
-    for f in sorted(os.listdir(csrc)):
-        if f.endswith(('.hip', '.h')):
-            h.update(open(os.path.join(csrc, f), 'rb').read())
+    for f in rec.get('sources', []):                 # the sources the measured kernels are built from
+        h.update(open(os.path.join(csrc, f), 'rb').read())
     if h.hexdigest()[:16] != rec.get('csrc_sha16'):
         return None, f"stale: measured at csrc {rec.get('csrc_sha16')} ({rec.get('commit')}), tree is {h.hexdigest()[:16]}"
     return rec['factors'].get(kernel), f"measured at commit {rec.get('commit')} (csrc {rec.get('csrc_sha16')})"

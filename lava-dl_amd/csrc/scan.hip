@@ -50,9 +50,14 @@ __device__ __forceinline__ float apply_affine(float A, float c, float B) {
 
 // Inclusive scan over the lanes, lowest lane first, of affine maps c -> B + A * c: afterwards (A, B) of lane l is
 // the composition of the maps of lanes 0 .. l (lane 0 applied first).
+// The plain composition (two instructions per step) is right whenever every partial result is finite: a cut's
+// 0 * b is then 0, which is what the cut means.  An Inf or a NaN anywhere in the wave survives into the final B of
+// its lane, so one test afterwards finds the rare wave that has one, and that wave repeats the scan with the cut
+// taken by a select (0 * Inf would be a NaN and would cross into the row below).  The same bits either way for
+// finite operands.
 __device__ __forceinline__ void scan_affine(float& A, float& B) {
-#define SLAYER_COMBINE(An, Bn) do { const float an_ = (An), bn_ = (Bn); const bool cut_ = A == 0.0f;            \
-        const float b2_ = __fmaf_rn(A, bn_, B), a2_ = A * an_; B = cut_ ? B : b2_; A = cut_ ? 0.0f : a2_; } while (0)
+    const float A0 = A, B0 = B;
+#define SLAYER_COMBINE(An, Bn) do { const float an_ = (An), bn_ = (Bn); B = __fmaf_rn(A, bn_, B); A = A * an_; } while (0)
     SLAYER_COMBINE(lane_below_in_row<1>(A, 1.0f), lane_below_in_row<1>(B, 0.0f));
     SLAYER_COMBINE(lane_below_in_row<2>(A, 1.0f), lane_below_in_row<2>(B, 0.0f));
     SLAYER_COMBINE(lane_below_in_row<4>(A, 1.0f), lane_below_in_row<4>(B, 0.0f));
@@ -60,6 +65,18 @@ __device__ __forceinline__ void scan_affine(float& A, float& B) {
     SLAYER_COMBINE(row_bcast15(A, 1.0f), row_bcast15(B, 0.0f));
     SLAYER_COMBINE(row_bcast31(A, 1.0f), row_bcast31(B, 0.0f));
 #undef SLAYER_COMBINE
+    if (__any(!(fabsf(B) <= 3.402823466e+38f))) {
+        A = A0; B = B0;
+#define SLAYER_COMBINE(An, Bn) do { const float an_ = (An), bn_ = (Bn); const bool cut_ = A == 0.0f;            \
+        const float b2_ = __fmaf_rn(A, bn_, B), a2_ = A * an_; B = cut_ ? B : b2_; A = cut_ ? 0.0f : a2_; } while (0)
+        SLAYER_COMBINE(lane_below_in_row<1>(A, 1.0f), lane_below_in_row<1>(B, 0.0f));
+        SLAYER_COMBINE(lane_below_in_row<2>(A, 1.0f), lane_below_in_row<2>(B, 0.0f));
+        SLAYER_COMBINE(lane_below_in_row<4>(A, 1.0f), lane_below_in_row<4>(B, 0.0f));
+        SLAYER_COMBINE(lane_below_in_row<8>(A, 1.0f), lane_below_in_row<8>(B, 0.0f));
+        SLAYER_COMBINE(row_bcast15(A, 1.0f), row_bcast15(B, 0.0f));
+        SLAYER_COMBINE(row_bcast31(A, 1.0f), row_bcast31(B, 0.0f));
+#undef SLAYER_COMBINE
+    }
 }
 
 // Inclusive sum over the lanes below that belong to the same run: lane l adds lanes l - reach .. l - 1.
@@ -296,12 +313,15 @@ __device__ __forceinline__ void delay_grad_fetch(DelayGradQuads& d, __amdgpu_buf
     const int kf = -k, u0 = 4 * pos + kf;
     d.sp = scan_load_at(src_s, in_span, r, u0 - 1, T);
     const bool first = in_span && pos == 0 && kf >= 1, last = in_span && pos == QR - 1 && kf < 0;
-    d.ag = scan_load_at(src_g, first, r, kf - 1, T);
-    d.as = scan_load_at(src_s, first, r, kf - 1, T);
-    d.asp = scan_load_at(src_s, first, r, kf - 2, T);
-    d.bg = scan_load_at(src_g, last, r, T + kf, T);
-    d.bs = scan_load_at(src_s, last, r, T + kf, T);
-    d.bsp = scan_load_at(src_s, last, r, T + kf - 1, T);
+    d.ag = d.as = d.asp = d.bg = d.bs = d.bsp = 0.0f;
+    if (__any(first || last)) {                                       // most waves hold no end of a row
+        d.ag = scan_load_at(src_g, first, r, kf - 1, T);
+        d.as = scan_load_at(src_s, first, r, kf - 1, T);
+        d.asp = scan_load_at(src_s, first, r, kf - 2, T);
+        d.bg = scan_load_at(src_g, last, r, T + kf, T);
+        d.bs = scan_load_at(src_s, last, r, T + kf, T);
+        d.bsp = scan_load_at(src_s, last, r, T + kf - 1, T);
+    }
 }
 // g: the gradient quad in place (zeros where the row has no sample); place: what scan_place needs for d.s
 __device__ __forceinline__ float delay_grad_terms(DelayGradQuads& d, float4 g, int place, float inv_ts) {
@@ -573,14 +593,13 @@ __device__ __forceinline__ Cx apply_affine_complex(Cx A, Cx z, Cx B) {
     return Cx{cut ? B.re : v.re, cut ? B.im : v.im};
 }
 
-// inclusive scan over the lanes of complex affine maps z -> B + A * z (see scan_affine)
+// inclusive scan over the lanes of complex affine maps z -> B + A * z (see scan_affine: the plain composition
+// first, the one with selected cuts only in a wave that holds an Inf or a NaN)
 __device__ __forceinline__ void scan_affine_complex(Cx& A, Cx& B) {
+    const Cx A0 = A, B0 = B;
 #define SLAYER_COMBINE(M) do {                                                                                  \
         const Cx an_{M(A.re, 1.0f), M(A.im, 0.0f)}, bn_{M(B.re, 0.0f), M(B.im, 0.0f)};                          \
-        const bool cut_ = A.re == 0.0f && A.im == 0.0f;                                                         \
-        const Cx b2_ = cfma(A, bn_, B), a2_ = cmul(A, an_);                                                     \
-        B = Cx{cut_ ? B.re : b2_.re, cut_ ? B.im : b2_.im};                                                     \
-        A = Cx{cut_ ? 0.0f : a2_.re, cut_ ? 0.0f : a2_.im}; } while (0)
+        B = cfma(A, bn_, B); A = cmul(A, an_); } while (0)
     SLAYER_COMBINE(lane_below_in_row<1>);
     SLAYER_COMBINE(lane_below_in_row<2>);
     SLAYER_COMBINE(lane_below_in_row<4>);
@@ -588,6 +607,22 @@ __device__ __forceinline__ void scan_affine_complex(Cx& A, Cx& B) {
     SLAYER_COMBINE(row_bcast15);
     SLAYER_COMBINE(row_bcast31);
 #undef SLAYER_COMBINE
+    if (__any(!(fabsf(B.re) <= 3.402823466e+38f) || !(fabsf(B.im) <= 3.402823466e+38f))) {
+        A = A0; B = B0;
+#define SLAYER_COMBINE(M) do {                                                                                  \
+        const Cx an_{M(A.re, 1.0f), M(A.im, 0.0f)}, bn_{M(B.re, 0.0f), M(B.im, 0.0f)};                          \
+        const bool cut_ = A.re == 0.0f && A.im == 0.0f;                                                         \
+        const Cx b2_ = cfma(A, bn_, B), a2_ = cmul(A, an_);                                                     \
+        B = Cx{cut_ ? B.re : b2_.re, cut_ ? B.im : b2_.im};                                                     \
+        A = Cx{cut_ ? 0.0f : a2_.re, cut_ ? 0.0f : a2_.im}; } while (0)
+        SLAYER_COMBINE(lane_below_in_row<1>);
+        SLAYER_COMBINE(lane_below_in_row<2>);
+        SLAYER_COMBINE(lane_below_in_row<4>);
+        SLAYER_COMBINE(lane_below_in_row<8>);
+        SLAYER_COMBINE(row_bcast15);
+        SLAYER_COMBINE(row_bcast31);
+#undef SLAYER_COMBINE
+    }
 }
 
 // SURR = 0: g_re / g_im are the incoming gradients of the two states (resonator backward).

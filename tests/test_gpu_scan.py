@@ -43,7 +43,12 @@ def test_li_bwd_scan_against_oracle_and_sequential_kernel(slayer, shape, nd):
         d[1] = 4096.0                              # nothing carried at all
     gi, gd = L._bwd(g.to(dev()), y.to(dev()), d.to(dev()))
     seq = L._bwd_naive(g.to(dev()), d.to(dev()))
-    assert_scale(gi, seq.cpu(), 'scan vs step-by-step kernel')
+    # two float32 evaluations of the same recurrence: within 1e-5 of the largest value while the rows are short
+    # enough for that to be a meaningful scale; on the rows of several hundred thousand steps a pure integrator is a
+    # random walk whose terms sum to a thousand times its largest value, and the bar is the one against float64 below
+    long_rows = shape[-1] > 65536
+    if not long_rows:
+        assert_scale(gi, seq.cpu(), 'scan vs step-by-step kernel')
     # the oracle on slabs of rows (whole tensor when it is small enough for the python loop over time)
     rows = g.reshape(-1, shape[-1])
     M = rows.shape[0]
@@ -57,9 +62,14 @@ def test_li_bwd_scan_against_oracle_and_sequential_kernel(slayer, shape, nd):
     for t in range(shape[-1] - 1, -1, -1):
         acc = a * acc + go[:, t:t + 1]
         ref[:, t:t + 1] = acc
-    assert_scale(gi.reshape(-1, shape[-1])[pick.to(dev())], ref, 'scan vs step-by-step recurrence (float32)')
     want64, mag64 = li_bwd_f64(go, a.float())          # every element against the magnitudes of its own terms
-    assert_sum(gi.reshape(-1, shape[-1])[pick.to(dev())], want64, mag64, 'scan vs float64 recurrence, elementwise')
+    got = gi.reshape(-1, shape[-1])[pick.to(dev())]
+    assert_sum(got, want64, mag64, 'scan vs float64 recurrence, elementwise')
+    if long_rows:
+        assert_sum(seq.reshape(-1, shape[-1])[pick.to(dev())], want64, mag64, 'step-by-step kernel vs float64 recurrence')
+        assert_sum(ref, want64, mag64, 'step-by-step recurrence (float32) vs float64 recurrence')
+    else:
+        assert_scale(got, ref, 'scan vs step-by-step recurrence (float32)')
     # decay gradient in float64 from the sequential result
     assert_sum(gd, *li_decay_grad_f64(seq, y, nd), 'grad_decay')
 
