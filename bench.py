@@ -667,9 +667,11 @@ class ConvSynapse(Cuba):
     the input spikes.  The synapse kernel works on the time-innermost layout as it is; the neuron reads its output in
     place.  Weights are multiples of 1/64 (quantised, as a SLAYER synapse's are), so the weighted spikes are exact
     and the forward parity check stays bit for bit.  Bytes per neuron-timestep of the output tensor."""
-    name = 'Conv synapse (3x3, 8 -> 16 channels) -> fused CUBA neuron, fwd+bwd (input gradient)'
+    name = 'Conv synapse (3x3, 8 -> 16 channels) -> fused CUBA neuron, fwd+bwd (input and weight gradients)'
     ops = [('conv_synapse', 'synapse_conv_row_kernel', 6), ('cuba_fwd', 'stream_kernel_staged<CubaFwd>', 16),
-           ('cuba_bwd', 'cuba_bwd_scan_kernel', 16), ('conv_synapse_bwd', 'synapse_conv_row_kernel', 6)]
+           ('cuba_bwd', 'cuba_bwd_scan_kernel', 16), ('conv_synapse_bwd', 'synapse_conv_row_kernel', 6),
+           ('conv_synapse_wgrad', 'synapse_wgrad_kernel', 6)]
+    weight_gradient = True
     note = Cuba.note + '; input spikes Bernoulli(0.05) on 8 channels, weights round(N(0, 0.3) * 64) / 64'
     in_channels = 8
 
@@ -699,6 +701,9 @@ class ConvSynapse(Cuba):
             g_z, _, _ = self.F._bwd(self.g, vol, cur, self.d_i, self.d_v, self.thr, 1.0, 1.0, False)
         with t('conv_synapse_bwd'):
             g_s = self.synapse_back(g_z)
+        if self.weight_gradient:
+            with t('conv_synapse_wgrad'):
+                self.g_w = self.syn._weight_gradient(self.s, self.wgt.shape, g_z, (1, 1), (1, 1), (1, 1))
         return spk, g_s
 
     def cpu_step(self, n, sl=None):
@@ -720,10 +725,12 @@ class ConvSynapse(Cuba):
 
 class ConvSynapseLibrary(ConvSynapse):
     """The same stack with the reference's own call for the synapse: the library convolution transposes the tensor to
-    channels-last and back around its kernel (three extra passes each way)."""
-    name = 'Conv synapse by F.conv3d (library kernel + layout transposes) -> fused CUBA neuron, fwd+bwd (input gradient)'
+    channels-last and back around its kernel (three extra passes each way).  Without the weight gradient:
+    torch.nn.grad.conv3d_weight takes 1.3 s per call on this tensor on this platform."""
+    name = 'Conv synapse by F.conv3d (library kernel + layout transposes) -> fused CUBA neuron, fwd+bwd (input gradient only)'
     ops = [('conv_synapse', 'F.conv3d: library conv + batched_transpose x3', 6), ('cuba_fwd', 'stream_kernel_staged<CubaFwd>', 16),
            ('cuba_bwd', 'cuba_bwd_scan_kernel', 16), ('conv_synapse_bwd', 'conv3d_input: library conv + transposes', 6)]
+    weight_gradient = False
 
     def synapse(self, s):
         return torch.nn.functional.conv3d(s, self.wgt, None, (1, 1, 1), (1, 1, 0))

@@ -44,7 +44,7 @@ extern "C" {
 
 #define SLAYER_EINVAL   (-1)   /* inconsistent sizes (M, T, neurons_per_batch, num_params, ...) */
 #define SLAYER_ENULL    (-2)   /* a required pointer is NULL */
-#define SLAYER_ERANGE   (-3)   /* a size exceeds what the kernels index (M*T >= 2^40, T >= 2^31, K > 4096 ...) */
+#define SLAYER_ERANGE   (-3)   /* a size exceeds what the kernels index (M*T >= 2^40, T >= 2^31, min(K, T) > 12288 ...) */
 #define SLAYER_ESCRATCH (-4)   /* a size exceeds the library's built-in scratch buffer (slayer_li_bwd_static) */
 #define SLAYER_ENOFLAG  (-5)   /* the range flag could not be set up (slayer_range_status) */
 
@@ -293,7 +293,8 @@ int slayer_delay_bwd(float *grad_in, float *grad_sum, const float *grad_out, con
 /* ---- temporal filter ---------------------------------------------------------------------- */
 
 /* Replaces conv fwd (utils/filter/conv.cu:80-125): out[m][t] = Ts * sum_{i<K, t-i>=0} filt[i] * in[m][t-i].
- * K <= 4096 (SLAYER_ERANGE beyond).  float32 throughout; for 32 < K <= 128 the products are formed on the matrix
+ * Any K: only the first min(K, T) taps can meet a sample of the row, and only they are read (SLAYER_ERANGE when
+ * min(K, T) > 12288: rows and filters both longer than that).  float32 throughout; for 32 < K <= 128 the products are formed on the matrix
  * cores from three bfloat16 parts per operand (each operand to within 2^-27, sums in float32): as close to the
  * exact sum as float32 multiply-adds, for every finite operand of at least about 3e-33 in magnitude (smaller
  * ones enter with an absolute error of up to 1.2e-38). */
@@ -319,6 +320,21 @@ int slayer_conv_synapse(float *out, const float *in, const float *weight,
                         int64_t N, int64_t Ci, int64_t Co, int64_t H, int64_t W, int64_t T,
                         int64_t kh, int64_t kw, int64_t stride_h, int64_t stride_w,
                         int64_t pad_h, int64_t pad_w, int64_t dil_h, int64_t dil_w, void *stream);
+
+/* The gradient of the synapse's weights (what autograd obtains from conv3d's backward, synapse/layer.py:297-323):
+ * grad_weight[co][ci][y][x] = sum over n, ho, wo, t of grad_out[n][co][ho][wo][t] *
+ *                             in[n][ci][ho * stride_h + y * dil_h - pad_h][wo * stride_w + x * dil_w - pad_w][t],
+ * reduced along time on the matrix cores (float32), the partial tiles of the waves added in double in a fixed
+ * order.  workspace: slayer_conv_synapse_wgrad_workspace(...) floats of device memory, 16-byte aligned, contents
+ * undefined afterwards (that function returns a negative error code for sizes the entry point refuses).  Same
+ * limits as slayer_conv_synapse, up to 4096 taps. */
+int64_t slayer_conv_synapse_wgrad_workspace(int64_t N, int64_t Ci, int64_t Co, int64_t H, int64_t W, int64_t T,
+                                            int64_t kh, int64_t kw, int64_t stride_h, int64_t pad_h, int64_t dil_h);
+int slayer_conv_synapse_wgrad(float *grad_weight, const float *grad_out, const float *in,
+                              int64_t N, int64_t Ci, int64_t Co, int64_t H, int64_t W, int64_t T,
+                              int64_t kh, int64_t kw, int64_t stride_h, int64_t stride_w,
+                              int64_t pad_h, int64_t pad_w, int64_t dil_h, int64_t dil_w,
+                              float *workspace, int64_t workspace_floats, void *stream);
 
 /* ---- sigma-delta ---------------------------------------------------------------------------- */
 

@@ -17,7 +17,7 @@ namespace slayer {
 
 constexpr int kOutPerLane = 8;
 constexpr int kSeg = kWave * kOutPerLane;      // outputs per workgroup
-constexpr int kMaxTaps = 4096;
+constexpr int kMaxTaps = 12288;          // window of 512 + K samples in 64 KB of LDS
 
 // LDS index of window position p (one pad word per 8 samples).  For p = 8*lane + d this is
 // 9*lane + d + (d >> 3): the lane part is computed once, the rest is wave-uniform (scalar ALU).
@@ -519,6 +519,9 @@ static int conv_launch(float* out, const float* in, const float* filt, int64_t K
     if (M == 0 || T == 0) return 0;
     if (!out || !in || !filt) return SLAYER_ENULL;
     if (K < 1) return SLAYER_EINVAL;
+    // tap i meets sample t - i (conv) or t + i (corr) of the same row: taps from T on meet nothing and are not read
+    // (the reference's kernels skip them one by one, utils/filter/conv.cu:42-46)
+    if (K > T) K = T;
     if (K > kMaxTaps) return SLAYER_ERANGE;
     // the matrix kernel walks the tensor as one flat stream of whole quads: rows of any length from 16 steps on, as
     // long as the tensor as a whole is a whole number of quads

@@ -18,6 +18,8 @@
 
 namespace slayer {
 
+int launch_zero_fill(float* p, int64_t n, hipStream_t stream);          // li.hip
+
 typedef float syn_f4 __attribute__((ext_vector_type(4)));
 
 constexpr int kSynTile = 64;            // time steps per tile
@@ -226,6 +228,157 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_row_kernel(con
     }
 }
 
+// Gradient of the weights: grad_w[co][k] = sum over batch, output pixels and time of grad_out[co][pixel][t] *
+// (input row of tap k at that pixel)[t] -- a [Co x P] x [P x K] product with P = N * Ho * Wo * T positions, reduced
+// along time on the matrix cores: lane (kk, j) loads steps 4 kk .. 4 kk + 3 of a 16-step group of the gradient row of
+// channel co0 + j (the A operand of four products) and of the input row of tap 16 tt + j (the B operand), so that
+// a group of 16 steps costs 1 + NTT loads and 4 NTT products and adds to NTT accumulator tiles [16 channels x 16
+// taps].  A wave owns one output row of one batch entry and a share of the time axis, walks the row pixel by pixel
+// and leaves its tiles in the workspace; synapse_wgrad_reduce_kernel adds the tiles of all waves in double, in a
+// fixed order.  Filters of more than 16 NTT taps take several passes (grid dimension z).
+struct SynapseWgrad {
+    float* partial;                     // [items][passes][NTT][64] quads
+    const float* grad_out;
+    const float* in;
+    int N, Ci, Co, H, W, Ho, Wo, T;
+    int kh, kw, sh, sw, ph, pw, dh, dw;
+    int K, passes;                      // taps, passes of 16 NTT taps
+    int tparts, tlen;                   // shares of the time axis, steps per share (a multiple of 32)
+    int items;                          // (share of time, output row) pairs of one (batch entry, channel block)
+};
+
+template <int NTT>
+__global__ __launch_bounds__(kSynWaves * kWave) void synapse_wgrad_kernel(const SynapseWgrad p) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    constexpr int Kp = NTT * 16;
+    int* tap_off = reinterpret_cast<int*>(lds);         // [Kp] bytes
+    int* tap_dy = tap_off + Kp;                         // [Kp]
+    int* tap_dx = tap_dy + Kp;                          // [Kp]
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int groups = (p.items + kSynWaves - 1) / kSynWaves;
+    const int cobs = (p.Co + 15) / 16;
+    int b = blockIdx.x;
+    const int ig = b % groups; b /= groups;
+    const int cob = b % cobs;
+    const int n = b / cobs;
+    const int co0 = cob * 16;
+    const int pass = blockIdx.y;
+    const int k0 = pass * Kp;
+
+    for (int kl = tid; kl < Kp; kl += kSynWaves * kWave) {
+        const int k = k0 + kl;
+        const int ci = k / (p.kh * p.kw), r = k - ci * (p.kh * p.kw), y = r / p.kw, x = r - y * p.kw;
+        const int dy = y * p.dh - p.ph, dx = x * p.dw - p.pw;
+        tap_dy[kl] = k < p.K ? dy : (1 << 28);                           // a tap that does not exist: always outside
+        tap_dx[kl] = dx;
+        tap_off[kl] = (((ci * p.H + dy) * p.W) + dx) * p.T * 4;
+    }
+    __syncthreads();
+
+    const int item = ig * kSynWaves + wave;
+    if (item >= p.items) return;
+    const int tpart = item % p.tparts;
+    const int ho = item / p.tparts;
+    const int kk = lane >> 4, j = lane & 15;
+    const int hin = ho * p.sh;
+    const int64_t in_plane = (int64_t)p.Ci * p.H * p.W * p.T;
+    const __amdgpu_buffer_rsrc_t src = make_rsrc(p.in + (int64_t)n * in_plane, (unsigned)(in_plane * 4));
+    const int64_t out_plane = (int64_t)p.Co * p.Ho * p.Wo * p.T;
+    const __amdgpu_buffer_rsrc_t grd = make_rsrc(p.grad_out + (int64_t)n * out_plane, (unsigned)(out_plane * 4));
+    const int col = p.T * 4;
+    const bool co_ok = co0 + j < p.Co;
+    const int g_row = (co0 + j) * (p.Ho * p.Wo * col) + ho * p.Wo * col;  // gradient row of this lane's channel
+    // this lane's taps: offset of the input row relative to the pixel, and whether its image row exists
+    int my_off[NTT], my_dx[NTT];
+    bool my_row[NTT];
+#pragma unroll
+    for (int tt = 0; tt < NTT; ++tt) {
+        my_off[tt] = tap_off[16 * tt + j];
+        my_dx[tt] = tap_dx[16 * tt + j];
+        my_row[tt] = (unsigned)(hin + tap_dy[16 * tt + j]) < (unsigned)p.H;
+    }
+    syn_f4 acc[NTT][2];                                                  // two chains per tile: no product waits for the one before
+#pragma unroll
+    for (int tt = 0; tt < NTT; ++tt) acc[tt][0] = acc[tt][1] = syn_f4{0.f, 0.f, 0.f, 0.f};
+
+    const int t_lo = tpart * p.tlen, t_hi = (t_lo + p.tlen) < p.T ? (t_lo + p.tlen) : p.T;
+    for (int t0 = t_lo; t0 < t_hi; t0 += 32) {                           // one 128-byte line of every row per visit
+        for (int wo = 0; wo < p.Wo; ++wo) {
+            const int win = wo * p.sw;
+            const int pix = ((hin * p.W) + win) * col;
+            float4 g[2], q[2][NTT];
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int t = t0 + 16 * u + 4 * kk;
+                const bool t_ok = t < t_hi;                              // T and the shares are whole quads
+                g[u] = buf_load4<false>(grd, (t_ok && co_ok) ? g_row + wo * col + t * 4 : kOutOfRange);
+#pragma unroll
+                for (int tt = 0; tt < NTT; ++tt) {
+                    const bool ok = t_ok && my_row[tt] && (unsigned)(win + my_dx[tt]) < (unsigned)p.W;
+                    q[u][tt] = buf_load4<false>(src, ok ? pix + my_off[tt] + t * 4 : kOutOfRange);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+#pragma unroll
+                for (int tt = 0; tt < NTT; ++tt) {
+                    acc[tt][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(g[u].x, q[u][tt].x, acc[tt][0], 0, 0, 0);
+                    acc[tt][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(g[u].y, q[u][tt].y, acc[tt][1], 0, 0, 0);
+                }
+#pragma unroll
+                for (int tt = 0; tt < NTT; ++tt) {
+                    acc[tt][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(g[u].z, q[u][tt].z, acc[tt][0], 0, 0, 0);
+                    acc[tt][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(g[u].w, q[u][tt].w, acc[tt][1], 0, 0, 0);
+                }
+            }
+        }
+    }
+    // lane (q, j) of tile tt: channels co0 + 4 q + i, tap k0 + 16 tt + j
+    float4* dst = reinterpret_cast<float4*>(p.partial) +
+                  ((((int64_t)(n * cobs + cob) * p.items + item) * p.passes + pass) * NTT) * kWave + lane;
+#pragma unroll
+    for (int tt = 0; tt < NTT; ++tt)
+        dst[tt * kWave] = make_float4(acc[tt][0][0] + acc[tt][1][0], acc[tt][0][1] + acc[tt][1][1],
+                                      acc[tt][0][2] + acc[tt][1][2], acc[tt][0][3] + acc[tt][1][3]);
+}
+
+// grad_w[co][k] = sum over batch entries and items of the waves' tiles, in double, in a fixed order: sixteen
+// partial sums (every sixteenth tile each), then those in turn.
+constexpr int kWgradParts = 16;
+template <int NTT>
+__global__ __launch_bounds__(kWgradParts * kWave) void synapse_wgrad_reduce_kernel(
+        float* __restrict__ grad_w, const float* __restrict__ partial, int N, int Co, int K, int items, int passes) {
+    __shared__ double sums[kWgradParts][kWave][4];
+    const int lane = threadIdx.x & (kWave - 1), part = threadIdx.x >> 6, q = lane >> 4, j = lane & 15;
+    const int tt = blockIdx.x % NTT;
+    int b = blockIdx.x / NTT;
+    const int pass = b % passes;
+    const int cob = b / passes;
+    const int cobs = (Co + 15) / 16;
+    const int k = (pass * NTT + tt) * 16 + j;
+    double s[4] = {0.0, 0.0, 0.0, 0.0};
+    const float4* src = reinterpret_cast<const float4*>(partial);
+    const int64_t total = (int64_t)N * items;
+    for (int64_t at = part; at < total; at += kWgradParts) {
+        const int64_t n = at / items, item = at - n * items;
+        const float4 v = src[((((n * cobs + cob) * items + item) * passes + pass) * NTT + tt) * kWave + lane];
+        s[0] += v.x; s[1] += v.y; s[2] += v.z; s[3] += v.w;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sums[part][lane][i] = s[i];
+    __syncthreads();
+    if (part != 0) return;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        double tot = 0.0;
+        for (int pp = 0; pp < kWgradParts; ++pp) tot += sums[pp][lane][i];
+        const int co = cob * 16 + 4 * q + i;
+        if (co < Co && k < K) grad_w[(int64_t)co * K + k] = (float)tot;
+    }
+}
+
 }  // namespace slayer
 
 using namespace slayer;
@@ -295,5 +448,84 @@ extern "C" int slayer_conv_synapse(float* out, const float* in, const float* wei
         hipLaunchKernelGGL((synapse_conv_kernel<true>), grid, block, lds, st, p);
     else
         hipLaunchKernelGGL((synapse_conv_kernel<false>), grid, block, lds, st, p);
+    return (int)hipGetLastError();
+}
+
+namespace {
+
+// tap tiles per pass of the weight-gradient kernel and the shares the time axis is cut into
+int wgrad_tiles(int64_t K) { return K <= 16 ? 1 : (K <= 32 ? 2 : 5); }
+void wgrad_shape(int64_t N, int64_t Co, int64_t Ho, int64_t T, int64_t K, SynapseWgrad& p) {
+    const int ntt = wgrad_tiles(K);
+    p.passes = (int)((K + 16 * ntt - 1) / (16 * ntt));
+    // enough waves for four rounds of the chip, shares of whole 128-byte lines
+    const int64_t base = N * ((Co + 15) / 16) * Ho;
+    int64_t parts = 1;
+    while (base * parts < 16 * 1024 && parts * 2 * 32 <= T) parts *= 2;
+    int64_t len = ((T + parts - 1) / parts + 31) / 32 * 32;
+    p.tparts = (int)((T + len - 1) / len);
+    p.tlen = (int)len;
+    p.items = (int)(Ho * p.tparts);
+}
+
+}  // namespace
+
+extern "C" int64_t slayer_conv_synapse_wgrad_workspace(int64_t N, int64_t Ci, int64_t Co, int64_t H, int64_t W,
+                                                       int64_t T, int64_t kh, int64_t kw, int64_t stride_h,
+                                                       int64_t pad_h, int64_t dil_h) {
+    if (N < 0 || Ci < 1 || Co < 1 || H < 1 || W < 1 || T < 0 || kh < 1 || kw < 1 || stride_h < 1 || pad_h < 0 ||
+        dil_h < 1)
+        return SLAYER_EINVAL;
+    const int64_t Ho = (H + 2 * pad_h - dil_h * (kh - 1) - 1) / stride_h + 1;
+    if (Ho < 1) return SLAYER_EINVAL;
+    const int64_t K = Ci * kh * kw;
+    if (K > 4096 || Ho > (1 << 20) || T > (1 << 24)) return SLAYER_ERANGE;
+    SynapseWgrad p;
+    wgrad_shape(N, Co, Ho, T, K, p);
+    return N * ((Co + 15) / 16) * p.items * p.passes * wgrad_tiles(K) * 256;
+}
+
+extern "C" int slayer_conv_synapse_wgrad(float* grad_weight, const float* grad_out, const float* in,
+                                         int64_t N, int64_t Ci, int64_t Co, int64_t H, int64_t W, int64_t T,
+                                         int64_t kh, int64_t kw, int64_t stride_h, int64_t stride_w,
+                                         int64_t pad_h, int64_t pad_w, int64_t dil_h, int64_t dil_w,
+                                         float* workspace, int64_t workspace_floats, void* stream) {
+    if (N < 0 || Ci < 1 || Co < 1 || H < 1 || W < 1 || T < 0 || kh < 1 || kw < 1 || stride_h < 1 || stride_w < 1 ||
+        pad_h < 0 || pad_w < 0 || dil_h < 1 || dil_w < 1)
+        return SLAYER_EINVAL;
+    const int64_t Ho = (H + 2 * pad_h - dil_h * (kh - 1) - 1) / stride_h + 1;
+    const int64_t Wo = (W + 2 * pad_w - dil_w * (kw - 1) - 1) / stride_w + 1;
+    if (Ho < 1 || Wo < 1) return SLAYER_EINVAL;
+    if (!grad_weight) return SLAYER_ENULL;
+    const int64_t K = Ci * kh * kw, lim = (int64_t)1 << 31;
+    hipStream_t st = (hipStream_t)stream;
+    if (N == 0 || T == 0) return launch_zero_fill(grad_weight, Co * K, st);
+    if (!grad_out || !in || !workspace) return SLAYER_ENULL;
+    if ((T % 4) != 0 || !aligned16(grad_out) || !aligned16(in) || !aligned16(workspace)) return SLAYER_ERANGE;
+    if (Ci * H * W * T * 4 >= lim || Co * Ho * Wo * T * 4 >= lim || K > 4096 || pad_h > 4096 || pad_w > 4096 ||
+        H * stride_h > (1 << 20) || W * stride_w > (1 << 20) || Ho > (1 << 20) || T > (1 << 24))
+        return SLAYER_ERANGE;
+    SynapseWgrad p;
+    p.partial = workspace; p.grad_out = grad_out; p.in = in;
+    p.N = (int)N; p.Ci = (int)Ci; p.Co = (int)Co; p.H = (int)H; p.W = (int)W; p.Ho = (int)Ho; p.Wo = (int)Wo; p.T = (int)T;
+    p.kh = (int)kh; p.kw = (int)kw; p.sh = (int)stride_h; p.sw = (int)stride_w; p.ph = (int)pad_h; p.pw = (int)pad_w;
+    p.dh = (int)dil_h; p.dw = (int)dil_w;
+    p.K = (int)K;
+    wgrad_shape(N, Co, Ho, T, K, p);
+    const int ntt = wgrad_tiles(K);
+    const int64_t cobs = (Co + 15) / 16;
+    if (workspace_floats < N * cobs * p.items * p.passes * ntt * 256) return SLAYER_ERANGE;
+    const int64_t blocks = N * cobs * ((p.items + kSynWaves - 1) / kSynWaves);
+    if (blocks > 0x7fffffffLL || p.passes > 65535) return SLAYER_ERANGE;
+    const dim3 grid((unsigned)blocks, (unsigned)p.passes), block(kSynWaves * kWave);
+    const dim3 rgrid((unsigned)(cobs * p.passes * ntt));
+#define SLAYER_WGRAD(NTT)                                                                                         \
+    do {                                                                                                          \
+        hipLaunchKernelGGL((synapse_wgrad_kernel<NTT>), grid, block, NTT * 16 * 3 * sizeof(int), st, p);          \
+        hipLaunchKernelGGL((synapse_wgrad_reduce_kernel<NTT>), rgrid, dim3(kWgradParts * kWave), 0, st, grad_weight, workspace,  \
+                           (int)N, (int)Co, (int)K, p.items, p.passes);                                           \
+    } while (0)
+    if (ntt == 1) SLAYER_WGRAD(1); else if (ntt == 2) SLAYER_WGRAD(2); else SLAYER_WGRAD(5);
+#undef SLAYER_WGRAD
     return (int)hipGetLastError();
 }

@@ -4,8 +4,9 @@ Interface of lava.lib.dl.slayer.synapse.Conv (synapse/layer.py:178-323 in the re
 applied at every time step of an NCHWT tensor.  The reference calls ``F.conv3d`` with a kernel of (kh, kw, 1); the
 library behind it wants channels last and transposes the tensor there and back around its kernel.  Here
 slayer_conv_synapse of libslayer_hip.so computes it where the tensor lies, so the neuron that follows reads the
-result in place.  What the kernel does not take (grouped convolutions, rows that are not whole quads of time steps)
-goes to ``F.conv3d`` as before; the weight gradient always does (``torch.nn.grad.conv3d_weight``).
+result in place; the input gradient is the same kernel on the flipped, transposed weights and the weight gradient
+slayer_conv_synapse_wgrad.  What the kernels do not take (grouped convolutions, rows that are not whole quads of
+time steps) goes to ``F.conv3d`` and its gradients as before.
 """
 import torch
 import torch.nn.functional as F
@@ -70,9 +71,33 @@ class _ConvSynapse(torch.autograd.Function):
                 grad_input = torch.nn.grad.conv3d_input(input.shape, weight, grad_output, stride + (1,),
                                                         padding + (0,), dilation + (1,), 1)
         if ctx.needs_input_grad[1]:
-            grad_weight = torch.nn.grad.conv3d_weight(input, weight.shape, grad_output, stride + (1,), padding + (0,),
-                                                      dilation + (1,), 1)
+            grad_weight = _weight_gradient(input, weight.shape, grad_output, stride, padding, dilation)
+            if grad_weight is None:
+                grad_weight = torch.nn.grad.conv3d_weight(input, weight.shape, grad_output, stride + (1,),
+                                                          padding + (0,), dilation + (1,), 1)
         return grad_input, grad_weight, None, None, None
+
+
+def _weight_gradient(input, weight_shape, grad_output, stride, padding, dilation):
+    """[Co, Ci, kh, kw, 1] gradient of the weights or None (None: outside what the kernel takes)."""
+    n, ci, h, w, t = input.shape
+    co, _, kh, kw, _ = weight_shape
+    lib = N.lib()
+    floats = lib.slayer_conv_synapse_wgrad_workspace(n, ci, co, h, w, t, kh, kw, stride[0], padding[0], dilation[0])
+    if floats == _ERANGE:
+        return None
+    if floats < 0:
+        N.check(int(floats))
+    grad = torch.empty((co, ci, kh, kw, 1), dtype=torch.float32, device=input.device)
+    workspace = torch.empty(max(int(floats), 4), dtype=torch.float32, device=input.device)
+    with N.device_guard(input.device):
+        code = lib.slayer_conv_synapse_wgrad(N.ptr(grad), N.ptr(grad_output), N.ptr(input), n, ci, co, h, w, t, kh, kw,
+                                             stride[0], stride[1], padding[0], padding[1], dilation[0], dilation[1],
+                                             N.ptr(workspace), workspace.numel(), N.stream_handle())
+    if code == _ERANGE:
+        return None
+    N.check(code)
+    return grad
 
 
 def conv_synapse(input, weight, stride=1, padding=0, dilation=1, groups=1):

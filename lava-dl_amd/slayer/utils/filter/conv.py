@@ -66,8 +66,9 @@ def conv(input, filter, sampling_time=1):
     """Convolution in time; the last axis of ``input`` is time, ``filter`` is
     flattened to 1-D.  Output has the shape of ``input``.
 
-    Two deviations from the reference: filters longer than 4096 taps raise (the reference accepts any
-    length), and for filters of 9 to 128 taps a non-finite input sample also makes the few neighbouring
+    Filters of any length are accepted: only the first ``min(K, T)`` taps can meet a sample of a row, and only
+    they are read (rows *and* filters longer than 12288 raise).  One deviation from the reference: for filters
+    of 9 to 128 taps a non-finite input sample also makes the few neighbouring
     outputs of its row NaN whose window holds it beyond the filter's support (the matrix-core kernel
     multiplies those samples by zero taps instead of skipping them); finite inputs give the same sums."""
     if input.dim() == 1:

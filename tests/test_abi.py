@@ -66,7 +66,7 @@ def test_argument_validation_happens_before_any_launch():
     code = L.slayer_range_status(ctypes.byref(raised), 0)
     assert code == (0 if torch.cuda.is_available() else -5)
     assert b'range flag' in L.slayer_error_string(-5)
-    assert L.slayer_conv(one, one, one, 5000, 1.0, 8, 8, None) == ERANGE
+    assert L.slayer_conv(one, one, one, 13000, 1.0, 8, 13000, None) == ERANGE      # rows and filter beyond the window
     assert L.slayer_shift(one, one, None, 1, 1.0, 8, 3, 8, None) == EINVAL
     assert L.slayer_spike_fwd(one, one, one, 3, 0.0, 0, 1.0, 8, None) == EINVAL             # 3 thresholds for 8 samples
     assert L.slayer_ath_fwd(one, one, one, one, one, one, one, 1 << 40, 0, 64, 8, 4, 1, 1, 1, 1, 8, None) == ERANGE

@@ -1,6 +1,7 @@
 """The convolution synapse on time-innermost tensors (csrc/synapse.hip, slayer.synapse.Conv) against the oracle's
 float64 evaluation of the reference's call (synapse/layer.py:297-323: F.conv3d with a (kh, kw, 1) kernel on NCHWT),
-every output element to 1e-5 of the sum of the magnitudes of its terms; the input gradient against float64 autograd;
+every output element to 1e-5 of the sum of the magnitudes of its terms; the gradients of the input and of the
+weights (slayer_conv_synapse_wgrad) against float64 autograd to the same bar;
 shapes the kernel does not take go to the library call and give the same result."""
 import pytest
 import torch
@@ -40,7 +41,7 @@ def _check(slayer, shape, co, kernel, stride, padding, dilation, what, backward=
         xa, wa = x.abs().double().requires_grad_(), wt.abs().double().requires_grad_()
         F.conv3d(xa, wa, None, tuple(stride) + (1,), tuple(padding) + (0,), tuple(dilation) + (1,)).backward(g.abs().double())
         assert_sum(xg.grad, xd.grad, xa.grad, what + ' grad input')
-        assert_sum(wg.grad, wd.grad, wa.grad, what + ' grad weight', rel=1e-4)      # torch's own kernel, float32 sums
+        assert_sum(wg.grad, wd.grad, wa.grad, what + ' grad weight')
 
 
 @pytest.mark.parametrize('shape,co,kernel,stride,padding,dilation', [
@@ -50,6 +51,9 @@ def _check(slayer, shape, co, kernel, stride, padding, dilation, what, backward=
     ((2, 4, 12, 10, 100), 40, (3, 2), (1, 2), (0, 1), (2, 1)),      # three blocks of output channels, mixed geometry
     ((3, 16, 8, 8, 36), 32, (1, 1), (1, 1), (0, 0), (1, 1)),        # 1x1: a dense synapse per pixel
     ((1, 5, 10, 12, 260), 7, (3, 3), (1, 1), (0, 0), (2, 2)),       # no padding, dilation 2
+    ((2, 16, 7, 9, 72), 8, (3, 3), (1, 1), (1, 1), (1, 1)),         # 144 taps: two passes of the weight gradient
+    ((3, 1, 9, 8, 132), 4, (3, 3), (1, 1), (1, 1), (1, 1)),         # 9 taps: one tile of taps
+    ((1, 20, 5, 5, 1032), 3, (3, 3), (1, 1), (2, 2), (1, 1)),       # 180 taps, long rows: several shares of time
 ])
 def test_conv_synapse_against_the_oracle(slayer, shape, co, kernel, stride, padding, dilation):
     _check(slayer, shape, co, kernel, stride, padding, dilation, f'{shape} -> {co}')
@@ -100,3 +104,28 @@ def test_conv_synapse_at_the_size_of_the_benchmark_tensor(slayer):
     neuron = slayer.neuron.cuba.Neuron(1.0, 0.25, 0.03).to(dev())
     spikes = neuron(z)
     assert spikes.shape == z.shape and 0 < float(spikes.sum()) < spikes.numel()
+
+
+def test_weight_gradient_at_the_size_of_the_benchmark_tensor(slayer):
+    """grad_weight of the synapse above at full size against nine float64 matrix products over the shifted views
+    (the defining sum), 1e-5 of the sum of the terms' magnitudes."""
+    gen = torch.Generator(device=dev()).manual_seed(10)
+    shape = (32, 8, 32, 32, 300)
+    x = (torch.rand(shape, device=dev(), generator=gen) < 0.05).float()
+    g = torch.randn((32, 16, 32, 32, 300), device=dev(), generator=gen)
+    w = (torch.randn(16, 8, 3, 3, 1, device=dev(), generator=gen) * 0.3).requires_grad_()
+    slayer.synapse.conv_synapse(x, w, 1, 1, 1).backward(g)
+    want = torch.empty(16, 8, 3, 3, dtype=torch.float64, device=dev())
+    mag = torch.empty_like(want)
+    xp = F.pad(x, (0, 0, 1, 1, 1, 1))
+    for n0 in range(0, 32, 8):                                     # float64 copies of a quarter of the batch at a time
+        gf = g[n0:n0 + 8].permute(1, 0, 2, 3, 4).reshape(16, -1).double()
+        for y in range(3):
+            for xx in range(3):
+                v = xp[n0:n0 + 8, :, y:y + 32, xx:xx + 32, :].permute(1, 0, 2, 3, 4).reshape(8, -1).double()
+                if n0 == 0:
+                    want[:, :, y, xx] = 0
+                    mag[:, :, y, xx] = 0
+                want[:, :, y, xx] += gf @ v.t()
+                mag[:, :, y, xx] += gf.abs() @ v.t()
+    assert_sum(w.grad[..., 0], want, mag, 'grad weight at [32,8,32,32,300]')

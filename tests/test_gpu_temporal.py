@@ -100,6 +100,43 @@ def test_conv_corr(slayer, shape, K):
     assert np.allclose(y, np.convolve(row, f.double().numpy())[:row.size], rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize('shape,K', [((6, 300), 5000), ((3, 40), 4097), ((2, 3, 9000), 6000), ((4, 100), 100000),
+                                     ((2, 5000), 12288), ((5, 129), 129), ((3, 12), 13)])
+def test_filters_longer_than_the_rows_or_than_4096_taps(slayer, shape, K):
+    """The reference takes filters of any length (utils/filter/conv.cu:42-46 skips the taps that meet no sample one
+    by one).  Only the first min(K, T) taps can meet a sample: results equal those of the truncated filter bit for
+    bit and scipy.signal.lfilter with the whole filter in float64; a non-finite tap beyond the row length changes
+    nothing, as in the reference."""
+    from scipy.signal import lfilter
+    gen = torch.Generator().manual_seed(seed_of('long filter', shape, K))
+    x = torch.randn(shape, generator=gen)
+    f = torch.randn(K, generator=gen) / K ** 0.5
+    T = shape[-1]
+    rows = x.reshape(-1, T).double().numpy()
+    fd = f.double().numpy()
+    conv_ref = lfilter(fd, [1.0], rows, axis=-1)
+    corr_ref = lfilter(fd, [1.0], rows[:, ::-1], axis=-1)[:, ::-1]
+    y = slayer.utils.filter.conv(x.to(dev()), f.to(dev()), 0.5)
+    z = slayer.utils.filter.corr(x.to(dev()), f.to(dev()), 0.5)
+    scale = 0.5 * np.abs(fd[:T]).sum() * np.abs(rows).max()
+    assert np.abs(y.reshape(-1, T).cpu().double().numpy() - 0.5 * conv_ref).max() <= 1e-5 * scale
+    assert np.abs(z.reshape(-1, T).cpu().double().numpy() - 0.5 * corr_ref).max() <= 1e-5 * scale
+    if K > T:
+        short = f[:T].contiguous().to(dev())
+        assert torch.equal(y, slayer.utils.filter.conv(x.to(dev()), short, 0.5))
+        assert torch.equal(z, slayer.utils.filter.corr(x.to(dev()), short, 0.5))
+        wild = f.clone()
+        wild[T:] = float('inf')
+        assert torch.equal(y, slayer.utils.filter.conv(x.to(dev()), wild.to(dev()), 0.5))
+
+
+def test_rows_and_filters_both_beyond_the_window_are_refused(slayer):
+    x = torch.zeros(1, 12292, device=dev())
+    with pytest.raises(RuntimeError, match='-3'):
+        slayer.utils.filter.conv(x, torch.ones(12289, device=dev()))
+    slayer.utils.filter.conv(x, torch.ones(12288, device=dev()))
+
+
 @pytest.mark.parametrize('shape,K', [((16, 64), 9), ((5, 3, 16), 16), ((37, 132), 17), ((3, 700, 48), 32), ((2, 9, 1000), 33),
                                      ((64, 256, 100), 64), ((1, 20, 2048), 64), ((130, 4), 64), ((50, 260), 65),
                                      ((7, 11, 300), 100), ((33, 520), 128), ((33, 520), 129), ((4, 12), 40),
