@@ -344,38 +344,209 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_wgrad_kernel(const 
                                       acc[tt][0][2] + acc[tt][1][2], acc[tt][0][3] + acc[tt][1][3]);
 }
 
-// grad_w[co][k] = sum over batch entries and items of the waves' tiles, in double, in a fixed order: sixteen
-// partial sums (every sixteenth tile each), then those in turn.
+// The common case again (unit stride and dilation along the image row, KW taps per row): the taps of a tile are 16
+// (input channel, kernel row) pairs at one input column, and that column meets KW output pixels, one per tap of the
+// row -- so the wave walks the input columns of its image row, keeps the gradient quads of the last KW pixels in
+// registers (one new load per column), and a column costs 1 + NPT loads for KW * NPT * 4 products per 16 steps instead
+// of 1 + KW * NPT / ... loads of the form above.  Accumulator tile (x, pt): [16 channels x 16 pairs] for tap x.
+#ifndef SLAYER_WGRAD_GROUPS
+#define SLAYER_WGRAD_GROUPS 4
+#endif
+constexpr int kWgU = SLAYER_WGRAD_GROUPS;      // groups of 16 steps per visit of a column
+
+template <int KW, int NPT>
+__global__ __launch_bounds__(kSynWaves * kWave) void synapse_wgrad_row_kernel(const SynapseWgrad p) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    constexpr int Pp = NPT * 16;
+    int* pair_off = reinterpret_cast<int*>(lds);        // [Pp] bytes, relative to the start of the wave's image row
+    int* pair_dy = pair_off + Pp;                       // [Pp]
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int groups = (p.items + kSynWaves - 1) / kSynWaves;
+    const int cobs = (p.Co + 15) / 16;
+    int b = blockIdx.x;
+    const int ig = b % groups; b /= groups;
+    const int cob = b % cobs;
+    const int n = b / cobs;
+    const int co0 = cob * 16;
+    const int pass = blockIdx.y;
+    const int col = p.T * 4;
+
+    for (int pl = tid; pl < Pp; pl += kSynWaves * kWave) {
+        const int pr = pass * Pp + pl;
+        const int ci = pr / p.kh, y = pr - ci * p.kh;
+        const int dy = y * p.dh - p.ph;
+        pair_dy[pl] = pr < p.Ci * p.kh ? dy : (1 << 28);                 // a pair that does not exist: always outside
+        pair_off[pl] = ((ci * p.H + dy) * p.W) * col;
+    }
+    __syncthreads();
+
+    const int item = ig * kSynWaves + wave;
+    if (item >= p.items) return;
+    const int tpart = item % p.tparts;
+    const int ho = item / p.tparts;
+    const int kk = lane >> 4, j = lane & 15;
+    const int hin = ho * p.sh;
+    const int64_t in_plane = (int64_t)p.Ci * p.H * p.W * p.T;
+    const __amdgpu_buffer_rsrc_t src = make_rsrc(p.in + (int64_t)n * in_plane, (unsigned)(in_plane * 4));
+    const int64_t out_plane = (int64_t)p.Co * p.Ho * p.Wo * p.T;
+    const __amdgpu_buffer_rsrc_t grd = make_rsrc(p.grad_out + (int64_t)n * out_plane, (unsigned)(out_plane * 4));
+    const bool co_ok = co0 + j < p.Co;
+    const int g_row = (co0 + j) * (p.Ho * p.Wo * col) + ho * p.Wo * col;  // gradient row of this lane's channel
+    const int s_row = hin * p.W * col;                                   // the wave's image row, before the pairs' offsets
+    int my_off[NPT];
+    bool my_row[NPT];
+#pragma unroll
+    for (int pt = 0; pt < NPT; ++pt) {
+        my_off[pt] = s_row + pair_off[16 * pt + j];
+        my_row[pt] = (unsigned)(hin + pair_dy[16 * pt + j]) < (unsigned)p.H;
+    }
+    syn_f4 acc[KW][NPT];
+#pragma unroll
+    for (int x = 0; x < KW; ++x)
+#pragma unroll
+        for (int pt = 0; pt < NPT; ++pt) acc[x][pt] = syn_f4{0.f, 0.f, 0.f, 0.f};
+
+    const int t_lo = tpart * p.tlen, t_hi = (t_lo + p.tlen) < p.T ? (t_lo + p.tlen) : p.T;
+    for (int t0 = t_lo; t0 < t_hi; t0 += 16 * kWgU) {                    // whole 128-byte lines of every row per visit
+        int toff[kWgU];
+        bool t_ok[kWgU];
+#pragma unroll
+        for (int u = 0; u < kWgU; ++u) {
+            const int t = t0 + 16 * u + 4 * kk;
+            t_ok[u] = t < t_hi;                                          // T and the shares are whole quads
+            toff[u] = t * 4;
+        }
+        auto grad_at = [&](int wo, int u) {
+            return buf_load4<false>(grd, (t_ok[u] && co_ok && (unsigned)wo < (unsigned)p.Wo) ? g_row + wo * col + toff[u]
+                                                                                             : kOutOfRange);
+        };
+        // gw[x][u]: the gradient at pixel c + pw - x for the column c at hand; gw[0] arrives with the column
+        float4 gw[KW][kWgU];
+#pragma unroll
+        for (int x = 1; x < KW; ++x)
+#pragma unroll
+            for (int u = 0; u < kWgU; ++u) gw[x][u] = grad_at(p.pw - x, u);
+        for (int c = 0; c < p.W; ++c) {
+            float4 q[kWgU][NPT];
+#pragma unroll
+            for (int u = 0; u < kWgU; ++u) {
+                gw[0][u] = grad_at(c + p.pw, u);
+#pragma unroll
+                for (int pt = 0; pt < NPT; ++pt)
+                    q[u][pt] = buf_load4<false>(src, (t_ok[u] && my_row[pt]) ? my_off[pt] + c * col + toff[u] : kOutOfRange);
+            }
+#pragma unroll
+            for (int u = 0; u < kWgU; ++u) {
+#pragma unroll
+                for (int x = 0; x < KW; ++x)
+#pragma unroll
+                    for (int pt = 0; pt < NPT; ++pt) {
+                        acc[x][pt] = __builtin_amdgcn_mfma_f32_16x16x4f32(gw[x][u].x, q[u][pt].x, acc[x][pt], 0, 0, 0);
+                    }
+#pragma unroll
+                for (int x = 0; x < KW; ++x)
+#pragma unroll
+                    for (int pt = 0; pt < NPT; ++pt) {
+                        acc[x][pt] = __builtin_amdgcn_mfma_f32_16x16x4f32(gw[x][u].y, q[u][pt].y, acc[x][pt], 0, 0, 0);
+                    }
+#pragma unroll
+                for (int x = 0; x < KW; ++x)
+#pragma unroll
+                    for (int pt = 0; pt < NPT; ++pt) {
+                        acc[x][pt] = __builtin_amdgcn_mfma_f32_16x16x4f32(gw[x][u].z, q[u][pt].z, acc[x][pt], 0, 0, 0);
+                    }
+#pragma unroll
+                for (int x = 0; x < KW; ++x)
+#pragma unroll
+                    for (int pt = 0; pt < NPT; ++pt) {
+                        acc[x][pt] = __builtin_amdgcn_mfma_f32_16x16x4f32(gw[x][u].w, q[u][pt].w, acc[x][pt], 0, 0, 0);
+                    }
+            }
+#pragma unroll
+            for (int x = KW - 1; x >= 1; --x)
+#pragma unroll
+                for (int u = 0; u < kWgU; ++u) gw[x][u] = gw[x - 1][u];
+        }
+    }
+    // lane (q, j) of tile (x, pt): channels co0 + 4 q + i, pair 16 (pass NPT + pt) + j, tap x of its row
+    float4* dst = reinterpret_cast<float4*>(p.partial) +
+                  ((((int64_t)(n * cobs + cob) * p.items + item) * p.passes + pass) * (KW * NPT)) * kWave + lane;
+#pragma unroll
+    for (int x = 0; x < KW; ++x)
+#pragma unroll
+        for (int pt = 0; pt < NPT; ++pt)
+            dst[(x * NPT + pt) * kWave] = make_float4(acc[x][pt][0], acc[x][pt][1], acc[x][pt][2], acc[x][pt][3]);
+}
+
+// grad_w[co][k] = sum over batch entries and items of the waves' tiles, in double, in a fixed order, in two
+// launches: block (tile, chunk) adds the tiles of its chunk of the (batch entry, item) pairs -- sixteen partial sums
+// (every sixteenth pair each), then those in turn -- into stage[chunk][tile]; the second launch adds the chunks and
+// writes the gradient.  `tiles` tiles per wave and pass; tile tl holds taps k = 16 (pass tiles + tl) + j
+// (row_kw == 0) or, for the row kernel, pairs 16 (pass npt + tl % npt) + j at tap x = tl / npt of their row:
+// k = pair * row_kw + x.
 constexpr int kWgradParts = 16;
-template <int NTT>
+constexpr int kWgradChunks = 32;
 __global__ __launch_bounds__(kWgradParts * kWave) void synapse_wgrad_reduce_kernel(
-        float* __restrict__ grad_w, const float* __restrict__ partial, int N, int Co, int K, int items, int passes) {
+        double* __restrict__ stage, const float* __restrict__ partial, int N, int Co, int items, int passes, int tiles) {
     __shared__ double sums[kWgradParts][kWave][4];
-    const int lane = threadIdx.x & (kWave - 1), part = threadIdx.x >> 6, q = lane >> 4, j = lane & 15;
-    const int tt = blockIdx.x % NTT;
-    int b = blockIdx.x / NTT;
+    const int lane = threadIdx.x & (kWave - 1), part = threadIdx.x >> 6;
+    const int tl = blockIdx.x % tiles;
+    int b = blockIdx.x / tiles;
     const int pass = b % passes;
     const int cob = b / passes;
     const int cobs = (Co + 15) / 16;
-    const int k = (pass * NTT + tt) * 16 + j;
     double s[4] = {0.0, 0.0, 0.0, 0.0};
     const float4* src = reinterpret_cast<const float4*>(partial);
     const int64_t total = (int64_t)N * items;
-    for (int64_t at = part; at < total; at += kWgradParts) {
+    const int64_t per = (total + kWgradChunks - 1) / kWgradChunks;
+    const int64_t lo = blockIdx.y * per, hi = (lo + per) < total ? (lo + per) : total;
+    for (int64_t at = lo + part; at < hi; at += kWgradParts) {
         const int64_t n = at / items, item = at - n * items;
-        const float4 v = src[((((n * cobs + cob) * items + item) * passes + pass) * NTT + tt) * kWave + lane];
+        const float4 v = src[((((n * cobs + cob) * items + item) * passes + pass) * tiles + tl) * kWave + lane];
         s[0] += v.x; s[1] += v.y; s[2] += v.z; s[3] += v.w;
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) sums[part][lane][i] = s[i];
     __syncthreads();
     if (part != 0) return;
+    double* dst = stage + (((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * kWave + lane) * 4;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         double tot = 0.0;
         for (int pp = 0; pp < kWgradParts; ++pp) tot += sums[pp][lane][i];
+        dst[i] = tot;
+    }
+}
+
+__global__ __launch_bounds__(kWave) void synapse_wgrad_final_kernel(float* __restrict__ grad_w,
+                                                                     const double* __restrict__ stage, int Co, int K,
+                                                                     int passes, int tiles, int row_kw, int npt) {
+    const int lane = threadIdx.x, q = lane >> 4, j = lane & 15;
+    const int tl = blockIdx.x % tiles;
+    int b = blockIdx.x / tiles;
+    const int pass = b % passes;
+    const int cob = b / passes;
+    int k;
+    if (row_kw == 0) {
+        k = (pass * tiles + tl) * 16 + j;
+    } else {
+        const int x = tl / npt, pt = tl - x * npt;
+        const int pair = (pass * npt + pt) * 16 + j;
+        k = pair * row_kw + x;
+        if (pair * row_kw >= K) k = K;                                   // a pair that does not exist
+    }
+    double tot[4] = {0.0, 0.0, 0.0, 0.0};
+    for (int c = 0; c < kWgradChunks; ++c) {
+        const double* src = stage + (((int64_t)c * gridDim.x + blockIdx.x) * kWave + lane) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) tot[i] += src[i];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
         const int co = cob * 16 + 4 * q + i;
-        if (co < Co && k < K) grad_w[(int64_t)co * K + k] = (float)tot;
+        if (co < Co && k < K) grad_w[(int64_t)co * K + k] = (float)tot[i];
     }
 }
 
@@ -453,16 +624,39 @@ extern "C" int slayer_conv_synapse(float* out, const float* in, const float* wei
 
 namespace {
 
-// tap tiles per pass of the weight-gradient kernel and the shares the time axis is cut into
-int wgrad_tiles(int64_t K) { return K <= 16 ? 1 : (K <= 32 ? 2 : 5); }
-void wgrad_shape(int64_t N, int64_t Co, int64_t Ho, int64_t T, int64_t K, SynapseWgrad& p) {
-    const int ntt = wgrad_tiles(K);
-    p.passes = (int)((K + 16 * ntt - 1) / (16 * ntt));
-    // enough waves for four rounds of the chip, shares of whole 128-byte lines
+// The form of the weight-gradient kernels for a geometry: the row kernel (tiles of 16 (channel, kernel row) pairs,
+// row_kw taps each) for unit stride and dilation along the image row with 3 or 5 taps per row, else tiles of 16
+// taps; `tiles` accumulator tiles per wave and pass; the shares the time axis is cut into.
+struct WgradForm { int row_kw, npt, tiles; };
+WgradForm wgrad_form(int64_t Ci, int64_t kh, int64_t kw, int64_t stride_w, int64_t dil_w) {
+    WgradForm f;
+    if (stride_w == 1 && dil_w == 1 && (kw == 3 || kw == 5)) {
+        const int64_t pairs = Ci * kh;
+        f.row_kw = (int)kw;
+        f.npt = pairs <= 16 ? 1 : 2;
+        f.tiles = f.row_kw * f.npt;
+    } else {
+        const int64_t K = Ci * kh * kw;
+        f.row_kw = 0;
+        f.npt = 0;
+        f.tiles = K <= 16 ? 1 : (K <= 32 ? 2 : 5);
+    }
+    return f;
+}
+void wgrad_shape(int64_t N, int64_t Ci, int64_t Co, int64_t Ho, int64_t T, int64_t kh, int64_t kw, const WgradForm& f,
+                 SynapseWgrad& p) {
+    if (f.row_kw) p.passes = (int)((Ci * kh + 16 * f.npt - 1) / (16 * f.npt));
+    else p.passes = (int)((Ci * kh * kw + 16 * f.tiles - 1) / (16 * f.tiles));
+    // about four thousand waves (one per SIMD and occupancy slot), shares of whole visits of 64 steps: a wave's
+    // set-up (tables, the gradient window) is paid once per share
+#ifndef SLAYER_WGRAD_WAVES
+#define SLAYER_WGRAD_WAVES 4096
+#endif
     const int64_t base = N * ((Co + 15) / 16) * Ho;
-    int64_t parts = 1;
-    while (base * parts < 16 * 1024 && parts * 2 * 32 <= T) parts *= 2;
-    int64_t len = ((T + parts - 1) / parts + 31) / 32 * 32;
+    const int64_t visits = (T + 63) / 64;
+    int64_t parts = (SLAYER_WGRAD_WAVES + base - 1) / base;
+    parts = parts > visits ? visits : (parts < 1 ? 1 : parts);
+    const int64_t len = (visits + parts - 1) / parts * 64;
     p.tparts = (int)((T + len - 1) / len);
     p.tlen = (int)len;
     p.items = (int)(Ho * p.tparts);
@@ -480,9 +674,16 @@ extern "C" int64_t slayer_conv_synapse_wgrad_workspace(int64_t N, int64_t Ci, in
     if (Ho < 1) return SLAYER_EINVAL;
     const int64_t K = Ci * kh * kw;
     if (K > 4096 || Ho > (1 << 20) || T > (1 << 24)) return SLAYER_ERANGE;
-    SynapseWgrad p;
-    wgrad_shape(N, Co, Ho, T, K, p);
-    return N * ((Co + 15) / 16) * p.items * p.passes * wgrad_tiles(K) * 256;
+    // enough for either form of the kernel (which one runs depends on stride and dilation along the image row)
+    int64_t need = 0;
+    for (int64_t stride_w : {1, 2}) {
+        const WgradForm f = wgrad_form(Ci, kh, kw, stride_w, 1);
+        SynapseWgrad p;
+        wgrad_shape(N, Ci, Co, Ho, T, kh, kw, f, p);
+        const int64_t floats = (N * p.items + 2 * kWgradChunks) * ((Co + 15) / 16) * p.passes * f.tiles * 256;
+        need = floats > need ? floats : need;
+    }
+    return need;
 }
 
 extern "C" int slayer_conv_synapse_wgrad(float* grad_weight, const float* grad_out, const float* in,
@@ -511,21 +712,31 @@ extern "C" int slayer_conv_synapse_wgrad(float* grad_weight, const float* grad_o
     p.kh = (int)kh; p.kw = (int)kw; p.sh = (int)stride_h; p.sw = (int)stride_w; p.ph = (int)pad_h; p.pw = (int)pad_w;
     p.dh = (int)dil_h; p.dw = (int)dil_w;
     p.K = (int)K;
-    wgrad_shape(N, Co, Ho, T, K, p);
-    const int ntt = wgrad_tiles(K);
+    const WgradForm f = wgrad_form(Ci, kh, kw, stride_w, dil_w);
+    wgrad_shape(N, Ci, Co, Ho, T, kh, kw, f, p);
     const int64_t cobs = (Co + 15) / 16;
-    if (workspace_floats < N * cobs * p.items * p.passes * ntt * 256) return SLAYER_ERANGE;
+    // the waves' tiles, then the chunk sums of the first reduction launch (doubles)
+    const int64_t tile_floats = N * cobs * p.items * p.passes * f.tiles * 256;
+    const int64_t stage_floats = 2 * kWgradChunks * cobs * p.passes * f.tiles * 256;
+    if (workspace_floats < tile_floats + stage_floats) return SLAYER_ERANGE;
+    double* stage = reinterpret_cast<double*>(workspace + tile_floats);
     const int64_t blocks = N * cobs * ((p.items + kSynWaves - 1) / kSynWaves);
     if (blocks > 0x7fffffffLL || p.passes > 65535) return SLAYER_ERANGE;
     const dim3 grid((unsigned)blocks, (unsigned)p.passes), block(kSynWaves * kWave);
-    const dim3 rgrid((unsigned)(cobs * p.passes * ntt));
-#define SLAYER_WGRAD(NTT)                                                                                         \
-    do {                                                                                                          \
-        hipLaunchKernelGGL((synapse_wgrad_kernel<NTT>), grid, block, NTT * 16 * 3 * sizeof(int), st, p);          \
-        hipLaunchKernelGGL((synapse_wgrad_reduce_kernel<NTT>), rgrid, dim3(kWgradParts * kWave), 0, st, grad_weight, workspace,  \
-                           (int)N, (int)Co, (int)K, p.items, p.passes);                                           \
-    } while (0)
-    if (ntt == 1) SLAYER_WGRAD(1); else if (ntt == 2) SLAYER_WGRAD(2); else SLAYER_WGRAD(5);
+#define SLAYER_WGRAD(NTT) hipLaunchKernelGGL((synapse_wgrad_kernel<NTT>), grid, block, NTT * 16 * 3 * sizeof(int), st, p)
+#define SLAYER_WGRAD_ROW(KW, NPT) \
+    hipLaunchKernelGGL((synapse_wgrad_row_kernel<KW, NPT>), grid, block, NPT * 16 * 2 * sizeof(int), st, p)
+    if (f.row_kw == 3) { if (f.npt == 1) SLAYER_WGRAD_ROW(3, 1); else SLAYER_WGRAD_ROW(3, 2); }
+    else if (f.row_kw == 5) { if (f.npt == 1) SLAYER_WGRAD_ROW(5, 1); else SLAYER_WGRAD_ROW(5, 2); }
+    else if (f.tiles == 1) SLAYER_WGRAD(1);
+    else if (f.tiles == 2) SLAYER_WGRAD(2);
+    else SLAYER_WGRAD(5);
+#undef SLAYER_WGRAD_ROW
 #undef SLAYER_WGRAD
+    const unsigned tile_blocks = (unsigned)(cobs * p.passes * f.tiles);
+    hipLaunchKernelGGL(synapse_wgrad_reduce_kernel, dim3(tile_blocks, kWgradChunks), dim3(kWgradParts * kWave), 0, st,
+                       stage, workspace, (int)N, (int)Co, p.items, p.passes, f.tiles);
+    hipLaunchKernelGGL(synapse_wgrad_final_kernel, dim3(tile_blocks), dim3(kWave), 0, st, grad_weight, stage, (int)Co,
+                       (int)K, p.passes, f.tiles, f.row_kw, f.npt);
     return (int)hipGetLastError();
 }

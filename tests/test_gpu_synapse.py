@@ -54,6 +54,9 @@ def _check(slayer, shape, co, kernel, stride, padding, dilation, what, backward=
     ((2, 16, 7, 9, 72), 8, (3, 3), (1, 1), (1, 1), (1, 1)),         # 144 taps: two passes of the weight gradient
     ((3, 1, 9, 8, 132), 4, (3, 3), (1, 1), (1, 1), (1, 1)),         # 9 taps: one tile of taps
     ((1, 20, 5, 5, 1032), 3, (3, 3), (1, 1), (2, 2), (1, 1)),       # 180 taps, long rows: several shares of time
+    ((2, 3, 9, 9, 40), 6, (5, 5), (1, 1), (2, 2), (1, 1)),          # five taps per row, one tile of pairs
+    ((1, 7, 8, 8, 36), 20, (5, 3), (1, 1), (2, 1), (1, 1)),         # 35 pairs: two tiles and a second pass; kw = 3, kh = 5
+    ((1, 7, 8, 8, 36), 20, (3, 5), (1, 1), (1, 2), (1, 1)),         # kw = 5, kh = 3
 ])
 def test_conv_synapse_against_the_oracle(slayer, shape, co, kernel, stride, padding, dilation):
     _check(slayer, shape, co, kernel, stride, padding, dilation, f'{shape} -> {co}')
