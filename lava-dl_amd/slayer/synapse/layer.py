@@ -1,4 +1,4 @@
-"""Convolution synapse on time-innermost tensors.
+"""Synapse layers on time-innermost tensors: the convolution synapse and the dense synapse.
 
 Interface of lava.lib.dl.slayer.synapse.Conv (synapse/layer.py:178-323 in the reference): a spatial convolution
 applied at every time step of an NCHWT tensor.  The reference calls ``F.conv3d`` with a kernel of (kh, kw, 1); the
@@ -117,29 +117,11 @@ def conv_synapse(input, weight, stride=1, padding=0, dilation=1, groups=1):
     return _ConvSynapse.apply(input, weight, stride, padding, dilation)
 
 
-class Conv(torch.nn.Conv3d):
-    """Convolution synapse layer (synapse/layer.py:178-323 in the reference).
+class _SynapseLayer:
+    """What the synapse layers share (GenericLayer, synapse/layer.py:15-69 in the reference): weight
+    normalisation on demand, a pre-hook applied to the weight before every forward pass, ``shape``."""
 
-    Parameters
-    ----------
-    in_features, out_features : int
-    kernel_size, stride, padding, dilation : int or (height, width)
-    groups : int
-    weight_scale : int
-        weight initialization scale factor.
-    weight_norm : bool
-        weight normalization (``torch.nn.utils.weight_norm`` over the output channels, as in the reference).
-    pre_hook_fx : callable or None
-        applied to the weight before every forward pass (typically a quantizer).
-    """
-
-    def __init__(self, in_features, out_features, kernel_size, stride=1, padding=0, dilation=1, groups=1,
-                 weight_scale=1, weight_norm=False, pre_hook_fx=None):
-        kernel = _pair(kernel_size, 'kernel_size')
-        self._stride2, self._padding2, self._dilation2 = _pair(stride, 'stride'), _pair(padding, 'padding'), \
-            _pair(dilation, 'dilation')
-        super().__init__(in_features, out_features, kernel + (1,), self._stride2 + (1,), self._padding2 + (0,),
-                         self._dilation2 + (1,), groups, bias=False)
+    def _finish(self, weight_scale, weight_norm, pre_hook_fx):
         if weight_scale != 1:
             self.weight = torch.nn.Parameter(weight_scale * self.weight)
         self._pre_hook_fx = pre_hook_fx
@@ -164,7 +146,79 @@ class Conv(torch.nn.Conv3d):
     def pre_hook_fx(self, fx):
         self._pre_hook_fx = fx
 
+    @property
+    def shape(self):
+        return self.weight.shape
+
+    def _weight(self):
+        return self.weight if self._pre_hook_fx is None else self._pre_hook_fx(self.weight)
+
+
+class Dense(torch.nn.Conv3d, _SynapseLayer):
+    """Dense synapse layer (synapse/layer.py:72-175 in the reference): every output neuron sums all input
+    neurons of the same time step.  The reference writes it as ``F.conv3d`` with a kernel that covers the whole
+    input; it is a matrix product of the [out, in] weights with the [N, in, T] spikes, and that is what runs
+    here (``torch.matmul``: one batched GEMM whose result is time innermost, which the neuron kernels read in
+    place).
+
+    Parameters
+    ----------
+    in_neurons : int or (width, height) or (width, height, channels)
+    out_neurons : int
+    weight_scale, weight_norm, pre_hook_fx : as for :class:`Conv`.
+    """
+
+    def __init__(self, in_neurons, out_neurons, weight_scale=1, weight_norm=False, pre_hook_fx=None):
+        if type(in_neurons) == int:
+            kernel, in_channels = (1, 1, 1), in_neurons
+        elif len(in_neurons) == 2:
+            kernel, in_channels = (in_neurons[1], in_neurons[0], 1), 1
+        elif len(in_neurons) == 3:
+            kernel, in_channels = (in_neurons[1], in_neurons[0], 1), in_neurons[2]
+        else:
+            raise Exception(f'in_neurons should not be more than 3 dimension. Found {in_neurons=}')
+        if type(out_neurons) != int:
+            raise Exception(f'out_neurons should not be more than 1 dimension. Found {out_neurons=}')
+        super().__init__(in_channels, out_neurons, kernel, bias=False)
+        self._finish(weight_scale, weight_norm, pre_hook_fx)
+
+    def forward(self, input):
+        """Weighted spikes for NCT spikes ([N, out, T]) or NCHWT spikes ([N, out, 1, 1, T] when the image is the
+        size of the kernel, the sliding convolution otherwise)."""
+        weight = self._weight()
+        if input.dim() == 3:
+            return torch.matmul(weight.reshape(weight.shape[0], -1), input)
+        if tuple(input.shape[1:4]) == tuple(weight.shape[1:4]):
+            n, t = input.shape[0], input.shape[-1]
+            return torch.matmul(weight.reshape(weight.shape[0], -1), input.reshape(n, -1, t)).reshape(n, -1, 1, 1, t)
+        return F.conv3d(input, weight, self.bias, self.stride, self.padding, self.dilation, self.groups)
+
+
+class Conv(torch.nn.Conv3d, _SynapseLayer):
+    """Convolution synapse layer (synapse/layer.py:178-323 in the reference).
+
+    Parameters
+    ----------
+    in_features, out_features : int
+    kernel_size, stride, padding, dilation : int or (height, width)
+    groups : int
+    weight_scale : int
+        weight initialization scale factor.
+    weight_norm : bool
+        weight normalization (``torch.nn.utils.weight_norm`` over the output channels, as in the reference).
+    pre_hook_fx : callable or None
+        applied to the weight before every forward pass (typically a quantizer).
+    """
+
+    def __init__(self, in_features, out_features, kernel_size, stride=1, padding=0, dilation=1, groups=1,
+                 weight_scale=1, weight_norm=False, pre_hook_fx=None):
+        kernel = _pair(kernel_size, 'kernel_size')
+        self._stride2, self._padding2, self._dilation2 = _pair(stride, 'stride'), _pair(padding, 'padding'), \
+            _pair(dilation, 'dilation')
+        super().__init__(in_features, out_features, kernel + (1,), self._stride2 + (1,), self._padding2 + (0,),
+                         self._dilation2 + (1,), groups, bias=False)
+        self._finish(weight_scale, weight_norm, pre_hook_fx)
+
     def forward(self, input):
         """Weighted spikes [N, out_features, Ho, Wo, T] for spikes [N, in_features, H, W, T]."""
-        weight = self.weight if self._pre_hook_fx is None else self._pre_hook_fx(self.weight)
-        return conv_synapse(input, weight, self._stride2, self._padding2, self._dilation2, self.groups)
+        return conv_synapse(input, self._weight(), self._stride2, self._padding2, self._dilation2, self.groups)

@@ -142,3 +142,28 @@ def test_sizes_the_step_kernels_refuse(slayer):
         N.ptr(one), N.ptr(one), N.ptr(one), N.ptr(one), 1.0, 0, 1.0, 64, 2, 1028, 1, 1, 1, 1, 4,
         N.ptr(ws), ws.numel(), N.stream_handle())
     assert code == -3
+
+
+@pytest.mark.parametrize('c', [24, 260])
+def test_recurrent_layer_with_the_dense_synapse_module(slayer, c):
+    """The recurrent synapse as the package's own Dense layer (what the reference's Recurrent blocks hold,
+    block/cuba.py:166-176): the kernels (one launch for 24 neurons, a launch per step for 260) and the plain loop
+    that calls the synapse module step by step give the same spikes and weight gradients."""
+    R = slayer.utils.recurrent
+    gen = torch.Generator().manual_seed(c)
+    n, t = 3, 40
+    z = (torch.randn(n, c, t, generator=gen) * 1.5).to(dev())
+    g = torch.rand(n, c, t, generator=gen).to(dev())
+    results = []
+    for loop in (False, True):
+        neuron = base._neuron(slayer)
+        syn = slayer.synapse.Dense(c, c, pre_hook_fx=neuron.quantize_8bit).to(dev())
+        with torch.no_grad():
+            syn.weight.copy_((torch.randn(c, c, generator=torch.Generator().manual_seed(5)) * 3.0 / c ** 0.5)
+                             .reshape(syn.weight.shape))
+        out = R.custom_recurrent_ground_truth_1(z, neuron, syn) if loop else R.custom_recurrent(z, neuron, syn)
+        out.backward(g)
+        results.append((out.detach(), syn.weight.grad))
+    assert 0.01 < float(results[0][0].mean()) < 0.9
+    assert torch.equal(results[0][0], results[1][0]), 'spikes'
+    assert results[0][1].shape == results[1][1].shape == (c, c, 1, 1, 1)
