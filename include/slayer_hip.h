@@ -314,8 +314,9 @@ int slayer_corr(float *out, const float *in, const float *filt, int64_t K, float
  * (zero outside the image), Ho = (H + 2 pad_h - dil_h (kh - 1) - 1) / stride_h + 1, Wo likewise; weight is
  * [Co][Ci][kh][kw] (the reference's [Co][Ci][kh][kw][1]).  float32 operands and accumulation on the matrix cores.
  * The gradient of the input is the same call on the gradient with the weights transposed and flipped.
- * SLAYER_ERANGE for what the kernel does not take (T not a multiple of 4, tensors not 16-byte aligned, a batch entry of
- * 2 GiB or more, more than about 860 taps Ci * kh * kw): the caller keeps its library convolution for those. */
+ * Rows of any length from four steps on, float-aligned tensors.  SLAYER_ERANGE for what the kernel does not take
+ * (T < 4, a batch entry of 2 GiB or more, more than about 860 taps Ci * kh * kw): the caller keeps its library
+ * convolution for those. */
 int slayer_conv_synapse(float *out, const float *in, const float *weight,
                         int64_t N, int64_t Ci, int64_t Co, int64_t H, int64_t W, int64_t T,
                         int64_t kh, int64_t kw, int64_t stride_h, int64_t stride_w,

@@ -22,6 +22,46 @@ int launch_zero_fill(float* p, int64_t n, hipStream_t stream);          // li.hi
 
 typedef float syn_f4 __attribute__((ext_vector_type(4)));
 
+// Rows of any length (T >= 4): a quad of steps is a 16-byte access at a dword-aligned address, and the last quad of
+// a row may hold fewer than four steps (nv of them).  Such a quad is loaded four steps before the end of its row --
+// never beyond it -- and moved into place: element e of the result is element e + 4 - nv of what was loaded, zero
+// behind the row's end.  Stores leave the steps that do not exist out.
+struct SynQuad {
+    int t_load;                         // step the quad is loaded at
+    int nv;                             // steps of the quad that exist (<= 0: none, the lane loads nothing)
+    template <bool TAIL>
+    __device__ __forceinline__ void set(int t, int t_end) {
+        nv = t_end - t;
+        t_load = (TAIL && nv > 0 && nv < 4) ? t_end - 4 : t;
+    }
+    __device__ __forceinline__ bool any() const { return nv > 0; }
+    __device__ __forceinline__ bool partial() const { return nv > 0 && nv < 4; }
+    // TAIL: the rows are not whole quads (decided on the host: a test per load would sit between the loads)
+    template <bool TAIL>
+    __device__ __forceinline__ float4 place(float4 q) const {
+        if (!TAIL || !__any(partial())) return q;                        // only the tile that holds the end of the rows
+        const int d = partial() ? 4 - nv : 0;
+        const float a[4] = {q.x, q.y, q.z, q.w};
+        float r[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int i = e + d;
+            r[e] = i == 0 ? a[0] : (i == 1 ? a[1] : (i == 2 ? a[2] : (i == 3 ? a[3] : 0.f)));
+        }
+        return make_float4(r[0], r[1], r[2], r[3]);
+    }
+};
+// the quad v at byte offset off, of which the first nv elements exist (nv <= 0: nothing is stored)
+template <bool STREAM, bool TAIL>
+__device__ __forceinline__ void syn_store_quad(__amdgpu_buffer_rsrc_t dst, bool on, int off, int nv, float4 v) {
+    buf_store4<STREAM>(dst, (on && nv >= 4) ? off : kOutOfRange, v);
+    if (TAIL && __any(on && nv > 0 && nv < 4)) {                                 // only the tile that holds the end of the rows
+        const float e[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 3; ++i) buf_store1<false>(dst, (on && nv < 4 && i < nv) ? off + 4 * i : kOutOfRange, e[i]);
+    }
+}
+
 constexpr int kSynTile = 64;            // time steps per tile
 constexpr int kSynWaves = 4;            // waves per workgroup: same output channels, same image row, different tiles
 
@@ -42,7 +82,7 @@ struct SynapseConv {
 // offset of its input row relative to the pixel's own position and its (row, column) displacement in the image.
 // A workgroup's four waves take four consecutive items of one (batch entry, channel block): an item is one tile
 // of 64 steps of a piece of one output row.
-template <bool STREAM>
+template <bool STREAM, bool TAIL>
 __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_kernel(const SynapseConv p) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int Kp = p.KG * 4;
@@ -81,7 +121,10 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_kernel(const S
     const int ho = item / (p.ttiles * p.wsplit);
     const int t0 = tile * kSynTile;
     const int kk = lane >> 4, j = lane & 15;
-    const bool t_ok = t0 + 4 * j < p.T;                                  // T is a whole number of quads
+    SynQuad tq;
+    tq.template set<TAIL>(t0 + 4 * j, p.T);
+    const int nv = tq.nv;
+    const bool t_ok = tq.any();
     const int hin = ho * p.sh;                                           // image row of tap (0, 0) before padding
     const int64_t in_plane = (int64_t)p.Ci * p.H * p.W * p.T;
     const __amdgpu_buffer_rsrc_t src = make_rsrc(p.in + (int64_t)n * in_plane, (unsigned)(in_plane * 4));
@@ -92,7 +135,7 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_kernel(const S
     const int w_lo = piece * per, w_hi = (w_lo + per) < p.Wo ? (w_lo + per) : p.Wo;
     for (int wo = w_lo; wo < w_hi; ++wo) {
         const int win = wo * p.sw;
-        const int pix = ((hin * p.W) + win) * p.T * 4 + (t0 + 4 * j) * 4;    // byte offset of tap (0,0,0)'s quad
+        const int pix = ((hin * p.W) + win) * p.T * 4 + tq.t_load * 4;       // byte offset of tap (0,0,0)'s quad
         syn_f4 acc[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc[e] = syn_f4{0.f, 0.f, 0.f, 0.f};
@@ -104,7 +147,7 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_kernel(const S
                 const int k = 4 * (g0 + u) + kk;
                 const int yy = hin + tap_dy[k], xx = win + tap_dx[k];
                 const bool ok = t_ok && (unsigned)yy < (unsigned)p.H && (unsigned)xx < (unsigned)p.W;
-                q[u] = buf_load4<false>(src, ok ? pix + tap_off[k] : kOutOfRange);
+                q[u] = tq.template place<TAIL>(buf_load4<false>(src, ok ? pix + tap_off[k] : kOutOfRange));
                 a[u] = wt[k * 16 + j];
             }
 #pragma unroll
@@ -120,9 +163,8 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_kernel(const S
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int co = co0 + 4 * kk + i;
-            const bool ok = t_ok && co < p.Co;
-            buf_store4<STREAM>(dst, ok ? co * (p.Ho * p.Wo * p.T * 4) + opix : kOutOfRange,
-                               make_float4(acc[0][i], acc[1][i], acc[2][i], acc[3][i]));
+            syn_store_quad<STREAM, TAIL>(dst, co < p.Co, co * (p.Ho * p.Wo * p.T * 4) + opix, nv,
+                                   make_float4(acc[0][i], acc[1][i], acc[2][i], acc[3][i]));
         }
     }
 }
@@ -134,7 +176,7 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_kernel(const S
 // (18 KB per pixel and tile of 64 steps), not by the matrix cores.
 // LDS: weights as above (tap k = pair * KW + x, pair = ci * kh + y), and per pair the byte offset of its input row
 // relative to the pixel block's own position and its row displacement.
-template <int KW, int PIX, bool STREAM>
+template <int KW, int PIX, bool STREAM, bool TAIL>
 __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_row_kernel(const SynapseConv p) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int PG = p.KG;                                // groups of four pairs
@@ -171,7 +213,10 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_row_kernel(con
     const int ho = item / (p.ttiles * p.wsplit);
     const int t0 = tile * kSynTile;
     const int kk = lane >> 4, j = lane & 15;
-    const bool t_ok = t0 + 4 * j < p.T;                                  // T is a whole number of quads
+    SynQuad tq;
+    tq.template set<TAIL>(t0 + 4 * j, p.T);
+    const int nv = tq.nv;
+    const bool t_ok = tq.any();
     const int hin = ho * p.sh;
     const int64_t in_plane = (int64_t)p.Ci * p.H * p.W * p.T;
     const __amdgpu_buffer_rsrc_t src = make_rsrc(p.in + (int64_t)n * in_plane, (unsigned)(in_plane * 4));
@@ -182,7 +227,7 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_row_kernel(con
     const int per = ((p.Wo + p.wsplit - 1) / p.wsplit + PIX - 1) / PIX * PIX;
     const int w_lo = piece * per, w_hi = (w_lo + per) < p.Wo ? (w_lo + per) : p.Wo;
     for (int wo0 = w_lo; wo0 < w_hi; wo0 += PIX) {
-        const int pix = ((hin * p.W) + wo0) * col + (t0 + 4 * j) * 4;
+        const int pix = ((hin * p.W) + wo0) * col + tq.t_load * 4;
         syn_f4 acc[PIX][4];
 #pragma unroll
         for (int i = 0; i < PIX; ++i)
@@ -197,7 +242,7 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_row_kernel(con
 #pragma unroll
             for (int c = 0; c < PIX + KW - 1; ++c) {
                 const bool ok = row_ok && (unsigned)(wo0 + c - p.pw) < (unsigned)p.W;
-                q[c] = buf_load4<false>(src, ok ? base + c * col : kOutOfRange);
+                q[c] = tq.template place<TAIL>(buf_load4<false>(src, ok ? base + c * col : kOutOfRange));
             }
             float a[KW];
 #pragma unroll
@@ -220,9 +265,8 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_row_kernel(con
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int co = co0 + 4 * kk + i;
-                const bool ok = t_ok && co < p.Co && wo0 + px < w_hi;
-                buf_store4<STREAM>(dst, ok ? co * (p.Ho * p.Wo * col) + opix : kOutOfRange,
-                                   make_float4(acc[px][0][i], acc[px][1][i], acc[px][2][i], acc[px][3][i]));
+                syn_store_quad<STREAM, TAIL>(dst, co < p.Co && wo0 + px < w_hi, co * (p.Ho * p.Wo * col) + opix, nv,
+                                       make_float4(acc[px][0][i], acc[px][1][i], acc[px][2][i], acc[px][3][i]));
             }
         }
     }
@@ -247,7 +291,7 @@ struct SynapseWgrad {
     int items;                          // (share of time, output row) pairs of one (batch entry, channel block)
 };
 
-template <int NTT>
+template <int NTT, bool TAIL>
 __global__ __launch_bounds__(kSynWaves * kWave) void synapse_wgrad_kernel(const SynapseWgrad p) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     constexpr int Kp = NTT * 16;
@@ -312,12 +356,14 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_wgrad_kernel(const 
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 const int t = t0 + 16 * u + 4 * kk;
-                const bool t_ok = t < t_hi;                              // T and the shares are whole quads
-                g[u] = buf_load4<false>(grd, (t_ok && co_ok) ? g_row + wo * col + t * 4 : kOutOfRange);
+                SynQuad tq;                                              // the shares are whole quads; a row's last quad may not be
+                tq.template set<TAIL>(t, t_hi);
+                const bool t_ok = tq.any();
+                g[u] = tq.template place<TAIL>(buf_load4<false>(grd, (t_ok && co_ok) ? g_row + wo * col + tq.t_load * 4 : kOutOfRange));
 #pragma unroll
                 for (int tt = 0; tt < NTT; ++tt) {
                     const bool ok = t_ok && my_row[tt] && (unsigned)(win + my_dx[tt]) < (unsigned)p.W;
-                    q[u][tt] = buf_load4<false>(src, ok ? pix + my_off[tt] + t * 4 : kOutOfRange);
+                    q[u][tt] = tq.template place<TAIL>(buf_load4<false>(src, ok ? pix + my_off[tt] + tq.t_load * 4 : kOutOfRange));
                 }
             }
 #pragma unroll
@@ -354,7 +400,7 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_wgrad_kernel(const 
 #endif
 constexpr int kWgU = SLAYER_WGRAD_GROUPS;      // groups of 16 steps per visit of a column
 
-template <int KW, int NPT>
+template <int KW, int NPT, bool TAIL>
 __global__ __launch_bounds__(kSynWaves * kWave) void synapse_wgrad_row_kernel(const SynapseWgrad p) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     constexpr int Pp = NPT * 16;
@@ -412,15 +458,17 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_wgrad_row_kernel(co
     for (int t0 = t_lo; t0 < t_hi; t0 += 16 * kWgU) {                    // whole 128-byte lines of every row per visit
         int toff[kWgU];
         bool t_ok[kWgU];
+        SynQuad tq[kWgU];
 #pragma unroll
         for (int u = 0; u < kWgU; ++u) {
             const int t = t0 + 16 * u + 4 * kk;
-            t_ok[u] = t < t_hi;                                          // T and the shares are whole quads
-            toff[u] = t * 4;
+            tq[u].template set<TAIL>(t, t_hi);                                          // the shares are whole quads; a row's last quad may not be
+            t_ok[u] = tq[u].any();
+            toff[u] = tq[u].t_load * 4;
         }
         auto grad_at = [&](int wo, int u) {
-            return buf_load4<false>(grd, (t_ok[u] && co_ok && (unsigned)wo < (unsigned)p.Wo) ? g_row + wo * col + toff[u]
-                                                                                             : kOutOfRange);
+            return tq[u].template place<TAIL>(buf_load4<false>(
+                grd, (t_ok[u] && co_ok && (unsigned)wo < (unsigned)p.Wo) ? g_row + wo * col + toff[u] : kOutOfRange));
         };
         // gw[x][u]: the gradient at pixel c + pw - x for the column c at hand; gw[0] arrives with the column
         float4 gw[KW][kWgU];
@@ -435,7 +483,8 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_wgrad_row_kernel(co
                 gw[0][u] = grad_at(c + p.pw, u);
 #pragma unroll
                 for (int pt = 0; pt < NPT; ++pt)
-                    q[u][pt] = buf_load4<false>(src, (t_ok[u] && my_row[pt]) ? my_off[pt] + c * col + toff[u] : kOutOfRange);
+                    q[u][pt] = tq[u].template place<TAIL>(buf_load4<false>(
+                        src, (t_ok[u] && my_row[pt]) ? my_off[pt] + c * col + toff[u] : kOutOfRange));
             }
 #pragma unroll
             for (int u = 0; u < kWgU; ++u) {
@@ -566,8 +615,9 @@ extern "C" int slayer_conv_synapse(float* out, const float* in, const float* wei
     if (Ho < 1 || Wo < 1) return SLAYER_EINVAL;
     if (N == 0 || T == 0) return 0;
     if (!out || !in || !weight) return SLAYER_ENULL;
-    // whole quads of time steps at 16-byte addresses, 32-bit byte offsets inside one batch entry
-    if ((T % 4) != 0 || !aligned16(out) || !aligned16(in)) return SLAYER_ERANGE;
+    // 32-bit byte offsets inside one batch entry; rows of any length from four steps on (16-byte accesses at
+    // dword-aligned addresses)
+    if (T < 4) return SLAYER_ERANGE;
     const int64_t K = Ci * kh * kw, lim = (int64_t)1 << 31;
     if (Ci * H * W * T * 4 >= lim || Co * Ho * Wo * T * 4 >= lim || K > 4096 || pad_h > 4096 || pad_w > 4096 ||
         H * stride_h > (1 << 20) || W * stride_w > (1 << 20))
@@ -597,28 +647,34 @@ extern "C" int slayer_conv_synapse(float* out, const float* in, const float* wei
     const int64_t blocks = N * ((Co + 15) / 16) * ((items + kSynWaves - 1) / kSynWaves);
     if (blocks > 0x7fffffffLL) return SLAYER_ERANGE;
     const bool streaming = N * Co * Ho * Wo * T * 4 > ((int64_t)64 << 20);
+    const bool tail = (T % 4) != 0;                                       // rows that end inside a quad
     const dim3 grid((unsigned)blocks), block(kSynWaves * kWave);
     hipStream_t st = (hipStream_t)stream;
     if (rows) {
         p.KG = (int)((Ci * kh + 3) / 4);                                  // groups of four (channel, kernel row) pairs
         const size_t lds = (size_t)p.KG * 4 * (kw * 16 * sizeof(float) + 2 * sizeof(int));
         if (lds > 64 * 1024) return SLAYER_ERANGE;
-#define SLAYER_SYN_ROW(KW)                                                                                          \
-        do {                                                                                                        \
-            if (streaming) hipLaunchKernelGGL((synapse_conv_row_kernel<KW, kRowPix, true>), grid, block, lds, st, p); \
-            else hipLaunchKernelGGL((synapse_conv_row_kernel<KW, kRowPix, false>), grid, block, lds, st, p);         \
+#define SLAYER_SYN_ROW_T(KW, TL)                                                                                         \
+        do {                                                                                                            \
+            if (streaming) hipLaunchKernelGGL((synapse_conv_row_kernel<KW, kRowPix, true, TL>), grid, block, lds, st, p); \
+            else hipLaunchKernelGGL((synapse_conv_row_kernel<KW, kRowPix, false, TL>), grid, block, lds, st, p);         \
         } while (0)
+#define SLAYER_SYN_ROW(KW) do { if (tail) SLAYER_SYN_ROW_T(KW, true); else SLAYER_SYN_ROW_T(KW, false); } while (0)
         if (kw == 3) SLAYER_SYN_ROW(3); else SLAYER_SYN_ROW(5);
+#undef SLAYER_SYN_ROW_T
 #undef SLAYER_SYN_ROW
         return (int)hipGetLastError();
     }
     p.KG = (int)(((K + 3) / 4 + kSynChunk - 1) / kSynChunk * kSynChunk);
     const size_t lds = (size_t)p.KG * 4 * (16 * sizeof(float) + 3 * sizeof(int));
     if (lds > 64 * 1024) return SLAYER_ERANGE;
-    if (streaming)
-        hipLaunchKernelGGL((synapse_conv_kernel<true>), grid, block, lds, st, p);
-    else
-        hipLaunchKernelGGL((synapse_conv_kernel<false>), grid, block, lds, st, p);
+    if (streaming) {
+        if (tail) hipLaunchKernelGGL((synapse_conv_kernel<true, true>), grid, block, lds, st, p);
+        else hipLaunchKernelGGL((synapse_conv_kernel<true, false>), grid, block, lds, st, p);
+    } else {
+        if (tail) hipLaunchKernelGGL((synapse_conv_kernel<false, true>), grid, block, lds, st, p);
+        else hipLaunchKernelGGL((synapse_conv_kernel<false, false>), grid, block, lds, st, p);
+    }
     return (int)hipGetLastError();
 }
 
@@ -702,7 +758,7 @@ extern "C" int slayer_conv_synapse_wgrad(float* grad_weight, const float* grad_o
     hipStream_t st = (hipStream_t)stream;
     if (N == 0 || T == 0) return launch_zero_fill(grad_weight, Co * K, st);
     if (!grad_out || !in || !workspace) return SLAYER_ENULL;
-    if ((T % 4) != 0 || !aligned16(grad_out) || !aligned16(in) || !aligned16(workspace)) return SLAYER_ERANGE;
+    if (T < 4 || !aligned16(workspace)) return SLAYER_ERANGE;
     if (Ci * H * W * T * 4 >= lim || Co * Ho * Wo * T * 4 >= lim || K > 4096 || pad_h > 4096 || pad_w > 4096 ||
         H * stride_h > (1 << 20) || W * stride_w > (1 << 20) || Ho > (1 << 20) || T > (1 << 24))
         return SLAYER_ERANGE;
@@ -723,9 +779,17 @@ extern "C" int slayer_conv_synapse_wgrad(float* grad_weight, const float* grad_o
     const int64_t blocks = N * cobs * ((p.items + kSynWaves - 1) / kSynWaves);
     if (blocks > 0x7fffffffLL || p.passes > 65535) return SLAYER_ERANGE;
     const dim3 grid((unsigned)blocks, (unsigned)p.passes), block(kSynWaves * kWave);
-#define SLAYER_WGRAD(NTT) hipLaunchKernelGGL((synapse_wgrad_kernel<NTT>), grid, block, NTT * 16 * 3 * sizeof(int), st, p)
-#define SLAYER_WGRAD_ROW(KW, NPT) \
-    hipLaunchKernelGGL((synapse_wgrad_row_kernel<KW, NPT>), grid, block, NPT * 16 * 2 * sizeof(int), st, p)
+    const bool tail = (T % 4) != 0;                                       // rows that end inside a quad
+#define SLAYER_WGRAD(NTT)                                                                                              \
+    do {                                                                                                               \
+        if (tail) hipLaunchKernelGGL((synapse_wgrad_kernel<NTT, true>), grid, block, NTT * 16 * 3 * sizeof(int), st, p); \
+        else hipLaunchKernelGGL((synapse_wgrad_kernel<NTT, false>), grid, block, NTT * 16 * 3 * sizeof(int), st, p);    \
+    } while (0)
+#define SLAYER_WGRAD_ROW(KW, NPT)                                                                                      \
+    do {                                                                                                               \
+        if (tail) hipLaunchKernelGGL((synapse_wgrad_row_kernel<KW, NPT, true>), grid, block, NPT * 16 * 2 * sizeof(int), st, p); \
+        else hipLaunchKernelGGL((synapse_wgrad_row_kernel<KW, NPT, false>), grid, block, NPT * 16 * 2 * sizeof(int), st, p);    \
+    } while (0)
     if (f.row_kw == 3) { if (f.npt == 1) SLAYER_WGRAD_ROW(3, 1); else SLAYER_WGRAD_ROW(3, 2); }
     else if (f.row_kw == 5) { if (f.npt == 1) SLAYER_WGRAD_ROW(5, 1); else SLAYER_WGRAD_ROW(5, 2); }
     else if (f.tiles == 1) SLAYER_WGRAD(1);

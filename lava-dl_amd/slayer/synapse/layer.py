@@ -5,8 +5,8 @@ applied at every time step of an NCHWT tensor.  The reference calls ``F.conv3d``
 library behind it wants channels last and transposes the tensor there and back around its kernel.  Here
 slayer_conv_synapse of libslayer_hip.so computes it where the tensor lies, so the neuron that follows reads the
 result in place; the input gradient is the same kernel on the flipped, transposed weights and the weight gradient
-slayer_conv_synapse_wgrad.  What the kernels do not take (grouped convolutions, rows that are not whole quads of
-time steps) goes to ``F.conv3d`` and its gradients as before.
+slayer_conv_synapse_wgrad.  What the kernels do not take (grouped convolutions, fewer than four time steps, more than
+about 860 taps) goes to ``F.conv3d`` and its gradients as before.
 """
 import torch
 import torch.nn.functional as F
@@ -103,15 +103,14 @@ def _weight_gradient(input, weight_shape, grad_output, stride, padding, dilation
 def conv_synapse(input, weight, stride=1, padding=0, dilation=1, groups=1):
     """``F.conv3d(input, weight, None, stride + (1,), padding + (0,), dilation + (1,), groups)`` for an NCHWT
     ``input`` and a ``weight`` of [Co, Ci / groups, kh, kw, 1], computed in place of the layout when the kernel
-    takes the shape (one group, float32 on the GPU, T a multiple of 4), by the library call otherwise."""
+    takes the shape (one group, float32 on the GPU, at least four time steps), by the library call otherwise."""
     stride, padding, dilation = _pair(stride, 'stride'), _pair(padding, 'padding'), _pair(dilation, 'dilation')
     takes = (groups == 1 and input.is_cuda and input.dtype == torch.float32 and weight.dtype == torch.float32
-             and input.dim() == 5 and weight.dim() == 5 and weight.shape[-1] == 1 and input.shape[-1] % 4 == 0
+             and input.dim() == 5 and weight.dim() == 5 and weight.shape[-1] == 1 and input.shape[-1] >= 4
              and input.shape[1] * weight.shape[2] * weight.shape[3] <= 860 and input.numel() > 0
              and input[0].numel() * 4 < 2 ** 31)
     if takes:
         input = input.contiguous()
-        takes = input.data_ptr() % 16 == 0
     if not takes:
         return F.conv3d(input, weight, None, stride + (1,), padding + (0,), dilation + (1,), groups)
     return _ConvSynapse.apply(input, weight, stride, padding, dilation)

@@ -55,6 +55,12 @@ def _check(slayer, shape, co, kernel, stride, padding, dilation, what, backward=
     ((3, 1, 9, 8, 132), 4, (3, 3), (1, 1), (1, 1), (1, 1)),         # 9 taps: one tile of taps
     ((1, 20, 5, 5, 1032), 3, (3, 3), (1, 1), (2, 2), (1, 1)),       # 180 taps, long rows: several shares of time
     ((2, 3, 9, 9, 40), 6, (5, 5), (1, 1), (2, 2), (1, 1)),          # five taps per row, one tile of pairs
+    # rows that are not whole quads of steps (T % 4 = 1, 2, 3), whole tiles of 64 steps and a few steps more
+    ((2, 8, 9, 9, 65), 16, (3, 3), (1, 1), (1, 1), (1, 1)),
+    ((1, 3, 6, 7, 350), 5, (3, 3), (1, 1), (1, 1), (1, 1)),
+    ((2, 4, 5, 6, 131), 20, (3, 3), (2, 1), (1, 1), (1, 1)),
+    ((1, 2, 12, 10, 7), 3, (5, 5), (2, 2), (2, 2), (1, 1)),
+    ((3, 5, 4, 4, 4), 2, (1, 1), (1, 1), (0, 0), (1, 1)),
     ((1, 7, 8, 8, 36), 20, (5, 3), (1, 1), (2, 1), (1, 1)),         # 35 pairs: two tiles and a second pass; kw = 3, kh = 5
     ((1, 7, 8, 8, 36), 20, (3, 5), (1, 1), (1, 2), (1, 1)),         # kw = 5, kh = 3
 ])
@@ -78,7 +84,7 @@ def test_conv_module_mirrors_the_reference_layer(slayer):
 
 def test_shapes_the_kernel_does_not_take_go_to_the_library_call(slayer):
     gen = torch.Generator().manual_seed(4)
-    x = torch.randn(2, 4, 6, 6, 10, generator=gen).to(dev())                 # T % 4 != 0
+    x = torch.randn(2, 4, 6, 6, 3, generator=gen).to(dev())                  # fewer than four steps
     w = torch.randn(6, 4, 3, 3, 1, generator=gen).to(dev())
     assert torch.equal(slayer.synapse.conv_synapse(x, w, 1, 1, 1), F.conv3d(x, w, None, (1, 1, 1), (1, 1, 0)))
     w2 = torch.randn(6, 2, 3, 3, 1, generator=gen).to(dev())                 # two groups
@@ -132,3 +138,30 @@ def test_weight_gradient_at_the_size_of_the_benchmark_tensor(slayer):
                 want[:, :, y, xx] += gf @ v.t()
                 mag[:, :, y, xx] += gf.abs() @ v.t()
     assert_sum(w.grad[..., 0], want, mag, 'grad weight at [32,8,32,32,300]')
+
+
+def test_tensors_at_dword_aligned_addresses(slayer):
+    """Input and gradient that start one float into their allocations (contiguous views): same results as the
+    aligned copies, bit for bit."""
+    gen = torch.Generator().manual_seed(21)
+    shape, co = (2, 4, 6, 7, 70), 6
+    x = (torch.rand(shape, generator=gen) < 0.3).float() * torch.randn(shape, generator=gen)
+    w = torch.randn(co, 4, 3, 3, 1, generator=gen).to(dev())
+    g = torch.randn((2, co, 6, 7, 70), generator=gen)
+
+    def off_by_one(t):
+        buf = torch.empty(t.numel() + 1, device=dev())
+        view = buf[1:].view(t.shape)
+        view.copy_(t)
+        assert view.data_ptr() % 16 == 4 and view.is_contiguous()
+        return view
+
+    results = []
+    for shifted in (False, True):
+        xs = (off_by_one(x) if shifted else x.to(dev())).requires_grad_()
+        ws = w.clone().requires_grad_()
+        y = slayer.synapse.conv_synapse(xs, ws, 1, 1, 1)
+        y.backward(off_by_one(g) if shifted else g.to(dev()))
+        results.append((y.detach(), xs.grad, ws.grad))
+    for a, b, what in zip(results[0], results[1], ('forward', 'grad input', 'grad weight')):
+        assert torch.equal(a, b), what
