@@ -322,6 +322,19 @@ int slayer_conv_synapse(float *out, const float *in, const float *weight,
                         int64_t kh, int64_t kw, int64_t stride_h, int64_t stride_w,
                         int64_t pad_h, int64_t pad_w, int64_t dil_h, int64_t dil_w, void *stream);
 
+/* The gradient of the synapse's input for any stride (what autograd obtains from conv3d's backward, and what the
+ * transposed convolution of synapse/layer.py:513-560 computes as a layer of its own):
+ * grad_in[n][ci][h][w][t] = sum over co, y, x of weight_t[ci][co][y][x] *
+ *                           grad_out[n][co][(h + pad_h - y * dil_h) / stride_h][(w + pad_w - x * dil_w) / stride_w][t]
+ * over the taps whose two quotients are exact and lie inside grad_out's [Ho][Wo].  N, Ci, Co, H, W, kh ... dil_w are
+ * those of the forward call; weight_t is [Ci][Co][kh][kw] (the forward weights with the channel axes exchanged,
+ * not flipped).  With unit strides slayer_conv_synapse on the flipped weights is the faster call.  SLAYER_ERANGE
+ * as for slayer_conv_synapse, and for strides above 16 or images beyond 65535 pixels a side. */
+int slayer_conv_synapse_input_grad(float *grad_in, const float *grad_out, const float *weight_t,
+                                   int64_t N, int64_t Ci, int64_t Co, int64_t H, int64_t W, int64_t T,
+                                   int64_t kh, int64_t kw, int64_t stride_h, int64_t stride_w,
+                                   int64_t pad_h, int64_t pad_w, int64_t dil_h, int64_t dil_w, void *stream);
+
 /* The gradient of the synapse's weights (what autograd obtains from conv3d's backward, synapse/layer.py:297-323):
  * grad_weight[co][ci][y][x] = sum over n, ho, wo, t of grad_out[n][co][ho][wo][t] *
  *                             in[n][ci][ho * stride_h + y * dil_h - pad_h][wo * stride_w + x * dil_w - pad_w][t],

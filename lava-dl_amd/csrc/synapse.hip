@@ -65,7 +65,7 @@ __device__ __forceinline__ void syn_store_quad(__amdgpu_buffer_rsrc_t dst, bool 
 constexpr int kSynTile = 64;            // time steps per tile
 constexpr int kSynWaves = 4;            // waves per workgroup: same output channels, same image row, different tiles
 
-constexpr int kSynChunk = 6;            // tap groups whose loads are in flight together
+constexpr int kSynChunk = 6;            // tap groups whose loads are in flight together (fewer for filters of a few taps)
 
 struct SynapseConv {
     float* out;
@@ -76,13 +76,21 @@ struct SynapseConv {
     int K, KG;                          // taps, groups of four taps (a whole number of chunks, padded with null taps)
     int ttiles, wsplit;                 // tiles of 64 steps per row, pieces an image row is cut into
     int items;                          // (tile, piece, output row) triples of one (batch entry, channel block)
+    float inv_sh, inv_sw;               // TRANSPOSED: 1 / stride
 };
 
+// TRANSPOSED: the gradient of the input of a convolution of any stride (what conv_transpose3d computes, the
+// ConvTranspose synapse of synapse/layer.py:513-560 in the reference): `in` is the gradient of the convolution's
+// output, [N][Ci][H][W][T] in this structure's names, `out` the gradient of its input, [N][Co][Ho][Wo][T], `weight`
+// [Co][Ci][kh][kw] (the convolution's weights with the two channel axes exchanged), and tap (ci, y, x) of output
+// pixel (ho, wo) reads source pixel ((ho + ph - y dh) / sh, (wo + pw - x dw) / sw) where both divisions are exact
+// and the result lies in the source image -- one tap in sh * sw on average.
+//
 // LDS: the weights of this workgroup's 16 output channels, tap-major (row k holds the 16 channels), and per tap the
 // offset of its input row relative to the pixel's own position and its (row, column) displacement in the image.
 // A workgroup's four waves take four consecutive items of one (batch entry, channel block): an item is one tile
 // of 64 steps of a piece of one output row.
-template <bool STREAM, bool TAIL>
+template <bool STREAM, bool TAIL, bool TRANSPOSED, int CHUNK>
 __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_kernel(const SynapseConv p) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int Kp = p.KG * 4;
@@ -107,10 +115,11 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_kernel(const S
     }
     for (int k = tid; k < Kp; k += kSynWaves * kWave) {
         const int ci = k / (p.kh * p.kw), r = k - ci * (p.kh * p.kw), y = r / p.kw, x = r - y * p.kw;
-        const int dy = y * p.dh - p.ph, dx = x * p.dw - p.pw;
-        tap_dy[k] = k < p.K ? dy : (1 << 28);                            // a tap that does not exist: always outside
+        const int dy = TRANSPOSED ? p.ph - y * p.dh : y * p.dh - p.ph;
+        const int dx = TRANSPOSED ? p.pw - x * p.dw : x * p.dw - p.pw;
+        tap_dy[k] = k < p.K ? dy : (TRANSPOSED ? -(1 << 28) : (1 << 28));   // a tap that does not exist: always outside
         tap_dx[k] = dx;
-        tap_off[k] = (((ci * p.H + dy) * p.W) + dx) * p.T * 4;
+        tap_off[k] = TRANSPOSED ? ci * p.H * p.W * p.T * 4 : (((ci * p.H + dy) * p.W) + dx) * p.T * 4;
     }
     __syncthreads();
 
@@ -125,7 +134,7 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_kernel(const S
     tq.template set<TAIL>(t0 + 4 * j, p.T);
     const int nv = tq.nv;
     const bool t_ok = tq.any();
-    const int hin = ho * p.sh;                                           // image row of tap (0, 0) before padding
+    const int hin = TRANSPOSED ? ho : ho * p.sh;                         // image row of tap (0, 0) before padding
     const int64_t in_plane = (int64_t)p.Ci * p.H * p.W * p.T;
     const __amdgpu_buffer_rsrc_t src = make_rsrc(p.in + (int64_t)n * in_plane, (unsigned)(in_plane * 4));
     const int64_t out_plane = (int64_t)p.Co * p.Ho * p.Wo * p.T;
@@ -134,24 +143,34 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_kernel(const S
     const int per = (p.Wo + p.wsplit - 1) / p.wsplit;
     const int w_lo = piece * per, w_hi = (w_lo + per) < p.Wo ? (w_lo + per) : p.Wo;
     for (int wo = w_lo; wo < w_hi; ++wo) {
-        const int win = wo * p.sw;
-        const int pix = ((hin * p.W) + win) * p.T * 4 + tq.t_load * 4;       // byte offset of tap (0,0,0)'s quad
+        const int win = TRANSPOSED ? wo : wo * p.sw;
+        // byte offset of tap (0,0,0)'s quad (TRANSPOSED: of the quad inside a row of the source)
+        const int pix = TRANSPOSED ? tq.t_load * 4 : ((hin * p.W) + win) * p.T * 4 + tq.t_load * 4;
         syn_f4 acc[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc[e] = syn_f4{0.f, 0.f, 0.f, 0.f};
-        for (int g0 = 0; g0 < p.KG; g0 += kSynChunk) {
-            float4 q[kSynChunk];
-            float a[kSynChunk];
+        for (int g0 = 0; g0 < p.KG; g0 += CHUNK) {
+            float4 q[CHUNK];
+            float a[CHUNK];
 #pragma unroll
-            for (int u = 0; u < kSynChunk; ++u) {
+            for (int u = 0; u < CHUNK; ++u) {
                 const int k = 4 * (g0 + u) + kk;
                 const int yy = hin + tap_dy[k], xx = win + tap_dx[k];
-                const bool ok = t_ok && (unsigned)yy < (unsigned)p.H && (unsigned)xx < (unsigned)p.W;
-                q[u] = tq.template place<TAIL>(buf_load4<false>(src, ok ? pix + tap_off[k] : kOutOfRange));
+                bool ok;
+                int off = pix + tap_off[k];
+                if (TRANSPOSED) {
+                    // exact quotients of small non-negative integers by way of float (coordinates below 2^16)
+                    const int yq = (int)(((float)yy + 0.5f) * p.inv_sh), xq = (int)(((float)xx + 0.5f) * p.inv_sw);
+                    ok = t_ok && yy >= 0 && xx >= 0 && yq * p.sh == yy && xq * p.sw == xx && yq < p.H && xq < p.W;
+                    off += (yq * p.W + xq) * p.T * 4;
+                } else {
+                    ok = t_ok && (unsigned)yy < (unsigned)p.H && (unsigned)xx < (unsigned)p.W;
+                }
+                q[u] = tq.template place<TAIL>(buf_load4<false>(src, ok ? off : kOutOfRange));
                 a[u] = wt[k * 16 + j];
             }
 #pragma unroll
-            for (int u = 0; u < kSynChunk; ++u) {
+            for (int u = 0; u < CHUNK; ++u) {
                 acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u], q[u].x, acc[0], 0, 0, 0);
                 acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u], q[u].y, acc[1], 0, 0, 0);
                 acc[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u], q[u].z, acc[2], 0, 0, 0);
@@ -603,6 +622,28 @@ __global__ __launch_bounds__(kWave) void synapse_wgrad_final_kernel(float* __res
 
 using namespace slayer;
 
+namespace {
+
+// the one-pixel kernel in its forward or transposed form: as many tap groups in flight as the filter has, up to six
+template <bool TRANSPOSED>
+int launch_synapse_conv(SynapseConv p, int64_t K, bool streaming, bool tail, dim3 grid, dim3 block, hipStream_t st) {
+    const int groups = (int)((K + 3) / 4);
+    const int chunk = groups <= 1 ? 1 : (groups == 2 ? 2 : kSynChunk);
+    p.KG = (groups + chunk - 1) / chunk * chunk;
+    const size_t lds = (size_t)p.KG * 4 * (16 * sizeof(float) + 3 * sizeof(int));
+    if (lds > 64 * 1024) return SLAYER_ERANGE;
+#define SLAYER_SYN_ONE(S, TL, CH) hipLaunchKernelGGL((synapse_conv_kernel<S, TL, TRANSPOSED, CH>), grid, block, lds, st, p)
+#define SLAYER_SYN_CH(S, TL) \
+    do { if (chunk == 1) SLAYER_SYN_ONE(S, TL, 1); else if (chunk == 2) SLAYER_SYN_ONE(S, TL, 2); else SLAYER_SYN_ONE(S, TL, kSynChunk); } while (0)
+    if (streaming) { if (tail) SLAYER_SYN_CH(true, true); else SLAYER_SYN_CH(true, false); }
+    else { if (tail) SLAYER_SYN_CH(false, true); else SLAYER_SYN_CH(false, false); }
+#undef SLAYER_SYN_CH
+#undef SLAYER_SYN_ONE
+    return (int)hipGetLastError();
+}
+
+}  // namespace
+
 extern "C" int slayer_conv_synapse(float* out, const float* in, const float* weight,
                                    int64_t N, int64_t Ci, int64_t Co, int64_t H, int64_t W, int64_t T,
                                    int64_t kh, int64_t kw, int64_t stride_h, int64_t stride_w,
@@ -665,16 +706,7 @@ extern "C" int slayer_conv_synapse(float* out, const float* in, const float* wei
 #undef SLAYER_SYN_ROW
         return (int)hipGetLastError();
     }
-    p.KG = (int)(((K + 3) / 4 + kSynChunk - 1) / kSynChunk * kSynChunk);
-    const size_t lds = (size_t)p.KG * 4 * (16 * sizeof(float) + 3 * sizeof(int));
-    if (lds > 64 * 1024) return SLAYER_ERANGE;
-    if (streaming) {
-        if (tail) hipLaunchKernelGGL((synapse_conv_kernel<true, true>), grid, block, lds, st, p);
-        else hipLaunchKernelGGL((synapse_conv_kernel<true, false>), grid, block, lds, st, p);
-    } else {
-        if (tail) hipLaunchKernelGGL((synapse_conv_kernel<false, true>), grid, block, lds, st, p);
-        else hipLaunchKernelGGL((synapse_conv_kernel<false, false>), grid, block, lds, st, p);
-    }
+    return launch_synapse_conv<false>(p, K, streaming, tail, grid, block, st);
     return (int)hipGetLastError();
 }
 
@@ -803,4 +835,50 @@ extern "C" int slayer_conv_synapse_wgrad(float* grad_weight, const float* grad_o
     hipLaunchKernelGGL(synapse_wgrad_final_kernel, dim3(tile_blocks), dim3(kWave), 0, st, grad_weight, stage, (int)Co,
                        (int)K, p.passes, f.tiles, f.row_kw, f.npt);
     return (int)hipGetLastError();
+}
+
+// The gradient of the input of slayer_conv_synapse for any stride (and, read as a layer of its own, the transposed
+// convolution): see TRANSPOSED in synapse_conv_kernel.
+extern "C" int slayer_conv_synapse_input_grad(float* grad_in, const float* grad_out, const float* weight_t,
+                                              int64_t N, int64_t Ci, int64_t Co, int64_t H, int64_t W, int64_t T,
+                                              int64_t kh, int64_t kw, int64_t stride_h, int64_t stride_w,
+                                              int64_t pad_h, int64_t pad_w, int64_t dil_h, int64_t dil_w, void* stream) {
+    if (N < 0 || Ci < 1 || Co < 1 || H < 1 || W < 1 || T < 0 || kh < 1 || kw < 1 || stride_h < 1 || stride_w < 1 ||
+        pad_h < 0 || pad_w < 0 || dil_h < 1 || dil_w < 1)
+        return SLAYER_EINVAL;
+    const int64_t Ho = (H + 2 * pad_h - dil_h * (kh - 1) - 1) / stride_h + 1;
+    const int64_t Wo = (W + 2 * pad_w - dil_w * (kw - 1) - 1) / stride_w + 1;
+    if (Ho < 1 || Wo < 1) return SLAYER_EINVAL;
+    if (N == 0 || T == 0) return 0;
+    if (!grad_in || !grad_out || !weight_t) return SLAYER_ENULL;
+    if (T < 4) return SLAYER_ERANGE;
+    const int64_t K = Co * kh * kw, lim = (int64_t)1 << 31;
+    // coordinates below 2^16 and strides up to 16: the quotients by the strides are taken in float
+    if (Ci * H * W * T * 4 >= lim || Co * Ho * Wo * T * 4 >= lim || K > 4096 || pad_h > 4096 || pad_w > 4096 ||
+        H + pad_h >= (1 << 16) || W + pad_w >= (1 << 16) || stride_h > 16 || stride_w > 16)
+        return SLAYER_ERANGE;
+    SynapseConv p;
+    p.out = grad_in; p.in = grad_out; p.weight = weight_t;
+    // in the kernel's names: the source is the gradient of the output, the result the gradient of the input
+    p.N = (int)N; p.Ci = (int)Co; p.Co = (int)Ci; p.H = (int)Ho; p.W = (int)Wo; p.Ho = (int)H; p.Wo = (int)W; p.T = (int)T;
+    p.kh = (int)kh; p.kw = (int)kw; p.sh = (int)stride_h; p.sw = (int)stride_w; p.ph = (int)pad_h; p.pw = (int)pad_w;
+    p.dh = (int)dil_h; p.dw = (int)dil_w;
+    p.inv_sh = 1.0f / (float)stride_h; p.inv_sw = 1.0f / (float)stride_w;
+    p.K = (int)K;
+    p.ttiles = (int)((T + kSynTile - 1) / kSynTile);
+    const int64_t cobs = (Ci + 15) / 16;
+    const int64_t base = N * cobs * H * p.ttiles;
+    int wsplit = 1;
+    while (base * wsplit < 16 * 1024 && wsplit * 2 <= W) wsplit *= 2;
+    p.wsplit = wsplit;
+    const int64_t items = H * wsplit * p.ttiles;
+    if (items > 0x7fffffffLL) return SLAYER_ERANGE;
+    p.items = (int)items;
+    const int64_t blocks = N * cobs * ((items + kSynWaves - 1) / kSynWaves);
+    if (blocks > 0x7fffffffLL) return SLAYER_ERANGE;
+    const bool streaming = N * Ci * H * W * T * 4 > ((int64_t)64 << 20);
+    const bool tail = (T % 4) != 0;
+    const dim3 grid((unsigned)blocks), block(kSynWaves * kWave);
+    hipStream_t st = (hipStream_t)stream;
+    return launch_synapse_conv<true>(p, K, streaming, tail, grid, block, st);
 }

@@ -57,6 +57,7 @@ _SIGNATURES = {
     'slayer_shift': (_INT, [_P, _P, _P, _I64, _F, _I64, _I64, _I64, _P]),
     'slayer_delay_bwd': (_INT, [_P, _P, _P, _P, _P, _I64, _F, _P, _I64, _I64, _I64, _P]),
     'slayer_conv_synapse': (_INT, [_P, _P, _P] + [_I64] * 14 + [_P]),
+    'slayer_conv_synapse_input_grad': (_INT, [_P, _P, _P] + [_I64] * 14 + [_P]),
     'slayer_conv_synapse_wgrad_workspace': (_I64, [_I64] * 11),
     'slayer_conv_synapse_wgrad': (_INT, [_P, _P, _P] + [_I64] * 14 + [_P, _I64, _P]),
     'slayer_conv': (_INT, [_P, _P, _P, _I64, _F, _I64, _I64, _P]),

@@ -1,3 +1,3 @@
-from .layer import Conv, Dense, conv_synapse
+from .layer import Conv, Dense, Pool, conv_synapse
 
-__all__ = ['Conv', 'Dense', 'conv_synapse']
+__all__ = ['Conv', 'Dense', 'Pool', 'conv_synapse']

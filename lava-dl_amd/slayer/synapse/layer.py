@@ -43,6 +43,22 @@ def _launch(input, weight4, stride, padding, dilation):
     return out
 
 
+def _launch_input_grad(grad_output, weight_t4, input_shape, stride, padding, dilation):
+    """Gradient of the input for any stride, or None (None: outside what the kernel takes).
+    weight_t4: [Ci, Co, kh, kw], the forward weights with the channel axes exchanged."""
+    n, ci, h, w, t = input_shape
+    _, co, kh, kw = weight_t4.shape
+    grad = torch.empty(tuple(input_shape), dtype=torch.float32, device=grad_output.device)
+    with N.device_guard(grad_output.device):
+        code = N.lib().slayer_conv_synapse_input_grad(N.ptr(grad), N.ptr(grad_output), N.ptr(weight_t4), n, ci, co, h, w,
+                                                      t, kh, kw, stride[0], stride[1], padding[0], padding[1],
+                                                      dilation[0], dilation[1], N.stream_handle())
+    if code == _ERANGE:
+        return None
+    N.check(code)
+    return grad
+
+
 class _ConvSynapse(torch.autograd.Function):
     @staticmethod
     def forward(ctx, input, weight, stride, padding, dilation):
@@ -68,6 +84,10 @@ class _ConvSynapse(torch.autograd.Function):
                 if back[0] >= 0 and back[1] >= 0:
                     grad_input = _launch(grad_output, flipped, (1, 1), back, dilation)
             if grad_input is None or grad_input.shape != input.shape:
+                # any stride: the transposed form of the kernel
+                grad_input = _launch_input_grad(grad_output, weight.detach()[..., 0].transpose(0, 1).contiguous(),
+                                                input.shape, stride, padding, dilation)
+            if grad_input is None:
                 grad_input = torch.nn.grad.conv3d_input(input.shape, weight, grad_output, stride + (1,),
                                                         padding + (0,), dilation + (1,), 1)
         if ctx.needs_input_grad[1]:
@@ -221,3 +241,42 @@ class Conv(torch.nn.Conv3d, _SynapseLayer):
     def forward(self, input):
         """Weighted spikes [N, out_features, Ho, Wo, T] for spikes [N, in_features, H, W, T]."""
         return conv_synapse(input, self._weight(), self._stride2, self._padding2, self._dilation2, self.groups)
+
+
+class Pool(torch.nn.Conv3d, _SynapseLayer):
+    """Pooling synapse layer (synapse/layer.py:326-510 in the reference): every channel is summed over windows of
+    ``kernel_size`` with a common weight (``weight_scale``, not trained).  The reference folds the channels into
+    the image height and applies a one-channel ``F.conv3d``; here the same tensor goes through the convolution
+    kernels of this package, its gradient through their transposed form.
+
+    Parameters
+    ----------
+    kernel_size, stride, padding, dilation : int or (height, width); ``stride`` defaults to ``kernel_size``.
+    weight_scale, weight_norm, pre_hook_fx : as for :class:`Conv`.
+    """
+
+    def __init__(self, kernel_size, stride=None, padding=0, dilation=1, weight_scale=1, weight_norm=False,
+                 pre_hook_fx=None):
+        kernel = _pair(kernel_size, 'kernel_size')
+        self._stride2 = kernel if stride is None else _pair(stride, 'stride')
+        self._padding2, self._dilation2 = _pair(padding, 'padding'), _pair(dilation, 'dilation')
+        super().__init__(1, 1, kernel + (1,), self._stride2 + (1,), self._padding2 + (0,), self._dilation2 + (1,),
+                         bias=False)
+        self.weight = torch.nn.Parameter(weight_scale * torch.ones_like(self.weight), requires_grad=False)
+        self._finish(1, weight_norm, pre_hook_fx)
+
+    def forward(self, input):
+        """Pooled spikes [N, C, Ho, Wo, T] for spikes [N, C, H, W, T]."""
+        kh, kw = self.weight.shape[2], self.weight.shape[3]
+        # as the reference does it: H % kh (W % kw) rows (columns) of zeros behind an image that is not a whole
+        # number of windows, then the channels folded into the height
+        if input.shape[2] % kh != 0:
+            input = torch.cat((input, input.new_zeros(input.shape[0], input.shape[1], input.shape[2] % kh,
+                                                      input.shape[3], input.shape[4])), 2)
+        if input.shape[3] % kw != 0:
+            input = torch.cat((input, input.new_zeros(input.shape[0], input.shape[1], input.shape[2],
+                                                      input.shape[3] % kw, input.shape[4])), 3)
+        n, c, h, w, t = input.shape
+        result = conv_synapse(input.reshape(n, 1, c * h, w, t), self._weight(), self._stride2, self._padding2,
+                              self._dilation2)
+        return result.reshape(n, c, -1, result.shape[3], t)

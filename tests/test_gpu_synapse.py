@@ -165,3 +165,38 @@ def test_tensors_at_dword_aligned_addresses(slayer):
         results.append((y.detach(), xs.grad, ws.grad))
     for a, b, what in zip(results[0], results[1], ('forward', 'grad input', 'grad weight')):
         assert torch.equal(a, b), what
+
+
+@pytest.mark.parametrize('shape,kernel,stride,scale', [((2, 3, 8, 6, 20), 2, None, 1.0), ((1, 4, 7, 9, 64), 2, None, 0.5),
+                                                        ((2, 2, 9, 8, 33), (3, 2), None, 2.0), ((1, 16, 32, 32, 100), 2, None, 1.0),
+                                                        ((2, 3, 9, 8, 12), 3, 3, 1.0), ((1, 2, 12, 10, 18), (4, 2), (4, 2), 1.0)])
+def test_pool_layer(slayer, shape, kernel, stride, scale):
+    """slayer.synapse.Pool (synapse/layer.py:326-510 in the reference) through the convolution kernels: the sums
+    over the windows as the reference forms them (channels folded into the height, zero rows behind an image that
+    is not a whole number of windows), and the gradient of the input through the transposed kernel, against
+    float64 autograd of the same expression."""
+    gen = torch.Generator().manual_seed(seed_of('pool', shape, kernel, stride))
+    pool = slayer.synapse.Pool(kernel, stride, weight_scale=scale).to(dev())
+    x = (torch.rand(shape, generator=gen) < 0.3).float() * torch.randn(shape, generator=gen)
+    xg = x.to(dev()).requires_grad_()
+    y = pool(xg)
+
+    def reference(v):
+        kh, kw = pool.weight.shape[2], pool.weight.shape[3]
+        if v.shape[2] % kh:
+            v = torch.cat((v, v.new_zeros(v.shape[0], v.shape[1], v.shape[2] % kh, v.shape[3], v.shape[4])), 2)
+        if v.shape[3] % kw:
+            v = torch.cat((v, v.new_zeros(v.shape[0], v.shape[1], v.shape[2], v.shape[3] % kw, v.shape[4])), 3)
+        n, c, h, w, t = v.shape
+        r = F.conv3d(v.reshape(n, 1, c * h, w, t), pool.weight.detach().cpu().to(v.dtype), None, pool.stride)
+        return r.reshape(n, c, -1, r.shape[3], t)
+
+    xd, xa = x.double().requires_grad_(), x.abs().double().requires_grad_()
+    want, mag = reference(xd), reference(xa)
+    assert y.shape == want.shape
+    assert_sum(y, want.detach(), mag.detach() + 1e-30, 'pooled spikes')
+    g = torch.randn(want.shape, generator=gen)
+    y.backward(g.to(dev()))
+    want.backward(g.double())
+    mag.backward(g.abs().double())
+    assert_sum(xg.grad, xd.grad, xa.grad + 1e-30, 'gradient of the input')

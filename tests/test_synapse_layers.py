@@ -45,3 +45,16 @@ def test_weight_norm_and_pre_hook_of_the_layers():
         layer.pre_hook_fx = lambda w: w * 0
         x = torch.ones(1, 6, 4) if isinstance(layer, slayer.synapse.Dense) else torch.ones(1, 2, 4, 4, 5)
         assert float(layer(x).abs().max()) == 0.0
+
+
+def test_pool_folds_the_channels_into_the_height_as_the_reference_does():
+    gen = torch.Generator().manual_seed(6)
+    pool = slayer.synapse.Pool(2, weight_scale=1.5)
+    assert tuple(pool.weight.shape) == (1, 1, 2, 2, 1) and not pool.weight.requires_grad
+    assert float(pool.weight.min()) == float(pool.weight.max()) == 1.5
+    x = torch.randn(2, 3, 6, 8, 5, generator=gen)
+    want = F.conv3d(x.reshape(2, 1, 18, 8, 5), 1.5 * torch.ones(1, 1, 2, 2, 1), None, (2, 2, 1)).reshape(2, 3, -1, 4, 5)
+    assert torch.allclose(pool(x), want)
+    # every output is the weighted sum of its own window of its own channel
+    assert torch.allclose(pool(x)[1, 2, 1, 3], 1.5 * x[1, 2, 2:4, 6:8].sum(dim=(0, 1)))
+    assert slayer.synapse.Pool((2, 3))(torch.randn(1, 2, 5, 7, 4, generator=gen)).shape == (1, 2, 3, 2, 4)
