@@ -312,7 +312,8 @@ int slayer_corr(float *out, const float *in, const float *filt, int64_t K, float
  * out[n][co][ho][wo][t] = sum over ci, y, x of weight[co][ci][y][x] *
  *                         in[n][ci][ho * stride_h + y * dil_h - pad_h][wo * stride_w + x * dil_w - pad_w][t]
  * (zero outside the image), Ho = (H + 2 pad_h - dil_h (kh - 1) - 1) / stride_h + 1, Wo likewise; weight is
- * [Co][Ci][kh][kw] (the reference's [Co][Ci][kh][kw][1]).  float32 operands and accumulation on the matrix cores.
+ * [Co][Ci][kh][kw] (the reference's [Co][Ci][kh][kw][1]).  float32 operands and accumulation on the matrix cores
+ * (on the vector units when Ci = Co = 1: the pooling layers, which fold their channels into the image height).
  * The gradient of the input is the same call on the gradient with the weights transposed and flipped.
  * Rows of any length from four steps on, float-aligned tensors.  SLAYER_ERANGE for what the kernel does not take
  * (T < 4, a batch entry of 2 GiB or more, more than about 860 taps Ci * kh * kw): the caller keeps its library
@@ -328,8 +329,10 @@ int slayer_conv_synapse(float *out, const float *in, const float *weight,
  *                           grad_out[n][co][(h + pad_h - y * dil_h) / stride_h][(w + pad_w - x * dil_w) / stride_w][t]
  * over the taps whose two quotients are exact and lie inside grad_out's [Ho][Wo].  N, Ci, Co, H, W, kh ... dil_w are
  * those of the forward call; weight_t is [Ci][Co][kh][kw] (the forward weights with the channel axes exchanged,
- * not flipped).  With unit strides slayer_conv_synapse on the flipped weights is the faster call.  SLAYER_ERANGE
- * as for slayer_conv_synapse, and for strides above 16 or images beyond 65535 pixels a side. */
+ * not flipped).  One launch per residue class of the pixels modulo the strides (stride_h * stride_w launches, each
+ * a plain convolution over the taps that class meets); a single launch on the vector units when Ci = Co = 1 (the
+ * pooling layers).  SLAYER_ERANGE as for slayer_conv_synapse, and for strides above 16 or images beyond 65535
+ * pixels a side. */
 int slayer_conv_synapse_input_grad(float *grad_in, const float *grad_out, const float *weight_t,
                                    int64_t N, int64_t Ci, int64_t Co, int64_t H, int64_t W, int64_t T,
                                    int64_t kh, int64_t kw, int64_t stride_h, int64_t stride_w,

@@ -70,27 +70,36 @@ constexpr int kSynChunk = 6;            // tap groups whose loads are in flight 
 struct SynapseConv {
     float* out;
     const float* in;
-    const float* weight;                // [Co][Ci][kh][kw]
+    const float* weight;                // [Co][Ci][kh_full][kw_full]
     int N, Ci, Co, H, W, Ho, Wo, T;
-    int kh, kw, sh, sw, ph, pw, dh, dw;
+    int kh, kw, sh, sw, ph, pw, dh, dw; // ph, pw: may be negative (a window that begins inside the image)
     int K, KG;                          // taps, groups of four taps (a whole number of chunks, padded with null taps)
     int ttiles, wsplit;                 // tiles of 64 steps per row, pieces an image row is cut into
     int items;                          // (tile, piece, output row) triples of one (batch entry, channel block)
-    float inv_sh, inv_sw;               // TRANSPOSED: 1 / stride
+    // The taps may be a sub-lattice of a larger filter and the outputs a sub-lattice of a larger image (identity for
+    // a plain convolution): row iy of the kh x kw taps is row ky0 + iy * kys of the weight tensor's kh_full rows,
+    // output pixel (ho, wo) is pixel (oy0 + ho * oys, ox0 + wo * oxs) of a tensor [Co][Ho_full][Wo_full][T].
+    int kh_full, kw_full, ky0, kys, kx0, kxs;
+    int Ho_full, Wo_full, oy0, oys, ox0, oxs;
+    __device__ __forceinline__ int weight_index(int ci, int iy, int ix) const {
+        return (ci * kh_full + ky0 + iy * kys) * kw_full + kx0 + ix * kxs;
+    }
+    __device__ __forceinline__ int out_pixel(int ho, int wo) const {     // in pixels of the full output image
+        return (oy0 + ho * oys) * Wo_full + ox0 + wo * oxs;
+    }
 };
 
-// TRANSPOSED: the gradient of the input of a convolution of any stride (what conv_transpose3d computes, the
-// ConvTranspose synapse of synapse/layer.py:513-560 in the reference): `in` is the gradient of the convolution's
-// output, [N][Ci][H][W][T] in this structure's names, `out` the gradient of its input, [N][Co][Ho][Wo][T], `weight`
-// [Co][Ci][kh][kw] (the convolution's weights with the two channel axes exchanged), and tap (ci, y, x) of output
-// pixel (ho, wo) reads source pixel ((ho + ph - y dh) / sh, (wo + pw - x dw) / sw) where both divisions are exact
-// and the result lies in the source image -- one tap in sh * sw on average.
+// The gradient of the input of a convolution with strides (what conv_transpose3d computes, the ConvTranspose synapse
+// of synapse/layer.py:513-560 in the reference) is one plain convolution per residue class of the output pixels: the
+// pixels (ry + m sh, rx + m' sw) meet only the taps y with (ry + ph - y dh) divisible by sh (x likewise), and over
+// m, m' those taps slide across the source with unit stride.  Each class is a launch of the kernels below on its
+// sub-lattices of taps and of outputs (slayer_conv_synapse_input_grad), a fraction 1 / (sh sw) of the taps each.
 //
 // LDS: the weights of this workgroup's 16 output channels, tap-major (row k holds the 16 channels), and per tap the
 // offset of its input row relative to the pixel's own position and its (row, column) displacement in the image.
 // A workgroup's four waves take four consecutive items of one (batch entry, channel block): an item is one tile
 // of 64 steps of a piece of one output row.
-template <bool STREAM, bool TAIL, bool TRANSPOSED, int CHUNK>
+template <bool STREAM, bool TAIL, int CHUNK>
 __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_kernel(const SynapseConv p) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int Kp = p.KG * 4;
@@ -109,17 +118,19 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_kernel(const S
     const int n = b / ((p.Co + 15) / 16);
     const int co0 = cob * 16;
 
+    const int64_t k_full = (int64_t)p.Ci * p.kh_full * p.kw_full;
     for (int i = tid; i < Kp * 16; i += kSynWaves * kWave) {
         const int k = i >> 4, m = i & 15;
-        wt[i] = (k < p.K && co0 + m < p.Co) ? p.weight[(int64_t)(co0 + m) * p.K + k] : 0.0f;
+        const int ci = k / (p.kh * p.kw), r = k - ci * (p.kh * p.kw), y = r / p.kw, x = r - y * p.kw;
+        wt[i] = (k < p.K && co0 + m < p.Co) ? p.weight[(int64_t)(co0 + m) * k_full + p.weight_index(ci, y, x)] : 0.0f;
     }
     for (int k = tid; k < Kp; k += kSynWaves * kWave) {
         const int ci = k / (p.kh * p.kw), r = k - ci * (p.kh * p.kw), y = r / p.kw, x = r - y * p.kw;
-        const int dy = TRANSPOSED ? p.ph - y * p.dh : y * p.dh - p.ph;
-        const int dx = TRANSPOSED ? p.pw - x * p.dw : x * p.dw - p.pw;
-        tap_dy[k] = k < p.K ? dy : (TRANSPOSED ? -(1 << 28) : (1 << 28));   // a tap that does not exist: always outside
+        const int dy = y * p.dh - p.ph;
+        const int dx = x * p.dw - p.pw;
+        tap_dy[k] = k < p.K ? dy : (1 << 28);                             // a tap that does not exist: always outside
         tap_dx[k] = dx;
-        tap_off[k] = TRANSPOSED ? ci * p.H * p.W * p.T * 4 : (((ci * p.H + dy) * p.W) + dx) * p.T * 4;
+        tap_off[k] = (((ci * p.H + dy) * p.W) + dx) * p.T * 4;
     }
     __syncthreads();
 
@@ -134,18 +145,17 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_kernel(const S
     tq.template set<TAIL>(t0 + 4 * j, p.T);
     const int nv = tq.nv;
     const bool t_ok = tq.any();
-    const int hin = TRANSPOSED ? ho : ho * p.sh;                         // image row of tap (0, 0) before padding
+    const int hin = ho * p.sh;                                           // image row of tap (0, 0) before padding
     const int64_t in_plane = (int64_t)p.Ci * p.H * p.W * p.T;
     const __amdgpu_buffer_rsrc_t src = make_rsrc(p.in + (int64_t)n * in_plane, (unsigned)(in_plane * 4));
-    const int64_t out_plane = (int64_t)p.Co * p.Ho * p.Wo * p.T;
+    const int64_t out_plane = (int64_t)p.Co * p.Ho_full * p.Wo_full * p.T;
     const __amdgpu_buffer_rsrc_t dst = make_rsrc(p.out + (int64_t)n * out_plane, (unsigned)(out_plane * 4));
 
     const int per = (p.Wo + p.wsplit - 1) / p.wsplit;
     const int w_lo = piece * per, w_hi = (w_lo + per) < p.Wo ? (w_lo + per) : p.Wo;
     for (int wo = w_lo; wo < w_hi; ++wo) {
-        const int win = TRANSPOSED ? wo : wo * p.sw;
-        // byte offset of tap (0,0,0)'s quad (TRANSPOSED: of the quad inside a row of the source)
-        const int pix = TRANSPOSED ? tq.t_load * 4 : ((hin * p.W) + win) * p.T * 4 + tq.t_load * 4;
+        const int win = wo * p.sw;
+        const int pix = ((hin * p.W) + win) * p.T * 4 + tq.t_load * 4;   // byte offset of tap (0,0,0)'s quad
         syn_f4 acc[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc[e] = syn_f4{0.f, 0.f, 0.f, 0.f};
@@ -156,17 +166,8 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_kernel(const S
             for (int u = 0; u < CHUNK; ++u) {
                 const int k = 4 * (g0 + u) + kk;
                 const int yy = hin + tap_dy[k], xx = win + tap_dx[k];
-                bool ok;
-                int off = pix + tap_off[k];
-                if (TRANSPOSED) {
-                    // exact quotients of small non-negative integers by way of float (coordinates below 2^16)
-                    const int yq = (int)(((float)yy + 0.5f) * p.inv_sh), xq = (int)(((float)xx + 0.5f) * p.inv_sw);
-                    ok = t_ok && yy >= 0 && xx >= 0 && yq * p.sh == yy && xq * p.sw == xx && yq < p.H && xq < p.W;
-                    off += (yq * p.W + xq) * p.T * 4;
-                } else {
-                    ok = t_ok && (unsigned)yy < (unsigned)p.H && (unsigned)xx < (unsigned)p.W;
-                }
-                q[u] = tq.template place<TAIL>(buf_load4<false>(src, ok ? off : kOutOfRange));
+                const bool ok = t_ok && (unsigned)yy < (unsigned)p.H && (unsigned)xx < (unsigned)p.W;
+                q[u] = tq.template place<TAIL>(buf_load4<false>(src, ok ? pix + tap_off[k] : kOutOfRange));
                 a[u] = wt[k * 16 + j];
             }
 #pragma unroll
@@ -178,11 +179,11 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_kernel(const S
             }
         }
         // lane (kk, j): output channels co0 + 4 kk + i, steps t0 + 4 j + e
-        const int opix = ((ho * p.Wo) + wo) * p.T * 4 + (t0 + 4 * j) * 4;
+        const int opix = p.out_pixel(ho, wo) * p.T * 4 + (t0 + 4 * j) * 4;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int co = co0 + 4 * kk + i;
-            syn_store_quad<STREAM, TAIL>(dst, co < p.Co, co * (p.Ho * p.Wo * p.T * 4) + opix, nv,
+            syn_store_quad<STREAM, TAIL>(dst, co < p.Co, co * (p.Ho_full * p.Wo_full * p.T * 4) + opix, nv,
                                    make_float4(acc[0][i], acc[1][i], acc[2][i], acc[3][i]));
         }
     }
@@ -213,9 +214,11 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_row_kernel(con
     const int n = b / ((p.Co + 15) / 16);
     const int co0 = cob * 16;
 
+    const int64_t k_full = (int64_t)p.Ci * p.kh_full * p.kw_full;
     for (int i = tid; i < Kp * 16; i += kSynWaves * kWave) {
         const int k = i >> 4, m = i & 15;
-        wt[i] = (k < p.K && co0 + m < p.Co) ? p.weight[(int64_t)(co0 + m) * p.K + k] : 0.0f;
+        const int pr = k / KW, x = k - pr * KW, ci = pr / p.kh, y = pr - ci * p.kh;
+        wt[i] = (k < p.K && co0 + m < p.Co) ? p.weight[(int64_t)(co0 + m) * k_full + p.weight_index(ci, y, x)] : 0.0f;
     }
     for (int pr = tid; pr < 4 * PG; pr += kSynWaves * kWave) {
         const int ci = pr / p.kh, y = pr - ci * p.kh;
@@ -239,7 +242,7 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_row_kernel(con
     const int hin = ho * p.sh;
     const int64_t in_plane = (int64_t)p.Ci * p.H * p.W * p.T;
     const __amdgpu_buffer_rsrc_t src = make_rsrc(p.in + (int64_t)n * in_plane, (unsigned)(in_plane * 4));
-    const int64_t out_plane = (int64_t)p.Co * p.Ho * p.Wo * p.T;
+    const int64_t out_plane = (int64_t)p.Co * p.Ho_full * p.Wo_full * p.T;
     const __amdgpu_buffer_rsrc_t dst = make_rsrc(p.out + (int64_t)n * out_plane, (unsigned)(out_plane * 4));
     const int col = p.T * 4;                                             // bytes from a pixel to its right neighbour
 
@@ -280,14 +283,74 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_row_kernel(con
         // lane (kk, j): output channels co0 + 4 kk + i, steps t0 + 4 j + e
 #pragma unroll
         for (int px = 0; px < PIX; ++px) {
-            const int opix = ((ho * p.Wo) + wo0 + px) * col + (t0 + 4 * j) * 4;
+            const int opix = p.out_pixel(ho, wo0 + px) * col + (t0 + 4 * j) * 4;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int co = co0 + 4 * kk + i;
-                syn_store_quad<STREAM, TAIL>(dst, co < p.Co && wo0 + px < w_hi, co * (p.Ho * p.Wo * col) + opix, nv,
+                syn_store_quad<STREAM, TAIL>(dst, co < p.Co && wo0 + px < w_hi, co * (p.Ho_full * p.Wo_full * col) + opix, nv,
                                        make_float4(acc[px][0][i], acc[px][1][i], acc[px][2][i], acc[px][3][i]));
             }
         }
+    }
+}
+
+// One input and one output channel (the pooling layers, which fold their channels into the image height,
+// synapse/layer.py:438-508 and :770-838 in the reference): there is no contraction for the matrix cores, and a wave
+// that owns 16 channels x 64 steps of one pixel would move 256 bytes per instruction.  One thread per quad of output
+// steps on the vector units instead: a block row of the grid is an image row of the output, grid.z the batch.
+// SPREAD: the gradient of the input (the unpooling layer's forward pass): output pixel (h, w) sums the taps (y, x)
+// whose source coordinates (h + ph - y dh) / sh, (w + pw - x dw) / sw are exact; which taps those are, and the
+// quotients less h / sh, depend on h mod sh alone and come from a table in LDS (quot_y[ry * kh + y], likewise x).
+constexpr int kPlaneThreads = 256;
+template <bool SPREAD, bool STREAM, bool TAIL>
+__global__ __launch_bounds__(kPlaneThreads) void synapse_plane_kernel(const SynapseConv p, int quads, int rows) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    float* wt = lds;                                                      // [kh * kw]
+    int* quot_y = reinterpret_cast<int*>(lds + p.kh * p.kw);              // SPREAD: [sh * kh]
+    int* quot_x = quot_y + p.sh * p.kh;                                   // SPREAD: [sw * kw]
+    const int none = 1 << 28;
+    for (int i = threadIdx.x; i < p.kh * p.kw; i += kPlaneThreads) wt[i] = p.weight[i];
+    if (SPREAD) {
+        for (int i = threadIdx.x; i < p.sh * p.kh; i += kPlaneThreads) {
+            const int c = i / p.kh + p.ph - (i % p.kh) * p.dh;
+            quot_y[i] = c % p.sh == 0 ? c / p.sh : none;
+        }
+        for (int i = threadIdx.x; i < p.sw * p.kw; i += kPlaneThreads) {
+            const int c = i / p.kw + p.pw - (i % p.kw) * p.dw;
+            quot_x[i] = c % p.sw == 0 ? c / p.sw : none;
+        }
+    }
+    __syncthreads();
+    const int n = blockIdx.z;
+    const int idx = blockIdx.x * kPlaneThreads + threadIdx.x;
+    const int wo = idx / quads, j = idx - wo * quads;
+    const bool on = wo < p.Wo;
+    SynQuad tq;
+    tq.template set<TAIL>(4 * j, p.T);
+    const int64_t in_plane = (int64_t)p.H * p.W * p.T;
+    const __amdgpu_buffer_rsrc_t src = make_rsrc(p.in + (int64_t)n * in_plane, (unsigned)(in_plane * 4));
+    const int64_t out_plane = (int64_t)p.Ho * p.Wo * p.T;
+    const __amdgpu_buffer_rsrc_t dst = make_rsrc(p.out + (int64_t)n * out_plane, (unsigned)(out_plane * 4));
+    // SPREAD: the pixel as quotient and residue of the strides (the row's are the same for the whole block)
+    const int wq = SPREAD ? wo / p.sw : 0, rx = SPREAD ? (on ? wo - wq * p.sw : 0) : 0;
+    // a block takes `rows` image rows one after the other: the tables above are set up once for all of them
+    for (int ho = blockIdx.y * rows; ho < p.Ho && ho < (blockIdx.y + 1) * rows; ++ho) {
+        const int hq = SPREAD ? ho / p.sh : 0, ry = SPREAD ? ho - hq * p.sh : 0;
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int y = 0; y < p.kh; ++y) {
+            const int yy = SPREAD ? hq + quot_y[ry * p.kh + y] : ho * p.sh + y * p.dh - p.ph;
+            if ((unsigned)yy >= (unsigned)p.H) continue;                  // the same for the whole block
+            for (int x = 0; x < p.kw; ++x) {
+                const int xx = SPREAD ? wq + quot_x[rx * p.kw + x] : wo * p.sw + x * p.dw - p.pw;
+                const bool ok = on && tq.any() && (unsigned)xx < (unsigned)p.W;
+                const float4 q = tq.template place<TAIL>(
+                    buf_load4<false>(src, ok ? ((yy * p.W + xx) * p.T + tq.t_load) * 4 : kOutOfRange));
+                const float f = wt[y * p.kw + x];
+                acc.x = __fmaf_rn(f, q.x, acc.x); acc.y = __fmaf_rn(f, q.y, acc.y);
+                acc.z = __fmaf_rn(f, q.z, acc.z); acc.w = __fmaf_rn(f, q.w, acc.w);
+            }
+        }
+        syn_store_quad<STREAM, TAIL>(dst, on, ((ho * p.Wo + wo) * p.T + 4 * j) * 4, tq.nv, acc);
     }
 }
 
@@ -624,15 +687,56 @@ using namespace slayer;
 
 namespace {
 
-// the one-pixel kernel in its forward or transposed form: as many tap groups in flight as the filter has, up to six
-template <bool TRANSPOSED>
-int launch_synapse_conv(SynapseConv p, int64_t K, bool streaming, bool tail, dim3 grid, dim3 block, hipStream_t st) {
+#ifndef SLAYER_SYN_PIX
+#define SLAYER_SYN_PIX 4
+#endif
+
+// One launch of the convolution kernels for the geometry in p (tensors, sizes, taps and sub-lattices filled in by the
+// caller): the row kernel for unit stride and dilation along the image row with 3 or 5 taps per row, else the
+// one-pixel kernel with as many tap groups in flight as the filter has, up to six.  A filter without taps (K = 0)
+// clears its outputs.
+int launch_synapse_conv(SynapseConv p, bool streaming, hipStream_t st) {
+    constexpr int kRowPix = SLAYER_SYN_PIX;
+    const int64_t K = (int64_t)p.Ci * p.kh * p.kw;
+    p.K = (int)K;
+    p.ttiles = (p.T + kSynTile - 1) / kSynTile;
+    // blocks of four neighbouring pixels that share their input columns: unit stride and dilation along the row
+    const bool rows = p.sw == 1 && p.dw == 1 && (p.kw == 2 || p.kw == 3 || p.kw == 5) && p.Wo >= kRowPix;
+    // enough waves for four rounds of the chip (16 waves on each of 256 compute units), so that the last, partly
+    // filled round weighs little; image rows cut into as few pieces as that takes
+    const int64_t cobs = (p.Co + 15) / 16;
+    const int64_t base = (int64_t)p.N * cobs * p.Ho * p.ttiles;
+    int wsplit = 1;
+    while (base * wsplit < 16 * 1024 && wsplit * 2 * (rows ? kRowPix : 1) <= p.Wo) wsplit *= 2;
+    p.wsplit = wsplit;
+    const int64_t items = (int64_t)p.Ho * wsplit * p.ttiles;
+    if (items > 0x7fffffffLL) return SLAYER_ERANGE;
+    p.items = (int)items;
+    const int64_t blocks = p.N * cobs * ((items + kSynWaves - 1) / kSynWaves);
+    if (blocks > 0x7fffffffLL) return SLAYER_ERANGE;
+    const bool tail = (p.T % 4) != 0;                                     // rows that end inside a quad
+    const dim3 grid((unsigned)blocks), block(kSynWaves * kWave);
+    if (rows) {
+        p.KG = (p.Ci * p.kh + 3) / 4;                                     // groups of four (channel, kernel row) pairs
+        const size_t lds = (size_t)p.KG * 4 * (p.kw * 16 * sizeof(float) + 2 * sizeof(int));
+        if (lds > 64 * 1024) return SLAYER_ERANGE;
+#define SLAYER_SYN_ROW_T(KW, TL)                                                                                         \
+        do {                                                                                                            \
+            if (streaming) hipLaunchKernelGGL((synapse_conv_row_kernel<KW, kRowPix, true, TL>), grid, block, lds, st, p); \
+            else hipLaunchKernelGGL((synapse_conv_row_kernel<KW, kRowPix, false, TL>), grid, block, lds, st, p);         \
+        } while (0)
+#define SLAYER_SYN_ROW(KW) do { if (tail) SLAYER_SYN_ROW_T(KW, true); else SLAYER_SYN_ROW_T(KW, false); } while (0)
+        if (p.kw == 2) SLAYER_SYN_ROW(2); else if (p.kw == 3) SLAYER_SYN_ROW(3); else SLAYER_SYN_ROW(5);
+#undef SLAYER_SYN_ROW_T
+#undef SLAYER_SYN_ROW
+        return (int)hipGetLastError();
+    }
     const int groups = (int)((K + 3) / 4);
     const int chunk = groups <= 1 ? 1 : (groups == 2 ? 2 : kSynChunk);
     p.KG = (groups + chunk - 1) / chunk * chunk;
     const size_t lds = (size_t)p.KG * 4 * (16 * sizeof(float) + 3 * sizeof(int));
     if (lds > 64 * 1024) return SLAYER_ERANGE;
-#define SLAYER_SYN_ONE(S, TL, CH) hipLaunchKernelGGL((synapse_conv_kernel<S, TL, TRANSPOSED, CH>), grid, block, lds, st, p)
+#define SLAYER_SYN_ONE(S, TL, CH) hipLaunchKernelGGL((synapse_conv_kernel<S, TL, CH>), grid, block, lds, st, p)
 #define SLAYER_SYN_CH(S, TL) \
     do { if (chunk == 1) SLAYER_SYN_ONE(S, TL, 1); else if (chunk == 2) SLAYER_SYN_ONE(S, TL, 2); else SLAYER_SYN_ONE(S, TL, kSynChunk); } while (0)
     if (streaming) { if (tail) SLAYER_SYN_CH(true, true); else SLAYER_SYN_CH(true, false); }
@@ -640,6 +744,53 @@ int launch_synapse_conv(SynapseConv p, int64_t K, bool streaming, bool tail, dim
 #undef SLAYER_SYN_CH
 #undef SLAYER_SYN_ONE
     return (int)hipGetLastError();
+}
+
+// The one-channel form (synapse_plane_kernel) for a plain convolution (spread = false: p as for
+// launch_synapse_conv) or for the gradient of its input (spread = true: p.in the gradient of the output [H][W],
+// p.out the gradient of the input [Ho][Wo], strides, padding and dilation those of the convolution).
+// false: not a geometry it takes.
+bool launch_synapse_plane(const SynapseConv& p, bool spread, bool streaming, hipStream_t st, int* code) {
+    const int64_t quads = (p.T + 3) / 4;
+    const int64_t blocks = ((int64_t)p.Wo * quads + kPlaneThreads - 1) / kPlaneThreads;
+    const size_t lds = ((size_t)p.kh * p.kw + (spread ? (size_t)p.sh * p.kh + (size_t)p.sw * p.kw : 0)) * 4;
+    if (p.Ci != 1 || p.Co != 1 || p.N > 65535 || blocks > 0x7fffffffLL || p.kh * p.kw > 1024 ||
+        lds > 48 * 1024)
+        return false;
+    // measured on [32,16,32,32,300] with 2x2 windows: the sums 136 us a row at a time (142 at two, 150 at four), the
+    // spread form 227 us a row at a time, 129 at four, 121 at eight, 123 at sixteen
+    const int rows = spread ? 8 : 1;
+    const dim3 grid((unsigned)blocks, (unsigned)((p.Ho + rows - 1) / rows), (unsigned)p.N), block(kPlaneThreads);
+    const bool tail = (p.T % 4) != 0;
+#define SLAYER_SYN_PLANE(SP, S, TL) hipLaunchKernelGGL((synapse_plane_kernel<SP, S, TL>), grid, block, lds, st, p, (int)quads, rows)
+#define SLAYER_SYN_PLANE_T(SP, S) do { if (tail) SLAYER_SYN_PLANE(SP, S, true); else SLAYER_SYN_PLANE(SP, S, false); } while (0)
+    if (spread) { if (streaming) SLAYER_SYN_PLANE_T(true, true); else SLAYER_SYN_PLANE_T(true, false); }
+    else { if (streaming) SLAYER_SYN_PLANE_T(false, true); else SLAYER_SYN_PLANE_T(false, false); }
+#undef SLAYER_SYN_PLANE_T
+#undef SLAYER_SYN_PLANE
+    *code = (int)hipGetLastError();
+    return true;
+}
+
+// the taps y of a filter row that output pixels of residue r (mod stride) meet in a transposed convolution:
+// (r + pad - y * dil) divisible by stride; they are y_last, y_last - step, ... (count of them), and the source
+// coordinate of y_last for the first pixel of the class, (r + pad - y_last * dil) / stride, is `first`
+struct TapClass { int count, y_last, step, first; };
+TapClass tap_class(int r, int k, int stride, int pad, int dil) {
+    TapClass c{0, 0, 1, 0};
+    int y_first = -1;
+    for (int y = 0; y < k; ++y) {
+        if ((r + pad - y * dil) % stride != 0) continue;
+        if (c.count == 0) y_first = y;
+        else if (c.count == 1) c.step = y - y_first;
+        c.y_last = y;
+        ++c.count;
+    }
+    if (c.count) {
+        const int num = r + pad - c.y_last * dil;                         // divisible by stride, of either sign
+        c.first = num / stride;
+    }
+    return c;
 }
 
 }  // namespace
@@ -668,46 +819,12 @@ extern "C" int slayer_conv_synapse(float* out, const float* in, const float* wei
     p.N = (int)N; p.Ci = (int)Ci; p.Co = (int)Co; p.H = (int)H; p.W = (int)W; p.Ho = (int)Ho; p.Wo = (int)Wo; p.T = (int)T;
     p.kh = (int)kh; p.kw = (int)kw; p.sh = (int)stride_h; p.sw = (int)stride_w; p.ph = (int)pad_h; p.pw = (int)pad_w;
     p.dh = (int)dil_h; p.dw = (int)dil_w;
-    p.K = (int)K;
-    p.ttiles = (int)((T + kSynTile - 1) / kSynTile);
-    // blocks of four neighbouring pixels that share their input columns: unit stride and dilation along the row
-#ifndef SLAYER_SYN_PIX
-#define SLAYER_SYN_PIX 4
-#endif
-    constexpr int kRowPix = SLAYER_SYN_PIX;
-    const bool rows = stride_w == 1 && dil_w == 1 && (kw == 3 || kw == 5) && Wo >= kRowPix;
-    // enough waves for four rounds of the chip (16 waves on each of 256 compute units), so that the last, partly
-    // filled round weighs little; image rows cut into as few pieces as that takes
-    const int64_t base = N * ((Co + 15) / 16) * Ho * p.ttiles;
-    int wsplit = 1;
-    while (base * wsplit < 16 * 1024 && wsplit * 2 * (rows ? kRowPix : 1) <= Wo) wsplit *= 2;
-    p.wsplit = wsplit;
-    const int64_t items = Ho * wsplit * p.ttiles;
-    if (items > 0x7fffffffLL) return SLAYER_ERANGE;
-    p.items = (int)items;
-    const int64_t blocks = N * ((Co + 15) / 16) * ((items + kSynWaves - 1) / kSynWaves);
-    if (blocks > 0x7fffffffLL) return SLAYER_ERANGE;
+    p.kh_full = p.kh; p.kw_full = p.kw; p.ky0 = p.kx0 = 0; p.kys = p.kxs = 1;
+    p.Ho_full = p.Ho; p.Wo_full = p.Wo; p.oy0 = p.ox0 = 0; p.oys = p.oxs = 1;
     const bool streaming = N * Co * Ho * Wo * T * 4 > ((int64_t)64 << 20);
-    const bool tail = (T % 4) != 0;                                       // rows that end inside a quad
-    const dim3 grid((unsigned)blocks), block(kSynWaves * kWave);
-    hipStream_t st = (hipStream_t)stream;
-    if (rows) {
-        p.KG = (int)((Ci * kh + 3) / 4);                                  // groups of four (channel, kernel row) pairs
-        const size_t lds = (size_t)p.KG * 4 * (kw * 16 * sizeof(float) + 2 * sizeof(int));
-        if (lds > 64 * 1024) return SLAYER_ERANGE;
-#define SLAYER_SYN_ROW_T(KW, TL)                                                                                         \
-        do {                                                                                                            \
-            if (streaming) hipLaunchKernelGGL((synapse_conv_row_kernel<KW, kRowPix, true, TL>), grid, block, lds, st, p); \
-            else hipLaunchKernelGGL((synapse_conv_row_kernel<KW, kRowPix, false, TL>), grid, block, lds, st, p);         \
-        } while (0)
-#define SLAYER_SYN_ROW(KW) do { if (tail) SLAYER_SYN_ROW_T(KW, true); else SLAYER_SYN_ROW_T(KW, false); } while (0)
-        if (kw == 3) SLAYER_SYN_ROW(3); else SLAYER_SYN_ROW(5);
-#undef SLAYER_SYN_ROW_T
-#undef SLAYER_SYN_ROW
-        return (int)hipGetLastError();
-    }
-    return launch_synapse_conv<false>(p, K, streaming, tail, grid, block, st);
-    return (int)hipGetLastError();
+    int code = 0;
+    if (launch_synapse_plane(p, false, streaming, (hipStream_t)stream, &code)) return code;
+    return launch_synapse_conv(p, streaming, (hipStream_t)stream);
 }
 
 namespace {
@@ -838,7 +955,7 @@ extern "C" int slayer_conv_synapse_wgrad(float* grad_weight, const float* grad_o
 }
 
 // The gradient of the input of slayer_conv_synapse for any stride (and, read as a layer of its own, the transposed
-// convolution): see TRANSPOSED in synapse_conv_kernel.
+// convolution): one plain convolution per residue class of the pixels of grad_in, see SynapseConv.
 extern "C" int slayer_conv_synapse_input_grad(float* grad_in, const float* grad_out, const float* weight_t,
                                               int64_t N, int64_t Ci, int64_t Co, int64_t H, int64_t W, int64_t T,
                                               int64_t kh, int64_t kw, int64_t stride_h, int64_t stride_w,
@@ -853,32 +970,42 @@ extern "C" int slayer_conv_synapse_input_grad(float* grad_in, const float* grad_
     if (!grad_in || !grad_out || !weight_t) return SLAYER_ENULL;
     if (T < 4) return SLAYER_ERANGE;
     const int64_t K = Co * kh * kw, lim = (int64_t)1 << 31;
-    // coordinates below 2^16 and strides up to 16: the quotients by the strides are taken in float
     if (Ci * H * W * T * 4 >= lim || Co * Ho * Wo * T * 4 >= lim || K > 4096 || pad_h > 4096 || pad_w > 4096 ||
-        H + pad_h >= (1 << 16) || W + pad_w >= (1 << 16) || stride_h > 16 || stride_w > 16)
+        dil_h > 4096 || dil_w > 4096 || H + pad_h >= (1 << 16) || W + pad_w >= (1 << 16) || stride_h > 16 || stride_w > 16)
         return SLAYER_ERANGE;
     SynapseConv p;
     p.out = grad_in; p.in = grad_out; p.weight = weight_t;
-    // in the kernel's names: the source is the gradient of the output, the result the gradient of the input
-    p.N = (int)N; p.Ci = (int)Co; p.Co = (int)Ci; p.H = (int)Ho; p.W = (int)Wo; p.Ho = (int)H; p.Wo = (int)W; p.T = (int)T;
-    p.kh = (int)kh; p.kw = (int)kw; p.sh = (int)stride_h; p.sw = (int)stride_w; p.ph = (int)pad_h; p.pw = (int)pad_w;
-    p.dh = (int)dil_h; p.dw = (int)dil_w;
-    p.inv_sh = 1.0f / (float)stride_h; p.inv_sw = 1.0f / (float)stride_w;
-    p.K = (int)K;
-    p.ttiles = (int)((T + kSynTile - 1) / kSynTile);
-    const int64_t cobs = (Ci + 15) / 16;
-    const int64_t base = N * cobs * H * p.ttiles;
-    int wsplit = 1;
-    while (base * wsplit < 16 * 1024 && wsplit * 2 <= W) wsplit *= 2;
-    p.wsplit = wsplit;
-    const int64_t items = H * wsplit * p.ttiles;
-    if (items > 0x7fffffffLL) return SLAYER_ERANGE;
-    p.items = (int)items;
-    const int64_t blocks = N * cobs * ((items + kSynWaves - 1) / kSynWaves);
-    if (blocks > 0x7fffffffLL) return SLAYER_ERANGE;
+    // in the kernels' names: the source is the gradient of the output, the result the gradient of the input
+    p.N = (int)N; p.Ci = (int)Co; p.Co = (int)Ci; p.H = (int)Ho; p.W = (int)Wo; p.T = (int)T;
+    p.sh = p.sw = 1;
+    p.kh_full = (int)kh; p.kw_full = (int)kw; p.Ho_full = (int)H; p.Wo_full = (int)W;
+    p.oys = (int)stride_h; p.oxs = (int)stride_w;
     const bool streaming = N * Ci * H * W * T * 4 > ((int64_t)64 << 20);
-    const bool tail = (T % 4) != 0;
-    const dim3 grid((unsigned)blocks), block(kSynWaves * kWave);
-    hipStream_t st = (hipStream_t)stream;
-    return launch_synapse_conv<true>(p, K, streaming, tail, grid, block, st);
+    {
+        SynapseConv q = p;                                                // one channel: every class in one launch
+        q.Ho = (int)H; q.Wo = (int)W; q.kh = (int)kh; q.kw = (int)kw; q.sh = (int)stride_h; q.sw = (int)stride_w;
+        q.ph = (int)pad_h; q.pw = (int)pad_w; q.dh = (int)dil_h; q.dw = (int)dil_w;
+        int code = 0;
+        if (launch_synapse_plane(q, true, streaming, (hipStream_t)stream, &code)) return code;
+    }
+    for (int ry = 0; ry < (int)stride_h && ry < (int)H; ++ry) {
+        const TapClass cy = tap_class(ry, (int)kh, (int)stride_h, (int)pad_h, (int)dil_h);
+        for (int rx = 0; rx < (int)stride_w && rx < (int)W; ++rx) {
+            const TapClass cx = tap_class(rx, (int)kw, (int)stride_w, (int)pad_w, (int)dil_w);
+            p.oy0 = ry; p.ox0 = rx;
+            p.Ho = ((int)H - ry + (int)stride_h - 1) / (int)stride_h;
+            p.Wo = ((int)W - rx + (int)stride_w - 1) / (int)stride_w;
+            const bool none = cy.count == 0 || cx.count == 0;            // pixels no tap reaches: zeros
+            // the taps in the order of rising source coordinate: from the last one down, a step of
+            // step * dil / stride pixels of the source each
+            p.kh = none ? 0 : cy.count; p.kw = none ? 0 : cx.count;
+            p.ky0 = cy.y_last; p.kys = -cy.step; p.kx0 = cx.y_last; p.kxs = -cx.step;
+            p.dh = cy.count > 1 ? cy.step * (int)dil_h / (int)stride_h : 1;
+            p.dw = cx.count > 1 ? cx.step * (int)dil_w / (int)stride_w : 1;
+            p.ph = -cy.first; p.pw = -cx.first;
+            const int code = launch_synapse_conv(p, streaming, (hipStream_t)stream);
+            if (code != 0) return code;
+        }
+    }
+    return 0;
 }

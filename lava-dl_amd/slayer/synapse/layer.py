@@ -1,4 +1,4 @@
-"""Synapse layers on time-innermost tensors: the convolution synapse and the dense synapse.
+"""Synapse layers on time-innermost tensors: dense, convolution, pooling and their transposed forms.
 
 Interface of lava.lib.dl.slayer.synapse.Conv (synapse/layer.py:178-323 in the reference): a spatial convolution
 applied at every time step of an NCHWT tensor.  The reference calls ``F.conv3d`` with a kernel of (kh, kw, 1); the
@@ -6,7 +6,8 @@ library behind it wants channels last and transposes the tensor there and back a
 slayer_conv_synapse of libslayer_hip.so computes it where the tensor lies, so the neuron that follows reads the
 result in place; the input gradient is the same kernel on the flipped, transposed weights and the weight gradient
 slayer_conv_synapse_wgrad.  What the kernels do not take (grouped convolutions, fewer than four time steps, more than
-about 860 taps) goes to ``F.conv3d`` and its gradients as before.
+about 860 taps) goes to ``F.conv3d`` and its gradients as before.  The transposed convolution
+(synapse/layer.py:511-658) and the unpooling layer (:661-838) are the same three kernels with their roles exchanged.
 """
 import torch
 import torch.nn.functional as F
@@ -136,6 +137,63 @@ def conv_synapse(input, weight, stride=1, padding=0, dilation=1, groups=1):
     return _ConvSynapse.apply(input, weight, stride, padding, dilation)
 
 
+class _ConvTransposeSynapse(torch.autograd.Function):
+    """The transposed convolution is the input gradient of a convolution from its output channels back to its
+    input channels, so its three passes are that convolution's three kernels with their roles exchanged."""
+
+    @staticmethod
+    def forward(ctx, input, weight, stride, padding, dilation):
+        n, _, h, w, t = input.shape
+        _, co, kh, kw, _ = weight.shape
+        shape = (n, co, (h - 1) * stride[0] - 2 * padding[0] + dilation[0] * (kh - 1) + 1,
+                 (w - 1) * stride[1] - 2 * padding[1] + dilation[1] * (kw - 1) + 1, t)
+        out = _launch_input_grad(input, weight.detach()[..., 0].transpose(0, 1).contiguous(), shape, stride, padding,
+                                 dilation)
+        if out is None:                                              # a limit conv_transpose_synapse() does not know
+            out = F.conv_transpose3d(input, weight.detach(), None, stride + (1,), padding + (0,), 0, 1, dilation + (1,))
+        ctx.save_for_backward(input, weight)
+        ctx.cfg = (stride, padding, dilation)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        input, weight = ctx.saved_tensors
+        stride, padding, dilation = ctx.cfg
+        grad_output = grad_output.contiguous()
+        grad_input = grad_weight = None
+        if ctx.needs_input_grad[0]:
+            grad_input = _launch(grad_output, weight.detach()[..., 0].contiguous(), stride, padding, dilation)
+            if grad_input is None:
+                grad_input = F.conv3d(grad_output, weight, None, stride + (1,), padding + (0,), dilation + (1,))
+        if ctx.needs_input_grad[1]:
+            # the weights of the convolution that runs backwards: its input is this layer's output
+            grad_weight = _weight_gradient(grad_output, weight.shape, input, stride, padding, dilation)
+            if grad_weight is None:
+                grad_weight = torch.nn.grad.conv3d_weight(grad_output, weight.shape, input, stride + (1,),
+                                                          padding + (0,), dilation + (1,), 1)
+        return grad_input, grad_weight, None, None, None
+
+
+def conv_transpose_synapse(input, weight, stride=1, padding=0, dilation=1, groups=1):
+    """``F.conv_transpose3d(input, weight, None, stride + (1,), padding + (0,), 0, groups, dilation + (1,))`` for an
+    NCHWT ``input`` and a ``weight`` of [Ci, Co / groups, kh, kw, 1], computed in place of the layout when the
+    kernels take the shape (one group, float32 on the GPU, at least four time steps, strides up to 16), by the
+    library call otherwise."""
+    stride, padding, dilation = _pair(stride, 'stride'), _pair(padding, 'padding'), _pair(dilation, 'dilation')
+    takes = (groups == 1 and input.is_cuda and input.dtype == torch.float32 and weight.dtype == torch.float32
+             and input.dim() == 5 and weight.dim() == 5 and weight.shape[-1] == 1 and input.shape[-1] >= 4
+             and input.numel() > 0 and max(stride) <= 16)
+    if takes:
+        _, co, kh, kw, _ = weight.shape
+        ho = (input.shape[2] - 1) * stride[0] - 2 * padding[0] + dilation[0] * (kh - 1) + 1
+        wo = (input.shape[3] - 1) * stride[1] - 2 * padding[1] + dilation[1] * (kw - 1) + 1
+        takes = (0 < ho <= 60000 and 0 < wo <= 60000 and input.shape[1] * kh * kw <= 4096
+                 and max(input[0].numel(), co * ho * wo * input.shape[-1]) * 4 < 2 ** 31)
+    if not takes:
+        return F.conv_transpose3d(input, weight, None, stride + (1,), padding + (0,), 0, groups, dilation + (1,))
+    return _ConvTransposeSynapse.apply(input.contiguous(), weight, stride, padding, dilation)
+
+
 class _SynapseLayer:
     """What the synapse layers share (GenericLayer, synapse/layer.py:15-69 in the reference): weight
     normalisation on demand, a pre-hook applied to the weight before every forward pass, ``shape``."""
@@ -156,6 +214,12 @@ class _SynapseLayer:
     def disable_weight_norm(self):
         torch.nn.utils.remove_weight_norm(self, name='weight')
         self.weight_norm_enabled = False
+
+    @property
+    def grad_norm(self):
+        """Norm of the weight gradient over its number of elements (0 before any backward pass)."""
+        grad = (self.weight_g if self.weight_norm_enabled else self.weight).grad
+        return 0 if grad is None else torch.norm(grad).item() / torch.numel(grad)
 
     @property
     def pre_hook_fx(self):
@@ -279,4 +343,60 @@ class Pool(torch.nn.Conv3d, _SynapseLayer):
         n, c, h, w, t = input.shape
         result = conv_synapse(input.reshape(n, 1, c * h, w, t), self._weight(), self._stride2, self._padding2,
                               self._dilation2)
+        return result.reshape(n, c, -1, result.shape[3], t)
+
+
+class ConvTranspose(torch.nn.ConvTranspose3d, _SynapseLayer):
+    """Transposed convolution synapse layer (synapse/layer.py:511-658 in the reference).
+
+    Parameters
+    ----------
+    in_features, out_features : int
+    kernel_size, stride, padding, dilation : int or (height, width)
+    groups : int
+    weight_scale, weight_norm, pre_hook_fx : as for :class:`Conv`.
+    """
+
+    def __init__(self, in_features, out_features, kernel_size, stride=1, padding=0, dilation=1, groups=1,
+                 weight_scale=1, weight_norm=False, pre_hook_fx=None):
+        kernel = _pair(kernel_size, 'kernel_size')
+        self._stride2, self._padding2, self._dilation2 = _pair(stride, 'stride'), _pair(padding, 'padding'), \
+            _pair(dilation, 'dilation')
+        super().__init__(in_features, out_features, kernel + (1,), self._stride2 + (1,), self._padding2 + (0,), 0,
+                         groups, False, self._dilation2 + (1,))
+        self._finish(weight_scale, weight_norm, pre_hook_fx)
+
+    def forward(self, input):
+        """Weighted spikes [N, out_features, Ho, Wo, T] for spikes [N, in_features, H, W, T],
+        Ho = (H - 1) stride - 2 padding + dilation (kh - 1) + 1."""
+        return conv_transpose_synapse(input, self._weight(), self._stride2, self._padding2, self._dilation2,
+                                      self.groups)
+
+
+class Unpool(torch.nn.ConvTranspose3d, _SynapseLayer):
+    """Unpooling synapse layer (synapse/layer.py:661-838 in the reference): every sample of a channel is spread
+    over a window of ``kernel_size`` with a common weight (``weight_scale``, not trained).  As in the reference
+    the channels are folded into the image height around a one-channel transposed convolution.
+
+    Parameters
+    ----------
+    kernel_size, stride, padding, dilation : int or (height, width); ``stride`` defaults to ``kernel_size``.
+    weight_scale, weight_norm, pre_hook_fx : as for :class:`Conv`.
+    """
+
+    def __init__(self, kernel_size, stride=None, padding=0, dilation=1, weight_scale=1, weight_norm=False,
+                 pre_hook_fx=None):
+        kernel = _pair(kernel_size, 'kernel_size')
+        self._stride2 = kernel if stride is None else _pair(stride, 'stride')
+        self._padding2, self._dilation2 = _pair(padding, 'padding'), _pair(dilation, 'dilation')
+        super().__init__(1, 1, kernel + (1,), self._stride2 + (1,), self._padding2 + (0,), 0, 1, False,
+                         self._dilation2 + (1,))
+        self.weight = torch.nn.Parameter(weight_scale * torch.ones_like(self.weight), requires_grad=False)
+        self._finish(1, weight_norm, pre_hook_fx)
+
+    def forward(self, input):
+        """Spread spikes [N, C, Ho, Wo, T] for spikes [N, C, H, W, T]."""
+        n, c, h, w, t = input.shape
+        result = conv_transpose_synapse(input.reshape(n, 1, c * h, w, t), self._weight(), self._stride2,
+                                        self._padding2, self._dilation2)
         return result.reshape(n, c, -1, result.shape[3], t)

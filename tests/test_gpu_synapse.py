@@ -200,3 +200,77 @@ def test_pool_layer(slayer, shape, kernel, stride, scale):
     want.backward(g.double())
     mag.backward(g.abs().double())
     assert_sum(xg.grad, xd.grad, xa.grad + 1e-30, 'gradient of the input')
+
+
+@pytest.mark.parametrize('shape,co,kernel,stride,padding,dilation', [
+    ((2, 5, 6, 7, 8), 3, (3, 3), (1, 1), (1, 1), (1, 1)),
+    ((1, 16, 17, 17, 300), 2, (5, 5), (2, 2), (2, 2), (1, 1)),      # what a decoder holds: few maps out of many
+    ((2, 8, 9, 9, 64), 16, (2, 2), (2, 2), (0, 0), (1, 1)),          # kernel = stride: every output has one term
+    ((2, 4, 6, 5, 101), 20, (3, 2), (1, 2), (0, 1), (2, 1)),
+    ((1, 3, 5, 6, 37), 7, (4, 4), (3, 3), (1, 1), (1, 1)),           # T % 4 = 1, stride 3
+    ((3, 6, 4, 4, 4), 5, (1, 1), (1, 1), (0, 0), (1, 1)),
+])
+def test_conv_transpose_synapse(slayer, shape, co, kernel, stride, padding, dilation):
+    """slayer.synapse.conv_transpose_synapse (the reference's F.conv_transpose3d call, synapse/layer.py:630-658)
+    on the convolution kernels with their roles exchanged: output and both gradients against float64 evaluation of
+    that call, every element to 1e-5 of the sum of the magnitudes of its terms."""
+    n, ci, h, w, t = shape
+    gen = torch.Generator().manual_seed(seed_of('conv-transpose', shape, co, kernel, stride, padding, dilation))
+    x = (torch.rand(shape, generator=gen) < 0.3).float() * torch.randn(shape, generator=gen)
+    wt = torch.randn(ci, co, kernel[0], kernel[1], 1, generator=gen)
+    xg, wg = x.to(dev()).requires_grad_(), wt.to(dev()).requires_grad_()
+    calls = []
+    plain = slayer.synapse.layer._launch_input_grad
+    slayer.synapse.layer._launch_input_grad = lambda *a: calls.append(1) or plain(*a)
+    try:
+        got = slayer.synapse.conv_transpose_synapse(xg, wg, stride, padding, dilation)
+    finally:
+        slayer.synapse.layer._launch_input_grad = plain
+    assert calls, 'the library call ran instead of the kernel'
+
+    def reference(a, b):
+        return F.conv_transpose3d(a, b, None, tuple(stride) + (1,), tuple(padding) + (0,), 0, 1, tuple(dilation) + (1,))
+
+    xd, wd = x.double().requires_grad_(), wt.double().requires_grad_()
+    xa, wa = x.abs().double().requires_grad_(), wt.abs().double().requires_grad_()
+    want, mag = reference(xd, wd), reference(xa, wa)
+    assert got.shape == want.shape and got.is_contiguous()
+    assert_sum(got, want.detach(), mag.detach() + 1e-30, 'forward')
+    g = torch.randn(want.shape, generator=gen)
+    got.backward(g.to(dev()))
+    want.backward(g.double())
+    mag.backward(g.abs().double())
+    assert_sum(xg.grad, xd.grad, xa.grad + 1e-30, 'grad input')
+    assert_sum(wg.grad, wd.grad, wa.grad + 1e-30, 'grad weight')
+
+
+def test_transposed_layers_mirror_the_reference_layers(slayer):
+    """ConvTranspose and Unpool (synapse/layer.py:511-838): module attributes, the weight pre-hook, the channels of
+    the unpooling layer folded into the height; what the kernels do not take goes to the library call."""
+    gen = torch.Generator().manual_seed(77)
+    quant = lambda v: (v * 8).round() / 8
+    up = slayer.synapse.ConvTranspose(6, 4, 3, stride=2, padding=1, weight_scale=2, pre_hook_fx=quant).to(dev())
+    assert tuple(up.shape) == (6, 4, 3, 3, 1) and up.bias is None and up.complex is False
+    x = torch.randn(2, 6, 5, 7, 24, generator=gen)
+    y = up(x.to(dev()))
+    want = F.conv_transpose3d(x.double(), quant(up.weight.detach().cpu()).double(), None, (2, 2, 1), (1, 1, 0))
+    assert y.shape == want.shape == (2, 4, 9, 13, 24)
+    assert float((y.cpu().double() - want).abs().max()) < 1e-4
+    grouped = slayer.synapse.ConvTranspose(6, 4, 3, groups=2).to(dev())         # groups: the library call
+    assert grouped(x.to(dev())).shape == (2, 4, 7, 9, 24)
+    assert slayer.synapse.ConvTranspose(6, 4, 3).to(dev())(x[..., :3].to(dev())).shape == (2, 4, 7, 9, 3)   # T < 4
+
+    unpool = slayer.synapse.Unpool(2, weight_scale=0.5).to(dev())
+    assert tuple(unpool.weight.shape) == (1, 1, 2, 2, 1) and not unpool.weight.requires_grad
+    xg = x.to(dev()).requires_grad_()
+    z = unpool(xg)
+    assert z.shape == (2, 6, 10, 14, 24)
+    # every sample spread over its own window of its own channel
+    assert torch.equal(z.detach().cpu(), 0.5 * x.repeat_interleave(2, 2).repeat_interleave(2, 3))
+    g = torch.randn(z.shape, generator=gen)
+    z.backward(g.to(dev()))
+    want = 0.5 * g.reshape(2, 6, 5, 2, 7, 2, 24).double().sum(dim=(3, 5))
+    assert float((xg.grad.cpu().double() - want).abs().max()) < 1e-5
+    pair = slayer.synapse.complex.ConvTranspose(6, 4, 3, stride=2).to(dev())
+    re, im = pair(x.to(dev()))
+    assert re.shape == im.shape == (2, 4, 11, 15, 24) and not torch.equal(re, im)

@@ -2,6 +2,7 @@
 the reference writes as a convolution whose kernel covers the whole input: against F.conv3d as the reference calls
 it, for the three ways of naming the input (neurons, (width, height), (width, height, channels)), with a weight
 pre-hook and weight normalisation, and the gradients through it."""
+import pytest
 import torch
 import torch.nn.functional as F
 
@@ -58,3 +59,54 @@ def test_pool_folds_the_channels_into_the_height_as_the_reference_does():
     # every output is the weighted sum of its own window of its own channel
     assert torch.allclose(pool(x)[1, 2, 1, 3], 1.5 * x[1, 2, 2:4, 6:8].sum(dim=(0, 1)))
     assert slayer.synapse.Pool((2, 3))(torch.randn(1, 2, 5, 7, 4, generator=gen)).shape == (1, 2, 3, 2, 4)
+
+
+def test_transposed_layers_are_the_references_calls():
+    """ConvTranspose and Unpool (synapse/layer.py:511-838 in the reference) on tensors the kernels do not take (CPU
+    here): F.conv_transpose3d as the reference calls it, the unpooling layer with its channels folded into the
+    height."""
+    gen = torch.Generator().manual_seed(8)
+    up = slayer.synapse.ConvTranspose(3, 5, (3, 2), stride=(2, 1), padding=(1, 0), dilation=(1, 2), weight_scale=3)
+    assert tuple(up.shape) == (3, 5, 3, 2, 1) and up.stride == (2, 1, 1) and up.padding == (1, 0, 0)
+    assert up.dilation == (1, 2, 1) and up.output_padding == (0, 0, 0) and up.bias is None
+    x = torch.randn(2, 3, 4, 5, 6, generator=gen)
+    want = F.conv_transpose3d(x, up.weight, None, (2, 1, 1), (1, 0, 0), 0, 1, (1, 2, 1))
+    assert torch.equal(up(x), want) and want.shape == (2, 5, 7, 7, 6)
+    unpool = slayer.synapse.Unpool(2, weight_scale=1.5)
+    assert not unpool.weight.requires_grad and float(unpool.weight.min()) == float(unpool.weight.max()) == 1.5
+    assert torch.allclose(unpool(x), 1.5 * x.repeat_interleave(2, 2).repeat_interleave(2, 3))
+    assert slayer.synapse.Unpool((2, 3))(x).shape == (2, 3, 8, 15, 6)
+    # a pooling layer after an unpooling layer of the same window: every sample times the window's size
+    assert torch.allclose(slayer.synapse.Pool(2)(slayer.synapse.Unpool(2)(x)), 4 * x)
+
+
+def test_complex_synapses_are_pairs_of_real_ones():
+    """synapse/complex.py in the reference: the same spikes through a real and an imaginary synapse."""
+    C = slayer.synapse.complex
+    gen = torch.Generator().manual_seed(9)
+    quant = lambda w: (w * 16).round() / 16
+    x = torch.randn(2, 4, 6, 6, 5, generator=gen)
+    cases = [(C.Dense(4, 3, pre_hook_fx=quant), torch.randn(2, 4, 7, generator=gen), slayer.synapse.Dense),
+             (C.Conv(4, 3, 3, padding=1, pre_hook_fx=quant), x, slayer.synapse.Conv),
+             (C.Pool(2, pre_hook_fx=quant), x, slayer.synapse.Pool),
+             (C.ConvTranspose(4, 3, 2, stride=2, pre_hook_fx=quant), x, slayer.synapse.ConvTranspose),
+             (C.Unpool(2, pre_hook_fx=quant), x, slayer.synapse.Unpool)]
+    for pair, inp, kind in cases:
+        assert pair.complex is True and isinstance(pair.real, kind) and isinstance(pair.imag, kind)
+        assert pair.real.weight is not pair.imag.weight and pair.shape == pair.real.shape
+        assert pair.pre_hook_fx is quant
+        re, im = pair(inp)
+        assert torch.equal(re, pair.real(inp)) and torch.equal(im, pair.imag(inp))
+        assert len(list(pair.parameters())) == 2
+    pair = C.Conv(4, 3, 3, weight_norm=True)
+    assert pair.real.weight_norm_enabled and pair.imag.weight_norm_enabled and pair.grad_norm == 0
+    re, im = pair(x)
+    (re.sum() + 2 * im.sum()).backward()
+    assert pair.grad_norm > 0 and abs(pair.grad_norm ** 2 - pair.real.grad_norm ** 2 - pair.imag.grad_norm ** 2) < 1e-12
+    pair.disable_weight_norm()
+    assert not pair.real.weight_norm_enabled
+    pair.real.pre_hook_fx = quant
+    with pytest.raises(Exception, match='must be same'):
+        pair.pre_hook_fx
+    pair.pre_hook_fx = None
+    assert pair.real.pre_hook_fx is None and pair.imag.pre_hook_fx is None
