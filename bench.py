@@ -739,6 +739,46 @@ class ConvSynapseLibrary(ConvSynapse):
         return torch.nn.grad.conv3d_input(self.s.shape, self.wgt, g, (1, 1, 1), (1, 1, 0))
 
 
+class PoolSynapse(Workload):
+    """The pooling synapse behind config[1]'s spikes (synapse/layer.py:326-510 in the reference: the channels folded
+    into the image height, a one-channel F.conv3d with a constant 2x2 kernel and stride 2), forward and the gradient
+    of its input.  Nothing to contract: one thread per quad of steps on the vector units.  Bytes per sample of the
+    layer's input tensor: the forward pass reads it and writes a quarter of it, the backward pass the reverse."""
+    name = 'Pool synapse 2x2 on the spikes of the conv-layer tensor, fwd + input gradient'
+    shape = (32, 16, 32, 32, 300)
+    ops = [('pool_synapse', 'synapse_plane_kernel<false>', 5), ('pool_synapse_bwd', 'synapse_plane_kernel<true>', 5)]
+    note = 'input spikes Bernoulli(0.05), weight 1.0, upstream gradient N(0, 1)'
+
+    def __init__(self, dev):
+        super().__init__(dev, 1007)
+        import importlib
+        g = self.gen
+        n, c, h, w, t = self.shape
+        self.put(s=(torch.rand(self.shape, generator=g) < 0.05).float(),
+                 g=torch.randn(n, c, h // 2, w // 2, t, generator=g), wgt=torch.ones(1, 1, 2, 2))
+        self.syn = importlib.import_module('lava_dl_amd.slayer.synapse.layer')
+        self.folded = (n, 1, c * h, w, t)
+
+    def step(self, t):
+        n, c, h, w, steps = self.shape
+        with t('pool_synapse'):
+            y = self.syn._launch(self.s.view(self.folded), self.wgt, (2, 2), (0, 0), (1, 1))
+        with t('pool_synapse_bwd'):
+            g_s = self.syn._launch_input_grad(self.g.view(n, 1, c * h // 2, w // 2, steps), self.wgt, self.folded,
+                                              (2, 2), (0, 0), (1, 1))
+        return y.view(n, c, h // 2, w // 2, steps), g_s.view(self.shape)
+
+    def cpu_step(self, n, sl=None):
+        c = self.cpu
+        s, g = c['s'][:n].double(), c['g'][:n].double()
+        y = s[:, :, 0::2, 0::2] + s[:, :, 0::2, 1::2] + s[:, :, 1::2, 0::2] + s[:, :, 1::2, 1::2]
+        g_s = g.repeat_interleave(2, 2).repeat_interleave(2, 3)
+        sl = slice(None) if sl is None else sl
+        return y[:, sl].float(), g_s[:, sl].float()
+
+    parity_slab = (2, slice(0, 16))
+
+
 class DenseSynapse(Workload):
     """Dense synapse (the reference's 1x1x1 conv3d over [N, C, 1, 1, T], synapse/layer.py:144-175, written as the
     batched GEMM it is) feeding the fused CUBA kernel, forward only: the kernel list of this workload shows what runs
@@ -851,7 +891,7 @@ class RecurrentLoop(Recurrent):
 
 
 WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fused_lean': CubaFusedLean, 'cuba_inference': CubaInference, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'alif_fused': AlifFused, 'alif_fused_lean': AlifFusedLean, 'rf': Rf, 'rf_fused': RfFused, 'rf_fused_lean': RfFusedLean, 'rf_inference': RfInference, 'synapse': Synapse, 'synapse_fused': SynapseFused, 'synapse_folded': SynapseFolded, 'synapse_delay_grad': SynapseDelayGrad, 'block_tail': BlockTail, 'block_tail_folded': BlockTailFolded,
-             'conv_synapse': ConvSynapse, 'conv_synapse_library': ConvSynapseLibrary,
+             'conv_synapse': ConvSynapse, 'conv_synapse_library': ConvSynapseLibrary, 'pool_synapse': PoolSynapse,
              'dense_synapse': DenseSynapse, 'recurrent': Recurrent, 'recurrent_loop': RecurrentLoop}
 
 
@@ -935,7 +975,7 @@ def timed_median(job, iters, warmup):
 # sequence of the configuration, then the fused forms with their own smaller byte counts).
 OTHER = ['cuba_fwd_small', 'cuba_fused', 'cuba_fused_lean', 'alif', 'alif_fused', 'alif_fused_lean', 'rf', 'rf_fused',
          'synapse', 'synapse_fused', 'synapse_folded', 'synapse_delay_grad', 'block_tail', 'block_tail_folded',
-         'conv_synapse', 'conv_synapse_library', 'recurrent', 'recurrent_loop']
+         'conv_synapse', 'conv_synapse_library', 'pool_synapse', 'recurrent', 'recurrent_loop']
 
 
 def other_configs(dev, iters):

@@ -297,27 +297,43 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_row_kernel(con
 // One input and one output channel (the pooling layers, which fold their channels into the image height,
 // synapse/layer.py:438-508 and :770-838 in the reference): there is no contraction for the matrix cores, and a wave
 // that owns 16 channels x 64 steps of one pixel would move 256 bytes per instruction.  One thread per quad of output
-// steps on the vector units instead: a block row of the grid is an image row of the output, grid.z the batch.
+// steps on the vector units instead: a block row of the grid is ROWS image rows of the output, grid.z the batch.
 // SPREAD: the gradient of the input (the unpooling layer's forward pass): output pixel (h, w) sums the taps (y, x)
-// whose source coordinates (h + ph - y dh) / sh, (w + pw - x dw) / sw are exact; which taps those are, and the
-// quotients less h / sh, depend on h mod sh alone and come from a table in LDS (quot_y[ry * kh + y], likewise x).
+// whose source coordinates (h + ph - y dh) / sh, (w + pw - x dw) / sw are exact.  Which taps those are depends on
+// h mod sh alone: a table in LDS lists them per residue (at most ny per residue: tap_y, and quot_y = the quotient
+// less h / sh; likewise nx, tap_x, quot_x), so that a pixel visits ny * nx slots -- one for a pooling window that is
+// as large as its stride -- instead of all kh * kw taps.
 constexpr int kPlaneThreads = 256;
-template <bool SPREAD, bool STREAM, bool TAIL>
-__global__ __launch_bounds__(kPlaneThreads) void synapse_plane_kernel(const SynapseConv p, int quads, int rows) {
+#ifndef SLAYER_PLANE_ROWS_SUM
+#define SLAYER_PLANE_ROWS_SUM 1
+#endif
+#ifndef SLAYER_PLANE_ROWS_SPREAD
+#define SLAYER_PLANE_ROWS_SPREAD 8
+#endif
+constexpr int kPlaneRowsSum = SLAYER_PLANE_ROWS_SUM, kPlaneRowsSpread = SLAYER_PLANE_ROWS_SPREAD;
+template <bool SPREAD, bool STREAM, bool TAIL, int ROWS>
+__global__ __launch_bounds__(kPlaneThreads) void synapse_plane_kernel(const SynapseConv p, int quads, int ny, int nx) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     float* wt = lds;                                                      // [kh * kw]
-    int* quot_y = reinterpret_cast<int*>(lds + p.kh * p.kw);              // SPREAD: [sh * kh]
-    int* quot_x = quot_y + p.sh * p.kh;                                   // SPREAD: [sw * kw]
+    int* quot_y = reinterpret_cast<int*>(lds + p.kh * p.kw);              // SPREAD: [sh * ny]
+    int* tap_y = quot_y + p.sh * ny;                                      //         [sh * ny], times kw
+    int* quot_x = tap_y + p.sh * ny;                                      //         [sw * nx]
+    int* tap_x = quot_x + p.sw * nx;                                      //         [sw * nx]
     const int none = 1 << 28;
     for (int i = threadIdx.x; i < p.kh * p.kw; i += kPlaneThreads) wt[i] = p.weight[i];
     if (SPREAD) {
-        for (int i = threadIdx.x; i < p.sh * p.kh; i += kPlaneThreads) {
-            const int c = i / p.kh + p.ph - (i % p.kh) * p.dh;
-            quot_y[i] = c % p.sh == 0 ? c / p.sh : none;
-        }
-        for (int i = threadIdx.x; i < p.sw * p.kw; i += kPlaneThreads) {
-            const int c = i / p.kw + p.pw - (i % p.kw) * p.dw;
-            quot_x[i] = c % p.sw == 0 ? c / p.sw : none;
+        for (int r = threadIdx.x; r < p.sh + p.sw; r += kPlaneThreads) {
+            const bool rows = r < p.sh;
+            const int res = rows ? r : r - p.sh, k = rows ? p.kh : p.kw, stride = rows ? p.sh : p.sw;
+            const int pad = rows ? p.ph : p.pw, dil = rows ? p.dh : p.dw, slots = rows ? ny : nx;
+            int* quot = (rows ? quot_y : quot_x) + res * slots;
+            int* tap = (rows ? tap_y : tap_x) + res * slots;
+            int found = 0;
+            for (int y = 0; y < k; ++y) {
+                const int c = res + pad - y * dil;
+                if (c % stride == 0) { quot[found] = c / stride; tap[found] = rows ? y * p.kw : y; ++found; }
+            }
+            for (; found < slots; ++found) { quot[found] = none; tap[found] = 0; }
         }
     }
     __syncthreads();
@@ -327,31 +343,52 @@ __global__ __launch_bounds__(kPlaneThreads) void synapse_plane_kernel(const Syna
     const bool on = wo < p.Wo;
     SynQuad tq;
     tq.template set<TAIL>(4 * j, p.T);
+    const bool lane_on = on && tq.any();
     const int64_t in_plane = (int64_t)p.H * p.W * p.T;
     const __amdgpu_buffer_rsrc_t src = make_rsrc(p.in + (int64_t)n * in_plane, (unsigned)(in_plane * 4));
     const int64_t out_plane = (int64_t)p.Ho * p.Wo * p.T;
     const __amdgpu_buffer_rsrc_t dst = make_rsrc(p.out + (int64_t)n * out_plane, (unsigned)(out_plane * 4));
-    // SPREAD: the pixel as quotient and residue of the strides (the row's are the same for the whole block)
+    // SPREAD: the pixel as quotient and residue of the strides (the rows' are the same for the whole block)
     const int wq = SPREAD ? wo / p.sw : 0, rx = SPREAD ? (on ? wo - wq * p.sw : 0) : 0;
-    // a block takes `rows` image rows one after the other: the tables above are set up once for all of them
-    for (int ho = blockIdx.y * rows; ho < p.Ho && ho < (blockIdx.y + 1) * rows; ++ho) {
-        const int hq = SPREAD ? ho / p.sh : 0, ry = SPREAD ? ho - hq * p.sh : 0;
-        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-        for (int y = 0; y < p.kh; ++y) {
-            const int yy = SPREAD ? hq + quot_y[ry * p.kh + y] : ho * p.sh + y * p.dh - p.ph;
-            if ((unsigned)yy >= (unsigned)p.H) continue;                  // the same for the whole block
-            for (int x = 0; x < p.kw; ++x) {
-                const int xx = SPREAD ? wq + quot_x[rx * p.kw + x] : wo * p.sw + x * p.dw - p.pw;
-                const bool ok = on && tq.any() && (unsigned)xx < (unsigned)p.W;
-                const float4 q = tq.template place<TAIL>(
-                    buf_load4<false>(src, ok ? ((yy * p.W + xx) * p.T + tq.t_load) * 4 : kOutOfRange));
-                const float f = wt[y * p.kw + x];
-                acc.x = __fmaf_rn(f, q.x, acc.x); acc.y = __fmaf_rn(f, q.y, acc.y);
-                acc.z = __fmaf_rn(f, q.z, acc.z); acc.w = __fmaf_rn(f, q.w, acc.w);
+    // A block takes ROWS image rows at once: the tables above are set up once for all of them, and a slot is
+    // loaded for all the rows before the first product waits for it.
+    const int ho0 = blockIdx.y * ROWS;
+    int hq[ROWS], ry[ROWS];
+    float4 acc[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        hq[r] = SPREAD ? (ho0 + r) / p.sh : 0;
+        ry[r] = SPREAD ? (ho0 + r < p.Ho ? ho0 + r - hq[r] * p.sh : 0) : 0;
+        acc[r] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    for (int y = 0; y < (SPREAD ? ny : p.kh); ++y) {
+        int row_off[ROWS], w_row[ROWS];                                   // source row of this slot or none, its weights
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            const int yy = SPREAD ? hq[r] + quot_y[ry[r] * ny + y] : (ho0 + r) * p.sh + y * p.dh - p.ph;
+            row_off[r] = (ho0 + r < p.Ho && (unsigned)yy < (unsigned)p.H) ? yy * p.W : -1;
+            w_row[r] = SPREAD ? tap_y[ry[r] * ny + y] : y * p.kw;
+        }
+        for (int x = 0; x < (SPREAD ? nx : p.kw); ++x) {
+            const int xx = SPREAD ? wq + quot_x[rx * nx + x] : wo * p.sw + x * p.dw - p.pw;
+            const int w_col = SPREAD ? tap_x[rx * nx + x] : x;
+            const bool ok = lane_on && (unsigned)xx < (unsigned)p.W;
+            float4 q[ROWS];
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r)
+                q[r] = buf_load4<false>(src, (ok && row_off[r] >= 0) ? ((row_off[r] + xx) * p.T + tq.t_load) * 4 : kOutOfRange);
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) {
+                const float f = wt[w_row[r] + w_col];
+                const float4 v = tq.template place<TAIL>(q[r]);
+                acc[r].x = __fmaf_rn(f, v.x, acc[r].x); acc[r].y = __fmaf_rn(f, v.y, acc[r].y);
+                acc[r].z = __fmaf_rn(f, v.z, acc[r].z); acc[r].w = __fmaf_rn(f, v.w, acc[r].w);
             }
         }
-        syn_store_quad<STREAM, TAIL>(dst, on, ((ho * p.Wo + wo) * p.T + 4 * j) * 4, tq.nv, acc);
     }
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r)
+        syn_store_quad<STREAM, TAIL>(dst, on && ho0 + r < p.Ho, (((ho0 + r) * p.Wo + wo) * p.T + 4 * j) * 4, tq.nv, acc[r]);
 }
 
 // Gradient of the weights: grad_w[co][k] = sum over batch, output pixels and time of grad_out[co][pixel][t] *
@@ -746,6 +783,17 @@ int launch_synapse_conv(SynapseConv p, bool streaming, hipStream_t st) {
     return (int)hipGetLastError();
 }
 
+// the most taps of a filter row of k taps that pixels of one residue (mod stride) meet in a transposed convolution
+int most_taps_per_residue(int k, int stride, int pad, int dil) {
+    int most = 0;
+    for (int r = 0; r < stride; ++r) {
+        int found = 0;
+        for (int y = 0; y < k; ++y) found += (r + pad - y * dil) % stride == 0;
+        most = found > most ? found : most;
+    }
+    return most;
+}
+
 // The one-channel form (synapse_plane_kernel) for a plain convolution (spread = false: p as for
 // launch_synapse_conv) or for the gradient of its input (spread = true: p.in the gradient of the output [H][W],
 // p.out the gradient of the input [Ho][Wo], strides, padding and dilation those of the convolution).
@@ -753,16 +801,17 @@ int launch_synapse_conv(SynapseConv p, bool streaming, hipStream_t st) {
 bool launch_synapse_plane(const SynapseConv& p, bool spread, bool streaming, hipStream_t st, int* code) {
     const int64_t quads = (p.T + 3) / 4;
     const int64_t blocks = ((int64_t)p.Wo * quads + kPlaneThreads - 1) / kPlaneThreads;
-    const size_t lds = ((size_t)p.kh * p.kw + (spread ? (size_t)p.sh * p.kh + (size_t)p.sw * p.kw : 0)) * 4;
-    if (p.Ci != 1 || p.Co != 1 || p.N > 65535 || blocks > 0x7fffffffLL || p.kh * p.kw > 1024 ||
-        lds > 48 * 1024)
-        return false;
-    // measured on [32,16,32,32,300] with 2x2 windows: the sums 136 us a row at a time (142 at two, 150 at four), the
-    // spread form 227 us a row at a time, 129 at four, 121 at eight, 123 at sixteen
-    const int rows = spread ? 8 : 1;
+    if (p.Ci != 1 || p.Co != 1 || p.N > 65535 || blocks > 0x7fffffffLL || p.kh * p.kw > 1024) return false;
+    const int ny = spread ? most_taps_per_residue(p.kh, p.sh, p.ph, p.dh) : 0;
+    const int nx = spread ? most_taps_per_residue(p.kw, p.sw, p.pw, p.dw) : 0;
+    const size_t lds = ((size_t)p.kh * p.kw + 2 * ((size_t)p.sh * ny + (size_t)p.sw * nx)) * 4;
+    if (lds > 48 * 1024) return false;
+    const int rows = spread ? kPlaneRowsSpread : kPlaneRowsSum;
     const dim3 grid((unsigned)blocks, (unsigned)((p.Ho + rows - 1) / rows), (unsigned)p.N), block(kPlaneThreads);
     const bool tail = (p.T % 4) != 0;
-#define SLAYER_SYN_PLANE(SP, S, TL) hipLaunchKernelGGL((synapse_plane_kernel<SP, S, TL>), grid, block, lds, st, p, (int)quads, rows)
+#define SLAYER_SYN_PLANE(SP, S, TL)                                                                                      \
+    hipLaunchKernelGGL((synapse_plane_kernel<SP, S, TL, (SP ? kPlaneRowsSpread : kPlaneRowsSum)>), grid, block, lds, st, p, \
+                       (int)quads, ny, nx)
 #define SLAYER_SYN_PLANE_T(SP, S) do { if (tail) SLAYER_SYN_PLANE(SP, S, true); else SLAYER_SYN_PLANE(SP, S, false); } while (0)
     if (spread) { if (streaming) SLAYER_SYN_PLANE_T(true, true); else SLAYER_SYN_PLANE_T(true, false); }
     else { if (streaming) SLAYER_SYN_PLANE_T(false, true); else SLAYER_SYN_PLANE_T(false, false); }

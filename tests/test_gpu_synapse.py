@@ -63,6 +63,15 @@ def _check(slayer, shape, co, kernel, stride, padding, dilation, what, backward=
     ((3, 5, 4, 4, 4), 2, (1, 1), (1, 1), (0, 0), (1, 1)),
     ((1, 7, 8, 8, 36), 20, (5, 3), (1, 1), (2, 1), (1, 1)),         # 35 pairs: two tiles and a second pass; kw = 3, kh = 5
     ((1, 7, 8, 8, 36), 20, (3, 5), (1, 1), (1, 2), (1, 1)),         # kw = 5, kh = 3
+    # strides whose residue classes differ in their taps (the input gradient is one convolution per class): a common
+    # factor of stride and dilation, a stride beyond the kernel, a stride of 3 under 5 taps, strides of 16
+    ((2, 3, 11, 11, 20), 4, (3, 3), (2, 2), (1, 1), (2, 2)),
+    ((1, 4, 17, 12, 24), 6, (3, 2), (4, 4), (2, 0), (6, 2)),
+    ((2, 2, 14, 17, 12), 3, (2, 2), (3, 5), (0, 1), (1, 1)),
+    ((1, 5, 16, 16, 44), 16, (5, 5), (3, 3), (2, 2), (1, 1)),
+    ((1, 2, 40, 36, 8), 3, (3, 3), (16, 16), (1, 1), (1, 1)),
+    ((2, 1, 13, 12, 30), 1, (3, 3), (2, 2), (1, 1), (1, 1)),        # one channel in and out: the vector-unit kernel
+    ((1, 1, 9, 9, 21), 1, (2, 3), (1, 2), (1, 0), (2, 1)),
 ])
 def test_conv_synapse_against_the_oracle(slayer, shape, co, kernel, stride, padding, dilation):
     _check(slayer, shape, co, kernel, stride, padding, dilation, f'{shape} -> {co}')
@@ -209,6 +218,14 @@ def test_pool_layer(slayer, shape, kernel, stride, scale):
     ((2, 4, 6, 5, 101), 20, (3, 2), (1, 2), (0, 1), (2, 1)),
     ((1, 3, 5, 6, 37), 7, (4, 4), (3, 3), (1, 1), (1, 1)),           # T % 4 = 1, stride 3
     ((3, 6, 4, 4, 4), 5, (1, 1), (1, 1), (0, 0), (1, 1)),
+    # residue classes of the output pixels that differ in their taps: stride and dilation with a common factor
+    # (every other class meets no tap at all), a stride beyond the kernel (classes without taps, rows of zeros),
+    # a stride of 3 under 5 taps (classes of two taps and of one)
+    ((2, 3, 5, 5, 20), 4, (3, 3), (2, 2), (1, 1), (2, 2)),
+    ((1, 4, 4, 5, 24), 6, (3, 2), (4, 4), (2, 0), (6, 2)),
+    ((2, 2, 6, 4, 12), 3, (2, 2), (3, 5), (0, 1), (1, 1)),
+    ((1, 5, 6, 6, 44), 16, (5, 5), (3, 3), (2, 2), (1, 1)),
+    ((2, 1, 7, 6, 30), 1, (3, 3), (2, 2), (1, 1), (1, 1)),          # one channel in and out: the vector-unit kernel
 ])
 def test_conv_transpose_synapse(slayer, shape, co, kernel, stride, padding, dilation):
     """slayer.synapse.conv_transpose_synapse (the reference's F.conv_transpose3d call, synapse/layer.py:630-658)
