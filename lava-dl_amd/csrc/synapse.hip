@@ -744,6 +744,11 @@ namespace {
 // one-pixel kernel with as many tap groups in flight as the filter has, up to six.  A filter without taps (K = 0)
 // clears its outputs.
 int launch_synapse_conv(SynapseConv p, bool streaming, hipStream_t st) {
+    // Non-temporal stores only for the classes of a transposed convolution, which leave every line they touch
+    // unfinished for the next launch.  A plain convolution finishes the lines that two of its tiles share within
+    // microseconds, and the L2 puts the pieces together if it is allowed to keep them: [32,8,32,32,300] -> 16 channels
+    // forward 378 -> 329 us with cached stores (the transposed 4x4 stride-2 classes 251 -> 288 us).
+    if (p.oys == 1 && p.oxs == 1) streaming = false;
     constexpr int kRowPix = SLAYER_SYN_PIX;
     const int64_t K = (int64_t)p.Ci * p.kh * p.kw;
     p.K = (int)K;
