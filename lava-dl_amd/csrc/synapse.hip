@@ -209,7 +209,8 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_kernel(const S
 // LDS: weights as above (tap k = pair * KW + x, pair = ci * kh + y), and per pair the byte offset of its input row
 // relative to the pixel block's own position and its row displacement.
 template <int KW, int PIX, bool STREAM, bool TAIL>
-__global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_row_kernel(const SynapseConv p) {
+__global__ __launch_bounds__(kSynWaves * kWave) __attribute__((amdgpu_waves_per_eu(5)))
+void synapse_conv_row_kernel(const SynapseConv p) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int PG = p.KG;                                // groups of four pairs
     const int Kp = PG * 4 * KW;
