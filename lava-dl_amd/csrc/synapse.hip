@@ -209,8 +209,7 @@ __global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_kernel(const S
 // LDS: weights as above (tap k = pair * KW + x, pair = ci * kh + y), and per pair the byte offset of its input row
 // relative to the pixel block's own position and its row displacement.
 template <int KW, int PIX, bool STREAM, bool TAIL>
-__global__ __launch_bounds__(kSynWaves * kWave) __attribute__((amdgpu_waves_per_eu(5)))
-void synapse_conv_row_kernel(const SynapseConv p) {
+__device__ __forceinline__ void synapse_conv_row(const SynapseConv& p) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int PG = p.KG;                                // groups of four pairs
     const int Kp = PG * 4 * KW;
@@ -304,6 +303,16 @@ void synapse_conv_row_kernel(const SynapseConv p) {
             }
         }
     }
+}
+
+// Rows of whole quads at five waves per SIMD (88 registers, no spills; four waves otherwise: 2-3 % slower); the
+// forms for rows that end inside a quad need a few registers more and keep the compiler's own choice.
+template <int KW, int PIX, bool STREAM>
+__global__ __launch_bounds__(kSynWaves * kWave) __attribute__((amdgpu_waves_per_eu(5)))
+void synapse_conv_row_kernel(const SynapseConv p) { synapse_conv_row<KW, PIX, STREAM, false>(p); }
+template <int KW, int PIX, bool STREAM>
+__global__ __launch_bounds__(kSynWaves * kWave) void synapse_conv_row_tail_kernel(const SynapseConv p) {
+    synapse_conv_row<KW, PIX, STREAM, true>(p);
 }
 
 // One input and one output channel (the pooling layers, which fold their channels into the image height,
@@ -774,12 +783,13 @@ int launch_synapse_conv(SynapseConv p, bool streaming, hipStream_t st) {
         p.KG = (p.Ci * p.kh + 3) / 4;                                     // groups of four (channel, kernel row) pairs
         const size_t lds = (size_t)p.KG * 4 * (p.kw * 16 * sizeof(float) + 2 * sizeof(int));
         if (lds > 64 * 1024) return SLAYER_ERANGE;
-#define SLAYER_SYN_ROW_T(KW, TL)                                                                                         \
-        do {                                                                                                            \
-            if (streaming) hipLaunchKernelGGL((synapse_conv_row_kernel<KW, kRowPix, true, TL>), grid, block, lds, st, p); \
-            else hipLaunchKernelGGL((synapse_conv_row_kernel<KW, kRowPix, false, TL>), grid, block, lds, st, p);         \
+#define SLAYER_SYN_ROW_T(KERNEL, KW)                                                                      \
+        do {                                                                                             \
+            if (streaming) hipLaunchKernelGGL((KERNEL<KW, kRowPix, true>), grid, block, lds, st, p);      \
+            else hipLaunchKernelGGL((KERNEL<KW, kRowPix, false>), grid, block, lds, st, p);               \
         } while (0)
-#define SLAYER_SYN_ROW(KW) do { if (tail) SLAYER_SYN_ROW_T(KW, true); else SLAYER_SYN_ROW_T(KW, false); } while (0)
+#define SLAYER_SYN_ROW(KW)                                                                                \
+        do { if (tail) SLAYER_SYN_ROW_T(synapse_conv_row_tail_kernel, KW); else SLAYER_SYN_ROW_T(synapse_conv_row_kernel, KW); } while (0)
         if (p.kw == 2) SLAYER_SYN_ROW(2); else if (p.kw == 3) SLAYER_SYN_ROW(3); else SLAYER_SYN_ROW(5);
 #undef SLAYER_SYN_ROW_T
 #undef SLAYER_SYN_ROW
