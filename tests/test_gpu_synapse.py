@@ -291,3 +291,51 @@ def test_transposed_layers_mirror_the_reference_layers(slayer):
     pair = slayer.synapse.complex.ConvTranspose(6, 4, 3, stride=2).to(dev())
     re, im = pair(x.to(dev()))
     assert re.shape == im.shape == (2, 4, 11, 15, 24) and not torch.equal(re, im)
+
+
+def test_synapse_kernels_under_graph_capture_replays(slayer):
+    """The synapse entry points enqueue kernels only (the weight gradient clears nothing with a memset, its
+    workspace comes from the caller), so a training step of a convolution and a pooling layer can be captured in a
+    graph; every replay, with eager work in between, must equal the eager result bit for bit."""
+    L = slayer.synapse.layer
+    gen = torch.Generator().manual_seed(seed_of('synapse graph'))
+    x = torch.zeros(2, 3, 8, 8, 40, device=dev())
+    g = torch.zeros(2, 5, 4, 4, 40, device=dev())
+    w = torch.randn(5, 3, 3, 3, 1, generator=gen).to(dev())
+    pool_w = torch.ones(1, 1, 2, 2, device=dev())
+
+    def fill():
+        x.copy_(((torch.rand(x.shape, generator=gen) < 0.3).float() * torch.randn(x.shape, generator=gen)).to(dev()))
+        g.copy_(torch.randn(g.shape, generator=gen).to(dev()))
+
+    def step():
+        w4 = w[..., 0].contiguous()
+        z = L._launch(x, w4, (2, 2), (1, 1), (1, 1))                               # strided convolution
+        g_x = L._launch_input_grad(g, w4.transpose(0, 1).contiguous(), x.shape, (2, 2), (1, 1), (1, 1))
+        g_w = L._weight_gradient(x, w.shape, g, (2, 2), (1, 1), (1, 1))
+        n, c, h, wd, t = z.shape
+        pooled = L._launch(z.view(n, 1, c * h, wd, t), pool_w, (2, 2), (0, 0), (1, 1))
+        spread = L._launch_input_grad(pooled, pool_w, (n, 1, c * h, wd, t), (2, 2), (0, 0), (1, 1))
+        return z, g_x, g_w, pooled, spread
+
+    fill()
+    step()                                      # warm-up outside the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        step()
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            outs = step()
+    torch.cuda.synchronize()
+    for k in range(3):
+        fill()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in outs]
+        want = step()                           # eager work between the replays
+        torch.cuda.synchronize()
+        assert float(want[0].abs().sum()) > 0 and float(want[2].abs().sum()) > 0
+        for i, (a, b) in enumerate(zip(got, want)):
+            assert torch.equal(a, b), f'replay {k}: output {i} differs from the eager result'
