@@ -779,6 +779,53 @@ class PoolSynapse(Workload):
     parity_slab = (2, slice(0, 16))
 
 
+class ConvTransposeSynapse(Workload):
+    """A decoder stage (synapse/layer.py:511-658 in the reference: F.conv_transpose3d with a 4x4x1 kernel, stride 2,
+    padding 1 on NCHWT spikes): 16 maps of 16x16 to 8 maps of 32x32, forward and both gradients.  One plain
+    convolution per residue class of the output pixels (four launches forward), the strided convolution kernel for
+    the input gradient, the weight-gradient kernels with input and output exchanged.  Weights are multiples of 1/64,
+    so the forward result is exact.  Bytes per sample of the layer's output tensor (4 written + 8 read forward, 4
+    read + 8 written for the input gradient, 12 read for the weight gradient: output 8 channels, input 16 at a
+    quarter of the pixels)."""
+    name = 'ConvTranspose synapse 4x4 stride 2, 16 -> 8 channels, 16x16 -> 32x32, fwd + input and weight gradients'
+    shape = (32, 8, 32, 32, 300)
+    ops = [('conv_transpose', 'synapse_conv_row_kernel<2> x 4 residue classes', 6), ('conv_transpose_bwd', 'synapse_conv_kernel (stride 2)', 6),
+           ('conv_transpose_wgrad', 'synapse_wgrad_kernel', 6)]
+    note = 'input spikes Bernoulli(0.05) on 16 channels of 16x16, weights round(N(0, 0.3) * 64) / 64, upstream gradient N(0, 1)'
+
+    def __init__(self, dev):
+        super().__init__(dev, 1008)
+        import importlib
+        g = self.gen
+        n, co, h, w, t = self.shape
+        self.put(s=(torch.rand(n, 16, h // 2, w // 2, t, generator=g) < 0.05).float(),
+                 wgt=(torch.randn(16, co, 4, 4, 1, generator=g) * 0.3 * 64).round() / 64,
+                 g=torch.randn(self.shape, generator=g))
+        self.syn = importlib.import_module('lava_dl_amd.slayer.synapse.layer')
+        self.w4 = self.wgt[..., 0].contiguous()                      # [Ci, Co, kh, kw]: the backward convolution's weights
+        self.w4_t = self.wgt[..., 0].transpose(0, 1).contiguous()    # channel axes exchanged for the class launches
+
+    def step(self, t):
+        cfg = ((2, 2), (1, 1), (1, 1))
+        with t('conv_transpose'):
+            y = self.syn._launch_input_grad(self.s, self.w4_t, self.shape, *cfg)
+        with t('conv_transpose_bwd'):
+            g_s = self.syn._launch(self.g, self.w4, *cfg)
+        with t('conv_transpose_wgrad'):
+            self.g_w = self.syn._weight_gradient(self.g, self.wgt.shape, self.s, *cfg)
+        return y, g_s
+
+    def cpu_step(self, n, sl=None):
+        c = self.cpu
+        F = torch.nn.functional
+        y = F.conv_transpose3d(c['s'][:n].double(), c['wgt'].double(), None, (2, 2, 1), (1, 1, 0))
+        g_s = F.conv3d(c['g'][:n].double(), c['wgt'].double(), None, (2, 2, 1), (1, 1, 0))
+        sl = slice(None) if sl is None else sl
+        return y[:, sl].float(), g_s[:, sl].float()
+
+    parity_slab = (1, slice(0, 8))
+
+
 class DenseSynapse(Workload):
     """Dense synapse (the reference's 1x1x1 conv3d over [N, C, 1, 1, T], synapse/layer.py:144-175, written as the
     batched GEMM it is) feeding the fused CUBA kernel, forward only: the kernel list of this workload shows what runs
@@ -891,7 +938,7 @@ class RecurrentLoop(Recurrent):
 
 
 WORKLOADS = {'cuba': Cuba, 'cuba_fused': CubaFused, 'cuba_fused_lean': CubaFusedLean, 'cuba_inference': CubaInference, 'cuba_fwd_small': CubaFwdSmall, 'alif': Alif, 'alif_fused': AlifFused, 'alif_fused_lean': AlifFusedLean, 'rf': Rf, 'rf_fused': RfFused, 'rf_fused_lean': RfFusedLean, 'rf_inference': RfInference, 'synapse': Synapse, 'synapse_fused': SynapseFused, 'synapse_folded': SynapseFolded, 'synapse_delay_grad': SynapseDelayGrad, 'block_tail': BlockTail, 'block_tail_folded': BlockTailFolded,
-             'conv_synapse': ConvSynapse, 'conv_synapse_library': ConvSynapseLibrary, 'pool_synapse': PoolSynapse,
+             'conv_synapse': ConvSynapse, 'conv_synapse_library': ConvSynapseLibrary, 'pool_synapse': PoolSynapse, 'conv_transpose_synapse': ConvTransposeSynapse,
              'dense_synapse': DenseSynapse, 'recurrent': Recurrent, 'recurrent_loop': RecurrentLoop}
 
 
@@ -975,7 +1022,7 @@ def timed_median(job, iters, warmup):
 # sequence of the configuration, then the fused forms with their own smaller byte counts).
 OTHER = ['cuba_fwd_small', 'cuba_fused', 'cuba_fused_lean', 'alif', 'alif_fused', 'alif_fused_lean', 'rf', 'rf_fused',
          'synapse', 'synapse_fused', 'synapse_folded', 'synapse_delay_grad', 'block_tail', 'block_tail_folded',
-         'conv_synapse', 'conv_synapse_library', 'pool_synapse', 'recurrent', 'recurrent_loop']
+         'conv_synapse', 'conv_synapse_library', 'pool_synapse', 'conv_transpose_synapse', 'recurrent', 'recurrent_loop']
 
 
 def other_configs(dev, iters):
