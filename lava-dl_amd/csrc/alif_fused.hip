@@ -10,7 +10,9 @@
 namespace slayer {
 
 int launch_reduce_param_grad(float* grad, const float* partial, float* scratch, int64_t M, int64_t npb,
-                             int64_t num_params, hipStream_t stream);   // li.hip
+                             int64_t num_params, hipStream_t stream);  // li.hip
+int launch_reduce_param_grad_pair(float* grad_a, float* grad_b, const float* partial, float* scratch, int64_t M,
+                                  int64_t npb, int64_t num_a, int64_t num_b, hipStream_t stream);  // li.hip
 int launch_zero_fill(float* p, int64_t n, hipStream_t stream);          // li.hip
 bool bwd_scan_usable(int64_t M, int64_t npb, int64_t T);                // scan.hip
 int launch_cuba_bwd_scan(float* grad_in, float* partial_i, float* partial_v, const float* grad_spikes,
@@ -372,11 +374,8 @@ extern "C" int slayer_alif_bwd(float* grad_in, float* grad_i_decay, float* grad_
             if (int e = launch_zero_fill(grad_i_decay, num_i_decays, st)) return e;
             return launch_zero_fill(grad_v_decay, num_v_decays, st);
         }
-        float* scratch = workspace + 2 * M;
-        if (int e = launch_reduce_param_grad(grad_i_decay, workspace, scratch, M, neurons_per_batch, num_i_decays, st))
-            return e;
-        return launch_reduce_param_grad(grad_v_decay, workspace + M, scratch + 64 * num_i_decays, M,
-                                        neurons_per_batch, num_v_decays, st);
+        return launch_reduce_param_grad_pair(grad_i_decay, grad_v_decay, workspace, workspace + 2 * M, M, neurons_per_batch, num_i_decays,
+                                             num_v_decays, st);
     }
     return 0;
 }

@@ -92,11 +92,15 @@ struct LiBwd {
 constexpr int kRedBlock = 256;
 constexpr int kRedMaxSplit = 64;
 
+// (blockIdx.z = 1: the second gradient of a pair -- its partial sums follow the first's M, its slice sums the
+// first's num_params * kRedMaxSplit)
 __global__ __launch_bounds__(kRedBlock) void reduce_param_slices(float* scratch, const float* partial,
                                                                  int64_t M, int64_t npb, int64_t num_params,
                                                                  int split) {
     const int64_t j = blockIdx.x;
     const int s = blockIdx.y;
+    partial += (int64_t)blockIdx.z * M;
+    scratch += (int64_t)blockIdx.z * num_params * kRedMaxSplit;
     const int64_t block = num_params > 1 ? npb / num_params : npb;   // rows per batch element for parameter j
     const int64_t total = (M / npb) * block;
     const int64_t per = (total + split - 1) / split;
@@ -116,10 +120,11 @@ __global__ __launch_bounds__(kRedBlock) void reduce_param_slices(float* scratch,
     if (threadIdx.x == 0) scratch[j * split + s] = (float)red[0];
 }
 
-__global__ __launch_bounds__(kRedBlock) void reduce_param_final(float* grad, const float* scratch,
+__global__ __launch_bounds__(kRedBlock) void reduce_param_final(float* grad, float* grad_second, const float* scratch,
                                                                 int64_t num_params, int split) {
     const int64_t j = (int64_t)blockIdx.x * kRedBlock + threadIdx.x;
     if (j >= num_params) return;
+    if (blockIdx.z) { grad = grad_second; scratch += num_params * kRedMaxSplit; }
     double acc = 0.0;
     for (int s = 0; s < split; ++s) acc += (double)scratch[j * split + s];
     grad[j] = (float)acc;
@@ -155,7 +160,25 @@ int launch_reduce_param_grad(float* grad, const float* partial, float* scratch, 
                        scratch, partial, M, npb, num_params, split);
     if (int e = (int)hipGetLastError()) return e;
     hipLaunchKernelGGL(reduce_param_final, dim3((unsigned)((num_params + kRedBlock - 1) / kRedBlock)),
-                       dim3(kRedBlock), 0, stream, grad, scratch, num_params, split);
+                       dim3(kRedBlock), 0, stream, grad, (float*)nullptr, scratch, num_params, split);
+    return (int)hipGetLastError();
+}
+
+// Two gradients of one backward pass (both decays of a CUBA or ALIF neuron, sine and cosine of a resonator): their
+// partial sums lie one after the other (M floats each), their slice sums likewise (kRedMaxSplit per parameter).
+// With as many parameters each, the two reductions share their two launches.
+int launch_reduce_param_grad_pair(float* grad_a, float* grad_b, const float* partial, float* scratch, int64_t M,
+                                  int64_t npb, int64_t num_a, int64_t num_b, hipStream_t stream) {
+    if (num_a != num_b) {
+        if (int e = launch_reduce_param_grad(grad_a, partial, scratch, M, npb, num_a, stream)) return e;
+        return launch_reduce_param_grad(grad_b, partial + M, scratch + kRedMaxSplit * num_a, M, npb, num_b, stream);
+    }
+    const int split = param_grad_split(M, npb, num_a);
+    hipLaunchKernelGGL(reduce_param_slices, dim3((unsigned)num_a, (unsigned)split, 2), dim3(kRedBlock), 0, stream,
+                       scratch, partial, M, npb, num_a, split);
+    if (int e = (int)hipGetLastError()) return e;
+    hipLaunchKernelGGL(reduce_param_final, dim3((unsigned)((num_a + kRedBlock - 1) / kRedBlock), 1, 2),
+                       dim3(kRedBlock), 0, stream, grad_a, grad_b, scratch, num_a, split);
     return (int)hipGetLastError();
 }
 

@@ -5,7 +5,9 @@
 namespace slayer {
 
 int launch_reduce_param_grad(float* grad, const float* partial, float* scratch, int64_t M, int64_t npb,
-                             int64_t num_params, hipStream_t stream);   // li.hip
+                             int64_t num_params, hipStream_t stream);  // li.hip
+int launch_reduce_param_grad_pair(float* grad_a, float* grad_b, const float* partial, float* scratch, int64_t M,
+                                  int64_t npb, int64_t num_a, int64_t num_b, hipStream_t stream);  // li.hip
 int launch_zero_fill(float* p, int64_t n, hipStream_t stream);          // li.hip
 
 template <bool POW2, bool HAS_THR>
@@ -254,11 +256,8 @@ extern "C" int slayer_res_bwd(float* g_re_in, float* g_im_in, float* grad_sin, f
             if (int e = launch_zero_fill(grad_sin, num_decays, st)) return e;
             return launch_zero_fill(grad_cos, num_decays, st);
         }
-        float* scratch = workspace + 2 * M;
-        if (int e = launch_reduce_param_grad(grad_sin, workspace, scratch, M, neurons_per_batch, num_decays, st))
-            return e;
-        return launch_reduce_param_grad(grad_cos, workspace + M, scratch + 64 * num_decays, M, neurons_per_batch,
-                                        num_decays, st);
+        return launch_reduce_param_grad_pair(grad_sin, grad_cos, workspace, workspace + 2 * M, M, neurons_per_batch, num_decays,
+                                             num_decays, st);
     }
     return 0;
 }

@@ -32,6 +32,7 @@ def _trips(slayer, call):
     try:
         call()
     except OverflowError:
+        _raised(slayer)             # workgroups of the call that are still running raise the flag again: wait, then lower it
         return True
     return _raised(slayer)
 
