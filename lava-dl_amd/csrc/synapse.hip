@@ -227,10 +227,21 @@ __device__ __forceinline__ void synapse_conv_row(const SynapseConv& p) {
     const int co0 = cob * 16;
 
     const int64_t k_full = (int64_t)p.Ci * p.kh_full * p.kw_full;
-    for (int i = tid; i < Kp * 16; i += kSynWaves * kWave) {
-        const int k = i >> 4, m = i & 15;
-        const int pr = k / KW, x = k - pr * KW, ci = pr / p.kh, y = pr - ci * p.kh;
-        wt[i] = (k < p.K && co0 + m < p.Co) ? p.weight[(int64_t)(co0 + m) * k_full + p.weight_index(ci, y, x)] : 0.0f;
+    // eight loads of a thread in flight at a time (one after the other they were a fifth of a workgroup's life)
+    for (int i0 = tid; i0 < Kp * 16; i0 += 8 * kSynWaves * kWave) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = i0 + u * kSynWaves * kWave;
+            const int k = i >> 4, m = i & 15;
+            const int pr = k / KW, x = k - pr * KW, ci = pr / p.kh, y = pr - ci * p.kh;
+            v[u] = (k < p.K && co0 + m < p.Co) ? p.weight[(int64_t)(co0 + m) * k_full + p.weight_index(ci, y, x)] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = i0 + u * kSynWaves * kWave;
+            if (i < Kp * 16) wt[i] = v[u];
+        }
     }
     for (int pr = tid; pr < 4 * PG; pr += kSynWaves * kWave) {
         const int ci = pr / p.kh, y = pr - ci * p.kh;
