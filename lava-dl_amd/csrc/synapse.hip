@@ -761,7 +761,7 @@ namespace {
 #endif
 
 // One launch of the convolution kernels for the geometry in p (tensors, sizes, taps and sub-lattices filled in by the
-// caller): the row kernel for unit stride and dilation along the image row with 3 or 5 taps per row, else the
+// caller): the row kernel for unit stride and dilation along the image row with 2, 3 or 5 taps per row, else the
 // one-pixel kernel with as many tap groups in flight as the filter has, up to six.  A filter without taps (K = 0)
 // clears its outputs.
 int launch_synapse_conv(SynapseConv p, bool streaming, hipStream_t st) {
